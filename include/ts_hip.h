@@ -1,0 +1,187 @@
+/*
+ * ts_hip.h -- C ABI of the MI355X (gfx950) scatter / segment / gather kernels.
+ *
+ * This is the boundary a torch_scatter-style host layer binds against in place
+ * of the reference's csrc/cuda launchers (scatter_cuda.h, segment_csr_cuda.h, segment_coo_cuda.h). Plain pointers and sizes only:
+ * no torch types, no exceptions, no allocation, no host synchronisation. The
+ * caller owns every buffer (device memory), holds the device guard and passes
+ * the stream to launch on. Every function returns TS_OK or a TS_ERR_* code;
+ * ts_error_string() turns a code into text.
+ *
+ * Shapes use the reference's flattening (csrc/cuda/scatter_cuda.cu:105-110,
+ * segment_csr_cuda.cu:144-146, segment_coo_cuda.cu:208-212):
+ *   B  product of the dimensions before the reduced dimension
+ *   E  length of the reduced dimension of the edge-side tensor
+ *   K  product of the trailing (feature) dimensions
+ *   N  length of the reduced dimension of the node-side tensor
+ * src/out are contiguous row-major [B, E|N, K]. index / indptr are int64.
+ * arg outputs are int64 with E as the "empty slot" sentinel.
+ */
+#ifndef TS_HIP_H
+#define TS_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void *ts_stream_t; /* a hipStream_t; NULL is the default stream */
+
+/* element types of src/out (AT_DISPATCH_ALL_TYPES_AND2(Half, BFloat16),
+ * csrc/cuda/scatter_cuda.cu:114) */
+enum ts_dtype {
+  TS_F32 = 0, TS_F64 = 1, TS_F16 = 2, TS_BF16 = 3, TS_I32 = 4, TS_I64 = 5,
+  TS_I16 = 6, TS_I8 = 7, TS_U8 = 8
+};
+
+/* reduction codes, same order as the reference enum (csrc/cuda/reducer.cuh:8) */
+enum ts_reduce {
+  TS_SUM = 0, TS_MEAN = 1, TS_MUL = 2, TS_DIV = 3, TS_MIN = 4, TS_MAX = 5
+};
+
+enum ts_status {
+  TS_OK = 0,
+  TS_ERR_BAD_ARG = 1,     /* null pointer, negative size, unknown code */
+  TS_ERR_UNSUPPORTED = 2, /* combination this library has no kernel for */
+  TS_ERR_WORKSPACE = 3,   /* workspace missing or too small */
+  TS_ERR_LAUNCH = 4       /* the HIP runtime rejected a launch */
+};
+
+const char *ts_error_string(int status);
+
+/* HIP_VERSION this library was built against.
+ * Replaces scatter::cuda_version(), csrc/version.cpp:28-38. */
+int64_t ts_hip_version(void);
+
+/* ------------------------------------------------------------ segment_csr
+ * out[b, n, :] = reduce over e in [indptr[b, n], indptr[b, n+1]) of src[b, e, :]
+ * Replaces segment_csr_cuda, csrc/cuda/segment_csr_cuda.cu:97-168 (kernels
+ * :15-95). Every row of out is written (empty row: 0, arg = E); mean divides
+ * by max(count, 1). reduce in {SUM, MEAN, MIN, MAX}; arg_out is required for
+ * MIN/MAX and ignored otherwise.
+ *
+ * indptr holds N+1 entries per batch row, unit inner stride;
+ * indptr_batch_stride is the element distance between batch rows (0 when one
+ * indptr row is shared by all batches).
+ *
+ * workspace: ts_segment_csr_workspace_bytes() bytes of device scratch for the
+ * partial results of rows that cross a tile boundary (may be 0 -> NULL ok).
+ */
+size_t ts_segment_csr_workspace_bytes(int64_t B, int64_t N, int64_t E, int64_t K,
+                                      int dtype, int reduce);
+int ts_segment_csr(const void *src, const int64_t *indptr, void *out,
+                   int64_t *arg_out, int64_t B, int64_t N, int64_t E, int64_t K,
+                   int64_t indptr_batch_stride, int dtype, int reduce,
+                   void *workspace, size_t workspace_bytes, ts_stream_t stream);
+
+/* ------------------------------------------------------------- gather_csr
+ * out[b, e, :] = src[b, n, :] for e in [indptr[b, n], indptr[b, n+1])
+ * Replaces gather_csr_cuda, csrc/cuda/segment_csr_cuda.cu:219-281 (kernels
+ * :170-217). Positions of out not covered by any row are left untouched.
+ */
+int ts_gather_csr(const void *src, const int64_t *indptr, void *out, int64_t B,
+                  int64_t N, int64_t E, int64_t K, int64_t indptr_batch_stride,
+                  int dtype, ts_stream_t stream);
+
+/* Fused backward of segment_csr(mean):
+ *   grad_in[b, e, :] = grad_out[b, n, :] / (T)max(count_n, 1)
+ * One pass instead of the reference's gather + gather-of-count + divide,
+ * SegmentMeanCSR::backward, csrc/segment_csr.cpp:94-111. The count is cast to
+ * the element type before the division, as there. Floating types only.
+ */
+int ts_segment_mean_csr_backward(const void *grad_out, const int64_t *indptr,
+                                 void *grad_in, int64_t B, int64_t N, int64_t E,
+                                 int64_t K, int64_t indptr_batch_stride,
+                                 int dtype, ts_stream_t stream);
+
+/* ------------------------------------------------------------ segment_coo
+ * Reduction keyed by a non-decreasing index (index[b, e] in [0, N)).
+ * Replaces segment_coo_cuda, csrc/cuda/segment_coo_cuda.cu:152-283 (kernels
+ * :14-150).
+ *   out_given == 0: every row of out is written (row without entries: 0,
+ *                   arg = E).
+ *   out_given != 0: rows with entries are combined with their previous
+ *                   content (sum: prev + sum; mean: (prev + sum) / count;
+ *                   min/max: entries must strictly beat prev, else arg = E);
+ *                   other rows are left untouched. arg_out must be pre-filled
+ *                   with E by the caller in this mode.
+ * count_out (MEAN only, may be NULL): [B, N] element-typed, max(count, 1).
+ * index: unit inner stride, index_batch_stride elements between batch rows
+ * (0 when shared).
+ *
+ * workspace: ts_segment_coo_workspace_bytes() bytes; holds the row-pointer
+ * array derived from the index and the cross-tile partials.
+ */
+size_t ts_segment_coo_workspace_bytes(int64_t B, int64_t N, int64_t E, int64_t K,
+                                      int dtype, int reduce);
+int ts_segment_coo(const void *src, const int64_t *index, void *out,
+                   void *arg_out, void *count_out, int64_t B, int64_t N,
+                   int64_t E, int64_t K, int64_t index_batch_stride, int dtype,
+                   int reduce, int out_given, void *workspace,
+                   size_t workspace_bytes, ts_stream_t stream);
+
+/* ------------------------------------------------------------- gather_coo
+ * out[b, e, :] = src[b, index[b, e], :]
+ * Replaces gather_coo_cuda, csrc/cuda/segment_coo_cuda.cu:327-382 (kernels
+ * :285-325).
+ */
+int ts_gather_coo(const void *src, const int64_t *index, void *out, int64_t B,
+                  int64_t N, int64_t E, int64_t K, int64_t index_batch_stride,
+                  int dtype, ts_stream_t stream);
+
+/* Fused backward of segment_coo(mean):
+ *   grad_in[b, e, :] = grad_out[b, index[b,e], :] / count[b, index[b,e]]
+ * SegmentMeanCOO::backward, csrc/segment_coo.cpp:99-112. count is the
+ * element-typed [B, N] tensor the forward produced.
+ */
+int ts_segment_mean_coo_backward(const void *grad_out, const int64_t *index,
+                                 const void *count, void *grad_in, int64_t B,
+                                 int64_t N, int64_t E, int64_t K,
+                                 int64_t index_batch_stride, int dtype,
+                                 ts_stream_t stream);
+
+/* ---------------------------------------------------------------- scatter
+ * out[b, index[b,e,k], k] (op)= src[b, e, k]   for an unsorted index.
+ * Replaces scatter_cuda, csrc/cuda/scatter_cuda.cu:58-138 (kernels :13-56),
+ * including its helper passes: the initial fill, the init->0 masking and the
+ * arg resolution. reduce in {SUM, MUL, MIN, MAX} (mean is sum + ts_scatter_count
+ * + ts_divide_by_count, as ScatterMean does, csrc/scatter.cpp:115-161).
+ *   out_given == 0: out is initialised by the call; untouched slots end as 0
+ *                   (1 for MUL) with arg = E.
+ *   out_given != 0: accumulate into out; arg_out (MIN/MAX) is fully written:
+ *                   E where no entry strictly beat the previous content.
+ * Ties keep the smallest e (the CPU rule, csrc/cpu/reducer.h:63-67).
+ * The index element of (b, e, k) is index[b*sb + e*se + k*sk]; a 1-D index
+ * broadcast along dim is sb = 0, se = 1, sk = 0.
+ */
+int ts_scatter(const void *src, const int64_t *index, void *out,
+               int64_t *arg_out, int64_t B, int64_t E, int64_t K, int64_t N,
+               int64_t index_stride_b, int64_t index_stride_e,
+               int64_t index_stride_k, int dtype, int reduce, int out_given,
+               ts_stream_t stream);
+
+/* count[b, index[b*sb + e*se]] += 1 as float32, count pre-zeroed by the call.
+ * The count half of ScatterMean::forward, csrc/scatter.cpp:131-137. */
+int ts_scatter_count(const int64_t *index, float *count, int64_t B, int64_t E,
+                     int64_t N, int64_t index_stride_b, int64_t index_stride_e,
+                     ts_stream_t stream);
+
+/* out[b, n, k] = out[b, n, k] / (T)max(count[b, n], 1): true division for
+ * floating types, floor division for integers (csrc/scatter.cpp:138-141). */
+int ts_divide_by_count(void *out, const float *count, int64_t B, int64_t N,
+                       int64_t K, int dtype, ts_stream_t stream);
+
+/* Backward of every min/max flavour (csrc/scatter.cpp:184-196,
+ * segment_coo.cpp:132-144, segment_csr.cpp:130-142):
+ *   grad_in = 0; grad_in[b, arg[b,n,k], k] = grad_out[b,n,k] where arg < E.
+ */
+int ts_arg_backward(const void *grad_out, const int64_t *arg, void *grad_in,
+                    int64_t B, int64_t N, int64_t E, int64_t K, int dtype,
+                    ts_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TS_HIP_H */

@@ -1,0 +1,162 @@
+"""ctypes binding of the C ABI in ``include/ts_hip.h`` (``libts_hip.so``).
+
+Kernel-level entry points on flattened ``[B, E|N, K]`` buffers. PyTorch is used
+only to own device memory and to name the stream; every call launches on the
+current stream of the tensors' device and never synchronises. The library must
+have been built (``python -c "import __graft_entry__ as g; g.build()"`` or
+``make -C pytorch_scatter_amd/csrc``): there is no fallback path.
+"""
+import ctypes
+import os
+from typing import Optional
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libts_hip.so")
+
+SUM, MEAN, MUL, DIV, MIN, MAX = range(6)
+REDUCE = {"sum": SUM, "add": SUM, "mean": MEAN, "mul": MUL, "min": MIN, "max": MAX}
+DTYPE = {torch.float32: 0, torch.float64: 1, torch.float16: 2, torch.bfloat16: 3,
+         torch.int32: 4, torch.int64: 5, torch.int16: 6, torch.int8: 7, torch.uint8: 8}
+
+EXPORTS = (
+    "ts_error_string", "ts_hip_version",
+    "ts_segment_csr_workspace_bytes", "ts_segment_csr", "ts_gather_csr",
+    "ts_segment_mean_csr_backward",
+    "ts_segment_coo_workspace_bytes", "ts_segment_coo", "ts_gather_coo",
+    "ts_segment_mean_coo_backward",
+    "ts_scatter", "ts_scatter_count", "ts_divide_by_count", "ts_arg_backward",
+)
+
+_lib = None
+
+
+class TsError(RuntimeError):
+    pass
+
+
+def lib() -> ctypes.CDLL:
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(
+                f"{LIB_PATH} is missing: the HIP kernels are not built "
+                "(run `make -C pytorch_scatter_amd/csrc -j8`); there is no CPU fallback")
+        _lib = ctypes.CDLL(LIB_PATH)
+        _lib.ts_error_string.restype = ctypes.c_char_p
+        _lib.ts_hip_version.restype = ctypes.c_int64
+        _lib.ts_segment_csr_workspace_bytes.restype = ctypes.c_size_t
+        _lib.ts_segment_coo_workspace_bytes.restype = ctypes.c_size_t
+    return _lib
+
+
+def _check(rc: int):
+    if rc != 0:
+        raise TsError(f"ts_hip: {lib().ts_error_string(rc).decode()} (status {rc})")
+
+
+def _p(t: Optional[torch.Tensor]):
+    return ctypes.c_void_p(0 if t is None else t.data_ptr())
+
+
+def _i(v):
+    return ctypes.c_int64(int(v))
+
+
+def _stream(t: torch.Tensor):
+    return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+def _dev(*ts):
+    for t in ts:
+        if t is not None and not t.is_cuda:
+            raise TsError("ts_hip: all buffers must be device (HIP) tensors")
+
+
+def hip_version() -> int:
+    return int(lib().ts_hip_version())
+
+
+def segment_csr(src, indptr, out, arg_out, B, N, E, K, indptr_batch_stride, reduce: int):
+    _dev(src, indptr, out, arg_out)
+    L = lib()
+    nbytes = L.ts_segment_csr_workspace_bytes(_i(B), _i(N), _i(E), _i(K), DTYPE[out.dtype], reduce)
+    ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=out.device)
+    with torch.cuda.device(out.device):
+        _check(L.ts_segment_csr(_p(src), _p(indptr), _p(out), _p(arg_out), _i(B), _i(N), _i(E), _i(K),
+                                _i(indptr_batch_stride), DTYPE[out.dtype], reduce, _p(ws),
+                                ctypes.c_size_t(nbytes), _stream(out)))
+    return ws
+
+
+def gather_csr(src, indptr, out, B, N, E, K, indptr_batch_stride):
+    _dev(src, indptr, out)
+    with torch.cuda.device(out.device):
+        _check(lib().ts_gather_csr(_p(src), _p(indptr), _p(out), _i(B), _i(N), _i(E), _i(K),
+                                   _i(indptr_batch_stride), DTYPE[out.dtype], _stream(out)))
+
+
+def segment_mean_csr_backward(grad_out, indptr, grad_in, B, N, E, K, indptr_batch_stride):
+    _dev(grad_out, indptr, grad_in)
+    with torch.cuda.device(grad_in.device):
+        _check(lib().ts_segment_mean_csr_backward(_p(grad_out), _p(indptr), _p(grad_in), _i(B), _i(N),
+                                                  _i(E), _i(K), _i(indptr_batch_stride),
+                                                  DTYPE[grad_in.dtype], _stream(grad_in)))
+
+
+def segment_coo(src, index, out, arg_out, count_out, B, N, E, K, index_batch_stride, reduce: int,
+                out_given: bool):
+    _dev(src, index, out, arg_out, count_out)
+    L = lib()
+    nbytes = L.ts_segment_coo_workspace_bytes(_i(B), _i(N), _i(E), _i(K), DTYPE[out.dtype], reduce)
+    ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=out.device)
+    with torch.cuda.device(out.device):
+        _check(L.ts_segment_coo(_p(src), _p(index), _p(out), _p(arg_out), _p(count_out), _i(B), _i(N),
+                                _i(E), _i(K), _i(index_batch_stride), DTYPE[out.dtype], reduce,
+                                int(out_given), _p(ws), ctypes.c_size_t(nbytes), _stream(out)))
+    return ws
+
+
+def gather_coo(src, index, out, B, N, E, K, index_batch_stride):
+    _dev(src, index, out)
+    with torch.cuda.device(out.device):
+        _check(lib().ts_gather_coo(_p(src), _p(index), _p(out), _i(B), _i(N), _i(E), _i(K),
+                                   _i(index_batch_stride), DTYPE[out.dtype], _stream(out)))
+
+
+def segment_mean_coo_backward(grad_out, index, count, grad_in, B, N, E, K, index_batch_stride):
+    _dev(grad_out, index, count, grad_in)
+    with torch.cuda.device(grad_in.device):
+        _check(lib().ts_segment_mean_coo_backward(_p(grad_out), _p(index), _p(count), _p(grad_in), _i(B),
+                                                  _i(N), _i(E), _i(K), _i(index_batch_stride),
+                                                  DTYPE[grad_in.dtype], _stream(grad_in)))
+
+
+def scatter(src, index, out, arg_out, B, E, K, N, sb, se, sk, reduce: int, out_given: bool):
+    _dev(src, index, out, arg_out)
+    with torch.cuda.device(out.device):
+        _check(lib().ts_scatter(_p(src), _p(index), _p(out), _p(arg_out), _i(B), _i(E), _i(K), _i(N),
+                                _i(sb), _i(se), _i(sk), DTYPE[out.dtype], reduce, int(out_given),
+                                _stream(out)))
+
+
+def scatter_count(index, count, B, E, N, sb, se):
+    _dev(index, count)
+    with torch.cuda.device(count.device):
+        _check(lib().ts_scatter_count(_p(index), _p(count), _i(B), _i(E), _i(N), _i(sb), _i(se),
+                                      _stream(count)))
+
+
+def divide_by_count(out, count, B, N, K):
+    _dev(out, count)
+    with torch.cuda.device(out.device):
+        _check(lib().ts_divide_by_count(_p(out), _p(count), _i(B), _i(N), _i(K), DTYPE[out.dtype],
+                                        _stream(out)))
+
+
+def arg_backward(grad_out, arg, grad_in, B, N, E, K):
+    _dev(grad_out, arg, grad_in)
+    with torch.cuda.device(grad_in.device):
+        _check(lib().ts_arg_backward(_p(grad_out), _p(arg), _p(grad_in), _i(B), _i(N), _i(E), _i(K),
+                                     DTYPE[grad_in.dtype], _stream(grad_in)))

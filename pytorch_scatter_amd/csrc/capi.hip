@@ -1,0 +1,314 @@
+// The C ABI declared in include/ts_hip.h: argument checks, kernel plans and
+// dispatch on the element type. Nothing here allocates or synchronises.
+#include <hip/hip_runtime.h>
+#include <hip/hip_version.h>
+#include <stdlib.h>
+
+#include "csr_reduce.h"
+#include "csr_gather.h"
+#include "coo_gather.h"
+#include "scatter.h"
+#include "elementwise.h"
+
+using namespace ts;
+
+namespace {
+
+const int kElemBytes[9] = {4, 8, 2, 2, 4, 8, 2, 1, 1};
+const int kAccBytes[9] = {4, 8, 4, 4, 4, 8, 2, 1, 1};
+
+inline bool valid_dtype(int d) { return d >= 0 && d < 9; }
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+inline bool is_float_dtype(int d) { return d == TS_F32 || d == TS_F64 || d == TS_F16 || d == TS_BF16; }
+
+#define TS_DISPATCH(dtype, EXPR)                      \
+  switch (dtype) {                                    \
+  case TS_F32: { typedef float T; return EXPR; }      \
+  case TS_F64: { typedef double T; return EXPR; }     \
+  case TS_F16: { typedef f16_t T; return EXPR; }      \
+  case TS_BF16: { typedef bf16_t T; return EXPR; }    \
+  case TS_I32: { typedef int32_t T; return EXPR; }    \
+  case TS_I64: { typedef int64_t T; return EXPR; }    \
+  case TS_I16: { typedef int16_t T; return EXPR; }    \
+  case TS_I8: { typedef int8_t T; return EXPR; }      \
+  case TS_U8: { typedef uint8_t T; return EXPR; }     \
+  default: return TS_ERR_BAD_ARG;                     \
+  }
+
+int dispatch_csr_reduce(int dtype, const CsrReduceArgs &a, const CsrPlan &p, int64_t B, int reduce,
+                        hipStream_t s) {
+  TS_DISPATCH(dtype, launch_csr_reduce<T>(a, p, B, reduce, s))
+}
+int dispatch_csr_gather(int dtype, const CsrGatherArgs &a, const CsrPlan &p, int64_t B, bool divide,
+                        hipStream_t s) {
+  TS_DISPATCH(dtype, launch_csr_gather<T>(a, p, B, divide, s))
+}
+int dispatch_coo_gather(int dtype, const CooGatherArgs &a, const CooGatherPlan &p, int64_t B,
+                        bool divide, hipStream_t s) {
+  TS_DISPATCH(dtype, launch_coo_gather<T>(a, p, B, divide, s))
+}
+int dispatch_scatter(int dtype, const ScatterArgs &a, int reduce, int vec, hipStream_t s) {
+  TS_DISPATCH(dtype, launch_scatter<T>(a, reduce, vec, s))
+}
+int dispatch_divide(int dtype, void *out, const float *count, int64_t rows, int64_t K, hipStream_t s) {
+  TS_DISPATCH(dtype, launch_divide_by_count<T>(out, count, rows, K, s))
+}
+int dispatch_arg_backward(int dtype, const void *g, const int64_t *arg, void *gi, int64_t B, int64_t N,
+                          int64_t E, int64_t K, hipStream_t s) {
+  TS_DISPATCH(dtype, launch_arg_backward<T>(g, arg, gi, B, N, E, K, s))
+}
+
+// The reduction keeps edge positions in 32 bits inside a tile.
+inline bool sizes_ok(int64_t B, int64_t N, int64_t E, int64_t K) {
+  return B >= 0 && N >= 0 && E >= 0 && K >= 0 && E < 0x7FFFFFFFll && N < 0x7FFFFFFFll &&
+         B <= 65535 && K < ((int64_t)1 << 40);
+}
+
+int env_int(const char *name, int fallback) {
+  const char *v = getenv(name);
+  return v ? atoi(v) : fallback;
+}
+
+struct CsrWs {
+  size_t total, off_args, off_meta;
+};
+
+CsrWs csr_workspace(const CsrPlan &p, int64_t B, int64_t K, int dtype, int reduce) {
+  CsrWs w;
+  w.total = csr_ws_bytes(p, B, K, kAccBytes[dtype], reduce == TS_MIN || reduce == TS_MAX, &w.off_args,
+                         &w.off_meta);
+  return w;
+}
+
+int run_csr_reduce(const void *src, const int64_t *indptr, void *out, int64_t *arg_out, void *count_out,
+                   int64_t B, int64_t N, int64_t E, int64_t K, int64_t indptr_batch_stride, int dtype,
+                   int reduce, int accumulate, void *ws, size_t ws_bytes, hipStream_t stream) {
+  const bool al = aligned16(src) && aligned16(out);
+  const CsrPlan p = csr_plan(N, E, K, kElemBytes[dtype], al);
+  const CsrWs w = csr_workspace(p, B, K, dtype, reduce);
+  if (ws == nullptr || ws_bytes < w.total) return TS_ERR_WORKSPACE;
+  CsrReduceArgs a;
+  a.src = src;
+  a.indptr = indptr;
+  a.out = out;
+  a.arg_out = arg_out;
+  a.count_out = count_out;
+  a.N = N;
+  a.E = E;
+  a.K = K;
+  a.indptr_batch_stride = indptr_batch_stride;
+  a.accumulate = accumulate;
+  a.G = p.G;
+  a.BI = p.BI;
+  a.nblk = p.nblk;
+  a.ws_vals = ws;
+  a.ws_args = reinterpret_cast<int32_t *>(static_cast<char *>(ws) + w.off_args);
+  a.ws_meta = reinterpret_cast<int64_t *>(static_cast<char *>(ws) + w.off_meta);
+  return dispatch_csr_reduce(dtype, a, p, B, reduce, stream);
+}
+
+}  // namespace
+
+extern "C" {
+
+const char *ts_error_string(int status) {
+  switch (status) {
+  case TS_OK: return "ok";
+  case TS_ERR_BAD_ARG: return "bad argument (null pointer, negative size or unknown dtype/reduce code)";
+  case TS_ERR_UNSUPPORTED: return "unsupported combination of dtype / reduce / size";
+  case TS_ERR_WORKSPACE: return "workspace missing or too small";
+  case TS_ERR_LAUNCH: return "HIP kernel launch failed";
+  default: return "unknown status";
+  }
+}
+
+int64_t ts_hip_version(void) { return HIP_VERSION; }
+
+size_t ts_segment_csr_workspace_bytes(int64_t B, int64_t N, int64_t E, int64_t K, int dtype, int reduce) {
+  if (!valid_dtype(dtype) || !sizes_ok(B, N, E, K)) return 0;
+  // the plan may fall back to one element per lane for unaligned buffers; the
+  // tile count does not depend on that choice
+  const CsrPlan p = csr_plan(N, E, K, kElemBytes[dtype], true);
+  return csr_workspace(p, B, K, dtype, reduce).total;
+}
+
+int ts_segment_csr(const void *src, const int64_t *indptr, void *out, int64_t *arg_out, int64_t B,
+                   int64_t N, int64_t E, int64_t K, int64_t indptr_batch_stride, int dtype, int reduce,
+                   void *workspace, size_t workspace_bytes, ts_stream_t stream) {
+  if (!valid_dtype(dtype) || !sizes_ok(B, N, E, K)) return TS_ERR_BAD_ARG;
+  if (reduce != TS_SUM && reduce != TS_MEAN && reduce != TS_MIN && reduce != TS_MAX) return TS_ERR_UNSUPPORTED;
+  if (B * N * K == 0) return TS_OK;
+  if (!indptr || !out || (E * K > 0 && !src)) return TS_ERR_BAD_ARG;
+  if ((reduce == TS_MIN || reduce == TS_MAX) && !arg_out) return TS_ERR_BAD_ARG;
+  return run_csr_reduce(src, indptr, out, arg_out, nullptr, B, N, E, K, indptr_batch_stride, dtype,
+                        reduce, 0, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
+}
+
+int ts_gather_csr(const void *src, const int64_t *indptr, void *out, int64_t B, int64_t N, int64_t E,
+                  int64_t K, int64_t indptr_batch_stride, int dtype, ts_stream_t stream) {
+  if (!valid_dtype(dtype) || !sizes_ok(B, N, E, K)) return TS_ERR_BAD_ARG;
+  if (B * E * K == 0 || N == 0) return TS_OK;
+  if (!src || !indptr || !out) return TS_ERR_BAD_ARG;
+  const CsrPlan p = csr_plan(N, E, K, kElemBytes[dtype], aligned16(src) && aligned16(out));
+  CsrGatherArgs a;
+  a.src = src;
+  a.indptr = indptr;
+  a.out = out;
+  a.N = N;
+  a.E = E;
+  a.K = K;
+  a.indptr_batch_stride = indptr_batch_stride;
+  a.G = p.G;
+  a.BI = p.BI;
+  a.nblk = p.nblk;
+  return dispatch_csr_gather(dtype, a, p, B, false, static_cast<hipStream_t>(stream));
+}
+
+int ts_segment_mean_csr_backward(const void *grad_out, const int64_t *indptr, void *grad_in, int64_t B,
+                                 int64_t N, int64_t E, int64_t K, int64_t indptr_batch_stride, int dtype,
+                                 ts_stream_t stream) {
+  if (!valid_dtype(dtype) || !sizes_ok(B, N, E, K)) return TS_ERR_BAD_ARG;
+  if (!is_float_dtype(dtype)) return TS_ERR_UNSUPPORTED;
+  if (B * E * K == 0 || N == 0) return TS_OK;
+  if (!grad_out || !indptr || !grad_in) return TS_ERR_BAD_ARG;
+  const CsrPlan p = csr_plan(N, E, K, kElemBytes[dtype], aligned16(grad_out) && aligned16(grad_in));
+  CsrGatherArgs a;
+  a.src = grad_out;
+  a.indptr = indptr;
+  a.out = grad_in;
+  a.N = N;
+  a.E = E;
+  a.K = K;
+  a.indptr_batch_stride = indptr_batch_stride;
+  a.G = p.G;
+  a.BI = p.BI;
+  a.nblk = p.nblk;
+  return dispatch_csr_gather(dtype, a, p, B, true, static_cast<hipStream_t>(stream));
+}
+
+size_t ts_segment_coo_workspace_bytes(int64_t B, int64_t N, int64_t E, int64_t K, int dtype, int reduce) {
+  if (!valid_dtype(dtype) || !sizes_ok(B, N, E, K)) return 0;
+  const CsrPlan p = csr_plan(N, E, K, kElemBytes[dtype], true);
+  const size_t ptr_bytes = ((size_t)B * (N + 1) * 8 + 255) & ~(size_t)255;
+  return ptr_bytes + csr_workspace(p, B, K, dtype, reduce).total;
+}
+
+int ts_segment_coo(const void *src, const int64_t *index, void *out, void *arg_out, void *count_out,
+                   int64_t B, int64_t N, int64_t E, int64_t K, int64_t index_batch_stride, int dtype,
+                   int reduce, int out_given, void *workspace, size_t workspace_bytes, ts_stream_t stream) {
+  if (!valid_dtype(dtype) || !sizes_ok(B, N, E, K)) return TS_ERR_BAD_ARG;
+  if (reduce != TS_SUM && reduce != TS_MEAN && reduce != TS_MIN && reduce != TS_MAX) return TS_ERR_UNSUPPORTED;
+  if (B * N * K == 0) return TS_OK;
+  if (!out || (E > 0 && (!index || (K > 0 && !src)))) return TS_ERR_BAD_ARG;
+  if ((reduce == TS_MIN || reduce == TS_MAX) && !arg_out) return TS_ERR_BAD_ARG;
+  const size_t ptr_bytes = ((size_t)B * (N + 1) * 8 + 255) & ~(size_t)255;
+  if (!workspace || workspace_bytes < ptr_bytes) return TS_ERR_WORKSPACE;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  int64_t *ptr = static_cast<int64_t *>(workspace);
+  dim3 grid((unsigned)((E + 1 + kBlock - 1) / kBlock), (unsigned)B);
+  hipLaunchKernelGGL(coo_to_indptr_kernel, grid, dim3(kBlock), 0, s, index, ptr, N, E, index_batch_stride);
+  if (hipGetLastError() != hipSuccess) return TS_ERR_LAUNCH;
+  return run_csr_reduce(src, ptr, out, static_cast<int64_t *>(arg_out), count_out, B, N, E, K, N + 1, dtype,
+                        reduce, out_given ? 1 : 0, static_cast<char *>(workspace) + ptr_bytes,
+                        workspace_bytes - ptr_bytes, s);
+}
+
+int ts_gather_coo(const void *src, const int64_t *index, void *out, int64_t B, int64_t N, int64_t E,
+                  int64_t K, int64_t index_batch_stride, int dtype, ts_stream_t stream) {
+  if (!valid_dtype(dtype) || !sizes_ok(B, N, E, K)) return TS_ERR_BAD_ARG;
+  if (B * E * K == 0 || N == 0) return TS_OK;
+  if (!src || !index || !out) return TS_ERR_BAD_ARG;
+  const CooGatherPlan p = coo_gather_plan(E, K, kElemBytes[dtype], aligned16(src) && aligned16(out));
+  CooGatherArgs a;
+  a.src = src;
+  a.index = index;
+  a.count = nullptr;
+  a.out = out;
+  a.N = N;
+  a.E = E;
+  a.K = K;
+  a.index_batch_stride = index_batch_stride;
+  a.G = p.G;
+  a.epw = p.epw;
+  return dispatch_coo_gather(dtype, a, p, B, false, static_cast<hipStream_t>(stream));
+}
+
+int ts_segment_mean_coo_backward(const void *grad_out, const int64_t *index, const void *count,
+                                 void *grad_in, int64_t B, int64_t N, int64_t E, int64_t K,
+                                 int64_t index_batch_stride, int dtype, ts_stream_t stream) {
+  if (!valid_dtype(dtype) || !sizes_ok(B, N, E, K)) return TS_ERR_BAD_ARG;
+  if (!is_float_dtype(dtype)) return TS_ERR_UNSUPPORTED;
+  if (B * E * K == 0 || N == 0) return TS_OK;
+  if (!grad_out || !index || !count || !grad_in) return TS_ERR_BAD_ARG;
+  const CooGatherPlan p = coo_gather_plan(E, K, kElemBytes[dtype], aligned16(grad_out) && aligned16(grad_in));
+  CooGatherArgs a;
+  a.src = grad_out;
+  a.index = index;
+  a.count = count;
+  a.out = grad_in;
+  a.N = N;
+  a.E = E;
+  a.K = K;
+  a.index_batch_stride = index_batch_stride;
+  a.G = p.G;
+  a.epw = p.epw;
+  return dispatch_coo_gather(dtype, a, p, B, true, static_cast<hipStream_t>(stream));
+}
+
+int ts_scatter(const void *src, const int64_t *index, void *out, int64_t *arg_out, int64_t B, int64_t E,
+               int64_t K, int64_t N, int64_t index_stride_b, int64_t index_stride_e, int64_t index_stride_k,
+               int dtype, int reduce, int out_given, ts_stream_t stream) {
+  if (!valid_dtype(dtype) || !sizes_ok(B, N, E, K)) return TS_ERR_BAD_ARG;
+  if (reduce != TS_SUM && reduce != TS_MUL && reduce != TS_MIN && reduce != TS_MAX) return TS_ERR_UNSUPPORTED;
+  if (B * N * K == 0) return TS_OK;
+  if (!out || (B * E * K > 0 && (!src || !index))) return TS_ERR_BAD_ARG;
+  if ((reduce == TS_MIN || reduce == TS_MAX) && !arg_out) return TS_ERR_BAD_ARG;
+  ScatterArgs a;
+  a.src = src;
+  a.index = index;
+  a.out = out;
+  a.arg_out = arg_out;
+  a.B = B;
+  a.E = E;
+  a.K = K;
+  a.N = N;
+  a.sb = index_stride_b;
+  a.se = index_stride_e;
+  a.sk = index_stride_k;
+  a.out_given = out_given ? 1 : 0;
+  a.precheck = env_int("TS_SCATTER_PRECHECK", 1);
+  const int full = kVecBytes / kElemBytes[dtype];
+  const int vec = (full > 1 && K % full == 0 && aligned16(src)) ? full : 1;
+  return dispatch_scatter(dtype, a, reduce, vec, static_cast<hipStream_t>(stream));
+}
+
+int ts_scatter_count(const int64_t *index, float *count, int64_t B, int64_t E, int64_t N,
+                     int64_t index_stride_b, int64_t index_stride_e, ts_stream_t stream) {
+  if (B < 0 || E < 0 || N < 0) return TS_ERR_BAD_ARG;
+  if (B * N == 0) return TS_OK;
+  if (!count || (B * E > 0 && !index)) return TS_ERR_BAD_ARG;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  hipLaunchKernelGGL(fill_kernel<float>, dim3(grid_for(B * N)), dim3(kBlock), 0, s, count, B * N, 0.0f);
+  if (B * E > 0)
+    hipLaunchKernelGGL(scatter_count_kernel, dim3(grid_for(B * E)), dim3(kBlock), 0, s, index, count, B, E,
+                       N, index_stride_b, index_stride_e);
+  return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
+}
+
+int ts_divide_by_count(void *out, const float *count, int64_t B, int64_t N, int64_t K, int dtype,
+                       ts_stream_t stream) {
+  if (!valid_dtype(dtype) || B < 0 || N < 0 || K < 0) return TS_ERR_BAD_ARG;
+  if (B * N * K == 0) return TS_OK;
+  if (!out || !count) return TS_ERR_BAD_ARG;
+  return dispatch_divide(dtype, out, count, B * N, K, static_cast<hipStream_t>(stream));
+}
+
+int ts_arg_backward(const void *grad_out, const int64_t *arg, void *grad_in, int64_t B, int64_t N, int64_t E,
+                    int64_t K, int dtype, ts_stream_t stream) {
+  if (!valid_dtype(dtype) || B < 0 || N < 0 || E < 0 || K < 0) return TS_ERR_BAD_ARG;
+  if (B * E * K == 0) return TS_OK;
+  if (!grad_in || (B * N * K > 0 && (!grad_out || !arg))) return TS_ERR_BAD_ARG;
+  return dispatch_arg_backward(dtype, grad_out, arg, grad_in, B, N, E, K, static_cast<hipStream_t>(stream));
+}
+
+}  // extern "C"

@@ -1,0 +1,116 @@
+// out[b, e, :] = src[b, index[b, e], :]   (gather_coo) and the fused backward
+// of segment_coo(mean), which divides the gathered row by count[index].
+//
+// Edges are independent, so the split is a plain even one: each worker (G
+// lanes holding one 16-byte-per-lane slice of a row) takes `epw` consecutive
+// edges and keeps U index loads, then U row loads, in flight. A sorted index
+// makes consecutive edges hit the same source row, which then comes from the
+// vector L1 / L2 rather than from HBM.
+#pragma once
+
+#include "device_utils.h"
+
+namespace ts {
+
+struct CooGatherArgs {
+  const void *src;      // [B, N, K]
+  const int64_t *index; // [B, E] (batch stride may be 0)
+  const void *count;    // [B, N] element-typed, DIV only
+  void *out;            // [B, E, K]
+  int64_t N, E, K;
+  int64_t index_batch_stride;
+  int G;
+  int epw;              // edges per worker
+};
+
+template <typename T, int VEC, bool DIV>
+__global__ __launch_bounds__(kBlock) void coo_gather_kernel(CooGatherArgs a) {
+  constexpr int U = 4;
+  const int G = a.G;
+  const int W = kBlock / G;
+  const int w = threadIdx.x / G;
+  const int lg = threadIdx.x - w * G;
+  const int64_t col = (int64_t)blockIdx.y * (G * VEC) + (int64_t)lg * VEC;
+  if (col >= a.K) return;
+  const int64_t b = blockIdx.z;
+  const int64_t *idx = a.index + b * a.index_batch_stride;
+  const T *src_b = static_cast<const T *>(a.src) + b * a.N * a.K;
+  const T *cnt_b = DIV ? static_cast<const T *>(a.count) + b * a.N : nullptr;
+  T *out_b = static_cast<T *>(a.out) + b * a.E * a.K;
+
+  const int64_t e0 = ((int64_t)blockIdx.x * W + w) * a.epw;
+  int64_t e1 = e0 + a.epw;
+  if (e1 > a.E) e1 = a.E;
+  for (int64_t e = e0; e < e1; e += U) {
+    int64_t n[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      int64_t ee = e + u < e1 ? e + u : e1 - 1;
+      int64_t v = idx[ee];
+      // an index outside [0, N) must not read out of bounds
+      n[u] = v < 0 ? 0 : (v >= a.N ? a.N - 1 : v);
+    }
+    Vec<T, VEC> x[U];
+    T c[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      x[u] = load_vec<T, VEC>(src_b + n[u] * a.K + col);
+      if (DIV) c[u] = cnt_b[n[u]];
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (e + u < e1) {
+        if (DIV) {
+#pragma unroll
+          for (int v = 0; v < VEC; ++v) x[u].v[v] = div_elem<T>(x[u].v[v], c[u]);
+        }
+        store_vec_stream<T, VEC>(out_b + (e + u) * a.K + col, x[u]);
+      }
+    }
+  }
+}
+
+struct CooGatherPlan {
+  int vec, G, ychunks, epw;
+  int64_t nblk;
+};
+
+inline CooGatherPlan coo_gather_plan(int64_t E, int64_t K, int elem_bytes, bool aligned16) {
+  CooGatherPlan p;
+  const int full = kVecBytes / elem_bytes;
+  p.vec = (aligned16 && full > 1 && K % full == 0) ? full : 1;
+  const int64_t lanes = (K + p.vec - 1) / p.vec;
+  int G = 1;
+  while (G < lanes && G < kWave) G <<= 1;
+  p.G = G;
+  p.ychunks = (int)((K + (int64_t)G * p.vec - 1) / ((int64_t)G * p.vec));
+  const int W = kBlock / G;
+  p.epw = E >= (1 << 22) ? 32 : (E >= (1 << 18) ? 16 : 8);
+  const int64_t per_block = (int64_t)W * p.epw;
+  p.nblk = (E + per_block - 1) / per_block;
+  if (p.nblk < 1) p.nblk = 1;
+  return p;
+}
+
+template <typename T, int VEC>
+int launch_coo_gather_v(const CooGatherArgs &a, const CooGatherPlan &p, int64_t B, bool divide,
+                        hipStream_t stream) {
+  dim3 grid((unsigned)p.nblk, (unsigned)p.ychunks, (unsigned)B);
+  if (divide)
+    hipLaunchKernelGGL((coo_gather_kernel<T, VEC, true>), grid, dim3(kBlock), 0, stream, a);
+  else
+    hipLaunchKernelGGL((coo_gather_kernel<T, VEC, false>), grid, dim3(kBlock), 0, stream, a);
+  return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
+}
+
+template <typename T> int launch_coo_gather(const CooGatherArgs &a, const CooGatherPlan &p,
+                                            int64_t B, bool divide, hipStream_t stream);
+
+#define TS_INSTANTIATE_COO_GATHER(T, FULLVEC)                                                \
+  template <> int launch_coo_gather<T>(const CooGatherArgs &a, const CooGatherPlan &p,       \
+                                       int64_t B, bool divide, hipStream_t stream) {         \
+    if (p.vec == FULLVEC) return launch_coo_gather_v<T, FULLVEC>(a, p, B, divide, stream);   \
+    return launch_coo_gather_v<T, 1>(a, p, B, divide, stream);                               \
+  }
+
+}  // namespace ts

@@ -1,0 +1,448 @@
+// Segmented reduction over CSR row pointers (segment_csr, and segment_coo once
+// its sorted index has been turned into row pointers).
+//
+// One pass over src. The merged list of edges and row ends is cut into tiles of
+// `BI` items per workgroup and `BI / W` items per lane group ("worker": G lanes
+// that together hold one 16-byte-per-lane slice of a feature row). A worker
+// walks its edges in order with U loads in flight, keeps the running reduction
+// in registers and writes every row that starts and ends inside its range
+// straight to `out`. A row that crosses a worker boundary leaves partials in
+// LDS which the workgroup combines in edge order; a row that crosses a
+// workgroup boundary leaves partials in the global workspace, combined in tile
+// order by a small second kernel. The result is independent of scheduling: no
+// atomics, no spinning.
+//
+// Semantics follow the reference CPU loop (csrc/cpu/segment_csr_cpu.cpp:54-88):
+// accumulate in float for 16-bit floats, strict compare so the first index
+// wins ties, mean = T(sum) / T(count), empty row -> 0 with arg = E.
+#pragma once
+
+#include "device_utils.h"
+#include "merge_path.h"
+
+namespace ts {
+
+constexpr int kMaxBlockItems = 2048;  // rows + edges per workgroup tile
+constexpr int kLoadsInFlight = 8;     // U: independent 16-byte loads per lane
+
+struct CsrReduceArgs {
+  const void *src;
+  const int64_t *indptr;
+  void *out;
+  int64_t *arg_out;   // min/max
+  void *count_out;    // optional, mean: T(max(count, 1)) per row
+  int64_t N, E, K;
+  int64_t indptr_batch_stride;
+  int accumulate;     // combine with the previous content of out (segment_coo with out=)
+  int G;              // lanes per worker
+  int BI;             // items per workgroup tile
+  int64_t nblk;       // tiles per batch
+  // workspace
+  void *ws_vals;      // Acc [B][nblk][2][K]
+  int32_t *ws_args;   // int32 [B][nblk][2][K]  (min/max)
+  int64_t *ws_meta;   // int64 [B][nblk][4]: head_row, head_closes, tail_row, -
+};
+
+template <typename A, int REDUCE>
+__device__ __forceinline__ void reduce_step(A &acc, int32_t &arg, A v, int32_t e) {
+  if (REDUCE == TS_SUM || REDUCE == TS_MEAN) {
+    acc = acc + v;
+  } else if (REDUCE == TS_MIN) {
+    if (v < acc) { acc = v; arg = e; }
+  } else {
+    if (v > acc) { acc = v; arg = e; }
+  }
+}
+
+// Write one finished row slice. `count` is the full length of the row.
+template <typename T, int VEC, int REDUCE>
+__device__ __forceinline__ void finalize_row(const CsrReduceArgs &a, T *out_b, int64_t *arg_b,
+                                             T *count_b, int64_t row, int64_t col, int lg,
+                                             const typename Acc<T>::type *acc, const int32_t *arg,
+                                             int64_t count, bool col_ok) {
+  typedef typename Acc<T>::type A;
+  if (!col_ok) return;
+  if (a.accumulate && count == 0) return;  // rows without entries keep their content
+  T *op = out_b + row * a.K + col;
+  Vec<T, VEC> o;
+  int64_t oa[VEC];
+  Vec<T, VEC> prev;
+  if (a.accumulate) prev = load_vec<T, VEC>(op);
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) {
+    A x = acc[v];
+    if (REDUCE == TS_SUM || REDUCE == TS_MEAN) {
+      if (a.accumulate) x = to_acc<T>(prev.v[v]) + x;
+      T t = from_acc<T>(x);
+      if (REDUCE == TS_MEAN) t = div_elem<T>(t, count_as<T>(count > 0 ? count : 1));
+      o.v[v] = t;
+    } else {
+      if (a.accumulate) {
+        const A p = to_acc<T>(prev.v[v]);
+        const bool beats = (REDUCE == TS_MIN) ? (x < p) : (x > p);
+        o.v[v] = beats ? from_acc<T>(x) : prev.v[v];
+        oa[v] = beats ? (int64_t)arg[v] : a.E;
+      } else {
+        o.v[v] = count > 0 ? from_acc<T>(x) : zero_elem<T>();
+        oa[v] = count > 0 ? (int64_t)arg[v] : a.E;
+      }
+    }
+  }
+  store_vec<T, VEC>(op, o);
+  if (REDUCE == TS_MIN || REDUCE == TS_MAX) {
+    int64_t *ap = arg_b + row * a.K + col;
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) ap[v] = oa[v];
+  }
+  if (REDUCE == TS_MEAN && count_b != nullptr && col == 0 && lg == 0)
+    count_b[row] = count_as<T>(count > 0 ? count : 1);
+}
+
+template <typename T, int VEC, int REDUCE>
+__global__ __launch_bounds__(kBlock) void csr_reduce_kernel(CsrReduceArgs a) {
+  typedef typename Acc<T>::type A;
+  constexpr bool kArg = (REDUCE == TS_MIN || REDUCE == TS_MAX);
+  constexpr int U = kLoadsInFlight;
+
+  __shared__ int32_t s_ptr[kMaxBlockItems + 2];
+  __shared__ A s_val[2 * kBlock * VEC];
+  __shared__ int32_t s_arg[kArg ? 2 * kBlock * VEC : 1];
+  __shared__ int32_t s_head_row[kBlock];    // local row of the head partial, -1: none
+  __shared__ int32_t s_head_closes[kBlock];
+  __shared__ int32_t s_tail_row[kBlock];    // local row of the tail partial, -1: none
+  __shared__ int64_t s_cut[2];
+
+  const int tid = threadIdx.x;
+  const int G = a.G;
+  const int W = kBlock / G;
+  const int w = tid / G;
+  const int lg = tid - w * G;
+  const int CW = G * VEC;
+  const int64_t col = (int64_t)blockIdx.y * CW + (int64_t)lg * VEC;
+  const bool col_ok = col < a.K;
+  const int64_t b = blockIdx.z;
+
+  const int64_t *ptr = a.indptr + b * a.indptr_batch_stride;
+  const T *src_b = static_cast<const T *>(a.src) + b * a.E * a.K;
+  T *out_b = static_cast<T *>(a.out) + b * a.N * a.K;
+  int64_t *arg_b = kArg ? a.arg_out + b * a.N * a.K : nullptr;
+  T *count_b = a.count_out ? static_cast<T *>(a.count_out) + b * a.N : nullptr;
+
+  // ---- tile cut: two wavefronts search the two diagonals concurrently
+  const int64_t total = a.N + a.E;
+  const int64_t d0 = (int64_t)blockIdx.x * a.BI;
+  const int64_t d1 = d0 + a.BI < total ? d0 + a.BI : total;
+  const int wave = tid / kWave;
+  if (wave < 2) {
+    const int64_t i = merge_search_wave(ptr, a.N, a.E, wave == 0 ? d0 : d1);
+    if ((tid & (kWave - 1)) == 0) s_cut[wave] = i;
+  }
+  __syncthreads();
+  const int64_t i0 = s_cut[0], i1 = s_cut[1];
+  const int64_t j0 = d0 - i0;
+  const int nr = (int)(i1 - i0);         // row ends inside the tile
+  const int ne = (int)((d1 - i1) - j0);  // edges inside the tile
+
+  // ---- row pointers of the tile into LDS, relative to the tile's first edge
+  const int64_t last = i1 + 1 < a.N ? i1 + 1 : a.N;
+  const int nload = (int)(last - i0) + 1;  // ptr[i0 .. last]
+  for (int t = tid; t < nload; t += kBlock) s_ptr[t] = (int32_t)(ptr[i0 + t] - j0);
+  s_head_row[tid] = -1;
+  s_tail_row[tid] = -1;
+  __syncthreads();
+
+  // ---- worker cut
+  const int ipw = a.BI / W;
+  const int tile_items = nr + ne;
+  int dw0 = w * ipw;
+  int dw1 = dw0 + ipw;
+  dw0 = dw0 < tile_items ? dw0 : tile_items;
+  dw1 = dw1 < tile_items ? dw1 : tile_items;
+  const int ri0 = merge_search_lds(s_ptr, nr, ne, dw0);
+  const int ri1 = merge_search_lds(s_ptr, nr, ne, dw1);
+  const int je0 = dw0 - ri0;
+  const int je1 = dw1 - ri1;
+
+  auto row_end = [&](int r) -> int32_t { return (r + 1 < nload) ? s_ptr[r + 1] : INT32_MAX; };
+
+  A acc[VEC];
+  int32_t arg[VEC];
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) { acc[v] = acc_init<A, REDUCE>(); arg[v] = 0; }
+
+  const bool has_work = (ri1 > ri0) || (je1 > je0);
+  // the worker's first row began before the worker's first edge
+  const bool head_open = has_work && (i0 + ri0 < a.N) && (s_ptr[ri0] < je0);
+
+  A *my_head_val = s_val + (size_t)w * CW + lg * VEC;
+  A *my_tail_val = s_val + (size_t)kBlock * VEC + (size_t)w * CW + lg * VEC;
+  int32_t *my_head_arg = s_arg + (kArg ? (size_t)w * CW + lg * VEC : 0);
+  int32_t *my_tail_arg = s_arg + (kArg ? (size_t)kBlock * VEC + (size_t)w * CW + lg * VEC : 0);
+
+  int r = ri0;
+  int32_t rend = row_end(r);
+
+  auto flush = [&]() {
+    if (r == ri0 && head_open) {
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) {
+        my_head_val[v] = acc[v];
+        if (kArg) my_head_arg[v] = arg[v];
+      }
+      if (lg == 0) { s_head_row[w] = r; s_head_closes[w] = 1; }
+    } else {
+      finalize_row<T, VEC, REDUCE>(a, out_b, arg_b, count_b, i0 + r, col, lg, acc, arg,
+                                   (int64_t)rend - (int64_t)s_ptr[r], col_ok);
+    }
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) acc[v] = acc_init<A, REDUCE>();
+    ++r;
+    rend = row_end(r);
+  };
+
+  const int64_t col_ld = col_ok ? col : 0;  // idle lanes re-read column 0
+  const T *src_col = src_b + col_ld;
+  for (int e = je0; e < je1; e += U) {
+    Vec<T, VEC> x[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int ee = e + u < je1 ? e + u : je1 - 1;
+      x[u] = load_vec_stream<T, VEC>(src_col + (j0 + ee) * a.K);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int ce = e + u;
+      if (ce < je1) {
+        while (ce >= rend) flush();
+        const int32_t ge = (int32_t)(j0 + ce);
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) reduce_step<A, REDUCE>(acc[v], arg[v], to_acc<T>(x[u].v[v]), ge);
+      }
+    }
+  }
+  while (r < ri1) flush();
+
+  // edges of a row whose end lies beyond this worker
+  if (has_work && (i0 + r < a.N)) {
+    const int32_t rs = s_ptr[r];
+    const int first = rs > je0 ? rs : je0;
+    if (je1 > first) {
+      if (r == ri0 && head_open) {
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) {
+          my_head_val[v] = acc[v];
+          if (kArg) my_head_arg[v] = arg[v];
+        }
+        if (lg == 0) { s_head_row[w] = r; s_head_closes[w] = 0; }
+      } else {
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) {
+          my_tail_val[v] = acc[v];
+          if (kArg) my_tail_arg[v] = arg[v];
+        }
+        if (lg == 0) s_tail_row[w] = r;
+      }
+    }
+  }
+  __syncthreads();
+
+  // ---- combine partials of rows that cross worker boundaries, in edge order
+  A *ws_val_blk = static_cast<A *>(a.ws_vals) + ((b * a.nblk + blockIdx.x) * 2) * a.K;
+  int32_t *ws_arg_blk = kArg ? a.ws_args + ((b * a.nblk + blockIdx.x) * 2) * a.K : nullptr;
+  int64_t *meta = a.ws_meta + (b * a.nblk + blockIdx.x) * 4;
+
+  auto absorb_head = [&](int ww) {
+    const A *hv = s_val + (size_t)ww * CW + lg * VEC;
+    const int32_t *ha = s_arg + (kArg ? (size_t)ww * CW + lg * VEC : 0);
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) {
+      if (kArg)
+        reduce_step<A, REDUCE>(acc[v], arg[v], hv[v], ha[v]);
+      else
+        acc[v] = acc[v] + hv[v];
+    }
+  };
+
+  if (s_tail_row[w] >= 0) {
+    // this worker opened a row: gather the heads of the workers after it
+    const int row = s_tail_row[w];
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) { acc[v] = my_tail_val[v]; if (kArg) arg[v] = my_tail_arg[v]; }
+    bool closed = false;
+    for (int ww = w + 1; ww < W && !closed; ++ww) {
+      if (s_head_row[ww] < 0) continue;  // worker without items (tile end)
+      absorb_head(ww);
+      closed = s_head_closes[ww] != 0;
+    }
+    if (closed) {
+      finalize_row<T, VEC, REDUCE>(a, out_b, arg_b, count_b, i0 + row, col, lg, acc, arg,
+                                   (int64_t)s_ptr[row + 1] - (int64_t)s_ptr[row], col_ok);
+    } else {
+      if (col_ok) {
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) {
+          ws_val_blk[a.K + col + v] = acc[v];
+          if (kArg) ws_arg_blk[a.K + col + v] = arg[v];
+        }
+      }
+      if (lg == 0 && blockIdx.y == 0) meta[2] = i0 + row;
+    }
+  }
+  if (w == 0) {
+    // the row that entered the tile from the previous one
+    if (s_head_row[0] >= 0) {
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) { acc[v] = my_head_val[v]; if (kArg) arg[v] = my_head_arg[v]; }
+      bool closed = s_head_closes[0] != 0;
+      for (int ww = 1; ww < W && !closed; ++ww) {
+        if (s_head_row[ww] < 0) continue;
+        absorb_head(ww);
+        closed = s_head_closes[ww] != 0;
+      }
+      if (col_ok) {
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) {
+          ws_val_blk[col + v] = acc[v];
+          if (kArg) ws_arg_blk[col + v] = arg[v];
+        }
+      }
+      if (lg == 0 && blockIdx.y == 0) { meta[0] = i0 + s_head_row[0]; meta[1] = closed ? 1 : 0; }
+    } else if (lg == 0 && blockIdx.y == 0) {
+      meta[0] = -1;
+      meta[1] = 0;
+    }
+  }
+  // tiles that leave no open row say so (exactly one worker can hold the open row)
+  if (tid == 0 && blockIdx.y == 0) {
+    bool open = false;
+    for (int ww = 0; ww < W; ++ww) {
+      if (s_tail_row[ww] < 0) continue;
+      bool closed = false;
+      for (int w2 = ww + 1; w2 < W && !closed; ++w2)
+        if (s_head_row[w2] >= 0) closed = s_head_closes[w2] != 0;
+      if (!closed) open = true;
+    }
+    if (!open) meta[2] = -1;
+  }
+}
+
+// Second kernel: rows that cross workgroup tiles. One worker per tile that
+// opened such a row walks the following tiles' head partials in order.
+template <typename T, int VEC, int REDUCE>
+__global__ __launch_bounds__(kBlock) void csr_reduce_fixup_kernel(CsrReduceArgs a) {
+  typedef typename Acc<T>::type A;
+  constexpr bool kArg = (REDUCE == TS_MIN || REDUCE == TS_MAX);
+  const int G = a.G;
+  const int W = kBlock / G;
+  const int w = threadIdx.x / G;
+  const int lg = threadIdx.x - w * G;
+  const int64_t col = (int64_t)blockIdx.y * (G * VEC) + (int64_t)lg * VEC;
+  const bool col_ok = col < a.K;
+  const int64_t b = blockIdx.z;
+  const int64_t t = (int64_t)blockIdx.x * W + w;
+  if (t >= a.nblk) return;
+  const int64_t *meta = a.ws_meta + (b * a.nblk) * 4;
+  const int64_t row = meta[t * 4 + 2];
+  if (row < 0) return;
+  const A *vals = static_cast<const A *>(a.ws_vals) + (b * a.nblk) * 2 * a.K;
+  const int32_t *args = kArg ? a.ws_args + (b * a.nblk) * 2 * a.K : nullptr;
+
+  A acc[VEC];
+  int32_t arg[VEC];
+  const int64_t c = col_ok ? col : 0;
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) {
+    acc[v] = vals[(t * 2 + 1) * a.K + c + v];
+    arg[v] = kArg ? args[(t * 2 + 1) * a.K + c + v] : 0;
+  }
+  for (int64_t tt = t + 1; tt < a.nblk; ++tt) {
+    if (meta[tt * 4 + 0] != row) break;  // cannot happen for a well-formed indptr
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) {
+      const A hv = vals[(tt * 2) * a.K + c + v];
+      if (kArg)
+        reduce_step<A, REDUCE>(acc[v], arg[v], hv, args[(tt * 2) * a.K + c + v]);
+      else
+        acc[v] = acc[v] + hv;
+    }
+    if (meta[tt * 4 + 1] != 0) break;
+  }
+  const int64_t *ptr = a.indptr + b * a.indptr_batch_stride;
+  T *out_b = static_cast<T *>(a.out) + b * a.N * a.K;
+  int64_t *arg_b = kArg ? a.arg_out + b * a.N * a.K : nullptr;
+  T *count_b = a.count_out ? static_cast<T *>(a.count_out) + b * a.N : nullptr;
+  finalize_row<T, VEC, REDUCE>(a, out_b, arg_b, count_b, row, col, lg, acc, arg,
+                               ptr[row + 1] - ptr[row], col_ok);
+}
+
+// ---- host side -----------------------------------------------------------
+
+struct CsrPlan {
+  int vec;       // elements per lane (16 bytes worth, or 1)
+  int G;         // lanes per worker
+  int BI;        // items per tile
+  int64_t nblk;  // tiles per batch
+  int ychunks;   // column chunks
+};
+
+inline CsrPlan csr_plan(int64_t N, int64_t E, int64_t K, int elem_bytes, bool aligned16) {
+  CsrPlan p;
+  const int full = kVecBytes / elem_bytes;
+  p.vec = (aligned16 && full > 1 && K % full == 0) ? full : 1;
+  const int64_t lanes = (K + p.vec - 1) / p.vec;
+  int G = 1;
+  while (G < lanes && G < kWave) G <<= 1;
+  p.G = G;
+  p.ychunks = (int)((K + (int64_t)G * p.vec - 1) / ((int64_t)G * p.vec));
+  const int64_t items = N + E;
+  p.BI = items >= (4 << 20) ? 2048 : (items >= (1 << 20) ? 1024 : 512);
+  p.nblk = (items + p.BI - 1) / p.BI;
+  if (p.nblk < 1) p.nblk = 1;
+  return p;
+}
+
+inline size_t csr_ws_bytes(const CsrPlan &p, int64_t B, int64_t K, int acc_bytes, bool with_arg,
+                           size_t *off_args, size_t *off_meta) {
+  auto up = [](size_t x) { return (x + 255) & ~(size_t)255; };
+  size_t vals = up((size_t)B * p.nblk * 2 * K * acc_bytes);
+  size_t args = with_arg ? up((size_t)B * p.nblk * 2 * K * 4) : 0;
+  size_t meta = up((size_t)B * p.nblk * 4 * 8);
+  if (off_args) *off_args = vals;
+  if (off_meta) *off_meta = vals + args;
+  return vals + args + meta;
+}
+
+template <typename T, int VEC, int REDUCE>
+int launch_csr_reduce_t(const CsrReduceArgs &a, const CsrPlan &p, int64_t B, hipStream_t stream) {
+  dim3 grid((unsigned)p.nblk, (unsigned)p.ychunks, (unsigned)B);
+  hipLaunchKernelGGL((csr_reduce_kernel<T, VEC, REDUCE>), grid, dim3(kBlock), 0, stream, a);
+  const int W = kBlock / p.G;
+  dim3 grid2((unsigned)((p.nblk + W - 1) / W), (unsigned)p.ychunks, (unsigned)B);
+  hipLaunchKernelGGL((csr_reduce_fixup_kernel<T, VEC, REDUCE>), grid2, dim3(kBlock), 0, stream, a);
+  return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
+}
+
+template <typename T, int VEC>
+int launch_csr_reduce_v(const CsrReduceArgs &a, const CsrPlan &p, int64_t B, int reduce,
+                        hipStream_t stream) {
+  switch (reduce) {
+  case TS_SUM: return launch_csr_reduce_t<T, VEC, TS_SUM>(a, p, B, stream);
+  case TS_MEAN: return launch_csr_reduce_t<T, VEC, TS_MEAN>(a, p, B, stream);
+  case TS_MIN: return launch_csr_reduce_t<T, VEC, TS_MIN>(a, p, B, stream);
+  case TS_MAX: return launch_csr_reduce_t<T, VEC, TS_MAX>(a, p, B, stream);
+  default: return TS_ERR_UNSUPPORTED;
+  }
+}
+
+// One entry per element type, each defined in its own translation unit.
+template <typename T> int launch_csr_reduce(const CsrReduceArgs &a, const CsrPlan &p, int64_t B,
+                                            int reduce, hipStream_t stream);
+
+#define TS_INSTANTIATE_CSR_REDUCE(T, FULLVEC)                                               \
+  template <> int launch_csr_reduce<T>(const CsrReduceArgs &a, const CsrPlan &p, int64_t B, \
+                                       int reduce, hipStream_t stream) {                    \
+    if (p.vec == FULLVEC) return launch_csr_reduce_v<T, FULLVEC>(a, p, B, reduce, stream);  \
+    return launch_csr_reduce_v<T, 1>(a, p, B, reduce, stream);                              \
+  }
+
+}  // namespace ts

@@ -1,0 +1,14 @@
+// Kernel instantiations for element type bf16_t.
+#include "csr_reduce.h"
+#include "csr_gather.h"
+#include "coo_gather.h"
+#include "scatter.h"
+#include "elementwise.h"
+
+namespace ts {
+TS_INSTANTIATE_CSR_REDUCE(bf16_t, 8)
+TS_INSTANTIATE_CSR_GATHER(bf16_t, 8)
+TS_INSTANTIATE_COO_GATHER(bf16_t, 8)
+TS_INSTANTIATE_SCATTER(bf16_t, 8)
+TS_INSTANTIATE_ELEMENTWISE(bf16_t)
+}  // namespace ts

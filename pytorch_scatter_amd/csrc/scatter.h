@@ -1,0 +1,441 @@
+// Scatter with an unsorted index: out[b, index[b,e,k], k] (op)= src[b,e,k].
+//
+// sum / mul update `out` in place with device-scope atomics in the element
+// type (the reference accumulates in scalar_t as well, csrc/cpu/scatter_cpu.cpp
+// :74-76): native add for f32 / f64 / i32 / i64, packed pair add for bf16 / f16
+// when the pair is 4-byte aligned, compare-and-swap on the containing word
+// otherwise.
+//
+// min / max of element types up to 32 bits run in ONE pass over src: value
+// and position are packed into a 64-bit key
+//     key = order(value) << 32 | (0xFFFFFFFE - e)
+// and reduced with a 64-bit unsigned atomic max into the int64 arg_out buffer
+// itself, so no extra memory is needed. A larger value wins; among equal
+// values the smaller e wins, which is the CPU rule (first index wins,
+// csrc/cpu/reducer.h:63-67) and makes the result independent of scheduling.
+// The low word 0xFFFFFFFF marks "initial / previous content": an entry has to
+// beat it strictly. A cheap read of the current key skips the atomic for the
+// vast majority of entries (a running maximum is improved only O(log n)
+// times). A last pass over [B, N, K] unpacks value and arg.
+// 64-bit element types use the reference's two-pass scheme with a
+// deterministic arg (atomic min over matching positions).
+#pragma once
+
+#include <limits>
+
+#include "device_utils.h"
+
+namespace ts {
+
+// ---------------------------------------------------------------- atomics
+template <typename T, typename F>
+__device__ __forceinline__ void atomic_rmw_word(T *addr, F fn) {
+  // read-modify-write of a 1/2/4-byte element through its 32-bit container
+  static_assert(sizeof(T) <= 4, "");
+  uintptr_t a = reinterpret_cast<uintptr_t>(addr);
+  uint32_t *word = reinterpret_cast<uint32_t *>(a & ~(uintptr_t)3);
+  const int shift = (int)(a & 3) * 8;
+  const uint32_t mask = (sizeof(T) == 4) ? 0xFFFFFFFFu : (((1u << (sizeof(T) * 8)) - 1u) << shift);
+  uint32_t old = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  while (true) {
+    uint32_t bits = (old & mask) >> shift;
+    T cur;
+    __builtin_memcpy(&cur, &bits, sizeof(T));
+    T nv = fn(cur);
+    uint32_t nbits = 0;
+    __builtin_memcpy(&nbits, &nv, sizeof(T));
+    uint32_t desired = (old & ~mask) | ((nbits << shift) & mask);
+    if (desired == old) return;
+    if (__hip_atomic_compare_exchange_strong(word, &old, desired, __ATOMIC_RELAXED, __ATOMIC_RELAXED,
+                                             __HIP_MEMORY_SCOPE_AGENT))
+      return;
+  }
+}
+template <typename T, typename F>
+__device__ __forceinline__ void atomic_rmw_dword(T *addr, F fn) {
+  static_assert(sizeof(T) == 8, "");
+  uint64_t *word = reinterpret_cast<uint64_t *>(addr);
+  uint64_t old = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  while (true) {
+    T cur;
+    __builtin_memcpy(&cur, &old, 8);
+    T nv = fn(cur);
+    uint64_t desired;
+    __builtin_memcpy(&desired, &nv, 8);
+    if (desired == old) return;
+    if (__hip_atomic_compare_exchange_strong(word, &old, desired, __ATOMIC_RELAXED, __ATOMIC_RELAXED,
+                                             __HIP_MEMORY_SCOPE_AGENT))
+      return;
+  }
+}
+template <typename T, typename F> __device__ __forceinline__ void atomic_rmw(T *addr, F fn) {
+  if constexpr (sizeof(T) == 8)
+    atomic_rmw_dword<T>(addr, fn);
+  else
+    atomic_rmw_word<T>(addr, fn);
+}
+
+// element arithmetic in the element type (16-bit floats: via float, one rounding)
+template <typename T> __device__ __forceinline__ T add_elem(T a, T b) { return (T)(a + b); }
+template <> __device__ __forceinline__ bf16_t add_elem<bf16_t>(bf16_t a, bf16_t b) {
+  return float_to_bf16(bf16_to_float(a) + bf16_to_float(b));
+}
+template <> __device__ __forceinline__ f16_t add_elem<f16_t>(f16_t a, f16_t b) {
+  return (f16_t)((float)a + (float)b);
+}
+template <typename T> __device__ __forceinline__ T mul_elem(T a, T b) { return (T)(a * b); }
+template <> __device__ __forceinline__ bf16_t mul_elem<bf16_t>(bf16_t a, bf16_t b) {
+  return float_to_bf16(bf16_to_float(a) * bf16_to_float(b));
+}
+template <> __device__ __forceinline__ f16_t mul_elem<f16_t>(f16_t a, f16_t b) {
+  return (f16_t)((float)a * (float)b);
+}
+
+template <typename T> __device__ __forceinline__ void atomic_add_elem(T *p, T v) {
+  atomic_rmw<T>(p, [v](T cur) { return add_elem<T>(cur, v); });
+}
+template <> __device__ __forceinline__ void atomic_add_elem<float>(float *p, float v) {
+  unsafeAtomicAdd(p, v);  // global_atomic_add_f32, no return value
+}
+template <> __device__ __forceinline__ void atomic_add_elem<double>(double *p, double v) {
+  unsafeAtomicAdd(p, v);  // global_atomic_add_f64
+}
+template <> __device__ __forceinline__ void atomic_add_elem<int32_t>(int32_t *p, int32_t v) {
+  __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+template <> __device__ __forceinline__ void atomic_add_elem<int64_t>(int64_t *p, int64_t v) {
+  __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// ------------------------------------------------ order-preserving 32-bit keys
+// order(v) is monotone in v; -0.0 is folded onto +0.0 so that the two compare
+// equal as they do under the reference's `<` / `>`.
+template <typename T> struct Key;
+template <> struct Key<float> {
+  __device__ static uint32_t enc(float v) {
+    uint32_t u = __float_as_uint(v);
+    if (u == 0x80000000u) u = 0;
+    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+  }
+  __device__ static float dec(uint32_t k) {
+    return __uint_as_float((k & 0x80000000u) ? (k & 0x7FFFFFFFu) : ~k);
+  }
+  __device__ static bool is_nan(float v) { return v != v; }
+  static constexpr bool kFloat = true;
+};
+template <> struct Key<bf16_t> {
+  __device__ static uint32_t enc(bf16_t v) { return Key<float>::enc(bf16_to_float(v)); }
+  __device__ static bf16_t dec(uint32_t k) { bf16_t r; r.x = (uint16_t)(__float_as_uint(Key<float>::dec(k)) >> 16); return r; }
+  __device__ static bool is_nan(bf16_t v) { return (v.x & 0x7FFF) > 0x7F80; }
+  static constexpr bool kFloat = true;
+};
+template <> struct Key<f16_t> {
+  __device__ static uint32_t enc(f16_t v) { return Key<float>::enc((float)v); }
+  __device__ static f16_t dec(uint32_t k) { return (f16_t)Key<float>::dec(k); }
+  __device__ static bool is_nan(f16_t v) { return v != v; }
+  static constexpr bool kFloat = true;
+};
+template <typename I> struct IntKey {
+  __device__ static uint32_t enc(I v) { return (uint32_t)(int32_t)v ^ 0x80000000u; }
+  __device__ static I dec(uint32_t k) { return (I)(int32_t)(k ^ 0x80000000u); }
+  __device__ static bool is_nan(I) { return false; }
+  static constexpr bool kFloat = false;
+};
+template <> struct Key<int32_t> : IntKey<int32_t> {};
+template <> struct Key<int16_t> : IntKey<int16_t> {};
+template <> struct Key<int8_t> : IntKey<int8_t> {};
+template <> struct Key<uint8_t> : IntKey<uint8_t> {};
+
+constexpr uint32_t kKeepLow = 0xFFFFFFFFu;  // low word of "initial / previous content"
+
+template <typename T, bool IS_MAX> __device__ __forceinline__ uint64_t pack_key(T v, uint32_t low) {
+  uint32_t k = Key<T>::enc(v);
+  if (!IS_MAX) k = ~k;
+  return ((uint64_t)k << 32) | low;
+}
+
+// ------------------------------------------------------------------ kernels
+struct ScatterArgs {
+  const void *src;
+  const int64_t *index;
+  void *out;
+  int64_t *arg_out;
+  int64_t B, E, K, N;
+  int64_t sb, se, sk;  // index strides
+  int out_given;
+  int precheck;        // read before the atomic: 0 none, 1 cached, 2 device-coherent, 3 streaming
+};
+
+// grid-stride over the [B*E, K/VEC] vectors of src
+template <typename T, int VEC, int REDUCE>
+__global__ __launch_bounds__(kBlock) void scatter_atomic_kernel(ScatterArgs a) {
+  const T *src = static_cast<const T *>(a.src);
+  T *out = static_cast<T *>(a.out);
+  const int64_t kv = a.K / VEC;
+  const int64_t nvec = a.B * a.E * kv;
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < nvec; i += (int64_t)gridDim.x * kBlock) {
+    const int64_t be = i / kv;
+    const int64_t k0 = (i - be * kv) * VEC;
+    const int64_t b = be / a.E;
+    const int64_t e = be - b * a.E;
+    const Vec<T, VEC> x = load_vec_stream<T, VEC>(src + i * VEC);
+    const int64_t ibase = b * a.sb + e * a.se + k0 * a.sk;
+    int64_t idx = a.index[ibase];
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) {
+      if (v > 0 && a.sk != 0) idx = a.index[ibase + v * a.sk];
+      if (idx < 0 || idx >= a.N) continue;
+      T *p = out + (b * a.N + idx) * a.K + k0 + v;
+      const T val = x.v[v];
+      if (REDUCE == TS_SUM)
+        atomic_add_elem<T>(p, val);
+      else
+        atomic_rmw<T>(p, [val](T cur) { return mul_elem<T>(cur, val); });
+    }
+  }
+}
+
+// packed-pair add for 16-bit floats: two neighbouring columns in one atomic
+template <typename T>
+__global__ __launch_bounds__(kBlock) void scatter_add_pk16_kernel(ScatterArgs a) {
+  // requires K even, sk == 0, out 4-byte aligned
+  const T *src = static_cast<const T *>(a.src);
+  T *out = static_cast<T *>(a.out);
+  const int64_t kv = a.K / 2;
+  const int64_t nvec = a.B * a.E * kv;
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < nvec; i += (int64_t)gridDim.x * kBlock) {
+    const int64_t be = i / kv;
+    const int64_t k0 = (i - be * kv) * 2;
+    const int64_t b = be / a.E;
+    const int64_t e = be - b * a.E;
+    const int64_t idx = a.index[b * a.sb + e * a.se];
+    if (idx < 0 || idx >= a.N) continue;
+    T *p = out + (b * a.N + idx) * a.K + k0;
+    if constexpr (sizeof(T) == 2 && __is_same(T, bf16_t)) {
+      typedef short v2s __attribute__((ext_vector_type(2)));
+      v2s val = *reinterpret_cast<const v2s *>(src + i * 2);
+      __builtin_amdgcn_global_atomic_fadd_v2bf16(reinterpret_cast<v2s *>(p), val);
+    } else {
+      typedef _Float16 v2h __attribute__((ext_vector_type(2)));
+      v2h val = *reinterpret_cast<const v2h *>(src + i * 2);
+      __builtin_amdgcn_global_atomic_fadd_v2f16(reinterpret_cast<v2h *>(p), val);
+    }
+  }
+}
+
+// ---- packed-key min/max -----------------------------------------------------
+template <typename T, bool IS_MAX>
+__global__ __launch_bounds__(kBlock) void scatter_key_init_kernel(ScatterArgs a) {
+  const int64_t n = a.B * a.N * a.K;
+  const T *out = static_cast<const T *>(a.out);
+  uint64_t *keys = reinterpret_cast<uint64_t *>(a.arg_out);
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlock) {
+    uint64_t k;
+    if (a.out_given) {
+      const T prev = out[i];
+      // a NaN already in out can never be beaten (comparisons with it are false)
+      k = Key<T>::is_nan(prev) ? ~(uint64_t)0 : pack_key<T, IS_MAX>(prev, kKeepLow);
+    } else {
+      k = pack_key<T, IS_MAX>(IS_MAX ? ElemLim<T>::lowest() : ElemLim<T>::max(), kKeepLow);
+    }
+    keys[i] = k;
+  }
+}
+
+template <typename T, int VEC, bool IS_MAX>
+__global__ __launch_bounds__(kBlock) void scatter_key_kernel(ScatterArgs a) {
+  const T *src = static_cast<const T *>(a.src);
+  uint64_t *keys = reinterpret_cast<uint64_t *>(a.arg_out);
+  const int64_t kv = a.K / VEC;
+  const int64_t nvec = a.B * a.E * kv;
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < nvec; i += (int64_t)gridDim.x * kBlock) {
+    const int64_t be = i / kv;
+    const int64_t k0 = (i - be * kv) * VEC;
+    const int64_t b = be / a.E;
+    const int64_t e = be - b * a.E;
+    const Vec<T, VEC> x = load_vec_stream<T, VEC>(src + i * VEC);
+    const int64_t ibase = b * a.sb + e * a.se + k0 * a.sk;
+    int64_t idx = a.index[ibase];
+    const uint32_t low = 0xFFFFFFFEu - (uint32_t)e;
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) {
+      if (v > 0 && a.sk != 0) idx = a.index[ibase + v * a.sk];
+      if (idx < 0 || idx >= a.N) continue;
+      const T val = x.v[v];
+      if (Key<T>::is_nan(val)) continue;  // NaN never wins (csrc/cpu/reducer.h:63-67)
+      const uint64_t key = pack_key<T, IS_MAX>(val, low);
+      uint64_t *p = keys + (b * a.N + idx) * a.K + k0 + v;
+      if (a.precheck == 1) {
+        if (key <= *reinterpret_cast<volatile uint64_t *>(p)) continue;
+      } else if (a.precheck == 2) {
+        if (key <= __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) continue;
+      } else if (a.precheck == 3) {
+        if (key <= __builtin_nontemporal_load(p)) continue;
+      }
+      __hip_atomic_fetch_max(p, key, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
+}
+
+template <typename T, bool IS_MAX>
+__global__ __launch_bounds__(kBlock) void scatter_key_final_kernel(ScatterArgs a) {
+  const int64_t n = a.B * a.N * a.K;
+  const T *src = static_cast<const T *>(a.src);
+  T *out = static_cast<T *>(a.out);
+  uint64_t *keys = reinterpret_cast<uint64_t *>(a.arg_out);
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlock) {
+    const uint64_t key = keys[i];
+    const uint32_t low = (uint32_t)key;
+    if (low == kKeepLow) {  // nothing beat the initial / previous content
+      if (!a.out_given) out[i] = zero_elem<T>();
+      a.arg_out[i] = a.E;
+    } else {
+      const int64_t e = (int64_t)(0xFFFFFFFEu - low);
+      uint32_t k = (uint32_t)(key >> 32);
+      if (!IS_MAX) k = ~k;
+      T val = Key<T>::dec(k);
+      if (Key<T>::kFloat && k == 0x80000000u) {
+        // a zero: fetch it from src to keep the sign bit of the winning entry
+        const int64_t bn = i / a.K;
+        const int64_t kk = i - bn * a.K;
+        const int64_t b = bn / a.N;
+        val = src[(b * a.E + e) * a.K + kk];
+      }
+      out[i] = val;
+      a.arg_out[i] = e;
+    }
+  }
+}
+
+// ---- two-pass min/max for 64-bit element types --------------------------------
+template <typename T, bool IS_MAX>
+__global__ __launch_bounds__(kBlock) void scatter_minmax_wide_kernel(ScatterArgs a) {
+  const T *src = static_cast<const T *>(a.src);
+  T *out = static_cast<T *>(a.out);
+  const int64_t n = a.B * a.E * a.K;
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlock) {
+    const int64_t be = i / a.K;
+    const int64_t k = i - be * a.K;
+    const int64_t b = be / a.E;
+    const int64_t e = be - b * a.E;
+    const int64_t idx = a.index[b * a.sb + e * a.se + k * a.sk];
+    if (idx < 0 || idx >= a.N) continue;
+    const T val = src[i];
+    atomic_rmw<T>(out + (b * a.N + idx) * a.K + k, [val](T cur) {
+      return IS_MAX ? (val > cur ? val : cur) : (val < cur ? val : cur);
+    });
+  }
+}
+template <typename T>
+__global__ __launch_bounds__(kBlock) void scatter_arg_wide_kernel(ScatterArgs a) {
+  const T *src = static_cast<const T *>(a.src);
+  const T *out = static_cast<const T *>(a.out);
+  const int64_t n = a.B * a.E * a.K;
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlock) {
+    const int64_t be = i / a.K;
+    const int64_t k = i - be * a.K;
+    const int64_t b = be / a.E;
+    const int64_t e = be - b * a.E;
+    const int64_t idx = a.index[b * a.sb + e * a.se + k * a.sk];
+    if (idx < 0 || idx >= a.N) continue;
+    const int64_t o = (b * a.N + idx) * a.K + k;
+    if (src[i] == out[o]) __hip_atomic_fetch_min(a.arg_out + o, e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+
+// ---- elementwise helpers --------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(kBlock) void fill_kernel(T *p, int64_t n, T value) {
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlock)
+    p[i] = value;
+}
+// out[out == init] = 0 (csrc/cuda/scatter_cuda.cu:126-127)
+template <typename T>
+__global__ __launch_bounds__(kBlock) void mask_init_kernel(T *p, int64_t n, T init) {
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlock)
+    if (p[i] == init) p[i] = (T)0;
+}
+
+inline unsigned grid_for(int64_t n, int per_thread = 1) {
+  int64_t blocks = (n + (int64_t)kBlock * per_thread - 1) / ((int64_t)kBlock * per_thread);
+  if (blocks < 1) blocks = 1;
+  const int64_t cap = 256 * 32;  // 256 CUs x 32 workgroups: enough to fill the chip, grid-stride beyond
+  return (unsigned)(blocks < cap ? blocks : cap);
+}
+
+// ---- host side --------------------------------------------------------------------
+template <typename T> struct IsWide { static constexpr bool value = sizeof(T) == 8; };
+
+template <typename T, int VEC>
+int launch_scatter_v(const ScatterArgs &a, int reduce, hipStream_t stream) {
+  T *out = static_cast<T *>(a.out);
+  const int64_t n_out = a.B * a.N * a.K;
+  const int64_t n_src = a.B * a.E * a.K;
+  const unsigned g_src = grid_for(n_src / VEC);
+  const unsigned g_out = grid_for(n_out);
+  if (reduce == TS_SUM || reduce == TS_MUL) {
+    if (!a.out_given)
+      hipLaunchKernelGGL(fill_kernel<T>, dim3(g_out), dim3(kBlock), 0, stream, out, n_out,
+                         small_const<T>(reduce == TS_MUL ? 1 : 0));
+    if (n_src > 0) {
+      if (reduce == TS_SUM) {
+        if constexpr (__is_same(T, bf16_t) || __is_same(T, f16_t)) {
+          if (a.K % 2 == 0 && a.sk == 0 && (reinterpret_cast<uintptr_t>(a.out) & 3) == 0 &&
+              (reinterpret_cast<uintptr_t>(a.src) & 3) == 0) {
+            hipLaunchKernelGGL(scatter_add_pk16_kernel<T>, dim3(grid_for(n_src / 2)), dim3(kBlock), 0,
+                               stream, a);
+            return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
+          }
+        }
+        hipLaunchKernelGGL((scatter_atomic_kernel<T, VEC, TS_SUM>), dim3(g_src), dim3(kBlock), 0, stream, a);
+      } else {
+        hipLaunchKernelGGL((scatter_atomic_kernel<T, VEC, TS_MUL>), dim3(g_src), dim3(kBlock), 0, stream, a);
+      }
+    }
+  } else if (reduce == TS_MIN || reduce == TS_MAX) {
+    const bool is_max = reduce == TS_MAX;
+    if constexpr (IsWide<T>::value) {
+      const T init = is_max ? std::numeric_limits<T>::lowest() : std::numeric_limits<T>::max();
+      if (!a.out_given)
+        hipLaunchKernelGGL(fill_kernel<T>, dim3(g_out), dim3(kBlock), 0, stream, out, n_out, init);
+      hipLaunchKernelGGL(fill_kernel<int64_t>, dim3(g_out), dim3(kBlock), 0, stream, a.arg_out, n_out, a.E);
+      if (n_src > 0) {
+        if (is_max)
+          hipLaunchKernelGGL((scatter_minmax_wide_kernel<T, true>), dim3(g_src), dim3(kBlock), 0, stream, a);
+        else
+          hipLaunchKernelGGL((scatter_minmax_wide_kernel<T, false>), dim3(g_src), dim3(kBlock), 0, stream, a);
+      }
+      if (!a.out_given)
+        hipLaunchKernelGGL(mask_init_kernel<T>, dim3(g_out), dim3(kBlock), 0, stream, out, n_out, init);
+      if (n_src > 0)
+        hipLaunchKernelGGL(scatter_arg_wide_kernel<T>, dim3(g_src), dim3(kBlock), 0, stream, a);
+    } else {
+      if (a.E >= 0xFFFFFFFEll) return TS_ERR_UNSUPPORTED;
+      if (is_max) {
+        hipLaunchKernelGGL((scatter_key_init_kernel<T, true>), dim3(g_out), dim3(kBlock), 0, stream, a);
+        if (n_src > 0)
+          hipLaunchKernelGGL((scatter_key_kernel<T, VEC, true>), dim3(g_src), dim3(kBlock), 0, stream, a);
+        hipLaunchKernelGGL((scatter_key_final_kernel<T, true>), dim3(g_out), dim3(kBlock), 0, stream, a);
+      } else {
+        hipLaunchKernelGGL((scatter_key_init_kernel<T, false>), dim3(g_out), dim3(kBlock), 0, stream, a);
+        if (n_src > 0)
+          hipLaunchKernelGGL((scatter_key_kernel<T, VEC, false>), dim3(g_src), dim3(kBlock), 0, stream, a);
+        hipLaunchKernelGGL((scatter_key_final_kernel<T, false>), dim3(g_out), dim3(kBlock), 0, stream, a);
+      }
+    }
+  } else {
+    return TS_ERR_UNSUPPORTED;
+  }
+  return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
+}
+
+// vec: elements per lane the caller found safe (alignment, K divisible)
+template <typename T> int launch_scatter(const ScatterArgs &a, int reduce, int vec, hipStream_t stream);
+
+#define TS_INSTANTIATE_SCATTER(T, FULLVEC)                                                       \
+  template <> int launch_scatter<T>(const ScatterArgs &a, int reduce, int vec, hipStream_t stream) { \
+    if (vec == FULLVEC) return launch_scatter_v<T, FULLVEC>(a, reduce, stream);                  \
+    return launch_scatter_v<T, 1>(a, reduce, stream);                                            \
+  }
+
+}  // namespace ts

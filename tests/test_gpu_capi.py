@@ -1,0 +1,397 @@
+"""Parity of the HIP kernels, called through the C ABI (libts_hip.so), against
+the CPU oracle on the same seeded inputs.
+
+Bars: bit-exact for min/max values, every arg index and every gather output;
+for sum/mean |got - want| <= rtol * |want| + atol with rtol = 1e-5 (fp32) /
+1e-2 (bf16, fp16), atol = rtol * max over rows of sum(|src|) (sums of N(0,1)
+values cancel towards zero, so a purely relative bound is ill-posed).
+"""
+from itertools import product
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import random_values
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+RTOL = {torch.float32: 1e-5, torch.float64: 1e-12, torch.bfloat16: 1e-2, torch.float16: 1e-2}
+
+
+@pytest.fixture(scope="module")
+def capi():
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    from pytorch_scatter_amd import capi
+    capi.lib()
+    return capi
+
+
+def _bits(t):
+    return t.view({1: torch.uint8, 2: torch.int16, 4: torch.int32, 8: torch.int64}[t.element_size()])
+
+
+def assert_exact(got, want, what=""):
+    got = got.cpu()
+    assert got.shape == want.shape, (what, got.shape, want.shape)
+    if got.dtype.is_floating_point:
+        # +0.0 / -0.0 carry different bits but are the same value under the reference's compares
+        same = (_bits(got) == _bits(want)) | ((got == 0) & (want == 0))
+        assert bool(same.all()), (what, int((~same).sum()))
+    else:
+        assert torch.equal(got, want), (what, int((got != want).sum()))
+
+
+def assert_close(got, want, scale, dtype, what=""):
+    got = got.cpu().double()
+    want = want.double()
+    rtol = RTOL[dtype]
+    err = (got - want).abs()
+    bound = rtol * want.abs() + rtol * scale
+    assert bool((err <= bound).all()), (what, float((err - bound).max()))
+
+
+def degrees(kind, rng, n):
+    if kind == "short":
+        d = rng.integers(0, 6, size=n)
+    elif kind == "zipf":
+        d = np.minimum(rng.zipf(1.8, size=n), 5000)
+        d[rng.random(n) < 0.1] = 0
+    elif kind == "hub":  # rows that span many tiles, next to empty rows at both ends
+        d = rng.integers(0, 4, size=n)
+        d[:3] = 0
+        d[-3:] = 0
+        d[n // 3] = 9000
+        d[n // 2] = 2049
+        d[n // 2 + 1] = 700
+    elif kind == "uniform":
+        d = np.full(n, 7)
+    else:
+        raise ValueError(kind)
+    return d.astype(np.int64)
+
+
+def make_csr(kind, seed, n):
+    rng = np.random.default_rng(seed)
+    deg = degrees(kind, rng, n)
+    indptr = np.zeros(n + 1, dtype=np.int64)
+    np.cumsum(deg, out=indptr[1:])
+    index = np.repeat(np.arange(n, dtype=np.int64), deg)
+    return rng, torch.from_numpy(indptr), torch.from_numpy(index)
+
+
+def values(rng, shape, dtype, reduce):
+    if reduce in ("min", "max") or not dtype.is_floating_point:
+        return random_values(rng, shape, dtype, ties=True)
+    return torch.from_numpy(rng.standard_normal(size=shape)).to(dtype)
+
+
+CSR_CASES = [
+    # kind, rows, K
+    ("short", 300, 1), ("short", 1000, 4), ("zipf", 2000, 16), ("zipf", 3000, 64),
+    ("hub", 900, 64), ("hub", 500, 128), ("uniform", 257, 3), ("zipf", 700, 200),
+    ("hub", 300, 520), ("short", 5, 8), ("hub", 40, 1),
+]
+
+
+@pytest.mark.parametrize("case,reduce,dtype", product(
+    CSR_CASES, ["sum", "mean", "min", "max"], [torch.float32, torch.bfloat16]))
+def test_segment_csr(capi, oracle, case, reduce, dtype):
+    kind, n, K = case
+    rng, indptr, index = make_csr(kind, CSR_CASES.index(case), n)
+    E = index.numel()
+    src = values(rng, (E, K), dtype, reduce)
+    want, want_arg = oracle.segment_csr(src, indptr, None, reduce)
+    out = torch.full((n, K), 7, dtype=dtype, device=DEV)
+    arg = torch.full((n, K), -1, dtype=torch.long, device=DEV) if reduce in ("min", "max") else None
+    capi.segment_csr(src.to(DEV), indptr.to(DEV), out, arg, 1, n, E, K, 0, capi.REDUCE[reduce])
+    torch.cuda.synchronize()
+    if reduce in ("min", "max"):
+        assert_exact(out, want, "values")
+        assert_exact(arg, want_arg, "arg")
+    else:
+        scale = float(oracle.segment_csr(src.abs().double(), indptr, None, "sum")[0].max()) if E else 0.0
+        assert_close(out, want, scale, dtype, "values")
+
+
+@pytest.mark.parametrize("dtype,reduce", product(
+    [torch.float16, torch.float64, torch.int32, torch.int64, torch.int16, torch.int8, torch.uint8],
+    ["sum", "mean", "min", "max"]))
+def test_segment_csr_other_dtypes(capi, oracle, dtype, reduce):
+    rng, indptr, index = make_csr("hub", 5, 400)
+    E = index.numel()
+    K = 24
+    src = random_values(rng, (E, K), dtype, ties=True)
+    if reduce in ("sum", "mean") and dtype in (torch.int8, torch.uint8, torch.int16, torch.float16):
+        src = src.clamp(-1, 1) if dtype != torch.uint8 else src.clamp(0, 1)
+    if dtype == torch.uint8 and reduce == "mean":
+        pytest.skip("8-bit counts wrap to 0 on long rows: undefined upstream")
+    if dtype == torch.uint8 and reduce == "max":
+        src = src + 1  # a row that never beats the initial value 0 keeps a stale arg upstream: unpinned
+    want, want_arg = oracle.segment_csr(src, indptr, None, reduce)
+    out = torch.zeros((400, K), dtype=dtype, device=DEV)
+    arg = torch.zeros((400, K), dtype=torch.long, device=DEV) if reduce in ("min", "max") else None
+    capi.segment_csr(src.to(DEV), indptr.to(DEV), out, arg, 1, 400, E, K, 0, capi.REDUCE[reduce])
+    torch.cuda.synchronize()
+    if reduce in ("min", "max") or not dtype.is_floating_point:
+        if dtype == torch.int8 and reduce == "mean":
+            pytest.skip("8-bit counts wrap on long rows: undefined upstream")
+        assert_exact(out, want, "values")
+        if arg is not None:
+            assert_exact(arg, want_arg, "arg")
+    else:
+        scale = float(oracle.segment_csr(src.abs().double(), indptr, None, "sum")[0].max())
+        assert_close(out, want, scale, dtype)
+
+
+@pytest.mark.parametrize("reduce", ["sum", "mean", "min", "max"])
+def test_segment_csr_batched(capi, oracle, reduce):
+    rng = np.random.default_rng(21)
+    B, n, K = 3, 50, 8
+    E = 400
+    ptrs = []
+    for _ in range(B):
+        deg = rng.multinomial(E, np.ones(n) / n)
+        ptrs.append(np.concatenate([[0], np.cumsum(deg)]))
+    indptr = torch.from_numpy(np.stack(ptrs).astype(np.int64))
+    src = values(rng, (B, E, K), torch.float32, reduce)
+    for ip, stride in ((indptr, n + 1), (indptr[:1], 0)):
+        want, want_arg = oracle.segment_csr(src, ip, None, reduce)
+        out = torch.empty((B, n, K), dtype=torch.float32, device=DEV)
+        arg = torch.empty((B, n, K), dtype=torch.long, device=DEV) if reduce in ("min", "max") else None
+        capi.segment_csr(src.to(DEV), ip.contiguous().to(DEV), out, arg, B, n, E, K, stride, capi.REDUCE[reduce])
+        torch.cuda.synchronize()
+        if reduce in ("min", "max"):
+            assert_exact(out, want)
+            assert_exact(arg, want_arg)
+        else:
+            assert_close(out, want, float(src.abs().sum(1).max()), torch.float32)
+
+
+@pytest.mark.parametrize("case,dtype", product(CSR_CASES, [torch.float32, torch.bfloat16, torch.int64, torch.uint8]))
+def test_gather_csr(capi, oracle, case, dtype):
+    kind, n, K = case
+    rng, indptr, index = make_csr(kind, CSR_CASES.index(case), n)
+    E = index.numel()
+    src = random_values(rng, (n, K), dtype, ties=False)
+    want = oracle.gather_csr(src, indptr)
+    out = torch.full((E, K), 3, dtype=dtype, device=DEV)
+    capi.gather_csr(src.to(DEV), indptr.to(DEV), out, 1, n, E, K, 0)
+    torch.cuda.synchronize()
+    assert_exact(out, want)
+
+
+@pytest.mark.parametrize("case,dtype", product(CSR_CASES[:8], [torch.float32, torch.bfloat16, torch.float64]))
+def test_segment_mean_csr_backward(capi, oracle, case, dtype):
+    kind, n, K = case
+    rng, indptr, index = make_csr(kind, CSR_CASES.index(case), n)
+    E = index.numel()
+    g = torch.from_numpy(rng.standard_normal(size=(n, K))).to(dtype)
+    want = oracle.segment_mean_csr_backward(g, indptr, (E, K))
+    out = torch.empty((E, K), dtype=dtype, device=DEV)
+    capi.segment_mean_csr_backward(g.to(DEV), indptr.to(DEV), out, 1, n, E, K, 0)
+    torch.cuda.synchronize()
+    assert_exact(out, want)  # one correctly rounded division per element: bit-exact
+
+
+@pytest.mark.parametrize("case,reduce,dtype", product(
+    CSR_CASES[:9], ["sum", "mean", "min", "max"], [torch.float32, torch.bfloat16]))
+def test_segment_coo(capi, oracle, case, reduce, dtype):
+    kind, n, K = case
+    rng, indptr, index = make_csr(kind, CSR_CASES.index(case), n)
+    E = index.numel()
+    src = values(rng, (E, K), dtype, reduce)
+    want, want2 = oracle.segment_coo(src, index, None, n, reduce)
+    out = torch.full((n, K), 7, dtype=dtype, device=DEV)
+    arg = torch.full((n, K), -1, dtype=torch.long, device=DEV) if reduce in ("min", "max") else None
+    cnt = torch.full((n,), -1, dtype=dtype, device=DEV) if reduce == "mean" else None
+    capi.segment_coo(src.to(DEV), index.to(DEV), out, arg, cnt, 1, n, E, K, 0, capi.REDUCE[reduce], False)
+    torch.cuda.synchronize()
+    if reduce in ("min", "max"):
+        assert_exact(out, want)
+        assert_exact(arg, want2)
+    else:
+        scale = float(oracle.segment_csr(src.abs().double(), indptr, None, "sum")[0].max()) if E else 0.0
+        assert_close(out, want, scale, dtype)
+        if reduce == "mean":
+            assert_exact(cnt, want2)
+
+
+@pytest.mark.parametrize("reduce,dtype", product(["sum", "mean", "min", "max"], [torch.float32, torch.bfloat16]))
+def test_segment_coo_out_given(capi, oracle, reduce, dtype):
+    kind, n, K = "hub", 500, 16
+    rng, indptr, index = make_csr(kind, 33, n)
+    E = index.numel()
+    src = values(rng, (E, K), dtype, reduce)
+    prev = random_values(rng, (n, K), dtype, ties=True)
+    prev[0] = 1  # the oracle seeds the first run from row 0: keep both readings equal
+    deg = indptr[1:] - indptr[:-1]
+    first = int(index[0])
+    prev[first] = prev[0]
+    want = prev.clone()
+    oracle.segment_coo(src, index, want, None, reduce)
+    out = prev.clone().to(DEV)
+    arg = torch.full((n, K), E, dtype=torch.long, device=DEV) if reduce in ("min", "max") else None
+    capi.segment_coo(src.to(DEV), index.to(DEV), out, arg, None, 1, n, E, K, 0, capi.REDUCE[reduce], True)
+    torch.cuda.synchronize()
+    if reduce in ("min", "max"):
+        assert_exact(out, want)
+        # arg: E where the previous content survived, else first position of the winner
+        a = arg.cpu()
+        kept = (out.cpu() == prev) & (a == E)
+        won = a < E
+        assert bool((kept | won).all())
+        picked = torch.gather(src, 0, a.clamp(max=E - 1))
+        assert torch.equal(picked[won], out.cpu()[won])
+    else:
+        scale = float(oracle.segment_csr(src.abs().double(), indptr, None, "sum")[0].max()) + float(prev.abs().max())
+        assert_close(out, want, scale, dtype)
+    # rows without entries keep their content
+    assert_exact(out[(deg == 0).to(DEV)], prev[deg == 0])
+
+
+@pytest.mark.parametrize("case,dtype", product(CSR_CASES[:9], [torch.float32, torch.bfloat16, torch.int32]))
+def test_gather_coo_and_mean_backward(capi, oracle, case, dtype):
+    kind, n, K = case
+    rng, indptr, index = make_csr(kind, CSR_CASES.index(case), n)
+    E = index.numel()
+    if E == 0:
+        pytest.skip("empty")
+    src = random_values(rng, (n, K), dtype, ties=False)
+    want = oracle.gather_coo(src, index)
+    out = torch.empty((E, K), dtype=dtype, device=DEV)
+    capi.gather_coo(src.to(DEV), index.to(DEV), out, 1, n, E, K, 0)
+    torch.cuda.synchronize()
+    assert_exact(out, want)
+    if dtype.is_floating_point:
+        count = (indptr[1:] - indptr[:-1]).clamp(min=1).to(dtype)
+        want = oracle.segment_mean_coo_backward(src, index, count, (E, K))
+        capi.segment_mean_coo_backward(src.to(DEV), index.to(DEV), count.to(DEV), out, 1, n, E, K, 0)
+        torch.cuda.synchronize()
+        assert_exact(out, want)
+
+
+SCATTER_SHAPES = [
+    # B, E, K, N
+    (1, 1000, 1, 37), (1, 5000, 16, 300), (1, 3000, 32, 10), (2, 700, 5, 50), (3, 400, 8, 1),
+    (1, 20000, 4, 2000), (1, 64, 130, 7),
+]
+
+
+@pytest.mark.parametrize("shape,reduce,dtype", product(
+    SCATTER_SHAPES, ["sum", "mul", "min", "max"], [torch.float32, torch.bfloat16, torch.int32]))
+def test_scatter(capi, oracle, shape, reduce, dtype):
+    B, E, K, N = shape
+    rng = np.random.default_rng(B * 1000 + E + K)
+    src = values(rng, (B, E, K), dtype, reduce)
+    if reduce == "mul":
+        src = random_values(rng, (B, E, K), dtype, ties=True).clamp(-1, 1)
+        if dtype.is_floating_point:
+            src = torch.where(src == 0, torch.ones_like(src), src)
+    index1 = torch.from_numpy(rng.integers(0, N, size=E))
+    for mode in ("broadcast", "full"):
+        if mode == "broadcast":
+            index = index1.view(1, E, 1).expand(B, E, K)
+            strides = (0, 1, 0)
+            dev_index = index1.to(DEV)
+        else:
+            index = torch.from_numpy(rng.integers(0, N, size=(B, E, K)))
+            strides = (E * K, K, 1)
+            dev_index = index.to(DEV)
+        want, want_arg = oracle.scatter(src, index, 1, None, N, reduce)
+        out = torch.full((B, N, K), 9, dtype=dtype, device=DEV)
+        arg = torch.full((B, N, K), -5, dtype=torch.long, device=DEV) if reduce in ("min", "max") else None
+        capi.scatter(src.to(DEV), dev_index, out, arg, B, E, K, N, *strides, capi.REDUCE[reduce], False)
+        torch.cuda.synchronize()
+        if reduce in ("min", "max") or not dtype.is_floating_point or reduce == "mul":
+            assert_exact(out, want, mode)
+            if arg is not None:
+                assert_exact(arg, want_arg, mode + " arg")
+        else:
+            absum = oracle.scatter(src.abs().double(), index, 1, None, N, "sum")[0]
+            if dtype == torch.float32:
+                assert_close(out, want, float(absum.max()), dtype, mode)
+            else:
+                # bf16 atomics round after every add, in arrival order: compare with the exact sum
+                exact = oracle.scatter(src.double(), index, 1, None, N, "sum")[0]
+                err = (out.cpu().double() - exact).abs()
+                cnt = oracle.scatter(torch.ones(B, E, K, dtype=torch.double), index, 1, None, N, "sum")[0]
+                assert bool((err <= 2.0 ** -8 * cnt * absum.clamp(min=1e-30) + 1e-30).all()), mode
+
+
+@pytest.mark.parametrize("reduce,dtype", product(["sum", "min", "max"], [torch.float32, torch.float64, torch.int64]))
+def test_scatter_out_given_and_wide_types(capi, oracle, reduce, dtype):
+    B, E, K, N = 2, 3000, 6, 40
+    rng = np.random.default_rng(77)
+    src = random_values(rng, (B, E, K), dtype, ties=True)
+    index = torch.from_numpy(rng.integers(0, N - 3, size=(B, E, K)))
+    prev = random_values(rng, (B, N, K), dtype, ties=True) * 0 + (6 if reduce == "min" else -6 if reduce == "max" else 1)
+    prev[:, :5] = 100 if reduce == "max" else -100 if reduce == "min" else 2  # previous content that survives
+    want = prev.clone()
+    _, want_arg = oracle.scatter(src, index, 1, want, None, reduce)
+    out = prev.clone().to(DEV)
+    arg = torch.full((B, N, K), -5, dtype=torch.long, device=DEV) if reduce != "sum" else None
+    capi.scatter(src.to(DEV), index.to(DEV), out, arg, B, E, K, N, E * K, K, 1, capi.REDUCE[reduce], True)
+    torch.cuda.synchronize()
+    assert_exact(out, want)
+    if arg is not None:
+        assert_exact(arg, want_arg)
+    # fresh output with the same inputs
+    want, want_arg = oracle.scatter(src, index, 1, None, N, reduce)
+    out = torch.empty((B, N, K), dtype=dtype, device=DEV)
+    capi.scatter(src.to(DEV), index.to(DEV), out, arg, B, E, K, N, E * K, K, 1, capi.REDUCE[reduce], False)
+    torch.cuda.synchronize()
+    assert_exact(out, want)
+    if arg is not None:
+        assert_exact(arg, want_arg)
+
+
+def test_scatter_mean_pieces(capi, oracle):
+    B, E, K, N = 2, 2000, 8, 64
+    rng = np.random.default_rng(5)
+    for dtype in (torch.float32, torch.int32):
+        src = random_values(rng, (B, E, K), dtype, ties=True)
+        index1 = torch.from_numpy(rng.integers(0, N - 2, size=E))
+        want = oracle.op_scatter(src, index1, 1, None, N, "mean")
+        out = torch.empty((B, N, K), dtype=dtype, device=DEV)
+        cnt = torch.empty((N,), dtype=torch.float32, device=DEV)
+        capi.scatter(src.to(DEV), index1.to(DEV), out, None, B, E, K, N, 0, 1, 0, capi.SUM, False)
+        capi.scatter_count(index1.to(DEV), cnt, 1, E, N, 0, 1)
+        for b in range(B):
+            capi.divide_by_count(out[b], cnt, 1, N, K)
+        torch.cuda.synchronize()
+        if dtype == torch.int32:
+            assert_exact(out, want)
+        else:
+            assert_close(out, want, 8.0 * E / N * 4, dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float64])
+def test_arg_backward(capi, oracle, dtype):
+    rng, indptr, index = make_csr("zipf", 3, 500)
+    E = index.numel()
+    K = 12
+    src = random_values(rng, (E, K), torch.float32, ties=True)
+    _, arg = oracle.segment_csr(src, indptr, None, "max")
+    g = torch.from_numpy(rng.standard_normal(size=(500, K))).to(dtype)
+    want = oracle.arg_backward(g, arg, (E, K), 0)
+    out = torch.full((E, K), 5, dtype=dtype, device=DEV)
+    capi.arg_backward(g.to(DEV), arg.to(DEV), out, 1, 500, E, K)
+    torch.cuda.synchronize()
+    assert_exact(out, want)
+
+
+def test_error_codes(capi):
+    x = torch.zeros(4, 4, device=DEV)
+    ptr = torch.tensor([0, 2, 4], device=DEV)
+    with pytest.raises(capi.TsError, match="workspace"):
+        with torch.cuda.device(0):
+            rc = capi.lib().ts_segment_csr(capi._p(x), capi._p(ptr), capi._p(x), None, capi._i(1), capi._i(2),
+                                           capi._i(4), capi._i(4), capi._i(0), 0, capi.SUM, None, 0, None)
+            capi._check(rc)
+    with pytest.raises(capi.TsError, match="unsupported"):
+        capi.segment_csr(x, ptr, x, None, 1, 2, 4, 4, 0, capi.MUL)
+    with pytest.raises(capi.TsError, match="device"):
+        capi.gather_csr(x.cpu(), ptr, x, 1, 2, 4, 4, 0)
