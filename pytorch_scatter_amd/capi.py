@@ -13,7 +13,7 @@ from typing import Optional
 import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libts_hip.so")
+LIB_PATH = os.environ.get("TS_HIP_LIB", os.path.join(_HERE, "libts_hip.so"))  # env: tuning aid
 
 SUM, MEAN, MUL, DIV, MIN, MAX = range(6)
 REDUCE = {"sum": SUM, "add": SUM, "mean": MEAN, "mul": MUL, "min": MIN, "max": MAX}

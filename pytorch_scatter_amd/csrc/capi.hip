@@ -100,6 +100,7 @@ int run_csr_reduce(const void *src, const int64_t *indptr, void *out, int64_t *a
   a.accumulate = accumulate;
   a.G = p.G;
   a.BI = p.BI;
+  a.ipw = p.ipw;
   a.nblk = p.nblk;
   a.ws_vals = ws;
   a.ws_args = reinterpret_cast<int32_t *>(static_cast<char *>(ws) + w.off_args);
@@ -160,6 +161,7 @@ int ts_gather_csr(const void *src, const int64_t *indptr, void *out, int64_t B, 
   a.indptr_batch_stride = indptr_batch_stride;
   a.G = p.G;
   a.BI = p.BI;
+  a.ipw = p.ipw;
   a.nblk = p.nblk;
   return dispatch_csr_gather(dtype, a, p, B, false, static_cast<hipStream_t>(stream));
 }
@@ -182,6 +184,7 @@ int ts_segment_mean_csr_backward(const void *grad_out, const int64_t *indptr, vo
   a.indptr_batch_stride = indptr_batch_stride;
   a.G = p.G;
   a.BI = p.BI;
+  a.ipw = p.ipw;
   a.nblk = p.nblk;
   return dispatch_csr_gather(dtype, a, p, B, true, static_cast<hipStream_t>(stream));
 }

@@ -20,7 +20,7 @@ struct CsrGatherArgs {
   void *out;           // [B, E, K]
   int64_t N, E, K;
   int64_t indptr_batch_stride;
-  int G, BI;
+  int G, BI, ipw;
   int64_t nblk;
 };
 
@@ -63,7 +63,7 @@ __global__ __launch_bounds__(kBlock) void csr_gather_kernel(CsrGatherArgs a) {
   for (int t = tid; t < nload; t += kBlock) s_ptr[t] = (int32_t)(ptr[i0 + t] - j0);
   __syncthreads();
 
-  const int ipw = a.BI / W;
+  const int ipw = a.ipw;
   const int tile_items = nr + ne;
   int dw0 = w * ipw;
   int dw1 = dw0 + ipw;

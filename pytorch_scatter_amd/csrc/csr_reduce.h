@@ -17,13 +17,18 @@
 // wins ties, mean = T(sum) / T(count), empty row -> 0 with arg = E.
 #pragma once
 
+#include <stdlib.h>
+
 #include "device_utils.h"
 #include "merge_path.h"
 
 namespace ts {
 
 constexpr int kMaxBlockItems = 2048;  // rows + edges per workgroup tile
-constexpr int kLoadsInFlight = 8;     // U: independent 16-byte loads per lane
+#ifndef TS_CSR_U
+#define TS_CSR_U 4
+#endif
+constexpr int kLoadsInFlight = TS_CSR_U;  // U: 16-byte loads per lane per batch (two batches in flight)
 
 struct CsrReduceArgs {
   const void *src;
@@ -35,7 +40,8 @@ struct CsrReduceArgs {
   int64_t indptr_batch_stride;
   int accumulate;     // combine with the previous content of out (segment_coo with out=)
   int G;              // lanes per worker
-  int BI;             // items per workgroup tile
+  int BI;             // items per workgroup tile (= workers * ipw)
+  int ipw;            // items per worker
   int64_t nblk;       // tiles per batch
   // workspace
   void *ws_vals;      // Acc [B][nblk][2][K]
@@ -152,7 +158,7 @@ __global__ __launch_bounds__(kBlock) void csr_reduce_kernel(CsrReduceArgs a) {
   __syncthreads();
 
   // ---- worker cut
-  const int ipw = a.BI / W;
+  const int ipw = a.ipw;
   const int tile_items = nr + ne;
   int dw0 = w * ipw;
   int dw1 = dw0 + ipw;
@@ -202,13 +208,20 @@ __global__ __launch_bounds__(kBlock) void csr_reduce_kernel(CsrReduceArgs a) {
 
   const int64_t col_ld = col_ok ? col : 0;  // idle lanes re-read column 0
   const T *src_col = src_b + col_ld;
-  for (int e = je0; e < je1; e += U) {
-    Vec<T, VEC> x[U];
+  // Software pipeline: the loads of batch i+1 are issued before batch i is
+  // reduced, so a wavefront always has U to 2U 16-byte loads outstanding.
+  auto load_batch = [&](Vec<T, VEC> *x, int e) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const int ee = e + u < je1 ? e + u : je1 - 1;
+      int ee = e + u < je1 ? e + u : je1 - 1;
       x[u] = load_vec_stream<T, VEC>(src_col + (j0 + ee) * a.K);
     }
+  };
+  Vec<T, VEC> x[U];
+  if (je0 < je1) load_batch(x, je0);
+  for (int e = je0; e < je1; e += U) {
+    Vec<T, VEC> y[U];
+    load_batch(y, e + U);  // unconditional (addresses are clamped): keeps the wait counts exact
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int ce = e + u;
@@ -219,6 +232,8 @@ __global__ __launch_bounds__(kBlock) void csr_reduce_kernel(CsrReduceArgs a) {
         for (int v = 0; v < VEC; ++v) reduce_step<A, REDUCE>(acc[v], arg[v], to_acc<T>(x[u].v[v]), ge);
       }
     }
+#pragma unroll
+    for (int u = 0; u < U; ++u) x[u] = y[u];
   }
   while (r < ri1) flush();
 
@@ -381,6 +396,7 @@ struct CsrPlan {
   int vec;       // elements per lane (16 bytes worth, or 1)
   int G;         // lanes per worker
   int BI;        // items per tile
+  int ipw;       // items per worker
   int64_t nblk;  // tiles per batch
   int ychunks;   // column chunks
 };
@@ -395,7 +411,19 @@ inline CsrPlan csr_plan(int64_t N, int64_t E, int64_t K, int elem_bytes, bool al
   p.G = G;
   p.ychunks = (int)((K + (int64_t)G * p.vec - 1) / ((int64_t)G * p.vec));
   const int64_t items = N + E;
-  p.BI = items >= (4 << 20) ? 2048 : (items >= (1 << 20) ? 1024 : 512);
+  // Items per worker: an odd multiple of 8. Workers of a tile start their
+  // streams ipw rows apart; a power-of-two distance puts all of them on the
+  // same HBM channels and costs ~15 % of the read bandwidth.
+  const int W = kBlock / G;
+  const int cap = kMaxBlockItems / W;  // LDS holds the row pointers of one tile
+  int want = items >= ((int64_t)8 << 20) ? 120 : (items >= ((int64_t)1 << 20) ? 56 : 24);
+  if (const char *env = getenv("TS_CSR_IPW")) want = atoi(env);  // tuning aid
+  if (want > cap) want = cap;
+  int ipw = want >= 8 ? (((want / 8) - 1) | 1) * 8 + 0 : (want | 1);
+  if (ipw > cap) ipw = cap;
+  if (ipw < 1) ipw = 1;
+  p.ipw = ipw;
+  p.BI = W * ipw;
   p.nblk = (items + p.BI - 1) / p.BI;
   if (p.nblk < 1) p.nblk = 1;
   return p;
