@@ -1,0 +1,692 @@
+// PyTorch host layer: registers the reference's operator names
+// (torch.ops.torch_scatter.*: csrc/scatter.cpp:272-277, segment_coo.cpp:240-246,
+// segment_csr.cpp:233-239, version.cpp:41-42) with the same inferred schemas
+// and the same forward/backward wiring, on top of the C ABI in ts_hip.h.
+//
+// PyTorch is used for what it owns: tensors, the caching allocator, the
+// current stream and the autograd graph. All arithmetic runs in libts_hip.so.
+// There is no CPU path: a CPU tensor is an error, not a fallback.
+#include <torch/script.h>
+
+#include <c10/core/DeviceGuard.h>
+#include <c10/hip/HIPStream.h>
+
+#include "../../include/ts_hip.h"
+
+namespace {
+
+using torch::Tensor;
+using OptTensor = std::optional<Tensor>;
+using OptInt = std::optional<int64_t>;
+using torch::autograd::AutogradContext;
+using torch::autograd::Variable;
+using torch::autograd::variable_list;
+
+// ------------------------------------------------------------------ helpers
+void check_input(bool cond) {
+  // the reference's CHECK_INPUT (csrc/cuda/utils.cuh:7)
+  TORCH_CHECK(cond, "Input mismatch");
+}
+
+void check_device(const Tensor &t, const char *name) {
+  // the reference's CHECK_CUDA (csrc/cuda/utils.cuh:5-6); HIP tensors carry the CUDA device type
+  TORCH_CHECK(t.device().is_cuda(), name,
+              " must be CUDA tensor (this build has HIP kernels only, no CPU path)");
+}
+
+int dtype_code(const Tensor &t) {
+  switch (t.scalar_type()) {
+  case at::kFloat: return TS_F32;
+  case at::kDouble: return TS_F64;
+  case at::kHalf: return TS_F16;
+  case at::kBFloat16: return TS_BF16;
+  case at::kInt: return TS_I32;
+  case at::kLong: return TS_I64;
+  case at::kShort: return TS_I16;
+  case at::kChar: return TS_I8;
+  case at::kByte: return TS_U8;
+  default: TORCH_CHECK(false, "torch_scatter: unsupported dtype ", t.scalar_type());
+  }
+}
+
+int reduce_code(const std::string &reduce) {
+  // same strings as the reference's reduce2REDUCE (csrc/cuda/reducer.cuh:10-13);
+  // an unknown string throws std::out_of_range there as well
+  static const std::map<std::string, int> table = {
+      {"sum", TS_SUM}, {"mean", TS_MEAN}, {"mul", TS_MUL}, {"div", TS_DIV}, {"min", TS_MIN}, {"max", TS_MAX}};
+  return table.at(reduce);
+}
+
+ts_stream_t stream_of(const Tensor &t) {
+  return static_cast<ts_stream_t>(c10::hip::getCurrentHIPStream(t.device().index()).stream());
+}
+
+void check_status(int status, const char *what) {
+  TORCH_CHECK(status == TS_OK, "torch_scatter (", what, "): ", ts_error_string(status));
+}
+
+int64_t prod(c10::IntArrayRef sizes, int64_t lo, int64_t hi) {
+  int64_t p = 1;
+  for (int64_t i = lo; i < hi; ++i) p *= sizes[i];
+  return p;
+}
+
+// Element stride that addresses dims [lo, hi) of `t` by their row-major linear
+// index, if one exists (contiguous within the group, or broadcast).
+std::optional<int64_t> collapsed_stride(const Tensor &t, int64_t lo, int64_t hi) {
+  int64_t expect = -1;  // stride the next more-significant non-unit dim must have
+  int64_t inner = 0;
+  bool have = false;
+  for (int64_t i = hi - 1; i >= lo; --i) {
+    if (t.size(i) == 1) continue;
+    if (!have) {
+      inner = t.stride(i);
+      have = true;
+    } else if (t.stride(i) != expect) {
+      return std::nullopt;
+    }
+    expect = t.stride(i) * t.size(i);
+  }
+  return have ? inner : 0;
+}
+
+Tensor workspace(size_t bytes, const Tensor &like) {
+  return at::empty({static_cast<int64_t>(bytes > 0 ? bytes : 1)}, like.options().dtype(at::kByte));
+}
+
+// csrc/scatter.cpp:25-33
+Tensor broadcast(Tensor src, const Tensor &other, int64_t dim) {
+  if (src.dim() == 1)
+    for (int64_t i = 0; i < dim; i++) src = src.unsqueeze(0);
+  for (int64_t i = src.dim(); i < other.dim(); i++) src = src.unsqueeze(-1);
+  return src.expand(other.sizes().vec());
+}
+
+// [B, I] view of an index / indptr tensor whose leading dims were expanded to
+// src's: unit inner stride and one batch stride (0 when shared), copying only
+// when the layout cannot be described that way.
+struct BatchedIndex {
+  Tensor t;
+  int64_t batch_stride;
+};
+BatchedIndex batched_index(const Tensor &idx) {
+  const int64_t d = idx.dim() - 1;
+  auto bs = collapsed_stride(idx, 0, d);
+  const bool inner_ok = idx.size(d) <= 1 || idx.stride(d) == 1;
+  if (bs.has_value() && inner_ok) return {idx, bs.value()};
+  Tensor c = idx.contiguous();
+  return {c, c.size(d)};
+}
+
+// ------------------------------------------------------------------ scatter
+// host half of scatter_cuda (csrc/cuda/scatter_cuda.cu:58-138)
+std::tuple<Tensor, OptTensor> scatter_hip(Tensor src, Tensor index, int64_t dim, OptTensor optional_out,
+                                          OptInt dim_size, int reduce) {
+  check_device(src, "src");
+  check_device(index, "index");
+  if (optional_out.has_value()) check_device(optional_out.value(), "out");
+  c10::DeviceGuard guard(src.device());
+
+  check_input(src.dim() == index.dim());
+  for (int64_t i = 0; i < index.dim() - 1; i++) check_input(src.size(i) >= index.size(i));
+  TORCH_CHECK(index.scalar_type() == at::kLong, "index must be int64");
+
+  src = src.contiguous();
+  Tensor out;
+  if (optional_out.has_value()) {
+    out = optional_out.value().contiguous();
+    for (int64_t i = 0; i < out.dim(); i++)
+      if (i != dim) check_input(src.size(i) == out.size(i));
+  } else {
+    auto sizes = src.sizes().vec();
+    if (dim_size.has_value())
+      sizes[dim] = dim_size.value();
+    else if (index.numel() == 0)
+      sizes[dim] = 0;
+    else
+      sizes[dim] = 1 + index.max().item<int64_t>();  // host sync, as upstream
+    out = at::empty(sizes, src.options());
+  }
+  const bool minmax = reduce == TS_MIN || reduce == TS_MAX;
+  OptTensor arg_out;
+  if (minmax) arg_out = at::empty(out.sizes(), index.options());
+
+  if (src.numel() == 0) {
+    if (!optional_out.has_value()) out.fill_(0);
+    if (minmax) arg_out.value().fill_(src.size(dim));
+    return std::make_tuple(out, arg_out);
+  }
+  // the op layer always hands over an index broadcast to src's shape
+  check_input(index.sizes() == src.sizes());
+
+  const int64_t B = prod(src.sizes(), 0, dim);
+  const int64_t E = src.size(dim);
+  const int64_t K = prod(src.sizes(), dim + 1, src.dim());
+  const int64_t N = out.size(dim);
+
+  auto sb = collapsed_stride(index, 0, dim);
+  auto sk = collapsed_stride(index, dim + 1, index.dim());
+  int64_t se = index.stride(dim);
+  if (!sb.has_value() || !sk.has_value()) {
+    index = index.contiguous();
+    sb = E * K;
+    se = K;
+    sk = 1;
+  }
+  check_status(ts_scatter(src.data_ptr(), index.data_ptr<int64_t>(), out.data_ptr(),
+                          minmax ? arg_out.value().data_ptr<int64_t>() : nullptr, B, E, K, N, sb.value(), se,
+                          sk.value(), dtype_code(src), reduce, optional_out.has_value() ? 1 : 0, stream_of(src)),
+               "scatter");
+  return std::make_tuple(out, arg_out);
+}
+
+// ---------------------------------------------------------------- segment_csr
+struct CsrShape {
+  Tensor indptr;
+  int64_t batch_stride, dim, B;
+};
+CsrShape expand_indptr(const Tensor &src, Tensor indptr) {
+  check_input(src.dim() >= indptr.dim());
+  TORCH_CHECK(indptr.scalar_type() == at::kLong, "indptr must be int64");
+  auto sizes = indptr.sizes().vec();
+  for (int64_t i = 0; i < indptr.dim() - 1; i++) sizes[i] = src.size(i);
+  indptr = indptr.expand(sizes);
+  CsrShape s;
+  s.dim = indptr.dim() - 1;
+  s.B = prod(indptr.sizes(), 0, s.dim);
+  auto bi = batched_index(indptr);
+  s.indptr = bi.t;
+  s.batch_stride = bi.batch_stride;
+  return s;
+}
+
+// host half of segment_csr_cuda (csrc/cuda/segment_csr_cuda.cu:97-168)
+std::tuple<Tensor, OptTensor> segment_csr_hip(Tensor src, Tensor indptr, OptTensor optional_out, int reduce) {
+  check_device(src, "src");
+  check_device(indptr, "indptr");
+  if (optional_out.has_value()) check_device(optional_out.value(), "out");
+  c10::DeviceGuard guard(src.device());
+
+  CsrShape cs = expand_indptr(src, indptr);
+  const int64_t dim = cs.dim;
+  src = src.contiguous();
+
+  Tensor out;
+  if (optional_out.has_value()) {
+    out = optional_out.value().contiguous();
+    for (int64_t i = 0; i < out.dim(); i++)
+      if (i != dim) check_input(src.size(i) == out.size(i));
+    check_input(src.numel() == 0 || out.size(dim) == cs.indptr.size(dim) - 1);
+  } else {
+    auto sizes = src.sizes().vec();
+    sizes[dim] = std::max<int64_t>(cs.indptr.size(dim) - 1, 0);
+    out = at::empty(sizes, src.options());
+  }
+  const bool minmax = reduce == TS_MIN || reduce == TS_MAX;
+  OptTensor arg_out;
+  if (minmax) arg_out = at::empty(out.sizes(), cs.indptr.options());
+
+  if (src.numel() == 0) {
+    if (!optional_out.has_value()) out.fill_(0);
+    if (minmax) arg_out.value().fill_(src.size(dim));
+    return std::make_tuple(out, arg_out);
+  }
+  const int64_t N = out.size(dim);
+  const int64_t E = src.size(dim);
+  const int64_t K = (cs.B * N) > 0 ? out.numel() / (cs.B * N) : 0;
+  const size_t ws_bytes = ts_segment_csr_workspace_bytes(cs.B, N, E, K, dtype_code(src), reduce);
+  Tensor ws = workspace(ws_bytes, src);
+  check_status(ts_segment_csr(src.data_ptr(), cs.indptr.data_ptr<int64_t>(), out.data_ptr(),
+                              minmax ? arg_out.value().data_ptr<int64_t>() : nullptr, cs.B, N, E, K,
+                              cs.batch_stride, dtype_code(src), reduce, ws.data_ptr(), ws_bytes, stream_of(src)),
+               "segment_csr");
+  return std::make_tuple(out, arg_out);
+}
+
+// host half of gather_csr_cuda (csrc/cuda/segment_csr_cuda.cu:219-281);
+// `mean_backward` selects the fused gather-and-divide
+Tensor gather_csr_hip(Tensor src, Tensor indptr, OptTensor optional_out, bool mean_backward = false) {
+  check_device(src, "src");
+  check_device(indptr, "indptr");
+  if (optional_out.has_value()) check_device(optional_out.value(), "out");
+  c10::DeviceGuard guard(src.device());
+
+  CsrShape cs = expand_indptr(src, indptr);
+  const int64_t dim = cs.dim;
+  check_input(src.size(dim) == 0 || src.size(dim) == cs.indptr.size(dim) - 1);
+  src = src.contiguous();
+
+  Tensor out;
+  if (optional_out.has_value()) {
+    out = optional_out.value().contiguous();
+    for (int64_t i = 0; i < out.dim(); i++)
+      if (i != dim) check_input(src.size(i) == out.size(i));
+  } else {
+    auto sizes = src.sizes().vec();
+    sizes[dim] = src.numel() > 0 ? cs.indptr.flatten()[-1].item<int64_t>() : 0;  // host sync, as upstream
+    out = at::empty(sizes, src.options());
+  }
+  if (src.numel() == 0) {
+    if (!optional_out.has_value()) out.fill_(0);
+    return out;
+  }
+  const int64_t N = src.size(dim);
+  const int64_t E = out.size(dim);
+  const int64_t K = src.numel() / (cs.B * N);
+  if (mean_backward)
+    check_status(ts_segment_mean_csr_backward(src.data_ptr(), cs.indptr.data_ptr<int64_t>(), out.data_ptr(), cs.B, N,
+                                              E, K, cs.batch_stride, dtype_code(src), stream_of(src)),
+                 "segment_mean_csr backward");
+  else
+    check_status(ts_gather_csr(src.data_ptr(), cs.indptr.data_ptr<int64_t>(), out.data_ptr(), cs.B, N, E, K,
+                               cs.batch_stride, dtype_code(src), stream_of(src)),
+                 "gather_csr");
+  return out;
+}
+
+// ---------------------------------------------------------------- segment_coo
+struct CooShape {
+  Tensor index;
+  int64_t batch_stride, dim, B;
+};
+CooShape expand_index(const Tensor &src, Tensor index, bool expand) {
+  check_input(src.dim() >= index.dim());
+  TORCH_CHECK(index.scalar_type() == at::kLong, "index must be int64");
+  if (expand) {
+    auto sizes = index.sizes().vec();
+    for (int64_t i = 0; i < index.dim(); i++) sizes[i] = src.size(i);
+    index = index.expand(sizes);
+  }
+  CooShape s;
+  s.dim = index.dim() - 1;
+  s.B = prod(index.sizes(), 0, s.dim);
+  auto bi = batched_index(index);
+  s.index = bi.t;
+  s.batch_stride = bi.batch_stride;
+  return s;
+}
+
+// host half of segment_coo_cuda (csrc/cuda/segment_coo_cuda.cu:152-283).
+// Second result: arg_out (min/max), count (mean), nothing (sum).
+std::tuple<Tensor, OptTensor> segment_coo_hip(Tensor src, Tensor index, OptTensor optional_out, OptInt dim_size,
+                                              int reduce) {
+  check_device(src, "src");
+  check_device(index, "index");
+  if (optional_out.has_value()) check_device(optional_out.value(), "out");
+  c10::DeviceGuard guard(src.device());
+
+  CooShape cs = expand_index(src, index, true);
+  const int64_t dim = cs.dim;
+  src = src.contiguous();
+
+  Tensor out;
+  if (optional_out.has_value()) {
+    out = optional_out.value().contiguous();
+    for (int64_t i = 0; i < out.dim(); i++)
+      if (i != dim) check_input(src.size(i) == out.size(i));
+  } else {
+    auto sizes = src.sizes().vec();
+    if (dim_size.has_value())
+      sizes[dim] = dim_size.value();
+    else if (cs.index.numel() == 0)
+      sizes[dim] = 0;
+    else {
+      auto tmp = cs.index.select(dim, cs.index.size(dim) - 1);
+      tmp = tmp.numel() > 1 ? tmp.max() : tmp;
+      sizes[dim] = 1 + tmp.item<int64_t>();  // host sync, as upstream
+    }
+    out = at::empty(sizes, src.options());
+  }
+  const bool minmax = reduce == TS_MIN || reduce == TS_MAX;
+  OptTensor second;
+  if (minmax) {
+    // with `out` given the kernel only touches rows that have entries
+    second = optional_out.has_value() ? at::full(out.sizes(), src.size(dim), cs.index.options())
+                                      : at::empty(out.sizes(), cs.index.options());
+  } else if (reduce == TS_MEAN) {
+    auto sizes = cs.index.sizes().vec();
+    sizes[dim] = out.size(dim);
+    second = optional_out.has_value() ? at::ones(sizes, out.options()) : at::empty(sizes, out.options());
+  }
+  if (src.numel() == 0 || cs.index.numel() == 0) {
+    if (!optional_out.has_value()) out.fill_(0);
+    if (minmax) second.value().fill_(src.size(dim));
+    if (reduce == TS_MEAN) second.value().fill_(1);
+    return std::make_tuple(out, second);
+  }
+  const int64_t E = src.size(dim);
+  const int64_t N = out.size(dim);
+  const int64_t K = src.numel() / (cs.B * E);
+  const size_t ws_bytes = ts_segment_coo_workspace_bytes(cs.B, N, E, K, dtype_code(src), reduce);
+  Tensor ws = workspace(ws_bytes, src);
+  check_status(ts_segment_coo(src.data_ptr(), cs.index.data_ptr<int64_t>(), out.data_ptr(),
+                              minmax ? second.value().data_ptr() : nullptr,
+                              reduce == TS_MEAN ? second.value().data_ptr() : nullptr, cs.B, N, E, K,
+                              cs.batch_stride, dtype_code(src), reduce, optional_out.has_value() ? 1 : 0,
+                              ws.data_ptr(), ws_bytes, stream_of(src)),
+               "segment_coo");
+  return std::make_tuple(out, second);
+}
+
+// host half of gather_coo_cuda (csrc/cuda/segment_coo_cuda.cu:327-382);
+// with `count` given: the fused backward of segment_coo(mean)
+Tensor gather_coo_hip(Tensor src, Tensor index, OptTensor optional_out, OptTensor count = std::nullopt) {
+  check_device(src, "src");
+  check_device(index, "index");
+  if (optional_out.has_value()) check_device(optional_out.value(), "out");
+  c10::DeviceGuard guard(src.device());
+
+  check_input(src.dim() >= index.dim());
+  auto sizes = index.sizes().vec();
+  for (int64_t i = 0; i < index.dim() - 1; i++) sizes[i] = src.size(i);
+  index = index.expand(sizes);
+  CooShape cs = expand_index(src, index, false);
+  const int64_t dim = cs.dim;
+  src = src.contiguous();
+
+  Tensor out;
+  if (optional_out.has_value()) {
+    out = optional_out.value().contiguous();
+    for (int64_t i = 0; i < src.dim(); i++)
+      if (i != dim) check_input(src.size(i) == out.size(i));
+    check_input(cs.index.size(dim) == out.size(dim));
+  } else {
+    auto osizes = src.sizes().vec();
+    osizes[dim] = cs.index.size(dim);
+    out = at::empty(osizes, src.options());
+  }
+  if (src.numel() == 0 || out.numel() == 0) {
+    if (!optional_out.has_value()) out.fill_(0);
+    return out;
+  }
+  const int64_t E = cs.index.size(dim);
+  const int64_t N = src.size(dim);
+  const int64_t K = out.numel() / (cs.B * E);
+  if (count.has_value()) {
+    Tensor c = count.value().contiguous();
+    check_status(ts_segment_mean_coo_backward(src.data_ptr(), cs.index.data_ptr<int64_t>(), c.data_ptr(),
+                                              out.data_ptr(), cs.B, N, E, K, cs.batch_stride, dtype_code(src),
+                                              stream_of(src)),
+                 "segment_mean_coo backward");
+  } else {
+    check_status(ts_gather_coo(src.data_ptr(), cs.index.data_ptr<int64_t>(), out.data_ptr(), cs.B, N, E, K,
+                               cs.batch_stride, dtype_code(src), stream_of(src)),
+                 "gather_coo");
+  }
+  return out;
+}
+
+// Backward of every min/max flavour: the gradient of each output slot goes to
+// the position that won it (csrc/scatter.cpp:184-196, segment_coo.cpp:132-144,
+// segment_csr.cpp:130-142 do this with a scatter_ into a buffer that has one
+// extra slot for the sentinel).
+Tensor arg_backward_hip(Tensor grad_out, const Tensor &arg_out, const std::vector<int64_t> &src_shape, int64_t dim) {
+  c10::DeviceGuard guard(grad_out.device());
+  grad_out = grad_out.contiguous();
+  Tensor arg = arg_out.contiguous();
+  Tensor grad_in = at::empty(src_shape, grad_out.options());
+  const int64_t B = prod(src_shape, 0, dim);
+  const int64_t E = src_shape[dim];
+  const int64_t K = prod(src_shape, dim + 1, static_cast<int64_t>(src_shape.size()));
+  const int64_t N = grad_out.size(dim);
+  check_status(ts_arg_backward(grad_out.data_ptr(), arg.data_ptr<int64_t>(), grad_in.data_ptr(), B, N, E, K,
+                               dtype_code(grad_out), stream_of(grad_out)),
+               "min/max backward");
+  return grad_in;
+}
+
+std::vector<int64_t> saved_shape(AutogradContext *ctx) {
+  return ctx->saved_data["src_shape"].toIntVector();
+}
+
+// ------------------------------------------------------- autograd: scatter
+// one Function per reduction, wired as ScatterSum/Mul/Mean/Min/Max in csrc/scatter.cpp:54-233
+template <int REDUCE> struct ScatterFn : public torch::autograd::Function<ScatterFn<REDUCE>> {
+  static variable_list forward(AutogradContext *ctx, Variable src, Variable index, int64_t dim,
+                               std::optional<Variable> optional_out, OptInt dim_size) {
+    dim = dim < 0 ? src.dim() + dim : dim;
+    ctx->saved_data["dim"] = dim;
+    ctx->saved_data["src_shape"] = src.sizes();
+    Variable old_index = index;
+    index = broadcast(index, src, dim);
+    auto result = scatter_hip(src, index, dim, optional_out, dim_size, REDUCE == TS_MEAN ? TS_SUM : REDUCE);
+    Variable out = std::get<0>(result);
+    if (optional_out.has_value()) ctx->mark_dirty({optional_out.value()});
+    if (REDUCE == TS_SUM) {
+      ctx->save_for_backward({index});
+      return {out};
+    }
+    if (REDUCE == TS_MUL) {
+      ctx->save_for_backward({src, index, out});
+      return {out};
+    }
+    if (REDUCE == TS_MEAN) {
+      // count over the index as given (csrc/scatter.cpp:131-141)
+      auto ones = at::ones(old_index.sizes(), src.options());
+      const int64_t cdim = old_index.dim() <= dim ? old_index.dim() - 1 : dim;
+      Variable count = std::get<0>(scatter_hip(ones, old_index, cdim, std::nullopt, out.size(dim), TS_SUM));
+      count.masked_fill_(count < 1, 1);
+      count = broadcast(count, out, dim);
+      if (out.is_floating_point())
+        out.true_divide_(count);
+      else
+        out.div_(count, "floor");
+      ctx->save_for_backward({index, count});
+      return {out};
+    }
+    Variable arg_out = std::get<1>(result).value();
+    ctx->save_for_backward({index, arg_out});
+    ctx->mark_non_differentiable({arg_out});
+    return {out, arg_out};
+  }
+
+  static variable_list backward(AutogradContext *ctx, variable_list grad_outs) {
+    auto grad_out = grad_outs[0];
+    auto saved = ctx->get_saved_variables();
+    const int64_t dim = ctx->saved_data["dim"].toInt();
+    Variable grad_in;
+    if (REDUCE == TS_SUM) {
+      grad_in = at::gather(grad_out, dim, saved[0], false);
+    } else if (REDUCE == TS_MUL) {
+      grad_in = at::gather(grad_out * saved[2], dim, saved[1], false).div_(saved[0]);
+      grad_in.masked_fill_(grad_in.isnan(), 0);
+    } else if (REDUCE == TS_MEAN) {
+      auto count = at::gather(saved[1], dim, saved[0], false);
+      grad_in = at::gather(grad_out, dim, saved[0], false);
+      grad_in.true_divide_(count);
+    } else {
+      grad_in = arg_backward_hip(grad_out, saved[1], saved_shape(ctx), dim);
+    }
+    return {grad_in, Variable(), Variable(), Variable(), Variable()};
+  }
+};
+
+// --------------------------------------------------- autograd: segment_csr
+// SegmentSum/Mean/Min/MaxCSR, csrc/segment_csr.cpp:57-174
+template <int REDUCE> struct SegmentCsrFn : public torch::autograd::Function<SegmentCsrFn<REDUCE>> {
+  static variable_list forward(AutogradContext *ctx, Variable src, Variable indptr,
+                               std::optional<Variable> optional_out) {
+    ctx->saved_data["src_shape"] = src.sizes();
+    auto result = segment_csr_hip(src, indptr, optional_out, REDUCE);
+    Variable out = std::get<0>(result);
+    if (optional_out.has_value()) ctx->mark_dirty({optional_out.value()});
+    if (REDUCE == TS_MIN || REDUCE == TS_MAX) {
+      Variable arg_out = std::get<1>(result).value();
+      ctx->save_for_backward({indptr, arg_out});
+      ctx->mark_non_differentiable({arg_out});
+      return {out, arg_out};
+    }
+    ctx->save_for_backward({indptr});
+    return {out};
+  }
+
+  static variable_list backward(AutogradContext *ctx, variable_list grad_outs) {
+    auto grad_out = grad_outs[0];
+    auto saved = ctx->get_saved_variables();
+    auto indptr = saved[0];
+    auto src_shape = saved_shape(ctx);
+    Variable grad_in;
+    if (REDUCE == TS_MIN || REDUCE == TS_MAX) {
+      grad_in = arg_backward_hip(grad_out, saved[1], src_shape, indptr.dim() - 1);
+    } else {
+      grad_in = at::empty(src_shape, grad_out.options());
+      // mean: one fused gather-and-divide instead of upstream's two gathers
+      // and a division (csrc/segment_csr.cpp:100-109)
+      if (grad_in.numel() > 0) gather_csr_hip(grad_out, indptr, grad_in, REDUCE == TS_MEAN);
+    }
+    return {grad_in, Variable(), Variable()};
+  }
+};
+
+// GatherCSR, csrc/segment_csr.cpp:176-199
+struct GatherCsrFn : public torch::autograd::Function<GatherCsrFn> {
+  static variable_list forward(AutogradContext *ctx, Variable src, Variable indptr,
+                               std::optional<Variable> optional_out) {
+    ctx->saved_data["src_shape"] = src.sizes();
+    Variable out = gather_csr_hip(src, indptr, optional_out);
+    ctx->save_for_backward({indptr});
+    if (optional_out.has_value()) ctx->mark_dirty({optional_out.value()});
+    return {out};
+  }
+  static variable_list backward(AutogradContext *ctx, variable_list grad_outs) {
+    auto grad_out = grad_outs[0];
+    auto indptr = ctx->get_saved_variables()[0];
+    Variable grad_in = at::empty(saved_shape(ctx), grad_out.options());
+    segment_csr_hip(grad_out, indptr, grad_in, TS_SUM);
+    return {grad_in, Variable(), Variable()};
+  }
+};
+
+// --------------------------------------------------- autograd: segment_coo
+// SegmentSum/Mean/Min/MaxCOO, csrc/segment_coo.cpp:57-177
+template <int REDUCE> struct SegmentCooFn : public torch::autograd::Function<SegmentCooFn<REDUCE>> {
+  static variable_list forward(AutogradContext *ctx, Variable src, Variable index,
+                               std::optional<Variable> optional_out, OptInt dim_size) {
+    ctx->saved_data["src_shape"] = src.sizes();
+    auto result = segment_coo_hip(src, index, optional_out, dim_size, REDUCE);
+    Variable out = std::get<0>(result);
+    if (optional_out.has_value()) ctx->mark_dirty({optional_out.value()});
+    if (REDUCE == TS_SUM) {
+      ctx->save_for_backward({index});
+      return {out};
+    }
+    Variable second = std::get<1>(result).value();
+    ctx->save_for_backward({index, second});
+    if (REDUCE == TS_MEAN) return {out};
+    ctx->mark_non_differentiable({second});
+    return {out, second};
+  }
+
+  static variable_list backward(AutogradContext *ctx, variable_list grad_outs) {
+    auto grad_out = grad_outs[0];
+    auto saved = ctx->get_saved_variables();
+    auto index = saved[0];
+    auto src_shape = saved_shape(ctx);
+    Variable grad_in;
+    if (REDUCE == TS_MIN || REDUCE == TS_MAX) {
+      grad_in = arg_backward_hip(grad_out, saved[1], src_shape, index.dim() - 1);
+    } else {
+      grad_in = at::empty(src_shape, grad_out.options());
+      if (grad_in.numel() > 0) {
+        if (REDUCE == TS_MEAN)
+          gather_coo_hip(grad_out, index, grad_in, saved[1]);  // fused gather / count
+        else
+          gather_coo_hip(grad_out, index, grad_in);
+      }
+    }
+    return {grad_in, Variable(), Variable(), Variable()};
+  }
+};
+
+// GatherCOO, csrc/segment_coo.cpp:179-202
+struct GatherCooFn : public torch::autograd::Function<GatherCooFn> {
+  static variable_list forward(AutogradContext *ctx, Variable src, Variable index,
+                               std::optional<Variable> optional_out) {
+    ctx->saved_data["src_shape"] = src.sizes();
+    Variable out = gather_coo_hip(src, index, optional_out);
+    ctx->save_for_backward({index});
+    if (optional_out.has_value()) ctx->mark_dirty({optional_out.value()});
+    return {out};
+  }
+  static variable_list backward(AutogradContext *ctx, variable_list grad_outs) {
+    auto grad_out = grad_outs[0];
+    auto index = ctx->get_saved_variables()[0];
+    auto src_shape = saved_shape(ctx);
+    Variable grad_in = at::zeros(src_shape, grad_out.options());
+    if (grad_out.numel() > 0) segment_coo_hip(grad_out, index, grad_in, std::nullopt, TS_SUM);
+    return {grad_in, Variable(), Variable()};
+  }
+};
+
+// ------------------------------------------------------- registered functions
+Tensor scatter_sum(Tensor src, Tensor index, int64_t dim, OptTensor out, OptInt dim_size) {
+  return ScatterFn<TS_SUM>::apply(src, index, dim, out, dim_size)[0];
+}
+Tensor scatter_mul(Tensor src, Tensor index, int64_t dim, OptTensor out, OptInt dim_size) {
+  return ScatterFn<TS_MUL>::apply(src, index, dim, out, dim_size)[0];
+}
+Tensor scatter_mean(Tensor src, Tensor index, int64_t dim, OptTensor out, OptInt dim_size) {
+  return ScatterFn<TS_MEAN>::apply(src, index, dim, out, dim_size)[0];
+}
+std::tuple<Tensor, Tensor> scatter_min(Tensor src, Tensor index, int64_t dim, OptTensor out, OptInt dim_size) {
+  auto r = ScatterFn<TS_MIN>::apply(src, index, dim, out, dim_size);
+  return std::make_tuple(r[0], r[1]);
+}
+std::tuple<Tensor, Tensor> scatter_max(Tensor src, Tensor index, int64_t dim, OptTensor out, OptInt dim_size) {
+  auto r = ScatterFn<TS_MAX>::apply(src, index, dim, out, dim_size);
+  return std::make_tuple(r[0], r[1]);
+}
+
+Tensor segment_sum_csr(Tensor src, Tensor indptr, OptTensor out) {
+  return SegmentCsrFn<TS_SUM>::apply(src, indptr, out)[0];
+}
+Tensor segment_mean_csr(Tensor src, Tensor indptr, OptTensor out) {
+  return SegmentCsrFn<TS_MEAN>::apply(src, indptr, out)[0];
+}
+std::tuple<Tensor, Tensor> segment_min_csr(Tensor src, Tensor indptr, OptTensor out) {
+  auto r = SegmentCsrFn<TS_MIN>::apply(src, indptr, out);
+  return std::make_tuple(r[0], r[1]);
+}
+std::tuple<Tensor, Tensor> segment_max_csr(Tensor src, Tensor indptr, OptTensor out) {
+  auto r = SegmentCsrFn<TS_MAX>::apply(src, indptr, out);
+  return std::make_tuple(r[0], r[1]);
+}
+Tensor gather_csr(Tensor src, Tensor indptr, OptTensor out) { return GatherCsrFn::apply(src, indptr, out)[0]; }
+
+Tensor segment_sum_coo(Tensor src, Tensor index, OptTensor out, OptInt dim_size) {
+  return SegmentCooFn<TS_SUM>::apply(src, index, out, dim_size)[0];
+}
+Tensor segment_mean_coo(Tensor src, Tensor index, OptTensor out, OptInt dim_size) {
+  return SegmentCooFn<TS_MEAN>::apply(src, index, out, dim_size)[0];
+}
+std::tuple<Tensor, Tensor> segment_min_coo(Tensor src, Tensor index, OptTensor out, OptInt dim_size) {
+  auto r = SegmentCooFn<TS_MIN>::apply(src, index, out, dim_size);
+  return std::make_tuple(r[0], r[1]);
+}
+std::tuple<Tensor, Tensor> segment_max_coo(Tensor src, Tensor index, OptTensor out, OptInt dim_size) {
+  auto r = SegmentCooFn<TS_MAX>::apply(src, index, out, dim_size);
+  return std::make_tuple(r[0], r[1]);
+}
+Tensor gather_coo(Tensor src, Tensor index, OptTensor out) { return GatherCooFn::apply(src, index, out)[0]; }
+
+int64_t cuda_version() { return ts_hip_version(); }  // csrc/version.cpp:28-38 returns HIP_VERSION on ROCm
+
+}  // namespace
+
+static auto registry = torch::RegisterOperators()
+                           .op("torch_scatter::cuda_version", &cuda_version)
+                           .op("torch_scatter::scatter_sum", &scatter_sum)
+                           .op("torch_scatter::scatter_mul", &scatter_mul)
+                           .op("torch_scatter::scatter_mean", &scatter_mean)
+                           .op("torch_scatter::scatter_min", &scatter_min)
+                           .op("torch_scatter::scatter_max", &scatter_max)
+                           .op("torch_scatter::segment_sum_csr", &segment_sum_csr)
+                           .op("torch_scatter::segment_mean_csr", &segment_mean_csr)
+                           .op("torch_scatter::segment_min_csr", &segment_min_csr)
+                           .op("torch_scatter::segment_max_csr", &segment_max_csr)
+                           .op("torch_scatter::gather_csr", &gather_csr)
+                           .op("torch_scatter::segment_sum_coo", &segment_sum_coo)
+                           .op("torch_scatter::segment_mean_coo", &segment_mean_coo)
+                           .op("torch_scatter::segment_min_coo", &segment_min_coo)
+                           .op("torch_scatter::segment_max_coo", &segment_max_coo)
+                           .op("torch_scatter::gather_coo", &gather_coo);

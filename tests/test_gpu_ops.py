@@ -1,0 +1,319 @@
+"""The registered operators (torch.ops.torch_scatter.* through the Python API)
+on the GPU against the reference's known-answer tables, with the reference's
+own test matrix: forward (eager and TorchScript), gradcheck, `out=`,
+non-contiguous inputs, zero-size tensors, broadcasting, composites.
+Follows test/test_scatter.py, test_segment.py, test_gather.py,
+test_zero_tensors.py, test_broadcasting.py and test/composite/*."""
+from itertools import product
+
+import numpy as np
+import pytest
+import torch
+from torch.autograd import gradcheck
+
+from helpers import DTYPES, REDUCTIONS, load_cases, random_csr, random_values, tensor
+
+pytestmark = pytest.mark.gpu
+DEV = torch.device("cuda:0")
+
+SCATTER = load_cases("scatter_cases")
+SEGMENT = load_cases("segment_cases")
+GATHER = load_cases("gather_cases")
+
+
+@pytest.fixture(scope="module")
+def ts():
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    import pytorch_scatter_amd
+    return pytorch_scatter_amd
+
+
+@pytest.mark.parametrize("ci,reduce,dtype", product(range(len(SCATTER)), REDUCTIONS + ["mul"], DTYPES))
+def test_scatter_forward(ts, ci, reduce, dtype):
+    case = SCATTER[ci]
+    if reduce not in case:
+        pytest.skip("table has no entry for this reduction")
+    src = tensor(case["src"], dtype, DEV)
+    index = tensor(case["index"], torch.long, DEV)
+    expected = tensor(case[reduce], dtype, DEV)
+    fn = getattr(ts, "scatter_" + reduce)
+    jit = torch.jit.script(fn)
+    out1 = fn(src, index, case["dim"])
+    out2 = jit(src, index, case["dim"])
+    if isinstance(out1, tuple):
+        out1, arg1 = out1
+        out2, arg2 = out2
+        if "arg_" + reduce in case:
+            assert torch.all(arg1 == tensor(case["arg_" + reduce], torch.long, DEV))
+        assert arg1.tolist() == arg2.tolist()
+    assert torch.all(out1 == expected)
+    assert out1.tolist() == out2.tolist()
+
+
+@pytest.mark.parametrize("ci,reduce", product(range(6), REDUCTIONS + ["mul"]))
+def test_scatter_backward(ts, ci, reduce):
+    case = SCATTER[ci]
+    src = tensor(case["src"], torch.double, DEV).requires_grad_()
+    index = tensor(case["index"], torch.long, DEV)
+    assert gradcheck(ts.scatter, (src, index, case["dim"], None, None, reduce))
+
+
+@pytest.mark.parametrize("ci,reduce,dtype", product(range(6), REDUCTIONS + ["mul"], DTYPES))
+def test_scatter_out(ts, ci, reduce, dtype):
+    case = SCATTER[ci]
+    src = tensor(case["src"], dtype, DEV)
+    index = tensor(case["index"], torch.long, DEV)
+    expected = tensor(case[reduce], dtype, DEV)
+    out = torch.full_like(expected, -2)
+    getattr(ts, "scatter_" + reduce)(src, index, case["dim"], out)
+    if reduce in ("sum", "add"):
+        expected = expected - 2
+    elif reduce in ("mul", "mean"):
+        expected = out  # not checkable from the table (as upstream)
+    elif reduce == "min":
+        expected = expected.fill_(-2)
+    elif reduce == "max":
+        expected[expected == 0] = -2
+    assert torch.all(out == expected)
+
+
+@pytest.mark.parametrize("ci,reduce,dtype", product(range(6), REDUCTIONS + ["mul"], DTYPES))
+def test_scatter_non_contiguous(ts, ci, reduce, dtype):
+    case = SCATTER[ci]
+    src = tensor(case["src"], dtype, DEV)
+    index = tensor(case["index"], torch.long, DEV)
+    expected = tensor(case[reduce], dtype, DEV)
+    if src.dim() > 1:
+        src = src.transpose(0, 1).contiguous().transpose(0, 1)
+    if index.dim() > 1:
+        index = index.transpose(0, 1).contiguous().transpose(0, 1)
+    out = getattr(ts, "scatter_" + reduce)(src, index, case["dim"])
+    if isinstance(out, tuple):
+        out, arg = out
+        assert torch.all(arg == tensor(case["arg_" + reduce], torch.long, DEV))
+    assert torch.all(out == expected)
+
+
+@pytest.mark.parametrize("ci,reduce,dtype", product(range(len(SEGMENT)), REDUCTIONS, DTYPES))
+def test_segment_forward(ts, ci, reduce, dtype):
+    case = SEGMENT[ci]
+    if reduce not in case:
+        pytest.skip("table has no entry for this reduction")
+    src = tensor(case["src"], dtype, DEV)
+    index = tensor(case["index"], torch.long, DEV)
+    indptr = tensor(case["indptr"], torch.long, DEV)
+    expected = tensor(case[reduce], dtype, DEV)
+    for name, idx in (("_csr", indptr), ("_coo", index)):
+        fn = getattr(ts, "segment_" + reduce + name)
+        jit = torch.jit.script(fn)
+        out1 = fn(src, idx)
+        out2 = jit(src, idx)
+        if isinstance(out1, tuple):
+            out1, arg1 = out1
+            out2, arg2 = out2
+            assert torch.all(arg1 == tensor(case["arg_" + reduce], torch.long, DEV))
+            assert arg1.tolist() == arg2.tolist()
+        assert torch.all(out1 == expected), name
+        assert out1.tolist() == out2.tolist()
+
+
+@pytest.mark.parametrize("ci,reduce", product(range(6), REDUCTIONS))
+def test_segment_backward(ts, ci, reduce):
+    case = SEGMENT[ci]
+    src = tensor(case["src"], torch.double, DEV).requires_grad_()
+    index = tensor(case["index"], torch.long, DEV)
+    indptr = tensor(case["indptr"], torch.long, DEV)
+    assert gradcheck(ts.segment_csr, (src, indptr, None, reduce))
+    assert gradcheck(ts.segment_coo, (src, index, None, None, reduce))
+
+
+@pytest.mark.parametrize("ci,reduce,dtype", product(range(6), REDUCTIONS, DTYPES))
+def test_segment_out(ts, ci, reduce, dtype):
+    case = SEGMENT[ci]
+    src = tensor(case["src"], dtype, DEV)
+    index = tensor(case["index"], torch.long, DEV)
+    indptr = tensor(case["indptr"], torch.long, DEV)
+    expected = tensor(case[reduce], dtype, DEV)
+    out = torch.full_like(expected, -2)
+    getattr(ts, "segment_" + reduce + "_csr")(src, indptr, out)   # csr overwrites
+    assert torch.all(out == expected)
+    out.fill_(-2)
+    getattr(ts, "segment_" + reduce + "_coo")(src, index, out)    # coo accumulates
+    if reduce in ("sum", "add"):
+        expected = expected - 2
+    elif reduce == "mean":
+        expected = out
+    elif reduce == "min":
+        expected = expected.fill_(-2)
+    elif reduce == "max":
+        expected[expected == 0] = -2
+    assert torch.all(out == expected)
+
+
+@pytest.mark.parametrize("ci,reduce,dtype", product(range(6), REDUCTIONS, DTYPES))
+def test_segment_non_contiguous(ts, ci, reduce, dtype):
+    case = SEGMENT[ci]
+    src = tensor(case["src"], dtype, DEV)
+    index = tensor(case["index"], torch.long, DEV)
+    indptr = tensor(case["indptr"], torch.long, DEV)
+    expected = tensor(case[reduce], dtype, DEV)
+    if src.dim() > 1:
+        src = src.transpose(0, 1).contiguous().transpose(0, 1)
+    if index.dim() > 1:
+        index = index.transpose(0, 1).contiguous().transpose(0, 1)
+    if indptr.dim() > 1:
+        indptr = indptr.transpose(0, 1).contiguous().transpose(0, 1)
+    for name, idx in (("_csr", indptr), ("_coo", index)):
+        out = getattr(ts, "segment_" + reduce + name)(src, idx)
+        if isinstance(out, tuple):
+            out, arg = out
+            assert torch.all(arg == tensor(case["arg_" + reduce], torch.long, DEV))
+        assert torch.all(out == expected)
+
+
+@pytest.mark.parametrize("ci,dtype", product(range(len(GATHER)), DTYPES))
+def test_gather_forward_out_non_contiguous(ts, ci, dtype):
+    case = GATHER[ci]
+    src = tensor(case["src"], dtype, DEV)
+    index = tensor(case["index"], torch.long, DEV)
+    indptr = tensor(case["indptr"], torch.long, DEV)
+    expected = tensor(case["expected"], dtype, DEV)
+    assert torch.all(ts.gather_csr(src, indptr) == expected)
+    assert torch.all(ts.gather_coo(src, index) == expected)
+    size = list(src.size())
+    size[index.dim() - 1] = index.size(-1)
+    out = src.new_full(size, -2)
+    ts.gather_csr(src, indptr, out)
+    assert torch.all(out == expected)
+    out.fill_(-2)
+    ts.gather_coo(src, index, out)
+    assert torch.all(out == expected)
+    if src.dim() > 1:
+        src = src.transpose(0, 1).contiguous().transpose(0, 1)
+    if index.dim() > 1:
+        index = index.transpose(0, 1).contiguous().transpose(0, 1)
+        indptr = indptr.transpose(0, 1).contiguous().transpose(0, 1)
+    assert torch.all(ts.gather_csr(src, indptr) == expected)
+    assert torch.all(ts.gather_coo(src, index) == expected)
+
+
+@pytest.mark.parametrize("ci", range(len(GATHER)))
+def test_gather_backward(ts, ci):
+    case = GATHER[ci]
+    src = tensor(case["src"], torch.double, DEV).requires_grad_()
+    index = tensor(case["index"], torch.long, DEV)
+    indptr = tensor(case["indptr"], torch.long, DEV)
+    assert gradcheck(ts.gather_csr, (src, indptr, None)) is True
+    assert gradcheck(ts.gather_coo, (src, index, None)) is True
+
+
+@pytest.mark.parametrize("reduce,dtype", product(REDUCTIONS, [torch.float, torch.double]))
+def test_zero_elements(ts, reduce, dtype):
+    x = torch.randn(0, 0, 0, 16, dtype=dtype, device=DEV, requires_grad=True)
+    index = tensor([], torch.long, DEV)
+    indptr = tensor([], torch.long, DEV)
+    for out in (ts.scatter(x, index, dim=0, dim_size=0, reduce=reduce),
+                ts.segment_coo(x, index, dim_size=0, reduce=reduce),
+                ts.gather_coo(x, index),
+                ts.segment_csr(x, indptr, reduce=reduce),
+                ts.gather_csr(x, indptr)):
+        out.backward(torch.randn_like(out))
+        assert out.size() == (0, 0, 0, 16)
+
+
+@pytest.mark.parametrize("reduce", REDUCTIONS)
+def test_broadcasting(ts, reduce):
+    B, C, H, W = (4, 3, 8, 8)
+    src = torch.randn((B, C, H, W), device=DEV)
+    index = torch.randint(0, H, (H,)).to(DEV, torch.long)
+    assert ts.scatter(src, index, dim=2, dim_size=H, reduce=reduce).size() == (B, C, H, W)
+    index = torch.randint(0, H, (B, 1, H, W)).to(DEV, torch.long)
+    assert ts.scatter(src, index, dim=2, dim_size=H, reduce=reduce).size() == (B, C, H, W)
+
+
+def test_scatter_matches_oracle_with_full_shape_index(ts, oracle):
+    rng = np.random.default_rng(0)
+    src = random_values(rng, (4, 3, 8, 5), torch.float, ties=True)
+    for shape, dim in (((8,), 2), ((4, 1, 8, 5), 2), ((4, 3, 8, 5), 1), ((5,), 3), ((4,), 0)):
+        index = torch.from_numpy(rng.integers(0, 6, size=shape))
+        if len(shape) == 4 and shape[1] == 1:
+            index = index.expand(4, 3, 8, 5)
+        for reduce in ("sum", "mean", "min", "max", "mul"):
+            want = oracle.op_scatter(src, index, dim, None, 7, reduce)
+            got = getattr(ts, "scatter_" + reduce)(src.to(DEV), index.to(DEV), dim, None, 7)
+            if isinstance(got, tuple):
+                assert torch.equal(got[1].cpu(), want[1]), (shape, dim, reduce)
+                got, want = got[0], want[0]
+            assert torch.allclose(got.cpu(), want, rtol=1e-5, atol=1e-5), (shape, dim, reduce)
+
+
+def test_fused_mean_backward_matches_closed_form(ts, oracle):
+    rng = np.random.default_rng(1)
+    indptr, index = random_csr(rng, 300, 40)
+    E = index.numel()
+    for dtype in (torch.float, torch.bfloat16):
+        src = torch.from_numpy(rng.standard_normal((E, 24))).to(dtype).to(DEV).requires_grad_()
+        g = torch.from_numpy(rng.standard_normal((300, 24))).to(dtype)
+        ts.segment_csr(src, indptr.to(DEV), reduce="mean").backward(g.to(DEV))
+        want = oracle.segment_mean_csr_backward(g, indptr, (E, 24))
+        assert torch.equal(src.grad.cpu(), want)
+        src.grad = None
+        ts.segment_coo(src, index.to(DEV), dim_size=300, reduce="mean").backward(g.to(DEV))
+        _, count = oracle.segment_coo(src.detach().cpu(), index, None, 300, "mean")
+        want = oracle.segment_mean_coo_backward(g, index, count, (E, 24))
+        assert torch.equal(src.grad.cpu(), want)
+        src.grad = None
+
+
+def test_min_max_backward_matches_reference_formula(ts, oracle):
+    rng = np.random.default_rng(2)
+    indptr, index = random_csr(rng, 200, 12)
+    E = index.numel()
+    src_cpu = random_values(rng, (E, 6), torch.double, ties=True)
+    g = torch.from_numpy(rng.standard_normal((200, 6)))
+    perm = torch.from_numpy(rng.permutation(E))
+    for reduce in ("min", "max"):
+        for fn, idx in ((ts.segment_csr, indptr), (ts.segment_coo, index)):
+            src = src_cpu.clone().to(DEV).requires_grad_()
+            args = (src, idx.to(DEV), None, reduce) if fn is ts.segment_csr else (src, idx.to(DEV), None, 200, reduce)
+            fn(*args).backward(g.to(DEV))
+            _, arg = oracle.segment_csr(src_cpu, indptr, None, reduce)
+            assert torch.equal(src.grad.cpu(), oracle.arg_backward(g, arg, (E, 6), 0))
+        src = src_cpu[perm].clone().to(DEV).requires_grad_()
+        ts.scatter(src, index[perm].to(DEV), 0, None, 200, reduce).backward(g.to(DEV))
+        _, arg = oracle.scatter(src_cpu[perm], oracle.broadcast(index[perm], src_cpu, 0), 0, None, 200, reduce)
+        assert torch.equal(src.grad.cpu(), oracle.arg_backward(g, arg, (E, 6), 0))
+
+
+def test_composites_against_dense_torch(ts):
+    # test/composite/test_softmax.py, test_logsumexp.py, test_std.py
+    src = torch.tensor([0.2, 0, 0.2, -2.1, 3.2, 7, -1, float("-inf")], device=DEV)
+    index = torch.tensor([0, 1, 0, 1, 1, 2, 4, 4], device=DEV)
+    out = ts.scatter_softmax(src, index)
+    groups = [[0, 2], [1, 3, 4], [5], [6, 7]]
+    for g in groups:
+        assert torch.allclose(out[g], torch.softmax(src[g], dim=-1))
+    out = ts.scatter_log_softmax(src, index)
+    for g in groups:
+        assert torch.allclose(out[g], torch.log_softmax(src[g], dim=-1))
+    out = ts.scatter_logsumexp(src, index)
+    want = torch.stack([torch.logsumexp(src[g], dim=-1) for g in groups[:3]] +
+                       [torch.tensor(0.0, device=DEV), torch.logsumexp(src[groups[3]], dim=-1)])
+    assert torch.allclose(out, want)
+    src = torch.tensor([[2.0, 0, 1, 4, 3], [0, 2, 1, 3, 4]], device=DEV, requires_grad=True)
+    index = torch.tensor([[0, 0, 0, 0, 0], [1, 1, 1, 1, 1]], device=DEV)
+    out = ts.scatter_std(src, index, dim=-1, unbiased=True)
+    std = src.std(dim=-1, unbiased=True)[0]
+    assert torch.allclose(out, torch.tensor([[std, 0], [0, std]], device=DEV))
+    out.backward(torch.randn_like(out))
+
+
+def test_errors_follow_reference_conventions(ts):
+    src = torch.randn(6, 4, device=DEV)
+    with pytest.raises(RuntimeError, match="Input mismatch"):
+        ts.segment_csr(src, torch.tensor([0, 3, 6], device=DEV), torch.empty(5, 4, device=DEV))
+    with pytest.raises(RuntimeError, match="Input mismatch"):
+        ts.gather_csr(src, torch.tensor([0, 3, 6], device=DEV))
+    with pytest.raises(RuntimeError, match="must be CUDA tensor"):
+        ts.scatter_sum(src, torch.tensor([0, 1, 0, 1, 2, 2]), 0)
