@@ -1,0 +1,272 @@
+#!/usr/bin/env python3
+"""Throughput of the scatter / segment / gather hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--configs C1,C2,...]
+
+Headline (`value`): configuration C2 of BASELINE.json -- segment_csr sum,
+segment_csr mean and gather_csr of the result back to the edges, 100000
+segments with Zipf(2.0) degrees, fp32 [E, 64] -- as effective HBM GB/s:
+algorithmic bytes (every input and output tensor counted once) divided by the
+wall time of K steps, inputs resident in HBM, called through the registered
+operators (torch.ops.torch_scatter.*). One step = the three ops once.
+
+The same JSON line carries
+  roofline      the dominant kernel of the headline (the CSR reduction), timed
+                with HIP events on the launch stream, against the 8 TB/s peak;
+  cpu_baseline  the reference's CPU kernels (oracle/_ref, else the C oracle)
+                timed on the host for the same workload, one thread;
+  configs       effective GB/s of every op of configurations C1..C5, timed the
+                same way (events around back-to-back launches).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for p in (ROOT, os.path.join(ROOT, "oracle")):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+PEAK_GBS = 8000.0  # MI355X HBM3E
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--configs", default="C1,C2,C2m,C3,C4,C5",
+                    help="comma list of side configurations to time (C2 is always run)")
+    ap.add_argument("--iters", type=int, default=20, help="launches per op in the per-config table")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    return ap.parse_args()
+
+
+def event_time(fn, iters, warm=3):
+    """Average seconds per call, HIP events on the current stream."""
+    import torch
+    for _ in range(warm):
+        fn()
+    torch.cuda.synchronize()
+    a = torch.cuda.Event(enable_timing=True)
+    b = torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(iters):
+        fn()
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) * 1e-3 / iters
+
+
+def gbs(nbytes, seconds):
+    return nbytes / seconds / 1e9
+
+
+def entry(nbytes, seconds, elems):
+    g = gbs(nbytes, seconds)
+    return {"GBps": round(g, 1), "pct_of_peak": round(100 * g / PEAK_GBS, 1), "us": round(seconds * 1e6, 1),
+            "Gelem_per_s": round(elems / seconds / 1e9, 2), "MB": round(nbytes / 1e6, 1)}
+
+
+def bench_csr_config(ts, wl, w, dev, iters, ops, uniform=False):
+    """segment / gather ops of one CSR-shaped workload through the operators."""
+    import torch
+    s = torch.empty(0, dtype=w.dtype).element_size()
+    src = wl.edge_values(w, dev, uniform=uniform)
+    indptr = w.indptr.to(dev)
+    index = w.index.to(dev)
+    out = torch.empty((w.N, w.K), dtype=w.dtype, device=dev)
+    res = {"N": w.N, "E": w.E, "K": w.K, "dtype": str(w.dtype).replace("torch.", ""),
+           "mean_degree": round(w.E / w.N, 2)}
+    EK = w.E * w.K
+    with torch.no_grad():
+        for op in ops:
+            if op in ("segment_csr_sum", "segment_csr_mean"):
+                r = op.rsplit("_", 1)[1]
+                t = event_time(lambda: ts.segment_csr(src, indptr, out, r), iters)
+                res[op] = entry(wl.bytes_segment(w.E, w.N, w.K, s), t, EK)
+            elif op == "segment_csr_max":
+                t = event_time(lambda: ts.segment_max_csr(src, indptr, out), iters)
+                res[op] = entry(wl.bytes_segment(w.E, w.N, w.K, s, True), t, EK)
+            elif op == "segment_coo_max":
+                t = event_time(lambda: ts.segment_max_coo(src, index, None, w.N), iters)
+                res[op] = entry(wl.bytes_segment(w.E, w.N, w.K, s, True, coo=True), t, EK)
+            elif op == "segment_coo_sum":
+                t = event_time(lambda: ts.segment_sum_coo(src, index, None, w.N), iters)
+                res[op] = entry(wl.bytes_segment(w.E, w.N, w.K, s, coo=True), t, EK)
+            elif op == "gather_csr":
+                t = event_time(lambda: ts.gather_csr(out, indptr, src), iters)
+                res[op] = entry(wl.bytes_gather(w.E, w.N, w.K, s), t, EK)
+            elif op == "gather_coo":
+                t = event_time(lambda: ts.gather_coo(out, index, src), iters)
+                res[op] = entry(wl.bytes_gather(w.E, w.N, w.K, s, coo=True), t, EK)
+            elif op == "segment_csr_mean_backward":
+                from pytorch_scatter_amd import capi
+                t = event_time(lambda: capi.segment_mean_csr_backward(out, indptr, src, 1, w.N, w.E, w.K, 0), iters)
+                res[op] = entry(wl.bytes_gather(w.E, w.N, w.K, s), t, EK)
+    del src, out
+    torch.cuda.empty_cache()
+    return res
+
+
+def bench_scatter_config(ts, wl, w, dev, iters, reduces):
+    import torch
+    src = wl.scatter_values(w, dev)
+    index = w.index.to(dev)
+    res = {"N": w.N, "E": w.E, "K": w.K, "dtype": "float32"}
+    with torch.no_grad():
+        for r in reduces:
+            if r == "sum":
+                t = event_time(lambda: ts.scatter_sum(src, index, 0, None, w.N), iters)
+                res["scatter_sum"] = entry(wl.bytes_scatter(w.E, w.N, w.K, 4), t, w.E * w.K)
+            else:
+                fn = ts.scatter_max if r == "max" else ts.scatter_min
+                t = event_time(lambda: fn(src, index, 0, None, w.N), iters)
+                res["scatter_" + r] = entry(wl.bytes_scatter(w.E, w.N, w.K, 4, True), t, w.E * w.K)
+    del src
+    torch.cuda.empty_cache()
+    return res
+
+
+def cpu_baseline(wl, w):
+    """The same three ops of C2 on the host, single thread: the reference's own
+    CPU kernels when oracle/_ref is built, else the C restatement."""
+    import torch
+    torch.set_num_threads(1)
+    g = torch.Generator().manual_seed(0)
+    src = torch.randn((w.E, w.K), generator=g, dtype=torch.float32)
+    out = torch.empty((w.N, w.K), dtype=torch.float32)
+    back = torch.empty_like(src)
+    kind = "port"
+    ref_path = os.path.join(ROOT, "oracle", "_ref", "libts_ref_cpu.so")
+    run = None
+    if os.path.exists(ref_path):
+        try:
+            torch.ops.load_library(ref_path)
+            ops = torch.ops.ts_ref
+
+            def run():
+                ops.segment_csr(src, w.indptr, out, "sum")
+                ops.segment_csr(src, w.indptr, out, "mean")
+                ops.gather_csr(out, w.indptr, back)
+            run()
+            kind = "reference"
+        except Exception:  # library built against another torch: fall back to the port
+            run = None
+    if run is None:
+        import ts_oracle
+
+        def run():
+            ts_oracle.segment_csr(src, w.indptr, out, "sum")
+            ts_oracle.segment_csr(src, w.indptr, out, "mean")
+            ts_oracle.gather_csr(out, w.indptr, back)
+        run()
+    reps = 5
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        run()
+    dt = (time.perf_counter() - t0) / reps
+    nbytes = 2 * wl.bytes_segment(w.E, w.N, w.K, 4) + wl.bytes_gather(w.E, w.N, w.K, 4)
+    return {"value": round(gbs(nbytes, dt), 3), "unit": "GB/s", "cores": 1, "kind": kind,
+            "host_cores_available": os.cpu_count(),
+            "sample": f"full C2 workload (E={w.E}, N={w.N}, K={w.K}, fp32), {reps} passes of "
+                      f"segment_csr sum + mean + gather_csr, {dt * 1e3:.1f} ms per pass"}
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU; every box of this run has a single MI355X, "
+              "so --gpus above 1 is not supported (the path shards by node range without any "
+              "exchange; see DESIGN.md).", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    import pytorch_scatter_amd as ts
+    from pytorch_scatter_amd import workloads as wl
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    # ---------------- headline: C2 through the registered operators
+    w2 = wl.c2_segment_csr()
+    src = wl.edge_values(w2, dev)
+    indptr = w2.indptr.to(dev)
+    out = torch.empty((w2.N, w2.K), dtype=torch.float32, device=dev)
+    back = torch.empty_like(src)
+    step_bytes = 2 * wl.bytes_segment(w2.E, w2.N, w2.K, 4) + wl.bytes_gather(w2.E, w2.N, w2.K, 4)
+
+    def step():
+        ts.segment_csr(src, indptr, out, "sum")
+        ts.segment_csr(src, indptr, out, "mean")
+        ts.gather_csr(out, indptr, back)
+
+    with torch.no_grad():
+        for _ in range(args.warmup):
+            step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            step()
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - t0) / args.steps
+        # dominant kernel: the CSR reduction (segment_csr sum), HIP events on the launch stream
+        t_kernel = event_time(lambda: ts.segment_csr(src, indptr, out, "sum"), max(args.steps, 20))
+    kernel_bytes = wl.bytes_segment(w2.E, w2.N, w2.K, 4)
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "traffic.json")
+    if os.path.exists(tpath):
+        traffic = json.load(open(tpath)).get("C2_segment_csr_sum_bytes_per_launch")
+    roofline = {"bound": "hbm", "kernel": "ts::csr_reduce_kernel<float, 4, SUM> (+ its fix-up launch)",
+                "achieved": round(gbs(kernel_bytes, t_kernel), 1), "peak": PEAK_GBS, "unit": "GB/s",
+                "frac": round(gbs(kernel_bytes, t_kernel) / PEAK_GBS, 4), "traffic": traffic,
+                "algorithmic_bytes_per_launch": kernel_bytes, "us_per_launch": round(t_kernel * 1e6, 2)}
+    del src, back, out
+    torch.cuda.empty_cache()
+
+    # ---------------- side table: every configuration
+    want = set(args.configs.split(",")) if args.configs else set()
+    table = {}
+    it = args.iters
+    if "C1" in want:
+        table["C1"] = bench_scatter_config(ts, wl, wl.c1_scatter_sum(), dev, it, ["sum"])
+    if "C2" in want:
+        table["C2"] = bench_csr_config(ts, wl, w2, dev, it, ["segment_csr_sum", "segment_csr_mean", "gather_csr"])
+    if "C2m" in want:
+        table["C2-mean16"] = bench_csr_config(ts, wl, wl.c2_segment_csr(mean16=True), dev, it,
+                                              ["segment_csr_sum", "segment_csr_mean", "gather_csr"])
+    if "C3" in want:
+        table["C3"] = bench_csr_config(ts, wl, wl.c3_segment_coo(), dev, it, ["segment_coo_max"], uniform=True)
+    if "C4" in want:
+        for K in (1, 32):
+            table[f"C4-K{K}"] = bench_scatter_config(ts, wl, wl.c4_scatter_minmax(K), dev, max(it // 2, 3),
+                                                     ["max", "min"])
+    if "C5" in want:
+        table["C5"] = bench_csr_config(ts, wl, wl.c5_gnn(), dev, max(it // 2, 3),
+                                       ["gather_csr", "segment_csr_mean", "segment_csr_mean_backward"])
+
+    cpu = None if args.no_cpu else cpu_baseline(wl, w2)
+
+    line = {
+        "metric": "effective HBM GB/s, segment_csr sum + mean + gather_csr (BASELINE config C2), 1 MI355X",
+        "value": round(gbs(step_bytes, dt), 1),
+        "unit": "GB/s",
+        "pct_of_8TBps_peak": round(100 * gbs(step_bytes, dt) / PEAK_GBS, 1),
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(dt * 1e3, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "C2: segment_csr sum+mean, gather_csr; 100000 segments, degrees "
+                               "clip(Zipf(2.0),1,512), src fp32 [E,64], numpy default_rng(0)",
+                   "N": w2.N, "E": w2.E, "K": w2.K, "algorithmic_bytes_per_step": step_bytes,
+                   "api": "torch.ops.torch_scatter.* (eager, out= preallocated)"},
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+        "configs": table,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()
