@@ -164,61 +164,113 @@ struct ScatterArgs {
   int64_t sb, se, sk;  // index strides
   int out_given;
   int precheck;        // read before the atomic: 0 none, 1 cached, 2 device-coherent, 3 streaming
+  int lds_cache;       // reduce hot slots in LDS first: 0 never, 1 for large inputs, 2 always
+  int64_t lds_epb;     // entries per workgroup chunk of that variant, 0 = default
+  int debug_skip;      // timing experiments only (wrong results): 1 skip misses, 2 skip flush, 4 skip hits
 };
 
-// grid-stride over the [B*E, K/VEC] vectors of src
+// ---- thread -> (edge, column) mapping shared by the scatter kernels ------------
+// A workgroup covers `epp` edges per pass with `L` lanes per edge, each lane
+// holding VEC consecutive columns; the column of a lane never changes, so the
+// hot loops are free of integer division. Rows wider than the workgroup are
+// covered by a loop over column chunks.
+struct EdgeLanes {
+  int L;    // lanes per edge
+  int epp;  // edges per pass of the workgroup
+  int el;   // this thread's edge slot, < epp (threads beyond are idle)
+  int cl;   // this thread's column lane, < L
+  bool active;
+};
+__device__ __forceinline__ EdgeLanes edge_lanes(int64_t kv, int block) {
+  EdgeLanes m;
+  m.L = kv < block ? (int)kv : block;
+  m.epp = block / m.L;
+  m.el = (int)threadIdx.x / m.L;
+  m.cl = (int)threadIdx.x - m.el * m.L;
+  m.active = m.el < m.epp;
+  return m;
+}
+// flat edge number -> (batch, position); the division only happens for batched inputs
+__device__ __forceinline__ void split_edge(const int64_t be, const int64_t B, const int64_t E, int64_t &b,
+                                           int64_t &e) {
+  if (B == 1) {
+    b = 0;
+    e = be;
+  } else {
+    b = be / E;
+    e = be - b * E;
+  }
+}
+
+// sum / mul: one atomic per element, consecutive lanes on consecutive columns
 template <typename T, int VEC, int REDUCE>
 __global__ __launch_bounds__(kBlock) void scatter_atomic_kernel(ScatterArgs a) {
+  constexpr int U = 4;
   const T *src = static_cast<const T *>(a.src);
   T *out = static_cast<T *>(a.out);
   const int64_t kv = a.K / VEC;
-  const int64_t nvec = a.B * a.E * kv;
-  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < nvec; i += (int64_t)gridDim.x * kBlock) {
-    const int64_t be = i / kv;
-    const int64_t k0 = (i - be * kv) * VEC;
-    const int64_t b = be / a.E;
-    const int64_t e = be - b * a.E;
-    const Vec<T, VEC> x = load_vec_stream<T, VEC>(src + i * VEC);
-    const int64_t ibase = b * a.sb + e * a.se + k0 * a.sk;
-    int64_t idx = a.index[ibase];
+  const EdgeLanes m = edge_lanes(kv, kBlock);
+  if (!m.active) return;
+  const int64_t n_edges = a.B * a.E;
+  const int64_t stride = (int64_t)gridDim.x * m.epp;
+  for (int64_t be0 = (int64_t)blockIdx.x * m.epp + m.el; be0 < n_edges; be0 += stride * U) {
+    for (int64_t cv = m.cl; cv < kv; cv += m.L) {
+      const int64_t k0 = cv * VEC;
+      Vec<T, VEC> x[U];
+      int64_t idx[U], bb[U], ee[U];
 #pragma unroll
-    for (int v = 0; v < VEC; ++v) {
-      if (v > 0 && a.sk != 0) idx = a.index[ibase + v * a.sk];
-      if (idx < 0 || idx >= a.N) continue;
-      T *p = out + (b * a.N + idx) * a.K + k0 + v;
-      const T val = x.v[v];
-      if (REDUCE == TS_SUM)
-        atomic_add_elem<T>(p, val);
-      else
-        atomic_rmw<T>(p, [val](T cur) { return mul_elem<T>(cur, val); });
+      for (int u = 0; u < U; ++u) {
+        const int64_t be = be0 + u * stride;
+        split_edge(be < n_edges ? be : be0, a.B, a.E, bb[u], ee[u]);
+        x[u] = load_vec_stream<T, VEC>(src + (bb[u] * a.E + ee[u]) * a.K + k0);
+        idx[u] = a.index[bb[u] * a.sb + ee[u] * a.se + k0 * a.sk];
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        if (be0 + u * stride >= n_edges) continue;
+        int64_t id = idx[u];
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) {
+          if (v > 0 && a.sk != 0) id = a.index[bb[u] * a.sb + ee[u] * a.se + (k0 + v) * a.sk];
+          if (id < 0 || id >= a.N) continue;
+          T *p = out + (bb[u] * a.N + id) * a.K + k0 + v;
+          const T val = x[u].v[v];
+          if (REDUCE == TS_SUM)
+            atomic_add_elem<T>(p, val);
+          else
+            atomic_rmw<T>(p, [val](T cur) { return mul_elem<T>(cur, val); });
+        }
+      }
     }
   }
 }
 
 // packed-pair add for 16-bit floats: two neighbouring columns in one atomic
+// (requires K even, one index per row, 4-byte aligned src/out)
 template <typename T>
 __global__ __launch_bounds__(kBlock) void scatter_add_pk16_kernel(ScatterArgs a) {
-  // requires K even, sk == 0, out 4-byte aligned
   const T *src = static_cast<const T *>(a.src);
   T *out = static_cast<T *>(a.out);
   const int64_t kv = a.K / 2;
-  const int64_t nvec = a.B * a.E * kv;
-  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < nvec; i += (int64_t)gridDim.x * kBlock) {
-    const int64_t be = i / kv;
-    const int64_t k0 = (i - be * kv) * 2;
-    const int64_t b = be / a.E;
-    const int64_t e = be - b * a.E;
+  const EdgeLanes m = edge_lanes(kv, kBlock);
+  if (!m.active) return;
+  const int64_t n_edges = a.B * a.E;
+  for (int64_t be = (int64_t)blockIdx.x * m.epp + m.el; be < n_edges; be += (int64_t)gridDim.x * m.epp) {
+    int64_t b, e;
+    split_edge(be, a.B, a.E, b, e);
     const int64_t idx = a.index[b * a.sb + e * a.se];
     if (idx < 0 || idx >= a.N) continue;
-    T *p = out + (b * a.N + idx) * a.K + k0;
-    if constexpr (sizeof(T) == 2 && __is_same(T, bf16_t)) {
-      typedef short v2s __attribute__((ext_vector_type(2)));
-      v2s val = *reinterpret_cast<const v2s *>(src + i * 2);
-      __builtin_amdgcn_global_atomic_fadd_v2bf16(reinterpret_cast<v2s *>(p), val);
-    } else {
-      typedef _Float16 v2h __attribute__((ext_vector_type(2)));
-      v2h val = *reinterpret_cast<const v2h *>(src + i * 2);
-      __builtin_amdgcn_global_atomic_fadd_v2f16(reinterpret_cast<v2h *>(p), val);
+    for (int64_t cv = m.cl; cv < kv; cv += m.L) {
+      const int64_t k0 = cv * 2;
+      T *p = out + (b * a.N + idx) * a.K + k0;
+      const T *q = src + be * a.K + k0;
+      if constexpr (__is_same(T, bf16_t)) {
+        typedef short v2s __attribute__((ext_vector_type(2)));
+        __builtin_amdgcn_global_atomic_fadd_v2bf16(reinterpret_cast<v2s *>(p), *reinterpret_cast<const v2s *>(q));
+      } else {
+        typedef _Float16 v2h __attribute__((ext_vector_type(2)));
+        __builtin_amdgcn_global_atomic_fadd_v2f16(reinterpret_cast<v2h *>(p), *reinterpret_cast<const v2h *>(q));
+      }
     }
   }
 }
@@ -242,38 +294,192 @@ __global__ __launch_bounds__(kBlock) void scatter_key_init_kernel(ScatterArgs a)
   }
 }
 
+// keys of one lane's VEC columns against the global table: read the current
+// keys first (one vector load), then issue atomics only for the improvements
+template <int VEC>
+__device__ __forceinline__ void keys_to_global(uint64_t *p, const uint64_t *key, int precheck) {
+  uint64_t cur[VEC];
+  if (precheck != 0) {
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) {
+      if (precheck == 2)
+        cur[v] = __hip_atomic_load(p + v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      else if (precheck == 3)
+        cur[v] = __builtin_nontemporal_load(p + v);
+      else
+        cur[v] = p[v];  // cached read: a stale value only costs a spare atomic
+    }
+  }
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) {
+    if (key[v] == 0) continue;  // nothing to contribute (NaN or index out of range)
+    if (precheck != 0 && key[v] <= cur[v]) continue;
+    __hip_atomic_fetch_max(p + v, key[v], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+
+// keys of the VEC columns a lane holds for one edge; 0 = nothing to contribute
+template <typename T, int VEC, bool IS_MAX>
+__device__ __forceinline__ void make_keys(const Vec<T, VEC> &x, int64_t e, uint64_t *key) {
+  const uint32_t low = 0xFFFFFFFEu - (uint32_t)e;
+#pragma unroll
+  for (int v = 0; v < VEC; ++v)
+    key[v] = Key<T>::is_nan(x.v[v]) ? 0 : pack_key<T, IS_MAX>(x.v[v], low);  // NaN never wins
+}
+
+// straight to the global table (per-element index, small inputs, very wide rows)
 template <typename T, int VEC, bool IS_MAX>
 __global__ __launch_bounds__(kBlock) void scatter_key_kernel(ScatterArgs a) {
+  constexpr int U = 4;
   const T *src = static_cast<const T *>(a.src);
   uint64_t *keys = reinterpret_cast<uint64_t *>(a.arg_out);
   const int64_t kv = a.K / VEC;
-  const int64_t nvec = a.B * a.E * kv;
-  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < nvec; i += (int64_t)gridDim.x * kBlock) {
-    const int64_t be = i / kv;
-    const int64_t k0 = (i - be * kv) * VEC;
-    const int64_t b = be / a.E;
-    const int64_t e = be - b * a.E;
-    const Vec<T, VEC> x = load_vec_stream<T, VEC>(src + i * VEC);
-    const int64_t ibase = b * a.sb + e * a.se + k0 * a.sk;
-    int64_t idx = a.index[ibase];
-    const uint32_t low = 0xFFFFFFFEu - (uint32_t)e;
+  const EdgeLanes m = edge_lanes(kv, kBlock);
+  if (!m.active) return;
+  const int64_t n_edges = a.B * a.E;
+  const int64_t stride = (int64_t)gridDim.x * m.epp;
+  for (int64_t be0 = (int64_t)blockIdx.x * m.epp + m.el; be0 < n_edges; be0 += stride * U) {
+    for (int64_t cv = m.cl; cv < kv; cv += m.L) {
+      const int64_t k0 = cv * VEC;
+      Vec<T, VEC> x[U];
+      int64_t idx[U], bb[U], ee[U];
 #pragma unroll
-    for (int v = 0; v < VEC; ++v) {
-      if (v > 0 && a.sk != 0) idx = a.index[ibase + v * a.sk];
-      if (idx < 0 || idx >= a.N) continue;
-      const T val = x.v[v];
-      if (Key<T>::is_nan(val)) continue;  // NaN never wins (csrc/cpu/reducer.h:63-67)
-      const uint64_t key = pack_key<T, IS_MAX>(val, low);
-      uint64_t *p = keys + (b * a.N + idx) * a.K + k0 + v;
-      if (a.precheck == 1) {
-        if (key <= *reinterpret_cast<volatile uint64_t *>(p)) continue;
-      } else if (a.precheck == 2) {
-        if (key <= __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) continue;
-      } else if (a.precheck == 3) {
-        if (key <= __builtin_nontemporal_load(p)) continue;
+      for (int u = 0; u < U; ++u) {
+        const int64_t be = be0 + u * stride;
+        split_edge(be < n_edges ? be : be0, a.B, a.E, bb[u], ee[u]);  // re-doing an edge is harmless under max
+        x[u] = load_vec_stream<T, VEC>(src + (bb[u] * a.E + ee[u]) * a.K + k0);
+        idx[u] = a.index[bb[u] * a.sb + ee[u] * a.se + k0 * a.sk];
       }
-      __hip_atomic_fetch_max(p, key, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        uint64_t key[VEC];
+        make_keys<T, VEC, IS_MAX>(x[u], ee[u], key);
+        if (a.sk == 0) {
+          if (idx[u] < 0 || idx[u] >= a.N) continue;
+          keys_to_global<VEC>(keys + (bb[u] * a.N + idx[u]) * a.K + k0, key, a.precheck);
+        } else {
+#pragma unroll
+          for (int v = 0; v < VEC; ++v) {
+            const int64_t id = v == 0 ? idx[u] : a.index[bb[u] * a.sb + ee[u] * a.se + (k0 + v) * a.sk];
+            if (id < 0 || id >= a.N) continue;
+            keys_to_global<1>(keys + (bb[u] * a.N + id) * a.K + k0 + v, key + v, a.precheck);
+          }
+        }
+      }
     }
+  }
+}
+
+// ---- packed-key min/max with a workgroup-private cache of hot slots ---------
+// Skewed indices (a hub node owning 20 % of the entries) would serialise on a
+// handful of global addresses. Each workgroup therefore reduces its chunk of
+// entries into an LDS table first -- direct-mapped on the node id, one row of K
+// keys per cached node, claimed with a compare-and-swap on the tag -- and only
+// writes the per-node winners to global memory once per chunk. Entries whose
+// table row is taken by another node go to global memory directly, after the
+// same read-before-atomic test. One index per row is required (sk == 0).
+constexpr int kLdsKeys = 4096;        // 32 KB of 64-bit keys
+constexpr int kLdsBlock = 256;  // 3 workgroups per CU (LDS-limited) at <= 168 VGPRs
+
+template <typename T, int VEC, bool IS_MAX>
+__global__ __launch_bounds__(kLdsBlock) void scatter_key_lds_kernel(ScatterArgs a, int tn_mask, int64_t epb) {
+  constexpr int U = VEC == 1 ? 8 : 4;
+  __shared__ uint64_t s_keys[kLdsKeys];
+  __shared__ int32_t s_tags[kLdsKeys];
+  const int K = (int)a.K;
+  const int tn = tn_mask + 1;
+  for (int i = threadIdx.x; i < tn * K; i += kLdsBlock) s_keys[i] = 0;
+  for (int i = threadIdx.x; i < tn; i += kLdsBlock) s_tags[i] = -1;
+  __syncthreads();
+
+  const T *src = static_cast<const T *>(a.src);
+  uint64_t *gkeys = reinterpret_cast<uint64_t *>(a.arg_out);
+  const int kv = K / VEC;
+  const EdgeLanes m = edge_lanes(kv, kLdsBlock);
+  const int64_t be_lo = (int64_t)blockIdx.x * epb;
+  int64_t be_hi = be_lo + epb;
+  if (be_hi > a.B * a.E) be_hi = a.B * a.E;
+
+  if (m.active) {
+    for (int64_t be0 = be_lo + m.el; be0 < be_hi; be0 += (int64_t)m.epp * U) {
+      for (int cv = m.cl; cv < kv; cv += m.L) {
+        const int k0 = cv * VEC;
+        Vec<T, VEC> x[U];
+        int64_t idx[U], bb[U], ee[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const int64_t be = be0 + (int64_t)u * m.epp;
+          split_edge(be < be_hi ? be : be0, a.B, a.E, bb[u], ee[u]);
+          x[u] = load_vec_stream<T, VEC>(src + (bb[u] * a.E + ee[u]) * a.K + k0);
+          idx[u] = a.index[bb[u] * a.sb + ee[u] * a.se];
+        }
+        uint64_t key[U][VEC];
+        int64_t miss_node[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          miss_node[u] = -1;
+          if (idx[u] < 0 || idx[u] >= a.N) continue;
+          make_keys<T, VEC, IS_MAX>(x[u], ee[u], key[u]);
+          const int node = (int)(bb[u] * a.N + idx[u]);
+          const int row = node & tn_mask;
+          int tag = s_tags[row];
+          if (tag == -1) {
+            const int old = atomicCAS(&s_tags[row], -1, node);
+            tag = old == -1 ? node : old;
+          }
+          if (tag == node) {
+            if (a.debug_skip & 4) continue;
+            uint64_t *p = &s_keys[row * K + k0];
+#pragma unroll
+            for (int v = 0; v < VEC; ++v)
+              if (key[u][v] > *reinterpret_cast<volatile uint64_t *>(p + v))
+                __hip_atomic_fetch_max(p + v, key[u][v], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+          } else if (!(a.debug_skip & 1)) {
+            miss_node[u] = node;
+          }
+        }
+        // entries whose table row belongs to another node: all reads first, then the atomics
+        uint64_t cur[U][VEC];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          if (miss_node[u] < 0) continue;
+          const uint64_t *p = gkeys + miss_node[u] * a.K + k0;
+#pragma unroll
+          for (int v = 0; v < VEC; ++v) cur[u][v] = p[v];  // cached read: a stale value only costs a spare atomic
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          if (miss_node[u] < 0) continue;
+          uint64_t *p = gkeys + miss_node[u] * a.K + k0;
+#pragma unroll
+          for (int v = 0; v < VEC; ++v)
+            if (key[u][v] > cur[u][v])
+              __hip_atomic_fetch_max(p + v, key[u][v], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+      }
+    }
+  }
+  __syncthreads();
+  if (a.debug_skip & 2) return;
+  // per-node winners of this chunk -> global table
+  for (int i0 = threadIdx.x; i0 < tn * K; i0 += kLdsBlock * 4) {
+    uint64_t key[4], cur[4];
+    uint64_t *p[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int i = i0 + j * kLdsBlock;
+      key[j] = i < tn * K ? s_keys[i] : 0;
+      p[j] = nullptr;
+      if (key[j] != 0) {
+        const int row = i / K;
+        p[j] = gkeys + (int64_t)s_tags[row] * a.K + (i - row * K);
+        cur[j] = *p[j];
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if (key[j] != 0 && key[j] > cur[j])
+        __hip_atomic_fetch_max(p[j], key[j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
 }
 
@@ -366,35 +572,50 @@ inline unsigned grid_for(int64_t n, int per_thread = 1) {
 // ---- host side --------------------------------------------------------------------
 template <typename T> struct IsWide { static constexpr bool value = sizeof(T) == 8; };
 
+// workgroups needed so that every edge is visited once: `block` threads cover
+// block / min(kv, block) edges per pass and U passes per loop trip
+inline unsigned scatter_grid(int64_t n_edges, int64_t kv, int block, int U) {
+  const int64_t L = kv < block ? kv : block;
+  const int64_t per_block = (block / L) * U;
+  int64_t blocks = (n_edges + per_block - 1) / per_block;
+  if (blocks < 1) blocks = 1;
+  const int64_t cap = 256 * 64;
+  return (unsigned)(blocks < cap ? blocks : cap);
+}
+
 template <typename T, int VEC>
 int launch_scatter_v(const ScatterArgs &a, int reduce, hipStream_t stream) {
   T *out = static_cast<T *>(a.out);
   const int64_t n_out = a.B * a.N * a.K;
   const int64_t n_src = a.B * a.E * a.K;
-  const unsigned g_src = grid_for(n_src / VEC);
+  const int64_t n_edges = a.B * a.E;
   const unsigned g_out = grid_for(n_out);
   if (reduce == TS_SUM || reduce == TS_MUL) {
     if (!a.out_given)
       hipLaunchKernelGGL(fill_kernel<T>, dim3(g_out), dim3(kBlock), 0, stream, out, n_out,
                          small_const<T>(reduce == TS_MUL ? 1 : 0));
     if (n_src > 0) {
+      // one element per lane: the 64 atomics of a wavefront then cover whole cache lines
+      // (4 lines per instruction for fp32 instead of 16 with 4 elements per lane)
+      const unsigned g = scatter_grid(n_edges, a.K, kBlock, 4);
       if (reduce == TS_SUM) {
         if constexpr (__is_same(T, bf16_t) || __is_same(T, f16_t)) {
           if (a.K % 2 == 0 && a.sk == 0 && (reinterpret_cast<uintptr_t>(a.out) & 3) == 0 &&
               (reinterpret_cast<uintptr_t>(a.src) & 3) == 0) {
-            hipLaunchKernelGGL(scatter_add_pk16_kernel<T>, dim3(grid_for(n_src / 2)), dim3(kBlock), 0,
-                               stream, a);
+            hipLaunchKernelGGL(scatter_add_pk16_kernel<T>, dim3(scatter_grid(n_edges, a.K / 2, kBlock, 1)),
+                               dim3(kBlock), 0, stream, a);
             return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
           }
         }
-        hipLaunchKernelGGL((scatter_atomic_kernel<T, VEC, TS_SUM>), dim3(g_src), dim3(kBlock), 0, stream, a);
+        hipLaunchKernelGGL((scatter_atomic_kernel<T, 1, TS_SUM>), dim3(g), dim3(kBlock), 0, stream, a);
       } else {
-        hipLaunchKernelGGL((scatter_atomic_kernel<T, VEC, TS_MUL>), dim3(g_src), dim3(kBlock), 0, stream, a);
+        hipLaunchKernelGGL((scatter_atomic_kernel<T, 1, TS_MUL>), dim3(g), dim3(kBlock), 0, stream, a);
       }
     }
   } else if (reduce == TS_MIN || reduce == TS_MAX) {
     const bool is_max = reduce == TS_MAX;
     if constexpr (IsWide<T>::value) {
+      const unsigned g_src = grid_for(n_src);
       const T init = is_max ? std::numeric_limits<T>::lowest() : std::numeric_limits<T>::max();
       if (!a.out_given)
         hipLaunchKernelGGL(fill_kernel<T>, dim3(g_out), dim3(kBlock), 0, stream, out, n_out, init);
@@ -411,15 +632,41 @@ int launch_scatter_v(const ScatterArgs &a, int reduce, hipStream_t stream) {
         hipLaunchKernelGGL(scatter_arg_wide_kernel<T>, dim3(g_src), dim3(kBlock), 0, stream, a);
     } else {
       if (a.E >= 0xFFFFFFFEll) return TS_ERR_UNSUPPORTED;
+      // LDS-cached variant: one index per row, at least 64 table rows, node ids that fit 31 bits,
+      // and enough entries per output slot for repeats inside a chunk to be likely (a uniform
+      // index with few entries per slot is served better by the direct kernel)
+      int tn = 1;
+      while ((int64_t)tn * 2 * a.K <= kLdsKeys) tn *= 2;
+      const bool use_lds = a.lds_cache && a.sk == 0 && tn >= 64 && a.B * a.N < 0x7FFFFFFFll &&
+                           (a.lds_cache == 2 || (n_src >= ((int64_t)1 << 20) && n_edges >= 32 * a.B * a.N));
+      // entries per workgroup chunk: large enough to amortise writing the table back,
+      // small enough to leave a few thousand workgroups
+      int64_t epb = a.lds_epb > 0 ? a.lds_epb : ((int64_t)1 << 15) / a.K;
+      if (a.lds_epb <= 0) {
+        while (epb > 256 && n_edges / epb < 2048) epb /= 2;
+      }
+      if (epb < 64) epb = 64;
+      const unsigned g_lds = (unsigned)((n_edges + epb - 1) / epb);
+      const unsigned g_key = scatter_grid(n_edges, a.K / VEC, kBlock, 4);
       if (is_max) {
         hipLaunchKernelGGL((scatter_key_init_kernel<T, true>), dim3(g_out), dim3(kBlock), 0, stream, a);
-        if (n_src > 0)
-          hipLaunchKernelGGL((scatter_key_kernel<T, VEC, true>), dim3(g_src), dim3(kBlock), 0, stream, a);
+        if (n_src > 0) {
+          if (use_lds)
+            hipLaunchKernelGGL((scatter_key_lds_kernel<T, VEC, true>), dim3(g_lds), dim3(kLdsBlock), 0, stream, a,
+                               tn - 1, epb);
+          else
+            hipLaunchKernelGGL((scatter_key_kernel<T, VEC, true>), dim3(g_key), dim3(kBlock), 0, stream, a);
+        }
         hipLaunchKernelGGL((scatter_key_final_kernel<T, true>), dim3(g_out), dim3(kBlock), 0, stream, a);
       } else {
         hipLaunchKernelGGL((scatter_key_init_kernel<T, false>), dim3(g_out), dim3(kBlock), 0, stream, a);
-        if (n_src > 0)
-          hipLaunchKernelGGL((scatter_key_kernel<T, VEC, false>), dim3(g_src), dim3(kBlock), 0, stream, a);
+        if (n_src > 0) {
+          if (use_lds)
+            hipLaunchKernelGGL((scatter_key_lds_kernel<T, VEC, false>), dim3(g_lds), dim3(kLdsBlock), 0, stream, a,
+                               tn - 1, epb);
+          else
+            hipLaunchKernelGGL((scatter_key_kernel<T, VEC, false>), dim3(g_key), dim3(kBlock), 0, stream, a);
+        }
         hipLaunchKernelGGL((scatter_key_final_kernel<T, false>), dim3(g_out), dim3(kBlock), 0, stream, a);
       }
     }

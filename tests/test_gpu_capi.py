@@ -321,6 +321,36 @@ def test_scatter(capi, oracle, shape, reduce, dtype):
                 assert bool((err <= 2.0 ** -8 * cnt * absum.clamp(min=1e-30) + 1e-30).all()), mode
 
 
+@pytest.mark.parametrize("shape,reduce,dtype", product(
+    [(1, 30000, 1, 500), (1, 9000, 32, 300), (2, 5000, 8, 40), (1, 4000, 12, 70000)],
+    ["min", "max"], [torch.float32, torch.bfloat16, torch.int32]))
+def test_scatter_minmax_lds_cached_variant(capi, oracle, shape, reduce, dtype, monkeypatch):
+    """The workgroup-private table variant (forced on, with a small chunk so that
+    several workgroups meet on the same slots), skewed index with heavy ties."""
+    monkeypatch.setenv("TS_SCATTER_LDS", "2")
+    monkeypatch.setenv("TS_SCATTER_EPB", "700")
+    B, E, K, N = shape
+    rng = np.random.default_rng(E + K)
+    src = random_values(rng, (B, E, K), dtype, ties=True)
+    p = np.arange(1, N + 1, dtype=np.float64) ** -1.2
+    index1 = torch.from_numpy(rng.choice(N, size=E, p=p / p.sum()))
+    index = index1.view(1, E, 1).expand(B, E, K)
+    for out_given in (False, True):
+        if out_given:
+            prev = random_values(rng, (B, N, K), dtype, ties=True)
+            want = prev.clone()
+            _, want_arg = oracle.scatter(src, index, 1, want, None, reduce)
+            out = prev.clone().to(DEV)
+        else:
+            want, want_arg = oracle.scatter(src, index, 1, None, N, reduce)
+            out = torch.empty((B, N, K), dtype=dtype, device=DEV)
+        arg = torch.empty((B, N, K), dtype=torch.long, device=DEV)
+        capi.scatter(src.to(DEV), index1.to(DEV), out, arg, B, E, K, N, 0, 1, 0, capi.REDUCE[reduce], out_given)
+        torch.cuda.synchronize()
+        assert_exact(out, want)
+        assert_exact(arg, want_arg)
+
+
 @pytest.mark.parametrize("reduce,dtype", product(["sum", "min", "max"], [torch.float32, torch.float64, torch.int64]))
 def test_scatter_out_given_and_wide_types(capi, oracle, reduce, dtype):
     B, E, K, N = 2, 3000, 6, 40
