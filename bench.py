@@ -179,8 +179,8 @@ def main():
     args = parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU; every box of this run has a single MI355X, "
-              "so --gpus above 1 is not supported (the path shards by node range without any "
-              "exchange; see DESIGN.md).", file=sys.stderr)
+              "so --gpus above 1 is not supported (segment / gather ops would shard by node range "
+              "without any exchange).", file=sys.stderr)
         sys.exit(2)
     import torch
     assert torch.cuda.is_available(), "bench.py needs a GPU"
