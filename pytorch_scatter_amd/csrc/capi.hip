@@ -282,7 +282,6 @@ int ts_scatter(const void *src, const int64_t *index, void *out, int64_t *arg_ou
   a.precheck = env_int("TS_SCATTER_PRECHECK", 1);   // tuning aids
   a.lds_cache = env_int("TS_SCATTER_LDS", 1);
   a.lds_epb = env_int("TS_SCATTER_EPB", 0);
-  a.debug_skip = env_int("TS_SCATTER_DEBUG_SKIP", 0);
   const int full = kVecBytes / kElemBytes[dtype];
   const int vec = (full > 1 && K % full == 0 && aligned16(src)) ? full : 1;
   return dispatch_scatter(dtype, a, reduce, vec, static_cast<hipStream_t>(stream));

@@ -34,7 +34,6 @@ __global__ __launch_bounds__(kBlock) void csr_gather_kernel(CsrGatherArgs a) {
 
   const int tid = threadIdx.x;
   const int G = a.G;
-  const int W = kBlock / G;
   const int w = tid / G;
   const int lg = tid - w * G;
   const int64_t col = (int64_t)blockIdx.y * (G * VEC) + (int64_t)lg * VEC;

@@ -166,7 +166,6 @@ struct ScatterArgs {
   int precheck;        // read before the atomic: 0 none, 1 cached, 2 device-coherent, 3 streaming
   int lds_cache;       // reduce hot slots in LDS first: 0 never, 1 for large inputs, 2 always
   int64_t lds_epb;     // entries per workgroup chunk of that variant, 0 = default
-  int debug_skip;      // timing experiments only (wrong results): 1 skip misses, 2 skip flush, 4 skip hits
 };
 
 // ---- thread -> (edge, column) mapping shared by the scatter kernels ------------
@@ -428,13 +427,12 @@ __global__ __launch_bounds__(kLdsBlock) void scatter_key_lds_kernel(ScatterArgs 
             tag = old == -1 ? node : old;
           }
           if (tag == node) {
-            if (a.debug_skip & 4) continue;
             uint64_t *p = &s_keys[row * K + k0];
 #pragma unroll
             for (int v = 0; v < VEC; ++v)
               if (key[u][v] > *reinterpret_cast<volatile uint64_t *>(p + v))
                 __hip_atomic_fetch_max(p + v, key[u][v], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-          } else if (!(a.debug_skip & 1)) {
+          } else {
             miss_node[u] = node;
           }
         }
@@ -460,7 +458,6 @@ __global__ __launch_bounds__(kLdsBlock) void scatter_key_lds_kernel(ScatterArgs 
     }
   }
   __syncthreads();
-  if (a.debug_skip & 2) return;
   // per-node winners of this chunk -> global table
   for (int i0 = threadIdx.x; i0 < tn * K; i0 += kLdsBlock * 4) {
     uint64_t key[4], cur[4];
