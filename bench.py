@@ -41,6 +41,9 @@ def parse_args():
                     help="comma list of side configurations to time (C2 is always run)")
     ap.add_argument("--iters", type=int, default=20, help="launches per op in the per-config table")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--probe", action="store_true",
+                    help="counter-collection mode for rocprofv3 --pmc: a few launches of the dominant kernels "
+                         "next to copies of known size, nothing timed")
     return ap.parse_args()
 
 
@@ -175,8 +178,49 @@ def cpu_baseline(wl, w):
                       f"segment_csr sum + mean + gather_csr, {dt * 1e3:.1f} ms per pass"}
 
 
+def probe():
+    """Launch sequence for `rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE -- python3 bench.py --probe`:
+    1. torch copy of 1 GiB (plain loads/stores, known size: calibrates the counters);
+    2. segment_csr sum with one entry per segment over 1 GiB of fp32 [4Mi, 64]: a copy through the
+       reduction kernel itself (same non-temporal loads), known size;
+    3. C2 segment_csr sum x3, C5 segment_csr mean x2, C5 gather_csr x2."""
+    import torch
+    import pytorch_scatter_amd as ts
+    from pytorch_scatter_amd import workloads as wl
+    dev = torch.device("cuda:0")
+    a = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+    b = torch.empty_like(a)
+    b.copy_(a)
+    n = 1 << 22
+    x = torch.ones((n, 64), dtype=torch.float32, device=dev)
+    ident = torch.arange(n + 1, device=dev)
+    y = torch.empty_like(x)
+    with torch.no_grad():
+        ts.segment_csr(x, ident, y, "sum")
+        del a, b, x, y
+        w2 = wl.c2_segment_csr()
+        src = wl.edge_values(w2, dev)
+        out = torch.empty((w2.N, w2.K), dtype=torch.float32, device=dev)
+        for _ in range(3):
+            ts.segment_csr(src, w2.indptr.to(dev), out, "sum")
+        del src, out
+        w5 = wl.c5_gnn()
+        src = wl.edge_values(w5, dev)
+        out = torch.empty((w5.N, w5.K), dtype=torch.bfloat16, device=dev)
+        ip = w5.indptr.to(dev)
+        for _ in range(2):
+            ts.segment_csr(src, ip, out, "mean")
+        for _ in range(2):
+            ts.gather_csr(out, ip, src)
+    torch.cuda.synchronize()
+    print(json.dumps({"probe": "done", "copy_bytes": 1 << 30, "identity_rows": n, "C2": [w2.N, w2.E, w2.K],
+                      "C5": [w5.N, w5.E, w5.K]}))
+
+
 def main():
     args = parse_args()
+    if args.probe:
+        return probe()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU; every box of this run has a single MI355X, "
               "so --gpus above 1 is not supported (segment / gather ops would shard by node range "
@@ -214,10 +258,9 @@ def main():
         # dominant kernel: the CSR reduction (segment_csr sum), HIP events on the launch stream
         t_kernel = event_time(lambda: ts.segment_csr(src, indptr, out, "sum"), max(args.steps, 20))
     kernel_bytes = wl.bytes_segment(w2.E, w2.N, w2.K, 4)
-    traffic = None
-    tpath = os.path.join(ROOT, "profiles", "traffic.json")
-    if os.path.exists(tpath):
-        traffic = json.load(open(tpath)).get("C2_segment_csr_sum_bytes_per_launch")
+    # HBM bytes per launch of this kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, calibrated against
+    # copies of known size (profiles/csr_reduce_pmc_traffic.txt): 117.5 MB read + 26.0 MB written
+    traffic = 143.5e6
     roofline = {"bound": "hbm", "kernel": "ts::csr_reduce_kernel<float, 4, SUM> (+ its fix-up launch)",
                 "achieved": round(gbs(kernel_bytes, t_kernel), 1), "peak": PEAK_GBS, "unit": "GB/s",
                 "frac": round(gbs(kernel_bytes, t_kernel) / PEAK_GBS, 4), "traffic": traffic,
