@@ -150,7 +150,7 @@ int ts_gather_csr(const void *src, const int64_t *indptr, void *out, int64_t B, 
   if (!valid_dtype(dtype) || !sizes_ok(B, N, E, K)) return TS_ERR_BAD_ARG;
   if (B * E * K == 0 || N == 0) return TS_OK;
   if (!src || !indptr || !out) return TS_ERR_BAD_ARG;
-  const CsrPlan p = csr_plan(N, E, K, kElemBytes[dtype], aligned16(src) && aligned16(out));
+  const CsrPlan p = csr_plan(N, E, K, kElemBytes[dtype], aligned16(src) && aligned16(out), true);
   CsrGatherArgs a;
   a.src = src;
   a.indptr = indptr;
@@ -173,7 +173,7 @@ int ts_segment_mean_csr_backward(const void *grad_out, const int64_t *indptr, vo
   if (!is_float_dtype(dtype)) return TS_ERR_UNSUPPORTED;
   if (B * E * K == 0 || N == 0) return TS_OK;
   if (!grad_out || !indptr || !grad_in) return TS_ERR_BAD_ARG;
-  const CsrPlan p = csr_plan(N, E, K, kElemBytes[dtype], aligned16(grad_out) && aligned16(grad_in));
+  const CsrPlan p = csr_plan(N, E, K, kElemBytes[dtype], aligned16(grad_out) && aligned16(grad_in), true);
   CsrGatherArgs a;
   a.src = grad_out;
   a.indptr = indptr;
@@ -294,9 +294,36 @@ int ts_scatter_count(const int64_t *index, float *count, int64_t B, int64_t E, i
   if (!count || (B * E > 0 && !index)) return TS_ERR_BAD_ARG;
   hipStream_t s = static_cast<hipStream_t>(stream);
   hipLaunchKernelGGL(fill_kernel<float>, dim3(grid_for(B * N)), dim3(kBlock), 0, s, count, B * N, 0.0f);
-  if (B * E > 0)
-    hipLaunchKernelGGL(scatter_count_kernel, dim3(grid_for(B * E)), dim3(kBlock), 0, s, index, count, B, E,
-                       N, index_stride_b, index_stride_e);
+  if (B * E > 0) {
+    // a sum of ones with K = 1: same kernels as scatter sum (src == nullptr adds 1.0 per entry)
+    ScatterArgs a;
+    a.src = nullptr;
+    a.index = index;
+    a.out = count;
+    a.arg_out = nullptr;
+    a.B = B;
+    a.E = E;
+    a.K = 1;
+    a.N = N;
+    a.sb = index_stride_b;
+    a.se = index_stride_e;
+    a.sk = 0;
+    a.out_given = 1;
+    a.precheck = 1;
+    a.lds_cache = env_int("TS_SCATTER_LDS", 1);
+    a.lds_epb = env_int("TS_SCATTER_EPB", 0);
+    const bool contended = a.lds_cache == 2 || (a.lds_cache == 1 && B * E >= ((int64_t)1 << 20) && B * E >= 32 * B * N);
+    if (contended && B * N < 0x7FFFFFFFll) {
+      int64_t epb = a.lds_epb > 0 ? a.lds_epb : ((int64_t)1 << 15);
+      if (a.lds_epb <= 0)
+        while (epb > 256 && B * E / epb < 2048) epb /= 2;
+      hipLaunchKernelGGL(scatter_add_lds_kernel<float>, dim3((unsigned)((B * E + epb - 1) / epb)), dim3(kLdsBlock), 0,
+                         s, a, kLdsAccRows - 1, epb);
+    } else {
+      hipLaunchKernelGGL(scatter_count_kernel, dim3(grid_for(B * E)), dim3(kBlock), 0, s, index, count, B, E, N,
+                         index_stride_b, index_stride_e);
+    }
+  }
   return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
 }
 

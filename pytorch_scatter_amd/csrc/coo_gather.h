@@ -8,6 +8,8 @@
 // vector L1 / L2 rather than from HBM.
 #pragma once
 
+#include <stdlib.h>
+
 #include "device_utils.h"
 
 namespace ts {
@@ -41,21 +43,29 @@ __global__ __launch_bounds__(kBlock) void coo_gather_kernel(CooGatherArgs a) {
   const int64_t e0 = ((int64_t)blockIdx.x * W + w) * a.epw;
   int64_t e1 = e0 + a.epw;
   if (e1 > a.E) e1 = a.E;
-  for (int64_t e = e0; e < e1; e += U) {
-    int64_t n[U];
+  if (e0 >= e1) return;
+  // software pipeline on the index: the indices of batch i+1 are in flight while
+  // the rows of batch i are fetched and stored
+  auto load_idx = [&](int64_t *n, int64_t e) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      int64_t ee = e + u < e1 ? e + u : e1 - 1;
-      int64_t v = idx[ee];
-      // an index outside [0, N) must not read out of bounds
-      n[u] = v < 0 ? 0 : (v >= a.N ? a.N - 1 : v);
+      const int64_t ee = e + u < e1 ? e + u : e1 - 1;
+      n[u] = idx[ee];
     }
+  };
+  int64_t n[U];
+  load_idx(n, e0);
+  for (int64_t e = e0; e < e1; e += U) {
+    int64_t nn[U];
+    load_idx(nn, e + U < e1 ? e + U : e);
     Vec<T, VEC> x[U];
     T c[U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      x[u] = load_vec<T, VEC>(src_b + n[u] * a.K + col);
-      if (DIV) c[u] = cnt_b[n[u]];
+      // an index outside [0, N) must not read out of bounds
+      const int64_t r = n[u] < 0 ? 0 : (n[u] >= a.N ? a.N - 1 : n[u]);
+      x[u] = load_vec<T, VEC>(src_b + r * a.K + col);
+      if (DIV) c[u] = cnt_b[r];
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -67,6 +77,8 @@ __global__ __launch_bounds__(kBlock) void coo_gather_kernel(CooGatherArgs a) {
         store_vec_stream<T, VEC>(out_b + (e + u) * a.K + col, x[u]);
       }
     }
+#pragma unroll
+    for (int u = 0; u < U; ++u) n[u] = nn[u];
   }
 }
 
@@ -85,7 +97,8 @@ inline CooGatherPlan coo_gather_plan(int64_t E, int64_t K, int elem_bytes, bool 
   p.G = G;
   p.ychunks = (int)((K + (int64_t)G * p.vec - 1) / ((int64_t)G * p.vec));
   const int W = kBlock / G;
-  p.epw = E >= (1 << 22) ? 32 : (E >= (1 << 18) ? 16 : 8);
+  p.epw = 8;  // measured best from 0.5 M to 62 M edges: short ranges keep more workgroups in flight
+  if (const char *env = getenv("TS_COO_EPW")) p.epw = atoi(env) > 0 ? atoi(env) : p.epw;  // tuning aid
   const int64_t per_block = (int64_t)W * p.epw;
   p.nblk = (E + per_block - 1) / per_block;
   if (p.nblk < 1) p.nblk = 1;

@@ -80,7 +80,7 @@ __device__ __forceinline__ void finalize_row(const CsrReduceArgs &a, T *out_b, i
     if (REDUCE == TS_SUM || REDUCE == TS_MEAN) {
       if (a.accumulate) x = to_acc<T>(prev.v[v]) + x;
       T t = from_acc<T>(x);
-      if (REDUCE == TS_MEAN) t = div_elem<T>(t, count_as<T>(count > 0 ? count : 1));
+      if (REDUCE == TS_MEAN && count > 1) t = div_elem<T>(t, count_as<T>(count));  // x / 1 == x
       o.v[v] = t;
     } else {
       if (a.accumulate) {
@@ -401,7 +401,7 @@ struct CsrPlan {
   int ychunks;   // column chunks
 };
 
-inline CsrPlan csr_plan(int64_t N, int64_t E, int64_t K, int elem_bytes, bool aligned16) {
+inline CsrPlan csr_plan(int64_t N, int64_t E, int64_t K, int elem_bytes, bool aligned16, bool expand = false) {
   CsrPlan p;
   const int full = kVecBytes / elem_bytes;
   p.vec = (aligned16 && full > 1 && K % full == 0) ? full : 1;
@@ -416,10 +416,13 @@ inline CsrPlan csr_plan(int64_t N, int64_t E, int64_t K, int elem_bytes, bool al
   // same HBM channels and costs ~15 % of the read bandwidth.
   const int W = kBlock / G;
   const int cap = kMaxBlockItems / W;  // LDS holds the row pointers of one tile
-  int want = items >= ((int64_t)8 << 20) ? 120 : (items >= ((int64_t)1 << 20) ? 56 : 24);
+  // measured: reductions like 40 / 56 / 120 items per worker as the input grows; the write-bound
+  // expansion likes short ranges (16) until the grid is large anyway
+  int want = items >= ((int64_t)8 << 20) ? 120 : (items >= ((int64_t)1 << 20) ? 56 : 40);
+  if (expand && items < ((int64_t)8 << 20)) want = 16;
   if (const char *env = getenv("TS_CSR_IPW")) want = atoi(env);  // tuning aid
   if (want > cap) want = cap;
-  int ipw = want >= 8 ? (((want / 8) - 1) | 1) * 8 + 0 : (want | 1);
+  int ipw = want >= 24 ? (((want / 8) - 1) | 1) * 8 : want;
   if (ipw > cap) ipw = cap;
   if (ipw < 1) ipw = 1;
   p.ipw = ipw;

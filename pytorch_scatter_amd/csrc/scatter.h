@@ -480,6 +480,75 @@ __global__ __launch_bounds__(kLdsBlock) void scatter_key_lds_kernel(ScatterArgs 
   }
 }
 
+// ---- sum with a workgroup-private accumulator table ------------------------------
+// Same idea as the packed-key table above, for additions: a hub node that owns
+// 20 % of the entries would otherwise put two million atomics on one address
+// (measured: 29 ms for 10 M entries). Rows of fp32 accumulators are claimed per
+// node in LDS (ds_add_f32), written back with one global atomic per touched
+// element and chunk. 16-bit inputs gain accuracy on the way (fp32 partial sums,
+// one rounding per chunk instead of one per entry). src == nullptr adds 1.0 per
+// entry (the count of scatter mean).
+constexpr int kLdsAcc = 8192;         // 32 KB of fp32 accumulators
+constexpr int kLdsAccRows = 4096;     // 16 KB of tags
+
+template <typename T>
+__global__ __launch_bounds__(kLdsBlock) void scatter_add_lds_kernel(ScatterArgs a, int tn_mask, int64_t epb) {
+  constexpr int U = 4;
+  __shared__ float s_acc[kLdsAcc];
+  __shared__ int32_t s_tags[kLdsAccRows];
+  const int K = (int)a.K;
+  const int tn = tn_mask + 1;
+  for (int i = threadIdx.x; i < tn * K; i += kLdsBlock) s_acc[i] = 0.0f;
+  for (int i = threadIdx.x; i < tn; i += kLdsBlock) s_tags[i] = -1;
+  __syncthreads();
+
+  const T *src = static_cast<const T *>(a.src);
+  T *out = static_cast<T *>(a.out);
+  const EdgeLanes m = edge_lanes(K, kLdsBlock);
+  const int64_t be_lo = (int64_t)blockIdx.x * epb;
+  int64_t be_hi = be_lo + epb;
+  if (be_hi > a.B * a.E) be_hi = a.B * a.E;
+
+  if (m.active) {
+    for (int64_t be0 = be_lo + m.el; be0 < be_hi; be0 += (int64_t)m.epp * U) {
+      for (int k = m.cl; k < K; k += m.L) {
+        float x[U];
+        int64_t idx[U], bb[U], ee[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const int64_t be = be0 + (int64_t)u * m.epp;
+          split_edge(be < be_hi ? be : be0, a.B, a.E, bb[u], ee[u]);
+          x[u] = src ? (float)to_acc<T>(src[(bb[u] * a.E + ee[u]) * a.K + k]) : 1.0f;
+          idx[u] = a.index[bb[u] * a.sb + ee[u] * a.se];
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          if (be0 + (int64_t)u * m.epp >= be_hi) continue;
+          if (idx[u] < 0 || idx[u] >= a.N) continue;
+          const int node = (int)(bb[u] * a.N + idx[u]);
+          const int row = node & tn_mask;
+          int tag = s_tags[row];
+          if (tag == -1) {
+            const int old = atomicCAS(&s_tags[row], -1, node);
+            tag = old == -1 ? node : old;
+          }
+          if (tag == node)
+            __hip_atomic_fetch_add(&s_acc[row * K + k], x[u], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+          else
+            atomic_add_elem<T>(out + (int64_t)node * a.K + k, from_acc<T>((typename Acc<T>::type)x[u]));
+        }
+      }
+    }
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < tn * K; i += kLdsBlock) {
+    const float v = s_acc[i];
+    if (v == 0.0f) continue;
+    const int row = i / K;
+    atomic_add_elem<T>(out + (int64_t)s_tags[row] * a.K + (i - row * K), from_acc<T>((typename Acc<T>::type)v));
+  }
+}
+
 template <typename T, bool IS_MAX>
 __global__ __launch_bounds__(kBlock) void scatter_key_final_kernel(ScatterArgs a) {
   const int64_t n = a.B * a.N * a.K;
@@ -596,6 +665,22 @@ int launch_scatter_v(const ScatterArgs &a, int reduce, hipStream_t stream) {
       // (4 lines per instruction for fp32 instead of 16 with 4 elements per lane)
       const unsigned g = scatter_grid(n_edges, a.K, kBlock, 4);
       if (reduce == TS_SUM) {
+        if constexpr (__is_same(T, float) || __is_same(T, bf16_t) || __is_same(T, f16_t)) {
+          // many entries per output slot: reduce in LDS first (see scatter_add_lds_kernel)
+          int tn = 1;
+          while ((int64_t)tn * 2 * a.K <= kLdsAcc && tn * 2 <= kLdsAccRows) tn *= 2;
+          const bool use_lds = a.lds_cache && a.sk == 0 && tn >= 64 && a.B * a.N < 0x7FFFFFFFll &&
+                               (a.lds_cache == 2 || (n_src >= ((int64_t)1 << 20) && n_edges >= 32 * a.B * a.N));
+          if (use_lds) {
+            int64_t epb = a.lds_epb > 0 ? a.lds_epb : ((int64_t)1 << 15) / a.K;
+            if (a.lds_epb <= 0)
+              while (epb > 256 && n_edges / epb < 2048) epb /= 2;
+            if (epb < 64) epb = 64;
+            hipLaunchKernelGGL(scatter_add_lds_kernel<T>, dim3((unsigned)((n_edges + epb - 1) / epb)),
+                               dim3(kLdsBlock), 0, stream, a, tn - 1, epb);
+            return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
+          }
+        }
         if constexpr (__is_same(T, bf16_t) || __is_same(T, f16_t)) {
           if (a.K % 2 == 0 && a.sk == 0 && (reinterpret_cast<uintptr_t>(a.out) & 3) == 0 &&
               (reinterpret_cast<uintptr_t>(a.src) & 3) == 0) {

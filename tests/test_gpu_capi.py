@@ -351,6 +351,38 @@ def test_scatter_minmax_lds_cached_variant(capi, oracle, shape, reduce, dtype, m
         assert_exact(arg, want_arg)
 
 
+@pytest.mark.parametrize("shape,dtype", product(
+    [(1, 30000, 1, 500), (1, 9000, 32, 300), (2, 5000, 8, 40), (1, 4000, 12, 70000)],
+    [torch.float32, torch.bfloat16, torch.float16]))
+def test_scatter_sum_lds_aggregated_variant(capi, oracle, shape, dtype, monkeypatch):
+    """Sum through the workgroup-private accumulator table (forced on), skewed index;
+    also the count entry point, which shares the kernel."""
+    monkeypatch.setenv("TS_SCATTER_LDS", "2")
+    monkeypatch.setenv("TS_SCATTER_EPB", "700")
+    B, E, K, N = shape
+    rng = np.random.default_rng(E + K)
+    src = torch.from_numpy(rng.standard_normal(size=(B, E, K))).to(dtype)
+    p = np.arange(1, N + 1, dtype=np.float64) ** -1.2
+    index1 = torch.from_numpy(rng.choice(N, size=E, p=p / p.sum()))
+    index = index1.view(1, E, 1).expand(B, E, K)
+    exact = oracle.scatter(src.double(), index, 1, None, N, "sum")[0]
+    absum = oracle.scatter(src.double().abs(), index, 1, None, N, "sum")[0]
+    for out_given in (False, True):
+        prev = torch.from_numpy(rng.standard_normal(size=(B, N, K))).to(dtype)
+        out = prev.clone().to(DEV) if out_given else torch.empty((B, N, K), dtype=dtype, device=DEV)
+        capi.scatter(src.to(DEV), index1.to(DEV), out, None, B, E, K, N, 0, 1, 0, capi.SUM, out_given)
+        torch.cuda.synchronize()
+        want = exact + (prev.double() if out_given else 0)
+        rtol = 1e-5 if dtype == torch.float32 else 1e-2
+        err = (out.cpu().double() - want).abs()
+        bound = rtol * want.abs() + rtol * (absum + (prev.double().abs() if out_given else 0)).clamp(min=1e-30)
+        assert bool((err <= bound).all()), float((err - bound).max())
+    cnt = torch.empty((N,), dtype=torch.float32, device=DEV)
+    capi.scatter_count(index1.to(DEV), cnt, 1, E, N, 0, 1)
+    torch.cuda.synchronize()
+    assert torch.equal(cnt.cpu(), torch.bincount(index1, minlength=N).float())
+
+
 @pytest.mark.parametrize("reduce,dtype", product(["sum", "min", "max"], [torch.float32, torch.float64, torch.int64]))
 def test_scatter_out_given_and_wide_types(capi, oracle, reduce, dtype):
     B, E, K, N = 2, 3000, 6, 40
