@@ -380,11 +380,11 @@ __global__ __launch_bounds__(kBlock) void scatter_key_kernel(ScatterArgs a) {
 constexpr int kLdsKeys = 4096;        // 32 KB of 64-bit keys
 constexpr int kLdsBlock = 256;  // 3 workgroups per CU (LDS-limited) at <= 168 VGPRs
 
-template <typename T, int VEC, bool IS_MAX>
-__global__ __launch_bounds__(kLdsBlock) void scatter_key_lds_kernel(ScatterArgs a, int tn_mask, int64_t epb) {
+template <typename T, int VEC, bool IS_MAX, int TAGS>
+__global__ __launch_bounds__(kLdsBlock, (TAGS <= 256 ? 4 : 1)) void scatter_key_lds_kernel(ScatterArgs a, int tn_mask, int64_t epb) {
   constexpr int U = VEC == 1 ? 8 : 4;
   __shared__ uint64_t s_keys[kLdsKeys];
-  __shared__ int32_t s_tags[kLdsKeys];
+  __shared__ int32_t s_tags[TAGS];  // TAGS >= table rows: kLdsKeys for narrow rows, 256 for K >= 16
   const int K = (int)a.K;
   const int tn = tn_mask + 1;
   for (int i = threadIdx.x; i < tn * K; i += kLdsBlock) s_keys[i] = 0;
@@ -733,9 +733,12 @@ int launch_scatter_v(const ScatterArgs &a, int reduce, hipStream_t stream) {
       if (is_max) {
         hipLaunchKernelGGL((scatter_key_init_kernel<T, true>), dim3(g_out), dim3(kBlock), 0, stream, a);
         if (n_src > 0) {
-          if (use_lds)
-            hipLaunchKernelGGL((scatter_key_lds_kernel<T, VEC, true>), dim3(g_lds), dim3(kLdsBlock), 0, stream, a,
-                               tn - 1, epb);
+          if (use_lds && tn <= 256)
+            hipLaunchKernelGGL((scatter_key_lds_kernel<T, VEC, true, 256>), dim3(g_lds), dim3(kLdsBlock), 0, stream,
+                               a, tn - 1, epb);
+          else if (use_lds)
+            hipLaunchKernelGGL((scatter_key_lds_kernel<T, VEC, true, kLdsKeys>), dim3(g_lds), dim3(kLdsBlock), 0,
+                               stream, a, tn - 1, epb);
           else
             hipLaunchKernelGGL((scatter_key_kernel<T, VEC, true>), dim3(g_key), dim3(kBlock), 0, stream, a);
         }
@@ -743,9 +746,12 @@ int launch_scatter_v(const ScatterArgs &a, int reduce, hipStream_t stream) {
       } else {
         hipLaunchKernelGGL((scatter_key_init_kernel<T, false>), dim3(g_out), dim3(kBlock), 0, stream, a);
         if (n_src > 0) {
-          if (use_lds)
-            hipLaunchKernelGGL((scatter_key_lds_kernel<T, VEC, false>), dim3(g_lds), dim3(kLdsBlock), 0, stream, a,
-                               tn - 1, epb);
+          if (use_lds && tn <= 256)
+            hipLaunchKernelGGL((scatter_key_lds_kernel<T, VEC, false, 256>), dim3(g_lds), dim3(kLdsBlock), 0, stream,
+                               a, tn - 1, epb);
+          else if (use_lds)
+            hipLaunchKernelGGL((scatter_key_lds_kernel<T, VEC, false, kLdsKeys>), dim3(g_lds), dim3(kLdsBlock), 0,
+                               stream, a, tn - 1, epb);
           else
             hipLaunchKernelGGL((scatter_key_kernel<T, VEC, false>), dim3(g_key), dim3(kBlock), 0, stream, a);
         }
