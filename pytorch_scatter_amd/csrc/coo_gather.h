@@ -74,6 +74,7 @@ __global__ __launch_bounds__(kBlock) void coo_gather_kernel(CooGatherArgs a) {
 #pragma unroll
           for (int v = 0; v < VEC; ++v) x[u].v[v] = div_elem<T>(x[u].v[v], c[u]);
         }
+        // streaming stores keep the source rows (re-read by neighbouring edges) in cache
         store_vec_stream<T, VEC>(out_b + (e + u) * a.K + col, x[u]);
       }
     }
