@@ -317,3 +317,56 @@ def test_errors_follow_reference_conventions(ts):
         ts.gather_csr(src, torch.tensor([0, 3, 6], device=DEV))
     with pytest.raises(RuntimeError, match="must be CUDA tensor"):
         ts.scatter_sum(src, torch.tensor([0, 1, 0, 1, 2, 2]), 0)
+
+
+def test_ops_on_a_side_stream_and_in_a_hip_graph(ts, oracle):
+    """Launches go to the caller's current stream and nothing allocates outside the
+    caching allocator or synchronises (with `out` / `dim_size` given), so a step
+    can be captured into a HIP graph; every replay is checked against eager."""
+    rng = np.random.default_rng(3)
+    indptr_c, index_c = random_csr(rng, 4000, 30)
+    E = index_c.numel()
+    indptr, index = indptr_c.to(DEV), index_c.to(DEV)
+    perm = torch.from_numpy(rng.permutation(E)).to(DEV)
+    src = torch.randn(E, 32, device=DEV)
+    out_mean = torch.empty(4000, 32, device=DEV)
+    back = torch.empty(E, 32, device=DEV)
+
+    def step():
+        ts.segment_csr(src, indptr, out_mean, "mean")
+        ts.gather_csr(out_mean, indptr, back)
+        mx, arg = ts.scatter_max(back[perm], index[perm], 0, None, 4000)
+        sm = ts.segment_coo(src, index, None, 4000, "sum")
+        return mx, arg, sm
+
+    # side stream
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side), torch.no_grad():
+        mx_s, arg_s, sm_s = step()
+    side.synchronize()
+    with torch.no_grad():
+        mx_e, arg_e, sm_e = step()
+    torch.cuda.synchronize()
+    want_mean, _ = oracle.segment_csr(src.cpu(), indptr_c, None, "mean")
+    assert torch.allclose(out_mean.cpu(), want_mean, rtol=1e-5, atol=1e-5)
+    assert torch.equal(mx_s, mx_e) and torch.equal(arg_s, arg_e) and torch.equal(sm_s, sm_e)
+
+    # graph capture and replays with changing inputs
+    g = torch.cuda.CUDAGraph()
+    with torch.no_grad():
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            step()  # warm-up on the capture stream
+        torch.cuda.current_stream().wait_stream(side)
+        with torch.cuda.graph(g):
+            mx_g, arg_g, sm_g = step()
+        for i in range(3):
+            src.copy_(torch.randn(E, 32, device=DEV))
+            g.replay()
+            torch.cuda.synchronize()
+            got = (mx_g.clone(), arg_g.clone(), sm_g.clone(), out_mean.clone())
+            mx_e, arg_e, sm_e = step()
+            torch.cuda.synchronize()
+            assert torch.equal(got[0], mx_e) and torch.equal(got[1], arg_e), i
+            assert torch.equal(got[2], sm_e) and torch.equal(got[3], out_mean), i
