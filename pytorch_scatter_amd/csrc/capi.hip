@@ -314,9 +314,7 @@ int ts_scatter_count(const int64_t *index, float *count, int64_t B, int64_t E, i
     a.lds_epb = env_int("TS_SCATTER_EPB", 0);
     const bool contended = a.lds_cache == 2 || (a.lds_cache == 1 && B * E >= ((int64_t)1 << 20) && B * E >= 32 * B * N);
     if (contended && B * N < 0x7FFFFFFFll) {
-      int64_t epb = a.lds_epb > 0 ? a.lds_epb : ((int64_t)1 << 15);
-      if (a.lds_epb <= 0)
-        while (epb > 256 && B * E / epb < 2048) epb /= 2;
+      const int64_t epb = lds_chunk_edges(a.lds_epb, 1, B * E);
       hipLaunchKernelGGL(scatter_add_lds_kernel<float>, dim3((unsigned)((B * E + epb - 1) / epb)), dim3(kLdsBlock), 0,
                          s, a, kLdsAccRows - 1, epb);
     } else {
