@@ -419,7 +419,7 @@ inline CsrPlan csr_plan(int64_t N, int64_t E, int64_t K, int elem_bytes, bool al
   // measured: reductions like 40 / 56 / 120 items per worker as the input grows; the write-bound
   // expansion likes short ranges at every size (a workgroup then writes ~100 KB and retires)
   int want = items >= ((int64_t)8 << 20) ? 120 : (items >= ((int64_t)1 << 20) ? 56 : 40);
-  if (expand) want = 24;
+  if (expand) want = items >= ((int64_t)32 << 20) ? 8 : 24;
   if (const char *env = getenv("TS_CSR_IPW")) want = atoi(env);  // tuning aid
   if (want > cap) want = cap;
   int ipw = want >= 24 ? (((want / 8) - 1) | 1) * 8 : want;
