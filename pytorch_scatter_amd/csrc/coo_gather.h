@@ -1,11 +1,11 @@
 // out[b, e, :] = src[b, index[b, e], :]   (gather_coo) and the fused backward
 // of segment_coo(mean), which divides the gathered row by count[index].
 //
-// Edges are independent, so the split is a plain even one: each worker (G
-// lanes holding one 16-byte-per-lane slice of a row) takes `epw` consecutive
-// edges and keeps U index loads, then U row loads, in flight. A sorted index
-// makes consecutive edges hit the same source row, which then comes from the
-// vector L1 / L2 rather than from HBM.
+// Edges are independent, so the split is a plain even one: a workgroup takes
+// W * epw consecutive edges, its workers (G lanes holding one 16-byte-per-lane
+// slice of a row) interleave over them and keep U index loads, then U row
+// loads, in flight. A sorted index makes neighbouring edges hit the same source
+// row, which then comes from the vector L1 / L2 rather than from HBM.
 #pragma once
 
 #include <stdlib.h>
@@ -40,24 +40,28 @@ __global__ __launch_bounds__(kBlock) void coo_gather_kernel(CooGatherArgs a) {
   const T *cnt_b = DIV ? static_cast<const T *>(a.count) + b * a.N : nullptr;
   T *out_b = static_cast<T *>(a.out) + b * a.E * a.K;
 
-  const int64_t e0 = ((int64_t)blockIdx.x * W + w) * a.epw;
-  int64_t e1 = e0 + a.epw;
-  if (e1 > a.E) e1 = a.E;
-  if (e0 >= e1) return;
+  // Workers of a workgroup interleave: worker w takes edges base + w, base + w + W, ... so that one
+  // wavefront instruction covers 64 / G consecutive edges (contiguous in out, and in src for a sorted index).
+  const int64_t base = (int64_t)blockIdx.x * W * a.epw;
+  int64_t blk_end = base + (int64_t)W * a.epw;
+  if (blk_end > a.E) blk_end = a.E;
+  const int64_t e0 = base + w;
+  if (e0 >= blk_end) return;
+  const int64_t e_last = e0 + ((blk_end - 1 - e0) / W) * W;  // last edge of this worker
   // software pipeline on the index: the indices of batch i+1 are in flight while
   // the rows of batch i are fetched and stored
   auto load_idx = [&](int64_t *n, int64_t e) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const int64_t ee = e + u < e1 ? e + u : e1 - 1;
+      const int64_t ee = e + (int64_t)u * W <= e_last ? e + (int64_t)u * W : e_last;
       n[u] = idx[ee];
     }
   };
   int64_t n[U];
   load_idx(n, e0);
-  for (int64_t e = e0; e < e1; e += U) {
+  for (int64_t e = e0; e <= e_last; e += (int64_t)U * W) {
     int64_t nn[U];
-    load_idx(nn, e + U < e1 ? e + U : e);
+    load_idx(nn, e + (int64_t)U * W <= e_last ? e + (int64_t)U * W : e);
     Vec<T, VEC> x[U];
     T c[U];
 #pragma unroll
@@ -69,13 +73,14 @@ __global__ __launch_bounds__(kBlock) void coo_gather_kernel(CooGatherArgs a) {
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      if (e + u < e1) {
+      const int64_t eu = e + (int64_t)u * W;
+      if (eu <= e_last) {
         if (DIV) {
 #pragma unroll
           for (int v = 0; v < VEC; ++v) x[u].v[v] = div_elem<T>(x[u].v[v], c[u]);
         }
         // streaming stores keep the source rows (re-read by neighbouring edges) in cache
-        store_vec_stream<T, VEC>(out_b + (e + u) * a.K + col, x[u]);
+        store_vec_stream<T, VEC>(out_b + eu * a.K + col, x[u]);
       }
     }
 #pragma unroll
