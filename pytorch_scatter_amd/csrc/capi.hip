@@ -282,6 +282,7 @@ int ts_scatter(const void *src, const int64_t *index, void *out, int64_t *arg_ou
   a.precheck = env_int("TS_SCATTER_PRECHECK", 1);   // tuning aids
   a.lds_cache = env_int("TS_SCATTER_LDS", 1);
   a.lds_epb = env_int("TS_SCATTER_EPB", 0);
+  a.run_reduce = env_int("TS_SCATTER_RUNS", 1);
   const int full = kVecBytes / kElemBytes[dtype];
   const int vec = (full > 1 && K % full == 0 && aligned16(src)) ? full : 1;
   return dispatch_scatter(dtype, a, reduce, vec, static_cast<hipStream_t>(stream));
@@ -317,6 +318,12 @@ int ts_scatter_count(const int64_t *index, float *count, int64_t B, int64_t E, i
       const int64_t epb = lds_chunk_edges(a.lds_epb, 1, B * E);
       hipLaunchKernelGGL(scatter_add_lds_kernel<float>, dim3((unsigned)((B * E + epb - 1) / epb)), dim3(kLdsBlock), 0,
                          s, a, kLdsAccRows - 1, epb);
+    } else if (env_int("TS_SCATTER_RUNS", 1) && B * N < 0x7FFFFFFFll) {
+      // runs of equal neighbouring indices (sorted input) are counted in the wavefront first
+      const int rpw = run_rows_per_wave(B * E, kWave);
+      const int64_t waves = (B * E + (int64_t)rpw * kWave - 1) / ((int64_t)rpw * kWave);
+      const int64_t blocks = (waves + kBlock / kWave - 1) / (kBlock / kWave);
+      hipLaunchKernelGGL((scatter_add_run_kernel<float, 1>), dim3((unsigned)blocks), dim3(kBlock), 0, s, a, 0, rpw);
     } else {
       hipLaunchKernelGGL(scatter_count_kernel, dim3(grid_for(B * E)), dim3(kBlock), 0, s, index, count, B, E, N,
                          index_stride_b, index_stride_e);

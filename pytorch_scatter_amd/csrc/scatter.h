@@ -22,6 +22,7 @@
 #pragma once
 
 #include <limits>
+#include <stdlib.h>
 
 #include "device_utils.h"
 
@@ -166,6 +167,7 @@ struct ScatterArgs {
   int precheck;        // read before the atomic: 0 none, 1 cached, 2 device-coherent, 3 streaming
   int lds_cache;       // reduce hot slots in LDS first: 0 never, 1 for large inputs, 2 always
   int64_t lds_epb;     // entries per workgroup chunk of that variant, 0 = default
+  int run_reduce = 1;  // sum: pre-reduce runs of equal neighbouring indices in the wavefront
 };
 
 // ---- thread -> (edge, column) mapping shared by the scatter kernels ------------
@@ -274,6 +276,231 @@ __global__ __launch_bounds__(kBlock) void scatter_add_pk16_kernel(ScatterArgs a)
   }
 }
 
+// ---- wavefront pre-reduction of equal neighbouring indices -------------------------
+// Message-passing indices are sorted or nearly so: neighbouring entries address the
+// same output row, and one atomic per element would serialise them on one cache
+// line. Here a wavefront owns a contiguous range of entries and reads it row by
+// row (64 / L entries of L lanes each, C columns = up to 16 bytes per lane, fully
+// coalesced). Runs of equal node ids inside a row are combined across lanes with
+// shuffles; the run that reaches the end of a row is carried in registers into the
+// next row instead of being written, so a run of any length costs one atomic per
+// element and wavefront. An index without repeats degenerates to one atomic per
+// element. Finished runs go through a per-wavefront LDS buffer so that the atomics
+// of one instruction fall on consecutive addresses (whole cache lines) although a
+// lane holds C neighbouring columns. One index per row (sk == 0) and B * N < 2^31
+// are required.
+//
+// The policy P supplies the value type and its operations:
+//   P::A, P::C, P::EW          accumulator type, columns per lane, columns per atomic
+//   load(e, pos, col, x)       x[0..C) = columns col.. of entry e (position pos inside its batch)
+//   combine(x, y)              x = x (op) y, one column
+//   identity()
+//   emit(node, col, x)         combine EW columns x[0..EW) into the output slot with one atomic
+template <typename P>
+__device__ __forceinline__ void run_reduce_wave(const ScatterArgs &a, const int lshift, const int rows_per_wave,
+                                                const P &p, typename P::A *stage) {
+  typedef typename P::A A;
+  constexpr int U = P::U;
+  constexpr int C = P::C;
+  constexpr int EW = P::EW;
+  constexpr int cshift = C == 1 ? 0 : (C == 2 ? 1 : (C == 4 ? 2 : (C == 8 ? 3 : 4)));
+  static_assert((1 << cshift) == C && C % EW == 0, "");
+  const int lane = threadIdx.x & (kWave - 1);
+  const int L = 1 << lshift;       // lanes per entry
+  const int epr = kWave >> lshift; // entries per wavefront row
+  const int el = lane >> lshift;
+  const int cl = lane & (L - 1);
+  const int64_t colbase = (int64_t)blockIdx.y * (L * C);
+  const int64_t col = colbase + cl * C;
+  const bool col_ok = col < a.K;
+  const int64_t n_edges = a.B * a.E;
+  const int64_t wave = (int64_t)blockIdx.x * (kBlock / kWave) + (threadIdx.x / kWave);
+  const int64_t lo = wave * rows_per_wave * epr;
+  int64_t hi = lo + (int64_t)rows_per_wave * epr;
+  if (hi > n_edges) hi = n_edges;
+  if (lo >= hi) return;
+  // bit 0 of every entry slot of the wavefront
+  const uint64_t slot_bits = L == kWave ? 1ull : ~0ull / ((1ull << L) - 1ull);
+
+  // Write the slots named in `mask` (bit slot * L) to the output: node id per lane in n,
+  // values in v. Lanes re-read the values from LDS so that consecutive lanes hold
+  // consecutive columns of one slot.
+  auto write_slots = [&](const uint64_t mask, const int n, const A *v) {
+    if constexpr (C == EW) {  // one atomic per lane: consecutive lanes already hold consecutive columns
+      if (((mask >> (el << lshift)) & 1ull) && col_ok) p.emit(n, col, v);
+      return;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");  // earlier reads of the buffer are done
+#pragma unroll
+    for (int c = 0; c < C; ++c) stage[lane * C + c] = v[c];
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int it = 0; it < C / EW; ++it) {
+      const int f = (lane + kWave * it) * EW;          // element of the wavefront row
+      const int slot = f >> (lshift + cshift);
+      const int j = f & ((L << cshift) - 1);           // column inside the slot
+      const int node = __shfl(n, slot << lshift);
+      if (((mask >> (slot << lshift)) & 1ull) && colbase + j < a.K) p.emit(node, colbase + j, stage + f);
+    }
+  };
+
+  A carry[C];
+#pragma unroll
+  for (int c = 0; c < C; ++c) carry[c] = p.identity();
+  int carry_node = -1;
+
+  for (int64_t r0 = lo; r0 < hi; r0 += (int64_t)U * epr) {
+    int node[U];
+    A x[U][C];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int64_t e = r0 + (int64_t)u * epr + el;
+      const bool ok = e < hi;
+      const int64_t ec = ok ? e : hi - 1;
+      int64_t b, pos;
+      split_edge(ec, a.B, a.E, b, pos);
+      const int64_t idx = a.index[b * a.sb + pos * a.se];
+      node[u] = (ok && idx >= 0 && idx < a.N) ? (int)(b * a.N + idx) : -1;
+      p.load(ec, pos, col_ok ? col : 0, x[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (r0 + (int64_t)u * epr >= hi) break;  // uniform
+      const int n = node[u];
+      A v[C];
+#pragma unroll
+      for (int c = 0; c < C; ++c) v[c] = x[u][c];
+      // the run carried over from the previous row continues in slot 0, or is written now
+      const int n0 = __builtin_amdgcn_readfirstlane(n);
+      if (carry_node == n0) {
+        if (el == 0) {
+#pragma unroll
+          for (int c = 0; c < C; ++c) p.combine(v[c], carry[c]);
+        }
+      } else if (carry_node >= 0) {
+        write_slots(1ull, carry_node, carry);
+      }
+      int h_slot = 0;
+      if (epr > 1) {
+        const int prev = __shfl_up(n, L);
+        const bool head = (el == 0) || (n != prev);
+        const uint64_t hm = __ballot(head) & slot_bits;
+        // slots from this one to the end of its run
+        const uint64_t after = (el + 1 < epr) ? (hm >> ((el + 1) << lshift)) : 0ull;
+        const int rem = after ? ((__ffsll((unsigned long long)after) - 1) >> lshift) + 1 : epr - el;
+        if (hm != slot_bits) {  // a row without equal neighbours has nothing to combine
+          for (int d = 1; d < epr; d <<= 1) {
+#pragma unroll
+            for (int c = 0; c < C; ++c) {
+              const A t = __shfl_down(v[c], d << lshift);
+              if (d < rem) p.combine(v[c], t);
+            }
+          }
+        }
+        h_slot = (63 - __clzll((long long)hm)) >> lshift;  // head of the last run of the row
+        // heads of finished runs with a valid node
+        const uint64_t em = __ballot(head && el != h_slot && n >= 0) & slot_bits;
+        if (em != 0) write_slots(em, n, v);
+      }
+      carry_node = __shfl(n, h_slot << lshift);
+#pragma unroll
+      for (int c = 0; c < C; ++c) carry[c] = __shfl(v[c], (h_slot << lshift) + cl);
+    }
+  }
+  if (carry_node >= 0) write_slots(1ull, carry_node, carry);
+}
+
+// sum: up to 16 bytes per lane; 16-bit floats accumulate in fp32 and are written
+// with the packed-pair atomic. src == nullptr adds 1 per entry (the count of scatter mean).
+template <typename T, int C_>
+struct AddRun {
+  typedef typename Acc<T>::type A;
+  static constexpr int C = C_;
+  static constexpr int EW = sizeof(T) == 2 ? 2 : 1;
+  static constexpr int U = 4;
+  const T *src;
+  T *out;
+  int64_t K;
+  __device__ A identity() const { return (A)0; }
+  __device__ void load(int64_t e, int64_t, int64_t col, A *x) const {
+    if (src == nullptr) {
+#pragma unroll
+      for (int c = 0; c < C; ++c) x[c] = (A)1;
+      return;
+    }
+    const Vec<T, C> r = load_vec_stream<T, C>(src + e * K + col);
+#pragma unroll
+    for (int c = 0; c < C; ++c) x[c] = to_acc<T>(r.v[c]);
+  }
+  __device__ void combine(A &x, const A &y) const { x = x + y; }
+  __device__ void emit(int node, int64_t col, const A *x) const {
+    T *p = out + (int64_t)node * K + col;
+#ifdef TS_RUN_NO_EMIT
+    if (node != 0x12345) return;
+#endif
+    if constexpr (EW == 2) {
+      if constexpr (__is_same(T, bf16_t)) {
+        typedef short v2s __attribute__((ext_vector_type(2)));
+        v2s pk;
+        pk.x = (short)float_to_bf16(x[0]).x;
+        pk.y = (short)float_to_bf16(x[1]).x;
+        __builtin_amdgcn_global_atomic_fadd_v2bf16(reinterpret_cast<v2s *>(p), pk);
+      } else {
+        typedef _Float16 v2h __attribute__((ext_vector_type(2)));
+        v2h pk;
+        pk.x = (_Float16)x[0];
+        pk.y = (_Float16)x[1];
+        __builtin_amdgcn_global_atomic_fadd_v2f16(reinterpret_cast<v2h *>(p), pk);
+      }
+    } else {
+      atomic_add_elem<T>(p, from_acc<T>(x[0]));
+    }
+  }
+};
+
+template <typename T, int C>
+__global__ __launch_bounds__(kBlock) void scatter_add_run_kernel(ScatterArgs a, int lshift, int rows_per_wave) {
+  typedef typename Acc<T>::type A;
+  __shared__ A s_stage[kBlock / kWave][kWave * C];
+  AddRun<T, C> p;
+  p.src = static_cast<const T *>(a.src);
+  p.out = static_cast<T *>(a.out);
+  p.K = a.K;
+  run_reduce_wave(a, lshift, rows_per_wave, p, s_stage[threadIdx.x / kWave]);
+}
+
+// rows of a wavefront in the kernel above: long enough to carry runs across rows, short enough to
+// leave ~8 K wavefronts
+inline int run_rows_per_wave(int64_t n_edges, int epr) {
+  const int64_t rows = (n_edges + epr - 1) / epr;
+  int64_t rpw = rows / 8192;
+  if (rpw > 32) rpw = 32;
+  if (rpw < 1) rpw = 1;
+  if (const char *env = getenv("TS_RUN_RPW")) rpw = atoi(env) > 0 ? atoi(env) : rpw;  // tuning aid
+  return (int)(rpw <= 4 ? rpw : (rpw + 3) / 4 * 4);
+}
+// launch shape of the run kernels for rows of `kc` lanes
+struct RunGrid {
+  int lshift, rpw;
+  unsigned blocks, ychunks;
+  bool ok;
+};
+inline RunGrid run_grid(int64_t n_edges, int64_t kc) {
+  RunGrid g;
+  g.lshift = 0;
+  while ((1 << g.lshift) < kc && g.lshift < 6) ++g.lshift;
+  const int L = 1 << g.lshift, epr = kWave >> g.lshift;
+  g.rpw = run_rows_per_wave(n_edges, epr);
+  const int64_t waves = (n_edges + (int64_t)g.rpw * epr - 1) / ((int64_t)g.rpw * epr);
+  const int64_t blocks = (waves + kBlock / kWave - 1) / (kBlock / kWave);
+  const int64_t ychunks = (kc + L - 1) / L;
+  g.ok = blocks < 0x7FFFFFFFll && ychunks <= 65535;
+  g.blocks = (unsigned)blocks;
+  g.ychunks = (unsigned)ychunks;
+  return g;
+}
+
 // ---- packed-key min/max -----------------------------------------------------
 template <typename T, bool IS_MAX>
 __global__ __launch_bounds__(kBlock) void scatter_key_init_kernel(ScatterArgs a) {
@@ -367,6 +594,40 @@ __global__ __launch_bounds__(kBlock) void scatter_key_kernel(ScatterArgs a) {
       }
     }
   }
+}
+
+// packed keys with the wavefront pre-reduction of run_reduce_wave: the largest key of a run of equal
+// neighbouring indices goes to the table with one read and at most one atomic
+template <typename T, int C_, bool IS_MAX>
+struct KeyRun {
+  typedef uint64_t A;
+  static constexpr int C = C_;
+  static constexpr int EW = 1;
+  static constexpr int U = 4;
+  const T *src;
+  uint64_t *keys;
+  int64_t K;
+  int precheck;
+  __device__ A identity() const { return 0; }
+  __device__ void load(int64_t e, int64_t pos, int64_t col, A *x) const {
+    const Vec<T, C> r = load_vec_stream<T, C>(src + e * K + col);
+    make_keys<T, C, IS_MAX>(r, pos, x);
+  }
+  __device__ void combine(A &x, const A &y) const { x = x > y ? x : y; }
+  __device__ void emit(int node, int64_t col, const A *x) const {
+    keys_to_global<1>(keys + (int64_t)node * K + col, x, precheck);
+  }
+};
+
+template <typename T, int C, bool IS_MAX>
+__global__ __launch_bounds__(kBlock) void scatter_key_run_kernel(ScatterArgs a, int lshift, int rows_per_wave) {
+  __shared__ uint64_t s_stage[kBlock / kWave][kWave * C];
+  KeyRun<T, C, IS_MAX> p;
+  p.src = static_cast<const T *>(a.src);
+  p.keys = reinterpret_cast<uint64_t *>(a.arg_out);
+  p.K = a.K;
+  p.precheck = a.precheck;
+  run_reduce_wave(a, lshift, rows_per_wave, p, s_stage[threadIdx.x / kWave]);
 }
 
 // ---- packed-key min/max with a workgroup-private cache of hot slots ---------
@@ -692,6 +953,30 @@ int launch_scatter_v(const ScatterArgs &a, int reduce, hipStream_t stream) {
             return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
           }
         }
+        if constexpr (__is_same(T, float) || __is_same(T, double) || __is_same(T, int32_t) ||
+                      __is_same(T, int64_t) || __is_same(T, bf16_t) || __is_same(T, f16_t)) {
+          // one index per row: sum runs of equal neighbouring indices in the wavefront first
+          constexpr bool k16 = sizeof(T) == 2;
+          const bool pair_ok = a.K % 2 == 0 && (reinterpret_cast<uintptr_t>(a.out) & 3) == 0 &&
+                               (reinterpret_cast<uintptr_t>(a.src) & 3) == 0;
+          if (a.run_reduce && a.sk == 0 && a.B * a.N < 0x7FFFFFFFll && (!k16 || pair_ok)) {
+            constexpr int CN = k16 ? 2 : 1;               // columns per lane without 16-byte loads
+            constexpr int C = VEC > 1 ? VEC : CN;
+            // 16-byte loads pay once the instruction rate limits the stream; small inputs are bound by
+            // latency and do better with one atomic per lane straight from registers
+            const bool wide = C > CN && n_src * (int64_t)sizeof(T) > ((int64_t)32 << 20);
+            const RunGrid g = run_grid(n_edges, a.K / (wide ? C : CN));
+            if (g.ok) {
+              if (wide)
+                hipLaunchKernelGGL((scatter_add_run_kernel<T, C>), dim3(g.blocks, g.ychunks), dim3(kBlock), 0, stream,
+                                   a, g.lshift, g.rpw);
+              else
+                hipLaunchKernelGGL((scatter_add_run_kernel<T, CN>), dim3(g.blocks, g.ychunks), dim3(kBlock), 0, stream,
+                                   a, g.lshift, g.rpw);
+              return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
+            }
+          }
+        }
         if constexpr (__is_same(T, bf16_t) || __is_same(T, f16_t)) {
           if (a.K % 2 == 0 && a.sk == 0 && (reinterpret_cast<uintptr_t>(a.out) & 3) == 0 &&
               (reinterpret_cast<uintptr_t>(a.src) & 3) == 0) {
@@ -737,6 +1022,25 @@ int launch_scatter_v(const ScatterArgs &a, int reduce, hipStream_t stream) {
       const int64_t epb = lds_chunk_edges(a.lds_epb, a.K, n_edges);
       const unsigned g_lds = (unsigned)((n_edges + epb - 1) / epb);
       const unsigned g_key = scatter_grid(n_edges, a.K / VEC, kBlock, 4);
+      // one index per row, few entries per slot: combine runs of equal neighbouring indices in the
+      // wavefront before going to the table (a sorted index then costs one atomic per slot)
+      if (!use_lds && a.run_reduce && a.sk == 0 && a.B * a.N < 0x7FFFFFFFll && n_src > 0) {
+        constexpr int KC = VEC > 4 ? 4 : VEC;  // columns per lane: 64-bit keys, so at most four
+        const RunGrid g = run_grid(n_edges, a.K / KC);
+        if (g.ok) {
+          const dim3 gd(g.blocks, g.ychunks);
+          if (is_max) {
+            hipLaunchKernelGGL((scatter_key_init_kernel<T, true>), dim3(g_out), dim3(kBlock), 0, stream, a);
+            hipLaunchKernelGGL((scatter_key_run_kernel<T, KC, true>), gd, dim3(kBlock), 0, stream, a, g.lshift, g.rpw);
+            hipLaunchKernelGGL((scatter_key_final_kernel<T, true>), dim3(g_out), dim3(kBlock), 0, stream, a);
+          } else {
+            hipLaunchKernelGGL((scatter_key_init_kernel<T, false>), dim3(g_out), dim3(kBlock), 0, stream, a);
+            hipLaunchKernelGGL((scatter_key_run_kernel<T, KC, false>), gd, dim3(kBlock), 0, stream, a, g.lshift, g.rpw);
+            hipLaunchKernelGGL((scatter_key_final_kernel<T, false>), dim3(g_out), dim3(kBlock), 0, stream, a);
+          }
+          return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
+        }
+      }
       if (is_max) {
         hipLaunchKernelGGL((scatter_key_init_kernel<T, true>), dim3(g_out), dim3(kBlock), 0, stream, a);
         if (n_src > 0) {

@@ -383,6 +383,119 @@ def test_scatter_sum_lds_aggregated_variant(capi, oracle, shape, dtype, monkeypa
     assert torch.equal(cnt.cpu(), torch.bincount(index1, minlength=N).float())
 
 
+RUN_SHAPES = [
+    # B, E, K, N
+    (1, 5000, 1, 600), (1, 3000, 2, 40), (1, 2000, 3, 300), (2, 1500, 5, 64), (1, 4000, 16, 500),
+    (1, 1500, 17, 100), (1, 1200, 64, 90), (1, 700, 100, 50), (1, 300, 130, 9), (3, 900, 8, 2),
+]
+
+
+def run_index(kind, rng, E, N):
+    """Indices with runs of equal neighbours, as a message-passing index has them."""
+    idx = np.sort(rng.integers(0, N, size=E))
+    if kind == "sorted":
+        return idx
+    if kind == "hub":  # one node owns the middle third
+        idx[E // 3: 2 * E // 3] = idx[E // 3]
+        return idx
+    # runs kept, order of the runs shuffled: a node shows up in several separate runs
+    cuts = np.sort(rng.choice(np.arange(1, E), size=min(E - 1, 40), replace=False))
+    pieces = np.split(idx, cuts)
+    rng.shuffle(pieces)
+    return np.concatenate(pieces)
+
+
+@pytest.mark.parametrize("shape,kind,dtype", product(
+    RUN_SHAPES, ["sorted", "hub", "pieces"],
+    [torch.int32, torch.int64, torch.float32, torch.float64, torch.bfloat16, torch.float16]))
+def test_scatter_sum_runs_of_equal_indices(capi, oracle, shape, kind, dtype):
+    """Sum with the wavefront pre-reduction of neighbouring equal indices: exact for
+    integers, within tolerance of the exact sum for floats; count shares the kernel."""
+    B, E, K, N = shape
+    rng = np.random.default_rng(E * 7 + K)
+    if dtype.is_floating_point:
+        src = torch.from_numpy(rng.standard_normal(size=(B, E, K))).to(dtype)
+    else:
+        src = torch.from_numpy(rng.integers(-1000, 1000, size=(B, E, K))).to(dtype)
+    index1 = torch.from_numpy(run_index(kind, rng, E, N))
+    index = index1.view(1, E, 1).expand(B, E, K)
+    for out_given in (False, True):
+        if dtype.is_floating_point:
+            prev = torch.from_numpy(rng.standard_normal(size=(B, N, K))).to(dtype)
+        else:
+            prev = torch.from_numpy(rng.integers(-1000, 1000, size=(B, N, K))).to(dtype)
+        out = prev.clone().to(DEV) if out_given else torch.full((B, N, K), 9, dtype=dtype, device=DEV)
+        capi.scatter(src.to(DEV), index1.to(DEV), out, None, B, E, K, N, 0, 1, 0, capi.SUM, out_given)
+        torch.cuda.synchronize()
+        if not dtype.is_floating_point:
+            want = prev.clone() if out_given else None
+            want = oracle.scatter(src, index, 1, want, None if out_given else N, "sum")[0]
+            assert_exact(out, want, f"{kind} out_given={out_given}")
+        else:
+            exact = oracle.scatter(src.double(), index, 1, None, N, "sum")[0]
+            absum = oracle.scatter(src.double().abs(), index, 1, None, N, "sum")[0]
+            want = exact + (prev.double() if out_given else 0)
+            rtol = RTOL[dtype]
+            err = (out.cpu().double() - want).abs()
+            bound = rtol * want.abs() + rtol * (absum + (prev.double().abs() if out_given else 0)).clamp(min=1e-30)
+            if dtype in (torch.bfloat16, torch.float16) and K % 2 == 1:
+                # odd rows of 16-bit floats take the plain kernel: element-type atomics that round after
+                # every add (as the reference's do), so the error grows with the entries per slot
+                cnt = oracle.scatter(torch.ones(B, E, K, dtype=torch.double), index, 1, None, N, "sum")[0]
+                bound = bound + 2.0 ** -8 * cnt * absum
+            assert bool((err <= bound).all()), (kind, out_given, float((err - bound).max()))
+    cnt = torch.empty((N,), dtype=torch.float32, device=DEV)
+    capi.scatter_count(index1.to(DEV), cnt, 1, E, N, 0, 1)
+    torch.cuda.synchronize()
+    assert torch.equal(cnt.cpu(), torch.bincount(index1, minlength=N).float())
+
+
+@pytest.mark.parametrize("shape,kind,reduce,dtype", product(
+    RUN_SHAPES, ["sorted", "hub", "pieces"], ["min", "max"],
+    [torch.float32, torch.bfloat16, torch.float16, torch.int32, torch.uint8]))
+def test_scatter_minmax_runs_of_equal_indices(capi, oracle, shape, kind, reduce, dtype):
+    """min / max + arg with the wavefront pre-reduction of neighbouring equal indices,
+    heavy ties (the first position has to win), with and without a given out."""
+    B, E, K, N = shape
+    rng = np.random.default_rng(E * 11 + K)
+    src = random_values(rng, (B, E, K), dtype, ties=True)
+    if dtype == torch.uint8:
+        src = src.clamp(min=1) if reduce == "max" else src.clamp(max=254)  # stay off the initial value
+    index1 = torch.from_numpy(run_index(kind, rng, E, N))
+    index = index1.view(1, E, 1).expand(B, E, K)
+    for out_given in (False, True):
+        if out_given:
+            prev = random_values(rng, (B, N, K), dtype, ties=True)
+            want = prev.clone()
+            _, want_arg = oracle.scatter(src, index, 1, want, None, reduce)
+            out = prev.clone().to(DEV)
+        else:
+            want, want_arg = oracle.scatter(src, index, 1, None, N, reduce)
+            out = torch.empty((B, N, K), dtype=dtype, device=DEV)
+        arg = torch.empty((B, N, K), dtype=torch.long, device=DEV)
+        capi.scatter(src.to(DEV), index1.to(DEV), out, arg, B, E, K, N, 0, 1, 0, capi.REDUCE[reduce], out_given)
+        torch.cuda.synchronize()
+        assert_exact(out, want, f"{kind} out_given={out_given}")
+        assert_exact(arg, want_arg, f"{kind} out_given={out_given} arg")
+
+
+def test_scatter_sum_plain_atomic_kernel_still_covered(capi, oracle, monkeypatch):
+    """The one-atomic-per-element kernel (used for per-element indices) with a shared index."""
+    monkeypatch.setenv("TS_SCATTER_RUNS", "0")
+    B, E, K, N = 2, 3000, 6, 50
+    rng = np.random.default_rng(5)
+    src = torch.from_numpy(rng.integers(-1000, 1000, size=(B, E, K))).to(torch.int32)
+    index1 = torch.from_numpy(np.sort(rng.integers(0, N, size=E)))
+    want = oracle.scatter(src, index1.view(1, E, 1).expand(B, E, K), 1, None, N, "sum")[0]
+    out = torch.empty((B, N, K), dtype=torch.int32, device=DEV)
+    capi.scatter(src.to(DEV), index1.to(DEV), out, None, B, E, K, N, 0, 1, 0, capi.SUM, False)
+    cnt = torch.empty((N,), dtype=torch.float32, device=DEV)
+    capi.scatter_count(index1.to(DEV), cnt, 1, E, N, 0, 1)
+    torch.cuda.synchronize()
+    assert_exact(out, want)
+    assert torch.equal(cnt.cpu(), torch.bincount(index1, minlength=N).float())
+
+
 @pytest.mark.parametrize("reduce,dtype", product(["sum", "min", "max"], [torch.float32, torch.float64, torch.int64]))
 def test_scatter_out_given_and_wide_types(capi, oracle, reduce, dtype):
     B, E, K, N = 2, 3000, 6, 40
