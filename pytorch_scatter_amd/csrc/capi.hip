@@ -80,6 +80,14 @@ CsrWs csr_workspace(const CsrPlan &p, int64_t B, int64_t K, int dtype, int reduc
   return w;
 }
 
+// Workspace for either plan: buffers that are not 16-byte aligned take one element per lane,
+// which changes the tile size and with it the number of partial results.
+size_t csr_workspace_max(int64_t B, int64_t N, int64_t E, int64_t K, int dtype, int reduce) {
+  const size_t w1 = csr_workspace(csr_plan(N, E, K, kElemBytes[dtype], true), B, K, dtype, reduce).total;
+  const size_t w0 = csr_workspace(csr_plan(N, E, K, kElemBytes[dtype], false), B, K, dtype, reduce).total;
+  return w1 > w0 ? w1 : w0;
+}
+
 int run_csr_reduce(const void *src, const int64_t *indptr, void *out, int64_t *arg_out, void *count_out,
                    int64_t B, int64_t N, int64_t E, int64_t K, int64_t indptr_batch_stride, int dtype,
                    int reduce, int accumulate, void *ws, size_t ws_bytes, hipStream_t stream) {
@@ -129,8 +137,7 @@ size_t ts_segment_csr_workspace_bytes(int64_t B, int64_t N, int64_t E, int64_t K
   if (!valid_dtype(dtype) || !sizes_ok(B, N, E, K)) return 0;
   // the plan may fall back to one element per lane for unaligned buffers; the
   // tile count does not depend on that choice
-  const CsrPlan p = csr_plan(N, E, K, kElemBytes[dtype], true);
-  return csr_workspace(p, B, K, dtype, reduce).total;
+  return csr_workspace_max(B, N, E, K, dtype, reduce);
 }
 
 int ts_segment_csr(const void *src, const int64_t *indptr, void *out, int64_t *arg_out, int64_t B,
@@ -191,9 +198,8 @@ int ts_segment_mean_csr_backward(const void *grad_out, const int64_t *indptr, vo
 
 size_t ts_segment_coo_workspace_bytes(int64_t B, int64_t N, int64_t E, int64_t K, int dtype, int reduce) {
   if (!valid_dtype(dtype) || !sizes_ok(B, N, E, K)) return 0;
-  const CsrPlan p = csr_plan(N, E, K, kElemBytes[dtype], true);
   const size_t ptr_bytes = ((size_t)B * (N + 1) * 8 + 255) & ~(size_t)255;
-  return ptr_bytes + csr_workspace(p, B, K, dtype, reduce).total;
+  return ptr_bytes + csr_workspace_max(B, N, E, K, dtype, reduce);
 }
 
 int ts_segment_coo(const void *src, const int64_t *index, void *out, void *arg_out, void *count_out,
@@ -208,7 +214,8 @@ int ts_segment_coo(const void *src, const int64_t *index, void *out, void *arg_o
   if (!workspace || workspace_bytes < ptr_bytes) return TS_ERR_WORKSPACE;
   hipStream_t s = static_cast<hipStream_t>(stream);
   int64_t *ptr = static_cast<int64_t *>(workspace);
-  dim3 grid((unsigned)((E + 1 + kBlock - 1) / kBlock), (unsigned)B);
+  const int64_t per_block = (int64_t)kBlock * kCooPtrPerThread;
+  dim3 grid((unsigned)((E + 1 + per_block - 1) / per_block), (unsigned)B);
   hipLaunchKernelGGL(coo_to_indptr_kernel, grid, dim3(kBlock), 0, s, index, ptr, N, E, index_batch_stride);
   if (hipGetLastError() != hipSuccess) return TS_ERR_LAUNCH;
   return run_csr_reduce(src, ptr, out, static_cast<int64_t *>(arg_out), count_out, B, N, E, K, N + 1, dtype,

@@ -392,6 +392,23 @@ __global__ __launch_bounds__(kBlock) void csr_reduce_fixup_kernel(CsrReduceArgs 
 
 // ---- host side -----------------------------------------------------------
 
+// narrow rows (csr_small.h, csr_gather_small_kernel): at most 16 elements and 64 bytes per entry
+constexpr int kSmallMaxK = 16;
+constexpr int kSmallMaxRowBytes = 64;
+constexpr int kSmallStageBytes = 16 * 1024;  // entries of one tile
+inline bool csr_small_ok(int64_t K, int elem_bytes) {
+  if (const char *env = getenv("TS_CSR_SMALL")) {  // tuning aid: 0 sends narrow rows to the wide kernel
+    if (atoi(env) == 0) return false;
+  }
+  return K >= 1 && K <= kSmallMaxK && K * elem_bytes <= kSmallMaxRowBytes;
+}
+// items (rows + entries) per tile so that the entries fit the LDS stage
+inline int csr_small_tile_items(int64_t K, int elem_bytes) {
+  int bi = kSmallStageBytes / (int)(K * elem_bytes);
+  if (bi > kMaxBlockItems) bi = kMaxBlockItems;
+  return bi & ~63;
+}
+
 struct CsrPlan {
   int vec;       // elements per lane (16 bytes worth, or 1)
   int G;         // lanes per worker
@@ -399,10 +416,28 @@ struct CsrPlan {
   int ipw;       // items per worker
   int64_t nblk;  // tiles per batch
   int ychunks;   // column chunks
+  bool small;    // narrow rows: the LDS-staged kernel
 };
 
 inline CsrPlan csr_plan(int64_t N, int64_t E, int64_t K, int elem_bytes, bool aligned16, bool expand = false) {
   CsrPlan p;
+  p.small = false;
+  // narrow rows: always for the reduction; for the expansion when a row is at most 8 bytes or
+  // consists of whole, aligned 16-byte granules (other widths do better with the wide kernel)
+  const bool granules = aligned16 && (K * elem_bytes) % kVecBytes == 0;
+  if (csr_small_ok(K, elem_bytes) && (!expand || K * elem_bytes <= 8 || granules)) {
+    p.small = true;
+    p.vec = (expand && granules) ? kVecBytes / elem_bytes : 1;
+    p.G = 1;
+    while (p.G < K) p.G <<= 1;
+    p.ychunks = 1;
+    // the reduction stages the tile's entries in LDS; the expansion only its row pointers
+    p.BI = expand ? kMaxBlockItems : csr_small_tile_items(K, elem_bytes);
+    p.ipw = p.BI / (kBlock / p.G);
+    p.nblk = (N + E + p.BI - 1) / p.BI;
+    if (p.nblk < 1) p.nblk = 1;
+    return p;
+  }
   const int full = kVecBytes / elem_bytes;
   p.vec = (aligned16 && full > 1 && K % full == 0) ? full : 1;
   const int64_t lanes = (K + p.vec - 1) / p.vec;
@@ -469,9 +504,13 @@ int launch_csr_reduce_v(const CsrReduceArgs &a, const CsrPlan &p, int64_t B, int
 template <typename T> int launch_csr_reduce(const CsrReduceArgs &a, const CsrPlan &p, int64_t B,
                                             int reduce, hipStream_t stream);
 
+template <typename T>
+int launch_csr_reduce_small(const CsrReduceArgs &a, const CsrPlan &p, int64_t B, int reduce, hipStream_t stream);
+
 #define TS_INSTANTIATE_CSR_REDUCE(T, FULLVEC)                                               \
   template <> int launch_csr_reduce<T>(const CsrReduceArgs &a, const CsrPlan &p, int64_t B, \
                                        int reduce, hipStream_t stream) {                    \
+    if (p.small) return launch_csr_reduce_small<T>(a, p, B, reduce, stream);                \
     if (p.vec == FULLVEC) return launch_csr_reduce_v<T, FULLVEC>(a, p, B, reduce, stream);  \
     return launch_csr_reduce_v<T, 1>(a, p, B, reduce, stream);                              \
   }

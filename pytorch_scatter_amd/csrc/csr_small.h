@@ -1,0 +1,193 @@
+// Segmented reduction over CSR row pointers for narrow rows (K <= 16 elements,
+// at most 64 bytes per entry): attention scores, degrees, per-head scalars.
+//
+// With so few bytes per entry the wide kernel's lane groups would each chase
+// their own cache line. Here a workgroup stages the entries of its merge-path
+// tile in LDS with full 16-byte coalesced loads and then reduces from LDS:
+// one lane per (row, column) for ordinary rows, one wavefront per row for rows
+// with more than 64 entries inside the tile (64 lanes stride over the entries,
+// then a shuffle tree). Tiles, the workspace for rows that cross tiles and the
+// second kernel that combines them are those of the wide kernel. Results do not
+// depend on scheduling: no atomics.
+//
+// Semantics as in csr_reduce.h (csrc/cpu/segment_csr_cpu.cpp:54-88): strict
+// compare so the first index wins ties, mean = T(sum) / T(count), empty row -> 0
+// with arg = E.
+#pragma once
+
+#include "csr_reduce.h"
+
+namespace ts {
+
+constexpr int kSmallLongRow = 64;  // more entries than this inside a tile: one wavefront per row
+
+// LDS layout of a tile, in 16-byte units
+__host__ __device__ inline int csr_small_ptr_vecs(int BI) { return (BI + 2 + 3) / 4; }
+inline size_t csr_small_lds_bytes(int BI, int64_t K, int elem_bytes) {
+  return (size_t)csr_small_ptr_vecs(BI) * 16 + (((size_t)BI * K * elem_bytes + 15) / 16 + 1) * 16;
+}
+
+template <typename T, int REDUCE>
+__global__ __launch_bounds__(kBlock) void csr_reduce_small_kernel(CsrReduceArgs a) {
+  typedef typename Acc<T>::type A;
+  typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+  constexpr bool kArg = (REDUCE == TS_MIN || REDUCE == TS_MAX);
+
+  // dynamic LDS, sized by the tile: [row pointers: BI + 2, padded to 16 bytes][entries: BI * K elements + 16 bytes]
+  extern __shared__ u4 s_dyn[];
+  int32_t *s_ptr = reinterpret_cast<int32_t *>(s_dyn);
+  u4 *s_raw = s_dyn + csr_small_ptr_vecs(a.BI);
+  __shared__ int32_t s_long[kMaxBlockItems / kSmallLongRow + 2];
+  __shared__ int32_t s_nlong;
+  __shared__ int64_t s_cut[2];
+
+  const int tid = threadIdx.x;
+  const int K = (int)a.K;
+  const int64_t b = blockIdx.z;
+  const int64_t *ptr = a.indptr + b * a.indptr_batch_stride;
+  const T *src_b = static_cast<const T *>(a.src) + b * a.E * a.K;
+  T *out_b = static_cast<T *>(a.out) + b * a.N * a.K;
+  int64_t *arg_b = kArg ? a.arg_out + b * a.N * a.K : nullptr;
+  T *count_b = a.count_out ? static_cast<T *>(a.count_out) + b * a.N : nullptr;
+
+  // ---- tile cut: two wavefronts search the two diagonals concurrently
+  const int64_t total = a.N + a.E;
+  const int64_t d0 = (int64_t)blockIdx.x * a.BI;
+  const int64_t d1 = d0 + a.BI < total ? d0 + a.BI : total;
+  const int wave = tid / kWave;
+  const int lane = tid & (kWave - 1);
+  if (wave < 2) {
+    const int64_t i = merge_search_wave(ptr, a.N, a.E, wave == 0 ? d0 : d1);
+    if (lane == 0) s_cut[wave] = i;
+  }
+  if (tid == 0) s_nlong = 0;
+  __syncthreads();
+  const int64_t i0 = s_cut[0], i1 = s_cut[1];
+  const int64_t j0 = d0 - i0;
+  const int nr = (int)(i1 - i0);         // row ends inside the tile
+  const int ne = (int)((d1 - i1) - j0);  // entries inside the tile
+
+  // ---- row pointers, relative to the tile's first entry, and the entries themselves
+  const int64_t last = i1 + 1 < a.N ? i1 + 1 : a.N;
+  const int nload = (int)(last - i0) + 1;  // ptr[i0 .. last]
+  for (int t = tid; t < nload; t += kBlock) s_ptr[t] = (int32_t)(ptr[i0 + t] - j0);
+  // whole 16-byte granules around the tile's entries: a granule never crosses a page,
+  // so the bytes before the first and after the last entry are safe to read
+  const T *p_first = src_b + j0 * K;
+  const int shift = ne > 0 ? (int)((reinterpret_cast<uintptr_t>(p_first) & 15) / sizeof(T)) : 0;
+  const int nvec = ne > 0 ? (int)(((size_t)(shift + ne * K) * sizeof(T) + 15) / 16) : 0;
+  const u4 *p0 = reinterpret_cast<const u4 *>(p_first - shift);
+  for (int t = tid; t < nvec; t += kBlock) s_raw[t] = __builtin_nontemporal_load(p0 + t);
+  __syncthreads();
+  const T *s_src = reinterpret_cast<const T *>(s_raw) + shift;
+
+  // ---- which rows the tile sees
+  const bool has_open_row = i1 < a.N;                 // the row after the last row end
+  const bool head_exists = i0 < a.N && s_ptr[0] < 0;  // row i0 began in an earlier tile
+  const int nrows = nr + (has_open_row ? 1 : 0);
+  enum { kComplete = 0, kHead = 1, kTail = 2, kNone = 3 };
+  auto classify = [&](int r, int &lo, int &hi) -> int {
+    const bool open = r == nr;
+    lo = s_ptr[r] > 0 ? s_ptr[r] : 0;
+    hi = open ? ne : s_ptr[r + 1];
+    if (r == 0 && head_exists) return kHead;
+    if (open) return hi > lo ? kTail : kNone;
+    return kComplete;
+  };
+
+  A *ws_val_blk = static_cast<A *>(a.ws_vals) + ((b * a.nblk + blockIdx.x) * 2) * a.K;
+  int32_t *ws_arg_blk = kArg ? a.ws_args + ((b * a.nblk + blockIdx.x) * 2) * a.K : nullptr;
+  auto deliver = [&](int r, int k, int kind, A acc, int32_t arg) {
+    if (kind == kComplete) {
+      finalize_row<T, 1, REDUCE>(a, out_b, arg_b, count_b, i0 + r, k, k, &acc, &arg,
+                                 (int64_t)s_ptr[r + 1] - (int64_t)s_ptr[r], true);
+    } else if (kind == kHead) {
+      ws_val_blk[k] = acc;
+      if (kArg) ws_arg_blk[k] = arg;
+    } else if (kind == kTail) {
+      ws_val_blk[a.K + k] = acc;
+      if (kArg) ws_arg_blk[a.K + k] = arg;
+    }
+  };
+
+  // ---- one lane per (row, column); long rows are left to whole wavefronts
+  const int n_units = nrows * K;
+  for (int u = tid; u < n_units; u += kBlock) {
+    const int r = u / K;
+    const int k = u - r * K;
+    int lo, hi;
+    const int kind = classify(r, lo, hi);
+    if (kind == kNone) continue;
+    if (hi - lo > kSmallLongRow) {
+      if (k == 0) s_long[atomicAdd(&s_nlong, 1)] = r;
+      continue;
+    }
+    A acc = acc_init<A, REDUCE>();
+    int32_t arg = 0;
+    const T *q = s_src + lo * K + k;
+    for (int e = lo; e < hi; ++e, q += K) reduce_step<A, REDUCE>(acc, arg, to_acc<T>(*q), (int32_t)(j0 + e));
+    deliver(r, k, kind, acc, arg);
+  }
+  __syncthreads();
+
+  // ---- long rows: the lanes of a wavefront stride over the entries, then a shuffle tree
+  const int nlong = s_nlong;
+  for (int qi = wave; qi < nlong; qi += kBlock / kWave) {
+    const int r = s_long[qi];
+    int lo, hi;
+    const int kind = classify(r, lo, hi);
+    for (int k = 0; k < K; ++k) {
+      A acc = acc_init<A, REDUCE>();
+      int32_t arg = 0;
+      for (int e = lo + lane; e < hi; e += kWave)
+        reduce_step<A, REDUCE>(acc, arg, to_acc<T>(s_src[e * K + k]), (int32_t)(j0 + e));
+#pragma unroll
+      for (int off = kWave / 2; off >= 1; off >>= 1) {
+        const A oacc = __shfl_down(acc, off);
+        const int32_t oarg = __shfl_down(arg, off);
+        if (REDUCE == TS_SUM || REDUCE == TS_MEAN) {
+          acc = acc + oacc;
+        } else {
+          // equal values: the smaller position wins, as in a walk in entry order
+          const bool better = (REDUCE == TS_MIN ? oacc < acc : oacc > acc) || (oacc == acc && oarg < arg);
+          if (better) { acc = oacc; arg = oarg; }
+        }
+      }
+      if (lane == 0) deliver(r, k, kind, acc, arg);
+    }
+  }
+
+  // ---- what the second kernel needs to know about this tile
+  if (tid == 0 && blockIdx.y == 0) {
+    int64_t *meta = a.ws_meta + (b * a.nblk + blockIdx.x) * 4;
+    int lo, hi;
+    const bool tail = has_open_row && classify(nr, lo, hi) == kTail;
+    meta[0] = head_exists ? i0 : -1;
+    meta[1] = head_exists && nr > 0 ? 1 : 0;  // the head row ends inside this tile
+    meta[2] = tail ? i0 + nr : -1;
+  }
+}
+
+template <typename T, int REDUCE>
+int launch_csr_reduce_small_t(const CsrReduceArgs &a, const CsrPlan &p, int64_t B, hipStream_t stream) {
+  dim3 grid((unsigned)p.nblk, 1, (unsigned)B);
+  hipLaunchKernelGGL((csr_reduce_small_kernel<T, REDUCE>), grid, dim3(kBlock),
+                     csr_small_lds_bytes(p.BI, a.K, (int)sizeof(T)), stream, a);
+  const int W = kBlock / p.G;
+  dim3 grid2((unsigned)((p.nblk + W - 1) / W), 1, (unsigned)B);
+  hipLaunchKernelGGL((csr_reduce_fixup_kernel<T, 1, REDUCE>), grid2, dim3(kBlock), 0, stream, a);
+  return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
+}
+
+template <typename T>
+int launch_csr_reduce_small(const CsrReduceArgs &a, const CsrPlan &p, int64_t B, int reduce, hipStream_t stream) {
+  switch (reduce) {
+  case TS_SUM: return launch_csr_reduce_small_t<T, TS_SUM>(a, p, B, stream);
+  case TS_MEAN: return launch_csr_reduce_small_t<T, TS_MEAN>(a, p, B, stream);
+  case TS_MIN: return launch_csr_reduce_small_t<T, TS_MIN>(a, p, B, stream);
+  case TS_MAX: return launch_csr_reduce_small_t<T, TS_MAX>(a, p, B, stream);
+  default: return TS_ERR_UNSUPPORTED;
+  }
+}
+
+}  // namespace ts

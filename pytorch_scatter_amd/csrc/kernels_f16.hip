@@ -1,5 +1,6 @@
 // Kernel instantiations for element type f16_t.
 #include "csr_reduce.h"
+#include "csr_small.h"
 #include "csr_gather.h"
 #include "coo_gather.h"
 #include "scatter.h"

@@ -146,6 +146,68 @@ def test_segment_csr_other_dtypes(capi, oracle, dtype, reduce):
         assert_close(out, want, scale, dtype)
 
 
+NARROW_CASES = [
+    # kind, rows, K: rows of at most 32 bytes take the LDS-staged kernel
+    ("zipf", 3000, 1), ("zipf", 2500, 2), ("hub", 900, 3), ("hub", 700, 5), ("zipf", 2000, 8),
+    ("uniform", 5000, 1), ("hub", 300, 8), ("short", 6000, 2), ("hub", 1200, 4),
+]
+
+
+@pytest.mark.parametrize("case,reduce,dtype", product(
+    NARROW_CASES, ["sum", "mean", "min", "max"],
+    [torch.float32, torch.bfloat16, torch.float64, torch.int32, torch.int8]))
+def test_segment_csr_narrow_rows(capi, oracle, case, reduce, dtype):
+    """Narrow rows, every element type width, with the entries starting at an address
+    that is not 16-byte aligned (second pass) and long rows that cross many tiles."""
+    kind, n, K = case
+    rng, indptr, index = make_csr(kind, 100 + NARROW_CASES.index(case), n)
+    E = index.numel()
+    src = values(rng, (E, K), dtype, reduce)
+    if dtype == torch.int8 and reduce in ("sum", "mean"):
+        if kind != "short":
+            pytest.skip("8-bit sums and counts wrap on long rows: undefined upstream")
+        src = src.clamp(-1, 1)
+    want, want_arg = oracle.segment_csr(src, indptr, None, reduce)
+    for offset in (0, 1):
+        flat = torch.empty(E * K + 8, dtype=dtype, device=DEV)
+        dsrc = flat[offset:offset + E * K].view(E, K)
+        dsrc.copy_(src)
+        out = torch.full((n, K), 7, dtype=dtype, device=DEV)
+        arg = torch.full((n, K), -1, dtype=torch.long, device=DEV) if reduce in ("min", "max") else None
+        capi.segment_csr(dsrc, indptr.to(DEV), out, arg, 1, n, E, K, 0, capi.REDUCE[reduce])
+        torch.cuda.synchronize()
+        if reduce in ("min", "max") or not dtype.is_floating_point:
+            assert_exact(out, want, f"values offset={offset}")
+            if arg is not None:
+                assert_exact(arg, want_arg, f"arg offset={offset}")
+        else:
+            scale = float(oracle.segment_csr(src.abs().double(), indptr, None, "sum")[0].max()) if E else 0.0
+            assert_close(out, want, scale, dtype, f"values offset={offset}")
+
+
+@pytest.mark.parametrize("case,reduce", product(NARROW_CASES[:5], ["sum", "mean", "min", "max"]))
+def test_segment_coo_narrow_rows(capi, oracle, case, reduce):
+    kind, n, K = case
+    rng, indptr, index = make_csr(kind, 200 + NARROW_CASES.index(case), n)
+    E = index.numel()
+    src = values(rng, (E, K), torch.float32, reduce)
+    want, want2 = oracle.segment_coo(src, index, None, n, reduce)
+    out = torch.full((n, K), 7, dtype=torch.float32, device=DEV)
+    wa = reduce in ("min", "max")
+    arg = torch.full((n, K), -1, dtype=torch.long, device=DEV) if wa else None
+    count = torch.full((n,), -1, dtype=torch.float32, device=DEV) if reduce == "mean" else None
+    capi.segment_coo(src.to(DEV), index.to(DEV), out, arg, count, 1, n, E, K, 0, capi.REDUCE[reduce], False)
+    torch.cuda.synchronize()
+    if wa:
+        assert_exact(out, want)
+        assert_exact(arg, want2, "arg")
+    else:
+        scale = float(oracle.segment_csr(src.abs().double(), indptr, None, "sum")[0].max()) if E else 0.0
+        assert_close(out, want, scale, torch.float32)
+        if reduce == "mean":
+            assert_exact(count, want2, "count")
+
+
 @pytest.mark.parametrize("reduce", ["sum", "mean", "min", "max"])
 def test_segment_csr_batched(capi, oracle, reduce):
     rng = np.random.default_rng(21)
@@ -196,6 +258,40 @@ def test_segment_mean_csr_backward(capi, oracle, case, dtype):
     assert_exact(out, want)  # one correctly rounded division per element: bit-exact
 
 
+@pytest.mark.parametrize("case,dtype", product(
+    NARROW_CASES + [("zipf", 1500, 16), ("hub", 400, 12)],
+    [torch.float32, torch.bfloat16, torch.float64, torch.int64, torch.uint8]))
+def test_gather_csr_and_mean_backward_narrow_rows(capi, oracle, case, dtype):
+    """Narrow rows take the one-lane-per-16-bytes kernel; also with `out` off the 16-byte grid
+    and with a batch whose slices are not multiples of 16 bytes."""
+    kind, n, K = case
+    rng, indptr, index = make_csr(kind, 300 + n + K, n)
+    E = index.numel()
+    src = random_values(rng, (n, K), dtype, ties=False)
+    want = oracle.gather_csr(src, indptr)
+    for offset in (0, 1):
+        flat = torch.full((E * K + 8,), 3, dtype=dtype, device=DEV)
+        out = flat[offset:offset + E * K].view(E, K)
+        capi.gather_csr(src.to(DEV), indptr.to(DEV), out, 1, n, E, K, 0)
+        torch.cuda.synchronize()
+        assert_exact(out, want, f"offset={offset}")
+        assert bool((flat[:offset] == 3).all()) and bool((flat[offset + E * K:] == 3).all())
+    B = 3
+    srcb = random_values(rng, (B, n, K), dtype, ties=False)
+    wantb = oracle.gather_csr(srcb, indptr.view(1, -1).expand(B, -1))
+    outb = torch.full((B, E, K), 3, dtype=dtype, device=DEV)
+    capi.gather_csr(srcb.to(DEV), indptr.to(DEV), outb, B, n, E, K, 0)
+    torch.cuda.synchronize()
+    assert_exact(outb, wantb, "batched")
+    if dtype.is_floating_point:
+        g = torch.from_numpy(rng.standard_normal(size=(n, K))).to(dtype)
+        wantg = oracle.segment_mean_csr_backward(g, indptr, (E, K))
+        outg = torch.empty((E, K), dtype=dtype, device=DEV)
+        capi.segment_mean_csr_backward(g.to(DEV), indptr.to(DEV), outg, 1, n, E, K, 0)
+        torch.cuda.synchronize()
+        assert_exact(outg, wantg, "mean backward")
+
+
 @pytest.mark.parametrize("case,reduce,dtype", product(
     CSR_CASES[:9], ["sum", "mean", "min", "max"], [torch.float32, torch.bfloat16]))
 def test_segment_coo(capi, oracle, case, reduce, dtype):
@@ -219,9 +315,10 @@ def test_segment_coo(capi, oracle, case, reduce, dtype):
             assert_exact(cnt, want2)
 
 
-@pytest.mark.parametrize("reduce,dtype", product(["sum", "mean", "min", "max"], [torch.float32, torch.bfloat16]))
-def test_segment_coo_out_given(capi, oracle, reduce, dtype):
-    kind, n, K = "hub", 500, 16
+@pytest.mark.parametrize("reduce,dtype,K", product(["sum", "mean", "min", "max"], [torch.float32, torch.bfloat16],
+                                                   [16, 2]))
+def test_segment_coo_out_given(capi, oracle, reduce, dtype, K):
+    kind, n = "hub", 500
     rng, indptr, index = make_csr(kind, 33, n)
     E = index.numel()
     src = values(rng, (E, K), dtype, reduce)
