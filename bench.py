@@ -16,7 +16,8 @@ The same JSON line carries
   cpu_baseline  the reference's CPU kernels (oracle/_ref, else the C oracle)
                 timed on the host for the same workload, one thread;
   configs       effective GB/s of every op of configurations C1..C5, timed the
-                same way (events around back-to-back launches).
+                same way (events around back-to-back launches); the X-* rows are
+                extra shapes (sorted index given to scatter, one value per entry).
 """
 import argparse
 import json
@@ -37,7 +38,7 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--configs", default="C1,C2,C2m,C3,C4,C5",
+    ap.add_argument("--configs", default="C1,C2,C2m,C3,C4,C5,X",
                     help="comma list of side configurations to time (C2 is always run)")
     ap.add_argument("--iters", type=int, default=20, help="launches per op in the per-config table")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
@@ -288,6 +289,17 @@ def main():
     if "C5" in want:
         table["C5"] = bench_csr_config(ts, wl, wl.c5_gnn(), dev, max(it // 2, 3),
                                        ["gather_csr", "segment_csr_mean", "segment_csr_mean_backward"])
+
+    if "X" in want:
+        # not BASELINE configurations: the graph of C3 with a sorted index given to scatter (the usual
+        # message-passing call) and with one value per entry (attention scores, degrees)
+        import dataclasses
+        w3 = wl.c3_segment_coo()
+        sw = wl.ScatterWorkload("X-sorted-K64", w3.index, w3.N, w3.E, 64, torch.float32)
+        table["X-sorted-K64"] = bench_scatter_config(ts, wl, sw, dev, max(it // 2, 3), ["sum", "max"])
+        table["X-narrow-K1"] = bench_csr_config(ts, wl, dataclasses.replace(w3, K=1, name="X-narrow-K1"), dev, it,
+                                                ["segment_csr_sum", "segment_csr_max", "segment_coo_sum",
+                                                 "gather_csr", "gather_coo"], uniform=True)
 
     cpu = None if args.no_cpu else cpu_baseline(wl, w2)
 
