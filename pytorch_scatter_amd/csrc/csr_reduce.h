@@ -74,14 +74,13 @@ __device__ __forceinline__ void finalize_row(const CsrReduceArgs &a, T *out_b, i
   int64_t oa[VEC];
   Vec<T, VEC> prev;
   if (a.accumulate) prev = load_vec<T, VEC>(op);
-  const RowDivider<T> divide(REDUCE == TS_MEAN && count > 1 ? count : 1);
 #pragma unroll
   for (int v = 0; v < VEC; ++v) {
     A x = acc[v];
     if (REDUCE == TS_SUM || REDUCE == TS_MEAN) {
       if (a.accumulate) x = to_acc<T>(prev.v[v]) + x;
       T t = from_acc<T>(x);
-      if (REDUCE == TS_MEAN && count > 1) t = divide(t);  // x / 1 == x
+      if (REDUCE == TS_MEAN && count > 1) t = div_elem<T>(t, count_as<T>(count));  // x / 1 == x
       o.v[v] = t;
     } else {
       if (a.accumulate) {

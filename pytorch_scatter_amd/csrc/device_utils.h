@@ -2,8 +2,6 @@
 // 16-byte vector access, accumulate-type conversions and the reducer rules.
 #pragma once
 
-#include <type_traits>
-
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -116,40 +114,6 @@ template <> struct ElemLim<bf16_t> {
 template <> struct ElemLim<f16_t> {
   __device__ static f16_t max() { return (f16_t)65504.0f; }
   __device__ static f16_t lowest() { return (f16_t)-65504.0f; }
-};
-
-// Several elements divided by the same (scalar_t)count: the reciprocal is formed once
-// (one full division), each quotient then costs a multiply and one residual
-// correction, q' = q + (x - q c) / c, which restores the correctly rounded result
-// of x / c outside the overflow and subnormal ranges. A row end sits in divergent
-// code, where the full division sequence per element is paid once per lane group.
-// Integers keep the truncating division.
-template <typename T, bool IS_FLOAT = !std::is_integral<T>::value> struct RowDivider;
-template <typename T> struct RowDivider<T, false> {
-  T c;
-  __device__ explicit RowDivider(int64_t count) : c(count_as<T>(count)) {}
-  __device__ T operator()(T x) const { return div_elem<T>(x, c); }
-};
-template <typename T> struct RowDivider<T, true> {
-  typedef typename Acc<T>::type A;
-  A c, rc;
-  // counts are below 2^31, so the conversion may go through 32 bits (same single rounding)
-  __device__ explicit RowDivider(int64_t count) : c(to_acc<T>(count_as<T>((int64_t)(int32_t)count))) {
-    if constexpr (sizeof(A) == 4) {
-      // hardware reciprocal (1 ulp) plus one Newton step: correctly rounded 1 / c for these integers
-      const float r0 = __builtin_amdgcn_rcpf(c);
-      rc = __builtin_fmaf(__builtin_fmaf(-c, r0, 1.0f), r0, r0);
-    } else {
-      rc = (A)1 / c;
-    }
-  }
-  __device__ T operator()(T x) const {
-    const A xf = to_acc<T>(x);
-    A q = xf * rc;
-    const A big = Lim<A>::max();
-    if (q >= -big && q <= big && c <= big) q = __builtin_fma(__builtin_fma(-q, c, xf), rc, q);  // not for inf / nan
-    return from_acc<T>(q);
-  }
 };
 
 template <typename A, int REDUCE> __device__ __forceinline__ A acc_init() {
