@@ -46,7 +46,7 @@ struct CsrReduceArgs {
   // workspace
   void *ws_vals;      // Acc [B][nblk][2][K]
   int32_t *ws_args;   // int32 [B][nblk][2][K]  (min/max)
-  int64_t *ws_meta;   // int64 [B][nblk][4]: head_row, head_closes, tail_row, -
+  int64_t *ws_meta;   // int64 [B][nblk][4]: head_row, head_closes, tail_row, length of the tail row
 };
 
 template <typename A, int REDUCE>
@@ -300,7 +300,10 @@ __global__ __launch_bounds__(kBlock) void csr_reduce_kernel(CsrReduceArgs a) {
           if (kArg) ws_arg_blk[a.K + col + v] = arg[v];
         }
       }
-      if (lg == 0 && blockIdx.y == 0) meta[2] = i0 + row;
+      if (lg == 0 && blockIdx.y == 0) {
+        meta[2] = i0 + row;
+        meta[3] = (int64_t)s_ptr[row + 1] - (int64_t)s_ptr[row];  // full length of the row
+      }
     }
   }
   if (w == 0) {
@@ -357,37 +360,51 @@ __global__ __launch_bounds__(kBlock) void csr_reduce_fixup_kernel(CsrReduceArgs 
   const int64_t t = (int64_t)blockIdx.x * W + w;
   if (t >= a.nblk) return;
   const int64_t *meta = a.ws_meta + (b * a.nblk) * 4;
-  const int64_t row = meta[t * 4 + 2];
-  if (row < 0) return;
   const A *vals = static_cast<const A *>(a.ws_vals) + (b * a.nblk) * 2 * a.K;
   const int32_t *args = kArg ? a.ws_args + (b * a.nblk) * 2 * a.K : nullptr;
-
-  A acc[VEC];
-  int32_t arg[VEC];
   const int64_t c = col_ok ? col : 0;
+
+  // Nearly every open row ends in the next tile: everything that case needs is loaded at
+  // once (one memory latency instead of a chain of five), whether or not it turns out to be used.
+  const int64_t tn = t + 1 < a.nblk ? t + 1 : t;
+  const int64_t row = meta[t * 4 + 2];
+  const int64_t count = meta[t * 4 + 3];  // length of that row, left by the tile that opened it
+  int64_t next_row = meta[tn * 4 + 0];
+  int64_t next_closes = meta[tn * 4 + 1];
+  A acc[VEC], hv[VEC];
+  int32_t arg[VEC], ha[VEC];
 #pragma unroll
   for (int v = 0; v < VEC; ++v) {
     acc[v] = vals[(t * 2 + 1) * a.K + c + v];
     arg[v] = kArg ? args[(t * 2 + 1) * a.K + c + v] : 0;
+    hv[v] = vals[(tn * 2) * a.K + c + v];
+    ha[v] = kArg ? args[(tn * 2) * a.K + c + v] : 0;
   }
+  if (row < 0) return;
   for (int64_t tt = t + 1; tt < a.nblk; ++tt) {
-    if (meta[tt * 4 + 0] != row) break;  // cannot happen for a well-formed indptr
+    if (tt > t + 1) {
+      next_row = meta[tt * 4 + 0];
+      next_closes = meta[tt * 4 + 1];
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) {
+        hv[v] = vals[(tt * 2) * a.K + c + v];
+        ha[v] = kArg ? args[(tt * 2) * a.K + c + v] : 0;
+      }
+    }
+    if (next_row != row) break;  // cannot happen for a well-formed indptr
 #pragma unroll
     for (int v = 0; v < VEC; ++v) {
-      const A hv = vals[(tt * 2) * a.K + c + v];
       if (kArg)
-        reduce_step<A, REDUCE>(acc[v], arg[v], hv, args[(tt * 2) * a.K + c + v]);
+        reduce_step<A, REDUCE>(acc[v], arg[v], hv[v], ha[v]);
       else
-        acc[v] = acc[v] + hv;
+        acc[v] = acc[v] + hv[v];
     }
-    if (meta[tt * 4 + 1] != 0) break;
+    if (next_closes != 0) break;
   }
-  const int64_t *ptr = a.indptr + b * a.indptr_batch_stride;
   T *out_b = static_cast<T *>(a.out) + b * a.N * a.K;
   int64_t *arg_b = kArg ? a.arg_out + b * a.N * a.K : nullptr;
   T *count_b = a.count_out ? static_cast<T *>(a.count_out) + b * a.N : nullptr;
-  finalize_row<T, VEC, REDUCE>(a, out_b, arg_b, count_b, row, col, lg, acc, arg,
-                               ptr[row + 1] - ptr[row], col_ok);
+  finalize_row<T, VEC, REDUCE>(a, out_b, arg_b, count_b, row, col, lg, acc, arg, count, col_ok);
 }
 
 // ---- host side -----------------------------------------------------------

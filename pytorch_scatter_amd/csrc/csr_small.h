@@ -165,6 +165,7 @@ __global__ __launch_bounds__(kBlock) void csr_reduce_small_kernel(CsrReduceArgs 
     meta[0] = head_exists ? i0 : -1;
     meta[1] = head_exists && nr > 0 ? 1 : 0;  // the head row ends inside this tile
     meta[2] = tail ? i0 + nr : -1;
+    if (tail) meta[3] = (int64_t)s_ptr[nr + 1] - (int64_t)s_ptr[nr];  // full length of the open row
   }
 }
 

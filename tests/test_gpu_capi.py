@@ -185,6 +185,32 @@ def test_segment_csr_narrow_rows(capi, oracle, case, reduce, dtype):
             assert_close(out, want, scale, dtype, f"values offset={offset}")
 
 
+@pytest.mark.parametrize("reduce,dtype", product(["sum", "max"], [torch.float32, torch.bfloat16]))
+def test_segment_csr_wide_rows_unaligned(capi, oracle, reduce, dtype):
+    """Buffers off the 16-byte grid take one element per lane, a different tile size and
+    more partial results: the workspace size reported for the shape has to cover that plan too."""
+    kind, n, K = "hub", 900, 64
+    rng, indptr, index = make_csr(kind, 77, n)
+    E = index.numel()
+    src = values(rng, (E, K), dtype, reduce)
+    want, want_arg = oracle.segment_csr(src, indptr, None, reduce)
+    flat = torch.empty(E * K + 8, dtype=dtype, device=DEV)
+    dsrc = flat[1:1 + E * K].view(E, K)
+    dsrc.copy_(src)
+    oflat = torch.full((n * K + 8,), 7, dtype=dtype, device=DEV)
+    out = oflat[1:1 + n * K].view(n, K)
+    arg = torch.full((n, K), -1, dtype=torch.long, device=DEV) if reduce == "max" else None
+    capi.segment_csr(dsrc, indptr.to(DEV), out, arg, 1, n, E, K, 0, capi.REDUCE[reduce])
+    torch.cuda.synchronize()
+    if reduce == "max":
+        assert_exact(out, want, "values")
+        assert_exact(arg, want_arg, "arg")
+    else:
+        scale = float(oracle.segment_csr(src.abs().double(), indptr, None, "sum")[0].max())
+        assert_close(out, want, scale, dtype, "values")
+    assert bool((oflat[:1] == 7).all()) and bool((oflat[1 + n * K:] == 7).all())
+
+
 @pytest.mark.parametrize("case,reduce", product(NARROW_CASES[:5], ["sum", "mean", "min", "max"]))
 def test_segment_coo_narrow_rows(capi, oracle, case, reduce):
     kind, n, K = case
