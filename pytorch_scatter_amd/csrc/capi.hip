@@ -83,8 +83,9 @@ CsrWs csr_workspace(const CsrPlan &p, int64_t B, int64_t K, int dtype, int reduc
 // Workspace for either plan: buffers that are not 16-byte aligned take one element per lane,
 // which changes the tile size and with it the number of partial results.
 size_t csr_workspace_max(int64_t B, int64_t N, int64_t E, int64_t K, int dtype, int reduce) {
-  const size_t w1 = csr_workspace(csr_plan(N, E, K, kElemBytes[dtype], true), B, K, dtype, reduce).total;
-  const size_t w0 = csr_workspace(csr_plan(N, E, K, kElemBytes[dtype], false), B, K, dtype, reduce).total;
+  const bool wa = reduce == TS_MIN || reduce == TS_MAX;
+  const size_t w1 = csr_workspace(csr_plan(N, E, K, kElemBytes[dtype], true, false, wa), B, K, dtype, reduce).total;
+  const size_t w0 = csr_workspace(csr_plan(N, E, K, kElemBytes[dtype], false, false, wa), B, K, dtype, reduce).total;
   return w1 > w0 ? w1 : w0;
 }
 
@@ -92,7 +93,7 @@ int run_csr_reduce(const void *src, const int64_t *indptr, void *out, int64_t *a
                    int64_t B, int64_t N, int64_t E, int64_t K, int64_t indptr_batch_stride, int dtype,
                    int reduce, int accumulate, void *ws, size_t ws_bytes, hipStream_t stream) {
   const bool al = aligned16(src) && aligned16(out);
-  const CsrPlan p = csr_plan(N, E, K, kElemBytes[dtype], al);
+  const CsrPlan p = csr_plan(N, E, K, kElemBytes[dtype], al, false, reduce == TS_MIN || reduce == TS_MAX);
   const CsrWs w = csr_workspace(p, B, K, dtype, reduce);
   if (ws == nullptr || ws_bytes < w.total) return TS_ERR_WORKSPACE;
   CsrReduceArgs a;

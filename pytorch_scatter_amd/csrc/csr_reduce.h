@@ -104,8 +104,9 @@ __device__ __forceinline__ void finalize_row(const CsrReduceArgs &a, T *out_b, i
     count_b[row] = count_as<T>(count > 0 ? count : 1);
 }
 
+// sum / mean: at most 80 VGPRs so that six workgroups fit a CU (mean would take 82 and drop to five)
 template <typename T, int VEC, int REDUCE>
-__global__ __launch_bounds__(kBlock) void csr_reduce_kernel(CsrReduceArgs a) {
+__global__ __launch_bounds__(kBlock, (REDUCE == TS_MIN || REDUCE == TS_MAX) ? 4 : 6) void csr_reduce_kernel(CsrReduceArgs a) {
   typedef typename Acc<T>::type A;
   constexpr bool kArg = (REDUCE == TS_MIN || REDUCE == TS_MAX);
   constexpr int U = kLoadsInFlight;
@@ -436,7 +437,8 @@ struct CsrPlan {
   bool small;    // narrow rows: the LDS-staged kernel
 };
 
-inline CsrPlan csr_plan(int64_t N, int64_t E, int64_t K, int elem_bytes, bool aligned16, bool expand = false) {
+inline CsrPlan csr_plan(int64_t N, int64_t E, int64_t K, int elem_bytes, bool aligned16, bool expand = false,
+                        bool with_arg = false) {
   CsrPlan p;
   p.small = false;
   // narrow rows: always for the reduction; for the expansion when a row is at most 8 bytes or
@@ -468,9 +470,11 @@ inline CsrPlan csr_plan(int64_t N, int64_t E, int64_t K, int elem_bytes, bool al
   // same HBM channels and costs ~15 % of the read bandwidth.
   const int W = kBlock / G;
   const int cap = kMaxBlockItems / W;  // LDS holds the row pointers of one tile
-  // measured: reductions like 40 / 56 / 120 items per worker as the input grows; the write-bound
+  // measured: reductions like 24 / 72 / 120 items per worker as the input grows; the write-bound
   // expansion likes short ranges at every size (a workgroup then writes ~100 KB and retires)
-  int want = items >= ((int64_t)8 << 20) ? 120 : (items >= ((int64_t)1 << 20) ? 56 : 40);
+  int want = items >= ((int64_t)8 << 20) ? 120 : (items >= ((int64_t)1 << 20) ? 72 : 24);
+  // min / max carry the positions too (101 VGPRs, four workgroups per CU): fewer, longer ranges
+  if (with_arg && want < 40) want = 40;
   if (expand) want = items >= ((int64_t)32 << 20) ? 8 : 24;
   if (const char *env = getenv("TS_CSR_IPW")) want = atoi(env);  // tuning aid
   if (want > cap) want = cap;
