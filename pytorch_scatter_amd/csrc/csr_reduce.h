@@ -503,9 +503,11 @@ template <typename T, int VEC, int REDUCE>
 int launch_csr_reduce_t(const CsrReduceArgs &a, const CsrPlan &p, int64_t B, hipStream_t stream) {
   dim3 grid((unsigned)p.nblk, (unsigned)p.ychunks, (unsigned)B);
   hipLaunchKernelGGL((csr_reduce_kernel<T, VEC, REDUCE>), grid, dim3(kBlock), 0, stream, a);
-  const int W = kBlock / p.G;
-  dim3 grid2((unsigned)((p.nblk + W - 1) / W), (unsigned)p.ychunks, (unsigned)B);
-  hipLaunchKernelGGL((csr_reduce_fixup_kernel<T, VEC, REDUCE>), grid2, dim3(kBlock), 0, stream, a);
+  if (p.nblk > 1) {  // a single tile has no rows that cross tiles
+    const int W = kBlock / p.G;
+    dim3 grid2((unsigned)((p.nblk + W - 1) / W), (unsigned)p.ychunks, (unsigned)B);
+    hipLaunchKernelGGL((csr_reduce_fixup_kernel<T, VEC, REDUCE>), grid2, dim3(kBlock), 0, stream, a);
+  }
   return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
 }
 

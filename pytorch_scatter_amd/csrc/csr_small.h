@@ -174,9 +174,11 @@ int launch_csr_reduce_small_t(const CsrReduceArgs &a, const CsrPlan &p, int64_t 
   dim3 grid((unsigned)p.nblk, 1, (unsigned)B);
   hipLaunchKernelGGL((csr_reduce_small_kernel<T, REDUCE>), grid, dim3(kBlock),
                      csr_small_lds_bytes(p.BI, a.K, (int)sizeof(T)), stream, a);
-  const int W = kBlock / p.G;
-  dim3 grid2((unsigned)((p.nblk + W - 1) / W), 1, (unsigned)B);
-  hipLaunchKernelGGL((csr_reduce_fixup_kernel<T, 1, REDUCE>), grid2, dim3(kBlock), 0, stream, a);
+  if (p.nblk > 1) {  // a single tile has no rows that cross tiles
+    const int W = kBlock / p.G;
+    dim3 grid2((unsigned)((p.nblk + W - 1) / W), 1, (unsigned)B);
+    hipLaunchKernelGGL((csr_reduce_fixup_kernel<T, 1, REDUCE>), grid2, dim3(kBlock), 0, stream, a);
+  }
   return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
 }
 
