@@ -104,9 +104,14 @@ __device__ __forceinline__ void finalize_row(const CsrReduceArgs &a, T *out_b, i
     count_b[row] = count_as<T>(count > 0 ? count : 1);
 }
 
-// sum / mean: at most 80 VGPRs so that six workgroups fit a CU (mean would take 82 and drop to five)
+// Workgroups per CU the register allocation aims at: six for sum / mean of 4- and 8-byte types (80 VGPRs;
+// mean would take 82 and drop to five, measured 7 % slower on 146 MB inputs). The other instantiations keep
+// the compiler's choice (forcing five on the 16-bit mean cost 3 % on 16 GB inputs).
+template <typename T, int VEC, int REDUCE> constexpr int csr_reduce_min_blocks() {
+  return (REDUCE == TS_SUM || REDUCE == TS_MEAN) && sizeof(T) >= 4 ? 6 : 1;
+}
 template <typename T, int VEC, int REDUCE>
-__global__ __launch_bounds__(kBlock, (REDUCE == TS_MIN || REDUCE == TS_MAX) ? 4 : 6) void csr_reduce_kernel(CsrReduceArgs a) {
+__global__ __launch_bounds__(kBlock, (csr_reduce_min_blocks<T, VEC, REDUCE>())) void csr_reduce_kernel(CsrReduceArgs a) {
   typedef typename Acc<T>::type A;
   constexpr bool kArg = (REDUCE == TS_MIN || REDUCE == TS_MAX);
   constexpr int U = kLoadsInFlight;
