@@ -42,6 +42,8 @@ def parse_args():
                     help="comma list of side configurations to time (C2 is always run)")
     ap.add_argument("--iters", type=int, default=20, help="launches per op in the per-config table")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--probe-scatter", action="store_true",
+                    help="launch sequence for the L2 / atomic counters of the scatter kernels (see probe_scatter)")
     ap.add_argument("--probe", action="store_true",
                     help="counter-collection mode for rocprofv3 --pmc: a few launches of the dominant kernels "
                          "next to copies of known size, nothing timed")
@@ -218,10 +220,45 @@ def probe():
                       "C5": [w5.N, w5.E, w5.K]}))
 
 
+def probe_scatter():
+    """Launch sequence for `rocprofv3 --pmc TCC_HIT_sum TCC_MISS_sum TCC_ATOMIC_sum -- python3 bench.py
+    --probe-scatter`: C1 scatter sum x3, C4 scatter max with K = 1 and K = 32 x2 each, scatter sum and max
+    over the sorted index of C3 with K = 64 x2 each."""
+    import torch
+    import pytorch_scatter_amd as ts
+    from pytorch_scatter_amd import workloads as wl
+    dev = torch.device("cuda:0")
+    done = {}
+    with torch.no_grad():
+        w1 = wl.c1_scatter_sum()
+        src, index = wl.scatter_values(w1, dev), w1.index.to(dev)
+        for _ in range(3):
+            ts.scatter_sum(src, index, 0, None, w1.N)
+        done["C1"] = [w1.N, w1.E, w1.K]
+        for K in (1, 32):
+            w4 = wl.c4_scatter_minmax(K)
+            src, index = wl.scatter_values(w4, dev), w4.index.to(dev)
+            for _ in range(2):
+                ts.scatter_max(src, index, 0, None, w4.N)
+            done[f"C4-K{K}"] = [w4.N, w4.E, w4.K]
+        w3 = wl.c3_segment_coo()
+        index = w3.index.to(dev)
+        src = torch.randn((w3.E, 64), device=dev)
+        for _ in range(2):
+            ts.scatter_sum(src, index, 0, None, w3.N)
+        for _ in range(2):
+            ts.scatter_max(src, index, 0, None, w3.N)
+        done["X-sorted-K64"] = [w3.N, w3.E, 64]
+    torch.cuda.synchronize()
+    print(json.dumps({"probe": "scatter done", **done}))
+
+
 def main():
     args = parse_args()
     if args.probe:
         return probe()
+    if args.probe_scatter:
+        return probe_scatter()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU; every box of this run has a single MI355X, "
               "so --gpus above 1 is not supported (segment / gather ops would shard by node range "
