@@ -291,6 +291,7 @@ int ts_scatter(const void *src, const int64_t *index, void *out, int64_t *arg_ou
   a.lds_cache = env_int("TS_SCATTER_LDS", 1);
   a.lds_epb = env_int("TS_SCATTER_EPB", 0);
   a.run_reduce = env_int("TS_SCATTER_RUNS", 1);
+  a.lds_k1 = env_int("TS_SCATTER_LDS_K1", 1);
   const int full = kVecBytes / kElemBytes[dtype];
   const int vec = (full > 1 && K % full == 0 && aligned16(src)) ? full : 1;
   return dispatch_scatter(dtype, a, reduce, vec, static_cast<hipStream_t>(stream));

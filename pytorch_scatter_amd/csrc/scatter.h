@@ -168,6 +168,7 @@ struct ScatterArgs {
   int lds_cache;       // reduce hot slots in LDS first: 0 never, 1 for large inputs, 2 always
   int64_t lds_epb;     // entries per workgroup chunk of that variant, 0 = default
   int run_reduce = 1;  // sum: pre-reduce runs of equal neighbouring indices in the wavefront
+  int lds_k1 = 1;      // min/max with K == 1: the 512-lane table kernel
 };
 
 // ---- thread -> (edge, column) mapping shared by the scatter kernels ------------
@@ -744,6 +745,113 @@ __global__ __launch_bounds__(kLdsBlock, (TAGS <= 256 ? 4 : 1)) void scatter_key_
   }
 }
 
+// One value per entry (K == 1): the same table, written for occupancy. The general kernel above keeps
+// eight entries with their 64-bit bookkeeping per lane (143 VGPRs, three wavefronts per SIMD) and the
+// counters show it bound by latency, not by L2 or HBM; this one holds 32-bit state only, runs 512 lanes on
+// one 48 KB table (24 wavefronts per CU) and keeps the next batch of loads in flight while the current one
+// goes through the table.
+constexpr int kLdsBlockK1 = 512;
+
+template <typename T, bool IS_MAX>
+__global__ __launch_bounds__(kLdsBlockK1, 2) void scatter_key_lds_k1_kernel(ScatterArgs a, int64_t epb) {
+  constexpr int U = 4;
+  constexpr int mask = kLdsKeys - 1;
+  __shared__ uint64_t s_keys[kLdsKeys];
+  __shared__ int32_t s_tags[kLdsKeys];
+  for (int i = threadIdx.x; i < kLdsKeys; i += kLdsBlockK1) {
+    s_keys[i] = 0;
+    s_tags[i] = -1;
+  }
+  __syncthreads();
+
+  const T *src = static_cast<const T *>(a.src);
+  uint64_t *gkeys = reinterpret_cast<uint64_t *>(a.arg_out);
+  const int64_t lo = (int64_t)blockIdx.x * epb;
+  int64_t hi = lo + epb;
+  if (hi > a.B * a.E) hi = a.B * a.E;
+  const int n_batches = (int)((hi - lo + (int64_t)kLdsBlockK1 * U - 1) / ((int64_t)kLdsBlockK1 * U));
+
+  // loads of one batch: value, node id and position of U entries (entries past the end repeat the last one)
+  auto load = [&](int batch, T *x, int *node, uint32_t *pos) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      int64_t e = lo + ((int64_t)batch * U + u) * kLdsBlockK1 + threadIdx.x;
+      const bool ok = e < hi;
+      if (!ok) e = hi - 1;
+      int64_t b, p;
+      split_edge(e, a.B, a.E, b, p);
+      x[u] = src[e];
+      const int64_t idx = a.index[b * a.sb + p * a.se];
+      node[u] = (ok && idx >= 0 && idx < a.N) ? (int)(b * a.N + idx) : -1;
+      pos[u] = (uint32_t)p;
+    }
+  };
+
+  T x[U], xn[U];
+  int node[U], noden[U];
+  uint32_t pos[U], posn[U];
+  if (n_batches > 0) load(0, x, node, pos);
+  for (int batch = 0; batch < n_batches; ++batch) {
+    load(batch + 1 < n_batches ? batch + 1 : batch, xn, noden, posn);  // unconditional: exact wait counts
+    uint64_t key[U];
+    bool miss[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      miss[u] = false;
+      key[u] = 0;
+      if (node[u] < 0 || Key<T>::is_nan(x[u])) continue;  // NaN never wins
+      key[u] = pack_key<T, IS_MAX>(x[u], 0xFFFFFFFEu - pos[u]);
+      const int row = node[u] & mask;
+      int tag = s_tags[row];
+      if (tag == -1) {
+        const int old = atomicCAS(&s_tags[row], -1, node[u]);
+        tag = old == -1 ? node[u] : old;
+      }
+      if (tag == node[u]) {
+        // value half first (one 32-bit LDS read): an entry below the cached value cannot win
+        const uint32_t cur_hi = reinterpret_cast<const volatile uint32_t *>(&s_keys[row])[1];
+        if ((uint32_t)(key[u] >> 32) >= cur_hi)
+          __hip_atomic_fetch_max(&s_keys[row], key[u], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      } else {
+        miss[u] = true;
+      }
+    }
+    // entries whose table row belongs to another node: all reads first, then the atomics
+    uint64_t cur[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      if (miss[u]) cur[u] = gkeys[node[u]];  // cached read: a stale value only costs a spare atomic
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      if (miss[u] && key[u] > cur[u])
+        __hip_atomic_fetch_max(gkeys + node[u], key[u], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      x[u] = xn[u];
+      node[u] = noden[u];
+      pos[u] = posn[u];
+    }
+  }
+  __syncthreads();
+  // per-node winners of this chunk -> global table
+  constexpr int F = 4;
+  for (int i0 = threadIdx.x; i0 < kLdsKeys; i0 += kLdsBlockK1 * F) {
+    uint64_t key[F], cur[F];
+    int tag[F];
+#pragma unroll
+    for (int j = 0; j < F; ++j) {
+      const int i = i0 + j * kLdsBlockK1;
+      key[j] = i < kLdsKeys ? s_keys[i] : 0;
+      tag[j] = i < kLdsKeys ? s_tags[i] : 0;
+      if (key[j] != 0) cur[j] = gkeys[tag[j]];
+    }
+#pragma unroll
+    for (int j = 0; j < F; ++j)
+      if (key[j] != 0 && key[j] > cur[j])
+        __hip_atomic_fetch_max(gkeys + tag[j], key[j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+
 // ---- sum with a workgroup-private accumulator table ------------------------------
 // Same idea as the packed-key table above, for additions: a hub node that owns
 // 20 % of the entries would otherwise put two million atomics on one address
@@ -1040,6 +1148,22 @@ int launch_scatter_v(const ScatterArgs &a, int reduce, hipStream_t stream) {
           }
           return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
         }
+      }
+      if (use_lds && a.K == 1 && n_src > 0 && a.lds_k1) {
+        // one value per entry: the 512-lane variant; chunks of at least 16384 entries, ~512 workgroups
+        int64_t epb1 = a.lds_epb > 0 ? a.lds_epb : 16384;
+        while (a.lds_epb == 0 && n_edges / epb1 > 1024) epb1 *= 2;
+        const unsigned g1 = (unsigned)((n_edges + epb1 - 1) / epb1);
+        if (is_max) {
+          hipLaunchKernelGGL((scatter_key_init_kernel<T, true>), dim3(g_out), dim3(kBlock), 0, stream, a);
+          hipLaunchKernelGGL((scatter_key_lds_k1_kernel<T, true>), dim3(g1), dim3(kLdsBlockK1), 0, stream, a, epb1);
+          hipLaunchKernelGGL((scatter_key_final_kernel<T, true>), dim3(g_out), dim3(kBlock), 0, stream, a);
+        } else {
+          hipLaunchKernelGGL((scatter_key_init_kernel<T, false>), dim3(g_out), dim3(kBlock), 0, stream, a);
+          hipLaunchKernelGGL((scatter_key_lds_k1_kernel<T, false>), dim3(g1), dim3(kLdsBlockK1), 0, stream, a, epb1);
+          hipLaunchKernelGGL((scatter_key_final_kernel<T, false>), dim3(g_out), dim3(kBlock), 0, stream, a);
+        }
+        return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
       }
       if (is_max) {
         hipLaunchKernelGGL((scatter_key_init_kernel<T, true>), dim3(g_out), dim3(kBlock), 0, stream, a);
