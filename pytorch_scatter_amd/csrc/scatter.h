@@ -168,7 +168,7 @@ struct ScatterArgs {
   int lds_cache;       // reduce hot slots in LDS first: 0 never, 1 for large inputs, 2 always
   int64_t lds_epb;     // entries per workgroup chunk of that variant, 0 = default
   int run_reduce = 1;  // sum: pre-reduce runs of equal neighbouring indices in the wavefront
-  int lds_k1 = 1;      // min/max with K == 1: the 512-lane table kernel
+  int lds_k1 = 1;      // min/max with K == 1: the 1024-lane table kernel
 };
 
 // ---- thread -> (edge, column) mapping shared by the scatter kernels ------------
@@ -747,13 +747,14 @@ __global__ __launch_bounds__(kLdsBlock, (TAGS <= 256 ? 4 : 1)) void scatter_key_
 
 // One value per entry (K == 1): the same table, written for occupancy. The general kernel above keeps
 // eight entries with their 64-bit bookkeeping per lane (143 VGPRs, three wavefronts per SIMD) and the
-// counters show it bound by latency, not by L2 or HBM; this one holds 32-bit state only, runs 512 lanes on
-// one 48 KB table (24 wavefronts per CU) and keeps the next batch of loads in flight while the current one
-// goes through the table.
-constexpr int kLdsBlockK1 = 512;
+// counters show it bound by latency, not by L2 or HBM; this one holds 32-bit state only (58 VGPRs), runs
+// 1024 lanes on one 48 KB table and keeps the next batch of loads in flight while the current one goes
+// through the table.
+
+constexpr int kLdsBlockK1 = 1024;
 
 template <typename T, bool IS_MAX>
-__global__ __launch_bounds__(kLdsBlockK1, 2) void scatter_key_lds_k1_kernel(ScatterArgs a, int64_t epb) {
+__global__ __launch_bounds__(kLdsBlockK1) void scatter_key_lds_k1_kernel(ScatterArgs a, int64_t epb) {
   constexpr int U = 4;
   constexpr int mask = kLdsKeys - 1;
   __shared__ uint64_t s_keys[kLdsKeys];
@@ -1150,9 +1151,16 @@ int launch_scatter_v(const ScatterArgs &a, int reduce, hipStream_t stream) {
         }
       }
       if (use_lds && a.K == 1 && n_src > 0 && a.lds_k1) {
-        // one value per entry: the 512-lane variant; chunks of at least 16384 entries, ~512 workgroups
-        int64_t epb1 = a.lds_epb > 0 ? a.lds_epb : 16384;
-        while (a.lds_epb == 0 && n_edges / epb1 > 1024) epb1 *= 2;
+          // one workgroup of 1024 lanes per CU (or a small multiple): every workgroup writes its table back
+        // once, so fewer and larger chunks win as long as all CUs are busy (measured: 256 chunks of 39 k
+        // entries 83 us, 610 chunks of 16 k entries 98 us for 10 M entries)
+        int dev = 0, cus = 256;
+        if (hipGetDevice(&dev) == hipSuccess) hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+        if (cus < 1) cus = 256;
+        const int64_t rounds = (n_edges + (int64_t)cus * 131072 - 1) / ((int64_t)cus * 131072);
+        int64_t epb1 = (n_edges + cus * rounds - 1) / (cus * rounds);
+        if (epb1 < 16384) epb1 = 16384;
+        if (a.lds_epb > 0) epb1 = a.lds_epb;
         const unsigned g1 = (unsigned)((n_edges + epb1 - 1) / epb1);
         if (is_max) {
           hipLaunchKernelGGL((scatter_key_init_kernel<T, true>), dim3(g_out), dim3(kBlock), 0, stream, a);
