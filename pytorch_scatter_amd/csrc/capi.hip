@@ -324,8 +324,8 @@ int ts_scatter_count(const int64_t *index, float *count, int64_t B, int64_t E, i
     a.lds_epb = env_int("TS_SCATTER_EPB", 0);
     const bool contended = a.lds_cache == 2 || (a.lds_cache == 1 && B * E >= ((int64_t)1 << 20) && B * E >= 32 * B * N);
     if (contended && B * N < 0x7FFFFFFFll) {
-      const int64_t epb = lds_chunk_edges(a.lds_epb, 1, B * E);
-      hipLaunchKernelGGL(scatter_add_lds_kernel<float>, dim3((unsigned)((B * E + epb - 1) / epb)), dim3(kLdsBlock), 0,
+      const int64_t epb = per_cu_chunk_edges(a.lds_epb, B * E, 16384, 131072);
+      hipLaunchKernelGGL(scatter_add_lds_kernel<float>, dim3((unsigned)((B * E + epb - 1) / epb)), dim3(kLdsAddBlock), 0,
                          s, a, kLdsAccRows - 1, epb);
     } else if (env_int("TS_SCATTER_RUNS", 1) && B * N < 0x7FFFFFFFll) {
       // runs of equal neighbouring indices (sorted input) are counted in the wavefront first

@@ -863,21 +863,22 @@ __global__ __launch_bounds__(kLdsBlockK1) void scatter_key_lds_k1_kernel(Scatter
 // entry (the count of scatter mean).
 constexpr int kLdsAcc = 8192;         // 32 KB of fp32 accumulators
 constexpr int kLdsAccRows = 4096;     // 16 KB of tags
+constexpr int kLdsAddBlock = 1024;    // one table per 16 wavefronts: every workgroup adds its table to out once
 
 template <typename T>
-__global__ __launch_bounds__(kLdsBlock) void scatter_add_lds_kernel(ScatterArgs a, int tn_mask, int64_t epb) {
+__global__ __launch_bounds__(kLdsAddBlock) void scatter_add_lds_kernel(ScatterArgs a, int tn_mask, int64_t epb) {
   constexpr int U = 4;
   __shared__ float s_acc[kLdsAcc];
   __shared__ int32_t s_tags[kLdsAccRows];
   const int K = (int)a.K;
   const int tn = tn_mask + 1;
-  for (int i = threadIdx.x; i < tn * K; i += kLdsBlock) s_acc[i] = 0.0f;
-  for (int i = threadIdx.x; i < tn; i += kLdsBlock) s_tags[i] = -1;
+  for (int i = threadIdx.x; i < tn * K; i += kLdsAddBlock) s_acc[i] = 0.0f;
+  for (int i = threadIdx.x; i < tn; i += kLdsAddBlock) s_tags[i] = -1;
   __syncthreads();
 
   const T *src = static_cast<const T *>(a.src);
   T *out = static_cast<T *>(a.out);
-  const EdgeLanes m = edge_lanes(K, kLdsBlock);
+  const EdgeLanes m = edge_lanes(K, kLdsAddBlock);
   const int64_t be_lo = (int64_t)blockIdx.x * epb;
   int64_t be_hi = be_lo + epb;
   if (be_hi > a.B * a.E) be_hi = a.B * a.E;
@@ -914,7 +915,7 @@ __global__ __launch_bounds__(kLdsBlock) void scatter_add_lds_kernel(ScatterArgs 
     }
   }
   __syncthreads();
-  for (int i = threadIdx.x; i < tn * K; i += kLdsBlock) {
+  for (int i = threadIdx.x; i < tn * K; i += kLdsAddBlock) {
     const float v = s_acc[i];
     if (v == 0.0f) continue;
     const int row = i / K;
@@ -1022,6 +1023,19 @@ inline int64_t lds_chunk_edges(int64_t forced, int64_t K, int64_t n_edges) {
   return epb < 64 ? 64 : epb;
 }
 
+// Entries per workgroup when one large workgroup per CU (or a small multiple of the CU count) shares a
+// table: the table is written back once per workgroup, so fewer and larger chunks win as long as all CUs
+// are busy (measured for min/max with K = 1: 256 chunks of 39 k entries 83 us, 610 chunks of 16 k 98 us).
+inline int64_t per_cu_chunk_edges(int64_t forced, int64_t n_edges, int64_t min_epb, int64_t max_epb) {
+  if (forced > 0) return forced;
+  int dev = 0, cus = 256;
+  if (hipGetDevice(&dev) == hipSuccess) hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+  if (cus < 1) cus = 256;
+  const int64_t rounds = (n_edges + (int64_t)cus * max_epb - 1) / ((int64_t)cus * max_epb);
+  const int64_t epb = (n_edges + cus * rounds - 1) / (cus * rounds);
+  return epb < min_epb ? min_epb : epb;
+}
+
 // workgroups needed so that every edge is visited once: `block` threads cover
 // block / min(kv, block) edges per pass and U passes per loop trip
 inline unsigned scatter_grid(int64_t n_edges, int64_t kv, int block, int U) {
@@ -1056,9 +1070,10 @@ int launch_scatter_v(const ScatterArgs &a, int reduce, hipStream_t stream) {
           const bool use_lds = a.lds_cache && a.sk == 0 && tn >= 64 && a.B * a.N < 0x7FFFFFFFll &&
                                (a.lds_cache == 2 || (n_src >= ((int64_t)1 << 20) && n_edges >= 32 * a.B * a.N));
           if (use_lds) {
-            const int64_t epb = lds_chunk_edges(a.lds_epb, a.K, n_edges);
+            const int64_t epb = per_cu_chunk_edges(a.lds_epb, n_edges, 16384 / a.K > 256 ? 16384 / a.K : 256,
+                                                   131072 / a.K > 2048 ? 131072 / a.K : 2048);
             hipLaunchKernelGGL(scatter_add_lds_kernel<T>, dim3((unsigned)((n_edges + epb - 1) / epb)),
-                               dim3(kLdsBlock), 0, stream, a, tn - 1, epb);
+                               dim3(kLdsAddBlock), 0, stream, a, tn - 1, epb);
             return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
           }
         }
@@ -1151,16 +1166,7 @@ int launch_scatter_v(const ScatterArgs &a, int reduce, hipStream_t stream) {
         }
       }
       if (use_lds && a.K == 1 && n_src > 0 && a.lds_k1) {
-          // one workgroup of 1024 lanes per CU (or a small multiple): every workgroup writes its table back
-        // once, so fewer and larger chunks win as long as all CUs are busy (measured: 256 chunks of 39 k
-        // entries 83 us, 610 chunks of 16 k entries 98 us for 10 M entries)
-        int dev = 0, cus = 256;
-        if (hipGetDevice(&dev) == hipSuccess) hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
-        if (cus < 1) cus = 256;
-        const int64_t rounds = (n_edges + (int64_t)cus * 131072 - 1) / ((int64_t)cus * 131072);
-        int64_t epb1 = (n_edges + cus * rounds - 1) / (cus * rounds);
-        if (epb1 < 16384) epb1 = 16384;
-        if (a.lds_epb > 0) epb1 = a.lds_epb;
+          const int64_t epb1 = per_cu_chunk_edges(a.lds_epb, n_edges, 16384, 131072);
         const unsigned g1 = (unsigned)((n_edges + epb1 - 1) / epb1);
         if (is_max) {
           hipLaunchKernelGGL((scatter_key_init_kernel<T, true>), dim3(g_out), dim3(kBlock), 0, stream, a);
