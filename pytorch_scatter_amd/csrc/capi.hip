@@ -134,6 +134,7 @@ const char *ts_error_string(int status) {
 
 int64_t ts_hip_version(void) { return HIP_VERSION; }
 
+
 size_t ts_segment_csr_workspace_bytes(int64_t B, int64_t N, int64_t E, int64_t K, int dtype, int reduce) {
   if (!valid_dtype(dtype) || !sizes_ok(B, N, E, K)) return 0;
   // the plan may fall back to one element per lane for unaligned buffers; the

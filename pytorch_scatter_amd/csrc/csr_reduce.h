@@ -61,29 +61,32 @@ __device__ __forceinline__ void reduce_step(A &acc, int32_t &arg, A v, int32_t e
 }
 
 // Write one finished row slice. `count` is the full length of the row.
-template <typename T, int VEC, int REDUCE>
+// ACCUM: 0 = `out` is overwritten (known at compile time: the row-end code sits in divergent control flow,
+// where every instruction counts), -1 = decided by a.accumulate at run time.
+template <typename T, int VEC, int REDUCE, int ACCUM = -1>
 __device__ __forceinline__ void finalize_row(const CsrReduceArgs &a, T *out_b, int64_t *arg_b,
                                              T *count_b, int64_t row, int64_t col, int lg,
                                              const typename Acc<T>::type *acc, const int32_t *arg,
                                              int64_t count, bool col_ok) {
   typedef typename Acc<T>::type A;
   if (!col_ok) return;
-  if (a.accumulate && count == 0) return;  // rows without entries keep their content
+  const bool accumulate = ACCUM < 0 ? a.accumulate != 0 : ACCUM != 0;
+  if (accumulate && count == 0) return;  // rows without entries keep their content
   T *op = out_b + row * a.K + col;
   Vec<T, VEC> o;
   int64_t oa[VEC];
   Vec<T, VEC> prev;
-  if (a.accumulate) prev = load_vec<T, VEC>(op);
+  if (accumulate) prev = load_vec<T, VEC>(op);
 #pragma unroll
   for (int v = 0; v < VEC; ++v) {
     A x = acc[v];
     if (REDUCE == TS_SUM || REDUCE == TS_MEAN) {
-      if (a.accumulate) x = to_acc<T>(prev.v[v]) + x;
+      if (accumulate) x = to_acc<T>(prev.v[v]) + x;
       T t = from_acc<T>(x);
       if (REDUCE == TS_MEAN && count > 1) t = div_elem<T>(t, count_as<T>(count));  // x / 1 == x
       o.v[v] = t;
     } else {
-      if (a.accumulate) {
+      if (accumulate) {
         const A p = to_acc<T>(prev.v[v]);
         const bool beats = (REDUCE == TS_MIN) ? (x < p) : (x > p);
         o.v[v] = beats ? from_acc<T>(x) : prev.v[v];
@@ -110,13 +113,13 @@ __device__ __forceinline__ void finalize_row(const CsrReduceArgs &a, T *out_b, i
 template <typename T, int VEC, int REDUCE> constexpr int csr_reduce_min_blocks() {
   return (REDUCE == TS_SUM || REDUCE == TS_MEAN) && sizeof(T) >= 4 ? 6 : 1;
 }
-template <typename T, int VEC, int REDUCE>
+template <typename T, int VEC, int REDUCE, int ACCUM>
 __global__ __launch_bounds__(kBlock, (csr_reduce_min_blocks<T, VEC, REDUCE>())) void csr_reduce_kernel(CsrReduceArgs a) {
   typedef typename Acc<T>::type A;
   constexpr bool kArg = (REDUCE == TS_MIN || REDUCE == TS_MAX);
   constexpr int U = kLoadsInFlight;
 
-  __shared__ int32_t s_ptr[kMaxBlockItems + 2];
+  __shared__ int32_t s_ptr[kMaxBlockItems + 4];  // row pointers of the tile + one sentinel
   __shared__ A s_val[2 * kBlock * VEC];
   __shared__ int32_t s_arg[kArg ? 2 * kBlock * VEC : 1];
   __shared__ int32_t s_head_row[kBlock];    // local row of the head partial, -1: none
@@ -159,6 +162,7 @@ __global__ __launch_bounds__(kBlock, (csr_reduce_min_blocks<T, VEC, REDUCE>())) 
   const int64_t last = i1 + 1 < a.N ? i1 + 1 : a.N;
   const int nload = (int)(last - i0) + 1;  // ptr[i0 .. last]
   for (int t = tid; t < nload; t += kBlock) s_ptr[t] = (int32_t)(ptr[i0 + t] - j0);
+  if (tid == 0) s_ptr[nload] = INT32_MAX;  // rows past the last one never end
   s_head_row[tid] = -1;
   s_tail_row[tid] = -1;
   __syncthreads();
@@ -175,7 +179,7 @@ __global__ __launch_bounds__(kBlock, (csr_reduce_min_blocks<T, VEC, REDUCE>())) 
   const int je0 = dw0 - ri0;
   const int je1 = dw1 - ri1;
 
-  auto row_end = [&](int r) -> int32_t { return (r + 1 < nload) ? s_ptr[r + 1] : INT32_MAX; };
+  auto row_end = [&](int r) -> int32_t { return s_ptr[r + 1]; };  // r + 1 <= nload: the sentinel at the latest
 
   A acc[VEC];
   int32_t arg[VEC];
@@ -203,8 +207,8 @@ __global__ __launch_bounds__(kBlock, (csr_reduce_min_blocks<T, VEC, REDUCE>())) 
       }
       if (lg == 0) { s_head_row[w] = r; s_head_closes[w] = 1; }
     } else {
-      finalize_row<T, VEC, REDUCE>(a, out_b, arg_b, count_b, i0 + r, col, lg, acc, arg,
-                                   (int64_t)rend - (int64_t)s_ptr[r], col_ok);
+      finalize_row<T, VEC, REDUCE, ACCUM>(a, out_b, arg_b, count_b, i0 + r, col, lg, acc, arg,
+                                   (int64_t)(int32_t)(rend - s_ptr[r]), col_ok);  // a row length fits 32 bits
     }
 #pragma unroll
     for (int v = 0; v < VEC; ++v) acc[v] = acc_init<A, REDUCE>();
@@ -265,6 +269,8 @@ __global__ __launch_bounds__(kBlock, (csr_reduce_min_blocks<T, VEC, REDUCE>())) 
       }
     }
   }
+  // default: the tile leaves no open row; the worker that does overwrites this after the barrier
+  if (tid == 0 && blockIdx.y == 0) a.ws_meta[(b * a.nblk + blockIdx.x) * 4 + 2] = -1;
   __syncthreads();
 
   // ---- combine partials of rows that cross worker boundaries, in edge order
@@ -296,7 +302,7 @@ __global__ __launch_bounds__(kBlock, (csr_reduce_min_blocks<T, VEC, REDUCE>())) 
       closed = s_head_closes[ww] != 0;
     }
     if (closed) {
-      finalize_row<T, VEC, REDUCE>(a, out_b, arg_b, count_b, i0 + row, col, lg, acc, arg,
+      finalize_row<T, VEC, REDUCE, ACCUM>(a, out_b, arg_b, count_b, i0 + row, col, lg, acc, arg,
                                    (int64_t)s_ptr[row + 1] - (int64_t)s_ptr[row], col_ok);
     } else {
       if (col_ok) {
@@ -335,18 +341,6 @@ __global__ __launch_bounds__(kBlock, (csr_reduce_min_blocks<T, VEC, REDUCE>())) 
       meta[0] = -1;
       meta[1] = 0;
     }
-  }
-  // tiles that leave no open row say so (exactly one worker can hold the open row)
-  if (tid == 0 && blockIdx.y == 0) {
-    bool open = false;
-    for (int ww = 0; ww < W; ++ww) {
-      if (s_tail_row[ww] < 0) continue;
-      bool closed = false;
-      for (int w2 = ww + 1; w2 < W && !closed; ++w2)
-        if (s_head_row[w2] >= 0) closed = s_head_closes[w2] != 0;
-      if (!closed) open = true;
-    }
-    if (!open) meta[2] = -1;
   }
 }
 
@@ -507,7 +501,10 @@ inline size_t csr_ws_bytes(const CsrPlan &p, int64_t B, int64_t K, int acc_bytes
 template <typename T, int VEC, int REDUCE>
 int launch_csr_reduce_t(const CsrReduceArgs &a, const CsrPlan &p, int64_t B, hipStream_t stream) {
   dim3 grid((unsigned)p.nblk, (unsigned)p.ychunks, (unsigned)B);
-  hipLaunchKernelGGL((csr_reduce_kernel<T, VEC, REDUCE>), grid, dim3(kBlock), 0, stream, a);
+  if (a.accumulate)
+    hipLaunchKernelGGL((csr_reduce_kernel<T, VEC, REDUCE, -1>), grid, dim3(kBlock), 0, stream, a);
+  else
+    hipLaunchKernelGGL((csr_reduce_kernel<T, VEC, REDUCE, 0>), grid, dim3(kBlock), 0, stream, a);
   if (p.nblk > 1) {  // a single tile has no rows that cross tiles
     const int W = kBlock / p.G;
     dim3 grid2((unsigned)((p.nblk + W - 1) / W), (unsigned)p.ychunks, (unsigned)B);
