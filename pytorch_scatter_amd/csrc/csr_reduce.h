@@ -64,15 +64,13 @@ __device__ __forceinline__ void reduce_step(A &acc, int32_t &arg, A v, int32_t e
 // ACCUM: 0 = `out` is overwritten (known at compile time: the row-end code sits in divergent control flow,
 // where every instruction counts), -1 = decided by a.accumulate at run time.
 template <typename T, int VEC, int REDUCE, int ACCUM = -1>
-__device__ __forceinline__ void finalize_row(const CsrReduceArgs &a, T *out_b, int64_t *arg_b,
-                                             T *count_b, int64_t row, int64_t col, int lg,
-                                             const typename Acc<T>::type *acc, const int32_t *arg,
-                                             int64_t count, bool col_ok) {
+__device__ __forceinline__ void finalize_row_at(const CsrReduceArgs &a, T *op, int64_t *ap, T *count_slot,
+                                                const typename Acc<T>::type *acc, const int32_t *arg,
+                                                int64_t count) {
+  // op / ap: the row's slice in out / arg_out; count_slot: where the row's count goes (mean with a count output)
   typedef typename Acc<T>::type A;
-  if (!col_ok) return;
   const bool accumulate = ACCUM < 0 ? a.accumulate != 0 : ACCUM != 0;
   if (accumulate && count == 0) return;  // rows without entries keep their content
-  T *op = out_b + row * a.K + col;
   Vec<T, VEC> o;
   int64_t oa[VEC];
   Vec<T, VEC> prev;
@@ -99,12 +97,22 @@ __device__ __forceinline__ void finalize_row(const CsrReduceArgs &a, T *out_b, i
   }
   store_vec<T, VEC>(op, o);
   if (REDUCE == TS_MIN || REDUCE == TS_MAX) {
-    int64_t *ap = arg_b + row * a.K + col;
 #pragma unroll
     for (int v = 0; v < VEC; ++v) ap[v] = oa[v];
   }
-  if (REDUCE == TS_MEAN && count_b != nullptr && col == 0 && lg == 0)
-    count_b[row] = count_as<T>(count > 0 ? count : 1);
+  if (REDUCE == TS_MEAN && count_slot != nullptr) *count_slot = count_as<T>(count > 0 ? count : 1);
+}
+
+template <typename T, int VEC, int REDUCE, int ACCUM = -1>
+__device__ __forceinline__ void finalize_row(const CsrReduceArgs &a, T *out_b, int64_t *arg_b,
+                                             T *count_b, int64_t row, int64_t col, int lg,
+                                             const typename Acc<T>::type *acc, const int32_t *arg,
+                                             int64_t count, bool col_ok) {
+  if (!col_ok) return;
+  constexpr bool kArg = REDUCE == TS_MIN || REDUCE == TS_MAX;
+  finalize_row_at<T, VEC, REDUCE, ACCUM>(a, out_b + row * a.K + col, kArg ? arg_b + row * a.K + col : nullptr,
+                                         (count_b != nullptr && col == 0 && lg == 0) ? count_b + row : nullptr,
+                                         acc, arg, count);
 }
 
 // Workgroups per CU the register allocation aims at: six for sum / mean of 4- and 8-byte types (80 VGPRs;
@@ -162,7 +170,7 @@ __global__ __launch_bounds__(kBlock, (csr_reduce_min_blocks<T, VEC, REDUCE>())) 
   const int64_t last = i1 + 1 < a.N ? i1 + 1 : a.N;
   const int nload = (int)(last - i0) + 1;  // ptr[i0 .. last]
   for (int t = tid; t < nload; t += kBlock) s_ptr[t] = (int32_t)(ptr[i0 + t] - j0);
-  if (tid == 0) s_ptr[nload] = INT32_MAX;  // rows past the last one never end
+  if (tid == 0) { s_ptr[nload] = INT32_MAX; s_ptr[nload + 1] = INT32_MAX; }  // rows past the last one never end
   s_head_row[tid] = -1;
   s_tail_row[tid] = -1;
   __syncthreads();
@@ -179,7 +187,7 @@ __global__ __launch_bounds__(kBlock, (csr_reduce_min_blocks<T, VEC, REDUCE>())) 
   const int je0 = dw0 - ri0;
   const int je1 = dw1 - ri1;
 
-  auto row_end = [&](int r) -> int32_t { return s_ptr[r + 1]; };  // r + 1 <= nload: the sentinel at the latest
+  auto row_end = [&](int r) -> int32_t { return s_ptr[r + 1]; };  // r + 1 <= nload + 1: a sentinel at the latest
 
   A acc[VEC];
   int32_t arg[VEC];
@@ -196,7 +204,12 @@ __global__ __launch_bounds__(kBlock, (csr_reduce_min_blocks<T, VEC, REDUCE>())) 
   int32_t *my_tail_arg = s_arg + (kArg ? (size_t)kBlock * VEC + (size_t)w * CW + lg * VEC : 0);
 
   int r = ri0;
+  T *op_row = out_b + (i0 + r) * a.K + (col_ok ? col : 0);
+  int64_t *ap_row = kArg ? arg_b + (i0 + r) * a.K + (col_ok ? col : 0) : nullptr;
+  T *cp_row = (count_b != nullptr && col == 0 && lg == 0) ? count_b + (i0 + r) : nullptr;
+  int32_t rbeg = s_ptr[r];       // first edge of row r
   int32_t rend = row_end(r);
+  int32_t rnext = row_end(r + 1);  // read one row ahead: a row end then never waits for LDS
 
   auto flush = [&]() {
     if (r == ri0 && head_open) {
@@ -206,14 +219,19 @@ __global__ __launch_bounds__(kBlock, (csr_reduce_min_blocks<T, VEC, REDUCE>())) 
         if (kArg) my_head_arg[v] = arg[v];
       }
       if (lg == 0) { s_head_row[w] = r; s_head_closes[w] = 1; }
-    } else {
-      finalize_row<T, VEC, REDUCE, ACCUM>(a, out_b, arg_b, count_b, i0 + r, col, lg, acc, arg,
-                                   (int64_t)(int32_t)(rend - s_ptr[r]), col_ok);  // a row length fits 32 bits
+    } else if (col_ok) {
+      finalize_row_at<T, VEC, REDUCE, ACCUM>(a, op_row, ap_row, cp_row, acc, arg,
+                                             (int64_t)(int32_t)(rend - rbeg));  // a row length fits 32 bits
     }
 #pragma unroll
     for (int v = 0; v < VEC; ++v) acc[v] = acc_init<A, REDUCE>();
     ++r;
-    rend = row_end(r);
+    op_row += a.K;  // the slices of row r in out / arg_out / count: no 64-bit multiply per row end
+    if (kArg) ap_row += a.K;
+    if (cp_row != nullptr) ++cp_row;
+    rbeg = rend;
+    rend = rnext;
+    rnext = row_end(r + 1);
   };
 
   const int64_t col_ld = col_ok ? col : 0;  // idle lanes re-read column 0
