@@ -92,6 +92,38 @@ def test_c3_segment_coo_max_against_scatter_max(env):
     assert torch.equal(out, out3) and torch.equal(arg, arg3)
 
 
+@pytest.mark.parametrize("K", [1, 4, 8, 16])
+def test_c3_graph_narrow_rows(env, K):
+    """The 9 M-entry graph of C3 with 1 to 16 values per entry: the LDS-staged reduction, the
+    one-lane-per-16-bytes expansion and the run-combining scatter against each other and torch."""
+    ts, wl = env
+    w = wl.c3_segment_coo()
+    g = torch.Generator(device=DEV).manual_seed(K)
+    src = torch.randint(-8, 9, (w.E, K), generator=g, device=DEV).float()   # many exact ties, exact sums
+    indptr, index = w.indptr.to(DEV), w.index.to(DEV)
+    deg = indptr[1:] - indptr[:-1]
+    want = torch.zeros(w.N, K, device=DEV).index_add_(0, index, src)
+    got = ts.segment_csr(src, indptr, None, "sum")
+    assert torch.equal(got, want)                                          # small integers: exact in fp32
+    assert torch.equal(ts.segment_coo(src, index, None, w.N, "sum"), want)
+    assert torch.equal(ts.scatter_sum(src, index, 0, None, w.N), want)     # sorted index: runs combined in the wavefront
+    out, arg = ts.segment_max_csr(src, indptr)
+    out2, arg2 = ts.scatter_max(src, index, 0, None, w.N)
+    assert torch.equal(out, out2) and torch.equal(arg, arg2)
+    full = deg > 0
+    a = arg[full]
+    assert bool((a < w.E).all()) and torch.equal(torch.gather(src, 0, a), out[full])
+    assert bool((arg[~full] == w.E).all()) and bool((out[~full] == 0).all())
+    # first position wins: no earlier entry of the row holds the same value
+    first = indptr[:-1][full].unsqueeze(1)
+    probe = torch.minimum(a - 1, a).clamp(min=0)
+    earlier_same = (torch.gather(src, 0, probe) == out[full]) & (a - 1 >= first)
+    assert not bool(earlier_same.any())
+    back = ts.gather_csr(got, indptr)
+    assert torch.equal(back, torch.repeat_interleave(got, deg, dim=0))
+    assert torch.equal(back, ts.gather_coo(got, index))
+
+
 @pytest.mark.parametrize("K", [1, 32])
 @pytest.mark.parametrize("reduce", ["max", "min"])
 def test_c4_contended_scatter_against_sorted_reduction(env, K, reduce):
