@@ -182,7 +182,7 @@ int ts_segment_mean_csr_backward(const void *grad_out, const int64_t *indptr, vo
   if (!is_float_dtype(dtype)) return TS_ERR_UNSUPPORTED;
   if (B * E * K == 0 || N == 0) return TS_OK;
   if (!grad_out || !indptr || !grad_in) return TS_ERR_BAD_ARG;
-  const CsrPlan p = csr_plan(N, E, K, kElemBytes[dtype], aligned16(grad_out) && aligned16(grad_in), true);
+  const CsrPlan p = csr_plan(N, E, K, kElemBytes[dtype], aligned16(grad_out) && aligned16(grad_in), true, true);
   CsrGatherArgs a;
   a.src = grad_out;
   a.indptr = indptr;

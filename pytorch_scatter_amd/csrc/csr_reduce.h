@@ -454,6 +454,7 @@ struct CsrPlan {
   bool small;    // narrow rows: the LDS-staged kernel
 };
 
+// with_arg: the reduction is min / max (positions carried along); for the expansion: the variant that divides
 inline CsrPlan csr_plan(int64_t N, int64_t E, int64_t K, int elem_bytes, bool aligned16, bool expand = false,
                         bool with_arg = false) {
   CsrPlan p;
@@ -492,7 +493,10 @@ inline CsrPlan csr_plan(int64_t N, int64_t E, int64_t K, int elem_bytes, bool al
   int want = items >= ((int64_t)8 << 20) ? 120 : (items >= ((int64_t)1 << 20) ? 72 : 24);
   // min / max carry the positions too (101 VGPRs, four workgroups per CU): fewer, longer ranges
   if (with_arg && want < 40) want = 40;
-  if (expand) want = items >= ((int64_t)32 << 20) ? 8 : 24;
+  // expansion of very large inputs: 6 items per worker for the plain copy, 8 for the variant that divides
+  // (with_arg doubles as that flag here); both then reach 70.5 % of peak on 62 M entries of 256 bytes, the
+  // neighbouring values 63-67 %
+  if (expand) want = items >= ((int64_t)32 << 20) ? (with_arg ? 8 : 6) : 24;
   if (const char *env = getenv("TS_CSR_IPW")) want = atoi(env);  // tuning aid
   if (want > cap) want = cap;
   int ipw = want >= 24 ? (((want / 8) - 1) | 1) * 8 : want;
