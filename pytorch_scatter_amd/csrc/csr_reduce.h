@@ -483,14 +483,13 @@ inline CsrPlan csr_plan(int64_t N, int64_t E, int64_t K, int elem_bytes, bool al
   p.G = G;
   p.ychunks = (int)((K + (int64_t)G * p.vec - 1) / ((int64_t)G * p.vec));
   const int64_t items = N + E;
-  // Items per worker: an odd multiple of 8. Workers of a tile start their
-  // streams ipw rows apart; a power-of-two distance puts all of them on the
-  // same HBM channels and costs ~15 % of the read bandwidth.
   const int W = kBlock / G;
   const int cap = kMaxBlockItems / W;  // LDS holds the row pointers of one tile
-  // measured: reductions like 24 / 72 / 120 items per worker as the input grows; the write-bound
-  // expansion likes short ranges at every size (a workgroup then writes ~100 KB and retires)
-  int want = items >= ((int64_t)8 << 20) ? 120 : (items >= ((int64_t)1 << 20) ? 72 : 24);
+  // Items per worker, from sweeps on 146 MB / 366 MB / 6 GB / 16 GB inputs (the curve is flat within 1-2 %
+  // except for a few sharp optima): reductions 24 below 1 M items (more, shorter workgroups: the kernel is
+  // latency bound there), 72 up to 32 M, 64 above; the write-bound expansion likes short ranges at every size
+  // (a workgroup then writes ~100 KB and retires).
+  int want = items >= ((int64_t)32 << 20) ? 64 : (items >= ((int64_t)1 << 20) ? 72 : 24);
   // min / max carry the positions too (101 VGPRs, four workgroups per CU): fewer, longer ranges
   if (with_arg && want < 40) want = 40;
   // expansion of very large inputs: 6 items per worker for the plain copy, 8 for the variant that divides
@@ -499,7 +498,7 @@ inline CsrPlan csr_plan(int64_t N, int64_t E, int64_t K, int elem_bytes, bool al
   if (expand) want = items >= ((int64_t)32 << 20) ? (with_arg ? 8 : 6) : 24;
   if (const char *env = getenv("TS_CSR_IPW")) want = atoi(env);  // tuning aid
   if (want > cap) want = cap;
-  int ipw = want >= 24 ? (((want / 8) - 1) | 1) * 8 : want;
+  int ipw = want;
   if (ipw > cap) ipw = cap;
   if (ipw < 1) ipw = 1;
   p.ipw = ipw;
