@@ -22,6 +22,7 @@
 #pragma once
 
 #include <limits>
+#include <type_traits>
 #include <stdlib.h>
 
 #include "device_utils.h"
@@ -418,7 +419,7 @@ template <typename T, int C_>
 struct AddRun {
   typedef typename Acc<T>::type A;
   static constexpr int C = C_;
-  static constexpr int EW = sizeof(T) == 2 ? 2 : 1;
+  static constexpr int EW = sizeof(T) < 4 ? 4 / (int)sizeof(T) : 1;  // columns per atomic: one 32-bit word
   static constexpr int U = 4;
   const T *src;
   T *out;
@@ -437,10 +438,27 @@ struct AddRun {
   __device__ void combine(A &x, const A &y) const { x = x + y; }
   __device__ void emit(int node, int64_t col, const A *x) const {
     T *p = out + (int64_t)node * K + col;
-#ifdef TS_RUN_NO_EMIT
-    if (node != 0x12345) return;
-#endif
-    if constexpr (EW == 2) {
+    if constexpr (std::is_integral<T>::value && sizeof(T) < 4) {
+      // 8- and 16-bit integers: one compare-and-swap on the 32-bit word that holds EW neighbouring columns
+      // (a CAS per element would make the lanes of one word fight each other)
+      typedef typename std::make_unsigned<T>::type UT;
+      constexpr int bits = 8 * (int)sizeof(T);
+      uint32_t *word = reinterpret_cast<uint32_t *>(p);
+      uint32_t old = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      while (true) {
+        uint32_t nw = 0;
+#pragma unroll
+        for (int j = 0; j < EW; ++j) {
+          const T cur = (T)(UT)(old >> (bits * j));
+          const T nv = (T)(cur + x[j]);
+          nw |= (uint32_t)(UT)nv << (bits * j);
+        }
+        if (nw == old) return;
+        if (__hip_atomic_compare_exchange_strong(word, &old, nw, __ATOMIC_RELAXED, __ATOMIC_RELAXED,
+                                                 __HIP_MEMORY_SCOPE_AGENT))
+          return;
+      }
+    } else if constexpr (EW == 2) {
       if constexpr (__is_same(T, bf16_t)) {
         typedef short v2s __attribute__((ext_vector_type(2)));
         v2s pk;
@@ -1077,14 +1095,13 @@ int launch_scatter_v(const ScatterArgs &a, int reduce, hipStream_t stream) {
             return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
           }
         }
-        if constexpr (__is_same(T, float) || __is_same(T, double) || __is_same(T, int32_t) ||
-                      __is_same(T, int64_t) || __is_same(T, bf16_t) || __is_same(T, f16_t)) {
-          // one index per row: sum runs of equal neighbouring indices in the wavefront first
-          constexpr bool k16 = sizeof(T) == 2;
-          const bool pair_ok = a.K % 2 == 0 && (reinterpret_cast<uintptr_t>(a.out) & 3) == 0 &&
-                               (reinterpret_cast<uintptr_t>(a.src) & 3) == 0;
-          if (a.run_reduce && a.sk == 0 && a.B * a.N < 0x7FFFFFFFll && (!k16 || pair_ok)) {
-            constexpr int CN = k16 ? 2 : 1;               // columns per lane without 16-byte loads
+        {
+          // one index per row: sum runs of equal neighbouring indices in the wavefront first.
+          // Element types below 32 bits are written one 32-bit word (2 or 4 columns) at a time.
+          constexpr int CN = sizeof(T) < 4 ? 4 / (int)sizeof(T) : 1;  // columns per lane without 16-byte loads
+          const bool word_ok = CN == 1 || (a.K % CN == 0 && (reinterpret_cast<uintptr_t>(a.out) & 3) == 0 &&
+                                           (reinterpret_cast<uintptr_t>(a.src) & 3) == 0);
+          if (a.run_reduce && a.sk == 0 && a.B * a.N < 0x7FFFFFFFll && word_ok) {
             constexpr int C = VEC > 1 ? VEC : CN;
             // 16-byte loads pay once the instruction rate limits the stream; small inputs are bound by
             // latency and do better with one atomic per lane straight from registers

@@ -530,7 +530,8 @@ def run_index(kind, rng, E, N):
 
 @pytest.mark.parametrize("shape,kind,dtype", product(
     RUN_SHAPES, ["sorted", "hub", "pieces"],
-    [torch.int32, torch.int64, torch.float32, torch.float64, torch.bfloat16, torch.float16]))
+    [torch.int32, torch.int64, torch.float32, torch.float64, torch.bfloat16, torch.float16,
+     torch.int16, torch.int8, torch.uint8]))
 def test_scatter_sum_runs_of_equal_indices(capi, oracle, shape, kind, dtype):
     """Sum with the wavefront pre-reduction of neighbouring equal indices: exact for
     integers, within tolerance of the exact sum for floats; count shares the kernel."""
