@@ -181,6 +181,36 @@ int ts_arg_backward(const void *grad_out, const int64_t *arg, void *grad_in,
                     int64_t B, int64_t N, int64_t E, int64_t K, int dtype,
                     ts_stream_t stream);
 
+/* ---------------------------------------------------------- group softmax
+ * Softmax / log-softmax over the entries that share an index, one index per
+ * row (index[b*sb + e*se] addresses all K columns of entry e):
+ *   m = group max, s = group sum of exp(src - m)
+ *   log_space == 0:  out = exp(src - m) / s
+ *   log_space != 0:  out = (src - m) - log(s + eps)
+ * Replaces, in three passes over src, the op sequences of
+ * torch_scatter/composite/softmax.py:16-29 and :45-59 (scatter_max, gather,
+ * sub, exp, scatter_sum, gather, div); the reference has no single launcher
+ * for it. Floating types only. Entries whose index lies outside [0, N) belong
+ * to no group and yield 0. The backward call takes the forward result:
+ *   log_space == 0:  grad_in = result * (grad_out - S),  S = group sum of result * grad_out
+ *   log_space != 0:  grad_in = grad_out - exp(result) * G,  G = group sum of grad_out
+ * workspace: ts_group_softmax_workspace_bytes() bytes of device scratch,
+ * 16-byte aligned. TS_ERR_UNSUPPORTED when B * N does not fit 31 bits.
+ */
+size_t ts_group_softmax_workspace_bytes(int64_t B, int64_t N, int64_t K,
+                                        int dtype);
+int ts_group_softmax(const void *src, const int64_t *index, void *out,
+                     int64_t B, int64_t E, int64_t K, int64_t N,
+                     int64_t index_stride_b, int64_t index_stride_e, int dtype,
+                     int log_space, double eps, void *workspace,
+                     size_t workspace_bytes, ts_stream_t stream);
+int ts_group_softmax_backward(const void *result, const void *grad_out,
+                              const int64_t *index, void *grad_in, int64_t B,
+                              int64_t E, int64_t K, int64_t N,
+                              int64_t index_stride_b, int64_t index_stride_e,
+                              int dtype, int log_space, void *workspace,
+                              size_t workspace_bytes, ts_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

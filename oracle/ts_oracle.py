@@ -355,3 +355,92 @@ def segment_mean_coo_backward(grad_out, index, count, src_shape):
         count = count.unsqueeze(-1)
     grad_in.true_divide_(count)
     return grad_in
+
+
+# ------------------------------------------------- group statistics (Python layer)
+# The reference composes these in Python from scatter_max / scatter_sum, gather
+# and ATen elementwise ops; the same sequence here, on the oracle's scatter.
+# Pinned by the reference's own checks (test/composite/test_softmax.py:6-54,
+# test_logsumexp.py:5-45, test_std.py:5-20: per-group torch.softmax /
+# log_softmax / logsumexp / std) in tests/test_oracle_golden.py.
+def _py_broadcast(index, other, dim):
+    """torch_scatter/utils.py:4-13."""
+    dim = other.dim() + dim if dim < 0 else dim
+    return broadcast(index, other, dim), dim
+
+
+def scatter_softmax(src, index, dim=-1, dim_size=None):
+    """torch_scatter/composite/softmax.py:8-29."""
+    index, dim = _py_broadcast(index, src, dim)
+    group_max = scatter(src, index, dim, None, dim_size, "max")[0]
+    e = (src - group_max.gather(dim, index)).exp_()
+    total = scatter(e, index, dim, None, dim_size, "sum")[0]
+    return e.div(total.gather(dim, index))
+
+
+def scatter_log_softmax(src, index, dim=-1, eps=1e-12, dim_size=None):
+    """torch_scatter/composite/softmax.py:32-59."""
+    index, dim = _py_broadcast(index, src, dim)
+    group_max = scatter(src, index, dim, None, dim_size, "max")[0]
+    z = src - group_max.gather(dim, index)
+    total = scatter(z.exp(), index, dim, None, dim_size, "sum")[0]
+    return z.sub_(total.add_(eps).log_().gather(dim, index))
+
+
+def scatter_logsumexp(src, index, dim=-1, out=None, dim_size=None, eps=1e-12):
+    """torch_scatter/composite/logsumexp.py:8-57."""
+    index, dim = _py_broadcast(index, src, dim)
+    if out is not None:
+        dim_size = out.size(dim)
+    elif dim_size is None:
+        dim_size = int(index.max()) + 1
+    size = list(src.shape)
+    size[dim] = dim_size
+    group_max = torch.full(size, float("-inf"), dtype=src.dtype)
+    scatter(src, index, dim, group_max, dim_size, "max")
+    z = src - group_max.gather(dim, index)
+    z.masked_fill_(torch.isnan(z), float("-inf"))
+    orig = None
+    if out is not None:
+        orig = out.clone()
+        out = out.sub_(group_max).exp_()
+    total = scatter(z.exp_(), index, dim, out, dim_size, "sum")[0]
+    res = total.add_(eps).log_().add_(group_max)
+    if orig is None:
+        return res.nan_to_num_(neginf=0.0)
+    mask = ~res.isfinite()
+    res[mask] = orig[mask]
+    return res
+
+
+def scatter_std(src, index, dim=-1, out=None, dim_size=None, unbiased=True):
+    """torch_scatter/composite/std.py:8-41."""
+    if out is not None:
+        dim_size = out.size(dim)
+    dim = src.dim() + dim if dim < 0 else dim
+    count_dim = index.dim() - 1 if index.dim() <= dim else dim
+    ones = torch.ones(list(index.shape), dtype=src.dtype)
+    count = scatter(ones, index, count_dim, None, dim_size, "sum")[0]
+    index = broadcast(index, src, dim)
+    total = scatter(src, index, dim, None, dim_size, "sum")[0]
+    count = broadcast(count, total, dim).clamp(1)
+    mean = total.div(count)
+    dev = src - mean.gather(dim, index)
+    sq = scatter(dev * dev, index, dim, out, dim_size, "sum")[0]
+    if unbiased:
+        count = count.sub(1).clamp_(1)
+    return sq.div(count + 1e-6).sqrt()
+
+
+def scatter_softmax_backward(result, grad_out, index, dim=-1, dim_size=None, log_space=False):
+    """What autograd derives for the two functions above (closed form; the
+    reference has no explicit backward, it differentiates through its ops):
+    softmax: y * (g - sum_group(y * g)); log_softmax: g - exp(y) * sum_group(g)."""
+    index, dim = _py_broadcast(index, result, dim)
+    if dim_size is None:
+        dim_size = int(index.max()) + 1
+    if log_space:
+        total = scatter(grad_out, index, dim, None, dim_size, "sum")[0]
+        return grad_out - result.exp() * total.gather(dim, index)
+    total = scatter(result * grad_out, index, dim, None, dim_size, "sum")[0]
+    return result * (grad_out - total.gather(dim, index))

@@ -27,6 +27,7 @@ EXPORTS = (
     "ts_segment_coo_workspace_bytes", "ts_segment_coo", "ts_gather_coo",
     "ts_segment_mean_coo_backward",
     "ts_scatter", "ts_scatter_count", "ts_divide_by_count", "ts_arg_backward",
+    "ts_group_softmax_workspace_bytes", "ts_group_softmax", "ts_group_softmax_backward",
 )
 
 _lib = None
@@ -48,6 +49,7 @@ def lib() -> ctypes.CDLL:
         _lib.ts_hip_version.restype = ctypes.c_int64
         _lib.ts_segment_csr_workspace_bytes.restype = ctypes.c_size_t
         _lib.ts_segment_coo_workspace_bytes.restype = ctypes.c_size_t
+        _lib.ts_group_softmax_workspace_bytes.restype = ctypes.c_size_t
     return _lib
 
 
@@ -160,3 +162,29 @@ def arg_backward(grad_out, arg, grad_in, B, N, E, K):
     with torch.cuda.device(grad_in.device):
         _check(lib().ts_arg_backward(_p(grad_out), _p(arg), _p(grad_in), _i(B), _i(N), _i(E), _i(K),
                                      DTYPE[grad_in.dtype], _stream(grad_in)))
+
+
+def _group_workspace(like, B, N, K):
+    nbytes = lib().ts_group_softmax_workspace_bytes(_i(B), _i(N), _i(K), DTYPE[like.dtype])
+    return torch.empty(max(nbytes, 1), dtype=torch.uint8, device=like.device), nbytes
+
+
+def group_softmax(src, index, out, B, E, K, N, sb, se, log_space: bool, eps: float = 1e-12):
+    _dev(src, index, out)
+    ws, nbytes = _group_workspace(out, B, N, K)
+    with torch.cuda.device(out.device):
+        _check(lib().ts_group_softmax(_p(src), _p(index), _p(out), _i(B), _i(E), _i(K), _i(N), _i(sb), _i(se),
+                                      DTYPE[out.dtype], int(log_space), ctypes.c_double(eps), _p(ws),
+                                      ctypes.c_size_t(nbytes), _stream(out)))
+    return ws
+
+
+def group_softmax_backward(result, grad_out, index, grad_in, B, E, K, N, sb, se, log_space: bool):
+    _dev(result, grad_out, index, grad_in)
+    ws, nbytes = _group_workspace(grad_in, B, N, K)
+    with torch.cuda.device(grad_in.device):
+        _check(lib().ts_group_softmax_backward(_p(result), _p(grad_out), _p(index), _p(grad_in), _i(B), _i(E),
+                                               _i(K), _i(N), _i(sb), _i(se), DTYPE[grad_in.dtype],
+                                               int(log_space), _p(ws), ctypes.c_size_t(nbytes),
+                                               _stream(grad_in)))
+    return ws

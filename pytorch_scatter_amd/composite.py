@@ -1,7 +1,8 @@
-"""Group-wise statistics composed from the scatter operators: softmax,
-log-softmax, logsumexp and standard deviation over the entries that share an
-index (API of torch_scatter/composite/{softmax,logsumexp,std}.py). These are
-callers of the reduction kernels, not kernels of their own."""
+"""Group-wise statistics over the entries that share an index: softmax,
+log-softmax, logsumexp and standard deviation (API of
+torch_scatter/composite/{softmax,logsumexp,std}.py). Softmax and log-softmax
+are one fused operator; logsumexp and std are composed from the scatter
+operators."""
 from typing import Optional
 
 import torch
@@ -28,28 +29,22 @@ def _require_float(src: torch.Tensor, name: str):
                          "floating point data types.")
 
 
-def _shifted(src: torch.Tensor, index: torch.Tensor, dim: int, dim_size: Optional[int]):
-    """src minus the maximum of its group (the usual overflow guard)."""
-    group_max = scatter_max(src, index, dim, None, dim_size)[0]
-    return src - group_max.gather(dim, index)
-
-
 def scatter_softmax(src: torch.Tensor, index: torch.Tensor, dim: int = -1,
                     dim_size: Optional[int] = None) -> torch.Tensor:
+    """``exp(src - max) / sum(exp(src - max))`` over the entries that share an
+    index along ``dim`` (torch_scatter/composite/softmax.py:8-29). One operator:
+    three passes over ``src`` forward, two backward, when every column of a row
+    belongs to the same group; otherwise composed from the scatter operators."""
     _require_float(src, "scatter_softmax")
-    index = _expand_index(index, src, dim)
-    e = _shifted(src, index, dim, dim_size).exp_()
-    denom = scatter_sum(e, index, dim, None, dim_size).gather(dim, index)
-    return e.div(denom)
+    return torch.ops.torch_scatter.scatter_softmax(src, index, dim, dim_size, False, 0.0)
 
 
 def scatter_log_softmax(src: torch.Tensor, index: torch.Tensor, dim: int = -1,
                         eps: float = 1e-12, dim_size: Optional[int] = None) -> torch.Tensor:
+    """``(src - max) - log(sum(exp(src - max)) + eps)`` over the entries that
+    share an index (torch_scatter/composite/softmax.py:32-59)."""
     _require_float(src, "scatter_log_softmax")
-    index = _expand_index(index, src, dim)
-    z = _shifted(src, index, dim, dim_size)
-    log_denom = scatter_sum(z.exp(), index, dim, None, dim_size).add_(eps).log_()
-    return z.sub_(log_denom.gather(dim, index))
+    return torch.ops.torch_scatter.scatter_softmax(src, index, dim, dim_size, True, eps)
 
 
 def scatter_logsumexp(src: torch.Tensor, index: torch.Tensor, dim: int = -1,

@@ -9,6 +9,7 @@
 #include "coo_gather.h"
 #include "scatter.h"
 #include "elementwise.h"
+#include "group_softmax.h"
 
 using namespace ts;
 
@@ -56,6 +57,16 @@ int dispatch_divide(int dtype, void *out, const float *count, int64_t rows, int6
 int dispatch_arg_backward(int dtype, const void *g, const int64_t *arg, void *gi, int64_t B, int64_t N,
                           int64_t E, int64_t K, hipStream_t s) {
   TS_DISPATCH(dtype, launch_arg_backward<T>(g, arg, gi, B, N, E, K, s))
+}
+
+int dispatch_group_softmax(int dtype, const GroupArgs &g, int mode, int vec, hipStream_t s) {
+  switch (dtype) {
+  case TS_F32: return launch_group_softmax<float>(g, mode, vec, s);
+  case TS_F64: return launch_group_softmax<double>(g, mode, vec, s);
+  case TS_F16: return launch_group_softmax<f16_t>(g, mode, vec, s);
+  case TS_BF16: return launch_group_softmax<bf16_t>(g, mode, vec, s);
+  default: return TS_ERR_UNSUPPORTED;
+  }
 }
 
 // The reduction keeps edge positions in 32 bits inside a tile.
@@ -356,6 +367,61 @@ int ts_arg_backward(const void *grad_out, const int64_t *arg, void *grad_in, int
   if (B * E * K == 0) return TS_OK;
   if (!grad_in || (B * N * K > 0 && (!grad_out || !arg))) return TS_ERR_BAD_ARG;
   return dispatch_arg_backward(dtype, grad_out, arg, grad_in, B, N, E, K, static_cast<hipStream_t>(stream));
+}
+
+namespace {
+int run_group_softmax(const void *src, const void *grad, const int64_t *index, void *out, int64_t B, int64_t E,
+                      int64_t K, int64_t N, int64_t sb, int64_t se, int dtype, int mode, double eps, void *workspace,
+                      size_t workspace_bytes, hipStream_t stream) {
+  if (!valid_dtype(dtype) || !sizes_ok(B, N, E, K)) return TS_ERR_BAD_ARG;
+  if (!is_float_dtype(dtype)) return TS_ERR_UNSUPPORTED;
+  if (B * E * K == 0) return TS_OK;
+  if (!src || !index || !out) return TS_ERR_BAD_ARG;
+  if ((mode == GS_SOFTMAX_BWD || mode == GS_LOG_SOFTMAX_BWD) && !grad) return TS_ERR_BAD_ARG;
+  if (N == 0 || B * N >= 0x7FFFFFFFll) return TS_ERR_UNSUPPORTED;
+  const size_t need = group_workspace_bytes(B, N, K, kElemBytes[dtype]);
+  if (!workspace || workspace_bytes < need || !aligned16(workspace)) return TS_ERR_WORKSPACE;
+  GroupArgs g;
+  g.src = src;
+  g.grad = grad;
+  g.index = index;
+  g.out = out;
+  g.gmax = workspace;
+  g.gsum = static_cast<char *>(workspace) + need / 2;
+  g.B = B;
+  g.E = E;
+  g.K = K;
+  g.N = N;
+  g.sb = sb;
+  g.se = se;
+  g.eps = eps;
+  const int full = kVecBytes / kElemBytes[dtype];
+  const bool al = aligned16(src) && aligned16(out) && (!grad || aligned16(grad));
+  const int vec = (full > 1 && K % full == 0 && al) ? full : 1;
+  return dispatch_group_softmax(dtype, g, mode, vec, stream);
+}
+}  // namespace
+
+size_t ts_group_softmax_workspace_bytes(int64_t B, int64_t N, int64_t K, int dtype) {
+  if (!valid_dtype(dtype) || B < 0 || N < 0 || K < 0) return 0;
+  return group_workspace_bytes(B, N, K, kElemBytes[dtype]);
+}
+
+int ts_group_softmax(const void *src, const int64_t *index, void *out, int64_t B, int64_t E, int64_t K, int64_t N,
+                     int64_t index_stride_b, int64_t index_stride_e, int dtype, int log_space, double eps,
+                     void *workspace, size_t workspace_bytes, ts_stream_t stream) {
+  return run_group_softmax(src, nullptr, index, out, B, E, K, N, index_stride_b, index_stride_e, dtype,
+                           log_space ? GS_LOG_SOFTMAX : GS_SOFTMAX, eps, workspace, workspace_bytes,
+                           static_cast<hipStream_t>(stream));
+}
+
+int ts_group_softmax_backward(const void *result, const void *grad_out, const int64_t *index, void *grad_in,
+                              int64_t B, int64_t E, int64_t K, int64_t N, int64_t index_stride_b,
+                              int64_t index_stride_e, int dtype, int log_space, void *workspace,
+                              size_t workspace_bytes, ts_stream_t stream) {
+  return run_group_softmax(result, grad_out, index, grad_in, B, E, K, N, index_stride_b, index_stride_e, dtype,
+                           log_space ? GS_LOG_SOFTMAX_BWD : GS_SOFTMAX_BWD, 0.0, workspace, workspace_bytes,
+                           static_cast<hipStream_t>(stream));
 }
 
 }  // extern "C"

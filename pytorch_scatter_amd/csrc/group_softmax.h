@@ -1,0 +1,333 @@
+// Softmax and log-softmax over the entries that share an index, forward and
+// backward, for one index per row (the index addresses dim, every column of a
+// row belongs to the same group):
+//
+//   m[n,k]   = max over the group            (entries have to beat lowest(), NaN never wins;
+//                                             a group without a winner uses 0: what scatter_max
+//                                             hands to torch_scatter/composite/softmax.py:16-18)
+//   e[i,k]   = exp(src[i,k] - m[index[i],k])
+//   s[n,k]   = sum of e over the group
+//   softmax      out = e / s[index[i]]                          (composite/softmax.py:20-29)
+//   log_softmax  out = (src - m) - log(s + eps)[index[i]]       (composite/softmax.py:45-59)
+//
+// The reference runs this as two scatters, two gathers and four elementwise
+// passes. Here it is three passes over src: group maxima as order-preserving
+// integer keys (atomic max), group sums in the accumulate type (atomic add),
+// and the elementwise finish that recomputes e from src. The first two reuse
+// the wavefront pre-reduction of runs of equal neighbouring indices, so a
+// sorted index costs one atomic per group and wavefront. Every intermediate
+// that the reference holds in a tensor of the element type is rounded to the
+// element type here as well; the group sums accumulate in fp32 for 16-bit
+// floats (the reference adds in the element type).
+//
+// Backward (what autograd derives from the same formulas):
+//   softmax      grad_src = y * (g - S[index]),       S = group sum of y * g
+//   log_softmax  grad_src = g - exp(y) * G[index],    G = group sum of g
+#pragma once
+
+#include <math.h>
+
+#include "scatter.h"
+
+namespace ts {
+
+// order-preserving unsigned keys of the accumulate type; -0.0 folds onto +0.0
+template <typename F> struct OrdKey;
+template <> struct OrdKey<float> {
+  typedef uint32_t bits;
+  __device__ static bits enc(float v) { return Key<float>::enc(v); }
+  __device__ static float dec(bits k) { return Key<float>::dec(k); }
+};
+template <> struct OrdKey<double> {
+  typedef uint64_t bits;
+  __device__ static bits enc(double v) {
+    uint64_t u = (uint64_t)__double_as_longlong(v);
+    if (u == 0x8000000000000000ull) u = 0;
+    return (u >> 63) ? ~u : (u | 0x8000000000000000ull);
+  }
+  __device__ static double dec(bits k) {
+    return __longlong_as_double((long long)((k >> 63) ? (k & 0x7FFFFFFFFFFFFFFFull) : ~k));
+  }
+};
+
+__device__ __forceinline__ float exp_acc(float v) { return expf(v); }
+__device__ __forceinline__ double exp_acc(double v) { return exp(v); }
+__device__ __forceinline__ float log_acc(float v) { return logf(v); }
+__device__ __forceinline__ double log_acc(double v) { return log(v); }
+
+// a value of the accumulate type as the element type would hold it
+template <typename T> __device__ __forceinline__ typename Acc<T>::type round_elem(typename Acc<T>::type v) {
+  return to_acc<T>(from_acc<T>(v));
+}
+// key of "no entry has won": entries have to beat lowest() of the element type
+template <typename T> __device__ __forceinline__ typename OrdKey<typename Acc<T>::type>::bits group_empty_key() {
+  return OrdKey<typename Acc<T>::type>::enc(to_acc<T>(ElemLim<T>::lowest()));
+}
+
+enum { GS_SOFTMAX = 0, GS_LOG_SOFTMAX = 1, GS_SOFTMAX_BWD = 2, GS_LOG_SOFTMAX_BWD = 3 };
+
+struct GroupArgs {
+  const void *src;       // [B, E, K]: forward input; backward: the forward result y
+  const void *grad;      // [B, E, K]: backward only, gradient of the result
+  const int64_t *index;  // index[b * sb + e * se]
+  void *out;             // [B, E, K]
+  void *gmax;            // [B, N, K] keys of the group maxima (forward)
+  void *gsum;            // [B, N, K] group sums in the accumulate type
+  int64_t B, E, K, N;
+  int64_t sb, se;
+  double eps;
+};
+
+inline size_t group_align(size_t v) { return (v + 255) / 256 * 256; }
+// bytes of workspace: keys and sums, each [B, N, K] in 8 bytes at most
+inline size_t group_workspace_bytes(int64_t B, int64_t N, int64_t K, int elem_bytes) {
+  const size_t acc = elem_bytes == 8 ? 8 : 4;
+  return 2 * group_align((size_t)(B * N * K) * acc);
+}
+
+template <typename T>
+__global__ __launch_bounds__(kBlock) void group_init_kernel(GroupArgs g, int with_max) {
+  typedef typename Acc<T>::type F;
+  typedef typename OrdKey<F>::bits KB;
+  const int64_t n = g.B * g.N * g.K;
+  KB *gmax = static_cast<KB *>(g.gmax);
+  F *gsum = static_cast<F *>(g.gsum);
+  const KB empty = group_empty_key<T>();
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlock) {
+    if (with_max) gmax[i] = empty;
+    gsum[i] = (F)0;
+  }
+}
+
+// ---- pass 1: group maxima as keys
+template <typename T, int C_> struct GroupMaxRun {
+  typedef typename Acc<T>::type F;
+  typedef typename OrdKey<F>::bits A;
+  static constexpr int C = C_;
+  static constexpr int EW = 1;
+  static constexpr int U = 4;
+  const T *src;
+  A *gmax;
+  int64_t K;
+  __device__ A identity() const { return (A)0; }
+  __device__ void load(int64_t e, int64_t, int64_t col, int, A *x) const {
+    const Vec<T, C> r = load_vec_stream<T, C>(src + e * K + col);
+#pragma unroll
+    for (int c = 0; c < C; ++c) {
+      const F v = to_acc<T>(r.v[c]);
+      x[c] = v != v ? (A)0 : OrdKey<F>::enc(v);  // NaN never wins
+    }
+  }
+  __device__ void combine(A &x, const A &y) const { x = x > y ? x : y; }
+  __device__ void emit(int node, int64_t col, const A *x) const {
+    A *p = gmax + (int64_t)node * K + col;
+    // a running maximum is improved rarely; a stale read only costs a spare atomic
+    if (x[0] > *p) __hip_atomic_fetch_max(p, x[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+};
+
+template <typename T, int C>
+__global__ __launch_bounds__(kBlock) void group_max_run_kernel(ScatterArgs a, GroupArgs g, int lshift,
+                                                               int rows_per_wave) {
+  typedef typename GroupMaxRun<T, C>::A A;
+  __shared__ A s_stage[kBlock / kWave][kWave * C];
+  GroupMaxRun<T, C> p;
+  p.src = static_cast<const T *>(g.src);
+  p.gmax = static_cast<A *>(g.gmax);
+  p.K = g.K;
+  run_reduce_wave(a, lshift, rows_per_wave, p, s_stage[threadIdx.x / kWave]);
+}
+
+// the group maximum a row is shifted by
+template <typename T, int C>
+__device__ __forceinline__ void group_shift(const void *gmax, int64_t slot, typename Acc<T>::type *m) {
+  typedef typename Acc<T>::type F;
+  typedef typename OrdKey<F>::bits KB;
+  const Vec<KB, C> k = load_vec<KB, C>(static_cast<const KB *>(gmax) + slot);
+  const KB empty = group_empty_key<T>();
+#pragma unroll
+  for (int c = 0; c < C; ++c) m[c] = k.v[c] == empty ? (F)0 : OrdKey<F>::dec(k.v[c]);
+}
+
+// ---- pass 2: group sums of a per-entry term
+//   GS_SOFTMAX / GS_LOG_SOFTMAX   exp(src - m[node])
+//   GS_SOFTMAX_BWD                y * g
+//   GS_LOG_SOFTMAX_BWD            g
+template <typename T, int C_, int MODE> struct GroupSumRun {
+  typedef typename Acc<T>::type A;
+  static constexpr int C = C_;
+  static constexpr int EW = 1;
+  static constexpr int U = 4;
+  const T *src;
+  const T *grad;
+  const void *gmax;
+  A *gsum;
+  int64_t K;
+  __device__ A identity() const { return (A)0; }
+  __device__ void load(int64_t e, int64_t, int64_t col, int node, A *x) const {
+    if constexpr (MODE == GS_SOFTMAX || MODE == GS_LOG_SOFTMAX) {
+      const Vec<T, C> r = load_vec_stream<T, C>(src + e * K + col);
+      if (node < 0) {
+#pragma unroll
+        for (int c = 0; c < C; ++c) x[c] = (A)0;
+        return;
+      }
+      A m[C];
+      group_shift<T, C>(gmax, (int64_t)node * K + col, m);
+#pragma unroll
+      for (int c = 0; c < C; ++c) x[c] = round_elem<T>(exp_acc(round_elem<T>(to_acc<T>(r.v[c]) - m[c])));
+    } else if constexpr (MODE == GS_SOFTMAX_BWD) {
+      const Vec<T, C> y = load_vec_stream<T, C>(src + e * K + col);
+      const Vec<T, C> gr = load_vec_stream<T, C>(grad + e * K + col);
+#pragma unroll
+      for (int c = 0; c < C; ++c) x[c] = to_acc<T>(y.v[c]) * to_acc<T>(gr.v[c]);
+    } else {
+      const Vec<T, C> gr = load_vec_stream<T, C>(grad + e * K + col);
+#pragma unroll
+      for (int c = 0; c < C; ++c) x[c] = to_acc<T>(gr.v[c]);
+    }
+  }
+  __device__ void combine(A &x, const A &y) const { x = x + y; }
+  __device__ void emit(int node, int64_t col, const A *x) const {
+    atomic_add_elem<A>(gsum + (int64_t)node * K + col, x[0]);
+  }
+};
+
+template <typename T, int C, int MODE>
+__global__ __launch_bounds__(kBlock) void group_sum_run_kernel(ScatterArgs a, GroupArgs g, int lshift,
+                                                               int rows_per_wave) {
+  typedef typename Acc<T>::type A;
+  __shared__ A s_stage[kBlock / kWave][kWave * C];
+  GroupSumRun<T, C, MODE> p;
+  p.src = static_cast<const T *>(g.src);
+  p.grad = static_cast<const T *>(g.grad);
+  p.gmax = g.gmax;
+  p.gsum = static_cast<A *>(g.gsum);
+  p.K = g.K;
+  run_reduce_wave(a, lshift, rows_per_wave, p, s_stage[threadIdx.x / kWave]);
+}
+
+// ---- pass 3: the elementwise finish
+template <typename T, int VEC, int MODE>
+__global__ __launch_bounds__(kBlock) void group_finish_kernel(GroupArgs g) {
+  typedef typename Acc<T>::type F;
+  constexpr int U = 4;
+  const T *src = static_cast<const T *>(g.src);
+  const T *grad = static_cast<const T *>(g.grad);
+  const F *gsum = static_cast<const F *>(g.gsum);
+  T *out = static_cast<T *>(g.out);
+  const int64_t kv = g.K / VEC;
+  const EdgeLanes m = edge_lanes(kv, kBlock);
+  if (!m.active) return;
+  const int64_t n_edges = g.B * g.E;
+  const int64_t stride = (int64_t)gridDim.x * m.epp;
+  const F eps = (F)g.eps;
+  for (int64_t be0 = (int64_t)blockIdx.x * m.epp + m.el; be0 < n_edges; be0 += stride * U) {
+    for (int64_t cv = m.cl; cv < kv; cv += m.L) {
+      const int64_t k0 = cv * VEC;
+      Vec<T, VEC> x[U], y[U];
+      int64_t idx[U], bb[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int64_t be = be0 + u * stride < n_edges ? be0 + u * stride : be0;
+        int64_t ee;
+        split_edge(be, g.B, g.E, bb[u], ee);
+        x[u] = load_vec_stream<T, VEC>(src + be * g.K + k0);
+        if (MODE == GS_SOFTMAX_BWD || MODE == GS_LOG_SOFTMAX_BWD) y[u] = load_vec_stream<T, VEC>(grad + be * g.K + k0);
+        idx[u] = g.index[bb[u] * g.sb + ee * g.se];
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int64_t be = be0 + u * stride;
+        if (be >= n_edges) continue;
+        Vec<T, VEC> r;
+        if (idx[u] < 0 || idx[u] >= g.N) {  // an entry that belongs to no group
+#pragma unroll
+          for (int v = 0; v < VEC; ++v) r.v[v] = from_acc<T>((F)0);
+          store_vec_stream<T, VEC>(out + be * g.K + k0, r);
+          continue;
+        }
+        const int64_t slot = (bb[u] * g.N + idx[u]) * g.K + k0;
+        const Vec<F, VEC> s = load_vec<F, VEC>(gsum + slot);
+        F mx[VEC];
+        if (MODE == GS_SOFTMAX || MODE == GS_LOG_SOFTMAX) group_shift<T, VEC>(g.gmax, slot, mx);
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) {
+          const F xv = to_acc<T>(x[u].v[v]);
+          F res;
+          if (MODE == GS_SOFTMAX) {
+            const F e = round_elem<T>(exp_acc(round_elem<T>(xv - mx[v])));
+            res = e / round_elem<T>(s.v[v]);
+          } else if (MODE == GS_LOG_SOFTMAX) {
+            const F z = round_elem<T>(xv - mx[v]);
+            F l = round_elem<T>(log_acc(round_elem<T>(round_elem<T>(s.v[v]) + eps)));
+            // keeps the compiler from folding the subtraction's negation into the float -> half
+            // conversion as a two-element vector negation, which this backend cannot select
+            asm volatile("" : "+v"(l));
+            res = z - l;
+          } else if (MODE == GS_SOFTMAX_BWD) {
+            res = xv * (to_acc<T>(y[u].v[v]) - s.v[v]);
+          } else {
+            res = to_acc<T>(y[u].v[v]) - exp_acc(xv) * s.v[v];
+          }
+          r.v[v] = from_acc<T>(res);
+        }
+        store_vec_stream<T, VEC>(out + be * g.K + k0, r);
+      }
+    }
+  }
+}
+
+// ---- host side
+inline ScatterArgs group_index_args(const GroupArgs &g) {
+  ScatterArgs a = {};
+  a.index = g.index;
+  a.B = g.B;
+  a.E = g.E;
+  a.K = g.K;
+  a.N = g.N;
+  a.sb = g.sb;
+  a.se = g.se;
+  a.sk = 0;
+  return a;
+}
+
+template <typename T, int VEC, int MODE>
+int launch_group_softmax_m(const GroupArgs &g, hipStream_t stream) {
+  constexpr bool kForward = MODE == GS_SOFTMAX || MODE == GS_LOG_SOFTMAX;
+  const int64_t n_edges = g.B * g.E;
+  if (g.B * g.N >= 0x7FFFFFFFll) return TS_ERR_UNSUPPORTED;
+  const RunGrid rg = run_grid(n_edges, g.K / VEC);
+  if (!rg.ok) return TS_ERR_UNSUPPORTED;
+  const ScatterArgs a = group_index_args(g);
+  const dim3 gd(rg.blocks, rg.ychunks);
+  hipLaunchKernelGGL(group_init_kernel<T>, dim3(grid_for(g.B * g.N * g.K)), dim3(kBlock), 0, stream, g,
+                     kForward ? 1 : 0);
+  if (kForward)
+    hipLaunchKernelGGL((group_max_run_kernel<T, VEC>), gd, dim3(kBlock), 0, stream, a, g, rg.lshift, rg.rpw);
+  hipLaunchKernelGGL((group_sum_run_kernel<T, VEC, MODE>), gd, dim3(kBlock), 0, stream, a, g, rg.lshift, rg.rpw);
+  hipLaunchKernelGGL((group_finish_kernel<T, VEC, MODE>), dim3(scatter_grid(n_edges, g.K / VEC, kBlock, 4)),
+                     dim3(kBlock), 0, stream, g);
+  return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
+}
+
+template <typename T, int VEC>
+int launch_group_softmax_v(const GroupArgs &g, int mode, hipStream_t stream) {
+  switch (mode) {
+  case GS_SOFTMAX: return launch_group_softmax_m<T, VEC, GS_SOFTMAX>(g, stream);
+  case GS_LOG_SOFTMAX: return launch_group_softmax_m<T, VEC, GS_LOG_SOFTMAX>(g, stream);
+  case GS_SOFTMAX_BWD: return launch_group_softmax_m<T, VEC, GS_SOFTMAX_BWD>(g, stream);
+  case GS_LOG_SOFTMAX_BWD: return launch_group_softmax_m<T, VEC, GS_LOG_SOFTMAX_BWD>(g, stream);
+  default: return TS_ERR_BAD_ARG;
+  }
+}
+
+template <typename T> int launch_group_softmax(const GroupArgs &g, int mode, int vec, hipStream_t stream);
+
+#define TS_INSTANTIATE_GROUP_SOFTMAX(T, FULLVEC)                                                      \
+  template <> int launch_group_softmax<T>(const GroupArgs &g, int mode, int vec, hipStream_t stream) { \
+    if (vec == FULLVEC) return launch_group_softmax_v<T, FULLVEC>(g, mode, stream);                  \
+    return launch_group_softmax_v<T, 1>(g, mode, stream);                                            \
+  }
+
+}  // namespace ts

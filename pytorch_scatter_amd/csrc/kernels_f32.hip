@@ -5,6 +5,7 @@
 #include "coo_gather.h"
 #include "scatter.h"
 #include "elementwise.h"
+#include "group_softmax.h"
 
 namespace ts {
 TS_INSTANTIATE_CSR_REDUCE(float, 4)
@@ -12,4 +13,5 @@ TS_INSTANTIATE_CSR_GATHER(float, 4)
 TS_INSTANTIATE_COO_GATHER(float, 4)
 TS_INSTANTIATE_SCATTER(float, 4)
 TS_INSTANTIATE_ELEMENTWISE(float)
+TS_INSTANTIATE_GROUP_SOFTMAX(float, 4)
 }  // namespace ts

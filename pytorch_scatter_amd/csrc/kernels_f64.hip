@@ -5,6 +5,7 @@
 #include "coo_gather.h"
 #include "scatter.h"
 #include "elementwise.h"
+#include "group_softmax.h"
 
 namespace ts {
 TS_INSTANTIATE_CSR_REDUCE(double, 2)
@@ -12,4 +13,5 @@ TS_INSTANTIATE_CSR_GATHER(double, 2)
 TS_INSTANTIATE_COO_GATHER(double, 2)
 TS_INSTANTIATE_SCATTER(double, 2)
 TS_INSTANTIATE_ELEMENTWISE(double)
+TS_INSTANTIATE_GROUP_SOFTMAX(double, 2)
 }  // namespace ts

@@ -294,7 +294,8 @@ __global__ __launch_bounds__(kBlock) void scatter_add_pk16_kernel(ScatterArgs a)
 //
 // The policy P supplies the value type and its operations:
 //   P::A, P::C, P::EW          accumulator type, columns per lane, columns per atomic
-//   load(e, pos, col, x)       x[0..C) = columns col.. of entry e (position pos inside its batch)
+//   load(e, pos, col, node, x) x[0..C) = columns col.. of entry e (position pos inside its batch,
+//                              output row node or -1)
 //   combine(x, y)              x = x (op) y, one column
 //   identity()
 //   emit(node, col, x)         combine EW columns x[0..EW) into the output slot with one atomic
@@ -364,7 +365,7 @@ __device__ __forceinline__ void run_reduce_wave(const ScatterArgs &a, const int 
       split_edge(ec, a.B, a.E, b, pos);
       const int64_t idx = a.index[b * a.sb + pos * a.se];
       node[u] = (ok && idx >= 0 && idx < a.N) ? (int)(b * a.N + idx) : -1;
-      p.load(ec, pos, col_ok ? col : 0, x[u]);
+      p.load(ec, pos, col_ok ? col : 0, node[u], x[u]);
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -425,7 +426,7 @@ struct AddRun {
   T *out;
   int64_t K;
   __device__ A identity() const { return (A)0; }
-  __device__ void load(int64_t e, int64_t, int64_t col, A *x) const {
+  __device__ void load(int64_t e, int64_t, int64_t col, int, A *x) const {
     if (src == nullptr) {
 #pragma unroll
       for (int c = 0; c < C; ++c) x[c] = (A)1;
@@ -628,7 +629,7 @@ struct KeyRun {
   int64_t K;
   int precheck;
   __device__ A identity() const { return 0; }
-  __device__ void load(int64_t e, int64_t pos, int64_t col, A *x) const {
+  __device__ void load(int64_t e, int64_t pos, int64_t col, int, A *x) const {
     const Vec<T, C> r = load_vec_stream<T, C>(src + e * K + col);
     make_keys<T, C, IS_MAX>(r, pos, x);
   }

@@ -618,6 +618,69 @@ struct GatherCooFn : public torch::autograd::Function<GatherCooFn> {
   }
 };
 
+// ------------------------------------------------- autograd: group softmax
+// scatter_softmax / scatter_log_softmax of torch_scatter/composite/softmax.py:8-59 as one
+// operator (upstream composes them in Python from scatter_max, scatter_sum, gather and
+// elementwise ops). One index per row runs the fused kernels; an index that differs
+// between the columns of a row is composed from the registered operators as upstream does.
+struct GroupLayout {
+  bool fused;
+  int64_t B, E, K, sb, se;
+};
+GroupLayout group_layout(const Tensor &src, const Tensor &index, int64_t dim) {
+  GroupLayout l;
+  l.B = prod(src.sizes(), 0, dim);
+  l.E = src.size(dim);
+  l.K = prod(src.sizes(), dim + 1, src.dim());
+  auto sb = collapsed_stride(index, 0, dim);
+  auto sk = collapsed_stride(index, dim + 1, index.dim());
+  l.fused = sb.has_value() && sk.has_value() && (l.K == 1 || sk.value() == 0);
+  l.sb = sb.value_or(0);
+  l.se = index.stride(dim);
+  return l;
+}
+
+struct GroupSoftmaxFn : public torch::autograd::Function<GroupSoftmaxFn> {
+  static variable_list forward(AutogradContext *ctx, Variable src, Variable index, int64_t dim, int64_t N,
+                               bool log_space, double eps) {
+    check_device(src, "src");
+    check_device(index, "index");
+    c10::DeviceGuard guard(src.device());
+    src = src.contiguous();
+    const GroupLayout l = group_layout(src, index, dim);
+    Tensor out = at::empty_like(src);
+    Tensor ws = workspace(ts_group_softmax_workspace_bytes(l.B, N, l.K, dtype_code(src)), src);
+    check_status(ts_group_softmax(src.data_ptr(), index.data_ptr<int64_t>(), out.data_ptr(), l.B, l.E, l.K, N, l.sb,
+                                  l.se, dtype_code(src), log_space ? 1 : 0, eps, ws.data_ptr(),
+                                  static_cast<size_t>(ws.numel()), stream_of(src)),
+                 "scatter_softmax");
+    ctx->saved_data["dim"] = dim;
+    ctx->saved_data["N"] = N;
+    ctx->saved_data["log"] = log_space;
+    ctx->save_for_backward({out, index});
+    return {out};
+  }
+
+  static variable_list backward(AutogradContext *ctx, variable_list grad_outs) {
+    auto saved = ctx->get_saved_variables();
+    Tensor out = saved[0], index = saved[1];
+    Tensor grad_out = grad_outs[0].contiguous();
+    c10::DeviceGuard guard(out.device());
+    const int64_t dim = ctx->saved_data["dim"].toInt();
+    const int64_t N = ctx->saved_data["N"].toInt();
+    const bool log_space = ctx->saved_data["log"].toBool();
+    const GroupLayout l = group_layout(out, index, dim);
+    Tensor grad_in = at::empty_like(out);
+    Tensor ws = workspace(ts_group_softmax_workspace_bytes(l.B, N, l.K, dtype_code(out)), out);
+    check_status(ts_group_softmax_backward(out.data_ptr(), grad_out.data_ptr(), index.data_ptr<int64_t>(),
+                                           grad_in.data_ptr(), l.B, l.E, l.K, N, l.sb, l.se, dtype_code(out),
+                                           log_space ? 1 : 0, ws.data_ptr(), static_cast<size_t>(ws.numel()),
+                                           stream_of(out)),
+                 "scatter_softmax backward");
+    return {grad_in, Variable(), Variable(), Variable(), Variable(), Variable()};
+  }
+};
+
 // ------------------------------------------------------- registered functions
 Tensor scatter_sum(Tensor src, Tensor index, int64_t dim, OptTensor out, OptInt dim_size) {
   return ScatterFn<TS_SUM>::apply(src, index, dim, out, dim_size)[0];
@@ -669,6 +732,28 @@ std::tuple<Tensor, Tensor> segment_max_coo(Tensor src, Tensor index, OptTensor o
 }
 Tensor gather_coo(Tensor src, Tensor index, OptTensor out) { return GatherCooFn::apply(src, index, out)[0]; }
 
+Tensor scatter_softmax(Tensor src, Tensor index, int64_t dim, OptInt dim_size, bool log_space, double eps) {
+  TORCH_CHECK(src.is_floating_point(), log_space ? "`scatter_log_softmax`" : "`scatter_softmax`",
+              " can only be computed over tensors with floating point data types.");
+  dim = dim < 0 ? src.dim() + dim : dim;
+  index = broadcast(index, src, dim);
+  TORCH_CHECK(index.scalar_type() == at::kLong, "index must be int64");
+  if (src.numel() == 0) return at::empty_like(src);
+  const GroupLayout l = group_layout(src, index, dim);
+  const int64_t N = dim_size.has_value() ? dim_size.value() : 1 + index.max().item<int64_t>();
+  if (l.fused && N > 0 && l.B * N < 0x7FFFFFFFll)
+    return GroupSoftmaxFn::apply(src, index, dim, N, log_space, eps)[0];
+  // composite/softmax.py:16-29, :45-59
+  Tensor shift = std::get<0>(scatter_max(src, index, dim, std::nullopt, dim_size)).gather(dim, index);
+  Tensor z = src - shift;
+  if (!log_space) {
+    Tensor e = z.exp();
+    return e.div(scatter_sum(e, index, dim, std::nullopt, dim_size).gather(dim, index));
+  }
+  Tensor norm = scatter_sum(z.exp(), index, dim, std::nullopt, dim_size).add(eps).log().gather(dim, index);
+  return z.sub(norm);
+}
+
 int64_t cuda_version() { return ts_hip_version(); }  // csrc/version.cpp:28-38 returns HIP_VERSION on ROCm
 
 }  // namespace
@@ -689,4 +774,5 @@ static auto registry = torch::RegisterOperators()
                            .op("torch_scatter::segment_mean_coo", &segment_mean_coo)
                            .op("torch_scatter::segment_min_coo", &segment_min_coo)
                            .op("torch_scatter::segment_max_coo", &segment_max_coo)
-                           .op("torch_scatter::gather_coo", &gather_coo);
+                           .op("torch_scatter::gather_coo", &gather_coo)
+                           .op("torch_scatter::scatter_softmax", &scatter_softmax);

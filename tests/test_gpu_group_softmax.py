@@ -1,0 +1,196 @@
+"""The fused softmax / log-softmax over groups (ts_group_softmax and its
+backward through the C ABI, torch.ops.torch_scatter.scatter_softmax through the
+Python API) against the CPU oracle on the same seeded inputs.
+
+Bars. fp32 / fp64 compare with the oracle's result in the same type:
+rtol 1e-5 / 1e-12 (the two differ in the exp of the math library and in the
+order of the group sum). 16-bit floats compare with the oracle evaluated in
+fp64 on the same 16-bit inputs, within the roundings the reference's own
+sequence commits in the element type: the shifted value z = src - max is
+rounded to the element type before exp, so the bound grows with |z|."""
+from itertools import product
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+EPS_T = {torch.float32: 1e-5, torch.float64: 1e-12, torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -11}
+DTYPES = [torch.float32, torch.float64, torch.bfloat16, torch.float16]
+SHAPES = [
+    # B, E, K, N
+    (1, 5000, 1, 300), (2, 3000, 4, 50), (1, 2000, 8, 100), (1, 1500, 3, 40), (1, 900, 64, 20),
+    (1, 700, 130, 9), (3, 400, 16, 7), (1, 1, 1, 1), (1, 257, 2, 300),
+]
+
+
+@pytest.fixture(scope="module")
+def capi():
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    from pytorch_scatter_amd import capi
+    capi.lib()
+    return capi
+
+
+@pytest.fixture(scope="module")
+def ts():
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    import pytorch_scatter_amd
+    return pytorch_scatter_amd
+
+
+def make_index(kind, rng, E, N):
+    idx = rng.integers(0, N, size=E)
+    if kind == "sorted":
+        idx = np.sort(idx)
+    elif kind == "hub":
+        idx[E // 4: 3 * E // 4] = idx[0]
+    return torch.from_numpy(idx)
+
+
+def forward_bound(dtype, want64, z64, log_space):
+    e = EPS_T[dtype]
+    if dtype in (torch.float32, torch.float64):
+        return e * want64.abs() + e * (1.0 if log_space else 1e-30)
+    if log_space:
+        return e * (4.0 + want64.abs() + z64.abs())
+    # fp16 results below 2^-14 are subnormal: absolute spacing 2^-24, for e and for the quotient
+    return e * (4.0 + z64.abs()) * want64.abs() + (2.0 ** -23 if dtype == torch.float16 else 1e-30)
+
+
+@pytest.mark.parametrize("shape,kind,dtype", product(SHAPES, ["random", "sorted", "hub"], DTYPES))
+def test_forward_and_backward_capi(capi, oracle, shape, kind, dtype):
+    B, E, K, N = shape
+    rng = np.random.default_rng(E * 13 + K)
+    src = torch.from_numpy(rng.standard_normal(size=(B, E, K)) * 3).to(dtype)
+    grad = torch.from_numpy(rng.standard_normal(size=(B, E, K))).to(dtype)
+    index1 = make_index(kind, rng, E, N)
+    index = index1.view(1, E, 1).expand(B, E, K)
+    exact = dtype in (torch.float32, torch.float64)
+    ref_src = src if exact else src.double()
+    group_max = oracle.scatter(ref_src, index, 1, None, N, "max")[0]
+    z64 = (ref_src - group_max.gather(1, index)).double()
+    for log_space in (False, True):
+        out = torch.empty((B, E, K), dtype=dtype, device=DEV)
+        capi.group_softmax(src.to(DEV), index1.to(DEV), out, B, E, K, N, 0, 1, log_space)
+        torch.cuda.synchronize()
+        want = (oracle.scatter_log_softmax(ref_src, index, 1, 1e-12, N) if log_space
+                else oracle.scatter_softmax(ref_src, index, 1, N)).double()
+        err = (out.cpu().double() - want).abs()
+        bound = forward_bound(dtype, want, z64, log_space)
+        assert bool((err <= bound).all()), (log_space, float((err - bound).max()))
+
+        grad_in = torch.empty((B, E, K), dtype=dtype, device=DEV)
+        capi.group_softmax_backward(out, grad.to(DEV), index1.to(DEV), grad_in, B, E, K, N, 0, 1, log_space)
+        torch.cuda.synchronize()
+        y64, g64 = out.cpu().double(), grad.double()
+        want_g = oracle.scatter_softmax_backward(y64, g64, index, 1, N, log_space)
+        terms = (g64.abs() if log_space else (y64 * g64).abs())
+        spread = oracle.scatter(terms, index, 1, None, N, "sum")[0].gather(1, index)
+        scale = g64.abs() + y64.exp() * spread if log_space else y64.abs() * (g64.abs() + spread)
+        e = EPS_T[dtype]
+        gerr = (grad_in.cpu().double() - want_g).abs()
+        gbound = 8 * e * scale + (2.0 ** -23 if dtype == torch.float16 else 1e-30)  # fp16 subnormals
+        assert bool((gerr <= gbound).all()), ("backward", log_space, float((gerr - gbound).max()))
+
+
+def test_special_values_capi(capi, oracle):
+    """-inf entries, a group of only -inf, NaN in a group, entries outside [0, N), an empty group."""
+    src = torch.tensor([0.2, 0, 0.2, -2.1, 3.2, 7, -1, float("-inf"), float("-inf"), float("-inf"),
+                        1.0, float("nan"), 2.0, 5.0])
+    index = torch.tensor([0, 1, 0, 1, 1, 2, 4, 4, 5, 5, 6, 6, 6, 9])
+    E, N = src.numel(), 8
+    keep = index < N
+    for log_space in (False, True):
+        out = torch.empty(E, device=DEV)
+        capi.group_softmax(src.to(DEV), index.to(DEV), out, 1, E, 1, N, 0, 1, log_space)
+        torch.cuda.synchronize()
+        fn = oracle.scatter_log_softmax if log_space else oracle.scatter_softmax
+        want = fn(src[keep], index[keep], 0, dim_size=N) if not log_space else fn(src[keep], index[keep], 0, 1e-12, N)
+        got = out.cpu()
+        assert torch.allclose(got[keep], want, rtol=1e-5, atol=1e-7, equal_nan=True), (log_space, got, want)
+        assert float(got[~keep].abs().max()) == 0.0
+
+
+def test_workspace_and_argument_checks(capi):
+    import ctypes
+    L = capi.lib()
+    x = torch.zeros(8, device=DEV)
+    idx = torch.zeros(8, dtype=torch.long, device=DEV)
+    ws = torch.empty(16, dtype=torch.uint8, device=DEV)
+    args = (capi._p(x), capi._p(idx), capi._p(x), capi._i(1), capi._i(8), capi._i(1), capi._i(4), capi._i(0),
+            capi._i(1))
+    rc = L.ts_group_softmax(*args, capi.DTYPE[torch.float32], 0, ctypes.c_double(0.0), capi._p(ws),
+                            ctypes.c_size_t(16), None)
+    assert rc == 3  # TS_ERR_WORKSPACE
+    rc = L.ts_group_softmax(*args, capi.DTYPE[torch.int32], 0, ctypes.c_double(0.0), capi._p(ws),
+                            ctypes.c_size_t(16), None)
+    assert rc == 2  # TS_ERR_UNSUPPORTED: floating types only
+
+
+# ------------------------------------------------------------------ operator level
+def per_group(lib, src, index, dim, n):
+    out = torch.zeros_like(src)
+    for g in range(n):
+        sel = (index == g).nonzero().flatten()
+        if sel.numel() > 0:
+            out = out.index_copy(dim, sel, lib(src.index_select(dim, sel), dim))
+    return out
+
+
+@pytest.mark.parametrize("dim,shape,log_space", product([0, 1, 2, -1], [(40, 30, 20)], [False, True]))
+def test_operator_dims_and_autograd(ts, dim, shape, log_space):
+    g = torch.Generator().manual_seed(5)
+    d = dim if dim >= 0 else len(shape) + dim
+    src_cpu = torch.randn(shape, generator=g, dtype=torch.double) * 2
+    index = torch.randint(0, 6, (shape[d],), generator=g)
+    grad = torch.randn(shape, generator=g, dtype=torch.double)
+    lib = torch.log_softmax if log_space else torch.softmax
+    ref = src_cpu.clone().requires_grad_(True)
+    want = per_group(lib, ref, index, d, 6)
+    want.backward(grad)
+    fn = ts.scatter_log_softmax if log_space else ts.scatter_softmax
+    src = src_cpu.to(DEV).requires_grad_(True)
+    shape1 = [1] * len(shape)
+    shape1[d] = shape[d]
+    for idx in (index.to(DEV) if d == 0 or True else None, index.view(shape1).expand(shape).to(DEV)):
+        if idx.dim() == 1 and d != 0:
+            idx = idx.view(shape1[:d + 1])  # leading dims broadcast, trailing dims implied
+        src.grad = None
+        out = fn(src, idx, dim)
+        out.backward(grad.to(DEV))
+        assert torch.allclose(out.detach().cpu(), want.detach(), rtol=1e-9, atol=1e-9)
+        assert torch.allclose(src.grad.cpu(), ref.grad, rtol=1e-8, atol=1e-9)
+
+
+def test_operator_reference_cases_script_and_fallback(ts, oracle):
+    # test/composite/test_softmax.py:6-54
+    src = torch.tensor([0.2, 0, 0.2, -2.1, 3.2, 7, -1, float("-inf")], device=DEV, requires_grad=True)
+    index = torch.tensor([0, 1, 0, 1, 1, 2, 4, 4], device=DEV)
+    for fn, ofn in ((ts.scatter_softmax, oracle.scatter_softmax), (ts.scatter_log_softmax, oracle.scatter_log_softmax)):
+        out = fn(src, index)
+        assert torch.allclose(out.detach().cpu(), ofn(src.detach().cpu(), index.cpu()), equal_nan=True)
+        out.backward(torch.randn_like(out))
+        jit = torch.jit.script(fn)
+        assert jit(src, index).tolist() == out.tolist()
+    # an index that differs between the columns of a row: composed from the scatter operators
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(50, 6, generator=g)
+    idx = torch.randint(0, 5, (50, 6), generator=g)
+    got = ts.scatter_softmax(x.to(DEV), idx.to(DEV), 0)
+    assert torch.allclose(got.cpu(), oracle.scatter_softmax(x, idx, 0), rtol=1e-5, atol=1e-7)
+    got = ts.scatter_log_softmax(x.to(DEV), idx.to(DEV), 0, dim_size=7)
+    assert torch.allclose(got.cpu(), oracle.scatter_log_softmax(x, idx, 0, 1e-12, 7), rtol=1e-5, atol=1e-6)
+    # per-row index on the last dimension (B > 1, K = 1) is the fused path
+    x = torch.randn(7, 90, generator=g)
+    idx = torch.randint(0, 9, (7, 90), generator=g)
+    got = ts.scatter_softmax(x.to(DEV), idx.to(DEV), -1)
+    assert torch.allclose(got.cpu(), oracle.scatter_softmax(x, idx, -1), rtol=1e-5, atol=1e-7)
+    # zero-size input, integer input
+    assert ts.scatter_softmax(torch.empty(0, 4, device=DEV), torch.empty(0, dtype=torch.long, device=DEV), 0).shape == (0, 4)
+    with pytest.raises(ValueError):
+        ts.scatter_softmax(torch.ones(4, dtype=torch.long, device=DEV), torch.zeros(4, dtype=torch.long, device=DEV))
