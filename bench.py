@@ -152,6 +152,31 @@ def bench_scatter_config(ts, wl, w, dev, iters, reduces):
     return res
 
 
+def bench_softmax_config(ts, wl, w, dev, iters, K):
+    """scatter_softmax over the destination index of the C3 graph with K values per entry (attention
+    heads), sorted and in random order; bytes: src read once, index read once, result written once."""
+    import torch
+    index = w.index.to(dev)
+    shuffled = index[torch.randperm(w.E, device=dev)]
+    src = torch.randn((w.E, K), device=dev)
+    grad = torch.randn((w.E, K), device=dev)
+    res = {"N": w.N, "E": w.E, "K": K, "dtype": "float32"}
+    fwd_bytes = 2 * w.E * K * 4 + w.E * 8
+    bwd_bytes = 3 * w.E * K * 4 + w.E * 8
+    for name, idx in (("sorted", index), ("unsorted", shuffled)):
+        with torch.no_grad():
+            t = event_time(lambda: ts.scatter_softmax(src, idx, 0, w.N), iters)
+        res[f"softmax_{name}"] = entry(fwd_bytes, t, w.E * K)
+        x = src.clone().requires_grad_(True)
+        y = ts.scatter_softmax(x, idx, 0, w.N)
+        t = event_time(lambda: torch.autograd.grad(y, x, grad, retain_graph=True), iters)
+        res[f"softmax_backward_{name}"] = entry(bwd_bytes, t, w.E * K)
+        del x, y
+    del src, grad
+    torch.cuda.empty_cache()
+    return res
+
+
 def cpu_baseline(wl, w):
     """The same three ops of C2 on the host, single thread: the reference's own
     CPU kernels when oracle/_ref is built, else the C restatement."""
@@ -350,6 +375,14 @@ def main():
         w3 = wl.c3_segment_coo()
         sw = wl.ScatterWorkload("X-sorted-K64", w3.index, w3.N, w3.E, 64, torch.float32)
         table["X-sorted-K64"] = bench_scatter_config(ts, wl, sw, dev, max(it // 2, 3), ["sum", "max"])
+        # the same entries in random order: the hubs of a power-law index no longer form runs and every
+        # entry of a hub meets the others on one address unless the kernel keeps its hot rows in LDS
+        g = torch.Generator().manual_seed(0)
+        wz = wl.c4_scatter_minmax(1)
+        zipf_index = wz.index[torch.randperm(wz.E, generator=g)] * 10 % 1_000_000
+        sz = wl.ScatterWorkload("X-zipf-unsorted-K8", zipf_index, 1_000_000, wz.E, 8, torch.float32)
+        table["X-zipf-unsorted-K8"] = bench_scatter_config(ts, wl, sz, dev, max(it // 2, 3), ["sum", "max"])
+        table["X-softmax-K8"] = bench_softmax_config(ts, wl, w3, dev, max(it // 2, 3), 8)
         table["X-narrow-K1"] = bench_csr_config(ts, wl, dataclasses.replace(w3, K=1, name="X-narrow-K1"), dev, it,
                                                 ["segment_csr_sum", "segment_csr_max", "segment_coo_sum",
                                                  "gather_csr", "gather_coo"], uniform=True)

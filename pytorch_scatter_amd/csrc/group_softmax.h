@@ -119,6 +119,7 @@ template <typename T, int C_> struct GroupMaxRun {
     }
   }
   __device__ void combine(A &x, const A &y) const { x = x > y ? x : y; }
+  __device__ void begin_row(int, int) const {}
   __device__ void emit(int node, int64_t col, const A *x) const {
     A *p = gmax + (int64_t)node * K + col;
     // a running maximum is improved rarely; a stale read only costs a spare atomic
@@ -153,7 +154,7 @@ __device__ __forceinline__ void group_shift(const void *gmax, int64_t slot, type
 //   GS_SOFTMAX / GS_LOG_SOFTMAX   exp(src - m[node])
 //   GS_SOFTMAX_BWD                y * g
 //   GS_LOG_SOFTMAX_BWD            g
-template <typename T, int C_, int MODE> struct GroupSumRun {
+template <typename T, int C_, int MODE> struct GroupSumRun : HotState<typename Acc<T>::type> {
   typedef typename Acc<T>::type A;
   static constexpr int C = C_;
   static constexpr int EW = 1;
@@ -188,23 +189,33 @@ template <typename T, int C_, int MODE> struct GroupSumRun {
     }
   }
   __device__ void combine(A &x, const A &y) const { x = x + y; }
-  __device__ void emit(int node, int64_t col, const A *x) const {
+  __device__ void emit(int node, int64_t col, const A *x) {
+    if (this->template to_table<1>(node, col, x)) return;  // a hub group: summed in LDS first
+    to_memory(node, col, x);
+  }
+  __device__ void to_memory(int node, int64_t col, const A *x) const {
     atomic_add_elem<A>(gsum + (int64_t)node * K + col, x[0]);
   }
 };
 
 template <typename T, int C, int MODE>
 __global__ __launch_bounds__(kBlock) void group_sum_run_kernel(ScatterArgs a, GroupArgs g, int lshift,
-                                                               int rows_per_wave) {
+                                                               int rows_per_wave, int hot_rlog) {
   typedef typename Acc<T>::type A;
   __shared__ A s_stage[kBlock / kWave][kWave * C];
+  __shared__ A s_hot[kHotAcc];
+  __shared__ uint32_t s_tags[kHotRowsMax];
   GroupSumRun<T, C, MODE> p;
   p.src = static_cast<const T *>(g.src);
   p.grad = static_cast<const T *>(g.grad);
   p.gmax = g.gmax;
   p.gsum = static_cast<A *>(g.gsum);
   p.K = g.K;
+  p.hot_init(s_hot, s_tags, hot_rlog, lshift + LogC<C>::value);
   run_reduce_wave(a, lshift, rows_per_wave, p, s_stage[threadIdx.x / kWave]);
+  p.hot.template flush<1>([&](int node, int j, const A *x) {
+    if (p.colbase + j < p.K) p.to_memory(node, p.colbase + j, x);
+  });
 }
 
 // ---- pass 3: the elementwise finish
@@ -297,7 +308,7 @@ int launch_group_softmax_m(const GroupArgs &g, hipStream_t stream) {
   constexpr bool kForward = MODE == GS_SOFTMAX || MODE == GS_LOG_SOFTMAX;
   const int64_t n_edges = g.B * g.E;
   if (g.B * g.N >= 0x7FFFFFFFll) return TS_ERR_UNSUPPORTED;
-  const RunGrid rg = run_grid(n_edges, g.K / VEC);
+  const RunGrid rg = run_grid(n_edges, g.K / VEC, VEC);
   if (!rg.ok) return TS_ERR_UNSUPPORTED;
   const ScatterArgs a = group_index_args(g);
   const dim3 gd(rg.blocks, rg.ychunks);
@@ -305,7 +316,8 @@ int launch_group_softmax_m(const GroupArgs &g, hipStream_t stream) {
                      kForward ? 1 : 0);
   if (kForward)
     hipLaunchKernelGGL((group_max_run_kernel<T, VEC>), gd, dim3(kBlock), 0, stream, a, g, rg.lshift, rg.rpw);
-  hipLaunchKernelGGL((group_sum_run_kernel<T, VEC, MODE>), gd, dim3(kBlock), 0, stream, a, g, rg.lshift, rg.rpw);
+  hipLaunchKernelGGL((group_sum_run_kernel<T, VEC, MODE>), gd, dim3(kBlock), 0, stream, a, g, rg.lshift, rg.rpw,
+                     rg.hot_rlog);
   hipLaunchKernelGGL((group_finish_kernel<T, VEC, MODE>), dim3(scatter_grid(n_edges, g.K / VEC, kBlock, 4)),
                      dim3(kBlock), 0, stream, g);
   return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;

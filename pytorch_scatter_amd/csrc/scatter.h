@@ -109,6 +109,34 @@ template <> __device__ __forceinline__ void atomic_add_elem<int64_t>(int64_t *p,
   __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// One 16-bit float without a compare-and-swap loop (which collapses when many lanes add to the same
+// element): a packed-pair add on the 32-bit word that holds the element, with +0.0 for the
+// neighbour. x + 0.0 leaves every value alone (a -0.0 neighbour turns into +0.0, which compares
+// equal), so this is only used when the neighbour is an element of the same buffer [lo, hi).
+template <typename T> __device__ __forceinline__ void atomic_add_half(T *p, T v, const T *lo, const T *hi) {
+  static_assert(sizeof(T) == 2, "");
+  const uintptr_t a = reinterpret_cast<uintptr_t>(p);
+  T *w = reinterpret_cast<T *>(a & ~(uintptr_t)3);
+  if (w < lo || w + 2 > hi) {
+    atomic_add_elem<T>(p, v);
+    return;
+  }
+  const bool upper = (a & 2) != 0;
+  if constexpr (__is_same(T, bf16_t)) {
+    typedef short v2s __attribute__((ext_vector_type(2)));
+    v2s pk;
+    pk.x = upper ? (short)0 : (short)v.x;
+    pk.y = upper ? (short)v.x : (short)0;
+    __builtin_amdgcn_global_atomic_fadd_v2bf16(reinterpret_cast<v2s *>(w), pk);
+  } else {
+    typedef _Float16 v2h __attribute__((ext_vector_type(2)));
+    v2h pk;
+    pk.x = upper ? (_Float16)0 : (_Float16)v;
+    pk.y = upper ? (_Float16)v : (_Float16)0;
+    __builtin_amdgcn_global_atomic_fadd_v2f16(reinterpret_cast<v2h *>(w), pk);
+  }
+}
+
 // ------------------------------------------------ order-preserving 32-bit keys
 // order(v) is monotone in v; -0.0 is folded onto +0.0 so that the two compare
 // equal as they do under the reference's `<` / `>`.
@@ -238,9 +266,12 @@ __global__ __launch_bounds__(kBlock) void scatter_atomic_kernel(ScatterArgs a) {
           if (id < 0 || id >= a.N) continue;
           T *p = out + (bb[u] * a.N + id) * a.K + k0 + v;
           const T val = x[u].v[v];
-          if (REDUCE == TS_SUM)
-            atomic_add_elem<T>(p, val);
-          else
+          if (REDUCE == TS_SUM) {
+            if constexpr (__is_same(T, bf16_t) || __is_same(T, f16_t))
+              atomic_add_half<T>(p, val, out, out + a.B * a.N * a.K);
+            else
+              atomic_add_elem<T>(p, val);
+          } else
             atomic_rmw<T>(p, [val](T cur) { return mul_elem<T>(cur, val); });
         }
       }
@@ -299,9 +330,11 @@ __global__ __launch_bounds__(kBlock) void scatter_add_pk16_kernel(ScatterArgs a)
 //   combine(x, y)              x = x (op) y, one column
 //   identity()
 //   emit(node, col, x)         combine EW columns x[0..EW) into the output slot with one atomic
+//   begin_row(heads, entries)  called once per wavefront row of more than one entry, before the
+//                              emissions of its finished runs: number of runs and of entries in it
 template <typename P>
 __device__ __forceinline__ void run_reduce_wave(const ScatterArgs &a, const int lshift, const int rows_per_wave,
-                                                const P &p, typename P::A *stage) {
+                                                P &p, typename P::A *stage) {
   typedef typename P::A A;
   constexpr int U = P::U;
   constexpr int C = P::C;
@@ -389,6 +422,7 @@ __device__ __forceinline__ void run_reduce_wave(const ScatterArgs &a, const int 
         const int prev = __shfl_up(n, L);
         const bool head = (el == 0) || (n != prev);
         const uint64_t hm = __ballot(head) & slot_bits;
+        p.begin_row(__popcll(hm), epr);
         // slots from this one to the end of its run
         const uint64_t after = (el + 1 < epr) ? (hm >> ((el + 1) << lshift)) : 0ull;
         const int rem = after ? ((__ffsll((unsigned long long)after) - 1) >> lshift) + 1 : epr - el;
@@ -414,16 +448,114 @@ __device__ __forceinline__ void run_reduce_wave(const ScatterArgs &a, const int 
   if (carry_node >= 0) write_slots(1ull, carry_node, carry);
 }
 
+// ---- hot rows of a workgroup ------------------------------------------------------
+// An unsorted index with a hub (a node that owns 1 % or more of the entries, as in
+// power-law graphs) puts every entry of the hub on one address: about 10 ns per
+// atomic, one after the other (measured: 10 M entries with a 20 % hub take 20 ms
+// instead of 0.5 ms). The sum kernels therefore keep a small LDS table of
+// accumulator rows per workgroup. A row is handed to a node only when the node
+// shows up twice in a row among the emissions that hash to it: a hub passes that
+// test almost at once, the one-off nodes of a sorted or uniform index practically
+// never do, so they cost one LDS read and keep going to memory directly. Confirmed
+// rows never change owner; they are added to the output once, when the workgroup
+// is done. Every value is added exactly once, either to its node's confirmed row
+// or to memory.
+constexpr int kHotAcc = 2048;                    // accumulators per workgroup
+constexpr int kHotRowsMax = 512;
+constexpr uint32_t kHotConfirmed = 0x80000000u;  // tag bit: the row belongs to the node for good
+constexpr uint32_t kHotNone = 0x7FFFFFFFu;       // no candidate yet (node ids stay below 2^31 - 1)
+template <typename A> struct HotOk { static constexpr bool value = sizeof(A) >= 4; };  // LDS atomics: 32 / 64 bits
+
+template <typename A> struct HotRows {
+  A *acc;          // [rows][1 << wshift]
+  uint32_t *tags;  // [rows]
+  int rlog;        // log2(rows), < 0: no table
+  int wshift;      // log2 of the columns per row (the column chunk of the workgroup)
+  __device__ int row_of(int node) const { return (int)(((uint32_t)node * 0x9E3779B1u) >> (32 - rlog)); }
+  // true: x[0..EW) went into the workgroup's row of `node` at columns j..; false: the caller adds them to memory
+  template <int EW> __device__ bool add(int node, int j, const A *x) const {
+    if (rlog < 0) return false;
+    const int row = row_of(node);
+    const uint32_t mine = (uint32_t)node | kHotConfirmed;
+    const uint32_t t = __hip_atomic_load(&tags[row], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    if (t != mine) {
+      // only the lane of column 0 moves the tag, so the other columns of one entry cannot confirm it
+      if ((t & kHotConfirmed) || j != 0) return false;
+      if (t != (uint32_t)node) {  // remember as the candidate
+        atomicCAS(&tags[row], t, (uint32_t)node);
+        return false;
+      }
+      const uint32_t old = atomicCAS(&tags[row], t, mine);  // second time in a row: confirm
+      if (old != t && old != mine) return false;
+    }
+#pragma unroll
+    for (int w = 0; w < EW; ++w)
+      __hip_atomic_fetch_add(&acc[(row << wshift) + j + w], x[w], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    return true;
+  }
+  __device__ void clear() const {
+    if (rlog < 0) return;
+    for (int i = threadIdx.x; i < (1 << (rlog + wshift)); i += blockDim.x) acc[i] = (A)0;
+    for (int i = threadIdx.x; i < (1 << rlog); i += blockDim.x) tags[i] = kHotNone;
+    __syncthreads();
+  }
+  // add the confirmed rows to the output: emit(node, column inside the chunk, EW accumulators)
+  template <int EW, typename F> __device__ void flush(F emit) const {
+    if (rlog < 0) return;
+    __syncthreads();
+    for (int i = threadIdx.x * EW; i < (1 << (rlog + wshift)); i += blockDim.x * EW) {
+      const uint32_t t = tags[i >> wshift];
+      if (!(t & kHotConfirmed)) continue;
+      bool any = false;
+#pragma unroll
+      for (int w = 0; w < EW; ++w) any = any || acc[i + w] != (A)0;
+      if (any) emit((int)(t & ~kHotConfirmed), i & ((1 << wshift) - 1), acc + i);
+    }
+  }
+};
+// log2 of the rows of the table for column chunks of 1 << wshift columns; -1: chunk too wide for a table
+inline int hot_rows_log(int wshift) {
+  int rlog = 0;
+  while ((2 << rlog) <= kHotRowsMax && ((2 << rlog) << wshift) <= kHotAcc) ++rlog;
+  return rlog >= 3 ? rlog : -1;
+}
+
+// What a sum policy keeps to use the table. Rows of the wavefront in which at least half of the
+// entries continue a run look sorted: their few emissions go to memory directly and the table costs
+// them nothing. (Hub entries sprinkled over an otherwise sorted index are not caught that way.)
+template <typename A> struct HotState {
+  HotRows<A> hot;
+  int64_t colbase;  // first column of the workgroup's chunk
+  bool active;
+  __device__ void hot_init(A *acc, uint32_t *tags, int rlog, int wshift) {
+    hot.acc = acc;
+    hot.tags = tags;
+    hot.rlog = HotOk<A>::value ? rlog : -1;
+    hot.wshift = wshift;
+    colbase = (int64_t)blockIdx.y << wshift;
+    active = true;
+    hot.clear();
+  }
+  __device__ void begin_row(int heads, int entries) { active = heads * 2 > entries; }
+  template <int EW> __device__ bool to_table(int node, int64_t col, const A *x) {
+    if constexpr (HotOk<A>::value) return active && hot.template add<EW>(node, (int)(col - colbase), x);
+    return false;
+  }
+};
+
 // sum: up to 16 bytes per lane; 16-bit floats accumulate in fp32 and are written
 // with the packed-pair atomic. src == nullptr adds 1 per entry (the count of scatter mean).
-template <typename T, int C_>
-struct AddRun {
+// EW_ = columns per atomic: a whole 32-bit word for element types below 32 bits, or 1 (rows whose
+// length or alignment rules that out; the element then goes through a compare-and-swap on its word)
+template <typename T, int C_, int EW_ = (sizeof(T) < 4 ? 4 / (int)sizeof(T) : 1)>
+struct AddRun : HotState<typename Acc<T>::type> {
   typedef typename Acc<T>::type A;
   static constexpr int C = C_;
-  static constexpr int EW = sizeof(T) < 4 ? 4 / (int)sizeof(T) : 1;  // columns per atomic: one 32-bit word
+  static constexpr int EW = EW_;
   static constexpr int U = 4;
   const T *src;
   T *out;
+  const T *out_end;
   int64_t K;
   __device__ A identity() const { return (A)0; }
   __device__ void load(int64_t e, int64_t, int64_t col, int, A *x) const {
@@ -437,9 +569,13 @@ struct AddRun {
     for (int c = 0; c < C; ++c) x[c] = to_acc<T>(r.v[c]);
   }
   __device__ void combine(A &x, const A &y) const { x = x + y; }
-  __device__ void emit(int node, int64_t col, const A *x) const {
+  __device__ void emit(int node, int64_t col, const A *x) {
+    if (this->template to_table<EW>(node, col, x)) return;
+    to_memory(node, col, x);
+  }
+  __device__ void to_memory(int node, int64_t col, const A *x) const {
     T *p = out + (int64_t)node * K + col;
-    if constexpr (std::is_integral<T>::value && sizeof(T) < 4) {
+    if constexpr (EW > 1 && std::is_integral<T>::value && sizeof(T) < 4) {
       // 8- and 16-bit integers: one compare-and-swap on the 32-bit word that holds EW neighbouring columns
       // (a CAS per element would make the lanes of one word fight each other)
       typedef typename std::make_unsigned<T>::type UT;
@@ -473,29 +609,41 @@ struct AddRun {
         pk.y = (_Float16)x[1];
         __builtin_amdgcn_global_atomic_fadd_v2f16(reinterpret_cast<v2h *>(p), pk);
       }
+    } else if constexpr (__is_same(T, bf16_t) || __is_same(T, f16_t)) {
+      atomic_add_half<T>(p, from_acc<T>(x[0]), out, out_end);
     } else {
       atomic_add_elem<T>(p, from_acc<T>(x[0]));
     }
   }
 };
 
-template <typename T, int C>
-__global__ __launch_bounds__(kBlock) void scatter_add_run_kernel(ScatterArgs a, int lshift, int rows_per_wave) {
+template <int C> struct LogC { static constexpr int value = C == 1 ? 0 : (C == 2 ? 1 : (C == 4 ? 2 : (C == 8 ? 3 : 4))); };
+
+template <typename T, int C, int EW = (sizeof(T) < 4 ? 4 / (int)sizeof(T) : 1)>
+__global__ __launch_bounds__(kBlock) void scatter_add_run_kernel(ScatterArgs a, int lshift, int rows_per_wave,
+                                                                 int hot_rlog) {
   typedef typename Acc<T>::type A;
   __shared__ A s_stage[kBlock / kWave][kWave * C];
-  AddRun<T, C> p;
+  __shared__ A s_hot[HotOk<A>::value ? kHotAcc : 1];
+  __shared__ uint32_t s_tags[HotOk<A>::value ? kHotRowsMax : 1];
+  AddRun<T, C, EW> p;
   p.src = static_cast<const T *>(a.src);
   p.out = static_cast<T *>(a.out);
+  p.out_end = p.out + a.B * a.N * a.K;
   p.K = a.K;
+  p.hot_init(s_hot, s_tags, hot_rlog, lshift + LogC<C>::value);
   run_reduce_wave(a, lshift, rows_per_wave, p, s_stage[threadIdx.x / kWave]);
+  p.hot.template flush<EW>([&](int node, int j, const A *x) {
+    if (p.colbase + j < p.K) p.to_memory(node, p.colbase + j, x);
+  });
 }
 
 // rows of a wavefront in the kernel above: long enough to carry runs across rows, short enough to
 // leave ~8 K wavefronts
-inline int run_rows_per_wave(int64_t n_edges, int epr) {
+inline int run_rows_per_wave(int64_t n_edges, int epr, int cap = 32) {
   const int64_t rows = (n_edges + epr - 1) / epr;
   int64_t rpw = rows / 8192;
-  if (rpw > 32) rpw = 32;
+  if (rpw > cap) rpw = cap;
   if (rpw < 1) rpw = 1;
   if (const char *env = getenv("TS_RUN_RPW")) rpw = atoi(env) > 0 ? atoi(env) : rpw;  // tuning aid
   return (int)(rpw <= 4 ? rpw : (rpw + 3) / 4 * 4);
@@ -505,13 +653,22 @@ struct RunGrid {
   int lshift, rpw;
   unsigned blocks, ychunks;
   bool ok;
+  int hot_rlog;  // log2 of the rows of the hot-row table, -1: none
 };
-inline RunGrid run_grid(int64_t n_edges, int64_t kc) {
+// c > 0: a sum kernel with c columns per lane that may keep a hot-row table. The table pays once a
+// workgroup sees enough entries for a hub to repeat: large inputs, with longer ranges per wavefront.
+inline RunGrid run_grid(int64_t n_edges, int64_t kc, int c = 0) {
   RunGrid g;
   g.lshift = 0;
   while ((1 << g.lshift) < kc && g.lshift < 6) ++g.lshift;
   const int L = 1 << g.lshift, epr = kWave >> g.lshift;
-  g.rpw = run_rows_per_wave(n_edges, epr);
+  g.hot_rlog = -1;
+  if (c > 0 && n_edges >= ((int64_t)1 << 18) && !getenv("TS_SCATTER_NO_HOT")) {  // env: tuning aid
+    int cshift = 0;
+    while ((1 << cshift) < c) ++cshift;
+    g.hot_rlog = hot_rows_log(g.lshift + cshift);
+  }
+  g.rpw = run_rows_per_wave(n_edges, epr, g.hot_rlog >= 0 ? 64 : 32);
   const int64_t waves = (n_edges + (int64_t)g.rpw * epr - 1) / ((int64_t)g.rpw * epr);
   const int64_t blocks = (waves + kBlock / kWave - 1) / (kBlock / kWave);
   const int64_t ychunks = (kc + L - 1) / L;
@@ -634,6 +791,7 @@ struct KeyRun {
     make_keys<T, C, IS_MAX>(r, pos, x);
   }
   __device__ void combine(A &x, const A &y) const { x = x > y ? x : y; }
+  __device__ void begin_row(int, int) const {}
   __device__ void emit(int node, int64_t col, const A *x) const {
     keys_to_global<1>(keys + (int64_t)node * K + col, x, precheck);
   }
@@ -1102,19 +1260,28 @@ int launch_scatter_v(const ScatterArgs &a, int reduce, hipStream_t stream) {
           constexpr int CN = sizeof(T) < 4 ? 4 / (int)sizeof(T) : 1;  // columns per lane without 16-byte loads
           const bool word_ok = CN == 1 || (a.K % CN == 0 && (reinterpret_cast<uintptr_t>(a.out) & 3) == 0 &&
                                            (reinterpret_cast<uintptr_t>(a.src) & 3) == 0);
+          if (a.run_reduce && a.sk == 0 && a.B * a.N < 0x7FFFFFFFll && !word_ok) {
+            // rows that cannot be written word by word: one column per lane and atomic
+            const RunGrid g = run_grid(n_edges, a.K, 1);
+            if (g.ok) {
+              hipLaunchKernelGGL((scatter_add_run_kernel<T, 1, 1>), dim3(g.blocks, g.ychunks), dim3(kBlock), 0, stream, a,
+                                 g.lshift, g.rpw, g.hot_rlog);
+              return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
+            }
+          }
           if (a.run_reduce && a.sk == 0 && a.B * a.N < 0x7FFFFFFFll && word_ok) {
             constexpr int C = VEC > 1 ? VEC : CN;
             // 16-byte loads pay once the instruction rate limits the stream; small inputs are bound by
             // latency and do better with one atomic per lane straight from registers
             const bool wide = C > CN && n_src * (int64_t)sizeof(T) > ((int64_t)32 << 20);
-            const RunGrid g = run_grid(n_edges, a.K / (wide ? C : CN));
+            const RunGrid g = run_grid(n_edges, a.K / (wide ? C : CN), wide ? C : CN);
             if (g.ok) {
               if (wide)
                 hipLaunchKernelGGL((scatter_add_run_kernel<T, C>), dim3(g.blocks, g.ychunks), dim3(kBlock), 0, stream,
-                                   a, g.lshift, g.rpw);
+                                   a, g.lshift, g.rpw, g.hot_rlog);
               else
                 hipLaunchKernelGGL((scatter_add_run_kernel<T, CN>), dim3(g.blocks, g.ychunks), dim3(kBlock), 0, stream,
-                                   a, g.lshift, g.rpw);
+                                   a, g.lshift, g.rpw, g.hot_rlog);
               return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
             }
           }

@@ -603,6 +603,96 @@ def test_scatter_minmax_runs_of_equal_indices(capi, oracle, shape, kind, reduce,
         assert_exact(arg, want_arg, f"{kind} out_given={out_given} arg")
 
 
+HOT_INDEX_KINDS = ["hub", "zipf", "sorted_hub", "uniform"]
+
+
+def hot_index(kind, rng, E, N):
+    """Indices of more than 2^18 entries (the size from which the sum kernels keep their LDS table of
+    hot rows): a hub that owns a fifth of the entries, a Zipf law, hub entries sprinkled over a
+    sorted index, and a uniform index (no row gets confirmed)."""
+    if kind == "zipf":
+        return np.minimum(rng.zipf(1.3, size=E) - 1, N - 1)
+    idx = rng.integers(0, N, size=E)
+    if kind == "uniform":
+        return idx
+    if kind == "sorted_hub":
+        idx = np.sort(idx)
+    idx[rng.random(E) < 0.2] = N // 3
+    return idx
+
+
+@pytest.mark.parametrize("K,kind,dtype", product(
+    [1, 3, 8, 64, 100], HOT_INDEX_KINDS,
+    [torch.float32, torch.float64, torch.bfloat16, torch.float16, torch.int32, torch.int64]))
+def test_scatter_sum_hot_rows(capi, oracle, K, kind, dtype):
+    """Sum with the workgroup table of hot rows in play: exact for integers, within tolerance of
+    the exact sum for floats, with and without a given out; count shares the kernel."""
+    E = 300_000 if K <= 8 else 270_000
+    N = 5000
+    rng = np.random.default_rng(K * 101 + len(kind))
+    index1 = torch.from_numpy(hot_index(kind, rng, E, N))
+    index = index1.view(E, 1).expand(E, K)
+    if dtype.is_floating_point:
+        src = torch.from_numpy(rng.standard_normal(size=(E, K))).to(dtype)
+    else:
+        src = torch.from_numpy(rng.integers(-1000, 1000, size=(E, K))).to(dtype)
+    for out_given in (False, True):
+        prev = (torch.from_numpy(rng.standard_normal(size=(N, K))).to(dtype) if dtype.is_floating_point
+                else torch.from_numpy(rng.integers(-1000, 1000, size=(N, K))).to(dtype))
+        out = prev.clone().to(DEV) if out_given else torch.full((N, K), 9, dtype=dtype, device=DEV)
+        capi.scatter(src.to(DEV), index1.to(DEV), out, None, 1, E, K, N, 0, 1, 0, capi.SUM, out_given)
+        torch.cuda.synchronize()
+        if not dtype.is_floating_point:
+            want = oracle.scatter(src, index, 0, prev.clone() if out_given else None, None if out_given else N,
+                                  "sum")[0]
+            assert_exact(out, want, f"{kind} out_given={out_given}")
+            continue
+        exact = oracle.scatter(src.double(), index, 0, None, N, "sum")[0]
+        absum = oracle.scatter(src.double().abs(), index, 0, None, N, "sum")[0]
+        want = exact + (prev.double() if out_given else 0)
+        rtol = RTOL[dtype]
+        err = (out.cpu().double() - want).abs()
+        bound = rtol * want.abs() + rtol * (absum + (prev.double().abs() if out_given else 0)).clamp(min=1e-30)
+        if dtype in (torch.bfloat16, torch.float16):
+            # partial sums leave the table or the wavefront as 16-bit values: one rounding of the running
+            # total per partial sum, and a hub collects one partial sum per workgroup
+            bound = bound + 2.0 ** -8 * 64 * want.abs().clamp(min=1.0)
+        assert bool((err <= bound).all()), (kind, out_given, float((err - bound).max()))
+    cnt = torch.empty((N,), dtype=torch.float32, device=DEV)
+    capi.scatter_count(index1.to(DEV), cnt, 1, E, N, 0, 1)
+    torch.cuda.synchronize()
+    assert torch.equal(cnt.cpu(), torch.bincount(index1, minlength=N).float())
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_scatter_sum_single_16bit_columns_leave_neighbours_alone(capi, dtype):
+    """Rows of one 16-bit column are added with a packed-pair atomic whose other half is +0.0: the
+    neighbouring elements of a given out keep their bits (denormals, infinities, NaN; -0.0 may turn
+    into +0.0), also when out starts or ends in the middle of a 32-bit word."""
+    N = 64
+    specials = torch.tensor([1e-40, -1e-40, float("inf"), float("-inf"), float("nan"), -0.0, 0.0, 1.5, 6e-8, -6e-8])
+    for offset in (0, 1):
+        buf = torch.zeros(N + 2, dtype=dtype)
+        buf[:] = specials.to(dtype).repeat(7)[:N + 2]
+        prev = buf[offset:offset + N].clone()
+        dbuf = buf.to(DEV)
+        out = dbuf[offset:offset + N]
+        touched = torch.tensor([7, 8, 21, N - 1, 0])  # values 1.5 or zeros at those positions? set them
+        prev_touched = prev.clone()
+        src = torch.ones(len(touched), dtype=dtype)
+        capi.scatter(src.to(DEV), touched.to(DEV), out, None, 1, len(touched), 1, N, 0, 1, 0, capi.SUM, True)
+        torch.cuda.synchronize()
+        got = dbuf.cpu()
+        mask = torch.ones(N + 2, dtype=torch.bool)
+        mask[touched + offset] = False
+        a, b = _bits(got)[mask], _bits(buf)[mask]
+        same = (a == b) | ((got[mask] == 0) & (buf[mask] == 0))
+        assert bool(same.all()), (offset, got[mask][~same], buf[mask][~same])
+        want = (prev_touched[touched].float() + 1).to(dtype)
+        ok = (got[touched + offset] == want) | (want != want)
+        assert bool(ok.all()), (offset, got[touched + offset], want)
+
+
 def test_scatter_sum_plain_atomic_kernel_still_covered(capi, oracle, monkeypatch):
     """The one-atomic-per-element kernel (used for per-element indices) with a shared index."""
     monkeypatch.setenv("TS_SCATTER_RUNS", "0")
