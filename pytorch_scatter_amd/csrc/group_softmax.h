@@ -119,11 +119,13 @@ template <typename T, int C_> struct GroupMaxRun {
     }
   }
   __device__ void combine(A &x, const A &y) const { x = x > y ? x : y; }
-  __device__ void begin_row(int, int) const {}
+  // a running maximum is improved rarely, so read first (a stale read only costs a spare atomic);
+  // not in rows of the wavefront that look sorted, where each slot gets one atomic anyway
+  bool check = true;
+  __device__ void begin_row(int heads, int entries) { check = heads * 2 > entries; }
   __device__ void emit(int node, int64_t col, const A *x) const {
     A *p = gmax + (int64_t)node * K + col;
-    // a running maximum is improved rarely; a stale read only costs a spare atomic
-    if (x[0] > *p) __hip_atomic_fetch_max(p, x[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (!check || x[0] > *p) __hip_atomic_fetch_max(p, x[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
 };
 

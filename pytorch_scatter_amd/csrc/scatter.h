@@ -791,9 +791,14 @@ struct KeyRun {
     make_keys<T, C, IS_MAX>(r, pos, x);
   }
   __device__ void combine(A &x, const A &y) const { x = x > y ? x : y; }
-  __device__ void begin_row(int, int) const {}
+  // The read before the atomic pays where a slot collects many entries that do not sit next to each
+  // other (a hub in an unsorted index). In a row of the wavefront in which at least half of the
+  // entries continue a run the index looks sorted: one atomic per slot anyway, and the read would
+  // only make the wavefront wait for memory.
+  bool check = true;
+  __device__ void begin_row(int heads, int entries) { check = heads * 2 > entries; }
   __device__ void emit(int node, int64_t col, const A *x) const {
-    keys_to_global<1>(keys + (int64_t)node * K + col, x, precheck);
+    keys_to_global<1>(keys + (int64_t)node * K + col, x, check ? precheck : 0);
   }
 };
 
