@@ -211,6 +211,26 @@ int ts_group_softmax_backward(const void *result, const void *grad_out,
                               int dtype, int log_space, void *workspace,
                               size_t workspace_bytes, ts_stream_t stream);
 
+/* logsumexp over the entries that share an index, one index per row:
+ *   out[b, n, k] = log(sum_group exp(src - m) + eps) + m,  m = group max starting from -inf;
+ *   NaN entries drop out; NaN and -inf results (empty groups) become 0, +inf the largest finite value.
+ * Replaces the op sequence of torch_scatter/composite/logsumexp.py:8-57 for the call without `out`
+ * (the reference has no single launcher for it). out is [B, N, K] and fully written when E > 0.
+ * Backward: grad_in[b, e, k] = grad_out[b, n, k] * exp(src[b, e, k] - out[b, n, k]), n = index of e.
+ * Workspace as for ts_group_softmax. Floating types only.
+ */
+int ts_group_logsumexp(const void *src, const int64_t *index, void *out,
+                       int64_t B, int64_t E, int64_t K, int64_t N,
+                       int64_t index_stride_b, int64_t index_stride_e,
+                       int dtype, double eps, void *workspace,
+                       size_t workspace_bytes, ts_stream_t stream);
+int ts_group_logsumexp_backward(const void *src, const int64_t *index,
+                                const void *out, const void *grad_out,
+                                void *grad_in, int64_t B, int64_t E, int64_t K,
+                                int64_t N, int64_t index_stride_b,
+                                int64_t index_stride_e, int dtype,
+                                ts_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -444,3 +444,13 @@ def scatter_softmax_backward(result, grad_out, index, dim=-1, dim_size=None, log
         return grad_out - result.exp() * total.gather(dim, index)
     total = scatter(result * grad_out, index, dim, None, dim_size, "sum")[0]
     return result * (grad_out - total.gather(dim, index))
+
+
+def scatter_logsumexp_backward(src, result, grad_out, index, dim=-1):
+    """What autograd derives for scatter_logsumexp above (closed form):
+    grad_out[group] * exp(src - result[group]); entries that dropped out of the
+    forward sum (NaN) get 0."""
+    index, dim = _py_broadcast(index, src, dim)
+    w = (src - result.gather(dim, index)).exp()
+    w = torch.where(torch.isnan(w), torch.zeros_like(w), w)
+    return grad_out.gather(dim, index) * w

@@ -28,6 +28,7 @@ EXPORTS = (
     "ts_segment_mean_coo_backward",
     "ts_scatter", "ts_scatter_count", "ts_divide_by_count", "ts_arg_backward",
     "ts_group_softmax_workspace_bytes", "ts_group_softmax", "ts_group_softmax_backward",
+    "ts_group_logsumexp", "ts_group_logsumexp_backward",
 )
 
 _lib = None
@@ -188,3 +189,21 @@ def group_softmax_backward(result, grad_out, index, grad_in, B, E, K, N, sb, se,
                                                int(log_space), _p(ws), ctypes.c_size_t(nbytes),
                                                _stream(grad_in)))
     return ws
+
+
+def group_logsumexp(src, index, out, B, E, K, N, sb, se, eps: float = 1e-12):
+    _dev(src, index, out)
+    ws, nbytes = _group_workspace(out, B, N, K)
+    with torch.cuda.device(out.device):
+        _check(lib().ts_group_logsumexp(_p(src), _p(index), _p(out), _i(B), _i(E), _i(K), _i(N), _i(sb), _i(se),
+                                        DTYPE[out.dtype], ctypes.c_double(eps), _p(ws), ctypes.c_size_t(nbytes),
+                                        _stream(out)))
+    return ws
+
+
+def group_logsumexp_backward(src, index, out, grad_out, grad_in, B, E, K, N, sb, se):
+    _dev(src, index, out, grad_out, grad_in)
+    with torch.cuda.device(grad_in.device):
+        _check(lib().ts_group_logsumexp_backward(_p(src), _p(index), _p(out), _p(grad_out), _p(grad_in), _i(B),
+                                                 _i(E), _i(K), _i(N), _i(sb), _i(se), DTYPE[grad_in.dtype],
+                                                 _stream(grad_in)))

@@ -1,13 +1,13 @@
 """Group-wise statistics over the entries that share an index: softmax,
 log-softmax, logsumexp and standard deviation (API of
-torch_scatter/composite/{softmax,logsumexp,std}.py). Softmax and log-softmax
-are one fused operator; logsumexp and std are composed from the scatter
+torch_scatter/composite/{softmax,logsumexp,std}.py). Softmax, log-softmax
+and logsumexp are fused operators; std is composed from the scatter
 operators."""
 from typing import Optional
 
 import torch
 
-from .scatter import scatter_max, scatter_sum
+from .scatter import scatter_sum
 
 
 def _expand_index(index: torch.Tensor, like: torch.Tensor, dim: int) -> torch.Tensor:
@@ -50,30 +50,13 @@ def scatter_log_softmax(src: torch.Tensor, index: torch.Tensor, dim: int = -1,
 def scatter_logsumexp(src: torch.Tensor, index: torch.Tensor, dim: int = -1,
                       out: Optional[torch.Tensor] = None, dim_size: Optional[int] = None,
                       eps: float = 1e-12) -> torch.Tensor:
+    """``log(sum(exp(src)) + eps)`` over the entries that share an index, stabilised by
+    the group maximum; groups without entries give 0
+    (torch_scatter/composite/logsumexp.py:8-57). One fused operator (two passes over
+    ``src`` forward, one backward) unless ``out`` is given or the index differs between
+    the columns of a row; then the same sequence as upstream on the scatter operators."""
     _require_float(src, "scatter_logsumexp")
-    index = _expand_index(index, src, dim)
-    if out is not None:
-        dim_size = out.size(dim)
-    elif dim_size is None:
-        dim_size = int(index.max()) + 1
-    shape = list(src.size())
-    shape[dim] = dim_size
-    # groups without entries keep -inf so that they drop out of the result
-    group_max = torch.full(shape, float("-inf"), dtype=src.dtype, device=src.device)
-    scatter_max(src, index, dim, group_max, dim_size)
-    z = src - group_max.gather(dim, index)
-    z.masked_fill_(torch.isnan(z), float("-inf"))
-    previous: Optional[torch.Tensor] = None
-    if out is not None:
-        previous = out.clone()
-        out = out.sub_(group_max).exp_()
-    total = scatter_sum(z.exp_(), index, dim, out, dim_size)
-    result = total.add_(eps).log_().add_(group_max)
-    if previous is None:
-        return result.nan_to_num_(neginf=0.0)
-    bad = ~result.isfinite()
-    result[bad] = previous[bad]
-    return result
+    return torch.ops.torch_scatter.scatter_logsumexp(src, index, dim, out, dim_size, eps)
 
 
 def scatter_std(src: torch.Tensor, index: torch.Tensor, dim: int = -1,

@@ -394,6 +394,9 @@ int run_group_softmax(const void *src, const void *grad, const int64_t *index, v
   g.sb = sb;
   g.se = se;
   g.eps = eps;
+  g.node_out = nullptr;
+  g.node_grad = nullptr;
+  g.from_neg_inf = 0;
   const int full = kVecBytes / kElemBytes[dtype];
   const bool al = aligned16(src) && aligned16(out) && (!grad || aligned16(grad));
   const int vec = (full > 1 && K % full == 0 && al) ? full : 1;
@@ -421,6 +424,61 @@ int ts_group_softmax_backward(const void *result, const void *grad_out, const in
   return run_group_softmax(result, grad_out, index, grad_in, B, E, K, N, index_stride_b, index_stride_e, dtype,
                            log_space ? GS_LOG_SOFTMAX_BWD : GS_SOFTMAX_BWD, 0.0, workspace, workspace_bytes,
                            static_cast<hipStream_t>(stream));
+}
+
+int ts_group_logsumexp(const void *src, const int64_t *index, void *out, int64_t B, int64_t E, int64_t K, int64_t N,
+                       int64_t index_stride_b, int64_t index_stride_e, int dtype, double eps, void *workspace,
+                       size_t workspace_bytes, ts_stream_t stream) {
+  if (!valid_dtype(dtype) || !sizes_ok(B, N, E, K)) return TS_ERR_BAD_ARG;
+  if (!is_float_dtype(dtype)) return TS_ERR_UNSUPPORTED;
+  if (B * N * K == 0) return TS_OK;
+  if (!out || (B * E * K > 0 && (!src || !index))) return TS_ERR_BAD_ARG;
+  if (B * N >= 0x7FFFFFFFll) return TS_ERR_UNSUPPORTED;
+  const size_t need = group_workspace_bytes(B, N, K, kElemBytes[dtype]);
+  if (!workspace || workspace_bytes < need || !aligned16(workspace)) return TS_ERR_WORKSPACE;
+  GroupArgs g = {};
+  g.src = src;
+  g.index = index;
+  g.out = out;
+  g.gmax = workspace;
+  g.gsum = static_cast<char *>(workspace) + need / 2;
+  g.B = B;
+  g.E = E;
+  g.K = K;
+  g.N = N;
+  g.sb = index_stride_b;
+  g.se = index_stride_e;
+  g.eps = eps;
+  g.from_neg_inf = 1;
+  const int full = kVecBytes / kElemBytes[dtype];
+  const int vec = (full > 1 && K % full == 0 && aligned16(src)) ? full : 1;
+  return dispatch_group_softmax(dtype, g, GS_LSE, vec, static_cast<hipStream_t>(stream));
+}
+
+int ts_group_logsumexp_backward(const void *src, const int64_t *index, const void *out, const void *grad_out,
+                                void *grad_in, int64_t B, int64_t E, int64_t K, int64_t N, int64_t index_stride_b,
+                                int64_t index_stride_e, int dtype, ts_stream_t stream) {
+  if (!valid_dtype(dtype) || !sizes_ok(B, N, E, K)) return TS_ERR_BAD_ARG;
+  if (!is_float_dtype(dtype)) return TS_ERR_UNSUPPORTED;
+  if (B * E * K == 0) return TS_OK;
+  if (!src || !index || !out || !grad_out || !grad_in) return TS_ERR_BAD_ARG;
+  if (N == 0 || B * N >= 0x7FFFFFFFll) return TS_ERR_UNSUPPORTED;
+  GroupArgs g = {};
+  g.src = src;
+  g.index = index;
+  g.out = grad_in;
+  g.node_out = out;
+  g.node_grad = grad_out;
+  g.B = B;
+  g.E = E;
+  g.K = K;
+  g.N = N;
+  g.sb = index_stride_b;
+  g.se = index_stride_e;
+  const int full = kVecBytes / kElemBytes[dtype];
+  const bool al = aligned16(src) && aligned16(grad_in) && aligned16(out) && aligned16(grad_out);
+  const int vec = (full > 1 && K % full == 0 && al) ? full : 1;
+  return dispatch_group_softmax(dtype, g, GS_LSE_BWD, vec, static_cast<hipStream_t>(stream));
 }
 
 }  // extern "C"

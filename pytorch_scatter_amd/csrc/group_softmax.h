@@ -64,7 +64,7 @@ template <typename T> __device__ __forceinline__ typename OrdKey<typename Acc<T>
   return OrdKey<typename Acc<T>::type>::enc(to_acc<T>(ElemLim<T>::lowest()));
 }
 
-enum { GS_SOFTMAX = 0, GS_LOG_SOFTMAX = 1, GS_SOFTMAX_BWD = 2, GS_LOG_SOFTMAX_BWD = 3 };
+enum { GS_SOFTMAX = 0, GS_LOG_SOFTMAX = 1, GS_SOFTMAX_BWD = 2, GS_LOG_SOFTMAX_BWD = 3, GS_LSE = 4, GS_LSE_BWD = 5 };
 
 struct GroupArgs {
   const void *src;       // [B, E, K]: forward input; backward: the forward result y
@@ -76,6 +76,9 @@ struct GroupArgs {
   int64_t B, E, K, N;
   int64_t sb, se;
   double eps;
+  const void *node_out;   // [B, N, K]: logsumexp backward, the forward result
+  const void *node_grad;  // [B, N, K]: logsumexp backward, its gradient
+  int from_neg_inf;       // the group maximum starts from -inf (logsumexp) instead of lowest() (softmax)
 };
 
 inline size_t group_align(size_t v) { return (v + 255) / 256 * 256; }
@@ -92,7 +95,7 @@ __global__ __launch_bounds__(kBlock) void group_init_kernel(GroupArgs g, int wit
   const int64_t n = g.B * g.N * g.K;
   KB *gmax = static_cast<KB *>(g.gmax);
   F *gsum = static_cast<F *>(g.gsum);
-  const KB empty = group_empty_key<T>();
+  const KB empty = g.from_neg_inf ? OrdKey<F>::enc(-INFINITY) : group_empty_key<T>();
   for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlock) {
     if (with_max) gmax[i] = empty;
     gsum[i] = (F)0;
@@ -141,15 +144,16 @@ __global__ __launch_bounds__(kBlock) void group_max_run_kernel(ScatterArgs a, Gr
   run_reduce_wave(a, lshift, rows_per_wave, p, s_stage[threadIdx.x / kWave]);
 }
 
-// the group maximum a row is shifted by
-template <typename T, int C>
+// the group maximum a row is shifted by. Softmax: a group in which nothing beat lowest() shifts by 0
+// (scatter_max's result for an untouched slot); logsumexp starts from -inf and keeps it.
+template <typename T, int C, bool LSE = false>
 __device__ __forceinline__ void group_shift(const void *gmax, int64_t slot, typename Acc<T>::type *m) {
   typedef typename Acc<T>::type F;
   typedef typename OrdKey<F>::bits KB;
   const Vec<KB, C> k = load_vec<KB, C>(static_cast<const KB *>(gmax) + slot);
   const KB empty = group_empty_key<T>();
 #pragma unroll
-  for (int c = 0; c < C; ++c) m[c] = k.v[c] == empty ? (F)0 : OrdKey<F>::dec(k.v[c]);
+  for (int c = 0; c < C; ++c) m[c] = (!LSE && k.v[c] == empty) ? (F)0 : OrdKey<F>::dec(k.v[c]);
 }
 
 // ---- pass 2: group sums of a per-entry term
@@ -168,7 +172,7 @@ template <typename T, int C_, int MODE> struct GroupSumRun : HotState<typename A
   int64_t K;
   __device__ A identity() const { return (A)0; }
   __device__ void load(int64_t e, int64_t, int64_t col, int node, A *x) const {
-    if constexpr (MODE == GS_SOFTMAX || MODE == GS_LOG_SOFTMAX) {
+    if constexpr (MODE == GS_SOFTMAX || MODE == GS_LOG_SOFTMAX || MODE == GS_LSE) {
       const Vec<T, C> r = load_vec_stream<T, C>(src + e * K + col);
       if (node < 0) {
 #pragma unroll
@@ -176,9 +180,13 @@ template <typename T, int C_, int MODE> struct GroupSumRun : HotState<typename A
         return;
       }
       A m[C];
-      group_shift<T, C>(gmax, (int64_t)node * K + col, m);
+      group_shift<T, C, MODE == GS_LSE>(gmax, (int64_t)node * K + col, m);
 #pragma unroll
-      for (int c = 0; c < C; ++c) x[c] = round_elem<T>(exp_acc(round_elem<T>(to_acc<T>(r.v[c]) - m[c])));
+      for (int c = 0; c < C; ++c) {
+        A z = round_elem<T>(to_acc<T>(r.v[c]) - m[c]);
+        if (MODE == GS_LSE && z != z) z = -INFINITY;  // NaN entries and -inf - -inf drop out (logsumexp.py:41)
+        x[c] = round_elem<T>(exp_acc(z));
+      }
     } else if constexpr (MODE == GS_SOFTMAX_BWD) {
       const Vec<T, C> y = load_vec_stream<T, C>(src + e * K + col);
       const Vec<T, C> gr = load_vec_stream<T, C>(grad + e * K + col);
@@ -261,6 +269,19 @@ __global__ __launch_bounds__(kBlock) void group_finish_kernel(GroupArgs g) {
           continue;
         }
         const int64_t slot = (bb[u] * g.N + idx[u]) * g.K + k0;
+        if constexpr (MODE == GS_LSE_BWD) {
+          // d logsumexp / d src = exp(src - result) (= exp(z) / (sum + eps)); NaN entries dropped out forward
+          const Vec<T, VEC> o = load_vec<T, VEC>(static_cast<const T *>(g.node_out) + slot);
+          const Vec<T, VEC> go = load_vec<T, VEC>(static_cast<const T *>(g.node_grad) + slot);
+#pragma unroll
+          for (int v = 0; v < VEC; ++v) {
+            const F xv = to_acc<T>(x[u].v[v]);
+            const F w = exp_acc(xv - to_acc<T>(o.v[v]));
+            r.v[v] = from_acc<T>(xv != xv || w != w ? (F)0 : to_acc<T>(go.v[v]) * w);
+          }
+          store_vec_stream<T, VEC>(out + be * g.K + k0, r);
+          continue;
+        }
         const Vec<F, VEC> s = load_vec<F, VEC>(gsum + slot);
         F mx[VEC];
         if (MODE == GS_SOFTMAX || MODE == GS_LOG_SOFTMAX) group_shift<T, VEC>(g.gmax, slot, mx);
@@ -288,6 +309,27 @@ __global__ __launch_bounds__(kBlock) void group_finish_kernel(GroupArgs g) {
         store_vec_stream<T, VEC>(out + be * g.K + k0, r);
       }
     }
+  }
+}
+
+// logsumexp: result per group, log(sum + eps) + max with the reference's clean-up
+// (composite/logsumexp.py:51-54: NaN and -inf -> 0, +inf -> largest finite value)
+template <typename T>
+__global__ __launch_bounds__(kBlock) void group_lse_finish_kernel(GroupArgs g) {
+  typedef typename Acc<T>::type F;
+  typedef typename OrdKey<F>::bits KB;
+  const int64_t n = g.B * g.N * g.K;
+  const KB *gmax = static_cast<const KB *>(g.gmax);
+  const F *gsum = static_cast<const F *>(g.gsum);
+  T *out = static_cast<T *>(g.out);
+  const F eps = (F)g.eps;
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlock) {
+    const F m = OrdKey<F>::dec(gmax[i]);
+    const F l = round_elem<T>(log_acc(round_elem<T>(round_elem<T>(gsum[i]) + eps)));
+    F o = round_elem<T>(l + m);
+    if (o != o || o == -INFINITY) o = (F)0;
+    if (o == INFINITY) o = to_acc<T>(ElemLim<T>::max());
+    out[i] = from_acc<T>(o);
   }
 }
 
@@ -326,8 +368,32 @@ int launch_group_softmax_m(const GroupArgs &g, hipStream_t stream) {
 }
 
 template <typename T, int VEC>
+int launch_group_lse_v(const GroupArgs &g, bool backward, hipStream_t stream) {
+  const int64_t n_edges = g.B * g.E;
+  if (g.B * g.N >= 0x7FFFFFFFll) return TS_ERR_UNSUPPORTED;
+  if (backward) {
+    hipLaunchKernelGGL((group_finish_kernel<T, VEC, GS_LSE_BWD>), dim3(scatter_grid(n_edges, g.K / VEC, kBlock, 4)),
+                       dim3(kBlock), 0, stream, g);
+    return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
+  }
+  const RunGrid rg = run_grid(n_edges, g.K / VEC, VEC);
+  if (!rg.ok) return TS_ERR_UNSUPPORTED;
+  const ScatterArgs a = group_index_args(g);
+  const dim3 gd(rg.blocks, rg.ychunks);
+  const unsigned g_out = grid_for(g.B * g.N * g.K);
+  hipLaunchKernelGGL(group_init_kernel<T>, dim3(g_out), dim3(kBlock), 0, stream, g, 1);
+  hipLaunchKernelGGL((group_max_run_kernel<T, VEC>), gd, dim3(kBlock), 0, stream, a, g, rg.lshift, rg.rpw);
+  hipLaunchKernelGGL((group_sum_run_kernel<T, VEC, GS_LSE>), gd, dim3(kBlock), 0, stream, a, g, rg.lshift, rg.rpw,
+                     rg.hot_rlog);
+  hipLaunchKernelGGL(group_lse_finish_kernel<T>, dim3(g_out), dim3(kBlock), 0, stream, g);
+  return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
+}
+
+template <typename T, int VEC>
 int launch_group_softmax_v(const GroupArgs &g, int mode, hipStream_t stream) {
   switch (mode) {
+  case GS_LSE: return launch_group_lse_v<T, VEC>(g, false, stream);
+  case GS_LSE_BWD: return launch_group_lse_v<T, VEC>(g, true, stream);
   case GS_SOFTMAX: return launch_group_softmax_m<T, VEC, GS_SOFTMAX>(g, stream);
   case GS_LOG_SOFTMAX: return launch_group_softmax_m<T, VEC, GS_LOG_SOFTMAX>(g, stream);
   case GS_SOFTMAX_BWD: return launch_group_softmax_m<T, VEC, GS_SOFTMAX_BWD>(g, stream);

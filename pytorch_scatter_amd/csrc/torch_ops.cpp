@@ -681,6 +681,44 @@ struct GroupSoftmaxFn : public torch::autograd::Function<GroupSoftmaxFn> {
   }
 };
 
+// scatter_logsumexp of torch_scatter/composite/logsumexp.py:8-57 for the call without `out`
+struct GroupLogSumExpFn : public torch::autograd::Function<GroupLogSumExpFn> {
+  static variable_list forward(AutogradContext *ctx, Variable src, Variable index, int64_t dim, int64_t N,
+                               double eps) {
+    check_device(src, "src");
+    check_device(index, "index");
+    c10::DeviceGuard guard(src.device());
+    src = src.contiguous();
+    const GroupLayout l = group_layout(src, index, dim);
+    auto sizes = src.sizes().vec();
+    sizes[dim] = N;
+    Tensor out = at::empty(sizes, src.options());
+    Tensor ws = workspace(ts_group_softmax_workspace_bytes(l.B, N, l.K, dtype_code(src)), src);
+    check_status(ts_group_logsumexp(src.data_ptr(), index.data_ptr<int64_t>(), out.data_ptr(), l.B, l.E, l.K, N, l.sb,
+                                    l.se, dtype_code(src), eps, ws.data_ptr(), static_cast<size_t>(ws.numel()),
+                                    stream_of(src)),
+                 "scatter_logsumexp");
+    ctx->saved_data["dim"] = dim;
+    ctx->save_for_backward({src, index, out});
+    return {out};
+  }
+
+  static variable_list backward(AutogradContext *ctx, variable_list grad_outs) {
+    auto saved = ctx->get_saved_variables();
+    Tensor src = saved[0], index = saved[1], out = saved[2];
+    Tensor grad_out = grad_outs[0].contiguous();
+    c10::DeviceGuard guard(src.device());
+    const int64_t dim = ctx->saved_data["dim"].toInt();
+    const GroupLayout l = group_layout(src, index, dim);
+    Tensor grad_in = at::empty_like(src);
+    check_status(ts_group_logsumexp_backward(src.data_ptr(), index.data_ptr<int64_t>(), out.data_ptr(),
+                                             grad_out.data_ptr(), grad_in.data_ptr(), l.B, l.E, l.K, out.size(dim),
+                                             l.sb, l.se, dtype_code(src), stream_of(src)),
+                 "scatter_logsumexp backward");
+    return {grad_in, Variable(), Variable(), Variable(), Variable()};
+  }
+};
+
 // ------------------------------------------------------- registered functions
 Tensor scatter_sum(Tensor src, Tensor index, int64_t dim, OptTensor out, OptInt dim_size) {
   return ScatterFn<TS_SUM>::apply(src, index, dim, out, dim_size)[0];
@@ -754,6 +792,44 @@ Tensor scatter_softmax(Tensor src, Tensor index, int64_t dim, OptInt dim_size, b
   return z.sub(norm);
 }
 
+Tensor scatter_logsumexp(Tensor src, Tensor index, int64_t dim, OptTensor out, OptInt dim_size, double eps) {
+  TORCH_CHECK(src.is_floating_point(),
+              "`scatter_logsumexp` can only be computed over tensors with floating point data types.");
+  dim = dim < 0 ? src.dim() + dim : dim;
+  index = broadcast(index, src, dim);
+  TORCH_CHECK(index.scalar_type() == at::kLong, "index must be int64");
+  int64_t N;
+  if (out.has_value())
+    N = out.value().size(dim);
+  else if (dim_size.has_value())
+    N = dim_size.value();
+  else
+    N = index.numel() == 0 ? 0 : 1 + index.max().item<int64_t>();
+  auto sizes = src.sizes().vec();
+  sizes[dim] = N;
+  if (!out.has_value() && src.numel() > 0 && N > 0) {
+    const GroupLayout l = group_layout(src, index, dim);
+    if (l.fused && l.B * N < 0x7FFFFFFFll) return GroupLogSumExpFn::apply(src, index, dim, N, eps)[0];
+  }
+  // composite/logsumexp.py:29-57
+  const double neg_inf = -std::numeric_limits<double>::infinity();
+  Tensor group_max = at::full(sizes, neg_inf, src.options());
+  if (src.numel() > 0) scatter_max(src, index, dim, group_max, N);
+  Tensor z = src - group_max.gather(dim, index);
+  z.masked_fill_(z.isnan(), neg_inf);
+  OptTensor previous;
+  if (out.has_value()) {
+    previous = out.value().clone();
+    out = out.value().sub_(group_max).exp_();
+  }
+  Tensor total = scatter_sum(z.exp_(), index, dim, out, N);
+  Tensor result = total.add_(eps).log_().add_(group_max);
+  if (!previous.has_value()) return result.nan_to_num_(0.0, std::nullopt, 0.0);
+  Tensor bad = result.isfinite().logical_not();
+  result.index_put_({bad}, previous.value().index({bad}));
+  return result;
+}
+
 int64_t cuda_version() { return ts_hip_version(); }  // csrc/version.cpp:28-38 returns HIP_VERSION on ROCm
 
 }  // namespace
@@ -775,4 +851,5 @@ static auto registry = torch::RegisterOperators()
                            .op("torch_scatter::segment_min_coo", &segment_min_coo)
                            .op("torch_scatter::segment_max_coo", &segment_max_coo)
                            .op("torch_scatter::gather_coo", &gather_coo)
-                           .op("torch_scatter::scatter_softmax", &scatter_softmax);
+                           .op("torch_scatter::scatter_softmax", &scatter_softmax)
+                           .op("torch_scatter::scatter_logsumexp", &scatter_logsumexp);

@@ -1,6 +1,7 @@
-"""The fused softmax / log-softmax over groups (ts_group_softmax and its
-backward through the C ABI, torch.ops.torch_scatter.scatter_softmax through the
-Python API) against the CPU oracle on the same seeded inputs.
+"""The fused softmax / log-softmax / logsumexp over groups (ts_group_softmax,
+ts_group_logsumexp and their backward calls through the C ABI,
+torch.ops.torch_scatter.scatter_softmax / scatter_logsumexp through the Python
+API) against the CPU oracle on the same seeded inputs.
 
 Bars. fp32 / fp64 compare with the oracle's result in the same type:
 rtol 1e-5 / 1e-12 (the two differ in the exp of the math library and in the
@@ -157,7 +158,7 @@ def test_operator_dims_and_autograd(ts, dim, shape, log_space):
     src = src_cpu.to(DEV).requires_grad_(True)
     shape1 = [1] * len(shape)
     shape1[d] = shape[d]
-    for idx in (index.to(DEV) if d == 0 or True else None, index.view(shape1).expand(shape).to(DEV)):
+    for idx in (index.to(DEV), index.view(shape1).expand(shape).to(DEV)):
         if idx.dim() == 1 and d != 0:
             idx = idx.view(shape1[:d + 1])  # leading dims broadcast, trailing dims implied
         src.grad = None
@@ -194,3 +195,80 @@ def test_operator_reference_cases_script_and_fallback(ts, oracle):
     assert ts.scatter_softmax(torch.empty(0, 4, device=DEV), torch.empty(0, dtype=torch.long, device=DEV), 0).shape == (0, 4)
     with pytest.raises(ValueError):
         ts.scatter_softmax(torch.ones(4, dtype=torch.long, device=DEV), torch.zeros(4, dtype=torch.long, device=DEV))
+
+
+# ------------------------------------------------------------------ logsumexp
+@pytest.mark.parametrize("shape,kind,dtype", product(SHAPES, ["random", "sorted", "hub"], DTYPES))
+def test_logsumexp_forward_and_backward_capi(capi, oracle, shape, kind, dtype):
+    B, E, K, N = shape
+    N = N + 3  # the last groups stay empty
+    rng = np.random.default_rng(E * 17 + K)
+    src = torch.from_numpy(rng.standard_normal(size=(B, E, K)) * 3).to(dtype)
+    index1 = make_index(kind, rng, E, N - 3)
+    index = index1.view(1, E, 1).expand(B, E, K)
+    exact = dtype in (torch.float32, torch.float64)
+    ref_src = src if exact else src.double()
+    out = torch.full((B, N, K), 7, dtype=dtype, device=DEV)
+    capi.group_logsumexp(src.to(DEV), index1.to(DEV), out, B, E, K, N, 0, 1)
+    torch.cuda.synchronize()
+    want = oracle.scatter_logsumexp(ref_src, index, 1, None, N).double()
+    e = EPS_T[dtype]
+    err = (out.cpu().double() - want).abs()
+    # 16-bit floats: z is rounded before the exp (relative error of a term up to eps_T * |z|, |z| <~ 25 here)
+    bound = e * (1.0 + want.abs()) if exact else e * (30.0 + want.abs())
+    assert bool((err <= bound).all()), float((err - bound).max())
+    assert float(out[:, N - 3:, :].abs().max()) == 0.0
+
+    grad = torch.from_numpy(rng.standard_normal(size=(B, N, K))).to(dtype)
+    grad_in = torch.empty((B, E, K), dtype=dtype, device=DEV)
+    capi.group_logsumexp_backward(src.to(DEV), index1.to(DEV), out, grad.to(DEV), grad_in, B, E, K, N, 0, 1)
+    torch.cuda.synchronize()
+    y64 = out.cpu().double()
+    want_g = oracle.scatter_logsumexp_backward(src.double(), y64, grad.double(), index, 1)
+    gerr = (grad_in.cpu().double() - want_g).abs()
+    gbound = 8 * e * want_g.abs() * (1 + (src.double() - y64.gather(1, index)).abs()) + \
+        (2.0 ** -23 if dtype == torch.float16 else 1e-30)
+    assert bool((gerr <= gbound).all()), ("backward", float((gerr - gbound).max()))
+
+
+def test_logsumexp_operator(ts, oracle):
+    # test/composite/test_logsumexp.py:5-45
+    inputs = torch.tensor([0.5, 0.5, 0.0, -2.1, 3.2, 7.0, -1.0, -100.0], device=DEV, requires_grad=True)
+    index = torch.tensor([0, 0, 1, 1, 1, 2, 4, 4], device=DEV)
+    outputs = ts.scatter_logsumexp(inputs, index)
+    for part, got in zip(inputs.split([2, 3, 1, 0, 2]), outputs.unbind()):
+        if part.numel() > 0:
+            assert torch.allclose(got, torch.logsumexp(part, dim=0), rtol=1e-6)
+        else:
+            assert got.item() == 0.0
+    outputs.backward(torch.randn_like(outputs))
+    jit = torch.jit.script(ts.scatter_logsumexp)
+    assert jit(inputs, index).tolist() == outputs.tolist()
+    out = torch.tensor([-10.0, -10.0], device=DEV)
+    ts.scatter_logsumexp(src=torch.tensor([-1.0, -50.0], device=DEV), index=torch.tensor([0, 0], device=DEV), out=out)
+    assert out.cpu().allclose(torch.tensor([-0.9999, -10.0]), atol=1e-4)
+    # special values: NaN entries drop out, a group of only -inf gives 0
+    x = torch.tensor([1.0, float("nan"), 2.0, float("-inf"), float("-inf"), 3.0])
+    idx = torch.tensor([0, 0, 0, 1, 1, 3])
+    got = ts.scatter_logsumexp(x.to(DEV), idx.to(DEV), dim_size=5)
+    assert torch.allclose(got.cpu(), oracle.scatter_logsumexp(x, idx, -1, None, 5), rtol=1e-6)
+    # dims, autograd against the per-group library routine
+    g = torch.Generator().manual_seed(2)
+    src_cpu = torch.randn(12, 40, 6, generator=g, dtype=torch.double)
+    idx = torch.randint(0, 5, (40,), generator=g)
+    ref = src_cpu.clone().requires_grad_(True)
+    want = torch.stack([torch.logsumexp(ref.index_select(1, (idx == n).nonzero().flatten()), 1) for n in range(5)], 1)
+    grad = torch.randn(12, 5, 6, generator=g, dtype=torch.double)
+    want.backward(grad)
+    src = src_cpu.to(DEV).requires_grad_(True)
+    got = ts.scatter_logsumexp(src, idx.view(1, 40).to(DEV), 1, dim_size=5)
+    got.backward(grad.to(DEV))
+    assert torch.allclose(got.detach().cpu(), want.detach(), rtol=1e-9, atol=1e-9)
+    assert torch.allclose(src.grad.cpu(), ref.grad, rtol=1e-8, atol=1e-10)
+    # an index that differs between the columns of a row: composed from the scatter operators
+    x = torch.randn(50, 6, generator=g)
+    idx2 = torch.randint(0, 5, (50, 6), generator=g)
+    got = ts.scatter_logsumexp(x.to(DEV), idx2.to(DEV), 0)
+    assert torch.allclose(got.cpu(), oracle.scatter_logsumexp(x, idx2, 0), rtol=1e-5, atol=1e-6)
+    with pytest.raises(ValueError):
+        ts.scatter_logsumexp(torch.ones(4, dtype=torch.long, device=DEV), torch.zeros(4, dtype=torch.long, device=DEV))

@@ -93,3 +93,17 @@ def test_softmax_backward_closed_form(oracle, log_space):
          else oracle.scatter_softmax(src.detach(), index, 0, 9))
     got = oracle.scatter_softmax_backward(y, grad, index, 0, 9, log_space)
     assert torch.allclose(got, src.grad, rtol=1e-9, atol=1e-12)
+
+
+def test_logsumexp_backward_closed_form(oracle):
+    g = torch.Generator().manual_seed(4)
+    src = (torch.randn(150, 4, generator=g, dtype=torch.double) * 2).requires_grad_(True)
+    index = torch.randint(0, 8, (150,), generator=g)  # group 8 stays empty
+    grad = torch.randn(9, 4, generator=g, dtype=torch.double)
+    rows = []
+    for sel in _groups(index, 9):
+        rows.append(torch.logsumexp(src.index_select(0, sel), 0) if sel.numel() else torch.zeros(4, dtype=torch.double))
+    torch.stack(rows).backward(grad)
+    y = oracle.scatter_logsumexp(src.detach(), index, 0, None, 9)
+    got = oracle.scatter_logsumexp_backward(src.detach(), y, grad, index, 0)
+    assert torch.allclose(got, src.grad, rtol=1e-9, atol=1e-12)
