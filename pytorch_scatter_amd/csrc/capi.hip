@@ -4,6 +4,9 @@
 #include <hip/hip_version.h>
 #include <stdlib.h>
 
+#include <atomic>
+#include <chrono>
+
 #include "csr_reduce.h"
 #include "csr_gather.h"
 #include "coo_gather.h"
@@ -80,6 +83,12 @@ int env_int(const char *name, int fallback) {
   return v ? atoi(v) : fallback;
 }
 
+// Tag of one call's carry flags: a process-wide counter that starts at the clock, 1 .. 2^61.
+uint64_t next_nonce() {
+  static std::atomic<uint64_t> counter{(uint64_t)std::chrono::steady_clock::now().time_since_epoch().count()};
+  return (counter.fetch_add(1, std::memory_order_relaxed) & ((1ull << 61) - 1)) + 1;
+}
+
 struct CsrWs {
   size_t total, off_args, off_meta;
 };
@@ -125,6 +134,10 @@ int run_csr_reduce(const void *src, const int64_t *indptr, void *out, int64_t *a
   a.ws_vals = ws;
   a.ws_args = reinterpret_cast<int32_t *>(static_cast<char *>(ws) + w.off_args);
   a.ws_meta = reinterpret_cast<int64_t *>(static_cast<char *>(ws) + w.off_meta);
+  // rows that cross tiles are finished inside the kernel when the carries fit 32- / 64-bit atomics and the
+  // four words of workspace per tile give every column chunk its flag; else by the second kernel
+  a.lookback = !p.small && kAccBytes[dtype] >= 4 && p.ychunks <= 4 && p.nblk > 1 && env_int("TS_CSR_LOOKBACK", 1);
+  a.nonce = next_nonce();
   return dispatch_csr_reduce(dtype, a, p, B, reduce, stream);
 }
 

@@ -47,7 +47,45 @@ struct CsrReduceArgs {
   void *ws_vals;      // Acc [B][nblk][2][K]
   int32_t *ws_args;   // int32 [B][nblk][2][K]  (min/max)
   int64_t *ws_meta;   // int64 [B][nblk][4]: head_row, head_closes, tail_row, length of the tail row
+                      // (look-back mode: one carry flag per column chunk instead)
+  int lookback;       // rows that cross tiles are finished inside the kernel (see carry_* below)
+  uint64_t nonce;     // tag of this call's carry flags, never 0
 };
+
+// ---- rows that cross tiles, finished without a second kernel ---------------------------------
+// The tile in which such a row ends walks back over the tiles before it. A tile whose last row is
+// still open at its end publishes that row's partial result as its carry: kCarryTail when the row
+// began inside the tile, kCarryPass when it only passes through (then the walk continues with the
+// tile before). Carries and flags move through device-scope read-modify-write atomics, which execute
+// at the memory side and so are coherent between the XCDs' L2 caches without a cache write-back (a
+// release fence per workgroup was measured and made the kernel 4x slower). The flag is written
+// after the wavefront has received the returns of its carry writes, i.e. after they were performed.
+// Tiles only ever wait for tiles with a smaller index, which the dispatcher started earlier, and
+// publishing never waits, so the walk cannot deadlock; it is bounded all the same and gives up on an
+// indptr that is not monotone. A flag holds the call's nonce, so stale workspace content never
+// matches, and its reader clears it, so a replay of a captured launch (same nonce, same workspace)
+// starts clean.
+constexpr uint64_t kCarryTail = 1, kCarryPass = 2;
+constexpr int kCarrySpin = 1 << 20;
+
+template <typename A> struct CarryBits { typedef uint32_t type; };
+template <> struct CarryBits<double> { typedef uint64_t type; };
+template <> struct CarryBits<int64_t> { typedef uint64_t type; };
+
+template <typename A> __device__ __forceinline__ uint64_t carry_put(A *p, A v) {
+  typedef typename CarryBits<A>::type U;
+  static_assert(sizeof(U) == sizeof(A), "");
+  U bits;
+  __builtin_memcpy(&bits, &v, sizeof(A));
+  return (uint64_t)__hip_atomic_exchange(reinterpret_cast<U *>(p), bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+template <typename A> __device__ __forceinline__ A carry_get(A *p) {
+  typedef typename CarryBits<A>::type U;
+  const U bits = __hip_atomic_fetch_or(reinterpret_cast<U *>(p), (U)0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  A v;
+  __builtin_memcpy(&v, &bits, sizeof(A));
+  return v;
+}
 
 template <typename A, int REDUCE>
 __device__ __forceinline__ void reduce_step(A &acc, int32_t &arg, A v, int32_t e) {
@@ -287,14 +325,70 @@ __global__ __launch_bounds__(kBlock, (csr_reduce_min_blocks<T, VEC, REDUCE>())) 
       }
     }
   }
+  constexpr bool kCarryOk = sizeof(A) >= 4;  // carries move through 32- and 64-bit atomics
+  const bool lookback = kCarryOk && a.lookback != 0;
   // default: the tile leaves no open row; the worker that does overwrites this after the barrier
-  if (tid == 0 && blockIdx.y == 0) a.ws_meta[(b * a.nblk + blockIdx.x) * 4 + 2] = -1;
+  if (!lookback && tid == 0 && blockIdx.y == 0) a.ws_meta[(b * a.nblk + blockIdx.x) * 4 + 2] = -1;
   __syncthreads();
 
   // ---- combine partials of rows that cross worker boundaries, in edge order
   A *ws_val_blk = static_cast<A *>(a.ws_vals) + ((b * a.nblk + blockIdx.x) * 2) * a.K;
   int32_t *ws_arg_blk = kArg ? a.ws_args + ((b * a.nblk + blockIdx.x) * 2) * a.K : nullptr;
   int64_t *meta = a.ws_meta + (b * a.nblk + blockIdx.x) * 4;
+
+  // look-back mode: this tile's carry slot is the second of its two partial slots
+  uint64_t *carry_flags = reinterpret_cast<uint64_t *>(a.ws_meta) + (b * a.nblk) * 4 + blockIdx.y;
+  auto publish_carry = [&](uint64_t kind) {
+    if constexpr (kCarryOk) {
+    uint64_t sink = 0;
+    if (col_ok) {
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) {
+        sink |= carry_put<A>(ws_val_blk + a.K + col + v, acc[v]);
+        if (kArg) sink |= carry_put<int32_t>(ws_arg_blk + a.K + col + v, arg[v]);
+      }
+    }
+    asm volatile("" ::"v"(sink) : "memory");  // the returns are in: the carry is in memory
+    if (lg == 0)
+      __hip_atomic_exchange(carry_flags + (int64_t)blockIdx.x * 4, (a.nonce << 2) | kind, __ATOMIC_RELAXED,
+                            __HIP_MEMORY_SCOPE_AGENT);
+    }
+  };
+  // acc / arg hold the last part of a row that began in an earlier tile: put the carries of the tiles before in front
+  auto walk_back = [&]() {
+    if constexpr (kCarryOk) {
+    A *vals_b = static_cast<A *>(a.ws_vals) + (b * a.nblk) * 2 * a.K;
+    int32_t *args_b = kArg ? a.ws_args + (b * a.nblk) * 2 * a.K : nullptr;
+    const int64_t c = col_ok ? col : 0;
+    for (int64_t tt = (int64_t)blockIdx.x - 1; tt >= 0; --tt) {
+      uint64_t *flag = carry_flags + tt * 4;
+      uint64_t f = 0;
+      int spin = kCarrySpin;
+      while (true) {
+        f = __hip_atomic_fetch_or(flag, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if ((f >> 2) == a.nonce || --spin <= 0) break;
+        __builtin_amdgcn_s_sleep(4);
+      }
+      if ((f >> 2) != a.nonce) return;  // indptr not monotone: no tile will ever publish this
+      asm volatile("" ::: "memory");
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) {
+        A early = carry_get<A>(vals_b + (tt * 2 + 1) * a.K + c + v);
+        if (kArg) {
+          int32_t early_arg = carry_get<int32_t>(args_b + (tt * 2 + 1) * a.K + c + v);
+          reduce_step<A, REDUCE>(early, early_arg, acc[v], arg[v]);  // earlier entries win ties
+          arg[v] = early_arg;
+          acc[v] = early;
+        } else {
+          acc[v] = early + acc[v];
+        }
+      }
+      asm volatile("" ::: "memory");
+      if (lg == 0) __hip_atomic_exchange(flag, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // consumed
+      if ((f & 3) == kCarryTail) return;
+    }
+    }
+  };
 
   auto absorb_head = [&](int ww) {
     const A *hv = s_val + (size_t)ww * CW + lg * VEC;
@@ -322,6 +416,8 @@ __global__ __launch_bounds__(kBlock, (csr_reduce_min_blocks<T, VEC, REDUCE>())) 
     if (closed) {
       finalize_row<T, VEC, REDUCE, ACCUM>(a, out_b, arg_b, count_b, i0 + row, col, lg, acc, arg,
                                    (int64_t)s_ptr[row + 1] - (int64_t)s_ptr[row], col_ok);
+    } else if (lookback) {
+      publish_carry(kCarryTail);
     } else {
       if (col_ok) {
 #pragma unroll
@@ -347,6 +443,17 @@ __global__ __launch_bounds__(kBlock, (csr_reduce_min_blocks<T, VEC, REDUCE>())) 
         absorb_head(ww);
         closed = s_head_closes[ww] != 0;
       }
+      if (lookback) {
+        if (closed) {
+          walk_back();
+          const int row = s_head_row[0];
+          finalize_row<T, VEC, REDUCE, ACCUM>(a, out_b, arg_b, count_b, i0 + row, col, lg, acc, arg,
+                                              (int64_t)s_ptr[row + 1] - (int64_t)s_ptr[row], col_ok);
+        } else {
+          publish_carry(kCarryPass);
+        }
+        return;
+      }
       if (col_ok) {
 #pragma unroll
         for (int v = 0; v < VEC; ++v) {
@@ -355,7 +462,7 @@ __global__ __launch_bounds__(kBlock, (csr_reduce_min_blocks<T, VEC, REDUCE>())) 
         }
       }
       if (lg == 0 && blockIdx.y == 0) { meta[0] = i0 + s_head_row[0]; meta[1] = closed ? 1 : 0; }
-    } else if (lg == 0 && blockIdx.y == 0) {
+    } else if (!lookback && lg == 0 && blockIdx.y == 0) {
       meta[0] = -1;
       meta[1] = 0;
     }
@@ -526,7 +633,7 @@ int launch_csr_reduce_t(const CsrReduceArgs &a, const CsrPlan &p, int64_t B, hip
     hipLaunchKernelGGL((csr_reduce_kernel<T, VEC, REDUCE, -1>), grid, dim3(kBlock), 0, stream, a);
   else
     hipLaunchKernelGGL((csr_reduce_kernel<T, VEC, REDUCE, 0>), grid, dim3(kBlock), 0, stream, a);
-  if (p.nblk > 1) {  // a single tile has no rows that cross tiles
+  if (p.nblk > 1 && !a.lookback) {  // a single tile has no rows that cross tiles
     const int W = kBlock / p.G;
     dim3 grid2((unsigned)((p.nblk + W - 1) / W), (unsigned)p.ychunks, (unsigned)B);
     hipLaunchKernelGGL((csr_reduce_fixup_kernel<T, VEC, REDUCE>), grid2, dim3(kBlock), 0, stream, a);
