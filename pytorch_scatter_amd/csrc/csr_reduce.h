@@ -354,38 +354,71 @@ __global__ __launch_bounds__(kBlock, (csr_reduce_min_blocks<T, VEC, REDUCE>())) 
                             __HIP_MEMORY_SCOPE_AGENT);
     }
   };
-  // acc / arg hold the last part of a row that began in an earlier tile: put the carries of the tiles before in front
-  auto walk_back = [&]() {
+  // acc / arg hold the last part of a row that began in an earlier tile: put the carries of the tiles before
+  // in front. first_tile is the tile in which the row began (from its row pointer), so the tiles to visit
+  // are known in advance and are polled and read several at a time: a hub row that passes through hundreds
+  // of tiles costs a few memory round trips per batch, not per tile.
+  auto walk_back = [&](int64_t first_tile) {
     if constexpr (kCarryOk) {
+    constexpr int PF = VEC <= 4 ? 4 : 2;
     A *vals_b = static_cast<A *>(a.ws_vals) + (b * a.nblk) * 2 * a.K;
     int32_t *args_b = kArg ? a.ws_args + (b * a.nblk) * 2 * a.K : nullptr;
     const int64_t c = col_ok ? col : 0;
-    for (int64_t tt = (int64_t)blockIdx.x - 1; tt >= 0; --tt) {
-      uint64_t *flag = carry_flags + tt * 4;
-      uint64_t f = 0;
+    if (first_tile < 0) first_tile = 0;
+    for (int64_t hi = (int64_t)blockIdx.x - 1; hi >= first_tile; hi -= PF) {
+      const int n = hi - first_tile + 1 < PF ? (int)(hi - first_tile + 1) : PF;  // tiles hi, hi - 1, ...
+      bool ready[PF];
+#pragma unroll
+      for (int q = 0; q < PF; ++q) ready[q] = q >= n;
       int spin = kCarrySpin;
       while (true) {
-        f = __hip_atomic_fetch_or(flag, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if ((f >> 2) == a.nonce || --spin <= 0) break;
+        uint64_t f[PF];
+#pragma unroll
+        for (int q = 0; q < PF; ++q)
+          f[q] = ready[q] ? 0 : __hip_atomic_fetch_or(carry_flags + (hi - q) * 4, 0ull, __ATOMIC_RELAXED,
+                                                       __HIP_MEMORY_SCOPE_AGENT);
+        bool all = true;
+#pragma unroll
+        for (int q = 0; q < PF; ++q) {
+          ready[q] = ready[q] || (f[q] >> 2) == a.nonce;
+          all = all && ready[q];
+        }
+        if (all || --spin <= 0) break;
         __builtin_amdgcn_s_sleep(4);
       }
-      if ((f >> 2) != a.nonce) return;  // indptr not monotone: no tile will ever publish this
+      if (spin <= 0) return;  // indptr not monotone: these carries will never be published
       asm volatile("" ::: "memory");
+      A early[PF][VEC];
+      int32_t early_arg[PF][VEC];
 #pragma unroll
-      for (int v = 0; v < VEC; ++v) {
-        A early = carry_get<A>(vals_b + (tt * 2 + 1) * a.K + c + v);
-        if (kArg) {
-          int32_t early_arg = carry_get<int32_t>(args_b + (tt * 2 + 1) * a.K + c + v);
-          reduce_step<A, REDUCE>(early, early_arg, acc[v], arg[v]);  // earlier entries win ties
-          arg[v] = early_arg;
-          acc[v] = early;
-        } else {
-          acc[v] = early + acc[v];
+      for (int q = 0; q < PF; ++q) {
+        if (q >= n) break;
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) {
+          early[q][v] = carry_get<A>(vals_b + ((hi - q) * 2 + 1) * a.K + c + v);
+          if (kArg) early_arg[q][v] = carry_get<int32_t>(args_b + ((hi - q) * 2 + 1) * a.K + c + v);
+        }
+      }
+#pragma unroll
+      for (int q = 0; q < PF; ++q) {
+        if (q >= n) break;
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) {
+          if (kArg) {
+            reduce_step<A, REDUCE>(early[q][v], early_arg[q][v], acc[v], arg[v]);  // earlier entries win ties
+            arg[v] = early_arg[q][v];
+            acc[v] = early[q][v];
+          } else {
+            acc[v] = early[q][v] + acc[v];
+          }
         }
       }
       asm volatile("" ::: "memory");
-      if (lg == 0) __hip_atomic_exchange(flag, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // consumed
-      if ((f & 3) == kCarryTail) return;
+      if (lg == 0) {
+#pragma unroll
+        for (int q = 0; q < PF; ++q)
+          if (q < n) __hip_atomic_exchange(carry_flags + (hi - q) * 4, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
     }
     }
   };
@@ -445,8 +478,9 @@ __global__ __launch_bounds__(kBlock, (csr_reduce_min_blocks<T, VEC, REDUCE>())) 
       }
       if (lookback) {
         if (closed) {
-          walk_back();
           const int row = s_head_row[0];
+          // the row's first entry sits at merge position (row index + row pointer)
+          walk_back(((i0 + row) + ((int64_t)s_ptr[row] + j0)) / a.BI);
           finalize_row<T, VEC, REDUCE, ACCUM>(a, out_b, arg_b, count_b, i0 + row, col, lg, acc, arg,
                                               (int64_t)s_ptr[row + 1] - (int64_t)s_ptr[row], col_ok);
         } else {
@@ -506,17 +540,8 @@ __global__ __launch_bounds__(kBlock) void csr_reduce_fixup_kernel(CsrReduceArgs 
     ha[v] = kArg ? args[(tn * 2) * a.K + c + v] : 0;
   }
   if (row < 0) return;
-  for (int64_t tt = t + 1; tt < a.nblk; ++tt) {
-    if (tt > t + 1) {
-      next_row = meta[tt * 4 + 0];
-      next_closes = meta[tt * 4 + 1];
-#pragma unroll
-      for (int v = 0; v < VEC; ++v) {
-        hv[v] = vals[(tt * 2) * a.K + c + v];
-        ha[v] = kArg ? args[(tt * 2) * a.K + c + v] : 0;
-      }
-    }
-    if (next_row != row) break;  // cannot happen for a well-formed indptr
+  bool done = next_row != row;  // cannot happen for a well-formed indptr
+  if (!done) {
 #pragma unroll
     for (int v = 0; v < VEC; ++v) {
       if (kArg)
@@ -524,7 +549,40 @@ __global__ __launch_bounds__(kBlock) void csr_reduce_fixup_kernel(CsrReduceArgs 
       else
         acc[v] = acc[v] + hv[v];
     }
-    if (next_closes != 0) break;
+    done = next_closes != 0;
+  }
+  // A hub row passes through many tiles. Their partials are fetched several tiles at a time (the
+  // loads do not depend on each other) and combined in tile order, so the walk costs one memory
+  // latency per batch instead of one per tile.
+  constexpr int PF = VEC == 1 ? 16 : (VEC <= 4 ? 8 : (VEC <= 8 ? 4 : 2));
+  for (int64_t t0 = t + 2; !done && t0 < a.nblk; t0 += PF) {
+    int64_t nrow[PF], ncl[PF];
+    A bv[PF][VEC];
+    int32_t ba[PF][VEC];
+#pragma unroll
+    for (int q = 0; q < PF; ++q) {
+      const int64_t tt = t0 + q < a.nblk ? t0 + q : a.nblk - 1;
+      nrow[q] = meta[tt * 4 + 0];
+      ncl[q] = meta[tt * 4 + 1];
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) {
+        bv[q][v] = vals[(tt * 2) * a.K + c + v];
+        ba[q][v] = kArg ? args[(tt * 2) * a.K + c + v] : 0;
+      }
+    }
+#pragma unroll
+    for (int q = 0; q < PF; ++q) {
+      if (done) break;
+      if (t0 + q >= a.nblk || nrow[q] != row) { done = true; break; }
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) {
+        if (kArg)
+          reduce_step<A, REDUCE>(acc[v], arg[v], bv[q][v], ba[q][v]);
+        else
+          acc[v] = acc[v] + bv[q][v];
+      }
+      done = ncl[q] != 0;
+    }
   }
   T *out_b = static_cast<T *>(a.out) + b * a.N * a.K;
   int64_t *arg_b = kArg ? a.arg_out + b * a.N * a.K : nullptr;

@@ -162,10 +162,105 @@ __global__ __launch_bounds__(kBlock) void csr_reduce_small_kernel(CsrReduceArgs 
     int64_t *meta = a.ws_meta + (b * a.nblk + blockIdx.x) * 4;
     int lo, hi;
     const bool tail = has_open_row && classify(nr, lo, hi) == kTail;
-    meta[0] = head_exists ? i0 : -1;
-    meta[1] = head_exists && nr > 0 ? 1 : 0;  // the head row ends inside this tile
     meta[2] = tail ? i0 + nr : -1;
-    if (tail) meta[3] = (int64_t)s_ptr[nr + 1] - (int64_t)s_ptr[nr];  // full length of the open row
+    if (tail) {
+      meta[3] = (int64_t)s_ptr[nr + 1] - (int64_t)s_ptr[nr];  // full length of the open row
+      // the tile in which it ends: its row-end item sits at merge position row + indptr[row + 1]
+      meta[0] = ((i0 + nr) + ((int64_t)s_ptr[nr + 1] + j0)) / a.BI;
+    }
+  }
+}
+
+// Second kernel of the narrow-row reduction: rows that cross tiles. A group of G lanes (one lane per
+// column, 64 / G groups per wavefront) serves one tile that opened such a row; nearly always the row
+// ends in the next tile and everything that needs is requested at once. A hub row, however, passes
+// through hundreds of these small tiles. Its chain is not walked by one group: the tile in which the
+// row ends is known (the first kernel derives it from the row pointer), so the wavefront's groups take
+// every (64 / G)-th tile of the chain, several loads in flight each, and a shuffle tree combines them.
+// The order of the combination is fixed by the tiling (for min / max ties go to the smaller
+// position), so the result does not depend on timing.
+template <typename T, int REDUCE>
+__global__ __launch_bounds__(kBlock) void csr_reduce_fixup_wave_kernel(CsrReduceArgs a) {
+  typedef typename Acc<T>::type A;
+  constexpr bool kArg = (REDUCE == TS_MIN || REDUCE == TS_MAX);
+  constexpr int PF = 8;
+  const int G = a.G;  // power of two, at most 16
+  const int S = kWave / G;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int j = lane / G;
+  const int lg = lane - j * G;
+  const bool col_ok = lg < a.K;
+  const int64_t c = col_ok ? lg : 0;
+  const int64_t b = blockIdx.z;
+  const int64_t wave = (int64_t)blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave;
+  const int64_t t = wave * S + j;
+  const bool valid = t < a.nblk;
+  const int64_t tc = valid ? t : a.nblk - 1;
+  const int64_t *meta = a.ws_meta + (b * a.nblk) * 4;
+  const A *vals = static_cast<const A *>(a.ws_vals) + (b * a.nblk) * 2 * a.K;
+  const int32_t *args = kArg ? a.ws_args + (b * a.nblk) * 2 * a.K : nullptr;
+
+  auto absorb = [&](A &x, int32_t &xa, A y, int32_t ya) {
+    if (kArg) {
+      const bool better = (REDUCE == TS_MIN ? y < x : y > x) || (y == x && ya < xa);
+      if (better) { x = y; xa = ya; }
+    } else {
+      x = x + y;
+    }
+  };
+
+  // everything the usual case needs is requested at once
+  const int64_t row = meta[tc * 4 + 2];
+  const int64_t count = meta[tc * 4 + 3];
+  int64_t last = meta[tc * 4 + 0];  // the tile in which the row ends, left by the tile that opened it
+  const int64_t tn = tc + 1 < a.nblk ? tc + 1 : tc;
+  A acc = vals[(tc * 2 + 1) * a.K + c];
+  int32_t arg = kArg ? args[(tc * 2 + 1) * a.K + c] : 0;
+  const A next_val = vals[(tn * 2) * a.K + c];
+  const int32_t next_arg = kArg ? args[(tn * 2) * a.K + c] : 0;
+  const bool has = valid && row >= 0;
+  if (!has || last >= a.nblk) last = has ? a.nblk - 1 : tc;
+  if (has && last > t) absorb(acc, arg, next_val, next_arg);
+
+  // chains that go on beyond the next tile: the whole wavefront works on one at a time
+  uint64_t pending = __ballot(has && last > t + 1 && lg == 0);
+  while (pending != 0) {
+    const int leader = __ffsll((unsigned long long)pending) - 1;
+    pending &= pending - 1;
+    const int64_t t_s = __shfl(t, leader);
+    const int64_t last_s = __shfl(last, leader);
+    A part = acc_init<A, REDUCE>();
+    int32_t part_arg = 0x7FFFFFFF;
+    for (int64_t t0 = t_s + 2 + j; t0 <= last_s; t0 += (int64_t)S * PF) {
+      A hv[PF];
+      int32_t ha[PF];
+#pragma unroll
+      for (int q = 0; q < PF; ++q) {
+        const int64_t tt = t0 + (int64_t)q * S <= last_s ? t0 + (int64_t)q * S : last_s;
+        hv[q] = vals[(tt * 2) * a.K + c];
+        ha[q] = kArg ? args[(tt * 2) * a.K + c] : 0;
+      }
+#pragma unroll
+      for (int q = 0; q < PF; ++q) {
+        if (t0 + (int64_t)q * S > last_s) break;
+        absorb(part, part_arg, hv[q], ha[q]);
+      }
+    }
+    for (int off = S / 2; off >= 1; off >>= 1) {
+      const A o = __shfl_down(part, off * G);
+      const int32_t oa = __shfl_down(part_arg, off * G);
+      absorb(part, part_arg, o, oa);
+    }
+    // group 0 holds the chain's total: hand it to the group that owns the row
+    const A total = __shfl(part, lg);
+    const int32_t total_arg = __shfl(part_arg, lg);
+    if (j == leader / G) absorb(acc, arg, total, total_arg);
+  }
+  if (has) {
+    T *out_b = static_cast<T *>(a.out) + b * a.N * a.K;
+    int64_t *arg_b = kArg ? a.arg_out + b * a.N * a.K : nullptr;
+    T *count_b = a.count_out ? static_cast<T *>(a.count_out) + b * a.N : nullptr;
+    finalize_row<T, 1, REDUCE>(a, out_b, arg_b, count_b, row, lg, lg, &acc, &arg, count, col_ok);
   }
 }
 
@@ -175,9 +270,9 @@ int launch_csr_reduce_small_t(const CsrReduceArgs &a, const CsrPlan &p, int64_t 
   hipLaunchKernelGGL((csr_reduce_small_kernel<T, REDUCE>), grid, dim3(kBlock),
                      csr_small_lds_bytes(p.BI, a.K, (int)sizeof(T)), stream, a);
   if (p.nblk > 1) {  // a single tile has no rows that cross tiles
-    const int W = kBlock / p.G;
+    const int W = (kBlock / kWave) * (kWave / p.G);  // tiles per workgroup
     dim3 grid2((unsigned)((p.nblk + W - 1) / W), 1, (unsigned)B);
-    hipLaunchKernelGGL((csr_reduce_fixup_kernel<T, 1, REDUCE>), grid2, dim3(kBlock), 0, stream, a);
+    hipLaunchKernelGGL((csr_reduce_fixup_wave_kernel<T, REDUCE>), grid2, dim3(kBlock), 0, stream, a);
   }
   return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
 }

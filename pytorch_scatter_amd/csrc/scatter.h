@@ -1249,8 +1249,12 @@ int launch_scatter_v(const ScatterArgs &a, int reduce, hipStream_t stream) {
           // many entries per output slot: reduce in LDS first (see scatter_add_lds_kernel)
           int tn = 1;
           while ((int64_t)tn * 2 * a.K <= kLdsAcc && tn * 2 <= kLdsAccRows) tn *= 2;
+          // Rows of 32 and more columns do as well or better through the run kernel with its hot rows
+          // (measured, 10 M entries onto 100 k nodes: equal for an unsorted index, 4-5x faster for a sorted
+          // one such as the batch vector of a pooling layer, where the table's lanes collide on one address)
           const bool use_lds = a.lds_cache && a.sk == 0 && tn >= 64 && a.B * a.N < 0x7FFFFFFFll &&
-                               (a.lds_cache == 2 || (n_src >= ((int64_t)1 << 20) && n_edges >= 32 * a.B * a.N));
+                               (a.lds_cache == 2 ||
+                                (a.K < 32 && n_src >= ((int64_t)1 << 20) && n_edges >= 32 * a.B * a.N));
           if (use_lds) {
             const int64_t epb = per_cu_chunk_edges(a.lds_epb, n_edges, 16384 / a.K > 256 ? 16384 / a.K : 256,
                                                    131072 / a.K > 2048 ? 131072 / a.K : 2048);
