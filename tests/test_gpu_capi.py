@@ -68,6 +68,10 @@ def degrees(kind, rng, n):
         d[n // 2 + 1] = 700
     elif kind == "uniform":
         d = np.full(n, 7)
+    elif kind == "long":  # every row passes through dozens of tiles; two empty rows in between
+        d = rng.integers(20000, 40000, size=n)
+        d[n // 2] = 0
+        d[n // 2 + 1] = 0
     else:
         raise ValueError(kind)
     return d.astype(np.int64)
@@ -93,6 +97,7 @@ CSR_CASES = [
     ("short", 300, 1), ("short", 1000, 4), ("zipf", 2000, 16), ("zipf", 3000, 64),
     ("hub", 900, 64), ("hub", 500, 128), ("uniform", 257, 3), ("zipf", 700, 200),
     ("hub", 300, 520), ("short", 5, 8), ("hub", 40, 1),
+    ("long", 12, 8), ("long", 12, 64), ("long", 9, 1), ("hub", 120, 1100),
 ]
 
 
@@ -319,7 +324,7 @@ def test_gather_csr_and_mean_backward_narrow_rows(capi, oracle, case, dtype):
 
 
 @pytest.mark.parametrize("case,reduce,dtype", product(
-    CSR_CASES[:9], ["sum", "mean", "min", "max"], [torch.float32, torch.bfloat16]))
+    CSR_CASES[:9] + CSR_CASES[11:14], ["sum", "mean", "min", "max"], [torch.float32, torch.bfloat16]))
 def test_segment_coo(capi, oracle, case, reduce, dtype):
     kind, n, K = case
     rng, indptr, index = make_csr(kind, CSR_CASES.index(case), n)
