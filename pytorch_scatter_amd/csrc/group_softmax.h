@@ -141,7 +141,7 @@ __global__ __launch_bounds__(kBlock) void group_max_run_kernel(ScatterArgs a, Gr
   p.src = static_cast<const T *>(g.src);
   p.gmax = static_cast<A *>(g.gmax);
   p.K = g.K;
-  run_reduce_wave(a, lshift, rows_per_wave, p, s_stage[threadIdx.x / kWave]);
+  run_wave(a, lshift, rows_per_wave, p, s_stage[threadIdx.x / kWave]);
 }
 
 // the group maximum a row is shifted by. Softmax: a group in which nothing beat lowest() shifts by 0
@@ -222,7 +222,7 @@ __global__ __launch_bounds__(kBlock) void group_sum_run_kernel(ScatterArgs a, Gr
   p.gsum = static_cast<A *>(g.gsum);
   p.K = g.K;
   p.hot_init(s_hot, s_tags, hot_rlog, lshift + LogC<C>::value);
-  run_reduce_wave(a, lshift, rows_per_wave, p, s_stage[threadIdx.x / kWave]);
+  run_wave(a, lshift, rows_per_wave, p, s_stage[threadIdx.x / kWave]);
   p.hot.template flush<1>([&](int node, int j, const A *x) {
     if (p.colbase + j < p.K) p.to_memory(node, p.colbase + j, x);
   });

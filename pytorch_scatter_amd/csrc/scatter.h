@@ -448,6 +448,114 @@ __device__ __forceinline__ void run_reduce_wave(const ScatterArgs &a, const int 
   if (carry_node >= 0) write_slots(1ull, carry_node, carry);
 }
 
+// The same reduction for rows of 8 and more lanes (128 bytes and up per entry): with so few entries per
+// wavefront row the shuffles of the scheme above cost more than the loads. Here every entry slot of the
+// wavefront walks its OWN contiguous part of the wavefront's range, one entry per step, and keeps the
+// running value of its current run in registers: equal neighbours cost one add per column and no
+// cross-lane traffic at all; a run is written when the node id changes (through the same LDS transposition,
+// for all slots that changed in that step at once). Each slot reads 128 bytes or more of one entry per
+// load, so the memory system still sees whole lines. Runs cut at the border between two slots' parts cost
+// one extra atomic.
+template <typename P>
+__device__ __forceinline__ void run_serial_wave(const ScatterArgs &a, const int lshift, const int rows_per_wave,
+                                                P &p, typename P::A *stage) {
+  typedef typename P::A A;
+  constexpr int U = P::U;
+  constexpr int C = P::C;
+  constexpr int EW = P::EW;
+  constexpr int cshift = C == 1 ? 0 : (C == 2 ? 1 : (C == 4 ? 2 : (C == 8 ? 3 : 4)));
+  const int lane = threadIdx.x & (kWave - 1);
+  const int L = 1 << lshift;
+  const int epr = kWave >> lshift;  // entry slots of the wavefront
+  const int el = lane >> lshift;
+  const int cl = lane & (L - 1);
+  const int64_t colbase = (int64_t)blockIdx.y * (L * C);
+  const int64_t col = colbase + cl * C;
+  const bool col_ok = col < a.K;
+  const int64_t n_edges = a.B * a.E;
+  const int64_t wave = (int64_t)blockIdx.x * (kBlock / kWave) + (threadIdx.x / kWave);
+  const int64_t lo = wave * rows_per_wave * epr;
+  int64_t hi = lo + (int64_t)rows_per_wave * epr;
+  if (hi > n_edges) hi = n_edges;
+  if (lo >= hi) return;
+  const int64_t s_lo = lo + (int64_t)el * rows_per_wave;  // this slot's part
+  const int64_t s_hi = s_lo + rows_per_wave < hi ? s_lo + rows_per_wave : hi;
+  const uint64_t slot_bits = L == kWave ? 1ull : ~0ull / ((1ull << L) - 1ull);
+
+  auto write_slots = [&](const uint64_t mask, const int n, const A *v) {
+    if constexpr (C == EW) {
+      if (((mask >> (el << lshift)) & 1ull) && col_ok) p.emit(n, col, v);
+      return;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+#pragma unroll
+    for (int c = 0; c < C; ++c) stage[lane * C + c] = v[c];
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int it = 0; it < C / EW; ++it) {
+      const int f = (lane + kWave * it) * EW;
+      const int slot = f >> (lshift + cshift);
+      const int j = f & ((L << cshift) - 1);
+      const int node = __shfl(n, slot << lshift);
+      if (((mask >> (slot << lshift)) & 1ull) && colbase + j < a.K) p.emit(node, colbase + j, stage + f);
+    }
+  };
+
+  A acc[C];
+#pragma unroll
+  for (int c = 0; c < C; ++c) acc[c] = p.identity();
+  int cur = -1;
+  for (int r0 = 0; r0 < rows_per_wave; r0 += U) {
+    int node[U];
+    A x[U][C];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int64_t e = s_lo + r0 + u;
+      const bool ok = e < s_hi;
+      const int64_t ec = ok ? e : hi - 1;
+      int64_t b, pos;
+      split_edge(ec, a.B, a.E, b, pos);
+      const int64_t idx = a.index[b * a.sb + pos * a.se];
+      node[u] = (ok && idx >= 0 && idx < a.N) ? (int)(b * a.N + idx) : -1;
+      p.load(ec, pos, col_ok ? col : 0, node[u], x[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (r0 + u >= rows_per_wave) break;  // uniform
+      const int n = node[u];
+      const bool change = n != cur;
+      p.begin_row(__popcll(__ballot(change) & slot_bits), epr);
+      const uint64_t em = __ballot(change && cur >= 0) & slot_bits;
+      if (em != 0) write_slots(em, cur, acc);
+      if (change) {
+        cur = n;
+#pragma unroll
+        for (int c = 0; c < C; ++c) acc[c] = x[u][c];
+      } else {
+#pragma unroll
+        for (int c = 0; c < C; ++c) p.combine(acc[c], x[u][c]);
+      }
+    }
+  }
+  // what is left in the slots are runs cut by the end of a part; for a hub they all belong to one node,
+  // so they go out like the entries of an unsorted index (table of hot rows, read before the atomic)
+  p.begin_row(epr, epr);
+  const uint64_t em = __ballot(cur >= 0) & slot_bits;
+  if (em != 0) write_slots(em, cur, acc);
+}
+
+// the scheme by row width: shuffles for narrow rows, one slot per part of the range from 8 lanes per entry
+constexpr int kSerialLshift = 3;
+template <typename P>
+__device__ __forceinline__ void run_wave(const ScatterArgs &a, const int lshift, const int rows_per_wave, P &p,
+                                         typename P::A *stage) {
+  if (lshift >= kSerialLshift)
+    run_serial_wave(a, lshift, rows_per_wave, p, stage);
+  else
+    run_reduce_wave(a, lshift, rows_per_wave, p, stage);
+}
+
 // ---- hot rows of a workgroup ------------------------------------------------------
 // An unsorted index with a hub (a node that owns 1 % or more of the entries, as in
 // power-law graphs) puts every entry of the hub on one address: about 10 ns per
@@ -632,7 +740,7 @@ __global__ __launch_bounds__(kBlock) void scatter_add_run_kernel(ScatterArgs a, 
   p.out_end = p.out + a.B * a.N * a.K;
   p.K = a.K;
   p.hot_init(s_hot, s_tags, hot_rlog, lshift + LogC<C>::value);
-  run_reduce_wave(a, lshift, rows_per_wave, p, s_stage[threadIdx.x / kWave]);
+  run_wave(a, lshift, rows_per_wave, p, s_stage[threadIdx.x / kWave]);
   p.hot.template flush<EW>([&](int node, int j, const A *x) {
     if (p.colbase + j < p.K) p.to_memory(node, p.colbase + j, x);
   });
@@ -668,7 +776,10 @@ inline RunGrid run_grid(int64_t n_edges, int64_t kc, int c = 0) {
     while ((1 << cshift) < c) ++cshift;
     g.hot_rlog = hot_rows_log(g.lshift + cshift);
   }
-  g.rpw = run_rows_per_wave(n_edges, epr, g.hot_rlog >= 0 ? 64 : 32);
+  // longer ranges where a workgroup should see a hub repeat, and where every slot walks its own part
+  g.rpw = run_rows_per_wave(n_edges, epr, g.lshift >= kSerialLshift || g.hot_rlog >= 0 ? 64 : 32);
+  // a slot only combines what lies inside its own part: keep the parts at 16 entries or more
+  if (g.lshift >= kSerialLshift && g.rpw < 16 && !getenv("TS_RUN_RPW")) g.rpw = 16;
   const int64_t waves = (n_edges + (int64_t)g.rpw * epr - 1) / ((int64_t)g.rpw * epr);
   const int64_t blocks = (waves + kBlock / kWave - 1) / (kBlock / kWave);
   const int64_t ychunks = (kc + L - 1) / L;
@@ -810,7 +921,7 @@ __global__ __launch_bounds__(kBlock) void scatter_key_run_kernel(ScatterArgs a, 
   p.keys = reinterpret_cast<uint64_t *>(a.arg_out);
   p.K = a.K;
   p.precheck = a.precheck;
-  run_reduce_wave(a, lshift, rows_per_wave, p, s_stage[threadIdx.x / kWave]);
+  run_wave(a, lshift, rows_per_wave, p, s_stage[threadIdx.x / kWave]);
 }
 
 // ---- packed-key min/max with a workgroup-private cache of hot slots ---------
