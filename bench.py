@@ -340,7 +340,7 @@ def main():
     # HBM bytes per launch of this kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, calibrated against
     # copies of known size (profiles/csr_reduce_pmc_traffic.txt): 117.5 MB read + 26.0 MB written
     traffic = 143.5e6
-    roofline = {"bound": "hbm", "kernel": "ts::csr_reduce_kernel<float, 4, SUM> (+ its fix-up launch)",
+    roofline = {"bound": "hbm", "kernel": "ts::csr_reduce_kernel<float, 4, SUM>",
                 "achieved": round(gbs(kernel_bytes, t_kernel), 1), "peak": PEAK_GBS, "unit": "GB/s",
                 "frac": round(gbs(kernel_bytes, t_kernel) / PEAK_GBS, 4), "traffic": traffic,
                 "algorithmic_bytes_per_launch": kernel_bytes, "us_per_launch": round(t_kernel * 1e6, 2)}

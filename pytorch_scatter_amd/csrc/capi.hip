@@ -354,9 +354,8 @@ int ts_scatter_count(const int64_t *index, float *count, int64_t B, int64_t E, i
                          s, a, kLdsAccRows - 1, epb);
     } else if (env_int("TS_SCATTER_RUNS", 1) && B * N < 0x7FFFFFFFll) {
       // runs of equal neighbouring indices (sorted input) are counted in the wavefront first
-      const RunGrid g = run_grid(B * E, 1, 1);
-      hipLaunchKernelGGL((scatter_add_run_kernel<float, 1>), dim3(g.blocks), dim3(kBlock), 0, s, a, 0, g.rpw,
-                         g.hot_rlog);
+      const RunGrid g = run_grid(B * E, 1, 1, 4);
+      launch_add_run<float, 1, 1>(a, g, s);
     } else {
       hipLaunchKernelGGL(scatter_count_kernel, dim3(grid_for(B * E)), dim3(kBlock), 0, s, index, count, B, E, N,
                          index_stride_b, index_stride_e);

@@ -392,24 +392,26 @@ __global__ __launch_bounds__(kBlock, (csr_reduce_min_blocks<T, VEC, REDUCE>())) 
       int32_t early_arg[PF][VEC];
 #pragma unroll
       for (int q = 0; q < PF; ++q) {
-        if (q >= n) break;
+        if (q < n) {
 #pragma unroll
-        for (int v = 0; v < VEC; ++v) {
-          early[q][v] = carry_get<A>(vals_b + ((hi - q) * 2 + 1) * a.K + c + v);
-          if (kArg) early_arg[q][v] = carry_get<int32_t>(args_b + ((hi - q) * 2 + 1) * a.K + c + v);
+          for (int v = 0; v < VEC; ++v) {
+            early[q][v] = carry_get<A>(vals_b + ((hi - q) * 2 + 1) * a.K + c + v);
+            if (kArg) early_arg[q][v] = carry_get<int32_t>(args_b + ((hi - q) * 2 + 1) * a.K + c + v);
+          }
         }
       }
 #pragma unroll
       for (int q = 0; q < PF; ++q) {
-        if (q >= n) break;
+        if (q < n) {
 #pragma unroll
-        for (int v = 0; v < VEC; ++v) {
-          if (kArg) {
-            reduce_step<A, REDUCE>(early[q][v], early_arg[q][v], acc[v], arg[v]);  // earlier entries win ties
-            arg[v] = early_arg[q][v];
-            acc[v] = early[q][v];
-          } else {
-            acc[v] = early[q][v] + acc[v];
+          for (int v = 0; v < VEC; ++v) {
+            if (kArg) {
+              reduce_step<A, REDUCE>(early[q][v], early_arg[q][v], acc[v], arg[v]);  // earlier entries win ties
+              arg[v] = early_arg[q][v];
+              acc[v] = early[q][v];
+            } else {
+              acc[v] = early[q][v] + acc[v];
+            }
           }
         }
       }
@@ -572,16 +574,20 @@ __global__ __launch_bounds__(kBlock) void csr_reduce_fixup_kernel(CsrReduceArgs 
     }
 #pragma unroll
     for (int q = 0; q < PF; ++q) {
-      if (done) break;
-      if (t0 + q >= a.nblk || nrow[q] != row) { done = true; break; }
+      if (!done) {
+        if (t0 + q >= a.nblk || nrow[q] != row) {
+          done = true;
+        } else {
 #pragma unroll
-      for (int v = 0; v < VEC; ++v) {
-        if (kArg)
-          reduce_step<A, REDUCE>(acc[v], arg[v], bv[q][v], ba[q][v]);
-        else
-          acc[v] = acc[v] + bv[q][v];
+          for (int v = 0; v < VEC; ++v) {
+            if (kArg)
+              reduce_step<A, REDUCE>(acc[v], arg[v], bv[q][v], ba[q][v]);
+            else
+              acc[v] = acc[v] + bv[q][v];
+          }
+          done = ncl[q] != 0;
+        }
       }
-      done = ncl[q] != 0;
     }
   }
   T *out_b = static_cast<T *>(a.out) + b * a.N * a.K;

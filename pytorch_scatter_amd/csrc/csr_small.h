@@ -242,8 +242,7 @@ __global__ __launch_bounds__(kBlock) void csr_reduce_fixup_wave_kernel(CsrReduce
       }
 #pragma unroll
       for (int q = 0; q < PF; ++q) {
-        if (t0 + (int64_t)q * S > last_s) break;
-        absorb(part, part_arg, hv[q], ha[q]);
+        if (t0 + (int64_t)q * S <= last_s) absorb(part, part_arg, hv[q], ha[q]);
       }
     }
     for (int off = S / 2; off >= 1; off >>= 1) {

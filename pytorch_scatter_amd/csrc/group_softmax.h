@@ -104,6 +104,7 @@ __global__ __launch_bounds__(kBlock) void group_init_kernel(GroupArgs g, int wit
 
 // ---- pass 1: group maxima as keys
 template <typename T, int C_> struct GroupMaxRun {
+  typedef T Elem;
   typedef typename Acc<T>::type F;
   typedef typename OrdKey<F>::bits A;
   static constexpr int C = C_;
@@ -132,7 +133,7 @@ template <typename T, int C_> struct GroupMaxRun {
   }
 };
 
-template <typename T, int C>
+template <typename T, int C, bool SERIAL>
 __global__ __launch_bounds__(kBlock) void group_max_run_kernel(ScatterArgs a, GroupArgs g, int lshift,
                                                                int rows_per_wave) {
   typedef typename GroupMaxRun<T, C>::A A;
@@ -141,7 +142,7 @@ __global__ __launch_bounds__(kBlock) void group_max_run_kernel(ScatterArgs a, Gr
   p.src = static_cast<const T *>(g.src);
   p.gmax = static_cast<A *>(g.gmax);
   p.K = g.K;
-  run_wave(a, lshift, rows_per_wave, p, s_stage[threadIdx.x / kWave]);
+  run_wave<SERIAL>(a, lshift, rows_per_wave, p, s_stage[threadIdx.x / kWave]);
 }
 
 // the group maximum a row is shifted by. Softmax: a group in which nothing beat lowest() shifts by 0
@@ -161,6 +162,7 @@ __device__ __forceinline__ void group_shift(const void *gmax, int64_t slot, type
 //   GS_SOFTMAX_BWD                y * g
 //   GS_LOG_SOFTMAX_BWD            g
 template <typename T, int C_, int MODE> struct GroupSumRun : HotState<typename Acc<T>::type> {
+  typedef T Elem;
   typedef typename Acc<T>::type A;
   static constexpr int C = C_;
   static constexpr int EW = 1;
@@ -208,7 +210,7 @@ template <typename T, int C_, int MODE> struct GroupSumRun : HotState<typename A
   }
 };
 
-template <typename T, int C, int MODE>
+template <typename T, int C, int MODE, bool SERIAL>
 __global__ __launch_bounds__(kBlock) void group_sum_run_kernel(ScatterArgs a, GroupArgs g, int lshift,
                                                                int rows_per_wave, int hot_rlog) {
   typedef typename Acc<T>::type A;
@@ -222,7 +224,7 @@ __global__ __launch_bounds__(kBlock) void group_sum_run_kernel(ScatterArgs a, Gr
   p.gsum = static_cast<A *>(g.gsum);
   p.K = g.K;
   p.hot_init(s_hot, s_tags, hot_rlog, lshift + LogC<C>::value);
-  run_wave(a, lshift, rows_per_wave, p, s_stage[threadIdx.x / kWave]);
+  run_wave<SERIAL>(a, lshift, rows_per_wave, p, s_stage[threadIdx.x / kWave]);
   p.hot.template flush<1>([&](int node, int j, const A *x) {
     if (p.colbase + j < p.K) p.to_memory(node, p.colbase + j, x);
   });
@@ -352,16 +354,17 @@ int launch_group_softmax_m(const GroupArgs &g, hipStream_t stream) {
   constexpr bool kForward = MODE == GS_SOFTMAX || MODE == GS_LOG_SOFTMAX;
   const int64_t n_edges = g.B * g.E;
   if (g.B * g.N >= 0x7FFFFFFFll) return TS_ERR_UNSUPPORTED;
-  const RunGrid rg = run_grid(n_edges, g.K / VEC, VEC);
+  const RunGrid rg = run_grid(n_edges, g.K / VEC, VEC, VEC * (int)sizeof(T));
   if (!rg.ok) return TS_ERR_UNSUPPORTED;
   const ScatterArgs a = group_index_args(g);
   const dim3 gd(rg.blocks, rg.ychunks);
   hipLaunchKernelGGL(group_init_kernel<T>, dim3(grid_for(g.B * g.N * g.K)), dim3(kBlock), 0, stream, g,
                      kForward ? 1 : 0);
   if (kForward)
-    hipLaunchKernelGGL((group_max_run_kernel<T, VEC>), gd, dim3(kBlock), 0, stream, a, g, rg.lshift, rg.rpw);
-  hipLaunchKernelGGL((group_sum_run_kernel<T, VEC, MODE>), gd, dim3(kBlock), 0, stream, a, g, rg.lshift, rg.rpw,
-                     rg.hot_rlog);
+    TS_LAUNCH_RUN(rg.serial, (group_max_run_kernel<T, VEC, true>), (group_max_run_kernel<T, VEC, false>), gd, stream, a, g,
+                  rg.lshift, rg.rpw);
+  TS_LAUNCH_RUN(rg.serial, (group_sum_run_kernel<T, VEC, MODE, true>), (group_sum_run_kernel<T, VEC, MODE, false>), gd,
+                stream, a, g, rg.lshift, rg.rpw, rg.hot_rlog);
   hipLaunchKernelGGL((group_finish_kernel<T, VEC, MODE>), dim3(scatter_grid(n_edges, g.K / VEC, kBlock, 4)),
                      dim3(kBlock), 0, stream, g);
   return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
@@ -376,15 +379,16 @@ int launch_group_lse_v(const GroupArgs &g, bool backward, hipStream_t stream) {
                        dim3(kBlock), 0, stream, g);
     return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
   }
-  const RunGrid rg = run_grid(n_edges, g.K / VEC, VEC);
+  const RunGrid rg = run_grid(n_edges, g.K / VEC, VEC, VEC * (int)sizeof(T));
   if (!rg.ok) return TS_ERR_UNSUPPORTED;
   const ScatterArgs a = group_index_args(g);
   const dim3 gd(rg.blocks, rg.ychunks);
   const unsigned g_out = grid_for(g.B * g.N * g.K);
   hipLaunchKernelGGL(group_init_kernel<T>, dim3(g_out), dim3(kBlock), 0, stream, g, 1);
-  hipLaunchKernelGGL((group_max_run_kernel<T, VEC>), gd, dim3(kBlock), 0, stream, a, g, rg.lshift, rg.rpw);
-  hipLaunchKernelGGL((group_sum_run_kernel<T, VEC, GS_LSE>), gd, dim3(kBlock), 0, stream, a, g, rg.lshift, rg.rpw,
-                     rg.hot_rlog);
+  TS_LAUNCH_RUN(rg.serial, (group_max_run_kernel<T, VEC, true>), (group_max_run_kernel<T, VEC, false>), gd, stream, a, g,
+                rg.lshift, rg.rpw);
+  TS_LAUNCH_RUN(rg.serial, (group_sum_run_kernel<T, VEC, GS_LSE, true>), (group_sum_run_kernel<T, VEC, GS_LSE, false>), gd,
+                stream, a, g, rg.lshift, rg.rpw, rg.hot_rlog);
   hipLaunchKernelGGL(group_lse_finish_kernel<T>, dim3(g_out), dim3(kBlock), 0, stream, g);
   return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
 }

@@ -19,6 +19,13 @@
 // times). A last pass over [B, N, K] unpacks value and arg.
 // 64-bit element types use the reference's two-pass scheme with a
 // deterministic arg (atomic min over matching positions).
+//
+// With one index per row (the message-passing call) the kernels do not issue
+// one atomic per element: a wavefront combines runs of equal neighbouring
+// indices first (run_reduce_wave for narrow rows, run_serial_wave from 128
+// bytes per entry), sums keep the rows of hub nodes in a small LDS table per
+// workgroup (HotRows), and heavily contended inputs reduce into LDS tables of
+// accumulators or keys before they touch memory.
 #pragma once
 
 #include <limits>
@@ -545,12 +552,15 @@ __device__ __forceinline__ void run_serial_wave(const ScatterArgs &a, const int 
   if (em != 0) write_slots(em, cur, acc);
 }
 
-// the scheme by row width: shuffles for narrow rows, one slot per part of the range from 8 lanes per entry
-constexpr int kSerialLshift = 3;
-template <typename P>
+// the scheme by row width: shuffles for narrow rows, one slot per part of the range from 128 bytes per
+// entry (lane_bytes = bytes of src a lane loads per entry)
+__host__ __device__ inline bool run_is_serial(int lshift, int lane_bytes) { return (lane_bytes << lshift) >= 128; }
+// (a kernel holds one of the two: with both behind a run-time branch the small latency-bound launches
+// were 3 us slower, whichever branch they took)
+template <bool SERIAL, typename P>
 __device__ __forceinline__ void run_wave(const ScatterArgs &a, const int lshift, const int rows_per_wave, P &p,
                                          typename P::A *stage) {
-  if (lshift >= kSerialLshift)
+  if constexpr (SERIAL)
     run_serial_wave(a, lshift, rows_per_wave, p, stage);
   else
     run_reduce_wave(a, lshift, rows_per_wave, p, stage);
@@ -655,9 +665,10 @@ template <typename A> struct HotState {
 // with the packed-pair atomic. src == nullptr adds 1 per entry (the count of scatter mean).
 // EW_ = columns per atomic: a whole 32-bit word for element types below 32 bits, or 1 (rows whose
 // length or alignment rules that out; the element then goes through a compare-and-swap on its word)
-template <typename T, int C_, int EW_ = (sizeof(T) < 4 ? 4 / (int)sizeof(T) : 1)>
+template <typename T, int C_, int EW_ = (sizeof(T) < 4 ? 4 / (int)sizeof(T) : 1), bool HOT = true>
 struct AddRun : HotState<typename Acc<T>::type> {
   typedef typename Acc<T>::type A;
+  typedef T Elem;
   static constexpr int C = C_;
   static constexpr int EW = EW_;
   static constexpr int U = 4;
@@ -677,8 +688,13 @@ struct AddRun : HotState<typename Acc<T>::type> {
     for (int c = 0; c < C; ++c) x[c] = to_acc<T>(r.v[c]);
   }
   __device__ void combine(A &x, const A &y) const { x = x + y; }
+  __device__ void begin_row(int heads, int entries) {
+    if constexpr (HOT) HotState<A>::begin_row(heads, entries);
+  }
   __device__ void emit(int node, int64_t col, const A *x) {
-    if (this->template to_table<EW>(node, col, x)) return;
+    if constexpr (HOT) {
+      if (this->template to_table<EW>(node, col, x)) return;
+    }
     to_memory(node, col, x);
   }
   __device__ void to_memory(int node, int64_t col, const A *x) const {
@@ -727,24 +743,30 @@ struct AddRun : HotState<typename Acc<T>::type> {
 
 template <int C> struct LogC { static constexpr int value = C == 1 ? 0 : (C == 2 ? 1 : (C == 4 ? 2 : (C == 8 ? 3 : 4))); };
 
-template <typename T, int C, int EW = (sizeof(T) < 4 ? 4 / (int)sizeof(T) : 1)>
+// HOT = false: the variant for inputs too small for the table to pay (its code and LDS cost a
+// latency-bound launch about a microsecond even when it is switched off at run time)
+template <typename T, int C, int EW, bool SERIAL, bool HOT>
 __global__ __launch_bounds__(kBlock) void scatter_add_run_kernel(ScatterArgs a, int lshift, int rows_per_wave,
                                                                  int hot_rlog) {
   typedef typename Acc<T>::type A;
+  constexpr bool kTable = HOT && HotOk<A>::value;
   __shared__ A s_stage[kBlock / kWave][kWave * C];
-  __shared__ A s_hot[HotOk<A>::value ? kHotAcc : 1];
-  __shared__ uint32_t s_tags[HotOk<A>::value ? kHotRowsMax : 1];
-  AddRun<T, C, EW> p;
+  __shared__ A s_hot[kTable ? kHotAcc : 1];
+  __shared__ uint32_t s_tags[kTable ? kHotRowsMax : 1];
+  AddRun<T, C, EW, kTable> p;
   p.src = static_cast<const T *>(a.src);
   p.out = static_cast<T *>(a.out);
   p.out_end = p.out + a.B * a.N * a.K;
   p.K = a.K;
-  p.hot_init(s_hot, s_tags, hot_rlog, lshift + LogC<C>::value);
-  run_wave(a, lshift, rows_per_wave, p, s_stage[threadIdx.x / kWave]);
-  p.hot.template flush<EW>([&](int node, int j, const A *x) {
-    if (p.colbase + j < p.K) p.to_memory(node, p.colbase + j, x);
-  });
+  if constexpr (kTable) p.hot_init(s_hot, s_tags, hot_rlog, lshift + LogC<C>::value);
+  run_wave<SERIAL>(a, lshift, rows_per_wave, p, s_stage[threadIdx.x / kWave]);
+  if constexpr (kTable) {
+    p.hot.template flush<EW>([&](int node, int j, const A *x) {
+      if (p.colbase + j < p.K) p.to_memory(node, p.colbase + j, x);
+    });
+  }
 }
+
 
 // rows of a wavefront in the kernel above: long enough to carry runs across rows, short enough to
 // leave ~8 K wavefronts
@@ -762,10 +784,30 @@ struct RunGrid {
   unsigned blocks, ychunks;
   bool ok;
   int hot_rlog;  // log2 of the rows of the hot-row table, -1: none
+  bool serial;   // run_serial_wave instead of run_reduce_wave
 };
+// launches the SERIAL = true or false instantiation of a run kernel named by the macro arguments
+#define TS_LAUNCH_RUN(SERIAL_FLAG, KERNEL_T, KERNEL_F, GRID, STREAM, ...)                      \
+  do {                                                                                         \
+    if (SERIAL_FLAG)                                                                           \
+      hipLaunchKernelGGL(KERNEL_T, GRID, dim3(kBlock), 0, STREAM, __VA_ARGS__);                \
+    else                                                                                       \
+      hipLaunchKernelGGL(KERNEL_F, GRID, dim3(kBlock), 0, STREAM, __VA_ARGS__);                \
+  } while (0)
 // c > 0: a sum kernel with c columns per lane that may keep a hot-row table. The table pays once a
 // workgroup sees enough entries for a hub to repeat: large inputs, with longer ranges per wavefront.
-inline RunGrid run_grid(int64_t n_edges, int64_t kc, int c = 0) {
+// launches the instantiation of scatter_add_run_kernel for (serial, hot)
+template <typename T, int C, int EW>
+void launch_add_run(const ScatterArgs &a, const RunGrid &g, hipStream_t stream) {
+  const dim3 gd(g.blocks, g.ychunks);
+  if (g.hot_rlog >= 0)
+    TS_LAUNCH_RUN(g.serial, (scatter_add_run_kernel<T, C, EW, true, true>), (scatter_add_run_kernel<T, C, EW, false, true>),
+                  gd, stream, a, g.lshift, g.rpw, g.hot_rlog);
+  else
+    TS_LAUNCH_RUN(g.serial, (scatter_add_run_kernel<T, C, EW, true, false>),
+                  (scatter_add_run_kernel<T, C, EW, false, false>), gd, stream, a, g.lshift, g.rpw, g.hot_rlog);
+}
+inline RunGrid run_grid(int64_t n_edges, int64_t kc, int c, int lane_bytes) {
   RunGrid g;
   g.lshift = 0;
   while ((1 << g.lshift) < kc && g.lshift < 6) ++g.lshift;
@@ -777,9 +819,11 @@ inline RunGrid run_grid(int64_t n_edges, int64_t kc, int c = 0) {
     g.hot_rlog = hot_rows_log(g.lshift + cshift);
   }
   // longer ranges where a workgroup should see a hub repeat, and where every slot walks its own part
-  g.rpw = run_rows_per_wave(n_edges, epr, g.lshift >= kSerialLshift || g.hot_rlog >= 0 ? 64 : 32);
+  const bool serial = run_is_serial(g.lshift, lane_bytes);
+  g.serial = serial;
+  g.rpw = run_rows_per_wave(n_edges, epr, serial || g.hot_rlog >= 0 ? 64 : 32);
   // a slot only combines what lies inside its own part: keep the parts at 16 entries or more
-  if (g.lshift >= kSerialLshift && g.rpw < 16 && !getenv("TS_RUN_RPW")) g.rpw = 16;
+  if (serial && g.rpw < 16 && !getenv("TS_RUN_RPW")) g.rpw = 16;
   const int64_t waves = (n_edges + (int64_t)g.rpw * epr - 1) / ((int64_t)g.rpw * epr);
   const int64_t blocks = (waves + kBlock / kWave - 1) / (kBlock / kWave);
   const int64_t ychunks = (kc + L - 1) / L;
@@ -889,6 +933,7 @@ __global__ __launch_bounds__(kBlock) void scatter_key_kernel(ScatterArgs a) {
 template <typename T, int C_, bool IS_MAX>
 struct KeyRun {
   typedef uint64_t A;
+  typedef T Elem;
   static constexpr int C = C_;
   static constexpr int EW = 1;
   static constexpr int U = 4;
@@ -913,7 +958,7 @@ struct KeyRun {
   }
 };
 
-template <typename T, int C, bool IS_MAX>
+template <typename T, int C, bool IS_MAX, bool SERIAL>
 __global__ __launch_bounds__(kBlock) void scatter_key_run_kernel(ScatterArgs a, int lshift, int rows_per_wave) {
   __shared__ uint64_t s_stage[kBlock / kWave][kWave * C];
   KeyRun<T, C, IS_MAX> p;
@@ -921,7 +966,7 @@ __global__ __launch_bounds__(kBlock) void scatter_key_run_kernel(ScatterArgs a, 
   p.keys = reinterpret_cast<uint64_t *>(a.arg_out);
   p.K = a.K;
   p.precheck = a.precheck;
-  run_wave(a, lshift, rows_per_wave, p, s_stage[threadIdx.x / kWave]);
+  run_wave<SERIAL>(a, lshift, rows_per_wave, p, s_stage[threadIdx.x / kWave]);
 }
 
 // ---- packed-key min/max with a workgroup-private cache of hot slots ---------
@@ -1322,7 +1367,9 @@ inline int64_t lds_chunk_edges(int64_t forced, int64_t K, int64_t n_edges) {
 inline int64_t per_cu_chunk_edges(int64_t forced, int64_t n_edges, int64_t min_epb, int64_t max_epb) {
   if (forced > 0) return forced;
   int dev = 0, cus = 256;
-  if (hipGetDevice(&dev) == hipSuccess) hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+  if (hipGetDevice(&dev) == hipSuccess &&
+      hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
+    cus = 0;
   if (cus < 1) cus = 256;
   const int64_t rounds = (n_edges + (int64_t)cus * max_epb - 1) / ((int64_t)cus * max_epb);
   const int64_t epb = (n_edges + cus * rounds - 1) / (cus * rounds);
@@ -1382,10 +1429,9 @@ int launch_scatter_v(const ScatterArgs &a, int reduce, hipStream_t stream) {
                                            (reinterpret_cast<uintptr_t>(a.src) & 3) == 0);
           if (a.run_reduce && a.sk == 0 && a.B * a.N < 0x7FFFFFFFll && !word_ok) {
             // rows that cannot be written word by word: one column per lane and atomic
-            const RunGrid g = run_grid(n_edges, a.K, 1);
+            const RunGrid g = run_grid(n_edges, a.K, 1, (int)sizeof(T));
             if (g.ok) {
-              hipLaunchKernelGGL((scatter_add_run_kernel<T, 1, 1>), dim3(g.blocks, g.ychunks), dim3(kBlock), 0, stream, a,
-                                 g.lshift, g.rpw, g.hot_rlog);
+              launch_add_run<T, 1, 1>(a, g, stream);
               return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
             }
           }
@@ -1394,14 +1440,13 @@ int launch_scatter_v(const ScatterArgs &a, int reduce, hipStream_t stream) {
             // 16-byte loads pay once the instruction rate limits the stream; small inputs are bound by
             // latency and do better with one atomic per lane straight from registers
             const bool wide = C > CN && n_src * (int64_t)sizeof(T) > ((int64_t)32 << 20);
-            const RunGrid g = run_grid(n_edges, a.K / (wide ? C : CN), wide ? C : CN);
+            const RunGrid g = run_grid(n_edges, a.K / (wide ? C : CN), wide ? C : CN, (wide ? C : CN) * (int)sizeof(T));
             if (g.ok) {
+              constexpr int EWD = sizeof(T) < 4 ? 4 / (int)sizeof(T) : 1;  // a whole 32-bit word per atomic
               if (wide)
-                hipLaunchKernelGGL((scatter_add_run_kernel<T, C>), dim3(g.blocks, g.ychunks), dim3(kBlock), 0, stream,
-                                   a, g.lshift, g.rpw, g.hot_rlog);
+                launch_add_run<T, C, EWD>(a, g, stream);
               else
-                hipLaunchKernelGGL((scatter_add_run_kernel<T, CN>), dim3(g.blocks, g.ychunks), dim3(kBlock), 0, stream,
-                                   a, g.lshift, g.rpw, g.hot_rlog);
+                launch_add_run<T, CN, EWD>(a, g, stream);
               return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
             }
           }
@@ -1455,16 +1500,18 @@ int launch_scatter_v(const ScatterArgs &a, int reduce, hipStream_t stream) {
       // wavefront before going to the table (a sorted index then costs one atomic per slot)
       if (!use_lds && a.run_reduce && a.sk == 0 && a.B * a.N < 0x7FFFFFFFll && n_src > 0) {
         constexpr int KC = VEC > 4 ? 4 : VEC;  // columns per lane: 64-bit keys, so at most four
-        const RunGrid g = run_grid(n_edges, a.K / KC);
+        const RunGrid g = run_grid(n_edges, a.K / KC, 0, KC * (int)sizeof(T));
         if (g.ok) {
           const dim3 gd(g.blocks, g.ychunks);
           if (is_max) {
             hipLaunchKernelGGL((scatter_key_init_kernel<T, true>), dim3(g_out), dim3(kBlock), 0, stream, a);
-            hipLaunchKernelGGL((scatter_key_run_kernel<T, KC, true>), gd, dim3(kBlock), 0, stream, a, g.lshift, g.rpw);
+            TS_LAUNCH_RUN(g.serial, (scatter_key_run_kernel<T, KC, true, true>), (scatter_key_run_kernel<T, KC, true, false>),
+                          gd, stream, a, g.lshift, g.rpw);
             hipLaunchKernelGGL((scatter_key_final_kernel<T, true>), dim3(g_out), dim3(kBlock), 0, stream, a);
           } else {
             hipLaunchKernelGGL((scatter_key_init_kernel<T, false>), dim3(g_out), dim3(kBlock), 0, stream, a);
-            hipLaunchKernelGGL((scatter_key_run_kernel<T, KC, false>), gd, dim3(kBlock), 0, stream, a, g.lshift, g.rpw);
+            TS_LAUNCH_RUN(g.serial, (scatter_key_run_kernel<T, KC, false, true>),
+                          (scatter_key_run_kernel<T, KC, false, false>), gd, stream, a, g.lshift, g.rpw);
             hipLaunchKernelGGL((scatter_key_final_kernel<T, false>), dim3(g_out), dim3(kBlock), 0, stream, a);
           }
           return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
