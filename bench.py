@@ -338,8 +338,8 @@ def main():
         t_kernel = event_time(lambda: ts.segment_csr(src, indptr, out, "sum"), max(args.steps, 20))
     kernel_bytes = wl.bytes_segment(w2.E, w2.N, w2.K, 4)
     # HBM bytes per launch of this kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, calibrated against
-    # copies of known size (profiles/csr_reduce_pmc_traffic.txt): 117.5 MB read + 26.0 MB written
-    traffic = 143.5e6
+    # copies of known size (profiles/csr_reduce_pmc_traffic.txt): 107.7 MB read + 26.9 MB written
+    traffic = 134.6e6
     roofline = {"bound": "hbm", "kernel": "ts::csr_reduce_kernel<float, 4, SUM>",
                 "achieved": round(gbs(kernel_bytes, t_kernel), 1), "peak": PEAK_GBS, "unit": "GB/s",
                 "frac": round(gbs(kernel_bytes, t_kernel) / PEAK_GBS, 4), "traffic": traffic,
