@@ -461,7 +461,32 @@ template <int REDUCE> struct ScatterFn : public torch::autograd::Function<Scatte
       return {out};
     }
     if (REDUCE == TS_MEAN) {
-      // count over the index as given (csrc/scatter.cpp:131-141)
+      // count over the index as given (csrc/scatter.cpp:131-141). One index per row (a 1-D index along
+      // dim 0, or an index shaped like src's leading dims): the entries are counted straight from the
+      // index (no tensor of ones; fp32 counts) and one kernel clamps, casts and divides.
+      bool per_row = old_index.dim() == dim + 1 && src.numel() > 0 && out.numel() > 0 && old_index.size(dim) == src.size(dim);
+      for (int64_t i = 0; per_row && i < dim; i++) per_row = old_index.size(i) == src.size(i);
+      if (per_row) {
+        const int64_t B = prod(src.sizes(), 0, dim), E = src.size(dim), N = out.size(dim);
+        const int64_t K = prod(src.sizes(), dim + 1, src.dim());
+        const BatchedIndex bi = batched_index(old_index);
+        Tensor count_f = at::empty({B * N}, src.options().dtype(at::kFloat));
+        check_status(ts_scatter_count(bi.t.data_ptr<int64_t>(), count_f.data_ptr<float>(), B, E, N, bi.batch_stride, 1,
+                                      stream_of(src)),
+                     "scatter_mean count");
+        Tensor out_c = out.contiguous();
+        check_status(ts_divide_by_count(out_c.data_ptr(), count_f.data_ptr<float>(), B, N, K, dtype_code(out_c),
+                                        stream_of(src)),
+                     "scatter_mean divide");
+        if (!out_c.is_same(out)) out.copy_(out_c);
+        if (src.requires_grad()) {  // the count in the element type, as the backward pass divides by it
+          auto count_sizes = out.sizes().vec();
+          count_sizes.resize(dim + 1);
+          Variable count = broadcast(count_f.clamp_min_(1).to(src.scalar_type()).view(count_sizes), out, dim);
+          ctx->save_for_backward({index, count});
+        }
+        return {out};
+      }
       auto ones = at::ones(old_index.sizes(), src.options());
       const int64_t cdim = old_index.dim() <= dim ? old_index.dim() - 1 : dim;
       Variable count = std::get<0>(scatter_hip(ones, old_index, cdim, std::nullopt, out.size(dim), TS_SUM));

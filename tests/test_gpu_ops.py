@@ -405,3 +405,38 @@ def test_segment_csr_under_graph_replay(ts, oracle):
         # eager work between the replays, through the same operators
         eager = ts.segment_sum_csr(static_src, dptr)
         assert torch.allclose(eager, out_sum, rtol=1e-5, atol=1e-3)
+
+
+def test_scatter_mean_counts_from_the_index(ts, oracle):
+    """scatter_mean with one index per row counts the entries straight from the index (fp32 counts,
+    one clamp-cast-divide kernel): same results as the reference's sum / count on the oracle wherever
+    its count is exact, floor division for integers, batched [B, E] index, `out=`, and backward."""
+    g = torch.Generator().manual_seed(9)
+    for dtype in (torch.float32, torch.float64, torch.int32, torch.int64):
+        src = (torch.randn(500, 6, generator=g) * 50).to(dtype)
+        index = torch.randint(0, 40, (500,), generator=g)
+        got = ts.scatter_mean(src.to(DEV), index.to(DEV), 0, None, 45)
+        want = oracle.op_scatter(src, index, 0, None, 45, "mean")
+        if dtype.is_floating_point:
+            assert torch.allclose(got.cpu(), want, rtol=1e-5, atol=1e-5)
+        else:
+            assert torch.equal(got.cpu(), want)
+    # batched index along dim 1, accumulate into a given out (the whole of out is divided, as upstream)
+    src = torch.randn(3, 200, 5, generator=g)
+    index = torch.randint(0, 9, (3, 200), generator=g)
+    prev = torch.randn(3, 9, 5, generator=g)
+    out = prev.clone().to(DEV)
+    ts.scatter_mean(src.to(DEV), index.to(DEV), 1, out)
+    want = oracle.op_scatter(src, index, 1, prev.clone(), None, "mean")
+    assert torch.allclose(out.cpu(), want, rtol=1e-5, atol=1e-5)
+    # fp16 groups of ~1500 entries (sums of ones stay exact up to 2048 in fp16)
+    index = torch.randint(0, 3, (4500,), generator=g)
+    got = ts.scatter_mean(torch.ones(4500, 4, dtype=torch.float16, device=DEV), index.to(DEV), 0, None, 4)
+    assert torch.equal(got.cpu(), torch.tensor([[1.0] * 4] * 3 + [[0.0] * 4], dtype=torch.float16))
+    # backward: grad_out[group] / count
+    src = torch.randn(300, 4, generator=g, dtype=torch.double).to(DEV).requires_grad_(True)
+    index = torch.randint(0, 20, (300,), generator=g)
+    grad = torch.randn(25, 4, generator=g, dtype=torch.double)
+    ts.scatter_mean(src, index.to(DEV), 0, None, 25).backward(grad.to(DEV))
+    count = torch.bincount(index, minlength=25).clamp(min=1).double()
+    assert torch.allclose(src.grad.cpu(), (grad / count.view(-1, 1))[index], rtol=1e-12)
