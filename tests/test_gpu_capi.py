@@ -121,6 +121,25 @@ def test_segment_csr(capi, oracle, case, reduce, dtype):
         assert_close(out, want, scale, dtype, "values")
 
 
+@pytest.mark.parametrize("case", [("long", 12, 64), ("hub", 900, 64), ("long", 9, 1), ("zipf", 3000, 64)])
+def test_segment_csr_is_bit_reproducible(capi, case):
+    """Rows that cross tiles are combined in an order fixed by the tiling (carries collected by the tile in
+    which the row ends, or by the second kernel), never by arrival: repeated launches give identical bits."""
+    kind, n, K = case
+    rng, indptr, index = make_csr(kind, 31, n)
+    E = index.numel()
+    src = torch.from_numpy(rng.standard_normal(size=(E, K))).float().to(DEV)
+    dptr = indptr.to(DEV)
+    first = None
+    for rep in range(6):
+        out = torch.empty((n, K), device=DEV)
+        capi.segment_csr(src, dptr, out, None, 1, n, E, K, 0, capi.SUM)
+        torch.cuda.synchronize()
+        if first is None:
+            first = out.clone()
+        assert torch.equal(_bits(out), _bits(first)), rep
+
+
 @pytest.mark.parametrize("dtype,reduce", product(
     [torch.float16, torch.float64, torch.int32, torch.int64, torch.int16, torch.int8, torch.uint8],
     ["sum", "mean", "min", "max"]))
