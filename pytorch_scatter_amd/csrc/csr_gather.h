@@ -119,7 +119,7 @@ template <typename T, bool DIV, bool VROW>
 __global__ __launch_bounds__(kBlock) void csr_gather_small_kernel(CsrGatherArgs a, int vec_ok) {
   constexpr int VE = kVecBytes / (int)sizeof(T);
   __shared__ int32_t s_ptr[kMaxBlockItems + 2];
-  __shared__ int32_t s_row[kMaxBlockItems];  // local row of every entry of the tile
+  __shared__ int32_t s_row[VROW ? kMaxBlockItems : 1];  // local row of every entry of the tile (VROW)
   __shared__ int32_t s_wtot[kBlock / kWave];
   __shared__ int64_t s_cut[2];
 
@@ -149,6 +149,49 @@ __global__ __launch_bounds__(kBlock) void csr_gather_small_kernel(CsrGatherArgs 
   __syncthreads();
   const int rmax = nload - 2;  // last local row whose end is known; i0 + rmax <= N - 1
   if (rmax < 0) return;
+
+  if (!VROW) {
+    // Rows of 1-3 elements: a 16-byte granule of out covers several entries. Its first entry's row comes
+    // from a binary search of the tile's row pointers (about ten LDS reads), the following entries
+    // advance from there; no per-entry row table, no barriers.
+    const int64_t f0 = j0 * K, f1 = (j0 + ne) * K;
+    const int64_t g0 = f0 / VE, g1 = (f1 + VE - 1) / VE;
+    for (int64_t g = g0 + tid; g < g1; g += kBlock) {
+      const int64_t fb = g * VE > f0 ? g * VE : f0;
+      const int64_t fe = (g + 1) * VE < f1 ? (g + 1) * VE : f1;
+      const unsigned rel = (unsigned)(fb - f0);  // 32-bit arithmetic relative to the tile (f0 is a row start)
+      int e = (int)(rel / (unsigned)K);          // entry, relative to the tile
+      int k = (int)(rel - (unsigned)e * (unsigned)K);
+      int lo = 0, hi = rmax;  // the last row that starts at or before e (rows without entries share a start)
+      while (lo < hi) {
+        const int mid = (lo + hi + 1) >> 1;
+        if (s_ptr[mid] <= e) lo = mid; else hi = mid - 1;
+      }
+      int row = lo;
+      Vec<T, VE> y;
+#pragma unroll
+      for (int i = 0; i < VE; ++i) {
+        if (fb + i < fe) {
+          T v = src_b[(i0 + row) * a.K + k];
+          if (DIV) v = div_elem<T>(v, count_as<T>((int64_t)s_ptr[row + 1] - (int64_t)s_ptr[row]));
+          y.v[i] = v;
+          if (++k == K) {
+            k = 0;
+            ++e;
+            while (row < rmax && s_ptr[row + 1] <= e) ++row;
+          }
+        }
+      }
+      if (vec_ok && fe - fb == VE) {
+        store_vec<T, VE>(out_b + fb, y);
+      } else {
+#pragma unroll
+        for (int i = 0; i < VE; ++i)
+          if (fb + i < fe) out_b[fb + i] = y.v[i];
+      }
+    }
+    return;
+  }
 
   // ---- row of every entry of the tile: mark the first entry of each non-empty row, then a
   // running maximum over the entries (entries before the first mark belong to row 0)
@@ -219,31 +262,6 @@ __global__ __launch_bounds__(kBlock) void csr_gather_small_kernel(CsrGatherArgs 
       }
     }
     return;
-  }
-  for (int64_t g = g0 + tid; g < g1; g += kBlock) {
-    const int64_t fb = g * VE > f0 ? g * VE : f0;
-    const int64_t fe = (g + 1) * VE < f1 ? (g + 1) * VE : f1;
-    const unsigned rel = (unsigned)(fb - f0);  // 32-bit arithmetic relative to the tile (f0 is a row start)
-    int e = (int)(rel / (unsigned)K);    // entry, relative to the tile
-    int k = (int)(rel - (unsigned)e * (unsigned)K);
-    Vec<T, VE> y;
-#pragma unroll
-    for (int i = 0; i < VE; ++i) {
-      if (fb + i < fe) {
-        const int row = s_row[e];
-        T v = src_b[(i0 + row) * a.K + k];
-        if (DIV) v = div_elem<T>(v, count_as<T>((int64_t)s_ptr[row + 1] - (int64_t)s_ptr[row]));
-        y.v[i] = v;
-        if (++k == K) { k = 0; ++e; }
-      }
-    }
-    if (vec_ok && fe - fb == VE) {
-      store_vec<T, VE>(out_b + fb, y);
-    } else {
-#pragma unroll
-      for (int i = 0; i < VE; ++i)
-        if (fb + i < fe) out_b[fb + i] = y.v[i];
-    }
   }
 }
 
