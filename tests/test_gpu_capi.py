@@ -420,6 +420,35 @@ def test_gather_coo_and_mean_backward(capi, oracle, case, dtype):
         assert_exact(out, want)
 
 
+@pytest.mark.parametrize("K,dtype,B", product(
+    [1, 3, 5, 7, 17, 33, 47, 129], [torch.float32, torch.bfloat16, torch.float64, torch.int8], [1, 3]))
+def test_gather_coo_odd_widths(capi, oracle, K, dtype, B):
+    """Row widths that are no multiple of 16 bytes take the flat kernel (a lane owns 16 consecutive bytes
+    of out that may span several edges); batches whose slices leave the 16-byte grid, and out / src
+    buffers off that grid, take its one-element-per-lane form. Bit-exact, and nothing outside out is touched."""
+    n, E = 300, 2511
+    rng = np.random.default_rng(K * 7 + B)
+    index = torch.from_numpy(np.sort(rng.integers(0, n, size=(B, E)), axis=1))
+    src = random_values(rng, (B, n, K), dtype, ties=False)
+    want = torch.stack([oracle.gather_coo(src[b], index[b]) for b in range(B)])
+    for off in (0, 1):
+        sflat = torch.zeros(B * n * K + 8, dtype=dtype, device=DEV)
+        dsrc = sflat[off:off + B * n * K].view(B, n, K)
+        dsrc.copy_(src)
+        oflat = torch.full((B * E * K + 8,), 7, dtype=dtype, device=DEV)
+        out = oflat[off:off + B * E * K].view(B, E, K)
+        capi.gather_coo(dsrc, index.to(DEV), out, B, n, E, K, E)
+        torch.cuda.synchronize()
+        assert_exact(out, want, f"off={off}")
+        assert bool((oflat[:off] == 7).all()) and bool((oflat[off + B * E * K:] == 7).all())
+        if dtype.is_floating_point:
+            count = torch.stack([torch.bincount(index[b], minlength=n) for b in range(B)]).clamp(min=1).to(dtype)
+            want_b = torch.stack([oracle.segment_mean_coo_backward(src[b], index[b], count[b], (E, K)) for b in range(B)])
+            capi.segment_mean_coo_backward(dsrc, index.to(DEV), count.to(DEV), out, B, n, E, K, E)
+            torch.cuda.synchronize()
+            assert_exact(out, want_b, f"mean backward off={off}")
+
+
 SCATTER_SHAPES = [
     # B, E, K, N
     (1, 1000, 1, 37), (1, 5000, 16, 300), (1, 3000, 32, 10), (2, 700, 5, 50), (3, 400, 8, 1),
