@@ -153,7 +153,7 @@ def bench_scatter_config(ts, wl, w, dev, iters, reduces):
 
 
 def bench_softmax_config(ts, wl, w, dev, iters, K):
-    """scatter_softmax over the destination index of the C3 graph with K values per entry (attention
+    """scatter_softmax and scatter_std over the destination index of the C3 graph with K values per entry (attention
     heads), sorted and in random order; bytes: src read once, index read once, result written once."""
     import torch
     index = w.index.to(dev)
@@ -171,6 +171,16 @@ def bench_softmax_config(ts, wl, w, dev, iters, K):
         y = ts.scatter_softmax(x, idx, 0, w.N)
         t = event_time(lambda: torch.autograd.grad(y, x, grad, retain_graph=True), iters)
         res[f"softmax_backward_{name}"] = entry(bwd_bytes, t, w.E * K)
+        del x, y
+        # std: src read twice (group sums, then squared deviations), index twice, N*K result
+        with torch.no_grad():
+            t = event_time(lambda: ts.scatter_std(src, idx, 0, None, w.N), iters)
+        res[f"std_{name}"] = entry(2 * (w.E * K * 4 + w.E * 8) + w.N * K * 4, t, w.E * K)
+        x = src.clone().requires_grad_(True)
+        y = ts.scatter_std(x, idx, 0, None, w.N)
+        gn = grad[:w.N].contiguous()
+        t = event_time(lambda: torch.autograd.grad(y, x, gn, retain_graph=True), iters)
+        res[f"std_backward_{name}"] = entry(2 * w.E * K * 4 + w.E * 8, t, w.E * K)
         del x, y
     del src, grad
     torch.cuda.empty_cache()

@@ -231,6 +231,28 @@ int ts_group_logsumexp_backward(const void *src, const int64_t *index,
                                 int64_t index_stride_e, int dtype,
                                 ts_stream_t stream);
 
+/* Standard deviation over the entries that share an index, one index per row, given the group sums
+ * `total` ([B, N, K], element type: ts_scatter with SUM) and the entries per group `count` ([B, N]
+ * float: ts_scatter_count):
+ *   mean = total / max(count, 1);  out = sqrt(sum_group (src - mean)^2 / (d + 1e-6)),
+ *   d = max(count - 1, 1) if unbiased else max(count, 1).
+ * Replaces the second half of torch_scatter/composite/std.py:8-41 (gather of the mean, sub, mul,
+ * scatter_sum, div, sqrt) for the call without `out`; the reference has no single launcher for it.
+ * Backward: grad_in[b, e, k] = grad_out[b, n, k] * (src - mean) / (out[b, n, k] * (d + 1e-6)).
+ * Workspace as for ts_group_softmax. Floating types only.
+ */
+int ts_group_std(const void *src, const int64_t *index, const void *total,
+                 const float *count, void *out, int64_t B, int64_t E, int64_t K,
+                 int64_t N, int64_t index_stride_b, int64_t index_stride_e,
+                 int dtype, int unbiased, void *workspace, size_t workspace_bytes,
+                 ts_stream_t stream);
+int ts_group_std_backward(const void *src, const int64_t *index,
+                          const void *total, const float *count,
+                          const void *out, const void *grad_out, void *grad_in,
+                          int64_t B, int64_t E, int64_t K, int64_t N,
+                          int64_t index_stride_b, int64_t index_stride_e,
+                          int dtype, int unbiased, ts_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -432,6 +432,31 @@ def scatter_std(src, index, dim=-1, out=None, dim_size=None, unbiased=True):
     return sq.div(count + 1e-6).sqrt()
 
 
+def scatter_std_backward(src, grad_out, index, dim=-1, dim_size=None, unbiased=True):
+    """What autograd derives for scatter_std above: the same sequence
+    (composite/std.py:19-41) on differentiable torch ops (index_add for the
+    sums), differentiated by torch. Returns (std, grad_src). A group whose std is 0
+    gets NaN, from the derivative of sqrt at 0."""
+    index, dim = _py_broadcast(index, src, dim)
+    if dim_size is None:
+        dim_size = int(index.max()) + 1
+    x = src.detach().clone().requires_grad_(True)
+    shape = list(x.shape)
+    shape[dim] = dim_size
+
+    def group_sum(v):
+        return torch.zeros(shape, dtype=v.dtype).scatter_add(dim, index, v)
+
+    count = group_sum(torch.ones_like(x)).clamp(1)
+    dev = x - (group_sum(x) / count).gather(dim, index)
+    sq = group_sum(dev * dev)
+    if unbiased:
+        count = count.sub(1).clamp(1)
+    std = (sq / (count + 1e-6)).sqrt()
+    grad, = torch.autograd.grad(std, x, grad_out)
+    return std.detach(), grad
+
+
 def scatter_softmax_backward(result, grad_out, index, dim=-1, dim_size=None, log_space=False):
     """What autograd derives for the two functions above (closed form; the
     reference has no explicit backward, it differentiates through its ops):

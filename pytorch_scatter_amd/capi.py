@@ -29,6 +29,7 @@ EXPORTS = (
     "ts_scatter", "ts_scatter_count", "ts_divide_by_count", "ts_arg_backward",
     "ts_group_softmax_workspace_bytes", "ts_group_softmax", "ts_group_softmax_backward",
     "ts_group_logsumexp", "ts_group_logsumexp_backward",
+    "ts_group_std", "ts_group_std_backward",
 )
 
 _lib = None
@@ -207,3 +208,21 @@ def group_logsumexp_backward(src, index, out, grad_out, grad_in, B, E, K, N, sb,
         _check(lib().ts_group_logsumexp_backward(_p(src), _p(index), _p(out), _p(grad_out), _p(grad_in), _i(B),
                                                  _i(E), _i(K), _i(N), _i(sb), _i(se), DTYPE[grad_in.dtype],
                                                  _stream(grad_in)))
+
+
+def group_std(src, index, total, count, out, B, E, K, N, sb, se, unbiased: bool = True):
+    _dev(src, index, total, count, out)
+    ws, nbytes = _group_workspace(out, B, N, K)
+    with torch.cuda.device(out.device):
+        _check(lib().ts_group_std(_p(src), _p(index), _p(total), _p(count), _p(out), _i(B), _i(E), _i(K), _i(N),
+                                  _i(sb), _i(se), DTYPE[out.dtype], int(unbiased), _p(ws), ctypes.c_size_t(nbytes),
+                                  _stream(out)))
+    return ws
+
+
+def group_std_backward(src, index, total, count, out, grad_out, grad_in, B, E, K, N, sb, se, unbiased: bool = True):
+    _dev(src, index, total, count, out, grad_out, grad_in)
+    with torch.cuda.device(grad_in.device):
+        _check(lib().ts_group_std_backward(_p(src), _p(index), _p(total), _p(count), _p(out), _p(grad_out),
+                                           _p(grad_in), _i(B), _i(E), _i(K), _i(N), _i(sb), _i(se),
+                                           DTYPE[grad_in.dtype], int(unbiased), _stream(grad_in)))

@@ -1,26 +1,10 @@
 """Group-wise statistics over the entries that share an index: softmax,
 log-softmax, logsumexp and standard deviation (API of
-torch_scatter/composite/{softmax,logsumexp,std}.py). Softmax, log-softmax
-and logsumexp are fused operators; std is composed from the scatter
-operators."""
+torch_scatter/composite/{softmax,logsumexp,std}.py), each one registered
+operator."""
 from typing import Optional
 
 import torch
-
-from .scatter import scatter_sum
-
-
-def _expand_index(index: torch.Tensor, like: torch.Tensor, dim: int) -> torch.Tensor:
-    # a 1-D index addresses `dim`; missing trailing dims are broadcast
-    # (torch_scatter/utils.py:4-13)
-    dim = dim + like.dim() if dim < 0 else dim
-    if index.dim() == 1:
-        shape = [1] * like.dim()
-        shape[dim] = index.numel()
-        index = index.view(shape)
-    while index.dim() < like.dim():
-        index = index.unsqueeze(-1)
-    return index.expand(like.size())
 
 
 def _require_float(src: torch.Tensor, name: str):
@@ -62,16 +46,10 @@ def scatter_logsumexp(src: torch.Tensor, index: torch.Tensor, dim: int = -1,
 def scatter_std(src: torch.Tensor, index: torch.Tensor, dim: int = -1,
                 out: Optional[torch.Tensor] = None, dim_size: Optional[int] = None,
                 unbiased: bool = True) -> torch.Tensor:
-    if out is not None:
-        dim_size = out.size(dim)
-    dim = dim + src.dim() if dim < 0 else dim
-    count_dim = index.dim() - 1 if index.dim() <= dim else dim
-    count = scatter_sum(torch.ones(index.size(), dtype=src.dtype, device=src.device),
-                        index, count_dim, None, dim_size)
-    full_index = _expand_index(index, src, dim)
-    total = scatter_sum(src, full_index, dim, None, dim_size)
-    count = _expand_index(count, total, dim).clamp(1)
-    centred = src - total.div(count).gather(dim, full_index)
-    sq = scatter_sum(centred * centred, full_index, dim, out, dim_size)
-    denom = count.sub(1).clamp_(1) if unbiased else count
-    return sq.div(denom + 1e-6).sqrt()
+    """``sqrt(sum((src - mean)^2) / (count - 1 + 1e-6))`` over the entries that share an
+    index (``count`` instead of ``count - 1`` if not ``unbiased``;
+    torch_scatter/composite/std.py:8-41). Group sums and counts come from the scatter
+    kernels, the squared deviations from one fused pass; with ``out`` given or an index
+    that differs between the columns of a row, the same sequence as upstream on the
+    scatter operators. Counts are exact (fp32) where upstream counts in the element type."""
+    return torch.ops.torch_scatter.scatter_std(src, index, dim, out, dim_size, unbiased)

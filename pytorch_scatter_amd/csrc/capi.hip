@@ -409,6 +409,9 @@ int run_group_softmax(const void *src, const void *grad, const int64_t *index, v
   g.node_out = nullptr;
   g.node_grad = nullptr;
   g.from_neg_inf = 0;
+  g.total = nullptr;
+  g.count = nullptr;
+  g.unbiased = 0;
   const int full = kVecBytes / kElemBytes[dtype];
   const bool al = aligned16(src) && aligned16(out) && (!grad || aligned16(grad));
   const int vec = (full > 1 && K % full == 0 && al) ? full : 1;
@@ -491,6 +494,66 @@ int ts_group_logsumexp_backward(const void *src, const int64_t *index, const voi
   const bool al = aligned16(src) && aligned16(grad_in) && aligned16(out) && aligned16(grad_out);
   const int vec = (full > 1 && K % full == 0 && al) ? full : 1;
   return dispatch_group_softmax(dtype, g, GS_LSE_BWD, vec, static_cast<hipStream_t>(stream));
+}
+
+int ts_group_std(const void *src, const int64_t *index, const void *total, const float *count, void *out, int64_t B,
+                 int64_t E, int64_t K, int64_t N, int64_t index_stride_b, int64_t index_stride_e, int dtype,
+                 int unbiased, void *workspace, size_t workspace_bytes, ts_stream_t stream) {
+  if (!valid_dtype(dtype) || !sizes_ok(B, N, E, K)) return TS_ERR_BAD_ARG;
+  if (!is_float_dtype(dtype)) return TS_ERR_UNSUPPORTED;
+  if (B * N * K == 0) return TS_OK;
+  if (!out || !total || !count || (B * E * K > 0 && (!src || !index))) return TS_ERR_BAD_ARG;
+  if (B * N >= 0x7FFFFFFFll) return TS_ERR_UNSUPPORTED;
+  const size_t need = group_workspace_bytes(B, N, K, kElemBytes[dtype]);
+  if (!workspace || workspace_bytes < need || !aligned16(workspace)) return TS_ERR_WORKSPACE;
+  GroupArgs g = {};
+  g.src = src;
+  g.index = index;
+  g.out = out;
+  g.gmax = workspace;
+  g.gsum = static_cast<char *>(workspace) + need / 2;
+  g.total = total;
+  g.count = count;
+  g.unbiased = unbiased ? 1 : 0;
+  g.B = B;
+  g.E = E;
+  g.K = K;
+  g.N = N;
+  g.sb = index_stride_b;
+  g.se = index_stride_e;
+  const int full = kVecBytes / kElemBytes[dtype];
+  const int vec = (full > 1 && K % full == 0 && aligned16(src) && aligned16(total)) ? full : 1;
+  return dispatch_group_softmax(dtype, g, GS_STD, vec, static_cast<hipStream_t>(stream));
+}
+
+int ts_group_std_backward(const void *src, const int64_t *index, const void *total, const float *count,
+                          const void *out, const void *grad_out, void *grad_in, int64_t B, int64_t E, int64_t K,
+                          int64_t N, int64_t index_stride_b, int64_t index_stride_e, int dtype, int unbiased,
+                          ts_stream_t stream) {
+  if (!valid_dtype(dtype) || !sizes_ok(B, N, E, K)) return TS_ERR_BAD_ARG;
+  if (!is_float_dtype(dtype)) return TS_ERR_UNSUPPORTED;
+  if (B * E * K == 0) return TS_OK;
+  if (!src || !index || !total || !count || !out || !grad_out || !grad_in) return TS_ERR_BAD_ARG;
+  if (N == 0 || B * N >= 0x7FFFFFFFll) return TS_ERR_UNSUPPORTED;
+  GroupArgs g = {};
+  g.src = src;
+  g.index = index;
+  g.out = grad_in;
+  g.node_out = out;
+  g.node_grad = grad_out;
+  g.total = total;
+  g.count = count;
+  g.unbiased = unbiased ? 1 : 0;
+  g.B = B;
+  g.E = E;
+  g.K = K;
+  g.N = N;
+  g.sb = index_stride_b;
+  g.se = index_stride_e;
+  const int full = kVecBytes / kElemBytes[dtype];
+  const bool al = aligned16(src) && aligned16(grad_in) && aligned16(out) && aligned16(grad_out) && aligned16(total);
+  const int vec = (full > 1 && K % full == 0 && al) ? full : 1;
+  return dispatch_group_softmax(dtype, g, GS_STD_BWD, vec, static_cast<hipStream_t>(stream));
 }
 
 }  // extern "C"

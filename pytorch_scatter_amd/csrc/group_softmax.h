@@ -54,6 +54,8 @@ __device__ __forceinline__ float exp_acc(float v) { return expf(v); }
 __device__ __forceinline__ double exp_acc(double v) { return exp(v); }
 __device__ __forceinline__ float log_acc(float v) { return logf(v); }
 __device__ __forceinline__ double log_acc(double v) { return log(v); }
+__device__ __forceinline__ float sqrt_acc(float v) { return sqrtf(v); }
+__device__ __forceinline__ double sqrt_acc(double v) { return sqrt(v); }
 
 // a value of the accumulate type as the element type would hold it
 template <typename T> __device__ __forceinline__ typename Acc<T>::type round_elem(typename Acc<T>::type v) {
@@ -64,7 +66,10 @@ template <typename T> __device__ __forceinline__ typename OrdKey<typename Acc<T>
   return OrdKey<typename Acc<T>::type>::enc(to_acc<T>(ElemLim<T>::lowest()));
 }
 
-enum { GS_SOFTMAX = 0, GS_LOG_SOFTMAX = 1, GS_SOFTMAX_BWD = 2, GS_LOG_SOFTMAX_BWD = 3, GS_LSE = 4, GS_LSE_BWD = 5 };
+enum {
+  GS_SOFTMAX = 0, GS_LOG_SOFTMAX = 1, GS_SOFTMAX_BWD = 2, GS_LOG_SOFTMAX_BWD = 3, GS_LSE = 4, GS_LSE_BWD = 5,
+  GS_STD = 6, GS_STD_BWD = 7
+};
 
 struct GroupArgs {
   const void *src;       // [B, E, K]: forward input; backward: the forward result y
@@ -79,7 +84,27 @@ struct GroupArgs {
   const void *node_out;   // [B, N, K]: logsumexp backward, the forward result
   const void *node_grad;  // [B, N, K]: logsumexp backward, its gradient
   int from_neg_inf;       // the group maximum starts from -inf (logsumexp) instead of lowest() (softmax)
+  const void *total;      // [B, N, K]: std, the group sums of src in the element type
+  const float *count;     // [B, N]: std, entries per group
+  int unbiased;           // std: divide by count - 1
 };
+
+// std: the group mean as the reference forms it (composite/std.py:27-31: sum / clamp(count, 1), in the
+// element type) and the divisor of the squared deviations (:36-38: count or clamp(count - 1, 1), plus 1e-6)
+template <typename T> __device__ __forceinline__ typename Acc<T>::type group_mean(T total, float count) {
+  typedef typename Acc<T>::type F;
+  const F c = round_elem<T>((F)(count < 1.0f ? 1.0f : count));
+  return round_elem<T>(to_acc<T>(total) / c);
+}
+template <typename T> __device__ __forceinline__ typename Acc<T>::type group_divisor(float count, int unbiased) {
+  typedef typename Acc<T>::type F;
+  F c = round_elem<T>((F)(count < 1.0f ? 1.0f : count));
+  if (unbiased) {
+    c = round_elem<T>(c - (F)1);
+    if (c < (F)1) c = (F)1;
+  }
+  return round_elem<T>(c + (F)1e-6);
+}
 
 inline size_t group_align(size_t v) { return (v + 255) / 256 * 256; }
 // bytes of workspace: keys and sums, each [B, N, K] in 8 bytes at most
@@ -171,6 +196,8 @@ template <typename T, int C_, int MODE> struct GroupSumRun : HotState<typename A
   const T *grad;
   const void *gmax;
   A *gsum;
+  const T *total;
+  const float *count;
   int64_t K;
   __device__ A identity() const { return (A)0; }
   __device__ void load(int64_t e, int64_t, int64_t col, int node, A *x) const {
@@ -188,6 +215,20 @@ template <typename T, int C_, int MODE> struct GroupSumRun : HotState<typename A
         A z = round_elem<T>(to_acc<T>(r.v[c]) - m[c]);
         if (MODE == GS_LSE && z != z) z = -INFINITY;  // NaN entries and -inf - -inf drop out (logsumexp.py:41)
         x[c] = round_elem<T>(exp_acc(z));
+      }
+    } else if constexpr (MODE == GS_STD) {
+      const Vec<T, C> r = load_vec_stream<T, C>(src + e * K + col);
+      if (node < 0) {
+#pragma unroll
+        for (int c = 0; c < C; ++c) x[c] = (A)0;
+        return;
+      }
+      const Vec<T, C> tot = load_vec<T, C>(total + (int64_t)node * K + col);
+      const float cnt = count[node];
+#pragma unroll
+      for (int c = 0; c < C; ++c) {
+        const A d = round_elem<T>(to_acc<T>(r.v[c]) - group_mean<T>(tot.v[c], cnt));
+        x[c] = round_elem<T>(d * d);
       }
     } else if constexpr (MODE == GS_SOFTMAX_BWD) {
       const Vec<T, C> y = load_vec_stream<T, C>(src + e * K + col);
@@ -222,6 +263,8 @@ __global__ __launch_bounds__(kBlock) void group_sum_run_kernel(ScatterArgs a, Gr
   p.grad = static_cast<const T *>(g.grad);
   p.gmax = g.gmax;
   p.gsum = static_cast<A *>(g.gsum);
+  p.total = static_cast<const T *>(g.total);
+  p.count = g.count;
   p.K = g.K;
   p.hot_init(s_hot, s_tags, hot_rlog, lshift + LogC<C>::value);
   run_wave<SERIAL>(a, lshift, rows_per_wave, p, s_stage[threadIdx.x / kWave]);
@@ -271,6 +314,22 @@ __global__ __launch_bounds__(kBlock) void group_finish_kernel(GroupArgs g) {
           continue;
         }
         const int64_t slot = (bb[u] * g.N + idx[u]) * g.K + k0;
+        if constexpr (MODE == GS_STD_BWD) {
+          // d std / d src = (src - mean) / (std * divisor); a group whose std is 0 gets 0 / 0 = NaN,
+          // as autograd gives for the reference's sqrt at 0
+          const Vec<T, VEC> o = load_vec<T, VEC>(static_cast<const T *>(g.node_out) + slot);
+          const Vec<T, VEC> go = load_vec<T, VEC>(static_cast<const T *>(g.node_grad) + slot);
+          const Vec<T, VEC> tot = load_vec<T, VEC>(static_cast<const T *>(g.total) + slot);
+          const float cnt = g.count[bb[u] * g.N + idx[u]];
+          const F div = group_divisor<T>(cnt, g.unbiased);
+#pragma unroll
+          for (int v = 0; v < VEC; ++v) {
+            const F d = to_acc<T>(x[u].v[v]) - group_mean<T>(tot.v[v], cnt);
+            r.v[v] = from_acc<T>(to_acc<T>(go.v[v]) * d / (to_acc<T>(o.v[v]) * div));
+          }
+          store_vec_stream<T, VEC>(out + be * g.K + k0, r);
+          continue;
+        }
         if constexpr (MODE == GS_LSE_BWD) {
           // d logsumexp / d src = exp(src - result) (= exp(z) / (sum + eps)); NaN entries dropped out forward
           const Vec<T, VEC> o = load_vec<T, VEC>(static_cast<const T *>(g.node_out) + slot);
@@ -335,6 +394,19 @@ __global__ __launch_bounds__(kBlock) void group_lse_finish_kernel(GroupArgs g) {
   }
 }
 
+// std: result per group, sqrt(sum of squared deviations / divisor) (composite/std.py:33-39)
+template <typename T>
+__global__ __launch_bounds__(kBlock) void group_std_finish_kernel(GroupArgs g) {
+  typedef typename Acc<T>::type F;
+  const int64_t n = g.B * g.N * g.K;
+  const F *gsum = static_cast<const F *>(g.gsum);
+  T *out = static_cast<T *>(g.out);
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlock) {
+    const F div = group_divisor<T>(g.count[i / g.K], g.unbiased);
+    out[i] = from_acc<T>(sqrt_acc(round_elem<T>(round_elem<T>(gsum[i]) / div)));
+  }
+}
+
 // ---- host side
 inline ScatterArgs group_index_args(const GroupArgs &g) {
   ScatterArgs a = {};
@@ -394,8 +466,32 @@ int launch_group_lse_v(const GroupArgs &g, bool backward, hipStream_t stream) {
 }
 
 template <typename T, int VEC>
+int launch_group_std_v(const GroupArgs &g, bool backward, hipStream_t stream) {
+  const int64_t n_edges = g.B * g.E;
+  if (g.B * g.N >= 0x7FFFFFFFll) return TS_ERR_UNSUPPORTED;
+  if (backward) {
+    hipLaunchKernelGGL((group_finish_kernel<T, VEC, GS_STD_BWD>), dim3(scatter_grid(n_edges, g.K / VEC, kBlock, 4)),
+                       dim3(kBlock), 0, stream, g);
+    return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
+  }
+  const RunGrid rg = run_grid(n_edges, g.K / VEC, VEC, VEC * (int)sizeof(T));
+  if (!rg.ok) return TS_ERR_UNSUPPORTED;
+  const ScatterArgs a = group_index_args(g);
+  const dim3 gd(rg.blocks, rg.ychunks);
+  const unsigned g_out = grid_for(g.B * g.N * g.K);
+  hipLaunchKernelGGL(group_init_kernel<T>, dim3(g_out), dim3(kBlock), 0, stream, g, 0);
+  if (n_edges > 0)
+    TS_LAUNCH_RUN(rg.serial, (group_sum_run_kernel<T, VEC, GS_STD, true>), (group_sum_run_kernel<T, VEC, GS_STD, false>), gd,
+                  stream, a, g, rg.lshift, rg.rpw, rg.hot_rlog);
+  hipLaunchKernelGGL(group_std_finish_kernel<T>, dim3(g_out), dim3(kBlock), 0, stream, g);
+  return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
+}
+
+template <typename T, int VEC>
 int launch_group_softmax_v(const GroupArgs &g, int mode, hipStream_t stream) {
   switch (mode) {
+  case GS_STD: return launch_group_std_v<T, VEC>(g, false, stream);
+  case GS_STD_BWD: return launch_group_std_v<T, VEC>(g, true, stream);
   case GS_LSE: return launch_group_lse_v<T, VEC>(g, false, stream);
   case GS_LSE_BWD: return launch_group_lse_v<T, VEC>(g, true, stream);
   case GS_SOFTMAX: return launch_group_softmax_m<T, VEC, GS_SOFTMAX>(g, stream);

@@ -744,6 +744,51 @@ struct GroupLogSumExpFn : public torch::autograd::Function<GroupLogSumExpFn> {
   }
 };
 
+// scatter_std of torch_scatter/composite/std.py:8-41 for the call without `out`: group sums and
+// counts from the scatter kernels, then one pass for the squared deviations and one per group
+struct GroupStdFn : public torch::autograd::Function<GroupStdFn> {
+  static variable_list forward(AutogradContext *ctx, Variable src, Variable index, int64_t dim, int64_t N,
+                               bool unbiased) {
+    check_device(src, "src");
+    check_device(index, "index");
+    c10::DeviceGuard guard(src.device());
+    src = src.contiguous();
+    const GroupLayout l = group_layout(src, index, dim);
+    Tensor total = std::get<0>(scatter_hip(src, index, dim, std::nullopt, N, TS_SUM)).contiguous();
+    Tensor count = at::empty({l.B * N}, src.options().dtype(at::kFloat));
+    check_status(ts_scatter_count(index.data_ptr<int64_t>(), count.data_ptr<float>(), l.B, l.E, N, l.sb, l.se,
+                                  stream_of(src)),
+                 "scatter_std count");
+    Tensor out = at::empty_like(total);
+    Tensor ws = workspace(ts_group_softmax_workspace_bytes(l.B, N, l.K, dtype_code(src)), src);
+    check_status(ts_group_std(src.data_ptr(), index.data_ptr<int64_t>(), total.data_ptr(), count.data_ptr<float>(),
+                              out.data_ptr(), l.B, l.E, l.K, N, l.sb, l.se, dtype_code(src), unbiased ? 1 : 0,
+                              ws.data_ptr(), static_cast<size_t>(ws.numel()), stream_of(src)),
+                 "scatter_std");
+    ctx->saved_data["dim"] = dim;
+    ctx->saved_data["unbiased"] = unbiased;
+    ctx->save_for_backward({src, index, total, count, out});
+    return {out};
+  }
+
+  static variable_list backward(AutogradContext *ctx, variable_list grad_outs) {
+    auto saved = ctx->get_saved_variables();
+    Tensor src = saved[0], index = saved[1], total = saved[2], count = saved[3], out = saved[4];
+    Tensor grad_out = grad_outs[0].contiguous();
+    c10::DeviceGuard guard(src.device());
+    const int64_t dim = ctx->saved_data["dim"].toInt();
+    const bool unbiased = ctx->saved_data["unbiased"].toBool();
+    const GroupLayout l = group_layout(src, index, dim);
+    Tensor grad_in = at::empty_like(src);
+    check_status(ts_group_std_backward(src.data_ptr(), index.data_ptr<int64_t>(), total.data_ptr(),
+                                       count.data_ptr<float>(), out.data_ptr(), grad_out.data_ptr(),
+                                       grad_in.data_ptr(), l.B, l.E, l.K, out.size(dim), l.sb, l.se, dtype_code(src),
+                                       unbiased ? 1 : 0, stream_of(src)),
+                 "scatter_std backward");
+    return {grad_in, Variable(), Variable(), Variable(), Variable()};
+  }
+};
+
 // ------------------------------------------------------- registered functions
 Tensor scatter_sum(Tensor src, Tensor index, int64_t dim, OptTensor out, OptInt dim_size) {
   return ScatterFn<TS_SUM>::apply(src, index, dim, out, dim_size)[0];
@@ -855,6 +900,28 @@ Tensor scatter_logsumexp(Tensor src, Tensor index, int64_t dim, OptTensor out, O
   return result;
 }
 
+Tensor scatter_std(Tensor src, Tensor index, int64_t dim, OptTensor out, OptInt dim_size, bool unbiased) {
+  dim = dim < 0 ? src.dim() + dim : dim;
+  if (out.has_value()) dim_size = out.value().size(dim);
+  const Tensor index_given = index;
+  index = broadcast(index, src, dim);
+  TORCH_CHECK(index.scalar_type() == at::kLong, "index must be int64");
+  if (!out.has_value() && src.is_floating_point() && src.numel() > 0) {
+    const int64_t N = dim_size.has_value() ? dim_size.value() : 1 + index.max().item<int64_t>();
+    const GroupLayout l = group_layout(src, index, dim);
+    if (l.fused && N > 0 && l.B * N < 0x7FFFFFFFll) return GroupStdFn::apply(src, index, dim, N, unbiased)[0];
+  }
+  // composite/std.py:19-41
+  const int64_t count_dim = index_given.dim() <= dim ? index_given.dim() - 1 : dim;
+  Tensor count = scatter_sum(at::ones(index_given.sizes(), src.options()), index_given, count_dim, std::nullopt, dim_size);
+  Tensor total = scatter_sum(src, index, dim, std::nullopt, dim_size);
+  count = broadcast(count, total, dim).clamp(1);
+  Tensor centred = src - total.div(count).gather(dim, index);
+  Tensor sq = scatter_sum(centred * centred, index, dim, out, dim_size);
+  if (unbiased) count = count.sub(1).clamp_(1);
+  return sq.div(count + 1e-6).sqrt();
+}
+
 int64_t cuda_version() { return ts_hip_version(); }  // csrc/version.cpp:28-38 returns HIP_VERSION on ROCm
 
 }  // namespace
@@ -877,4 +944,5 @@ static auto registry = torch::RegisterOperators()
                            .op("torch_scatter::segment_max_coo", &segment_max_coo)
                            .op("torch_scatter::gather_coo", &gather_coo)
                            .op("torch_scatter::scatter_softmax", &scatter_softmax)
-                           .op("torch_scatter::scatter_logsumexp", &scatter_logsumexp);
+                           .op("torch_scatter::scatter_logsumexp", &scatter_logsumexp)
+                           .op("torch_scatter::scatter_std", &scatter_std);

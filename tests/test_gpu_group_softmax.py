@@ -1,7 +1,7 @@
-"""The fused softmax / log-softmax / logsumexp over groups (ts_group_softmax,
-ts_group_logsumexp and their backward calls through the C ABI,
-torch.ops.torch_scatter.scatter_softmax / scatter_logsumexp through the Python
-API) against the CPU oracle on the same seeded inputs.
+"""The fused softmax / log-softmax / logsumexp / std over groups (ts_group_softmax,
+ts_group_logsumexp, ts_group_std and their backward calls through the C ABI,
+torch.ops.torch_scatter.scatter_softmax / scatter_logsumexp / scatter_std through
+the Python API) against the CPU oracle on the same seeded inputs.
 
 Bars. fp32 / fp64 compare with the oracle's result in the same type:
 rtol 1e-5 / 1e-12 (the two differ in the exp of the math library and in the
@@ -272,3 +272,134 @@ def test_logsumexp_operator(ts, oracle):
     assert torch.allclose(got.cpu(), oracle.scatter_logsumexp(x, idx2, 0), rtol=1e-5, atol=1e-6)
     with pytest.raises(ValueError):
         ts.scatter_logsumexp(torch.ones(4, dtype=torch.long, device=DEV), torch.zeros(4, dtype=torch.long, device=DEV))
+
+
+# ------------------------------------------------------------------ std
+STD_SHAPES = [
+    # B, E, K, N
+    (1, 5000, 1, 600), (2, 3000, 4, 300), (1, 2000, 8, 250), (1, 1500, 3, 200), (1, 900, 64, 100),
+    (1, 700, 130, 80), (3, 400, 16, 50), (1, 1, 1, 1), (1, 257, 2, 300),
+]
+
+
+@pytest.mark.parametrize("shape,kind,dtype,unbiased",
+                         product(STD_SHAPES, ["random", "sorted", "hub"], DTYPES, [True, False]))
+def test_std_forward_and_backward_capi(capi, oracle, shape, kind, dtype, unbiased):
+    """fp32 / fp64 against the oracle's sequence in the same type. 16-bit floats against the
+    oracle in fp64 on the same inputs, within the roundings the reference's sequence commits in
+    the element type (deviation, square, sum, quotient, root: a few ulp of the result); no hub
+    groups there, whose sum in a 16-bit type the reference itself cannot hold."""
+    B, E, K, N = shape
+    exact = dtype in (torch.float32, torch.float64)
+    if kind == "hub" and not exact:
+        pytest.skip("a 16-bit group sum over hundreds of entries is not meaningful")
+    rng = np.random.default_rng(E * 17 + K)
+    src = torch.from_numpy(rng.standard_normal(size=(B, E, K)) * 3 + 1).to(dtype)
+    grad = torch.from_numpy(rng.standard_normal(size=(B, N, K))).to(dtype)
+    index1 = make_index(kind, rng, E, N)
+    index = index1.view(1, E, 1).expand(B, E, K)
+    src_d, idx_d = src.to(DEV), index1.to(DEV)
+    total = torch.empty((B, N, K), dtype=dtype, device=DEV)
+    capi.scatter(src_d, idx_d, total, None, B, E, K, N, 0, 1, 0, capi.SUM, False)
+    count = torch.empty((B, N), dtype=torch.float32, device=DEV)
+    capi.scatter_count(idx_d, count, B, E, N, 0, 1)
+    out = torch.empty((B, N, K), dtype=dtype, device=DEV)
+    capi.group_std(src_d, idx_d, total, count, out, B, E, K, N, 0, 1, unbiased)
+    torch.cuda.synchronize()
+    assert count.cpu().view(B, N)[0].tolist() == np.bincount(index1.numpy(), minlength=N).tolist()
+
+    ref_src = src if exact else src.double()
+    want = oracle.scatter_std(ref_src, index, 1, None, N, unbiased).double()
+    e = EPS_T[dtype]
+    err = (out.cpu().double() - want).abs()
+    cnt_n = count.cpu().double().view(B, N, 1).clamp(1).expand(B, N, K)
+    mean_abs = oracle.scatter(src.double().abs(), index, 1, None, N, "sum")[0] / cnt_n
+    if exact:
+        bound = e * want + (1e-6 if dtype == torch.float32 else 1e-12)
+    else:  # the mean carries the roundings of a sum in the element type; an offset of the mean adds to the std
+        bound = 8.0 * e * want + 2.0 * e * mean_abs * (1.0 + cnt_n.sqrt())
+    assert bool((err <= bound).all()), float((err - bound).max())
+
+    grad_in = torch.empty((B, E, K), dtype=dtype, device=DEV)
+    capi.group_std_backward(src_d, idx_d, total, count, out, grad.to(DEV), grad_in, B, E, K, N, 0, 1, unbiased)
+    torch.cuda.synchronize()
+    std64, want_g = oracle.scatter_std_backward(src.double(), grad.double(), index, 1, N, unbiased)
+    got_g = grad_in.cpu().double()
+    # a group whose std is 0 (one entry, or equal entries): NaN on both sides
+    dead = (std64 == 0).gather(1, index)
+    assert bool(torch.isnan(got_g[dead]).all()) and bool(torch.isnan(want_g[dead]).all())
+    live = ~dead & ~torch.isnan(want_g)
+    # the deviation src - mean cancels: its error is that of the mean, relative to the group's spread
+    scale = (grad.double().abs() / std64.clamp_min(1e-300)).gather(1, index)
+    cnt = cnt_n.gather(1, index)
+    gbound = (8 if exact else 16) * e * (want_g.abs() + scale * mean_abs.gather(1, index) / cnt)
+    gerr = (got_g - want_g).abs()
+    assert bool((gerr[live] <= gbound[live]).all()), float((gerr[live] - gbound[live]).max())
+
+
+@pytest.mark.parametrize("dim,unbiased", product([0, 1, 2, -1], [True, False]))
+def test_std_operator_dims_and_autograd(ts, oracle, dim, unbiased):
+    shape = (40, 30, 20)
+    g = torch.Generator().manual_seed(11)
+    d = dim if dim >= 0 else len(shape) + dim
+    src_cpu = torch.randn(shape, generator=g, dtype=torch.double) * 2 + 0.5
+    index = torch.randint(0, 6, (shape[d],), generator=g)
+    shape_g = list(shape)
+    shape_g[d] = 8  # two groups without entries
+    grad = torch.randn(shape_g, generator=g, dtype=torch.double)
+    want, want_g = oracle.scatter_std_backward(src_cpu, grad, index, d, 8, unbiased)
+    # torch's own std per group, where the group has more than one entry
+    for grp in range(6):
+        sel = (index == grp).nonzero().flatten()
+        if sel.numel() > 1:
+            lib = src_cpu.index_select(d, sel).std(d, unbiased=unbiased)
+            assert torch.allclose(want.select(d, grp), lib, rtol=1e-5)
+    src = src_cpu.to(DEV).requires_grad_(True)
+    shape1 = [1] * len(shape)
+    shape1[d] = shape[d]
+    for idx in (index.to(DEV), index.view(shape1).expand(shape).to(DEV)):
+        if idx.dim() == 1 and d != 0:
+            idx = idx.view(shape1[:d + 1])
+        src.grad = None
+        out = ts.scatter_std(src, idx, dim, dim_size=8, unbiased=unbiased)
+        out.backward(grad.to(DEV))
+        assert torch.allclose(out.detach().cpu(), want, rtol=1e-9, atol=1e-12)
+        assert float(out.detach().select(d, 7).abs().max()) == 0.0
+        assert torch.allclose(src.grad.cpu(), want_g, rtol=1e-7, atol=1e-9, equal_nan=True)
+
+
+def test_std_operator_reference_case_script_and_fallback(ts, oracle):
+    # test/composite/test_std.py:5-23
+    src = torch.tensor([[2.0, 0, 1, 4, 3], [0, 2, 1, 3, 4]], device=DEV, requires_grad=True)
+    index = torch.tensor([[0, 0, 0, 0, 0], [1, 1, 1, 1, 1]], device=DEV)
+    out = ts.scatter_std(src, index, dim=-1, unbiased=True)
+    std = src.std(dim=-1, unbiased=True)[0]
+    assert torch.allclose(out, torch.tensor([[std, 0], [0, std]], device=DEV))
+    out.backward(torch.randn_like(out))
+    jit = torch.jit.script(ts.scatter_std)
+    assert jit(src, index, dim=-1, unbiased=True).tolist() == out.tolist()
+    g = torch.Generator().manual_seed(2)
+    # an index that differs between the columns of a row, and `out` given: composed as upstream
+    x = torch.randn(60, 5, generator=g)
+    idx = torch.randint(0, 4, (60, 5), generator=g)
+    got = ts.scatter_std(x.to(DEV), idx.to(DEV), 0)
+    assert torch.allclose(got.cpu(), oracle.scatter_std(x, idx, 0), rtol=1e-5, atol=1e-6)
+    idx1 = torch.randint(0, 4, (60,), generator=g)
+    base = torch.rand(6, 5, generator=g)
+    got = ts.scatter_std(x.to(DEV), idx1.to(DEV), 0, out=base.clone().to(DEV), unbiased=False)
+    assert torch.allclose(got.cpu(), oracle.scatter_std(x, idx1, 0, base.clone(), None, False), rtol=1e-5, atol=1e-6)
+    # fused and composed agree (fp32, 1-D index along dim 0; last dim with a per-row index)
+    fused = ts.scatter_std(x.to(DEV), idx1.to(DEV), 0, dim_size=6)
+    assert torch.allclose(fused.cpu(), oracle.scatter_std(x, idx1, 0, None, 6), rtol=1e-5, atol=1e-6)
+    x = torch.randn(7, 90, generator=g)
+    idx = torch.randint(0, 9, (7, 90), generator=g)
+    got = ts.scatter_std(x.to(DEV), idx.to(DEV), -1)
+    assert torch.allclose(got.cpu(), oracle.scatter_std(x, idx, -1), rtol=1e-5, atol=1e-6)
+    # integer input goes through the composed sequence as upstream (count + 1e-6 promotes to float)
+    xi = torch.randint(0, 9, (50,), generator=g)
+    ii = torch.randint(0, 5, (50,), generator=g)
+    got = ts.scatter_std(xi.to(DEV), ii.to(DEV), 0)
+    assert torch.allclose(got.cpu(), oracle.scatter_std(xi, ii, 0), rtol=1e-5, atol=1e-6)
+    # zero-size input
+    assert ts.scatter_std(torch.empty(0, 4, device=DEV), torch.empty(0, dtype=torch.long, device=DEV), 0,
+                          dim_size=3).shape == (3, 4)

@@ -107,3 +107,23 @@ def test_logsumexp_backward_closed_form(oracle):
     y = oracle.scatter_logsumexp(src.detach(), index, 0, None, 9)
     got = oracle.scatter_logsumexp_backward(src.detach(), y, grad, index, 0)
     assert torch.allclose(got, src.grad, rtol=1e-9, atol=1e-12)
+
+
+@pytest.mark.parametrize("unbiased", [True, False])
+def test_std_backward_against_library_std(oracle, unbiased):
+    """The gradient the oracle derives for scatter_std is that of torch's own std taken
+    group by group (up to the 1e-6 in the divisor); a one-entry group gives NaN."""
+    g = torch.Generator().manual_seed(9)
+    src = torch.randn(150, 4, generator=g, dtype=torch.double) * 2 + 1
+    index = torch.randint(0, 7, (150,), generator=g)
+    index[0] = 7  # a group of one entry
+    grad = torch.randn(9, 4, generator=g, dtype=torch.double)
+    std, got = oracle.scatter_std_backward(src, grad, index, 0, 9, unbiased)
+    assert torch.equal(std, oracle.scatter_std(src, index.view(-1, 1).expand(150, 4), 0, None, 9, unbiased))
+    ref = src.clone().requires_grad_(True)
+    total = sum((ref.index_select(0, sel).std(0, unbiased=unbiased) * grad[grp]).sum()
+                for grp, sel in enumerate(_groups(index, 9)) if sel.numel() > 1)
+    total.backward()
+    keep = index != 7
+    assert torch.allclose(got[keep], ref.grad[keep], rtol=1e-5, atol=1e-9)
+    assert bool(torch.isnan(got[~keep]).all())
