@@ -253,6 +253,47 @@ int ts_group_std_backward(const void *src, const int64_t *index,
                           int64_t index_stride_b, int64_t index_stride_e,
                           int dtype, int unbiased, ts_stream_t stream);
 
+/* ---- index formats either side of the reductions. The reference has no operator for these steps:
+ * its benchmark takes `row` and `rowptr` from the same sparse matrix (benchmark/scatter_segment.py:38-41)
+ * and segment_coo's documentation asks the caller for a sorted index (torch_scatter/segment_coo.py:80-83).
+ */
+
+/* Sorted index [B, E] -> row pointers [B, N+1]: indptr[b, r] = first e with index[b, e] >= r. */
+int ts_index_to_indptr(const int64_t *index, int64_t *indptr, int64_t B, int64_t E,
+                       int64_t N, int64_t index_batch_stride, ts_stream_t stream);
+
+/* Row pointers [B, N+1] -> sorted index [B, E] (E = indptr[b, N]): index[b, e] = r for
+ * e in [indptr[b, r], indptr[b, r+1]). */
+size_t ts_indptr_to_index_workspace_bytes(int64_t B, int64_t N);
+int ts_indptr_to_index(const int64_t *indptr, int64_t *index, int64_t B, int64_t N,
+                       int64_t E, int64_t indptr_batch_stride, void *workspace,
+                       size_t workspace_bytes, ts_stream_t stream);
+
+/* One-time stable sort of an unsorted index [E] with values in [0, N):
+ *   perm[E] (int32): index[perm[0]] <= index[perm[1]] <= ..., equal values in order of position;
+ *   indptr[N+1]: row pointers of the sorted order.
+ * An index outside [0, N) sorts behind the last row: indptr[N] < E then tells the caller.
+ * E, N < 2^31 - 1. */
+size_t ts_sort_index_workspace_bytes(int64_t E, int64_t N);
+int ts_sort_index(const int64_t *index, int32_t *perm, int64_t *indptr, int64_t E,
+                  int64_t N, void *workspace, size_t workspace_bytes, ts_stream_t stream);
+
+/* ts_segment_csr over permuted rows: entry e of the row-pointer order is row perm[b, e] of src,
+ *   out[b, n, k] = reduce over e in [indptr[b, n], indptr[b, n+1]) of src[b, perm[b, e], k].
+ * With perm / indptr from ts_sort_index this is scatter (csrc/cuda/scatter_cuda.cu:54-138) for an
+ * index that is used many times: one pass over src, no atomics, the same bits on every call.
+ * arg_out (MIN / MAX) holds positions in src's order (perm applied); ties keep the smallest position
+ * as perm is stable. A slot without entries, or whose entries never beat scatter's initial value
+ * (lowest() / max() of the element type), reads 0 with position E (csrc/cpu/scatter_cpu.cpp:81-82).
+ * perm_batch_stride: 0 (one perm for all b) or E. */
+size_t ts_segment_csr_permuted_workspace_bytes(int64_t B, int64_t N, int64_t E, int64_t K,
+                                               int dtype, int reduce);
+int ts_segment_csr_permuted(const void *src, const int32_t *perm, const int64_t *indptr,
+                            void *out, int64_t *arg_out, int64_t B, int64_t N, int64_t E,
+                            int64_t K, int64_t perm_batch_stride,
+                            int64_t indptr_batch_stride, int dtype, int reduce,
+                            void *workspace, size_t workspace_bytes, ts_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

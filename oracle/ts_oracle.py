@@ -479,3 +479,36 @@ def scatter_logsumexp_backward(src, result, grad_out, index, dim=-1):
     w = (src - result.gather(dim, index)).exp()
     w = torch.where(torch.isnan(w), torch.zeros_like(w), w)
     return grad_out.gather(dim, index) * w
+
+
+# ---- index formats. The reference has no routine for these steps (its benchmark reads
+# row and rowptr from the same scipy matrix, benchmark/scatter_segment.py:38-41); the
+# definitions are restated with plain loops so that tests can pin them against
+# numpy / scipy library routines.
+def index_to_indptr(index, dim_size):
+    """indptr[r] = number of entries with index < r (1-D sorted index)."""
+    ptr = [0] * (dim_size + 1)
+    for v in index.tolist():
+        for r in range(max(v + 1, 0), dim_size + 1):
+            ptr[r] += 1
+    return torch.tensor(ptr, dtype=torch.long)
+
+
+def indptr_to_index(indptr):
+    out = []
+    p = indptr.tolist()
+    for r in range(len(p) - 1):
+        out.extend([r] * (p[r + 1] - p[r]))
+    return torch.tensor(out, dtype=torch.long)
+
+
+def sort_index(index, dim_size):
+    """Stable counting sort: (perm, indptr)."""
+    buckets = [[] for _ in range(dim_size)]
+    for e, v in enumerate(index.tolist()):
+        buckets[v].append(e)
+    perm, ptr = [], [0]
+    for b in buckets:
+        perm.extend(b)
+        ptr.append(len(perm))
+    return torch.tensor(perm, dtype=torch.long), torch.tensor(ptr, dtype=torch.long)

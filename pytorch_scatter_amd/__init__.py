@@ -41,6 +41,8 @@ from .segment_csr import (gather_csr, segment_add_csr, segment_csr,  # noqa: E40
                           segment_sum_csr)
 from .composite import (scatter_log_softmax, scatter_logsumexp,  # noqa: E402
                         scatter_softmax, scatter_std)
+from .index_format import (SortedIndex, index_to_indptr, indptr_to_index,  # noqa: E402
+                           scatter_sorted)
 
 __all__ = [
     "scatter_sum", "scatter_add", "scatter_mul", "scatter_mean", "scatter_min",
@@ -50,5 +52,6 @@ __all__ = [
     "segment_sum_coo", "segment_add_coo", "segment_mean_coo", "segment_min_coo",
     "segment_max_coo", "segment_coo", "gather_coo",
     "scatter_std", "scatter_logsumexp", "scatter_softmax", "scatter_log_softmax",
+    "SortedIndex", "index_to_indptr", "indptr_to_index", "scatter_sorted",
     "hip_version", "__version__",
 ]

@@ -30,6 +30,9 @@ EXPORTS = (
     "ts_group_softmax_workspace_bytes", "ts_group_softmax", "ts_group_softmax_backward",
     "ts_group_logsumexp", "ts_group_logsumexp_backward",
     "ts_group_std", "ts_group_std_backward",
+    "ts_index_to_indptr", "ts_indptr_to_index_workspace_bytes", "ts_indptr_to_index",
+    "ts_sort_index_workspace_bytes", "ts_sort_index",
+    "ts_segment_csr_permuted_workspace_bytes", "ts_segment_csr_permuted",
 )
 
 _lib = None
@@ -52,6 +55,9 @@ def lib() -> ctypes.CDLL:
         _lib.ts_segment_csr_workspace_bytes.restype = ctypes.c_size_t
         _lib.ts_segment_coo_workspace_bytes.restype = ctypes.c_size_t
         _lib.ts_group_softmax_workspace_bytes.restype = ctypes.c_size_t
+        _lib.ts_indptr_to_index_workspace_bytes.restype = ctypes.c_size_t
+        _lib.ts_sort_index_workspace_bytes.restype = ctypes.c_size_t
+        _lib.ts_segment_csr_permuted_workspace_bytes.restype = ctypes.c_size_t
     return _lib
 
 
@@ -226,3 +232,45 @@ def group_std_backward(src, index, total, count, out, grad_out, grad_in, B, E, K
         _check(lib().ts_group_std_backward(_p(src), _p(index), _p(total), _p(count), _p(out), _p(grad_out),
                                            _p(grad_in), _i(B), _i(E), _i(K), _i(N), _i(sb), _i(se),
                                            DTYPE[grad_in.dtype], int(unbiased), _stream(grad_in)))
+
+
+def index_to_indptr(index, indptr, B, E, N, index_batch_stride):
+    _dev(index, indptr)
+    with torch.cuda.device(indptr.device):
+        _check(lib().ts_index_to_indptr(_p(index), _p(indptr), _i(B), _i(E), _i(N), _i(index_batch_stride),
+                                        _stream(indptr)))
+
+
+def indptr_to_index(indptr, index, B, N, E, indptr_batch_stride):
+    _dev(indptr, index)
+    L = lib()
+    nbytes = L.ts_indptr_to_index_workspace_bytes(_i(B), _i(N))
+    ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=index.device)
+    with torch.cuda.device(index.device):
+        _check(L.ts_indptr_to_index(_p(indptr), _p(index), _i(B), _i(N), _i(E), _i(indptr_batch_stride), _p(ws),
+                                    ctypes.c_size_t(nbytes), _stream(index)))
+    return ws
+
+
+def sort_index(index, perm, indptr, E, N):
+    _dev(index, perm, indptr)
+    L = lib()
+    with torch.cuda.device(indptr.device):
+        nbytes = L.ts_sort_index_workspace_bytes(_i(E), _i(N))
+        ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=indptr.device)
+        _check(L.ts_sort_index(_p(index), _p(perm), _p(indptr), _i(E), _i(N), _p(ws), ctypes.c_size_t(nbytes),
+                               _stream(indptr)))
+    return ws
+
+
+def segment_csr_permuted(src, perm, indptr, out, arg_out, B, N, E, K, perm_batch_stride, indptr_batch_stride,
+                         reduce: int):
+    _dev(src, perm, indptr, out, arg_out)
+    L = lib()
+    nbytes = L.ts_segment_csr_permuted_workspace_bytes(_i(B), _i(N), _i(E), _i(K), DTYPE[out.dtype], reduce)
+    ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=out.device)
+    with torch.cuda.device(out.device):
+        _check(L.ts_segment_csr_permuted(_p(src), _p(perm), _p(indptr), _p(out), _p(arg_out), _i(B), _i(N), _i(E),
+                                         _i(K), _i(perm_batch_stride), _i(indptr_batch_stride), DTYPE[out.dtype],
+                                         reduce, _p(ws), ctypes.c_size_t(nbytes), _stream(out)))
+    return ws

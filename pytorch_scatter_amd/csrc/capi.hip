@@ -13,6 +13,7 @@
 #include "scatter.h"
 #include "elementwise.h"
 #include "group_softmax.h"
+#include "index_format.h"
 
 using namespace ts;
 
@@ -56,6 +57,10 @@ int dispatch_scatter(int dtype, const ScatterArgs &a, int reduce, int vec, hipSt
 }
 int dispatch_divide(int dtype, void *out, const float *count, int64_t rows, int64_t K, hipStream_t s) {
   TS_DISPATCH(dtype, launch_divide_by_count<T>(out, count, rows, K, s))
+}
+int dispatch_sorted_args(int dtype, void *out, int64_t *arg, const int32_t *perm, int64_t B, int64_t per_batch,
+                         int64_t E, int64_t perm_batch_stride, bool is_max, hipStream_t s) {
+  TS_DISPATCH(dtype, launch_sorted_args<T>(out, arg, perm, B, per_batch, E, perm_batch_stride, is_max, s))
 }
 int dispatch_arg_backward(int dtype, const void *g, const int64_t *arg, void *gi, int64_t B, int64_t N,
                           int64_t E, int64_t K, hipStream_t s) {
@@ -111,9 +116,12 @@ size_t csr_workspace_max(int64_t B, int64_t N, int64_t E, int64_t K, int dtype, 
 
 int run_csr_reduce(const void *src, const int64_t *indptr, void *out, int64_t *arg_out, void *count_out,
                    int64_t B, int64_t N, int64_t E, int64_t K, int64_t indptr_batch_stride, int dtype,
-                   int reduce, int accumulate, void *ws, size_t ws_bytes, hipStream_t stream) {
+                   int reduce, int accumulate, void *ws, size_t ws_bytes, hipStream_t stream,
+                   const int32_t *perm = nullptr, int64_t perm_batch_stride = 0) {
   const bool al = aligned16(src) && aligned16(out);
-  const CsrPlan p = csr_plan(N, E, K, kElemBytes[dtype], al, false, reduce == TS_MIN || reduce == TS_MAX);
+  // permuted rows always take the wide kernel (the narrow one stages consecutive entries)
+  const CsrPlan p = csr_plan(N, E, K, kElemBytes[dtype], al, false, reduce == TS_MIN || reduce == TS_MAX,
+                             perm == nullptr);
   const CsrWs w = csr_workspace(p, B, K, dtype, reduce);
   if (ws == nullptr || ws_bytes < w.total) return TS_ERR_WORKSPACE;
   CsrReduceArgs a;
@@ -138,6 +146,8 @@ int run_csr_reduce(const void *src, const int64_t *indptr, void *out, int64_t *a
   // four words of workspace per tile give every column chunk its flag; else by the second kernel
   a.lookback = !p.small && kAccBytes[dtype] >= 4 && p.ychunks <= 4 && p.nblk > 1 && env_int("TS_CSR_LOOKBACK", 1);
   a.nonce = next_nonce();
+  a.perm = perm;
+  a.perm_batch_stride = perm_batch_stride;
   return dispatch_csr_reduce(dtype, a, p, B, reduce, stream);
 }
 
@@ -220,6 +230,31 @@ int ts_segment_mean_csr_backward(const void *grad_out, const int64_t *indptr, vo
   a.ipw = p.ipw;
   a.nblk = p.nblk;
   return dispatch_csr_gather(dtype, a, p, B, true, static_cast<hipStream_t>(stream));
+}
+
+size_t ts_segment_csr_permuted_workspace_bytes(int64_t B, int64_t N, int64_t E, int64_t K, int dtype, int reduce) {
+  if (!valid_dtype(dtype) || !sizes_ok(B, N, E, K)) return 0;
+  const bool wa = reduce == TS_MIN || reduce == TS_MAX;
+  const size_t w1 = csr_workspace(csr_plan(N, E, K, kElemBytes[dtype], true, false, wa, false), B, K, dtype, reduce).total;
+  const size_t w0 = csr_workspace(csr_plan(N, E, K, kElemBytes[dtype], false, false, wa, false), B, K, dtype, reduce).total;
+  return w1 > w0 ? w1 : w0;
+}
+
+int ts_segment_csr_permuted(const void *src, const int32_t *perm, const int64_t *indptr, void *out,
+                            int64_t *arg_out, int64_t B, int64_t N, int64_t E, int64_t K,
+                            int64_t perm_batch_stride, int64_t indptr_batch_stride, int dtype, int reduce,
+                            void *workspace, size_t workspace_bytes, ts_stream_t stream) {
+  if (!valid_dtype(dtype) || !sizes_ok(B, N, E, K)) return TS_ERR_BAD_ARG;
+  if (reduce != TS_SUM && reduce != TS_MEAN && reduce != TS_MIN && reduce != TS_MAX) return TS_ERR_UNSUPPORTED;
+  if (E >= 0x7FFFFFFFll) return TS_ERR_UNSUPPORTED;  // 32-bit row numbers
+  if (B * N * K == 0) return TS_OK;
+  if (!indptr || !out || (E * K > 0 && (!src || !perm))) return TS_ERR_BAD_ARG;
+  if ((reduce == TS_MIN || reduce == TS_MAX) && !arg_out) return TS_ERR_BAD_ARG;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int rc = run_csr_reduce(src, indptr, out, arg_out, nullptr, B, N, E, K, indptr_batch_stride, dtype, reduce,
+                                0, workspace, workspace_bytes, s, perm, perm_batch_stride);
+  if (rc != TS_OK || (reduce != TS_MIN && reduce != TS_MAX)) return rc;
+  return dispatch_sorted_args(dtype, out, arg_out, perm, B, N * K, E, perm_batch_stride, reduce == TS_MAX, s);
 }
 
 size_t ts_segment_coo_workspace_bytes(int64_t B, int64_t N, int64_t E, int64_t K, int dtype, int reduce) {
@@ -554,6 +589,73 @@ int ts_group_std_backward(const void *src, const int64_t *index, const void *tot
   const bool al = aligned16(src) && aligned16(grad_in) && aligned16(out) && aligned16(grad_out) && aligned16(total);
   const int vec = (full > 1 && K % full == 0 && al) ? full : 1;
   return dispatch_group_softmax(dtype, g, GS_STD_BWD, vec, static_cast<hipStream_t>(stream));
+}
+
+// ---- index formats
+int ts_index_to_indptr(const int64_t *index, int64_t *indptr, int64_t B, int64_t E, int64_t N,
+                       int64_t index_batch_stride, ts_stream_t stream) {
+  if (B < 0 || E < 0 || N < 0) return TS_ERR_BAD_ARG;
+  if (B == 0) return TS_OK;
+  if (!indptr || (E > 0 && !index)) return TS_ERR_BAD_ARG;
+  const int64_t per_block = (int64_t)kBlock * kCooPtrPerThread;
+  dim3 grid((unsigned)((E + 1 + per_block - 1) / per_block), (unsigned)B);
+  hipLaunchKernelGGL(coo_to_indptr_kernel, grid, dim3(kBlock), 0, static_cast<hipStream_t>(stream), index, indptr, N,
+                     E, index_batch_stride);
+  return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
+}
+
+size_t ts_indptr_to_index_workspace_bytes(int64_t B, int64_t N) {
+  return B < 0 || N < 0 ? 0 : ((size_t)B * N * 8 + 255) & ~(size_t)255;
+}
+
+int ts_indptr_to_index(const int64_t *indptr, int64_t *index, int64_t B, int64_t N, int64_t E,
+                       int64_t indptr_batch_stride, void *workspace, size_t workspace_bytes, ts_stream_t stream) {
+  if (!sizes_ok(B, N, E, 1)) return TS_ERR_BAD_ARG;
+  if (B * E == 0 || N == 0) return TS_OK;
+  if (!indptr || !index) return TS_ERR_BAD_ARG;
+  if (!workspace || workspace_bytes < ts_indptr_to_index_workspace_bytes(B, N) || !aligned16(workspace))
+    return TS_ERR_WORKSPACE;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  // the row numbers 0 .. N-1 of every batch, expanded along the row pointers like any other source
+  int64_t *rows = static_cast<int64_t *>(workspace);
+  hipLaunchKernelGGL(row_numbers_kernel, dim3(index_grid(B * N)), dim3(kBlock), 0, s, rows, B * N, N);
+  if (hipGetLastError() != hipSuccess) return TS_ERR_LAUNCH;
+  return ts_gather_csr(rows, indptr, index, B, N, E, 1, indptr_batch_stride, TS_I64, stream);
+}
+
+static int sort_key_bits(int64_t N) {  // keys are 0 .. N (N: an index outside [0, N))
+  int bits = 1;
+  while (bits < 32 && ((int64_t)1 << bits) <= N) ++bits;
+  return bits;
+}
+static size_t sort_keys_bytes(int64_t E) { return ((size_t)E * 4 + 255) & ~(size_t)255; }
+
+size_t ts_sort_index_workspace_bytes(int64_t E, int64_t N) {
+  if (E < 0 || N < 0 || E >= 0x7FFFFFFFll || N >= 0x7FFFFFFFll) return 0;
+  return 2 * sort_keys_bytes(E) + ((sort_keys_temp_bytes(E, sort_key_bits(N)) + 255) & ~(size_t)255);
+}
+
+int ts_sort_index(const int64_t *index, int32_t *perm, int64_t *indptr, int64_t E, int64_t N, void *workspace,
+                  size_t workspace_bytes, ts_stream_t stream) {
+  if (E < 0 || N < 0) return TS_ERR_BAD_ARG;
+  if (E >= 0x7FFFFFFFll || N >= 0x7FFFFFFFll) return TS_ERR_UNSUPPORTED;
+  if (!indptr || (E > 0 && (!index || !perm))) return TS_ERR_BAD_ARG;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const size_t kb = sort_keys_bytes(E);
+  uint32_t *keys_in = static_cast<uint32_t *>(workspace);
+  uint32_t *keys_out = reinterpret_cast<uint32_t *>(static_cast<char *>(workspace) + kb);
+  if (E > 0) {
+    const int bits = sort_key_bits(N);
+    const size_t temp = sort_keys_temp_bytes(E, bits);
+    if (!workspace || !aligned16(workspace) || workspace_bytes < 2 * kb + temp) return TS_ERR_WORKSPACE;
+    hipLaunchKernelGGL(index_keys_kernel, dim3(index_grid(E)), dim3(kBlock), 0, s, index, keys_in, E, N);
+    if (hipGetLastError() != hipSuccess) return TS_ERR_LAUNCH;
+    const int rc = sort_keys_to_perm(static_cast<char *>(workspace) + 2 * kb, temp, keys_in, keys_out, perm, E, bits, s);
+    if (rc != TS_OK) return rc;
+  }
+  hipLaunchKernelGGL(keys_to_indptr_kernel, dim3((unsigned)((E + 1 + kBlock - 1) / kBlock)), dim3(kBlock), 0, s,
+                     keys_out, indptr, N, E);
+  return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
 }
 
 }  // extern "C"

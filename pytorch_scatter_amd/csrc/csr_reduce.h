@@ -28,6 +28,7 @@ constexpr int kMaxBlockItems = 2048;  // rows + edges per workgroup tile
 #ifndef TS_CSR_U
 #define TS_CSR_U 4
 #endif
+constexpr int kSharedWalkMin = 32;  // tiles a row must have passed through before the workgroup shares the walk
 constexpr int kLoadsInFlight = TS_CSR_U;  // U: 16-byte loads per lane per batch (two batches in flight)
 
 struct CsrReduceArgs {
@@ -50,6 +51,10 @@ struct CsrReduceArgs {
                       // (look-back mode: one carry flag per column chunk instead)
   int lookback;       // rows that cross tiles are finished inside the kernel (see carry_* below)
   uint64_t nonce;     // tag of this call's carry flags, never 0
+  // optional: entry e of the row-pointer order lives in row perm[e] of src (a scatter whose index was
+  // sorted once: perm = stable argsort of the index). Positions handed to arg_out stay in row-pointer order.
+  const int32_t *perm;
+  int64_t perm_batch_stride;
 };
 
 // ---- rows that cross tiles, finished without a second kernel ---------------------------------
@@ -156,16 +161,17 @@ __device__ __forceinline__ void finalize_row(const CsrReduceArgs &a, T *out_b, i
 // Workgroups per CU the register allocation aims at: six for sum / mean of 4- and 8-byte types (80 VGPRs;
 // mean would take 82 and drop to five, measured 7 % slower on 146 MB inputs). The other instantiations keep
 // the compiler's choice (forcing five on the 16-bit mean cost 3 % on 16 GB inputs).
-template <typename T, int VEC, int REDUCE> constexpr int csr_reduce_min_blocks() {
-  return (REDUCE == TS_SUM || REDUCE == TS_MEAN) && sizeof(T) >= 4 ? 6 : 1;
+template <typename T, int VEC, int REDUCE, bool PERM = false> constexpr int csr_reduce_min_blocks() {
+  return PERM ? 1 : ((REDUCE == TS_SUM || REDUCE == TS_MEAN) && sizeof(T) >= 4 ? 6 : 1);  // PERM: 8 KB more LDS
 }
-template <typename T, int VEC, int REDUCE, int ACCUM>
-__global__ __launch_bounds__(kBlock, (csr_reduce_min_blocks<T, VEC, REDUCE>())) void csr_reduce_kernel(CsrReduceArgs a) {
+template <typename T, int VEC, int REDUCE, int ACCUM, bool PERM = false>
+__global__ __launch_bounds__(kBlock, (csr_reduce_min_blocks<T, VEC, REDUCE, PERM>())) void csr_reduce_kernel(CsrReduceArgs a) {
   typedef typename Acc<T>::type A;
   constexpr bool kArg = (REDUCE == TS_MIN || REDUCE == TS_MAX);
   constexpr int U = kLoadsInFlight;
 
   __shared__ int32_t s_ptr[kMaxBlockItems + 4];  // row pointers of the tile + one sentinel
+  __shared__ int32_t s_perm[PERM ? kMaxBlockItems : 1];  // source rows of the tile's entries
   __shared__ A s_val[2 * kBlock * VEC];
   __shared__ int32_t s_arg[kArg ? 2 * kBlock * VEC : 1];
   __shared__ int32_t s_head_row[kBlock];    // local row of the head partial, -1: none
@@ -209,6 +215,10 @@ __global__ __launch_bounds__(kBlock, (csr_reduce_min_blocks<T, VEC, REDUCE>())) 
   const int nload = (int)(last - i0) + 1;  // ptr[i0 .. last]
   for (int t = tid; t < nload; t += kBlock) s_ptr[t] = (int32_t)(ptr[i0 + t] - j0);
   if (tid == 0) { s_ptr[nload] = INT32_MAX; s_ptr[nload + 1] = INT32_MAX; }  // rows past the last one never end
+  if constexpr (PERM) {
+    const int32_t *perm_b = a.perm + b * a.perm_batch_stride + j0;
+    for (int t = tid; t < ne; t += kBlock) s_perm[t] = perm_b[t];
+  }
   s_head_row[tid] = -1;
   s_tail_row[tid] = -1;
   __syncthreads();
@@ -280,7 +290,8 @@ __global__ __launch_bounds__(kBlock, (csr_reduce_min_blocks<T, VEC, REDUCE>())) 
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       int ee = e + u < je1 ? e + u : je1 - 1;
-      x[u] = load_vec_stream<T, VEC>(src_col + (j0 + ee) * a.K);
+      const int64_t srow = PERM ? (int64_t)s_perm[ee] : j0 + ee;
+      x[u] = load_vec_stream<T, VEC>(src_col + srow * a.K);
     }
   };
   Vec<T, VEC> x[U];
@@ -329,6 +340,7 @@ __global__ __launch_bounds__(kBlock, (csr_reduce_min_blocks<T, VEC, REDUCE>())) 
   const bool lookback = kCarryOk && a.lookback != 0;
   // default: the tile leaves no open row; the worker that does overwrites this after the barrier
   if (!lookback && tid == 0 && blockIdx.y == 0) a.ws_meta[(b * a.nblk + blockIdx.x) * 4 + 2] = -1;
+  if (PERM && tid == 0) s_cut[0] = -1;  // becomes the first tile of a walk that the workgroup shares
   __syncthreads();
 
   // ---- combine partials of rows that cross worker boundaries, in edge order
@@ -358,15 +370,18 @@ __global__ __launch_bounds__(kBlock, (csr_reduce_min_blocks<T, VEC, REDUCE>())) 
   // in front. first_tile is the tile in which the row began (from its row pointer), so the tiles to visit
   // are known in advance and are polled and read several at a time: a hub row that passes through hundreds
   // of tiles costs a few memory round trips per batch, not per tile.
-  auto walk_back = [&](int64_t first_tile) {
+  // (start, stride): the tiles start, start - stride, ... down to first_tile; one worker walking alone takes
+  // (blockIdx.x - 1, 1), the workers of a workgroup that share a long walk take every W-th tile each.
+  auto walk_back = [&](int64_t first_tile, int64_t start, int64_t stride) {
     if constexpr (kCarryOk) {
     constexpr int PF = VEC <= 4 ? 4 : 2;
     A *vals_b = static_cast<A *>(a.ws_vals) + (b * a.nblk) * 2 * a.K;
     int32_t *args_b = kArg ? a.ws_args + (b * a.nblk) * 2 * a.K : nullptr;
     const int64_t c = col_ok ? col : 0;
     if (first_tile < 0) first_tile = 0;
-    for (int64_t hi = (int64_t)blockIdx.x - 1; hi >= first_tile; hi -= PF) {
-      const int n = hi - first_tile + 1 < PF ? (int)(hi - first_tile + 1) : PF;  // tiles hi, hi - 1, ...
+    for (int64_t hi = start; hi >= first_tile; hi -= PF * stride) {
+      const int64_t left = (hi - first_tile) / stride + 1;
+      const int n = left < PF ? (int)left : PF;  // tiles hi, hi - stride, ...
       bool ready[PF];
 #pragma unroll
       for (int q = 0; q < PF; ++q) ready[q] = q >= n;
@@ -375,7 +390,7 @@ __global__ __launch_bounds__(kBlock, (csr_reduce_min_blocks<T, VEC, REDUCE>())) 
         uint64_t f[PF];
 #pragma unroll
         for (int q = 0; q < PF; ++q)
-          f[q] = ready[q] ? 0 : __hip_atomic_fetch_or(carry_flags + (hi - q) * 4, 0ull, __ATOMIC_RELAXED,
+          f[q] = ready[q] ? 0 : __hip_atomic_fetch_or(carry_flags + (hi - q * stride) * 4, 0ull, __ATOMIC_RELAXED,
                                                        __HIP_MEMORY_SCOPE_AGENT);
         bool all = true;
 #pragma unroll
@@ -395,8 +410,8 @@ __global__ __launch_bounds__(kBlock, (csr_reduce_min_blocks<T, VEC, REDUCE>())) 
         if (q < n) {
 #pragma unroll
           for (int v = 0; v < VEC; ++v) {
-            early[q][v] = carry_get<A>(vals_b + ((hi - q) * 2 + 1) * a.K + c + v);
-            if (kArg) early_arg[q][v] = carry_get<int32_t>(args_b + ((hi - q) * 2 + 1) * a.K + c + v);
+            early[q][v] = carry_get<A>(vals_b + ((hi - q * stride) * 2 + 1) * a.K + c + v);
+            if (kArg) early_arg[q][v] = carry_get<int32_t>(args_b + ((hi - q * stride) * 2 + 1) * a.K + c + v);
           }
         }
       }
@@ -419,7 +434,8 @@ __global__ __launch_bounds__(kBlock, (csr_reduce_min_blocks<T, VEC, REDUCE>())) 
       if (lg == 0) {
 #pragma unroll
         for (int q = 0; q < PF; ++q)
-          if (q < n) __hip_atomic_exchange(carry_flags + (hi - q) * 4, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          if (q < n)
+            __hip_atomic_exchange(carry_flags + (hi - q * stride) * 4, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
     }
     }
@@ -482,26 +498,73 @@ __global__ __launch_bounds__(kBlock, (csr_reduce_min_blocks<T, VEC, REDUCE>())) 
         if (closed) {
           const int row = s_head_row[0];
           // the row's first entry sits at merge position (row index + row pointer)
-          walk_back(((i0 + row) + ((int64_t)s_ptr[row] + j0)) / a.BI);
-          finalize_row<T, VEC, REDUCE, ACCUM>(a, out_b, arg_b, count_b, i0 + row, col, lg, acc, arg,
-                                              (int64_t)s_ptr[row + 1] - (int64_t)s_ptr[row], col_ok);
+          int64_t first_tile = ((i0 + row) + ((int64_t)s_ptr[row] + j0)) / a.BI;
+          if (first_tile < 0) first_tile = 0;
+          if (PERM && (int64_t)blockIdx.x - first_tile > kSharedWalkMin) {
+            // a hub row that passed through many tiles: the whole workgroup walks (below)
+#pragma unroll
+            for (int v = 0; v < VEC; ++v) { my_tail_val[v] = acc[v]; if (kArg) my_tail_arg[v] = arg[v]; }
+            if (lg == 0) s_cut[0] = first_tile;
+          } else {
+            walk_back(first_tile, (int64_t)blockIdx.x - 1, 1);
+            finalize_row<T, VEC, REDUCE, ACCUM>(a, out_b, arg_b, count_b, i0 + row, col, lg, acc, arg,
+                                                (int64_t)s_ptr[row + 1] - (int64_t)s_ptr[row], col_ok);
+          }
         } else {
           publish_carry(kCarryPass);
         }
-        return;
-      }
-      if (col_ok) {
+      } else {
+        if (col_ok) {
 #pragma unroll
-        for (int v = 0; v < VEC; ++v) {
-          ws_val_blk[col + v] = acc[v];
-          if (kArg) ws_arg_blk[col + v] = arg[v];
+          for (int v = 0; v < VEC; ++v) {
+            ws_val_blk[col + v] = acc[v];
+            if (kArg) ws_arg_blk[col + v] = arg[v];
+          }
         }
+        if (lg == 0 && blockIdx.y == 0) { meta[0] = i0 + s_head_row[0]; meta[1] = closed ? 1 : 0; }
       }
-      if (lg == 0 && blockIdx.y == 0) { meta[0] = i0 + s_head_row[0]; meta[1] = closed ? 1 : 0; }
     } else if (!lookback && lg == 0 && blockIdx.y == 0) {
       meta[0] = -1;
       meta[1] = 0;
     }
+  }
+
+  // ---- a long walk shared by the workgroup: worker w collects the carries of the tiles
+  // blockIdx.x - 1 - w, - W, ... into a partial of its own; worker 0 then folds the partials in worker order.
+  // The grouping is fixed by the tiling, so the result is the same on every call.
+  if constexpr (PERM && kCarryOk) {
+    if (!lookback) return;
+    __syncthreads();
+    const int64_t first_tile = s_cut[0];
+    if (first_tile < 0) return;
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) { acc[v] = acc_init<A, REDUCE>(); arg[v] = INT32_MAX; }
+    walk_back(first_tile, (int64_t)blockIdx.x - 1 - w, W);
+    A *part_val = s_val + (size_t)w * CW + lg * VEC;  // the head slots: read for the last time before the barrier
+    int32_t *part_arg = s_arg + (kArg ? (size_t)w * CW + lg * VEC : 0);
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) { part_val[v] = acc[v]; if (kArg) part_arg[v] = arg[v]; }
+    __syncthreads();
+    if (w != 0) return;
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) { acc[v] = my_tail_val[v]; if (kArg) arg[v] = my_tail_arg[v]; }
+    for (int ww = 0; ww < W; ++ww) {
+      const A *pv = s_val + (size_t)ww * CW + lg * VEC;
+      const int32_t *pa = s_arg + (kArg ? (size_t)ww * CW + lg * VEC : 0);
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) {
+        if (kArg) {
+          // any order: the better value, on ties the smaller position
+          const bool better = (REDUCE == TS_MIN) ? (pv[v] < acc[v]) : (pv[v] > acc[v]);
+          if (better || (pv[v] == acc[v] && pa[v] < arg[v])) { acc[v] = pv[v]; arg[v] = pa[v]; }
+        } else {
+          acc[v] = pv[v] + acc[v];
+        }
+      }
+    }
+    const int row = s_head_row[0];
+    finalize_row<T, VEC, REDUCE, ACCUM>(a, out_b, arg_b, count_b, i0 + row, col, lg, acc, arg,
+                                        (int64_t)s_ptr[row + 1] - (int64_t)s_ptr[row], col_ok);
   }
 }
 
@@ -627,13 +690,13 @@ struct CsrPlan {
 
 // with_arg: the reduction is min / max (positions carried along); for the expansion: the variant that divides
 inline CsrPlan csr_plan(int64_t N, int64_t E, int64_t K, int elem_bytes, bool aligned16, bool expand = false,
-                        bool with_arg = false) {
+                        bool with_arg = false, bool allow_small = true) {
   CsrPlan p;
   p.small = false;
   // narrow rows: always for the reduction; for the expansion when a row is at most 8 bytes or
   // consists of whole, aligned 16-byte granules (other widths do better with the wide kernel)
   const bool granules = aligned16 && (K * elem_bytes) % kVecBytes == 0;
-  if (csr_small_ok(K, elem_bytes) && (!expand || K * elem_bytes <= 8 || granules)) {
+  if (allow_small && csr_small_ok(K, elem_bytes) && (!expand || K * elem_bytes <= 8 || granules)) {
     p.small = true;
     p.vec = (expand && granules) ? kVecBytes / elem_bytes : 1;
     p.G = 1;
@@ -693,7 +756,10 @@ inline size_t csr_ws_bytes(const CsrPlan &p, int64_t B, int64_t K, int acc_bytes
 template <typename T, int VEC, int REDUCE>
 int launch_csr_reduce_t(const CsrReduceArgs &a, const CsrPlan &p, int64_t B, hipStream_t stream) {
   dim3 grid((unsigned)p.nblk, (unsigned)p.ychunks, (unsigned)B);
-  if (a.accumulate)
+  if (a.perm != nullptr) {
+    if (a.accumulate) return TS_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL((csr_reduce_kernel<T, VEC, REDUCE, 0, true>), grid, dim3(kBlock), 0, stream, a);
+  } else if (a.accumulate)
     hipLaunchKernelGGL((csr_reduce_kernel<T, VEC, REDUCE, -1>), grid, dim3(kBlock), 0, stream, a);
   else
     hipLaunchKernelGGL((csr_reduce_kernel<T, VEC, REDUCE, 0>), grid, dim3(kBlock), 0, stream, a);

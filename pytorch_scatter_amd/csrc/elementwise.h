@@ -70,6 +70,32 @@ __global__ __launch_bounds__(kBlock) void arg_backward_kernel(const T *__restric
   }
 }
 
+// After a min / max over permuted rows (a scatter through a sorted index): positions in row-pointer order
+// become positions in the caller's order, and a slot whose entries never beat scatter's initial value
+// (lowest() / max() of the element type) reads 0 with position E, as scatter leaves it
+// (csrc/cpu/scatter_cpu.cpp:81-82). A slot without entries already holds 0 and E.
+template <typename T, bool IS_MAX>
+__global__ __launch_bounds__(kBlock) void sorted_args_kernel(T *__restrict__ out, int64_t *__restrict__ arg,
+                                                             const int32_t *__restrict__ perm, int64_t total,
+                                                             int64_t per_batch, int64_t E, int64_t perm_batch_stride) {
+  typedef typename Acc<T>::type A;
+  const A lim = to_acc<T>(IS_MAX ? ElemLim<T>::lowest() : ElemLim<T>::max());
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < total; i += (int64_t)gridDim.x * kBlock) {
+    const int64_t a = arg[i];
+    if (a < 0 || a >= E) continue;
+    const A v = to_acc<T>(out[i]);
+    const bool beat = IS_MAX ? (v > lim) : (v < lim);
+    if (beat) {
+      arg[i] = perm[(i / per_batch) * perm_batch_stride + a];
+    } else {
+      out[i] = zero_elem<T>();
+      arg[i] = E;
+    }
+  }
+}
+
+template <typename T> int launch_sorted_args(void *out, int64_t *arg, const int32_t *perm, int64_t B, int64_t per_batch,
+                                             int64_t E, int64_t perm_batch_stride, bool is_max, hipStream_t stream);
 template <typename T> int launch_divide_by_count(void *out, const float *count, int64_t rows, int64_t K,
                                                  hipStream_t stream);
 template <typename T> int launch_arg_backward(const void *grad_out, const int64_t *arg, void *grad_in,
@@ -77,6 +103,20 @@ template <typename T> int launch_arg_backward(const void *grad_out, const int64_
                                               hipStream_t stream);
 
 #define TS_INSTANTIATE_ELEMENTWISE(T)                                                              \
+  template <> int launch_sorted_args<T>(void *out, int64_t *arg, const int32_t *perm, int64_t B,   \
+                                        int64_t per_batch, int64_t E, int64_t perm_batch_stride,   \
+                                        bool is_max, hipStream_t stream) {                         \
+    const int64_t total = B * per_batch;                                                           \
+    if (total > 0 && is_max)                                                                       \
+      hipLaunchKernelGGL((sorted_args_kernel<T, true>), dim3(grid_for(total)), dim3(kBlock), 0,    \
+                         stream, static_cast<T *>(out), arg, perm, total, per_batch, E,            \
+                         perm_batch_stride);                                                       \
+    else if (total > 0)                                                                            \
+      hipLaunchKernelGGL((sorted_args_kernel<T, false>), dim3(grid_for(total)), dim3(kBlock), 0,   \
+                         stream, static_cast<T *>(out), arg, perm, total, per_batch, E,            \
+                         perm_batch_stride);                                                       \
+    return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;                                \
+  }                                                                                                \
   template <> int launch_divide_by_count<T>(void *out, const float *count, int64_t rows, int64_t K, \
                                             hipStream_t stream) {                                  \
     if (rows * K > 0)                                                                              \

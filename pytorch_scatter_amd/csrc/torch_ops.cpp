@@ -789,6 +789,140 @@ struct GroupStdFn : public torch::autograd::Function<GroupStdFn> {
   }
 };
 
+// ------------------------------------------------- index formats and the sorted scatter
+// Not in the reference: its callers bring `row` and `rowptr` from the same sparse matrix
+// (benchmark/scatter_segment.py:38-41). index_to_indptr / indptr_to_index convert between the two,
+// sort_index turns an unsorted index into (perm, indptr) once, and scatter_sorted then runs scatter's
+// reductions as a segmented reduction over permuted rows: no atomics, the same bits on every call.
+void check_long_device(const Tensor &t, const char *name) {
+  check_device(t, name);
+  TORCH_CHECK(t.scalar_type() == at::kLong, name, " must be int64");
+}
+
+Tensor index_to_indptr(Tensor index, int64_t dim_size) {
+  check_long_device(index, "index");
+  TORCH_CHECK(index.dim() >= 1 && dim_size >= 0, "Input mismatch");
+  c10::DeviceGuard guard(index.device());
+  index = index.contiguous();
+  const int64_t E = index.size(-1), B = E > 0 ? index.numel() / E : prod(index.sizes(), 0, index.dim() - 1);
+  auto sizes = index.sizes().vec();
+  sizes.back() = dim_size + 1;
+  Tensor indptr = at::empty(sizes, index.options());
+  check_status(ts_index_to_indptr(index.data_ptr<int64_t>(), indptr.data_ptr<int64_t>(), B, E, dim_size, E,
+                                  stream_of(index)),
+               "index_to_indptr");
+  return indptr;
+}
+
+Tensor indptr_to_index(Tensor indptr, OptInt num_entries) {
+  check_long_device(indptr, "indptr");
+  TORCH_CHECK(indptr.dim() >= 1 && indptr.size(-1) >= 1, "Input mismatch");
+  c10::DeviceGuard guard(indptr.device());
+  indptr = indptr.contiguous();
+  const int64_t N = indptr.size(-1) - 1, B = indptr.numel() / (N + 1);
+  // every batch row must hold the same number of entries; without num_entries it is read back
+  const int64_t E = num_entries.has_value() ? num_entries.value()
+                                            : (indptr.numel() > 0 ? indptr.select(-1, N).max().item<int64_t>() : 0);
+  auto sizes = indptr.sizes().vec();
+  sizes.back() = E;
+  Tensor index = at::empty(sizes, indptr.options());
+  if (index.numel() == 0) return index;
+  Tensor ws = workspace(ts_indptr_to_index_workspace_bytes(B, N), indptr);
+  check_status(ts_indptr_to_index(indptr.data_ptr<int64_t>(), index.data_ptr<int64_t>(), B, N, E, N + 1, ws.data_ptr(),
+                                  static_cast<size_t>(ws.numel()), stream_of(indptr)),
+               "indptr_to_index");
+  return index;
+}
+
+std::tuple<Tensor, Tensor> sort_index(Tensor index, int64_t dim_size) {
+  check_long_device(index, "index");
+  TORCH_CHECK(index.dim() == 1, "sort_index expects a one-dimensional index");
+  TORCH_CHECK(dim_size >= 0, "Input mismatch");
+  c10::DeviceGuard guard(index.device());
+  index = index.contiguous();
+  const int64_t E = index.numel();
+  Tensor perm = at::empty({E}, index.options().dtype(at::kInt));
+  Tensor indptr = at::empty({dim_size + 1}, index.options());
+  Tensor ws = workspace(ts_sort_index_workspace_bytes(E, dim_size), index);
+  check_status(ts_sort_index(index.data_ptr<int64_t>(), perm.data_ptr<int32_t>(), indptr.data_ptr<int64_t>(), E,
+                             dim_size, ws.data_ptr(), static_cast<size_t>(ws.numel()), stream_of(index)),
+               "sort_index");
+  // one read-back at set-up: entries outside [0, dim_size) sort behind the last row
+  TORCH_CHECK(indptr[dim_size].item<int64_t>() == E, "sort_index: index out of range [0, ", dim_size, ")");
+  return std::make_tuple(perm, indptr);
+}
+
+template <int REDUCE> struct SortedScatterFn : public torch::autograd::Function<SortedScatterFn<REDUCE>> {
+  static variable_list forward(AutogradContext *ctx, Variable src, Variable index, Variable perm, Variable indptr,
+                               int64_t dim) {
+    check_device(src, "src");
+    check_long_device(index, "index");
+    check_long_device(indptr, "indptr");
+    check_device(perm, "perm");
+    TORCH_CHECK(perm.scalar_type() == at::kInt, "perm must be int32");
+    TORCH_CHECK(src.dim() >= 1, "Input mismatch");
+    dim = dim < 0 ? src.dim() + dim : dim;
+    TORCH_CHECK(dim >= 0 && dim < src.dim(), "Input mismatch");
+    TORCH_CHECK(index.dim() == 1 && perm.dim() == 1 && indptr.dim() == 1 && indptr.numel() >= 1, "Input mismatch");
+    const int64_t E = src.size(dim), N = indptr.numel() - 1;
+    TORCH_CHECK(index.numel() == E && perm.numel() == E, "Input mismatch");
+    c10::DeviceGuard guard(src.device());
+    src = src.contiguous();
+    perm = perm.contiguous();
+    indptr = indptr.contiguous();
+    const int64_t B = prod(src.sizes(), 0, dim), K = prod(src.sizes(), dim + 1, src.dim());
+    auto sizes = src.sizes().vec();
+    sizes[dim] = N;
+    constexpr bool kArg = REDUCE == TS_MIN || REDUCE == TS_MAX;
+    // integer mean: scatter divides with floor (csrc/scatter.cpp:138-141), the segmented kernel truncates
+    const bool int_mean = REDUCE == TS_MEAN && !src.is_floating_point();
+    const int reduce = int_mean ? TS_SUM : REDUCE;
+    Tensor out = at::empty(sizes, src.options());
+    Tensor arg_out = kArg ? at::empty(sizes, index.options()) : Tensor();
+    if (out.numel() > 0) {
+      Tensor ws = workspace(ts_segment_csr_permuted_workspace_bytes(B, N, E, K, dtype_code(src), reduce), src);
+      check_status(ts_segment_csr_permuted(src.data_ptr(), perm.data_ptr<int32_t>(), indptr.data_ptr<int64_t>(),
+                                           out.data_ptr(), kArg ? arg_out.data_ptr<int64_t>() : nullptr, B, N, E, K, 0,
+                                           0, dtype_code(src), reduce, ws.data_ptr(),
+                                           static_cast<size_t>(ws.numel()), stream_of(src)),
+                   "scatter_sorted");
+    }
+    ctx->saved_data["dim"] = dim;
+    ctx->saved_data["src_shape"] = src.sizes();
+    Variable index_b = broadcast(index, src, dim);
+    if (REDUCE == TS_MEAN) {
+      Tensor count = (indptr.slice(0, 1, N + 1) - indptr.slice(0, 0, N)).clamp_min_(1);
+      if (int_mean) out.div_(broadcast(count.to(src.scalar_type()), out, dim), "floor");
+      if (src.requires_grad()) ctx->save_for_backward({index_b, broadcast(count.to(src.scalar_type()), out, dim)});
+      return {out};
+    }
+    if (kArg) {
+      ctx->save_for_backward({index_b, arg_out});
+      ctx->mark_non_differentiable({arg_out});
+      return {out, arg_out};
+    }
+    ctx->save_for_backward({index_b});
+    return {out};
+  }
+
+  // as ScatterFn: csrc/scatter.cpp:70-81, 143-161, 184-196
+  static variable_list backward(AutogradContext *ctx, variable_list grad_outs) {
+    auto grad_out = grad_outs[0];
+    auto saved = ctx->get_saved_variables();
+    const int64_t dim = ctx->saved_data["dim"].toInt();
+    Variable grad_in;
+    if (REDUCE == TS_SUM) {
+      grad_in = at::gather(grad_out, dim, saved[0], false);
+    } else if (REDUCE == TS_MEAN) {
+      grad_in = at::gather(grad_out, dim, saved[0], false);
+      grad_in.true_divide_(at::gather(saved[1], dim, saved[0], false));
+    } else {
+      grad_in = arg_backward_hip(grad_out, saved[1], saved_shape(ctx), dim);
+    }
+    return {grad_in, Variable(), Variable(), Variable(), Variable()};
+  }
+};
+
 // ------------------------------------------------------- registered functions
 Tensor scatter_sum(Tensor src, Tensor index, int64_t dim, OptTensor out, OptInt dim_size) {
   return ScatterFn<TS_SUM>::apply(src, index, dim, out, dim_size)[0];
@@ -922,6 +1056,38 @@ Tensor scatter_std(Tensor src, Tensor index, int64_t dim, OptTensor out, OptInt 
   return sq.div(count + 1e-6).sqrt();
 }
 
+// (values, positions); positions is an empty tensor unless reduce is min or max
+std::tuple<Tensor, Tensor> scatter_sorted(Tensor src, Tensor index, Tensor perm, Tensor indptr, int64_t dim,
+                                          std::string reduce) {
+  const int code = reduce_code(reduce);
+  if ((code == TS_MIN || code == TS_MAX) && src.dim() >= 1 && indptr.dim() == 1 && indptr.numel() >= 1) {
+    // rows under 64 bytes: min / max through the atomic kernels are as exact and faster
+    const int64_t d = dim < 0 ? src.dim() + dim : dim;
+    if (d >= 0 && d < src.dim() && prod(src.sizes(), d + 1, src.dim()) * (int64_t)src.element_size() < 64 &&
+        index.numel() == src.size(d)) {
+      const int64_t N = indptr.numel() - 1;
+      return code == TS_MIN ? scatter_min(src, index, d, std::nullopt, N) : scatter_max(src, index, d, std::nullopt, N);
+    }
+  }
+  switch (code) {
+  case TS_SUM:
+    return std::make_tuple(SortedScatterFn<TS_SUM>::apply(src, index, perm, indptr, dim)[0],
+                           at::empty({0}, index.options()));
+  case TS_MEAN:
+    return std::make_tuple(SortedScatterFn<TS_MEAN>::apply(src, index, perm, indptr, dim)[0],
+                           at::empty({0}, index.options()));
+  case TS_MIN: {
+    auto r = SortedScatterFn<TS_MIN>::apply(src, index, perm, indptr, dim);
+    return std::make_tuple(r[0], r[1]);
+  }
+  case TS_MAX: {
+    auto r = SortedScatterFn<TS_MAX>::apply(src, index, perm, indptr, dim);
+    return std::make_tuple(r[0], r[1]);
+  }
+  default: TORCH_CHECK(false, "scatter_sorted: reduce must be sum, mean, min or max");
+  }
+}
+
 int64_t cuda_version() { return ts_hip_version(); }  // csrc/version.cpp:28-38 returns HIP_VERSION on ROCm
 
 }  // namespace
@@ -945,4 +1111,8 @@ static auto registry = torch::RegisterOperators()
                            .op("torch_scatter::gather_coo", &gather_coo)
                            .op("torch_scatter::scatter_softmax", &scatter_softmax)
                            .op("torch_scatter::scatter_logsumexp", &scatter_logsumexp)
-                           .op("torch_scatter::scatter_std", &scatter_std);
+                           .op("torch_scatter::scatter_std", &scatter_std)
+                           .op("torch_scatter::index_to_indptr", &index_to_indptr)
+                           .op("torch_scatter::indptr_to_index", &indptr_to_index)
+                           .op("torch_scatter::sort_index", &sort_index)
+                           .op("torch_scatter::scatter_sorted", &scatter_sorted);

@@ -1,0 +1,258 @@
+"""Index formats and the sorted scatter on the GPU: ts_index_to_indptr,
+ts_indptr_to_index, ts_sort_index and ts_segment_csr_permuted through the C ABI,
+SortedIndex / scatter_sorted through the Python API.
+
+Bars: permutations, row pointers, min / max values and arg positions are bit-exact
+against the CPU oracle (its plain-loop restatement at small sizes, numpy's stable
+argsort -- which the CPU suite pins to the same loops -- at large ones); sum / mean
+within rtol 1e-5 (fp32) / 1e-2 (16-bit floats) of the oracle's scatter, integers exact.
+"""
+from itertools import product
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import random_values
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+RTOL = {torch.float32: 1e-5, torch.float64: 1e-12, torch.bfloat16: 1e-2, torch.float16: 1e-2}
+ALL_DTYPES = [torch.float32, torch.float64, torch.float16, torch.bfloat16, torch.int32, torch.int64, torch.int16,
+              torch.int8, torch.uint8]
+
+
+@pytest.fixture(scope="module")
+def capi():
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    from pytorch_scatter_amd import capi
+    capi.lib()
+    return capi
+
+
+@pytest.fixture(scope="module")
+def ts():
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    import pytorch_scatter_amd
+    return pytorch_scatter_amd
+
+
+def make_index(kind, rng, E, N):
+    if kind == "hub":
+        idx = rng.integers(0, N, size=E)
+        idx[E // 4: 3 * E // 4] = N // 2
+    elif kind == "sorted":
+        idx = np.sort(rng.integers(0, N, size=E))
+    elif kind == "gaps":  # most rows empty
+        idx = rng.integers(0, max(N // 16, 1), size=E) * 16 % N
+    else:
+        idx = rng.integers(0, N, size=E)
+    return torch.from_numpy(idx.astype(np.int64))
+
+
+def sort_on_gpu(capi, index, N):
+    E = index.numel()
+    perm = torch.empty(E, dtype=torch.int32, device=DEV)
+    indptr = torch.empty(N + 1, dtype=torch.long, device=DEV)
+    capi.sort_index(index.to(DEV), perm, indptr, E, N)
+    torch.cuda.synchronize()
+    return perm, indptr
+
+
+@pytest.mark.parametrize("E,N,kind", [(0, 0, "random"), (0, 7, "random"), (1, 1, "random"), (300, 17, "random"),
+                                      (4000, 3, "hub"), (3000, 5000, "gaps"), (2500, 40, "sorted")])
+def test_sort_and_formats_against_oracle_loops(capi, oracle, E, N, kind):
+    rng = np.random.default_rng(E * 3 + N)
+    index = make_index(kind, rng, E, N) if E > 0 else torch.zeros(0, dtype=torch.long)
+    perm, indptr = sort_on_gpu(capi, index, N)
+    want_perm, want_ptr = oracle.sort_index(index, N)
+    assert torch.equal(perm.cpu().long(), want_perm)
+    assert torch.equal(indptr.cpu(), want_ptr)
+    srt = index[want_perm]
+    ptr2 = torch.empty(N + 1, dtype=torch.long, device=DEV)
+    capi.index_to_indptr(srt.to(DEV), ptr2, 1, E, N, E)
+    torch.cuda.synchronize()
+    assert torch.equal(ptr2.cpu(), oracle.index_to_indptr(srt, N))
+    back = torch.full((E,), -1, dtype=torch.long, device=DEV)
+    capi.indptr_to_index(ptr2, back, 1, N, E, N + 1)
+    torch.cuda.synchronize()
+    assert torch.equal(back.cpu(), oracle.indptr_to_index(want_ptr)) and torch.equal(back.cpu(), srt)
+
+
+@pytest.mark.parametrize("E,N,kind", [(1 << 20, 1000, "hub"), (3_000_001, 2_000_000, "random"),
+                                      (2_000_000, 70_000, "gaps"), (1 << 21, 1, "random")])
+def test_sort_large_against_numpy(capi, E, N, kind):
+    rng = np.random.default_rng(N)
+    index = make_index(kind, rng, E, N)
+    perm, indptr = sort_on_gpu(capi, index, N)
+    assert torch.equal(perm.cpu().long(), torch.from_numpy(np.argsort(index.numpy(), kind="stable")))
+    want_ptr = np.zeros(N + 1, dtype=np.int64)
+    want_ptr[1:] = np.cumsum(np.bincount(index.numpy(), minlength=N))
+    assert torch.equal(indptr.cpu(), torch.from_numpy(want_ptr))
+    # batched round trip of the formats: two batch rows that hold the same number of entries
+    srt = np.sort(index.numpy())
+    both = torch.from_numpy(np.stack([srt, np.sort((srt * 7 + 1) % N)])).to(DEV)
+    ptr = torch.empty((2, N + 1), dtype=torch.long, device=DEV)
+    capi.index_to_indptr(both, ptr, 2, E, N, E)
+    back = torch.empty((2, E), dtype=torch.long, device=DEV)
+    capi.indptr_to_index(ptr, back, 2, N, E, N + 1)
+    torch.cuda.synchronize()
+    assert torch.equal(back, both)
+    assert torch.equal(ptr[0].cpu(), torch.from_numpy(want_ptr))
+
+
+def test_sort_marks_entries_outside_the_range(capi):
+    index = torch.tensor([3, -1, 0, 9, 2, 3, 4], dtype=torch.long)
+    perm, indptr = sort_on_gpu(capi, index, 4)
+    assert indptr.tolist() == [0, 1, 1, 2, 4]  # indptr[N] = 4 < E = 7
+    assert perm.tolist()[:4] == [2, 4, 0, 5] and sorted(perm.tolist()[4:]) == [1, 3, 6]
+
+
+SHAPES = [
+    # B, E, K, N
+    (1, 5000, 1, 300), (2, 3000, 4, 50), (1, 2000, 8, 100), (1, 1500, 3, 40), (1, 900, 64, 20),
+    (1, 700, 130, 9), (3, 400, 16, 7), (1, 1, 1, 1), (1, 257, 2, 300), (1, 40000, 32, 1500),
+]
+
+
+@pytest.mark.parametrize("shape,kind,dtype", product(SHAPES, ["random", "hub", "gaps"], ALL_DTYPES))
+def test_permuted_reduce_against_oracle_scatter(capi, oracle, shape, kind, dtype):
+    B, E, K, N = shape
+    rng = np.random.default_rng(E * 5 + K)
+    index1 = make_index(kind, rng, E, N)
+    perm, indptr = sort_on_gpu(capi, index1, N)
+    index = index1.view(1, E, 1).expand(B, E, K)
+    for reduce in ("sum", "mean", "min", "max"):
+        small = dtype in (torch.int8, torch.uint8) and reduce in ("sum", "mean")
+        src = random_values(rng, (B, E, K), dtype, ties=True)
+        if small:  # keep 8-bit sums inside the type
+            src = (src.abs() > 6).to(dtype)
+            if kind != "random":  # more than 127 entries per slot: the reference's 8-bit count wraps
+                continue
+        want, want_arg = oracle.scatter(src, index, 1, None, N, reduce)
+        if reduce == "mean":  # the division belongs to the op layer (floor division for integers)
+            want = oracle.op_scatter(src, index1, 1, None, N, "mean")
+        out = torch.empty((B, N, K), dtype=dtype, device=DEV)
+        arg = torch.empty((B, N, K), dtype=torch.long, device=DEV) if reduce in ("min", "max") else None
+        code = capi.REDUCE[reduce]
+        if reduce == "mean" and not dtype.is_floating_point:
+            capi.segment_csr_permuted(src.to(DEV), perm, indptr, out, arg, B, N, E, K, 0, 0, capi.SUM)
+            cnt = (indptr[1:] - indptr[:-1]).clamp(min=1).view(1, N, 1)
+            out = torch.div(out, cnt, rounding_mode="floor").to(dtype)
+        else:
+            capi.segment_csr_permuted(src.to(DEV), perm, indptr, out, arg, B, N, E, K, 0, 0, code)
+        torch.cuda.synchronize()
+        if reduce in ("min", "max"):
+            assert torch.equal(out.cpu(), want), reduce
+            assert torch.equal(arg.cpu(), want_arg), reduce
+        elif dtype.is_floating_point:
+            scale = float(oracle.scatter(src.double().abs(), index, 1, None, N, "sum")[0].max())
+            err = (out.cpu().double() - want.double()).abs()
+            bound = RTOL[dtype] * want.double().abs() + RTOL[dtype] * scale
+            assert bool((err <= bound).all()), (reduce, float((err - bound).max()))
+        else:
+            assert torch.equal(out.cpu(), want), reduce
+
+
+def test_permuted_reduce_argument_checks(capi):
+    import ctypes
+    L = capi.lib()
+    x = torch.zeros((8, 4), device=DEV)
+    perm = torch.arange(8, dtype=torch.int32, device=DEV)
+    ptr = torch.tensor([0, 8], device=DEV)
+    out = torch.zeros((1, 4), device=DEV)
+    ws = torch.empty(1, dtype=torch.uint8, device=DEV)
+    args = (capi._p(x), capi._p(perm), capi._p(ptr), capi._p(out), None, capi._i(1), capi._i(1), capi._i(8), capi._i(4),
+            capi._i(0), capi._i(0), capi.DTYPE[torch.float32])
+    assert L.ts_segment_csr_permuted(*args, capi.MUL, capi._p(ws), ctypes.c_size_t(1), None) == 2  # unsupported
+    assert L.ts_segment_csr_permuted(*args, capi.MAX, capi._p(ws), ctypes.c_size_t(1), None) == 1  # arg_out missing
+    assert L.ts_segment_csr_permuted(*args, capi.SUM, None, ctypes.c_size_t(0), None) == 3         # workspace
+
+
+# ------------------------------------------------------------------ operator level
+@pytest.mark.parametrize("dim,reduce,dtype", product([0, 1, -1], ["sum", "mean", "min", "max"],
+                                                     [torch.float32, torch.float64, torch.bfloat16, torch.int64]))
+def test_scatter_sorted_matches_scatter(ts, dim, reduce, dtype):
+    shape = (60, 50, 24)
+    g = torch.Generator().manual_seed(13)
+    d = dim if dim >= 0 else len(shape) + dim
+    N = 11
+    index = torch.randint(0, N - 1, (shape[d],), generator=g).to(DEV)  # slot N-1 stays empty
+    src = torch.randint(-9, 10, shape, generator=g).to(dtype).to(DEV)
+    plan = ts.SortedIndex(index, N)
+    assert torch.equal(index[plan.perm.long()], plan.sorted_index())
+    if reduce in ("min", "max"):
+        out, arg = ts.scatter_sorted(src, plan, dim, reduce)
+        want, want_arg = (ts.scatter_min if reduce == "min" else ts.scatter_max)(src, index, dim, None, N)
+        assert torch.equal(out, want) and torch.equal(arg, want_arg)
+    else:
+        out = ts.scatter_sorted(src, plan, dim, reduce)
+        want = ts.scatter(src, index, dim, None, N, reduce)
+        assert torch.equal(out, want)  # small integers: every sum is exact in every type
+    again = ts.scatter_sorted(src, plan, dim, reduce)
+    assert torch.equal(out, again[0] if reduce in ("min", "max") else again)
+
+
+@pytest.mark.parametrize("reduce", ["sum", "mean", "min", "max"])
+def test_scatter_sorted_autograd(ts, reduce):
+    g = torch.Generator().manual_seed(17)
+    N = 40
+    index = torch.randint(0, N, (500,), generator=g).to(DEV)
+    x = torch.randn((3, 500, 6), generator=g, dtype=torch.double).to(DEV)
+    grad = torch.randn((3, N, 6), generator=g, dtype=torch.double).to(DEV)
+    plan = ts.SortedIndex(index, N)
+    a = x.clone().requires_grad_(True)
+    b = x.clone().requires_grad_(True)
+    got = ts.scatter_sorted(a, plan, 1, reduce)
+    want = ts.scatter(b, index, 1, None, N, reduce)
+    got = got[0] if reduce in ("min", "max") else got
+    got.backward(grad)
+    want.backward(grad)
+    assert torch.allclose(got, want, rtol=1e-12, atol=1e-12)
+    assert torch.allclose(a.grad, b.grad, rtol=1e-12, atol=1e-12)
+
+
+def test_scatter_sorted_is_bit_reproducible_and_close_to_scatter(ts):
+    g = torch.Generator().manual_seed(19)
+    E, N, K = 400_000, 5000, 32
+    index = torch.randint(0, N, (E,), generator=g)
+    index[: E // 3] = 7  # a hub
+    index = index[torch.randperm(E, generator=g)].to(DEV)
+    src = torch.randn((E, K), generator=g).to(DEV)
+    plan = ts.SortedIndex(index, N)
+    first = ts.scatter_sorted(src, plan, 0, "sum")
+    for _ in range(3):
+        assert torch.equal(first, ts.scatter_sorted(src, plan, 0, "sum"))
+    want = ts.scatter_sum(src.double(), index, 0, None, N)
+    scale = float(ts.scatter_sum(src.abs().double(), index, 0, None, N).max())
+    assert float((first.double() - want).abs().max()) <= 1e-5 * scale
+
+
+def test_formats_and_plan_operator_checks(ts):
+    index = torch.tensor([0, 0, 2, 2, 2, 5], device=DEV)
+    ptr = ts.index_to_indptr(index, 7)
+    assert ptr.tolist() == [0, 2, 2, 5, 5, 5, 6, 6]
+    assert torch.equal(ts.indptr_to_index(ptr), index)
+    assert torch.equal(ts.indptr_to_index(ptr, 6), index)
+    both = torch.stack([index, torch.tensor([1, 1, 1, 3, 6, 6], device=DEV)])
+    ptr2 = ts.index_to_indptr(both, 7)
+    assert ptr2.shape == (2, 8) and torch.equal(ts.indptr_to_index(ptr2), both)
+    assert ts.indptr_to_index(torch.zeros(4, dtype=torch.long, device=DEV)).shape == (0,)
+    with pytest.raises(RuntimeError, match="out of range"):
+        ts.SortedIndex(torch.tensor([0, 3, 9], device=DEV), 5)
+    with pytest.raises(ValueError):
+        ts.SortedIndex(both)
+    with pytest.raises(RuntimeError, match="must be CUDA tensor"):
+        ts.index_to_indptr(index.cpu(), 7)
+    plan = ts.SortedIndex(index)
+    assert plan.dim_size == 6
+    with pytest.raises(ValueError):
+        ts.scatter_sorted(torch.ones(6, device=DEV), plan, 0, "mul")
+    with pytest.raises(RuntimeError, match="Input mismatch"):
+        ts.scatter_sorted(torch.ones(5, device=DEV), plan, 0, "sum")
+    # a plan over no entries
+    empty = ts.SortedIndex(torch.zeros(0, dtype=torch.long, device=DEV), 3)
+    assert ts.scatter_sorted(torch.ones((0, 2), device=DEV), empty, 0, "sum").tolist() == [[0, 0]] * 3
