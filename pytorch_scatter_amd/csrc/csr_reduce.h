@@ -340,8 +340,15 @@ __global__ __launch_bounds__(kBlock, (csr_reduce_min_blocks<T, VEC, REDUCE, PERM
   const bool lookback = kCarryOk && a.lookback != 0;
   // default: the tile leaves no open row; the worker that does overwrites this after the barrier
   if (!lookback && tid == 0 && blockIdx.y == 0) a.ws_meta[(b * a.nblk + blockIdx.x) * 4 + 2] = -1;
-  if (PERM && tid == 0) s_cut[0] = -1;  // becomes the first tile of a walk that the workgroup shares
   __syncthreads();
+  // The row that entered the tile from the one before began more than kSharedWalkMin tiles back (a hub row):
+  // if it ends here, the walk over those tiles is shared by the whole workgroup. Every lane derives the same
+  // answer from LDS, so tiles without such a row, nearly all, pay two LDS reads and no barrier.
+  bool shared_walk = false;
+  if (lookback && s_head_row[0] >= 0) {
+    const int row0 = s_head_row[0];
+    shared_walk = (i0 + row0) + ((int64_t)s_ptr[row0] + j0) < ((int64_t)blockIdx.x - kSharedWalkMin) * a.BI;
+  }
 
   // ---- combine partials of rows that cross worker boundaries, in edge order
   A *ws_val_blk = static_cast<A *>(a.ws_vals) + ((b * a.nblk + blockIdx.x) * 2) * a.K;
@@ -500,8 +507,7 @@ __global__ __launch_bounds__(kBlock, (csr_reduce_min_blocks<T, VEC, REDUCE, PERM
           // the row's first entry sits at merge position (row index + row pointer)
           int64_t first_tile = ((i0 + row) + ((int64_t)s_ptr[row] + j0)) / a.BI;
           if (first_tile < 0) first_tile = 0;
-          if (PERM && (int64_t)blockIdx.x - first_tile > kSharedWalkMin) {
-            // a hub row that passed through many tiles: the whole workgroup walks (below)
+          if (shared_walk) {
 #pragma unroll
             for (int v = 0; v < VEC; ++v) { my_tail_val[v] = acc[v]; if (kArg) my_tail_arg[v] = arg[v]; }
             if (lg == 0) s_cut[0] = first_tile;
@@ -512,6 +518,7 @@ __global__ __launch_bounds__(kBlock, (csr_reduce_min_blocks<T, VEC, REDUCE, PERM
           }
         } else {
           publish_carry(kCarryPass);
+          if (shared_walk && lg == 0) s_cut[0] = -1;  // the row goes on: nothing to walk here
         }
       } else {
         if (col_ok) {
@@ -532,8 +539,8 @@ __global__ __launch_bounds__(kBlock, (csr_reduce_min_blocks<T, VEC, REDUCE, PERM
   // ---- a long walk shared by the workgroup: worker w collects the carries of the tiles
   // blockIdx.x - 1 - w, - W, ... into a partial of its own; worker 0 then folds the partials in worker order.
   // The grouping is fixed by the tiling, so the result is the same on every call.
-  if constexpr (PERM && kCarryOk) {
-    if (!lookback) return;
+  if constexpr (kCarryOk) {
+    if (!shared_walk) return;
     __syncthreads();
     const int64_t first_tile = s_cut[0];
     if (first_tile < 0) return;

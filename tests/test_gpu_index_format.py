@@ -256,3 +256,47 @@ def test_formats_and_plan_operator_checks(ts):
     # a plan over no entries
     empty = ts.SortedIndex(torch.zeros(0, dtype=torch.long, device=DEV), 3)
     assert ts.scatter_sorted(torch.ones((0, 2), device=DEV), empty, 0, "sum").tolist() == [[0, 0]] * 3
+
+
+@pytest.mark.parametrize("K,dtype", [(4, torch.float32), (32, torch.float32), (2, torch.float64), (64, torch.bfloat16),
+                                     (8, torch.int32)])
+def test_hub_row_through_many_tiles(capi, oracle, K, dtype):
+    """A row of 200 000 entries passes through about a hundred tiles: the walk over their partial results is
+    shared by the workgroup that ends the row. Small-integer values: every sum is exact and ties are
+    everywhere, so values and positions must match the oracle bit for bit, with and without a permutation."""
+    rng = np.random.default_rng(K)
+    N, E = 50, 300_000
+    deg = np.full(N, (E - 200_000) // (N - 1), dtype=np.int64)
+    deg[17] = 200_000
+    deg[-1] += E - deg.sum()
+    indptr = torch.zeros(N + 1, dtype=torch.long)
+    indptr[1:] = torch.from_numpy(np.cumsum(deg))
+    src = torch.from_numpy(rng.integers(-3, 4, size=(E, K)).astype(np.float64)).to(dtype)
+    order = torch.from_numpy(rng.permutation(E))
+    index = torch.repeat_interleave(torch.arange(N), torch.from_numpy(deg))
+    shuffled_index = torch.empty(E, dtype=torch.long)
+    shuffled_index[order] = index          # entry order[i] of the shuffled input is sorted entry i ...
+    shuffled_src = torch.empty_like(src)
+    shuffled_src[order] = src              # ... up to the order inside a row, which the stable sort fixes
+    perm, ptr_d = sort_on_gpu(capi, shuffled_index, N)
+    assert torch.equal(ptr_d.cpu(), indptr)
+    for reduce in ("sum", "min", "max"):
+        code = capi.REDUCE[reduce]
+        want, want_arg = oracle.segment_csr(src, indptr, None, reduce)
+        out = torch.empty((N, K), dtype=dtype, device=DEV)
+        arg = torch.empty((N, K), dtype=torch.long, device=DEV) if reduce != "sum" else None
+        capi.segment_csr(src.to(DEV), indptr.to(DEV), out, arg, 1, N, E, K, 0, code)
+        torch.cuda.synchronize()
+        assert torch.equal(out.cpu(), want), reduce
+        if arg is not None:
+            assert torch.equal(arg.cpu(), want_arg), reduce
+        want2, want_arg2 = oracle.scatter(shuffled_src.view(1, E, K), shuffled_index.view(1, E, 1).expand(1, E, K), 1,
+                                          None, N, reduce)
+        out2 = torch.empty((N, K), dtype=dtype, device=DEV)
+        arg2 = torch.empty((N, K), dtype=torch.long, device=DEV) if reduce != "sum" else None
+        capi.segment_csr_permuted(shuffled_src.to(DEV), perm, ptr_d, out2, arg2, 1, N, E, K, 0, 0, code)
+        torch.cuda.synchronize()
+        # sums against the segmented oracle: scatter's oracle adds 16-bit floats in the element type
+        assert torch.equal(out2.cpu(), want if reduce == "sum" else want2[0]), reduce
+        if arg2 is not None:
+            assert torch.equal(arg2.cpu(), want_arg2[0]), reduce
