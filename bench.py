@@ -152,6 +152,26 @@ def bench_scatter_config(ts, wl, w, dev, iters, reduces):
     return res
 
 
+def bench_sorted_config(ts, wl, w, dev, iters):
+    """The same scatter through an index sorted once (SortedIndex + scatter_sorted): the one-time sort, then
+    sum / max as a segmented reduction over permuted rows. Bytes as for scatter plus 4 per entry for perm."""
+    import torch
+    src = wl.scatter_values(w, dev)
+    index = w.index.to(dev)
+    res = {"N": w.N, "E": w.E, "K": w.K, "dtype": "float32"}
+    t = event_time(lambda: ts.SortedIndex(index, w.N), max(iters // 2, 3))
+    res["sort_index_us"] = round(t * 1e6, 1)
+    plan = ts.SortedIndex(index, w.N)
+    with torch.no_grad():
+        t = event_time(lambda: ts.scatter_sorted(src, plan, 0, "sum"), iters)
+        res["scatter_sorted_sum"] = entry(wl.bytes_scatter(w.E, w.N, w.K, 4) + 4 * w.E, t, w.E * w.K)
+        t = event_time(lambda: ts.scatter_sorted(src, plan, 0, "max"), iters)
+        res["scatter_sorted_max"] = entry(wl.bytes_scatter(w.E, w.N, w.K, 4, True) + 4 * w.E, t, w.E * w.K)
+    del src, plan
+    torch.cuda.empty_cache()
+    return res
+
+
 def bench_softmax_config(ts, wl, w, dev, iters, K):
     """scatter_softmax and scatter_std over the destination index of the C3 graph with K values per entry (attention
     heads), sorted and in random order; bytes: src read once, index read once, result written once."""
@@ -392,6 +412,10 @@ def main():
         zipf_index = wz.index[torch.randperm(wz.E, generator=g)] * 10 % 1_000_000
         sz = wl.ScatterWorkload("X-zipf-unsorted-K8", zipf_index, 1_000_000, wz.E, 8, torch.float32)
         table["X-zipf-unsorted-K8"] = bench_scatter_config(ts, wl, sz, dev, max(it // 2, 3), ["sum", "max"])
+        table["X-sorted-plan-C4-K32"] = bench_sorted_config(ts, wl, wl.c4_scatter_minmax(32), dev, max(it // 2, 3))
+        ss = wl.ScatterWorkload("X-sorted-plan-C3-shuffled-K64", w3.index[torch.randperm(w3.E, generator=g)], w3.N, w3.E,
+                                64, torch.float32)
+        table["X-sorted-plan-C3-shuffled-K64"] = bench_sorted_config(ts, wl, ss, dev, max(it // 2, 3))
         table["X-softmax-K8"] = bench_softmax_config(ts, wl, w3, dev, max(it // 2, 3), 8)
         table["X-narrow-K1"] = bench_csr_config(ts, wl, dataclasses.replace(w3, K=1, name="X-narrow-K1"), dev, it,
                                                 ["segment_csr_sum", "segment_csr_max", "segment_coo_sum",
