@@ -162,6 +162,20 @@ int ts_scatter(const void *src, const int64_t *index, void *out,
                int64_t index_stride_k, int dtype, int reduce, int out_given,
                ts_stream_t stream);
 
+/* ts_scatter with an optional workspace (ts_scatter_workspace_bytes; 0 = no use for one). With it,
+ * MIN / MAX of contended rows of 64 bytes and more first bin the entries by bucket of output rows
+ * (8 bytes per entry) and reduce every bucket in LDS: no atomics on the table in memory except one
+ * write-back per chunk. Same results as ts_scatter. No counterpart in the reference
+ * (scatter_cuda allocates nothing beyond its outputs, csrc/cuda/scatter_cuda.cu:54-138). */
+size_t ts_scatter_workspace_bytes(int64_t B, int64_t E, int64_t K, int64_t N,
+                                  int dtype, int reduce);
+int ts_scatter_with_workspace(const void *src, const int64_t *index, void *out,
+                              int64_t *arg_out, int64_t B, int64_t E, int64_t K,
+                              int64_t N, int64_t index_stride_b,
+                              int64_t index_stride_e, int64_t index_stride_k,
+                              int dtype, int reduce, int out_given, void *workspace,
+                              size_t workspace_bytes, ts_stream_t stream);
+
 /* count[b, index[b*sb + e*se]] += 1 as float32, count pre-zeroed by the call.
  * The count half of ScatterMean::forward, csrc/scatter.cpp:131-137. */
 int ts_scatter_count(const int64_t *index, float *count, int64_t B, int64_t E,

@@ -326,9 +326,23 @@ int ts_segment_mean_coo_backward(const void *grad_out, const int64_t *index, con
   return dispatch_coo_gather(dtype, a, p, B, true, static_cast<hipStream_t>(stream));
 }
 
+size_t ts_scatter_workspace_bytes(int64_t B, int64_t E, int64_t K, int64_t N, int dtype, int reduce) {
+  if (!valid_dtype(dtype) || !sizes_ok(B, N, E, K) || (reduce != TS_MIN && reduce != TS_MAX)) return 0;
+  if (kElemBytes[dtype] > 4) return 0;  // 64-bit elements do not use packed keys
+  return bin_plan(B, E, K, N, kElemBytes[dtype], nullptr, 0, env_int("TS_SCATTER_BINNED", 1) == 2).bytes;
+}
+
 int ts_scatter(const void *src, const int64_t *index, void *out, int64_t *arg_out, int64_t B, int64_t E,
                int64_t K, int64_t N, int64_t index_stride_b, int64_t index_stride_e, int64_t index_stride_k,
                int dtype, int reduce, int out_given, ts_stream_t stream) {
+  return ts_scatter_with_workspace(src, index, out, arg_out, B, E, K, N, index_stride_b, index_stride_e,
+                                   index_stride_k, dtype, reduce, out_given, nullptr, 0, stream);
+}
+
+int ts_scatter_with_workspace(const void *src, const int64_t *index, void *out, int64_t *arg_out, int64_t B,
+                              int64_t E, int64_t K, int64_t N, int64_t index_stride_b, int64_t index_stride_e,
+                              int64_t index_stride_k, int dtype, int reduce, int out_given, void *workspace,
+                              size_t workspace_bytes, ts_stream_t stream) {
   if (!valid_dtype(dtype) || !sizes_ok(B, N, E, K)) return TS_ERR_BAD_ARG;
   if (reduce != TS_SUM && reduce != TS_MUL && reduce != TS_MIN && reduce != TS_MAX) return TS_ERR_UNSUPPORTED;
   if (B * N * K == 0) return TS_OK;
@@ -352,6 +366,11 @@ int ts_scatter(const void *src, const int64_t *index, void *out, int64_t *arg_ou
   a.lds_epb = env_int("TS_SCATTER_EPB", 0);
   a.run_reduce = env_int("TS_SCATTER_RUNS", 1);
   a.lds_k1 = env_int("TS_SCATTER_LDS_K1", 1);
+  if (const int binned = env_int("TS_SCATTER_BINNED", 1)) {  // tuning aid: 0 never, 2 at any size
+    a.bin_ws = workspace;
+    a.bin_ws_bytes = workspace_bytes;
+    a.bin_any_size = binned == 2;
+  }
   const int full = kVecBytes / kElemBytes[dtype];
   const int vec = (full > 1 && K % full == 0 && aligned16(src)) ? full : 1;
   return dispatch_scatter(dtype, a, reduce, vec, static_cast<hipStream_t>(stream));

@@ -205,6 +205,9 @@ struct ScatterArgs {
   int64_t lds_epb;     // entries per workgroup chunk of that variant, 0 = default
   int run_reduce = 1;  // sum: pre-reduce runs of equal neighbouring indices in the wavefront
   int lds_k1 = 1;      // min/max with K == 1: the 1024-lane table kernel
+  void *bin_ws = nullptr;  // optional workspace: min/max of wide rows through buckets of output rows
+  size_t bin_ws_bytes = 0;
+  int bin_any_size = 0;    // tuning aid / tests: also for inputs below the size from which it pays
 };
 
 // ---- thread -> (edge, column) mapping shared by the scatter kernels ------------
@@ -1327,6 +1330,10 @@ __global__ __launch_bounds__(kBlock) void scatter_arg_wide_kernel(ScatterArgs a)
   }
 }
 
+}  // namespace ts
+#include "scatter_binned.h"
+namespace ts {
+
 // ---- elementwise helpers --------------------------------------------------------
 template <typename T>
 __global__ __launch_bounds__(kBlock) void fill_kernel(T *p, int64_t n, T value) {
@@ -1489,13 +1496,30 @@ int launch_scatter_v(const ScatterArgs &a, int reduce, hipStream_t stream) {
       // index with few entries per slot is served better by the direct kernel)
       int tn = 1;
       while ((int64_t)tn * 2 * a.K <= kLdsKeys) tn *= 2;
-      const bool use_lds = a.lds_cache && a.sk == 0 && tn >= 64 && a.B * a.N < 0x7FFFFFFFll &&
-                           (a.lds_cache == 2 || (n_src >= ((int64_t)1 << 20) && n_edges >= 32 * a.B * a.N));
+      const bool contended = a.lds_cache && a.sk == 0 && a.B * a.N < 0x7FFFFFFFll &&
+                             (a.lds_cache == 2 || (n_src >= ((int64_t)1 << 20) && n_edges >= 32 * a.B * a.N));
+      const bool use_lds = contended && tn >= 64;
       // entries per workgroup chunk: large enough to amortise writing the table back,
       // small enough to leave a few thousand workgroups
       const int64_t epb = lds_chunk_edges(a.lds_epb, a.K, n_edges);
       const unsigned g_lds = (unsigned)((n_edges + epb - 1) / epb);
       const unsigned g_key = scatter_grid(n_edges, a.K / VEC, kBlock, 4);
+      if ((contended || a.bin_any_size) && a.sk == 0 && a.bin_ws != nullptr && a.K % VEC == 0 && n_src > 0) {
+        // contended wide rows with a workspace: entries binned by bucket of output rows, no table misses
+        const BinPlan bp = bin_plan(a.B, a.E, a.K, a.N, (int)sizeof(T), a.bin_ws, a.bin_ws_bytes, a.bin_any_size != 0);
+        if (bp.ok) {
+          if (is_max) {
+            hipLaunchKernelGGL((scatter_key_init_kernel<T, true>), dim3(g_out), dim3(kBlock), 0, stream, a);
+            launch_binned_keys<T, VEC, true>(a, bp.p, stream);
+            hipLaunchKernelGGL((scatter_key_final_kernel<T, true>), dim3(g_out), dim3(kBlock), 0, stream, a);
+          } else {
+            hipLaunchKernelGGL((scatter_key_init_kernel<T, false>), dim3(g_out), dim3(kBlock), 0, stream, a);
+            launch_binned_keys<T, VEC, false>(a, bp.p, stream);
+            hipLaunchKernelGGL((scatter_key_final_kernel<T, false>), dim3(g_out), dim3(kBlock), 0, stream, a);
+          }
+          return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
+        }
+      }
       // one index per row, few entries per slot: combine runs of equal neighbouring indices in the
       // wavefront before going to the table (a sorted index then costs one atomic per slot)
       if (!use_lds && a.run_reduce && a.sk == 0 && a.B * a.N < 0x7FFFFFFFll && n_src > 0) {

@@ -1,0 +1,310 @@
+// scatter min / max for wide rows through buckets of output rows (included by scatter.h).
+//
+// The packed-key table of one workgroup (scatter_key_lds_kernel) holds 128 rows of 32 keys; with a heavy-tailed
+// index a quarter of the entries miss it and go to the table in memory one 256-byte row at a time. Here the
+// entries are first binned by bucket of R consecutive output rows, R * K keys = 64 KB of LDS, so that a
+// workgroup which reduces (a chunk of) one bucket holds every row it can meet: no misses, no tags, and the
+// only traffic besides the stream is the table written back once per chunk.
+//   count  : per workgroup, a histogram of its entries over the buckets (LDS), added to the bucket totals
+//   scan   : bucket starts, chunks per bucket, the (bucket, chunk) of every reducing workgroup
+//   place  : every entry -> (row inside its bucket, entry number) at its bucket's next free slot (8 bytes)
+//   reduce : a workgroup per chunk of a bucket: rows of src by entry number, packed keys into the LDS table,
+//            table -> global table with a read before each atomic
+// The order inside a bucket is whatever the placement gives; the packed keys carry the positions, so the result
+// (value, first position among equal values) does not depend on it.
+#pragma once
+
+namespace ts {
+
+constexpr int kBinKeys = 8192;        // keys of the LDS table: 64 KB, two workgroups per CU
+constexpr int kBinBlock = 1024;
+constexpr int kBinMaxBuckets = 4096;  // LDS histogram of count / place
+constexpr int kBinChunk = 16384;      // entries per workgroup in count / place and per chunk in reduce
+
+struct BinArgs {
+  int rshift;              // log2 of the rows per bucket
+  int nb;                  // buckets
+  int64_t n_place;         // workgroups of count / place
+  int64_t max_wgs;         // workgroups of reduce (upper bound of the chunks)
+  unsigned long long *totals;  // [nb] entries per bucket
+  unsigned long long *cursor;  // [nb] next free slot
+  int64_t *starts;         // [nb + 1]
+  int32_t *chunk_start;    // [nb + 1]
+  int32_t *wg_bucket;      // [max_wgs] bucket of a reducing workgroup, -1: none
+  int32_t *wg_hist;        // [n_place][nb]
+  uint64_t *binned;        // [B * E] (row in bucket << 32) | entry number
+};
+
+struct BinPlan {
+  bool ok;
+  BinArgs p;
+  size_t bytes;
+};
+
+inline BinPlan bin_plan(int64_t B, int64_t E, int64_t K, int64_t N, int elem_bytes, void *ws, size_t ws_bytes,
+                        bool any_size = false) {
+  BinPlan r;
+  r.ok = false;
+  r.bytes = 0;
+  const int64_t n_edges = B * E, rows = B * N;
+  // rows of 64 bytes and more, inputs from 200 MB (below, the five extra launches cost more than the misses)
+  if (K * elem_bytes < 64 || K > kBinKeys / 16 || (!any_size && n_edges * K * elem_bytes < (int64_t)200000000) ||
+      n_edges >= 0xFFFFFFFEll || rows >= 0x7FFFFFFFll || rows < 1)
+    return r;
+  int rshift = 0;
+  while (((int64_t)2 << rshift) * K <= kBinKeys) ++rshift;
+  const int64_t nb = (rows + ((int64_t)1 << rshift) - 1) >> rshift;
+  if (nb > kBinMaxBuckets) return r;
+  BinArgs &p = r.p;
+  p.rshift = rshift;
+  p.nb = (int)nb;
+  p.n_place = (n_edges + kBinChunk - 1) / kBinChunk;
+  p.max_wgs = n_edges / kBinChunk + nb + 1;
+  auto up = [](size_t x) { return (x + 255) & ~(size_t)255; };
+  size_t off = 0;
+  auto take = [&](size_t bytes) { const size_t o = off; off += up(bytes); return o; };
+  const size_t o_tot = take((size_t)nb * 8), o_cur = take((size_t)nb * 8), o_st = take((size_t)(nb + 1) * 8);
+  const size_t o_cs = take((size_t)(nb + 1) * 4), o_wb = take((size_t)p.max_wgs * 4);
+  const size_t o_wh = take((size_t)p.n_place * nb * 4), o_bin = take((size_t)n_edges * 8);
+  r.bytes = off;
+  if (ws == nullptr || ws_bytes < off || (reinterpret_cast<uintptr_t>(ws) & 15) != 0) return r;
+  char *base = static_cast<char *>(ws);
+  p.totals = reinterpret_cast<unsigned long long *>(base + o_tot);
+  p.cursor = reinterpret_cast<unsigned long long *>(base + o_cur);
+  p.starts = reinterpret_cast<int64_t *>(base + o_st);
+  p.chunk_start = reinterpret_cast<int32_t *>(base + o_cs);
+  p.wg_bucket = reinterpret_cast<int32_t *>(base + o_wb);
+  p.wg_hist = reinterpret_cast<int32_t *>(base + o_wh);
+  p.binned = reinterpret_cast<uint64_t *>(base + o_bin);
+  r.ok = true;
+  return r;
+}
+
+// node (b * N + index) of entry be, -1 for an index outside [0, N)
+__device__ __forceinline__ int64_t bin_node(const ScatterArgs &a, int64_t be) {
+  int64_t b = 0, e = be;
+  if (a.B > 1) { b = be / a.E; e = be - b * a.E; }
+  const int64_t idx = a.index[b * a.sb + e * a.se];
+  return (idx >= 0 && idx < a.N) ? b * a.N + idx : -1;
+}
+
+constexpr int kBinPer = kBinChunk / kBinBlock;  // entries per lane in count / place
+
+// buckets of the kBinPer entries of a lane, all index loads in flight at once; -1: no bucket
+__device__ __forceinline__ void bin_buckets(const ScatterArgs &a, const BinArgs &p, int64_t lo, int64_t hi,
+                                            int32_t *bucket, int32_t *local) {
+  int64_t node[kBinPer];
+#pragma unroll
+  for (int j = 0; j < kBinPer; ++j) {
+    const int64_t be = lo + threadIdx.x + (int64_t)j * kBinBlock;
+    node[j] = be < hi ? bin_node(a, be) : -1;
+  }
+#pragma unroll
+  for (int j = 0; j < kBinPer; ++j) {
+    bucket[j] = node[j] >= 0 ? (int32_t)(node[j] >> p.rshift) : -1;
+    if (local != nullptr) local[j] = (int32_t)(node[j] & (((int64_t)1 << p.rshift) - 1));
+  }
+}
+
+// Adds 1 to counter[bucket] for every lane with bucket >= 0 and returns the value before the lane's own
+// addition. The lanes that share the bucket of the wavefront's first lane (with a heavy-tailed index: most of
+// them, the bucket of the hubs) go through one atomic of their leader; the others add on their own.
+__device__ __forceinline__ int32_t bin_take(int32_t *counter, int32_t bucket) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int32_t first = __builtin_amdgcn_readfirstlane(bucket);
+  const uint64_t same = __ballot(bucket == first && first >= 0);
+  int32_t before = 0;
+  if (same != 0) {
+    const int leader = __ffsll((unsigned long long)same) - 1;
+    int32_t base = 0;
+    if (lane == leader) base = atomicAdd(&counter[first], __popcll(same));
+    base = __shfl(base, leader);
+    before = base + __popcll(same & (((uint64_t)1 << lane) - 1));
+  }
+  if (bucket >= 0 && !((same >> lane) & 1)) before = atomicAdd(&counter[bucket], 1);
+  return before;
+}
+
+static __global__ __launch_bounds__(kBinBlock) void bin_count_kernel(ScatterArgs a, BinArgs p) {
+  __shared__ int32_t s_hist[kBinMaxBuckets];
+  for (int i = threadIdx.x; i < p.nb; i += kBinBlock) s_hist[i] = 0;
+  __syncthreads();
+  const int64_t lo = (int64_t)blockIdx.x * kBinChunk;
+  const int64_t hi = lo + kBinChunk < a.B * a.E ? lo + kBinChunk : a.B * a.E;
+  int32_t bucket[kBinPer];
+  bin_buckets(a, p, lo, hi, bucket, nullptr);
+#pragma unroll
+  for (int j = 0; j < kBinPer; ++j) bin_take(s_hist, bucket[j]);
+  __syncthreads();
+  for (int i = threadIdx.x; i < p.nb; i += kBinBlock) {
+    const int32_t h = s_hist[i];
+    p.wg_hist[(int64_t)blockIdx.x * p.nb + i] = h;
+    if (h != 0) atomicAdd(&p.totals[i], (unsigned long long)h);
+  }
+}
+
+// one workgroup: prefix sums over the buckets and the list of reducing workgroups
+static __global__ __launch_bounds__(kBinBlock) void bin_scan_kernel(BinArgs p) {
+  constexpr int PER = kBinMaxBuckets / kBinBlock;
+  __shared__ int64_t s_t[kBinBlock];
+  __shared__ int64_t s_c[kBinBlock];
+  int64_t t[PER], c[PER], sum_t = 0, sum_c = 0;
+#pragma unroll
+  for (int j = 0; j < PER; ++j) {
+    const int i = threadIdx.x * PER + j;
+    t[j] = i < p.nb ? (int64_t)p.totals[i] : 0;
+    c[j] = (t[j] + kBinChunk - 1) / kBinChunk;
+    sum_t += t[j];
+    sum_c += c[j];
+  }
+  s_t[threadIdx.x] = sum_t;
+  s_c[threadIdx.x] = sum_c;
+  __syncthreads();
+  for (int d = 1; d < kBinBlock; d <<= 1) {  // inclusive scan over the threads
+    int64_t vt = 0, vc = 0;
+    if ((int)threadIdx.x >= d) { vt = s_t[threadIdx.x - d]; vc = s_c[threadIdx.x - d]; }
+    __syncthreads();
+    s_t[threadIdx.x] += vt;
+    s_c[threadIdx.x] += vc;
+    __syncthreads();
+  }
+  int64_t run_t = s_t[threadIdx.x] - sum_t, run_c = s_c[threadIdx.x] - sum_c;
+  const int64_t all_c = s_c[kBinBlock - 1];
+#pragma unroll
+  for (int j = 0; j < PER; ++j) {
+    const int i = threadIdx.x * PER + j;
+    if (i < p.nb) {
+      p.starts[i] = run_t;
+      p.cursor[i] = (unsigned long long)run_t;
+      p.chunk_start[i] = (int32_t)run_c;
+    }
+    if (i == p.nb) { p.starts[i] = run_t; p.chunk_start[i] = (int32_t)run_c; }
+    run_t += t[j];
+    run_c += c[j];
+  }
+  if (threadIdx.x == kBinBlock - 1 && p.nb == kBinMaxBuckets) {
+    p.starts[p.nb] = run_t;
+    p.chunk_start[p.nb] = (int32_t)run_c;
+  }
+  __syncthreads();  // chunk_start is complete (written and read by this one workgroup)
+  __threadfence_block();
+  for (int64_t k = threadIdx.x; k < p.max_wgs; k += kBinBlock) {
+    int32_t b = -1;
+    if (k < all_c) {  // the bucket whose chunks include k: last i with chunk_start[i] <= k
+      int lo = 0, hi = p.nb - 1;
+      while (lo < hi) {
+        const int mid = (lo + hi + 1) >> 1;
+        if (p.chunk_start[mid] <= k) lo = mid; else hi = mid - 1;
+      }
+      b = lo;
+    }
+    p.wg_bucket[k] = b;
+  }
+}
+
+static __global__ __launch_bounds__(kBinBlock) void bin_place_kernel(ScatterArgs a, BinArgs p) {
+  __shared__ uint32_t s_base[kBinMaxBuckets];
+  __shared__ int32_t s_cnt[kBinMaxBuckets];
+  for (int i = threadIdx.x; i < p.nb; i += kBinBlock) {
+    const int32_t h = p.wg_hist[(int64_t)blockIdx.x * p.nb + i];
+    s_base[i] = h != 0 ? (uint32_t)atomicAdd(&p.cursor[i], (unsigned long long)h) : 0u;
+    s_cnt[i] = 0;
+  }
+  __syncthreads();
+  const int64_t lo = (int64_t)blockIdx.x * kBinChunk;
+  const int64_t hi = lo + kBinChunk < a.B * a.E ? lo + kBinChunk : a.B * a.E;
+  int32_t bucket[kBinPer], local[kBinPer];
+  bin_buckets(a, p, lo, hi, bucket, local);
+#pragma unroll
+  for (int j = 0; j < kBinPer; ++j) {
+    const int32_t rank = bin_take(s_cnt, bucket[j]);
+    if (bucket[j] < 0) continue;
+    const int64_t be = lo + threadIdx.x + (int64_t)j * kBinBlock;
+    p.binned[s_base[bucket[j]] + (uint32_t)rank] = ((uint64_t)(uint32_t)local[j] << 32) | (uint32_t)be;
+  }
+}
+
+template <typename T, int VEC, bool IS_MAX>
+__global__ __launch_bounds__(kBinBlock) void bin_reduce_kernel(ScatterArgs a, BinArgs p) {
+  constexpr int U = 4;  // 63 VGPRs: two workgroups per CU (eight rows in flight per lane: 74 VGPRs, one workgroup)
+  // rows are K + 1 keys apart: with K a multiple of 32 the rows would all start in the same LDS bank and the
+  // lanes of a wavefront, which hold the same columns of different rows, would queue up behind each other
+  __shared__ uint64_t s_keys[kBinKeys + kBinKeys / 16];
+  const int bucket = p.wg_bucket[blockIdx.x];
+  if (bucket < 0) return;
+  const int K = (int)a.K;
+  const int KP = K + 1;
+  const int rows = 1 << p.rshift;
+  for (int i = threadIdx.x; i < rows * KP; i += kBinBlock) s_keys[i] = 0;
+  __syncthreads();
+
+  const T *src = static_cast<const T *>(a.src);
+  const int64_t lo = p.starts[bucket] + ((int64_t)blockIdx.x - p.chunk_start[bucket]) * kBinChunk;
+  int64_t hi = lo + kBinChunk;
+  if (hi > p.starts[bucket + 1]) hi = p.starts[bucket + 1];
+  const EdgeLanes m = edge_lanes(K / VEC, kBinBlock);  // K / VEC <= 512: one column slice per lane
+  if (m.active) {
+    const int k0 = m.cl * VEC;
+    for (int64_t s0 = lo + m.el; s0 < hi; s0 += (int64_t)m.epp * U) {
+      uint64_t ent[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int64_t s = s0 + (int64_t)u * m.epp;
+        ent[u] = p.binned[s < hi ? s : s0];
+      }
+      Vec<T, VEC> x[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) x[u] = load_vec_stream<T, VEC>(src + (int64_t)(uint32_t)ent[u] * a.K + k0);
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        if (s0 + (int64_t)u * m.epp >= hi) continue;
+        int64_t e = (int64_t)(uint32_t)ent[u];
+        if (a.B > 1) e -= (e / a.E) * a.E;  // position inside the batch
+        uint64_t key[VEC];
+        make_keys<T, VEC, IS_MAX>(x[u], e, key);
+        uint64_t *row = &s_keys[(int)(ent[u] >> 32) * KP + k0];
+        // filter on the value half (one 32-bit LDS read per element): below the cached key cannot win
+        const volatile uint32_t *hi32 = reinterpret_cast<const volatile uint32_t *>(row) + 1;
+#pragma unroll
+        for (int v = 0; v < VEC; ++v)
+          if (key[v] != 0 && (uint32_t)(key[v] >> 32) >= hi32[2 * v])
+            __hip_atomic_fetch_max(row + v, key[v], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      }
+    }
+  }
+  __syncthreads();
+  // the chunk's winners -> global table
+  uint64_t *gkeys = reinterpret_cast<uint64_t *>(a.arg_out) + ((int64_t)bucket << p.rshift) * a.K;
+  const int64_t limit = (a.B * a.N - ((int64_t)bucket << p.rshift)) * a.K;  // keys of rows that exist
+  const int table = K << p.rshift;
+  for (int i0 = threadIdx.x; i0 < table; i0 += kBinBlock * 4) {
+    uint64_t key[4], cur[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int i = i0 + j * kBinBlock;
+      key[j] = (i < table && i < limit) ? s_keys[i + i / K] : 0;  // row i / K starts i / K keys later
+      if (key[j] != 0) cur[j] = gkeys[i];
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if (key[j] != 0 && key[j] > cur[j])
+        __hip_atomic_fetch_max(gkeys + i0 + j * kBinBlock, key[j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+
+static __global__ __launch_bounds__(kBlock) void bin_clear_kernel(unsigned long long *totals, int n) {
+  const int i = blockIdx.x * kBlock + threadIdx.x;
+  if (i < n) totals[i] = 0;
+}
+
+// the passes between scatter_key_init_kernel and scatter_key_final_kernel
+template <typename T, int VEC, bool IS_MAX>
+void launch_binned_keys(const ScatterArgs &a, const BinArgs &p, hipStream_t stream) {
+  hipLaunchKernelGGL(bin_clear_kernel, dim3((p.nb + kBlock - 1) / kBlock), dim3(kBlock), 0, stream, p.totals, p.nb);
+  hipLaunchKernelGGL(bin_count_kernel, dim3((unsigned)p.n_place), dim3(kBinBlock), 0, stream, a, p);
+  hipLaunchKernelGGL(bin_scan_kernel, dim3(1), dim3(kBinBlock), 0, stream, p);
+  hipLaunchKernelGGL(bin_place_kernel, dim3((unsigned)p.n_place), dim3(kBinBlock), 0, stream, a, p);
+  hipLaunchKernelGGL((bin_reduce_kernel<T, VEC, IS_MAX>), dim3((unsigned)p.max_wgs), dim3(kBinBlock), 0, stream, a, p);
+}
+
+}  // namespace ts

@@ -173,9 +173,15 @@ std::tuple<Tensor, OptTensor> scatter_hip(Tensor src, Tensor index, int64_t dim,
     se = K;
     sk = 1;
   }
-  check_status(ts_scatter(src.data_ptr(), index.data_ptr<int64_t>(), out.data_ptr(),
-                          minmax ? arg_out.value().data_ptr<int64_t>() : nullptr, B, E, K, N, sb.value(), se,
-                          sk.value(), dtype_code(src), reduce, optional_out.has_value() ? 1 : 0, stream_of(src)),
+  // min / max of large inputs with wide rows can use scratch memory (entries binned by bucket of output rows)
+  const size_t ws_bytes = sk.value() == 0 ? ts_scatter_workspace_bytes(B, E, K, N, dtype_code(src), reduce) : 0;
+  Tensor ws;
+  if (ws_bytes > 0) ws = workspace(ws_bytes, src);
+  check_status(ts_scatter_with_workspace(src.data_ptr(), index.data_ptr<int64_t>(), out.data_ptr(),
+                                         minmax ? arg_out.value().data_ptr<int64_t>() : nullptr, B, E, K, N,
+                                         sb.value(), se, sk.value(), dtype_code(src), reduce,
+                                         optional_out.has_value() ? 1 : 0, ws_bytes > 0 ? ws.data_ptr() : nullptr,
+                                         ws_bytes, stream_of(src)),
                "scatter");
   return std::make_tuple(out, arg_out);
 }

@@ -527,6 +527,44 @@ def test_scatter_minmax_lds_cached_variant(capi, oracle, shape, reduce, dtype, m
         assert_exact(arg, want_arg)
 
 
+@pytest.mark.parametrize("shape,reduce,dtype", product(
+    [(1, 60000, 32, 300), (2, 40000, 16, 700), (1, 50000, 128, 90), (1, 30000, 24, 5000), (1, 20000, 64, 100000),
+     (3, 9000, 512, 5), (1, 70000, 17, 40)],
+    ["min", "max"], [torch.float32, torch.bfloat16, torch.int32, torch.int8]))
+def test_scatter_minmax_binned_variant(capi, oracle, shape, reduce, dtype, monkeypatch):
+    """min / max with a workspace: entries binned by bucket of output rows and reduced in LDS (forced on at
+    these sizes), skewed index with heavy ties, with and without previous content in out. Rows under 64 bytes
+    (int8 at K < 64, ...) keep the path without workspace."""
+    monkeypatch.setenv("TS_SCATTER_BINNED", "2")
+    B, E, K, N = shape
+    rng = np.random.default_rng(E + K)
+    src = random_values(rng, (B, E, K), dtype, ties=True)
+    p = np.arange(1, N + 1, dtype=np.float64) ** -1.2
+    idx = rng.choice(N, size=E, p=p / p.sum())
+    index1 = torch.from_numpy(idx)
+    index = index1.view(1, E, 1).expand(B, E, K)
+    for out_given in (False, True):
+        if out_given:
+            prev = random_values(rng, (B, N, K), dtype, ties=True)
+            want = prev.clone()
+            _, want_arg = oracle.scatter(src, index, 1, want, None, reduce)
+            out = prev.clone().to(DEV)
+        else:
+            want, want_arg = oracle.scatter(src, index, 1, None, N, reduce)
+            out = torch.empty((B, N, K), dtype=dtype, device=DEV)
+        arg = torch.empty((B, N, K), dtype=torch.long, device=DEV)
+        capi.scatter_with_workspace(src.to(DEV), index1.to(DEV), out, arg, B, E, K, N, 0, 1, 0, capi.REDUCE[reduce],
+                                    out_given)
+        torch.cuda.synchronize()
+        assert_exact(out, want)
+        assert_exact(arg, want_arg)
+    L = capi.lib()
+    need = L.ts_scatter_workspace_bytes(capi._i(B), capi._i(E), capi._i(K), capi._i(N), capi.DTYPE[dtype],
+                                        capi.REDUCE[reduce])
+    assert (need > 0) == (K * src.element_size() >= 64 and K <= 512)
+    assert L.ts_scatter_workspace_bytes(capi._i(B), capi._i(E), capi._i(K), capi._i(N), capi.DTYPE[dtype], capi.SUM) == 0
+
+
 @pytest.mark.parametrize("shape,dtype", product(
     [(1, 30000, 1, 500), (1, 9000, 32, 300), (2, 5000, 8, 40), (1, 4000, 12, 70000)],
     [torch.float32, torch.bfloat16, torch.float16]))
