@@ -55,6 +55,8 @@ struct CsrReduceArgs {
   // sorted once: perm = stable argsort of the index). Positions handed to arg_out stay in row-pointer order.
   const int32_t *perm;
   int64_t perm_batch_stride;
+  int perm_args;      // min / max with perm: the kernel itself writes positions in src's order and applies
+                      // scatter's rule for slots that never beat the initial value (no pass over arg_out after it)
 };
 
 // ---- rows that cross tiles, finished without a second kernel ---------------------------------
@@ -106,10 +108,10 @@ __device__ __forceinline__ void reduce_step(A &acc, int32_t &arg, A v, int32_t e
 // Write one finished row slice. `count` is the full length of the row.
 // ACCUM: 0 = `out` is overwritten (known at compile time: the row-end code sits in divergent control flow,
 // where every instruction counts), -1 = decided by a.accumulate at run time.
-template <typename T, int VEC, int REDUCE, int ACCUM = -1>
+template <typename T, int VEC, int REDUCE, int ACCUM = -1, bool PERM = false>
 __device__ __forceinline__ void finalize_row_at(const CsrReduceArgs &a, T *op, int64_t *ap, T *count_slot,
                                                 const typename Acc<T>::type *acc, const int32_t *arg,
-                                                int64_t count) {
+                                                int64_t count, const int32_t *perm_b = nullptr) {
   // op / ap: the row's slice in out / arg_out; count_slot: where the row's count goes (mean with a count output)
   typedef typename Acc<T>::type A;
   const bool accumulate = ACCUM < 0 ? a.accumulate != 0 : ACCUM != 0;
@@ -135,6 +137,20 @@ __device__ __forceinline__ void finalize_row_at(const CsrReduceArgs &a, T *op, i
       } else {
         o.v[v] = count > 0 ? from_acc<T>(x) : zero_elem<T>();
         oa[v] = count > 0 ? (int64_t)arg[v] : a.E;
+        if constexpr (PERM) {
+          if (perm_b != nullptr && count > 0) {
+            // scatter's view of the slot: the position in src's order, or 0 and E if nothing beat the initial
+            // value of the element type (csrc/cpu/scatter_cpu.cpp:81-82)
+            const A lim = to_acc<T>(REDUCE == TS_MAX ? ElemLim<T>::lowest() : ElemLim<T>::max());
+            const A xv = to_acc<T>(o.v[v]);
+            if ((REDUCE == TS_MAX) ? (xv > lim) : (xv < lim)) {
+              oa[v] = perm_b[arg[v]];
+            } else {
+              o.v[v] = zero_elem<T>();
+              oa[v] = a.E;
+            }
+          }
+        }
       }
     }
   }
@@ -146,16 +162,16 @@ __device__ __forceinline__ void finalize_row_at(const CsrReduceArgs &a, T *op, i
   if (REDUCE == TS_MEAN && count_slot != nullptr) *count_slot = count_as<T>(count > 0 ? count : 1);
 }
 
-template <typename T, int VEC, int REDUCE, int ACCUM = -1>
+template <typename T, int VEC, int REDUCE, int ACCUM = -1, bool PERM = false>
 __device__ __forceinline__ void finalize_row(const CsrReduceArgs &a, T *out_b, int64_t *arg_b,
                                              T *count_b, int64_t row, int64_t col, int lg,
                                              const typename Acc<T>::type *acc, const int32_t *arg,
-                                             int64_t count, bool col_ok) {
+                                             int64_t count, bool col_ok, const int32_t *perm_b = nullptr) {
   if (!col_ok) return;
   constexpr bool kArg = REDUCE == TS_MIN || REDUCE == TS_MAX;
-  finalize_row_at<T, VEC, REDUCE, ACCUM>(a, out_b + row * a.K + col, kArg ? arg_b + row * a.K + col : nullptr,
-                                         (count_b != nullptr && col == 0 && lg == 0) ? count_b + row : nullptr,
-                                         acc, arg, count);
+  finalize_row_at<T, VEC, REDUCE, ACCUM, PERM>(a, out_b + row * a.K + col, kArg ? arg_b + row * a.K + col : nullptr,
+                                               (count_b != nullptr && col == 0 && lg == 0) ? count_b + row : nullptr,
+                                               acc, arg, count, perm_b);
 }
 
 // Workgroups per CU the register allocation aims at: six for sum / mean of 4- and 8-byte types (80 VGPRs;
@@ -215,9 +231,11 @@ __global__ __launch_bounds__(kBlock, (csr_reduce_min_blocks<T, VEC, REDUCE, PERM
   const int nload = (int)(last - i0) + 1;  // ptr[i0 .. last]
   for (int t = tid; t < nload; t += kBlock) s_ptr[t] = (int32_t)(ptr[i0 + t] - j0);
   if (tid == 0) { s_ptr[nload] = INT32_MAX; s_ptr[nload + 1] = INT32_MAX; }  // rows past the last one never end
+  const int32_t *arg_perm = nullptr;  // set: positions leave the kernel in src's order
   if constexpr (PERM) {
-    const int32_t *perm_b = a.perm + b * a.perm_batch_stride + j0;
-    for (int t = tid; t < ne; t += kBlock) s_perm[t] = perm_b[t];
+    const int32_t *perm_b = a.perm + b * a.perm_batch_stride;
+    for (int t = tid; t < ne; t += kBlock) s_perm[t] = perm_b[j0 + t];
+    if (kArg && a.perm_args) arg_perm = perm_b;
   }
   s_head_row[tid] = -1;
   s_tail_row[tid] = -1;
@@ -268,8 +286,8 @@ __global__ __launch_bounds__(kBlock, (csr_reduce_min_blocks<T, VEC, REDUCE, PERM
       }
       if (lg == 0) { s_head_row[w] = r; s_head_closes[w] = 1; }
     } else if (col_ok) {
-      finalize_row_at<T, VEC, REDUCE, ACCUM>(a, op_row, ap_row, cp_row, acc, arg,
-                                             (int64_t)(int32_t)(rend - rbeg));  // a row length fits 32 bits
+      finalize_row_at<T, VEC, REDUCE, ACCUM, PERM>(a, op_row, ap_row, cp_row, acc, arg,
+                                                   (int64_t)(int32_t)(rend - rbeg), arg_perm);  // the length fits 32 bits
     }
 #pragma unroll
     for (int v = 0; v < VEC; ++v) acc[v] = acc_init<A, REDUCE>();
@@ -472,8 +490,8 @@ __global__ __launch_bounds__(kBlock, (csr_reduce_min_blocks<T, VEC, REDUCE, PERM
       closed = s_head_closes[ww] != 0;
     }
     if (closed) {
-      finalize_row<T, VEC, REDUCE, ACCUM>(a, out_b, arg_b, count_b, i0 + row, col, lg, acc, arg,
-                                   (int64_t)s_ptr[row + 1] - (int64_t)s_ptr[row], col_ok);
+      finalize_row<T, VEC, REDUCE, ACCUM, PERM>(a, out_b, arg_b, count_b, i0 + row, col, lg, acc, arg,
+                                                (int64_t)s_ptr[row + 1] - (int64_t)s_ptr[row], col_ok, arg_perm);
     } else if (lookback) {
       publish_carry(kCarryTail);
     } else {
@@ -513,8 +531,8 @@ __global__ __launch_bounds__(kBlock, (csr_reduce_min_blocks<T, VEC, REDUCE, PERM
             if (lg == 0) s_cut[0] = first_tile;
           } else {
             walk_back(first_tile, (int64_t)blockIdx.x - 1, 1);
-            finalize_row<T, VEC, REDUCE, ACCUM>(a, out_b, arg_b, count_b, i0 + row, col, lg, acc, arg,
-                                                (int64_t)s_ptr[row + 1] - (int64_t)s_ptr[row], col_ok);
+            finalize_row<T, VEC, REDUCE, ACCUM, PERM>(a, out_b, arg_b, count_b, i0 + row, col, lg, acc, arg,
+                                                      (int64_t)s_ptr[row + 1] - (int64_t)s_ptr[row], col_ok, arg_perm);
           }
         } else {
           publish_carry(kCarryPass);
@@ -570,8 +588,8 @@ __global__ __launch_bounds__(kBlock, (csr_reduce_min_blocks<T, VEC, REDUCE, PERM
       }
     }
     const int row = s_head_row[0];
-    finalize_row<T, VEC, REDUCE, ACCUM>(a, out_b, arg_b, count_b, i0 + row, col, lg, acc, arg,
-                                        (int64_t)s_ptr[row + 1] - (int64_t)s_ptr[row], col_ok);
+    finalize_row<T, VEC, REDUCE, ACCUM, PERM>(a, out_b, arg_b, count_b, i0 + row, col, lg, acc, arg,
+                                              (int64_t)s_ptr[row + 1] - (int64_t)s_ptr[row], col_ok, arg_perm);
   }
 }
 

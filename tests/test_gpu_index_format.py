@@ -300,3 +300,26 @@ def test_hub_row_through_many_tiles(capi, oracle, K, dtype):
         assert torch.equal(out2.cpu(), want if reduce == "sum" else want2[0]), reduce
         if arg2 is not None:
             assert torch.equal(arg2.cpu(), want_arg2[0]), reduce
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.int32, torch.uint8])
+def test_permuted_minmax_with_a_large_output(capi, oracle, dtype):
+    """From 8 M output elements on, the reduction writes the positions in src's order itself (no pass over
+    arg_out afterwards), including scatter's rule for slots that never beat the initial value (uint8 zeros
+    under max). Values and positions bit-exact against the oracle's scatter."""
+    rng = np.random.default_rng(23)
+    B, E, K, N = 1, 150_000, 128, 70_000
+    index1 = make_index("gaps", rng, E, N)
+    index1[: E // 5] = 31  # a row through many tiles
+    index1 = index1[torch.from_numpy(rng.permutation(E))]
+    perm, indptr = sort_on_gpu(capi, index1, N)
+    src = random_values(rng, (B, E, K), dtype, ties=True)
+    index = index1.view(1, E, 1).expand(B, E, K)
+    for reduce in ("min", "max"):
+        want, want_arg = oracle.scatter(src, index, 1, None, N, reduce)
+        out = torch.empty((B, N, K), dtype=dtype, device=DEV)
+        arg = torch.empty((B, N, K), dtype=torch.long, device=DEV)
+        capi.segment_csr_permuted(src.to(DEV), perm, indptr, out, arg, B, N, E, K, 0, 0, capi.REDUCE[reduce])
+        torch.cuda.synchronize()
+        assert torch.equal(out.cpu(), want), reduce
+        assert torch.equal(arg.cpu(), want_arg), reduce
