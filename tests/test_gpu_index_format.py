@@ -323,3 +323,41 @@ def test_permuted_minmax_with_a_large_output(capi, oracle, dtype):
         torch.cuda.synchronize()
         assert torch.equal(out.cpu(), want), reduce
         assert torch.equal(arg.cpu(), want_arg), reduce
+
+
+def test_sorted_and_binned_scatter_under_graph_replay(ts, oracle, monkeypatch):
+    """scatter_sorted (a hub row that the whole workgroup walks back over; carry flags in the workspace are
+    cleared by their readers) and scatter_max with its workspace path, captured once and replayed three times
+    with fresh inputs and eager work in between; every replay is checked."""
+    monkeypatch.setenv("TS_SCATTER_BINNED", "2")
+    g = torch.Generator().manual_seed(29)
+    E, N, K = 200_000, 300, 32
+    index = torch.randint(0, N, (E,), generator=g)
+    index[: E // 2] = 5  # 100 000 entries: about fifty tiles
+    index = index[torch.randperm(E, generator=g)]
+    d_index = index.to(DEV)
+    plan = ts.SortedIndex(d_index, N)
+    static_src = torch.zeros(E, K, device=DEV)
+    for _ in range(2):  # warm-up outside the capture
+        ts.scatter_sorted(static_src, plan, 0, "sum")
+        ts.scatter_sorted(static_src, plan, 0, "max")
+        ts.scatter_max(static_src, d_index, 0, None, N)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        s_sum = ts.scatter_sorted(static_src, plan, 0, "sum")
+        s_max, s_arg = ts.scatter_sorted(static_src, plan, 0, "max")
+        b_max, b_arg = ts.scatter_max(static_src, d_index, 0, None, N)
+    full = index.view(E, 1).expand(E, K)
+    for rep in range(3):
+        src = torch.randint(-20, 21, (E, K), generator=g).float()
+        static_src.copy_(src.to(DEV))
+        graph.replay()
+        torch.cuda.synchronize()
+        want_sum = oracle.scatter(src, full, 0, None, N, "sum")[0]
+        want_max, want_arg = oracle.scatter(src, full, 0, None, N, "max")
+        assert torch.equal(s_sum.cpu(), want_sum), rep  # small integers: exact
+        assert torch.equal(s_max.cpu(), want_max) and torch.equal(s_arg.cpu(), want_arg), rep
+        assert torch.equal(b_max.cpu(), want_max) and torch.equal(b_arg.cpu(), want_arg), rep
+        eager = ts.scatter_sorted(static_src, plan, 0, "sum")
+        assert torch.equal(eager, s_sum)
