@@ -31,6 +31,10 @@ torch.ops.load_library(_OPS_LIB)
 
 hip_version = torch.ops.torch_scatter.cuda_version()  # HIP_VERSION of the build
 
+from .index_format import (SortedIndex, index_to_indptr, indptr_to_index,  # noqa: E402
+                           scatter_sorted)
+from .index_reuse import (disable_index_reuse, enable_index_reuse,  # noqa: E402
+                          index_reuse_enabled)
 from .scatter import (scatter, scatter_add, scatter_max, scatter_mean,  # noqa: E402
                       scatter_min, scatter_mul, scatter_sum)
 from .segment_coo import (gather_coo, segment_add_coo, segment_coo,  # noqa: E402
@@ -41,8 +45,6 @@ from .segment_csr import (gather_csr, segment_add_csr, segment_csr,  # noqa: E40
                           segment_sum_csr)
 from .composite import (scatter_log_softmax, scatter_logsumexp,  # noqa: E402
                         scatter_softmax, scatter_std)
-from .index_format import (SortedIndex, index_to_indptr, indptr_to_index,  # noqa: E402
-                           scatter_sorted)
 
 __all__ = [
     "scatter_sum", "scatter_add", "scatter_mul", "scatter_mean", "scatter_min",
@@ -53,5 +55,6 @@ __all__ = [
     "segment_max_coo", "segment_coo", "gather_coo",
     "scatter_std", "scatter_logsumexp", "scatter_softmax", "scatter_log_softmax",
     "SortedIndex", "index_to_indptr", "indptr_to_index", "scatter_sorted",
+    "enable_index_reuse", "disable_index_reuse", "index_reuse_enabled",
     "hip_version", "__version__",
 ]

@@ -361,3 +361,58 @@ def test_sorted_and_binned_scatter_under_graph_replay(ts, oracle, monkeypatch):
         assert torch.equal(b_max.cpu(), want_max) and torch.equal(b_arg.cpu(), want_arg), rep
         eager = ts.scatter_sorted(static_src, plan, 0, "sum")
         assert torch.equal(eager, s_sum)
+
+
+def test_index_reuse_front_end(ts):
+    """Off: scatter runs the atomic kernels. On: the first call with an index still does, the second sorts the
+    index once and from then on scatter runs as a segmented reduction over permuted rows (bit-identical
+    results call after call, positions equal to scatter_max's); an in-place change of the index, another
+    dim_size, `out=`, narrow rows and a 2-D index are not taken from the cache."""
+    from pytorch_scatter_amd import index_reuse
+    g = torch.Generator().manual_seed(31)
+    E, N, K = 50_000, 700, 32
+    index = torch.randint(0, N, (E,), generator=g).to(DEV)
+    src = torch.randint(-9, 10, (E, K), generator=g).float().to(DEV)
+    assert not ts.index_reuse_enabled()
+    base_sum = ts.scatter_sum(src, index, 0, None, N)
+    base_max, base_arg = ts.scatter_max(src, index, 0, None, N)
+    assert len(index_reuse._cache) == 0
+    ts.enable_index_reuse(max_plans=3)
+    try:
+        first = ts.scatter_sum(src, index, 0, None, N)          # first sighting: remembered, no plan yet
+        (entry,) = index_reuse._cache.values()
+        assert entry[2] is None
+        second = ts.scatter_sum(src, index, 0, None, N)         # second sighting: sorted once
+        assert entry[2] is not None
+        plan = entry[2]
+        assert torch.equal(first, base_sum) and torch.equal(second, base_sum)  # small integers: exact sums
+        got_max, got_arg = ts.scatter_max(src, index, 0, None, N)
+        assert entry[2] is plan and torch.equal(got_max, base_max) and torch.equal(got_arg, base_arg)
+        x = src.clone().requires_grad_(True)
+        ts.scatter_mean(x, index, 0, None, N).sum().backward()
+        y = src.clone().requires_grad_(True)
+        torch.ops.torch_scatter.scatter_mean(y, index, 0, None, N).sum().backward()
+        assert torch.allclose(x.grad, y.grad)
+        # dim_size is part of the key; so is the version counter of the index
+        assert ts.scatter_sum(src, index, 0, None, N + 5).shape[0] == N + 5
+        assert len(index_reuse._cache) == 2
+        index[0] = (index[0] + 1) % N
+        moved = ts.scatter_sum(src, index, 0, None, N)
+        assert torch.equal(moved, torch.ops.torch_scatter.scatter_sum(src, index, 0, None, N))
+        assert torch.equal(ts.scatter_sum(src, index, 0, None, N), moved)  # plan of the changed index
+        assert len(index_reuse._cache) == 3
+        # not eligible: out given, rows under 64 bytes, an index of the shape of src
+        before = len(index_reuse._cache)
+        ts.scatter_sum(src, index, 0, torch.zeros(N, K, device=DEV))
+        ts.scatter_sum(src[:, :4].contiguous(), index, 0, None, N)
+        ts.scatter_sum(src, index.view(E, 1).expand(E, K), 0, None, N)
+        assert len(index_reuse._cache) == before
+        # least recently used out
+        for i in range(4):
+            ts.scatter_sum(src, torch.randint(0, N, (E,), generator=g).to(DEV), 0, None, N)
+        assert len(index_reuse._cache) == 3
+        # scripted wrappers keep going to the operator
+        assert torch.equal(torch.jit.script(ts.scatter_sum)(src, index, 0, None, N), moved)
+    finally:
+        ts.disable_index_reuse()
+    assert len(index_reuse._cache) == 0 and not ts.index_reuse_enabled()
