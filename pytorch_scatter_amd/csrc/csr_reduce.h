@@ -234,7 +234,11 @@ __global__ __launch_bounds__(kBlock, (csr_reduce_min_blocks<T, VEC, REDUCE, PERM
   const int32_t *arg_perm = nullptr;  // set: positions leave the kernel in src's order
   if constexpr (PERM) {
     const int32_t *perm_b = a.perm + b * a.perm_batch_stride;
-    for (int t = tid; t < ne; t += kBlock) s_perm[t] = perm_b[j0 + t];
+    const int32_t last_row = a.E > 0 ? (int32_t)(a.E - 1) : 0;
+    for (int t = tid; t < ne; t += kBlock) {
+      const int32_t r = perm_b[j0 + t];
+      s_perm[t] = r < 0 ? 0 : (r > last_row ? last_row : r);  // a malformed perm must not read outside src
+    }
     if (kArg && a.perm_args) arg_perm = perm_b;
   }
   s_head_row[tid] = -1;
