@@ -19,7 +19,9 @@ namespace ts {
 constexpr int kBinKeys = 8192;        // keys of the LDS table: 64 KB, two workgroups per CU
 constexpr int kBinBlock = 1024;
 constexpr int kBinMaxBuckets = 4096;  // LDS histogram of count / place
-constexpr int kBinChunk = 16384;      // entries per workgroup in count / place and per chunk in reduce
+constexpr int kBinChunk = 16384;      // entries per chunk of a bucket in reduce
+constexpr int kBinPlaceChunk = 16384;  // entries per workgroup in count / place: one batch of 16 per lane
+constexpr int kBinPlaceBlock = 1024;   // (measured slower: 256 lanes x 4 batches, 64 K entries per workgroup, 8 K)
 
 struct BinArgs {
   int rshift;              // log2 of the rows per bucket
@@ -58,7 +60,7 @@ inline BinPlan bin_plan(int64_t B, int64_t E, int64_t K, int64_t N, int elem_byt
   BinArgs &p = r.p;
   p.rshift = rshift;
   p.nb = (int)nb;
-  p.n_place = (n_edges + kBinChunk - 1) / kBinChunk;
+  p.n_place = (n_edges + kBinPlaceChunk - 1) / kBinPlaceChunk;
   p.max_wgs = n_edges / kBinChunk + nb + 1;
   auto up = [](size_t x) { return (x + 255) & ~(size_t)255; };
   size_t off = 0;
@@ -88,7 +90,8 @@ __device__ __forceinline__ int64_t bin_node(const ScatterArgs &a, int64_t be) {
   return (idx >= 0 && idx < a.N) ? b * a.N + idx : -1;
 }
 
-constexpr int kBinPer = kBinChunk / kBinBlock;  // entries per lane in count / place
+constexpr int kBinPer = 16;  // entries per lane and batch in count / place (all index loads of a batch in flight)
+constexpr int kBinBatch = kBinPer * kBinPlaceBlock;
 
 // buckets of the kBinPer entries of a lane, all index loads in flight at once; -1: no bucket
 __device__ __forceinline__ void bin_buckets(const ScatterArgs &a, const BinArgs &p, int64_t lo, int64_t hi,
@@ -96,7 +99,7 @@ __device__ __forceinline__ void bin_buckets(const ScatterArgs &a, const BinArgs 
   int64_t node[kBinPer];
 #pragma unroll
   for (int j = 0; j < kBinPer; ++j) {
-    const int64_t be = lo + threadIdx.x + (int64_t)j * kBinBlock;
+    const int64_t be = lo + threadIdx.x + (int64_t)j * kBinPlaceBlock;
     node[j] = be < hi ? bin_node(a, be) : -1;
   }
 #pragma unroll
@@ -107,36 +110,46 @@ __device__ __forceinline__ void bin_buckets(const ScatterArgs &a, const BinArgs 
 }
 
 // Adds 1 to counter[bucket] for every lane with bucket >= 0 and returns the value before the lane's own
-// addition. The lanes that share the bucket of the wavefront's first lane (with a heavy-tailed index: most of
-// them, the bucket of the hubs) go through one atomic of their leader; the others add on their own.
+// addition. Twice over, the lanes that share the bucket of the first lane still waiting go through one atomic
+// of their leader (with a heavy-tailed index nearly all lanes: the bucket of the hubs, which would otherwise
+// queue up on one LDS address); whoever is left adds on its own.
 __device__ __forceinline__ int32_t bin_take(int32_t *counter, int32_t bucket) {
   const int lane = threadIdx.x & (kWave - 1);
-  const int32_t first = __builtin_amdgcn_readfirstlane(bucket);
-  const uint64_t same = __ballot(bucket == first && first >= 0);
   int32_t before = 0;
-  if (same != 0) {
-    const int leader = __ffsll((unsigned long long)same) - 1;
+  bool waiting = bucket >= 0;
+#pragma unroll
+  for (int round = 0; round < 2; ++round) {
+    const uint64_t todo = __ballot(waiting);
+    if (todo == 0) break;
+    const int head = __ffsll((unsigned long long)todo) - 1;
+    const int32_t first = __shfl(bucket, head);
+    const uint64_t same = __ballot(waiting && bucket == first);
     int32_t base = 0;
-    if (lane == leader) base = atomicAdd(&counter[first], __popcll(same));
-    base = __shfl(base, leader);
-    before = base + __popcll(same & (((uint64_t)1 << lane) - 1));
+    if (lane == head) base = atomicAdd(&counter[first], __popcll(same));
+    base = __shfl(base, head);
+    if ((same >> lane) & 1) {
+      before = base + __popcll(same & (((uint64_t)1 << lane) - 1));
+      waiting = false;
+    }
   }
-  if (bucket >= 0 && !((same >> lane) & 1)) before = atomicAdd(&counter[bucket], 1);
+  if (waiting) before = atomicAdd(&counter[bucket], 1);
   return before;
 }
 
-static __global__ __launch_bounds__(kBinBlock) void bin_count_kernel(ScatterArgs a, BinArgs p) {
+static __global__ __launch_bounds__(kBinPlaceBlock) void bin_count_kernel(ScatterArgs a, BinArgs p) {
   __shared__ int32_t s_hist[kBinMaxBuckets];
-  for (int i = threadIdx.x; i < p.nb; i += kBinBlock) s_hist[i] = 0;
+  for (int i = threadIdx.x; i < p.nb; i += kBinPlaceBlock) s_hist[i] = 0;
   __syncthreads();
-  const int64_t lo = (int64_t)blockIdx.x * kBinChunk;
-  const int64_t hi = lo + kBinChunk < a.B * a.E ? lo + kBinChunk : a.B * a.E;
-  int32_t bucket[kBinPer];
-  bin_buckets(a, p, lo, hi, bucket, nullptr);
+  const int64_t lo = (int64_t)blockIdx.x * kBinPlaceChunk;
+  const int64_t hi = lo + kBinPlaceChunk < a.B * a.E ? lo + kBinPlaceChunk : a.B * a.E;
+  for (int64_t b0 = lo; b0 < hi; b0 += kBinBatch) {
+    int32_t bucket[kBinPer];
+    bin_buckets(a, p, b0, hi, bucket, nullptr);
 #pragma unroll
-  for (int j = 0; j < kBinPer; ++j) bin_take(s_hist, bucket[j]);
+    for (int j = 0; j < kBinPer; ++j) bin_take(s_hist, bucket[j]);
+  }
   __syncthreads();
-  for (int i = threadIdx.x; i < p.nb; i += kBinBlock) {
+  for (int i = threadIdx.x; i < p.nb; i += kBinPlaceBlock) {
     const int32_t h = s_hist[i];
     p.wg_hist[(int64_t)blockIdx.x * p.nb + i] = h;
     if (h != 0) atomicAdd(&p.totals[i], (unsigned long long)h);
@@ -202,25 +215,27 @@ static __global__ __launch_bounds__(kBinBlock) void bin_scan_kernel(BinArgs p) {
   }
 }
 
-static __global__ __launch_bounds__(kBinBlock) void bin_place_kernel(ScatterArgs a, BinArgs p) {
+static __global__ __launch_bounds__(kBinPlaceBlock) void bin_place_kernel(ScatterArgs a, BinArgs p) {
   __shared__ uint32_t s_base[kBinMaxBuckets];
   __shared__ int32_t s_cnt[kBinMaxBuckets];
-  for (int i = threadIdx.x; i < p.nb; i += kBinBlock) {
+  for (int i = threadIdx.x; i < p.nb; i += kBinPlaceBlock) {
     const int32_t h = p.wg_hist[(int64_t)blockIdx.x * p.nb + i];
     s_base[i] = h != 0 ? (uint32_t)atomicAdd(&p.cursor[i], (unsigned long long)h) : 0u;
     s_cnt[i] = 0;
   }
   __syncthreads();
-  const int64_t lo = (int64_t)blockIdx.x * kBinChunk;
-  const int64_t hi = lo + kBinChunk < a.B * a.E ? lo + kBinChunk : a.B * a.E;
-  int32_t bucket[kBinPer], local[kBinPer];
-  bin_buckets(a, p, lo, hi, bucket, local);
+  const int64_t lo = (int64_t)blockIdx.x * kBinPlaceChunk;
+  const int64_t hi = lo + kBinPlaceChunk < a.B * a.E ? lo + kBinPlaceChunk : a.B * a.E;
+  for (int64_t b0 = lo; b0 < hi; b0 += kBinBatch) {
+    int32_t bucket[kBinPer], local[kBinPer];
+    bin_buckets(a, p, b0, hi, bucket, local);
 #pragma unroll
-  for (int j = 0; j < kBinPer; ++j) {
-    const int32_t rank = bin_take(s_cnt, bucket[j]);
-    if (bucket[j] < 0) continue;
-    const int64_t be = lo + threadIdx.x + (int64_t)j * kBinBlock;
-    p.binned[s_base[bucket[j]] + (uint32_t)rank] = ((uint64_t)(uint32_t)local[j] << 32) | (uint32_t)be;
+    for (int j = 0; j < kBinPer; ++j) {
+      const int32_t rank = bin_take(s_cnt, bucket[j]);
+      if (bucket[j] < 0) continue;
+      const int64_t be = b0 + threadIdx.x + (int64_t)j * kBinPlaceBlock;
+      p.binned[s_base[bucket[j]] + (uint32_t)rank] = ((uint64_t)(uint32_t)local[j] << 32) | (uint32_t)be;
+    }
   }
 }
 
@@ -292,6 +307,86 @@ __global__ __launch_bounds__(kBinBlock) void bin_reduce_kernel(ScatterArgs a, Bi
   }
 }
 
+// The same reduction for rows held by a power-of-two number of lanes (<= 64): a wavefront reads 64 entry words
+// with one coalesced load (the next 64 are in flight while these are worked on) and hands them to its lane
+// groups by shuffle, so the rows of an entry are requested without first waiting for its entry word.
+template <typename T, int VEC, bool IS_MAX>
+__global__ __launch_bounds__(kBinBlock) void bin_reduce_wave_kernel(ScatterArgs a, BinArgs p, int lshift) {
+  constexpr int U = 4;  // eight rows in flight per lane: 90 VGPRs, one workgroup per CU, no gain
+  __shared__ uint64_t s_keys[kBinKeys + kBinKeys / 16];  // rows K + 1 keys apart (LDS banks, see above)
+  const int bucket = p.wg_bucket[blockIdx.x];
+  if (bucket < 0) return;
+  const int K = (int)a.K;
+  const int KP = K + 1;
+  const int rows = 1 << p.rshift;
+  for (int i = threadIdx.x; i < rows * KP; i += kBinBlock) s_keys[i] = 0;
+  __syncthreads();
+
+  const T *src = static_cast<const T *>(a.src);
+  const int64_t lo = p.starts[bucket] + ((int64_t)blockIdx.x - p.chunk_start[bucket]) * kBinChunk;
+  int64_t hi = lo + kBinChunk;
+  if (hi > p.starts[bucket + 1]) hi = p.starts[bucket + 1];
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  const int g = lane >> lshift;                 // lane group: one entry at a time
+  const int gpw = kWave >> lshift;              // lane groups per wavefront
+  const int k0 = (lane & ((1 << lshift) - 1)) * VEC;
+  constexpr int64_t kStride = (int64_t)(kBinBlock / kWave) * kWave;  // entries per pass of the workgroup
+  if (lo < hi) {
+    int64_t base = lo + (int64_t)wave * kWave;
+    uint64_t ent_next = p.binned[base + lane < hi ? base + lane : hi - 1];
+    for (; base < hi; base += kStride) {
+      const uint64_t ent = ent_next;
+      const int64_t nb = base + kStride;
+      ent_next = p.binned[nb + lane < hi ? nb + lane : hi - 1];  // unconditional: exact wait counts
+      const int n = hi - base < kWave ? (int)(hi - base) : kWave;
+      const uint32_t ent_lo = (uint32_t)ent, ent_hi = (uint32_t)(ent >> 32);
+      for (int i0 = 0; i0 < n; i0 += gpw * U) {
+        uint32_t e_row[U], e_ent[U];
+        Vec<T, VEC> x[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const int i = i0 + u * gpw + g;
+          const int from = i < n ? i : n - 1;
+          e_ent[u] = (uint32_t)__shfl((int)ent_lo, from);
+          e_row[u] = (uint32_t)__shfl((int)ent_hi, from);
+          x[u] = load_vec_stream<T, VEC>(src + (int64_t)e_ent[u] * a.K + k0);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          if (i0 + u * gpw + g >= n) continue;
+          int64_t e = (int64_t)e_ent[u];
+          if (a.B > 1) e -= (e / a.E) * a.E;  // position inside the batch
+          uint64_t key[VEC];
+          make_keys<T, VEC, IS_MAX>(x[u], e, key);
+          uint64_t *row = &s_keys[(int)e_row[u] * KP + k0];
+          const volatile uint32_t *hi32 = reinterpret_cast<const volatile uint32_t *>(row) + 1;
+#pragma unroll
+          for (int v = 0; v < VEC; ++v)
+            if (key[v] != 0 && (uint32_t)(key[v] >> 32) >= hi32[2 * v])
+              __hip_atomic_fetch_max(row + v, key[v], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        }
+      }
+    }
+  }
+  __syncthreads();
+  uint64_t *gkeys = reinterpret_cast<uint64_t *>(a.arg_out) + ((int64_t)bucket << p.rshift) * a.K;
+  const int64_t limit = (a.B * a.N - ((int64_t)bucket << p.rshift)) * a.K;  // keys of rows that exist
+  const int table = K << p.rshift;
+  for (int i0 = threadIdx.x; i0 < table; i0 += kBinBlock * 4) {
+    uint64_t key[4], cur[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int i = i0 + j * kBinBlock;
+      key[j] = (i < table && i < limit) ? s_keys[i + i / K] : 0;
+      if (key[j] != 0) cur[j] = gkeys[i];
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if (key[j] != 0 && key[j] > cur[j])
+        __hip_atomic_fetch_max(gkeys + i0 + j * kBinBlock, key[j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+
 static __global__ __launch_bounds__(kBlock) void bin_clear_kernel(unsigned long long *totals, int n) {
   const int i = blockIdx.x * kBlock + threadIdx.x;
   if (i < n) totals[i] = 0;
@@ -301,10 +396,17 @@ static __global__ __launch_bounds__(kBlock) void bin_clear_kernel(unsigned long 
 template <typename T, int VEC, bool IS_MAX>
 void launch_binned_keys(const ScatterArgs &a, const BinArgs &p, hipStream_t stream) {
   hipLaunchKernelGGL(bin_clear_kernel, dim3((p.nb + kBlock - 1) / kBlock), dim3(kBlock), 0, stream, p.totals, p.nb);
-  hipLaunchKernelGGL(bin_count_kernel, dim3((unsigned)p.n_place), dim3(kBinBlock), 0, stream, a, p);
+  hipLaunchKernelGGL(bin_count_kernel, dim3((unsigned)p.n_place), dim3(kBinPlaceBlock), 0, stream, a, p);
   hipLaunchKernelGGL(bin_scan_kernel, dim3(1), dim3(kBinBlock), 0, stream, p);
-  hipLaunchKernelGGL(bin_place_kernel, dim3((unsigned)p.n_place), dim3(kBinBlock), 0, stream, a, p);
-  hipLaunchKernelGGL((bin_reduce_kernel<T, VEC, IS_MAX>), dim3((unsigned)p.max_wgs), dim3(kBinBlock), 0, stream, a, p);
+  hipLaunchKernelGGL(bin_place_kernel, dim3((unsigned)p.n_place), dim3(kBinPlaceBlock), 0, stream, a, p);
+  const int64_t kv = a.K / VEC;
+  int lshift = 0;
+  while (((int64_t)1 << lshift) < kv) ++lshift;
+  if (((int64_t)1 << lshift) == kv && kv <= kWave && !getenv("TS_BIN_NO_WAVE"))  // env: tuning aid
+    hipLaunchKernelGGL((bin_reduce_wave_kernel<T, VEC, IS_MAX>), dim3((unsigned)p.max_wgs), dim3(kBinBlock), 0, stream, a,
+                       p, lshift);
+  else
+    hipLaunchKernelGGL((bin_reduce_kernel<T, VEC, IS_MAX>), dim3((unsigned)p.max_wgs), dim3(kBinBlock), 0, stream, a, p);
 }
 
 }  // namespace ts
