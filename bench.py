@@ -412,6 +412,8 @@ def main():
         zipf_index = wz.index[torch.randperm(wz.E, generator=g)] * 10 % 1_000_000
         sz = wl.ScatterWorkload("X-zipf-unsorted-K8", zipf_index, 1_000_000, wz.E, 8, torch.float32)
         table["X-zipf-unsorted-K8"] = bench_scatter_config(ts, wl, sz, dev, max(it // 2, 3), ["sum", "max"])
+        sw32 = dataclasses.replace(wl.c4_scatter_minmax(32), name="X-zipf-unsorted-K32")
+        table["X-zipf-unsorted-K32"] = bench_scatter_config(ts, wl, sw32, dev, max(it // 2, 3), ["sum"])
         table["X-sorted-plan-C4-K32"] = bench_sorted_config(ts, wl, wl.c4_scatter_minmax(32), dev, max(it // 2, 3))
         ss = wl.ScatterWorkload("X-sorted-plan-C3-shuffled-K64", w3.index[torch.randperm(w3.E, generator=g)], w3.N, w3.E,
                                 64, torch.float32)

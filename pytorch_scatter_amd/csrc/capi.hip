@@ -334,9 +334,15 @@ int ts_segment_mean_coo_backward(const void *grad_out, const int64_t *index, con
 }
 
 size_t ts_scatter_workspace_bytes(int64_t B, int64_t E, int64_t K, int64_t N, int dtype, int reduce) {
-  if (!valid_dtype(dtype) || !sizes_ok(B, N, E, K) || (reduce != TS_MIN && reduce != TS_MAX)) return 0;
-  if (kElemBytes[dtype] > 4) return 0;  // 64-bit elements do not use packed keys
-  return bin_plan(B, E, K, N, kElemBytes[dtype], nullptr, 0, env_int("TS_SCATTER_BINNED", 1) == 2).bytes;
+  if (!valid_dtype(dtype) || !sizes_ok(B, N, E, K)) return 0;
+  const bool any_size = env_int("TS_SCATTER_BINNED", 1) == 2;
+  if (reduce == TS_MIN || reduce == TS_MAX) {
+    if (kElemBytes[dtype] > 4) return 0;  // 64-bit elements do not use packed keys
+    return bin_plan(B, E, K, N, kElemBytes[dtype], nullptr, 0, any_size).bytes;
+  }
+  if (reduce == TS_SUM && kAccBytes[dtype] >= 4)  // table slots: int32 for int32, 8 bytes for the other types
+    return bin_plan(B, E, K, N, kElemBytes[dtype], nullptr, 0, any_size, dtype == TS_I32 ? 4 : 8).bytes;
+  return 0;
 }
 
 int ts_scatter(const void *src, const int64_t *index, void *out, int64_t *arg_out, int64_t B, int64_t E,

@@ -208,6 +208,7 @@ struct ScatterArgs {
   void *bin_ws = nullptr;  // optional workspace: min/max of wide rows through buckets of output rows
   size_t bin_ws_bytes = 0;
   int bin_any_size = 0;    // tuning aid / tests: also for inputs below the size from which it pays
+  const int *skip_flag = nullptr;  // sum kernels: leave at once if *skip_flag != 0 (the binned pass did the work)
 };
 
 // ---- thread -> (edge, column) mapping shared by the scatter kernels ------------
@@ -247,6 +248,7 @@ __device__ __forceinline__ void split_edge(const int64_t be, const int64_t B, co
 template <typename T, int VEC, int REDUCE>
 __global__ __launch_bounds__(kBlock) void scatter_atomic_kernel(ScatterArgs a) {
   constexpr int U = 4;
+  if (a.skip_flag != nullptr && *a.skip_flag != 0) return;
   const T *src = static_cast<const T *>(a.src);
   T *out = static_cast<T *>(a.out);
   const int64_t kv = a.K / VEC;
@@ -293,6 +295,7 @@ __global__ __launch_bounds__(kBlock) void scatter_atomic_kernel(ScatterArgs a) {
 // (requires K even, one index per row, 4-byte aligned src/out)
 template <typename T>
 __global__ __launch_bounds__(kBlock) void scatter_add_pk16_kernel(ScatterArgs a) {
+  if (a.skip_flag != nullptr && *a.skip_flag != 0) return;
   const T *src = static_cast<const T *>(a.src);
   T *out = static_cast<T *>(a.out);
   const int64_t kv = a.K / 2;
@@ -753,6 +756,7 @@ __global__ __launch_bounds__(kBlock) void scatter_add_run_kernel(ScatterArgs a, 
                                                                  int hot_rlog) {
   typedef typename Acc<T>::type A;
   constexpr bool kTable = HOT && HotOk<A>::value;
+  if (a.skip_flag != nullptr && *a.skip_flag != 0) return;
   __shared__ A s_stage[kBlock / kWave][kWave * C];
   __shared__ A s_hot[kTable ? kHotAcc : 1];
   __shared__ uint32_t s_tags[kTable ? kHotRowsMax : 1];
@@ -1209,6 +1213,7 @@ constexpr int kLdsAddBlock = 1024;    // one table per 16 wavefronts: every work
 template <typename T>
 __global__ __launch_bounds__(kLdsAddBlock) void scatter_add_lds_kernel(ScatterArgs a, int tn_mask, int64_t epb) {
   constexpr int U = 4;
+  if (a.skip_flag != nullptr && *a.skip_flag != 0) return;
   __shared__ float s_acc[kLdsAcc];
   __shared__ int32_t s_tags[kLdsAccRows];
   const int K = (int)a.K;
@@ -1395,7 +1400,8 @@ inline unsigned scatter_grid(int64_t n_edges, int64_t kv, int block, int U) {
 }
 
 template <typename T, int VEC>
-int launch_scatter_v(const ScatterArgs &a, int reduce, hipStream_t stream) {
+int launch_scatter_v(const ScatterArgs &args, int reduce, hipStream_t stream) {
+  ScatterArgs a = args;
   T *out = static_cast<T *>(a.out);
   const int64_t n_out = a.B * a.N * a.K;
   const int64_t n_src = a.B * a.E * a.K;
@@ -1405,6 +1411,24 @@ int launch_scatter_v(const ScatterArgs &a, int reduce, hipStream_t stream) {
     if (!a.out_given)
       hipLaunchKernelGGL(fill_kernel<T>, dim3(g_out), dim3(kBlock), 0, stream, out, n_out,
                          small_const<T>(reduce == TS_MUL ? 1 : 0));
+    if (reduce == TS_SUM && n_src > 0 && a.bin_ws != nullptr && a.sk == 0 && a.K % VEC == 0) {
+      // Large inputs with rows of 64 bytes and more, given a workspace: unless the index is sorted (found out by
+      // the first pass), the entries are binned by bucket of output rows and summed in LDS (scatter_binned.h);
+      // the kernels launched below then return at once. A sorted index stays with them: they combine its runs.
+      if constexpr (BinSlotOk<T>::value) {
+        const int64_t kv = a.K / VEC;
+        int lshift = 0;
+        while (((int64_t)1 << lshift) < kv) ++lshift;
+        if (((int64_t)1 << lshift) == kv && kv <= kWave) {
+          const BinPlan bp = bin_plan(a.B, a.E, a.K, a.N, (int)sizeof(T), a.bin_ws, a.bin_ws_bytes, a.bin_any_size != 0,
+                                      (int)sizeof(typename BinSlot<T>::type));
+          if (bp.ok) {
+            launch_binned_add<T, VEC>(a, bp.p, lshift, stream);
+            a.skip_flag = bp.p.unsorted;
+          }
+        }
+      }
+    }
     if (n_src > 0) {
       // one element per lane: the 64 atomics of a wavefront then cover whole cache lines
       // (4 lines per instruction for fp32 instead of 16 with 4 elements per lane)

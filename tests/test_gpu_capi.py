@@ -562,7 +562,56 @@ def test_scatter_minmax_binned_variant(capi, oracle, shape, reduce, dtype, monke
     need = L.ts_scatter_workspace_bytes(capi._i(B), capi._i(E), capi._i(K), capi._i(N), capi.DTYPE[dtype],
                                         capi.REDUCE[reduce])
     assert (need > 0) == (K * src.element_size() >= 64 and K <= 512)
-    assert L.ts_scatter_workspace_bytes(capi._i(B), capi._i(E), capi._i(K), capi._i(N), capi.DTYPE[dtype], capi.SUM) == 0
+    assert L.ts_scatter_workspace_bytes(capi._i(B), capi._i(E), capi._i(K), capi._i(N), capi.DTYPE[dtype], capi.MUL) == 0
+
+
+@pytest.mark.parametrize("shape,kind,dtype", product(
+    [(1, 60000, 32, 300), (2, 40000, 16, 700), (1, 50000, 128, 90), (1, 20000, 64, 100000), (3, 9000, 256, 5),
+     (1, 30000, 24, 500)],
+    ["zipf", "sorted", "one descent"],
+    [torch.float32, torch.float64, torch.bfloat16, torch.float16, torch.int32, torch.int64, torch.int16]))
+def test_scatter_sum_binned_variant(capi, oracle, shape, kind, dtype, monkeypatch):
+    """Sum with a workspace (forced on at these sizes): the first pass finds out whether the index is sorted;
+    if not, the entries are binned by bucket of output rows and added in LDS (double slots for floating
+    types), else the usual kernels run. Exact for integers (int16 and K = 24 keep the path without
+    workspace), within tolerance of the exact sum for floats, with and without previous content in out."""
+    monkeypatch.setenv("TS_SCATTER_BINNED", "2")
+    B, E, K, N = shape
+    rng = np.random.default_rng(E + K + len(kind))
+    p = np.arange(1, N + 1, dtype=np.float64) ** -1.2
+    idx = rng.choice(N, size=E, p=p / p.sum())
+    if kind != "zipf":
+        idx = np.sort(idx)
+    if kind == "one descent":
+        idx[E // 2] = N - 1
+        idx[E // 2 + 1] = 0
+    index1 = torch.from_numpy(idx)
+    index = index1.view(1, E, 1).expand(B, E, K)
+    if dtype.is_floating_point:
+        src = torch.from_numpy(rng.standard_normal(size=(B, E, K))).to(dtype)
+    else:
+        src = torch.from_numpy(rng.integers(-20, 20, size=(B, E, K))).to(dtype)
+    for out_given in (False, True):
+        prev = (torch.from_numpy(rng.standard_normal(size=(B, N, K))).to(dtype) if dtype.is_floating_point
+                else torch.from_numpy(rng.integers(-20, 20, size=(B, N, K))).to(dtype))
+        out = prev.clone().to(DEV) if out_given else torch.full((B, N, K), 9, dtype=dtype, device=DEV)
+        capi.scatter_with_workspace(src.to(DEV), index1.to(DEV), out, None, B, E, K, N, 0, 1, 0, capi.SUM, out_given)
+        torch.cuda.synchronize()
+        if not dtype.is_floating_point:
+            want = oracle.scatter(src, index, 1, prev.clone() if out_given else None, None if out_given else N,
+                                  "sum")[0]
+            assert_exact(out, want, f"{kind} out_given={out_given}")
+            continue
+        exact = oracle.scatter(src.double(), index, 1, None, N, "sum")[0]
+        absum = oracle.scatter(src.double().abs(), index, 1, None, N, "sum")[0]
+        want = exact + (prev.double() if out_given else 0)
+        rtol = RTOL[dtype]
+        err = (out.cpu().double() - want).abs()
+        bound = rtol * want.abs() + rtol * (absum + (prev.double().abs() if out_given else 0)).clamp(min=1e-30)
+        if dtype in (torch.bfloat16, torch.float16):
+            n_row = torch.bincount(index1, minlength=N).double().clamp(max=64).view(1, N, 1)
+            bound = bound + 2.0 ** -8 * 64 * want.abs().clamp(min=1.0) + 2.0 ** -9 * n_row * absum
+        assert bool((err <= bound).all()), (kind, out_given, float((err - bound).max()))
 
 
 @pytest.mark.parametrize("shape,dtype", product(
