@@ -256,7 +256,7 @@ __global__ __launch_bounds__(kBlock) void group_sum_run_kernel(ScatterArgs a, Gr
                                                                int rows_per_wave, int hot_rlog) {
   typedef typename Acc<T>::type A;
   __shared__ A s_stage[kBlock / kWave][kWave * C];
-  __shared__ A s_hot[kHotAcc];
+  __shared__ typename HotSlot<A>::type s_hot[kHotAcc];
   __shared__ uint32_t s_tags[kHotRowsMax];
   GroupSumRun<T, C, MODE> p;
   p.src = static_cast<const T *>(g.src);

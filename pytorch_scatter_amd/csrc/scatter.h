@@ -590,8 +590,14 @@ constexpr uint32_t kHotConfirmed = 0x80000000u;  // tag bit: the row belongs to 
 constexpr uint32_t kHotNone = 0x7FFFFFFFu;       // no candidate yet (node ids stay below 2^31 - 1)
 template <typename A> struct HotOk { static constexpr bool value = sizeof(A) >= 4; };  // LDS atomics: 32 / 64 bits
 
+// Slot type of the table: fp32 sums are kept in double slots. ds_add_f32 loses its rate when many lanes meet on one
+// address, which is what a hub row is; ds_add_f64 and the integer adds keep theirs.
+template <typename A> struct HotSlot { typedef A type; };
+template <> struct HotSlot<float> { typedef double type; };
+
 template <typename A> struct HotRows {
-  A *acc;          // [rows][1 << wshift]
+  typedef typename HotSlot<A>::type S;
+  S *acc;          // [rows][1 << wshift]
   uint32_t *tags;  // [rows]
   int rlog;        // log2(rows), < 0: no table
   int wshift;      // log2 of the columns per row (the column chunk of the workgroup)
@@ -614,12 +620,12 @@ template <typename A> struct HotRows {
     }
 #pragma unroll
     for (int w = 0; w < EW; ++w)
-      __hip_atomic_fetch_add(&acc[(row << wshift) + j + w], x[w], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      __hip_atomic_fetch_add(&acc[(row << wshift) + j + w], (S)x[w], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     return true;
   }
   __device__ void clear() const {
     if (rlog < 0) return;
-    for (int i = threadIdx.x; i < (1 << (rlog + wshift)); i += blockDim.x) acc[i] = (A)0;
+    for (int i = threadIdx.x; i < (1 << (rlog + wshift)); i += blockDim.x) acc[i] = (S)0;
     for (int i = threadIdx.x; i < (1 << rlog); i += blockDim.x) tags[i] = kHotNone;
     __syncthreads();
   }
@@ -631,9 +637,13 @@ template <typename A> struct HotRows {
       const uint32_t t = tags[i >> wshift];
       if (!(t & kHotConfirmed)) continue;
       bool any = false;
+      A x[EW];
 #pragma unroll
-      for (int w = 0; w < EW; ++w) any = any || acc[i + w] != (A)0;
-      if (any) emit((int)(t & ~kHotConfirmed), i & ((1 << wshift) - 1), acc + i);
+      for (int w = 0; w < EW; ++w) {
+        x[w] = (A)acc[i + w];
+        any = any || acc[i + w] != (S)0;
+      }
+      if (any) emit((int)(t & ~kHotConfirmed), i & ((1 << wshift) - 1), x);
     }
   }
 };
@@ -651,7 +661,7 @@ template <typename A> struct HotState {
   HotRows<A> hot;
   int64_t colbase;  // first column of the workgroup's chunk
   bool active;
-  __device__ void hot_init(A *acc, uint32_t *tags, int rlog, int wshift) {
+  __device__ void hot_init(typename HotSlot<A>::type *acc, uint32_t *tags, int rlog, int wshift) {
     hot.acc = acc;
     hot.tags = tags;
     hot.rlog = HotOk<A>::value ? rlog : -1;
@@ -758,7 +768,7 @@ __global__ __launch_bounds__(kBlock) void scatter_add_run_kernel(ScatterArgs a, 
   constexpr bool kTable = HOT && HotOk<A>::value;
   if (a.skip_flag != nullptr && *a.skip_flag != 0) return;
   __shared__ A s_stage[kBlock / kWave][kWave * C];
-  __shared__ A s_hot[kTable ? kHotAcc : 1];
+  __shared__ typename HotSlot<A>::type s_hot[kTable ? kHotAcc : 1];
   __shared__ uint32_t s_tags[kTable ? kHotRowsMax : 1];
   AddRun<T, C, EW, kTable> p;
   p.src = static_cast<const T *>(a.src);
@@ -1206,7 +1216,7 @@ __global__ __launch_bounds__(kLdsBlockK1) void scatter_key_lds_k1_kernel(Scatter
 // element and chunk. 16-bit inputs gain accuracy on the way (fp32 partial sums,
 // one rounding per chunk instead of one per entry). src == nullptr adds 1.0 per
 // entry (the count of scatter mean).
-constexpr int kLdsAcc = 8192;         // 32 KB of fp32 accumulators
+constexpr int kLdsAcc = 8192;         // accumulators of the table (64 KB of double slots)
 constexpr int kLdsAccRows = 4096;     // 16 KB of tags
 constexpr int kLdsAddBlock = 1024;    // one table per 16 wavefronts: every workgroup adds its table to out once
 
@@ -1214,11 +1224,14 @@ template <typename T>
 __global__ __launch_bounds__(kLdsAddBlock) void scatter_add_lds_kernel(ScatterArgs a, int tn_mask, int64_t epb) {
   constexpr int U = 4;
   if (a.skip_flag != nullptr && *a.skip_flag != 0) return;
-  __shared__ float s_acc[kLdsAcc];
+  // double slots: ds_add_f32 loses its rate when many lanes meet on one address (a hub, or a sorted index whose
+  // neighbouring entries share a row), ds_add_f64 does not (Zipf(1.2) index, K = 8: 391 -> 263 us; sorted: 476 -> 177 us)
+  typedef double LdsAcc;
+  __shared__ LdsAcc s_acc[kLdsAcc];
   __shared__ int32_t s_tags[kLdsAccRows];
   const int K = (int)a.K;
   const int tn = tn_mask + 1;
-  for (int i = threadIdx.x; i < tn * K; i += kLdsAddBlock) s_acc[i] = 0.0f;
+  for (int i = threadIdx.x; i < tn * K; i += kLdsAddBlock) s_acc[i] = (LdsAcc)0;
   for (int i = threadIdx.x; i < tn; i += kLdsAddBlock) s_tags[i] = -1;
   __syncthreads();
 
@@ -1253,7 +1266,7 @@ __global__ __launch_bounds__(kLdsAddBlock) void scatter_add_lds_kernel(ScatterAr
             tag = old == -1 ? node : old;
           }
           if (tag == node)
-            __hip_atomic_fetch_add(&s_acc[row * K + k], x[u], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            __hip_atomic_fetch_add(&s_acc[row * K + k], (LdsAcc)x[u], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
           else
             atomic_add_elem<T>(out + (int64_t)node * a.K + k, from_acc<T>((typename Acc<T>::type)x[u]));
         }
@@ -1262,7 +1275,7 @@ __global__ __launch_bounds__(kLdsAddBlock) void scatter_add_lds_kernel(ScatterAr
   }
   __syncthreads();
   for (int i = threadIdx.x; i < tn * K; i += kLdsAddBlock) {
-    const float v = s_acc[i];
+    const float v = (float)s_acc[i];
     if (v == 0.0f) continue;
     const int row = i / K;
     atomic_add_elem<T>(out + (int64_t)s_tags[row] * a.K + (i - row * K), from_acc<T>((typename Acc<T>::type)v));
