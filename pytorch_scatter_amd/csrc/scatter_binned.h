@@ -101,13 +101,30 @@ constexpr int kBinPer = 16;  // entries per lane and batch in count / place (all
 constexpr int kBinBatch = kBinPer * kBinPlaceBlock;
 
 // buckets of the kBinPer entries of a lane, all index loads in flight at once; -1: no bucket
+// descent (optional): set when an entry's node lies below that of the entry before it. The entry before is the
+// neighbouring lane's (a shuffle); only the first lane of a wavefront loads it.
 __device__ __forceinline__ void bin_buckets(const ScatterArgs &a, const BinArgs &p, int64_t lo, int64_t hi,
-                                            int32_t *bucket, int32_t *local) {
+                                            int32_t *bucket, int32_t *local, bool *descent = nullptr) {
   int64_t node[kBinPer];
 #pragma unroll
   for (int j = 0; j < kBinPer; ++j) {
     const int64_t be = lo + threadIdx.x + (int64_t)j * kBinPlaceBlock;
     node[j] = be < hi ? bin_node(a, be) : -1;
+  }
+  if (descent != nullptr) {
+    const int lane = threadIdx.x & (kWave - 1);
+    int64_t before[kBinPer];
+#pragma unroll
+    for (int j = 0; j < kBinPer; ++j) {
+      const int64_t be = lo + threadIdx.x + (int64_t)j * kBinPlaceBlock;
+      before[j] = (lane == 0 && be > 0 && be < hi) ? bin_node(a, be - 1) : -1;
+    }
+#pragma unroll
+    for (int j = 0; j < kBinPer; ++j) {
+      const int lo32 = __shfl_up((int)(uint32_t)node[j], 1), hi32 = __shfl_up((int)(node[j] >> 32), 1);
+      const int64_t prev = lane == 0 ? before[j] : (int64_t)(((uint64_t)(uint32_t)hi32 << 32) | (uint32_t)lo32);
+      *descent = *descent || (node[j] >= 0 && prev >= 0 && node[j] < prev);
+    }
   }
 #pragma unroll
   for (int j = 0; j < kBinPer; ++j) {
@@ -145,31 +162,26 @@ __device__ __forceinline__ int32_t bin_take(int32_t *counter, int32_t bucket) {
 
 static __global__ __launch_bounds__(kBinPlaceBlock) void bin_count_kernel(ScatterArgs a, BinArgs p) {
   __shared__ int32_t s_hist[kBinMaxBuckets];
+  __shared__ int s_hist_flag;
   for (int i = threadIdx.x; i < p.nb; i += kBinPlaceBlock) s_hist[i] = 0;
+  if (threadIdx.x == 0) s_hist_flag = 0;
   __syncthreads();
   const int64_t lo = (int64_t)blockIdx.x * kBinPlaceChunk;
   const int64_t hi = lo + kBinPlaceChunk < a.B * a.E ? lo + kBinPlaceChunk : a.B * a.E;
   bool descent = false;
   for (int64_t b0 = lo; b0 < hi; b0 += kBinBatch) {
     int32_t bucket[kBinPer];
-    bin_buckets(a, p, b0, hi, bucket, nullptr);
-    if (p.unsorted != nullptr) {
-      // an entry whose index is below that of the entry before it (the neighbour's load: a cache hit)
-#pragma unroll
-      for (int j = 0; j < kBinPer; ++j) {
-        const int64_t be = b0 + threadIdx.x + (int64_t)j * kBinPlaceBlock;
-        if (be < hi) {
-          int64_t b = 0, e = be;
-          if (a.B > 1) { b = be / a.E; e = be - b * a.E; }
-          if (e > 0) descent = descent || a.index[b * a.sb + e * a.se] < a.index[b * a.sb + (e - 1) * a.se];
-        }
-      }
-    }
+    bin_buckets(a, p, b0, hi, bucket, nullptr, p.unsorted != nullptr ? &descent : nullptr);
 #pragma unroll
     for (int j = 0; j < kBinPer; ++j) bin_take(s_hist, bucket[j]);
   }
-  if (p.unsorted != nullptr && __ballot(descent) != 0 && (threadIdx.x & (kWave - 1)) == 0) atomicOr(p.unsorted, 1);
+  // one flag for the whole launch: a workgroup that saw a descent sets it unless it reads as set already (ten
+  // thousand wavefronts doing so one by one on the same address cost 100 us)
+  if (__ballot(descent) != 0) s_hist_flag = 1;
   __syncthreads();
+  if (p.unsorted != nullptr && threadIdx.x == 0 && s_hist_flag != 0 &&
+      __hip_atomic_load(p.unsorted, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0)
+    atomicOr(p.unsorted, 1);
   for (int i = threadIdx.x; i < p.nb; i += kBinPlaceBlock) {
     const int32_t h = s_hist[i];
     p.wg_hist[(int64_t)blockIdx.x * p.nb + i] = h;
