@@ -293,8 +293,8 @@ def probe():
 
 def probe_scatter():
     """Launch sequence for `rocprofv3 --pmc TCC_HIT_sum TCC_MISS_sum TCC_ATOMIC_sum -- python3 bench.py
-    --probe-scatter`: C1 scatter sum x3, C4 scatter max with K = 1 and K = 32 x2 each, scatter sum and max
-    over the sorted index of C3 with K = 64 x2 each."""
+    --probe-scatter`: C1 scatter sum x3, C4 scatter max with K = 1 and K = 32 x2 each (K = 32 also as a sum and
+    through an index sorted once, x2 each), scatter sum and max over the sorted index of C3 with K = 64 x2 each."""
     import torch
     import pytorch_scatter_amd as ts
     from pytorch_scatter_amd import workloads as wl
@@ -312,6 +312,12 @@ def probe_scatter():
             for _ in range(2):
                 ts.scatter_max(src, index, 0, None, w4.N)
             done[f"C4-K{K}"] = [w4.N, w4.E, w4.K]
+            if K == 32:  # the same scatter as a sum, and through an index sorted once
+                for _ in range(2):
+                    ts.scatter_sum(src, index, 0, None, w4.N)
+                plan = ts.SortedIndex(index, w4.N)
+                for _ in range(2):
+                    ts.scatter_sorted(src, plan, 0, "max")
         w3 = wl.c3_segment_coo()
         index = w3.index.to(dev)
         src = torch.randn((w3.E, 64), device=dev)
