@@ -1,4 +1,4 @@
-// scatter min / max for wide rows through buckets of output rows (included by scatter.h).
+// scatter min / max / sum for wide rows through buckets of output rows (included by scatter.h).
 //
 // The packed-key table of one workgroup (scatter_key_lds_kernel) holds 128 rows of 32 keys; with a heavy-tailed
 // index a quarter of the entries miss it and go to the table in memory one 256-byte row at a time. Here the
@@ -11,7 +11,8 @@
 //   reduce : a workgroup per chunk of a bucket: rows of src by entry number, packed keys into the LDS table,
 //            table -> global table with a read before each atomic
 // The order inside a bucket is whatever the placement gives; the packed keys carry the positions, so the result
-// (value, first position among equal values) does not depend on it.
+// (value, first position among equal values) does not depend on it. Sums use the same passes with a table of
+// accumulators (bin_add_wave_kernel) unless the count pass finds the index sorted.
 #pragma once
 
 namespace ts {
@@ -273,6 +274,29 @@ static __global__ __launch_bounds__(kBinPlaceBlock) void bin_place_kernel(Scatte
   }
 }
 
+// The table of one chunk (rows K + 1 keys apart) -> the table in memory: a read first, an atomic only for a key
+// that improves on what is there.
+__device__ __forceinline__ void bin_flush_keys(const ScatterArgs &a, const BinArgs &p, int bucket,
+                                               const uint64_t *s_keys) {
+  const int K = (int)a.K;
+  uint64_t *gkeys = reinterpret_cast<uint64_t *>(a.arg_out) + ((int64_t)bucket << p.rshift) * a.K;
+  const int64_t limit = (a.B * a.N - ((int64_t)bucket << p.rshift)) * a.K;  // keys of rows that exist
+  const int table = K << p.rshift;
+  for (int i0 = threadIdx.x; i0 < table; i0 += kBinBlock * 4) {
+    uint64_t key[4], cur[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int i = i0 + j * kBinBlock;
+      key[j] = (i < table && i < limit) ? s_keys[i + i / K] : 0;  // row i / K starts i / K keys later
+      if (key[j] != 0) cur[j] = gkeys[i];
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if (key[j] != 0 && key[j] > cur[j])
+        __hip_atomic_fetch_max(gkeys + i0 + j * kBinBlock, key[j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+
 template <typename T, int VEC, bool IS_MAX>
 __global__ __launch_bounds__(kBinBlock) void bin_reduce_kernel(ScatterArgs a, BinArgs p) {
   constexpr int U = 4;  // 63 VGPRs: two workgroups per CU (eight rows in flight per lane: 74 VGPRs, one workgroup)
@@ -322,23 +346,7 @@ __global__ __launch_bounds__(kBinBlock) void bin_reduce_kernel(ScatterArgs a, Bi
     }
   }
   __syncthreads();
-  // the chunk's winners -> global table
-  uint64_t *gkeys = reinterpret_cast<uint64_t *>(a.arg_out) + ((int64_t)bucket << p.rshift) * a.K;
-  const int64_t limit = (a.B * a.N - ((int64_t)bucket << p.rshift)) * a.K;  // keys of rows that exist
-  const int table = K << p.rshift;
-  for (int i0 = threadIdx.x; i0 < table; i0 += kBinBlock * 4) {
-    uint64_t key[4], cur[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int i = i0 + j * kBinBlock;
-      key[j] = (i < table && i < limit) ? s_keys[i + i / K] : 0;  // row i / K starts i / K keys later
-      if (key[j] != 0) cur[j] = gkeys[i];
-    }
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-      if (key[j] != 0 && key[j] > cur[j])
-        __hip_atomic_fetch_max(gkeys + i0 + j * kBinBlock, key[j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  }
+  bin_flush_keys(a, p, bucket, s_keys);
 }
 
 // The same reduction for rows held by a power-of-two number of lanes (<= 64): a wavefront reads 64 entry words
@@ -403,22 +411,7 @@ __global__ __launch_bounds__(kBinBlock) void bin_reduce_wave_kernel(ScatterArgs 
     }
   }
   __syncthreads();
-  uint64_t *gkeys = reinterpret_cast<uint64_t *>(a.arg_out) + ((int64_t)bucket << p.rshift) * a.K;
-  const int64_t limit = (a.B * a.N - ((int64_t)bucket << p.rshift)) * a.K;  // keys of rows that exist
-  const int table = K << p.rshift;
-  for (int i0 = threadIdx.x; i0 < table; i0 += kBinBlock * 4) {
-    uint64_t key[4], cur[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int i = i0 + j * kBinBlock;
-      key[j] = (i < table && i < limit) ? s_keys[i + i / K] : 0;
-      if (key[j] != 0) cur[j] = gkeys[i];
-    }
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-      if (key[j] != 0 && key[j] > cur[j])
-        __hip_atomic_fetch_max(gkeys + i0 + j * kBinBlock, key[j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  }
+  bin_flush_keys(a, p, bucket, s_keys);
 }
 
 static __global__ __launch_bounds__(kBlock) void bin_clear_kernel(unsigned long long *totals, int n, int *flag) {
