@@ -25,7 +25,10 @@
 // indices first (run_reduce_wave for narrow rows, run_serial_wave from 128
 // bytes per entry), sums keep the rows of hub nodes in a small LDS table per
 // workgroup (HotRows), and heavily contended inputs reduce into LDS tables of
-// accumulators or keys before they touch memory.
+// accumulators or keys before they touch memory. Given scratch memory, large
+// inputs with rows of 64 bytes and more are first binned by bucket of output
+// rows, so that a workgroup's table holds every row it can meet
+// (scatter_binned.h).
 #pragma once
 
 #include <limits>
