@@ -128,6 +128,37 @@ def test_cpu_tensors_fail_loudly():
         ts.segment_csr(src, index, reduce="median")
 
 
+def test_added_operators_and_index_reuse_without_a_gpu():
+    """The operators this library adds are registered, their wrappers script, fail loudly on CPU tensors, and
+    the index-reuse front-end never touches a call it is not meant for (CPU tensors, switched off)."""
+    import pytorch_scatter_amd as ts
+    from pytorch_scatter_amd import index_reuse
+    for name in ("scatter_softmax", "scatter_logsumexp", "scatter_std", "index_to_indptr", "indptr_to_index",
+                 "sort_index", "scatter_sorted"):
+        assert hasattr(torch.ops.torch_scatter, name), name
+    for fn in (ts.scatter_mean, ts.scatter_min, ts.scatter_add, ts.scatter_std, ts.scatter_softmax,
+               ts.scatter_logsumexp, ts.index_to_indptr, ts.indptr_to_index):
+        torch.jit.script(fn)
+    index = torch.tensor([0, 1, 0, 1])
+    with pytest.raises(RuntimeError, match="must be CUDA tensor"):
+        ts.index_to_indptr(index.sort()[0], 2)
+    with pytest.raises(RuntimeError, match="must be CUDA tensor"):
+        ts.SortedIndex(index, 2)
+    assert not ts.index_reuse_enabled()
+    src = torch.ones(4, 32)
+    assert index_reuse.plan_for(src, index, 0, None, 2) is None
+    ts.enable_index_reuse(max_plans=2)
+    try:
+        assert index_reuse.plan_for(src, index, 0, None, 2) is None      # CPU tensors never qualify
+        assert index_reuse.plan_for(src, index, 0, None, 2) is None
+        assert len(index_reuse._cache) == 0
+        with pytest.raises(RuntimeError, match="must be CUDA tensor"):   # and still fail loudly
+            ts.scatter_sum(src, index, 0, None, 2)
+    finally:
+        ts.disable_index_reuse()
+    assert not ts.index_reuse_enabled()
+
+
 def test_product_does_not_import_the_oracle():
     pkg = os.path.join(ROOT, "pytorch_scatter_amd")
     for dirpath, _, files in os.walk(pkg):
