@@ -1454,12 +1454,14 @@ int launch_scatter_v(const ScatterArgs &args, int reduce, hipStream_t stream) {
           // many entries per output slot: reduce in LDS first (see scatter_add_lds_kernel)
           int tn = 1;
           while ((int64_t)tn * 2 * a.K <= kLdsAcc && tn * 2 <= kLdsAccRows) tn *= 2;
-          // Rows of 32 and more columns do as well or better through the run kernel with its hot rows
-          // (measured, 10 M entries onto 100 k nodes: equal for an unsorted index, 4-5x faster for a sorted
-          // one such as the batch vector of a pooling layer, where the table's lanes collide on one address)
+          // Rows of 32 and more columns: the table up to 300 MB of input (1 M entries onto 3000 nodes, K = 32:
+          // 70 / 58 / 106 us for a Zipf / sorted / uniform index against 275 / 174 / 126 us through the run kernel),
+          // the run kernel with its hot rows above (9-10 M entries: a sorted index, such as the batch vector of a
+          // pooling layer, takes 450 us there and 940 us through the table; an unsorted one has the workspace path)
           const bool use_lds = a.lds_cache && a.sk == 0 && tn >= 64 && a.B * a.N < 0x7FFFFFFFll &&
                                (a.lds_cache == 2 ||
-                                (a.K < 32 && n_src >= ((int64_t)1 << 20) && n_edges >= 32 * a.B * a.N));
+                                ((a.K < 32 || n_src * (int64_t)sizeof(T) < (int64_t)300000000) &&
+                                 n_src >= ((int64_t)1 << 20) && n_edges >= 32 * a.B * a.N));
           if (use_lds) {
             const int64_t epb = per_cu_chunk_edges(a.lds_epb, n_edges, 16384 / a.K > 256 ? 16384 / a.K : 256,
                                                    131072 / a.K > 2048 ? 131072 / a.K : 2048);
