@@ -20,12 +20,13 @@ namespace ts {
 constexpr int kBinKeys = 8192;        // keys of the LDS table: 64 KB, two workgroups per CU
 constexpr int kBinBlock = 1024;
 constexpr int kBinMaxBuckets = 4096;  // LDS histogram of count / place
-constexpr int kBinChunk = 8192;      // entries per chunk of a bucket in reduce
+constexpr int kBinChunk = 8192;       // entries per chunk of a bucket in reduce (fewer for inputs under 4 M entries)
 constexpr int kBinPlaceChunk = 16384;  // entries per workgroup in count / place: one batch of 16 per lane
 constexpr int kBinPlaceBlock = 1024;   // (measured slower: 256 lanes x 4 batches, 64 K entries per workgroup, 8 K)
 
 struct BinArgs {
   int rshift;              // log2 of the rows per bucket
+  int chunk;               // entries per reducing workgroup
   int nb;                  // buckets
   int64_t n_place;         // workgroups of count / place
   int64_t max_wgs;         // workgroups of reduce (upper bound of the chunks)
@@ -54,8 +55,9 @@ inline BinPlan bin_plan(int64_t B, int64_t E, int64_t K, int64_t N, int elem_byt
   r.ok = false;
   r.bytes = 0;
   const int64_t n_edges = B * E, rows = B * N;
-  // rows of 64 bytes and more, inputs from 200 MB (below, the five extra launches cost more than the misses)
-  if (K * elem_bytes < 64 || K > kBinKeys / 16 || (!any_size && n_edges * K * elem_bytes < (int64_t)200000000) ||
+  // rows of 64 bytes and more, inputs from 128 MB (below, the five extra launches cost more than the misses:
+  // 64 MB of 128-byte rows, Zipf index: 65 us without, 79 us with; 154 MB of 512-byte rows: 348 against 115 us)
+  if (K * elem_bytes < 64 || K > kBinKeys / 16 || (!any_size && n_edges * K * elem_bytes < ((int64_t)128 << 20)) ||
       n_edges >= 0xFFFFFFFEll || rows >= 0x7FFFFFFFll || rows < 1)
     return r;
   const int64_t slots = (int64_t)kBinKeys * 8 / slot_bytes;
@@ -68,7 +70,16 @@ inline BinPlan bin_plan(int64_t B, int64_t E, int64_t K, int64_t N, int elem_byt
   p.rshift = rshift;
   p.nb = (int)nb;
   p.n_place = (n_edges + kBinPlaceChunk - 1) / kBinPlaceChunk;
-  p.max_wgs = n_edges / kBinChunk + nb + 1;
+  // A reducing workgroup walks its chunk in steps of a few rows per lane group, each step a memory latency:
+  // 8 K entries take it about 200 us whatever the input, which is fine once there are a few workgroups per CU
+  // (4 M entries and more) and far too long for a smaller input. Those get shorter chunks: about 512 workgroups.
+  int64_t chunk = kBinChunk;
+  if (n_edges < (int64_t)512 * kBinChunk) {
+    chunk = (n_edges / 512 + 63) & ~(int64_t)63;
+    if (chunk < 1024) chunk = 1024;
+  }
+  p.chunk = (int)chunk;
+  p.max_wgs = n_edges / chunk + nb + 1;
   auto up = [](size_t x) { return (x + 255) & ~(size_t)255; };
   size_t off = 0;
   auto take = [&](size_t bytes) { const size_t o = off; off += up(bytes); return o; };
@@ -200,7 +211,7 @@ static __global__ __launch_bounds__(kBinBlock) void bin_scan_kernel(BinArgs p) {
   for (int j = 0; j < PER; ++j) {
     const int i = threadIdx.x * PER + j;
     t[j] = i < p.nb ? (int64_t)p.totals[i] : 0;
-    c[j] = (t[j] + kBinChunk - 1) / kBinChunk;
+    c[j] = (t[j] + p.chunk - 1) / p.chunk;
     sum_t += t[j];
     sum_c += c[j];
   }
@@ -312,8 +323,8 @@ __global__ __launch_bounds__(kBinBlock) void bin_reduce_kernel(ScatterArgs a, Bi
   __syncthreads();
 
   const T *src = static_cast<const T *>(a.src);
-  const int64_t lo = p.starts[bucket] + ((int64_t)blockIdx.x - p.chunk_start[bucket]) * kBinChunk;
-  int64_t hi = lo + kBinChunk;
+  const int64_t lo = p.starts[bucket] + ((int64_t)blockIdx.x - p.chunk_start[bucket]) * p.chunk;
+  int64_t hi = lo + p.chunk;
   if (hi > p.starts[bucket + 1]) hi = p.starts[bucket + 1];
   const EdgeLanes m = edge_lanes(K / VEC, kBinBlock);  // K / VEC <= 512: one column slice per lane
   if (m.active) {
@@ -365,8 +376,8 @@ __global__ __launch_bounds__(kBinBlock) void bin_reduce_wave_kernel(ScatterArgs 
   __syncthreads();
 
   const T *src = static_cast<const T *>(a.src);
-  const int64_t lo = p.starts[bucket] + ((int64_t)blockIdx.x - p.chunk_start[bucket]) * kBinChunk;
-  int64_t hi = lo + kBinChunk;
+  const int64_t lo = p.starts[bucket] + ((int64_t)blockIdx.x - p.chunk_start[bucket]) * p.chunk;
+  int64_t hi = lo + p.chunk;
   if (hi > p.starts[bucket + 1]) hi = p.starts[bucket + 1];
   const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
   const int g = lane >> lshift;                 // lane group: one entry at a time
@@ -447,8 +458,8 @@ __global__ __launch_bounds__(kBinBlock) void bin_add_wave_kernel(ScatterArgs a, 
   __syncthreads();
 
   const T *src = static_cast<const T *>(a.src);
-  const int64_t lo = p.starts[bucket] + ((int64_t)blockIdx.x - p.chunk_start[bucket]) * kBinChunk;
-  int64_t hi = lo + kBinChunk;
+  const int64_t lo = p.starts[bucket] + ((int64_t)blockIdx.x - p.chunk_start[bucket]) * p.chunk;
+  int64_t hi = lo + p.chunk;
   if (hi > p.starts[bucket + 1]) hi = p.starts[bucket + 1];
   const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
   const int g = lane >> lshift;
