@@ -1454,14 +1454,19 @@ int launch_scatter_v(const ScatterArgs &args, int reduce, hipStream_t stream) {
           // many entries per output slot: reduce in LDS first (see scatter_add_lds_kernel)
           int tn = 1;
           while ((int64_t)tn * 2 * a.K <= kLdsAcc && tn * 2 <= kLdsAccRows) tn *= 2;
-          // Rows of 32 and more columns: the table up to 300 MB of input (1 M entries onto 3000 nodes, K = 32:
+          // Rows under 32 columns: from 1 M elements on for a contended index, from 8 M elements on whatever the
+          // number of entries per output row (200 k x 16 floats onto 10 k rows are 4 us faster without the table). A
+          // skewed index gains a lot even at ten entries per row (10 M entries of a Zipf(1.2) index onto 1 M
+          // rows: K = 1 924 -> 135 us, K = 8 424 -> 239 us), a uniform one loses nothing (493 -> 483, 522 -> 494 us).
+          // Rows of 32 and more columns: for a contended index, the table up to 300 MB of input (1 M entries onto 3000 nodes, K = 32:
           // 70 / 58 / 106 us for a Zipf / sorted / uniform index against 275 / 174 / 126 us through the run kernel),
           // the run kernel with its hot rows above (9-10 M entries: a sorted index, such as the batch vector of a
           // pooling layer, takes 450 us there and 940 us through the table; an unsorted one has the workspace path)
           const bool use_lds = a.lds_cache && a.sk == 0 && tn >= 64 && a.B * a.N < 0x7FFFFFFFll &&
                                (a.lds_cache == 2 ||
-                                ((a.K < 32 || n_src * (int64_t)sizeof(T) < (int64_t)300000000) &&
-                                 n_src >= ((int64_t)1 << 20) && n_edges >= 32 * a.B * a.N));
+                                (n_src >= ((int64_t)1 << 20) &&
+                                 (n_edges >= 32 * a.B * a.N ? (a.K < 32 || n_src * (int64_t)sizeof(T) < (int64_t)300000000)
+                                                            : (a.K < 32 && n_src >= ((int64_t)1 << 23)))));
           if (use_lds) {
             const int64_t epb = per_cu_chunk_edges(a.lds_epb, n_edges, 16384 / a.K > 256 ? 16384 / a.K : 256,
                                                    131072 / a.K > 2048 ? 131072 / a.K : 2048);
@@ -1540,8 +1545,13 @@ int launch_scatter_v(const ScatterArgs &args, int reduce, hipStream_t stream) {
       // index with few entries per slot is served better by the direct kernel)
       int tn = 1;
       while ((int64_t)tn * 2 * a.K <= kLdsKeys) tn *= 2;
+      // one value per entry: the table kernel whatever the number of entries per output row (10 M entries onto
+      // 1 M rows, Zipf(1.2) index: 235 -> 77 us; uniform index: 266 -> 251 us); wider rows only when contended
+      // (a uniform index with ten entries per row loses: K = 8 554 -> 737 us)
       const bool contended = a.lds_cache && a.sk == 0 && a.B * a.N < 0x7FFFFFFFll &&
-                             (a.lds_cache == 2 || (n_src >= ((int64_t)1 << 20) && n_edges >= 32 * a.B * a.N));
+                             (a.lds_cache == 2 ||
+                              (n_src >= ((int64_t)1 << 20) &&
+                               ((a.K == 1 && n_src >= ((int64_t)1 << 23)) || n_edges >= 32 * a.B * a.N)));
       const bool use_lds = contended && tn >= 16;
       // entries per workgroup chunk: large enough to amortise writing the table back,
       // small enough to leave a few thousand workgroups
