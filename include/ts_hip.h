@@ -163,10 +163,12 @@ int ts_scatter(const void *src, const int64_t *index, void *out,
                ts_stream_t stream);
 
 /* ts_scatter with an optional workspace (ts_scatter_workspace_bytes; 0 = no use for one). With it,
- * MIN / MAX of contended rows of 64 bytes and more, and SUM of such rows under an index that is not
- * sorted, first bin the entries by bucket of output rows (8 bytes per entry) and reduce every bucket
- * in LDS: no atomics on the table in memory except one write-back per chunk. MIN / MAX: same results
- * as ts_scatter; SUM: the same sum in another order of additions. No counterpart in the reference
+ * MIN / MAX of large inputs with rows of 64 bytes and more, and SUM of such rows under an index that
+ * is not sorted, first bin the entries by bucket of output rows (8 bytes per entry) and reduce every
+ * bucket in LDS: no atomics on the table in memory except one write-back per chunk. MIN / MAX of
+ * other large inputs of 4-byte elements with few entries per output row ask for 256 bytes: one flag,
+ * written by a sample of the index, that picks the kernel for a skewed or an even index. MIN / MAX: same
+ * results as ts_scatter; SUM: the same sum in another order of additions. No counterpart in the reference
  * (scatter_cuda allocates nothing beyond its outputs, csrc/cuda/scatter_cuda.cu:54-138). */
 size_t ts_scatter_workspace_bytes(int64_t B, int64_t E, int64_t K, int64_t N,
                                   int dtype, int reduce);

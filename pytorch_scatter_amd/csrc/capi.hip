@@ -338,7 +338,11 @@ size_t ts_scatter_workspace_bytes(int64_t B, int64_t E, int64_t K, int64_t N, in
   const bool any_size = env_int("TS_SCATTER_BINNED", 1) == 2;
   if (reduce == TS_MIN || reduce == TS_MAX) {
     if (kElemBytes[dtype] > 4) return 0;  // 64-bit elements do not use packed keys
-    return bin_plan(B, E, K, N, kElemBytes[dtype], nullptr, 0, any_size).bytes;
+    const size_t binned = bin_plan(B, E, K, N, kElemBytes[dtype], nullptr, 0, any_size).bytes;
+    if (binned != 0) return binned;
+    // one flag for the sample of the index that picks the kernel when few entries meet in an output row
+    const int probe = env_int("TS_SCATTER_SKEW", 1);
+    return probe && skew_probe_shape(B, E, K, N, kElemBytes[dtype], probe == 2) ? 256 : 0;
   }
   if (reduce == TS_SUM && kAccBytes[dtype] >= 4)  // table slots: int32 for int32, 8 bytes for the other types
     return bin_plan(B, E, K, N, kElemBytes[dtype], nullptr, 0, any_size, dtype == TS_I32 ? 4 : 8).bytes;
@@ -379,6 +383,7 @@ int ts_scatter_with_workspace(const void *src, const int64_t *index, void *out, 
   a.lds_epb = env_int("TS_SCATTER_EPB", 0);
   a.run_reduce = env_int("TS_SCATTER_RUNS", 1);
   a.lds_k1 = env_int("TS_SCATTER_LDS_K1", 1);
+  a.skew_probe = env_int("TS_SCATTER_SKEW", 1);  // tuning aid: 0 never, 2 at any size
   if (const int binned = env_int("TS_SCATTER_BINNED", 1)) {  // tuning aid: 0 never, 2 at any size
     a.bin_ws = workspace;
     a.bin_ws_bytes = workspace_bytes;

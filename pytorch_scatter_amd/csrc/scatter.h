@@ -212,7 +212,18 @@ struct ScatterArgs {
   size_t bin_ws_bytes = 0;
   int bin_any_size = 0;    // tuning aid / tests: also for inputs below the size from which it pays
   const int *skip_flag = nullptr;  // sum kernels: leave at once if *skip_flag != 0 (the binned pass did the work)
+  int skew_probe = 1;              // min/max: sample the index for skew (needs 256 bytes of workspace): 0 never, 2 at any size
+  const int *skew_flag = nullptr;  // min/max kernels behind the probe: run only if (*skew_flag != 0) == (skew_want != 0)
+  int skew_want = 0;
 };
+
+// Inputs for which the min/max launcher samples the index (see index_skew_kernel): rows of 2-256 columns of
+// 4-byte elements (16 bf16 columns lose through the table: 762 -> 1025 us), at least 32 M elements (the sample
+// and the launch that returns at once cost 10-20 us), fewer than 32 entries per output row on average.
+inline bool skew_probe_shape(int64_t B, int64_t E, int64_t K, int64_t N, int elem_bytes, bool any_size) {
+  return elem_bytes == 4 && K > 1 && K <= 256 && B * E >= 8192 &&
+         (any_size || (B * E * K >= ((int64_t)1 << 25) && E < 32 * N));
+}
 
 // ---- thread -> (edge, column) mapping shared by the scatter kernels ------------
 // A workgroup covers `epp` edges per pass with `L` lanes per edge, each lane
@@ -981,6 +992,7 @@ struct KeyRun {
 template <typename T, int C, bool IS_MAX, bool SERIAL>
 __global__ __launch_bounds__(kBlock) void scatter_key_run_kernel(ScatterArgs a, int lshift, int rows_per_wave) {
   __shared__ uint64_t s_stage[kBlock / kWave][kWave * C];
+  if (a.skew_flag != nullptr && (*a.skew_flag != 0) != (a.skew_want != 0)) return;
   KeyRun<T, C, IS_MAX> p;
   p.src = static_cast<const T *>(a.src);
   p.keys = reinterpret_cast<uint64_t *>(a.arg_out);
@@ -1005,6 +1017,7 @@ __global__ __launch_bounds__(kLdsBlock, (TAGS <= 256 ? 4 : 1)) void scatter_key_
   constexpr int U = VEC == 1 ? 8 : 4;
   __shared__ uint64_t s_keys[kLdsKeys];
   __shared__ int32_t s_tags[TAGS];  // TAGS >= table rows: kLdsKeys for narrow rows, 256 for K >= 16
+  if (a.skew_flag != nullptr && (*a.skew_flag != 0) != (a.skew_want != 0)) return;
   const int K = (int)a.K;
   const int tn = tn_mask + 1;
   for (int i = threadIdx.x; i < tn * K; i += kLdsBlock) s_keys[i] = 0;
@@ -1101,6 +1114,57 @@ __global__ __launch_bounds__(kLdsBlock, (TAGS <= 256 ? 4 : 1)) void scatter_key_
       if (key[j] != 0 && key[j] > cur[j])
         __hip_atomic_fetch_max(p[j], key[j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
+}
+
+// Is the index skewed? The table kernel above gains 2x on an unsorted index in which a few output rows own
+// much of the input (10 M entries of 8 / 32 floats onto 1 M rows, Zipf(1.2): 486 -> 244 / 1166 -> 681 us) and
+// loses as much on a uniform or sorted one, and the average number of entries per row does not tell them
+// apart. One workgroup looks at 1024 entries spread evenly over the index: *flag = 1 if at least a quarter
+// of them repeat an output row seen before (a hash set in LDS) and the sampled neighbours are not in
+// ascending order (a sorted index stays with the run kernel), else 0. The two kernels launched behind it
+// read the flag and one of them returns at once.
+constexpr int kSkewSamples = 1024;  // one per lane: widely spaced loads, most of them miss the TLB
+constexpr int kSkewSlots = 2048;
+constexpr int kSkewBlock = 1024;
+
+static __global__ __launch_bounds__(kSkewBlock) void index_skew_kernel(ScatterArgs a, int *flag) {
+  __shared__ int s_set[kSkewSlots];
+  __shared__ int s_dup, s_desc;
+  for (int i = threadIdx.x; i < kSkewSlots; i += kSkewBlock) s_set[i] = -1;
+  if (threadIdx.x == 0) { s_dup = 0; s_desc = 0; }
+  __syncthreads();
+  const int64_t n = a.B * a.E;
+  const int64_t step = n / kSkewSamples;  // the host only launches this with n >= 2 * kSkewSamples
+  int dup = 0, desc = 0;
+  constexpr int PER = kSkewSamples / kSkewBlock;
+  int64_t idx[PER], nxt[PER], bb[PER];
+#pragma unroll
+  for (int j = 0; j < PER; ++j) {  // all loads first: one memory latency for the whole sample
+    const int64_t be = (int64_t)(threadIdx.x + j * kSkewBlock) * step;
+    int64_t e, b1, e1;
+    split_edge(be, a.B, a.E, bb[j], e);
+    split_edge(be + 1, a.B, a.E, b1, e1);
+    idx[j] = a.index[bb[j] * a.sb + e * a.se];
+    nxt[j] = a.index[b1 * a.sb + e1 * a.se];
+    if (b1 != bb[j]) nxt[j] = idx[j];
+  }
+#pragma unroll
+  for (int j = 0; j < PER; ++j) {
+    if (nxt[j] < idx[j]) ++desc;
+    if (idx[j] < 0 || idx[j] >= a.N) continue;
+    const int node = (int)(bb[j] * a.N + idx[j]);
+    unsigned h = ((unsigned)node * 2654435761u) >> 21;  // 11 bits
+    for (int probe = 0; probe < 16; ++probe) {
+      const int old = atomicCAS(&s_set[h], -1, node);
+      if (old == -1) break;
+      if (old == node) { ++dup; break; }
+      h = (h + 1) & (kSkewSlots - 1);
+    }
+  }
+  if (dup) atomicAdd(&s_dup, dup);
+  if (desc) atomicAdd(&s_desc, desc);
+  __syncthreads();
+  if (threadIdx.x == 0) *flag = (s_dup * 4 >= kSkewSamples && s_desc * 64 >= kSkewSamples) ? 1 : 0;
 }
 
 // One value per entry (K == 1): the same table, written for occupancy. The general kernel above keeps
@@ -1584,15 +1648,39 @@ int launch_scatter_v(const ScatterArgs &args, int reduce, hipStream_t stream) {
         const RunGrid g = run_grid(n_edges, a.K / KC, 0, KC * (int)sizeof(T));
         if (g.ok) {
           const dim3 gd(g.blocks, g.ychunks);
+          // few entries per output row on average, 256 bytes of workspace: the sample of the index decides
+          // between this kernel and the table kernel (index_skew_kernel); both are launched, one returns at once
+          const bool probe = a.skew_probe && a.lds_cache == 1 && a.K % VEC == 0 && a.bin_ws != nullptr &&
+                             a.bin_ws_bytes >= 256 && ((uintptr_t)a.bin_ws & 3) == 0 &&
+                             skew_probe_shape(a.B, a.E, a.K, a.N, (int)sizeof(T), a.skew_probe == 2);
+          ScatterArgs ar = a, al = a;
+          if (probe) {
+            ar.skew_flag = al.skew_flag = static_cast<const int *>(a.bin_ws);
+            ar.skew_want = 0;
+            al.skew_want = 1;
+            hipLaunchKernelGGL(index_skew_kernel, dim3(1), dim3(kSkewBlock), 0, stream, a, static_cast<int *>(a.bin_ws));
+          }
           if (is_max) {
             hipLaunchKernelGGL((scatter_key_init_kernel<T, true>), dim3(g_out), dim3(kBlock), 0, stream, a);
             TS_LAUNCH_RUN(g.serial, (scatter_key_run_kernel<T, KC, true, true>), (scatter_key_run_kernel<T, KC, true, false>),
-                          gd, stream, a, g.lshift, g.rpw);
+                          gd, stream, ar, g.lshift, g.rpw);
+            if (probe && tn <= 256)
+              hipLaunchKernelGGL((scatter_key_lds_kernel<T, VEC, true, 256>), dim3(g_lds), dim3(kLdsBlock), 0, stream,
+                                 al, tn - 1, epb);
+            else if (probe)
+              hipLaunchKernelGGL((scatter_key_lds_kernel<T, VEC, true, kLdsKeys>), dim3(g_lds), dim3(kLdsBlock), 0,
+                                 stream, al, tn - 1, epb);
             hipLaunchKernelGGL((scatter_key_final_kernel<T, true>), dim3(g_out), dim3(kBlock), 0, stream, a);
           } else {
             hipLaunchKernelGGL((scatter_key_init_kernel<T, false>), dim3(g_out), dim3(kBlock), 0, stream, a);
             TS_LAUNCH_RUN(g.serial, (scatter_key_run_kernel<T, KC, false, true>),
-                          (scatter_key_run_kernel<T, KC, false, false>), gd, stream, a, g.lshift, g.rpw);
+                          (scatter_key_run_kernel<T, KC, false, false>), gd, stream, ar, g.lshift, g.rpw);
+            if (probe && tn <= 256)
+              hipLaunchKernelGGL((scatter_key_lds_kernel<T, VEC, false, 256>), dim3(g_lds), dim3(kLdsBlock), 0, stream,
+                                 al, tn - 1, epb);
+            else if (probe)
+              hipLaunchKernelGGL((scatter_key_lds_kernel<T, VEC, false, kLdsKeys>), dim3(g_lds), dim3(kLdsBlock), 0,
+                                 stream, al, tn - 1, epb);
             hipLaunchKernelGGL((scatter_key_final_kernel<T, false>), dim3(g_out), dim3(kBlock), 0, stream, a);
           }
           return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;

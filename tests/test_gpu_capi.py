@@ -565,6 +565,64 @@ def test_scatter_minmax_binned_variant(capi, oracle, shape, reduce, dtype, monke
     assert L.ts_scatter_workspace_bytes(capi._i(B), capi._i(E), capi._i(K), capi._i(N), capi.DTYPE[dtype], capi.MUL) == 0
 
 
+@pytest.mark.parametrize("shape,kind,reduce,dtype", product(
+    [(1, 60000, 8, 3000), (2, 40000, 4, 700), (1, 50000, 32, 9000), (1, 9000, 64, 1000), (1, 30000, 6, 500),
+     (3, 9000, 16, 50000)],
+    ["zipf", "uniform", "sorted zipf", "hub in sorted"], ["min", "max"],
+    [torch.float32, torch.bfloat16, torch.int32, torch.uint8]))
+def test_scatter_minmax_skew_probe(capi, oracle, shape, kind, reduce, dtype, monkeypatch):
+    """min / max with 256 bytes of workspace and few entries per output row: a sample of the index picks the
+    table kernel (skewed, unsorted index) or the run kernel (uniform or sorted index); forced on at these sizes.
+    Both must give the oracle's values and arg indices, with and without previous content in out."""
+    monkeypatch.setenv("TS_SCATTER_SKEW", "2")
+    B, E, K, N = shape
+    rng = np.random.default_rng(E + K)
+    src = random_values(rng, (B, E, K), dtype, ties=True)
+    if kind == "uniform":
+        idx = rng.integers(0, N, size=E)
+    else:
+        p = np.arange(1, N + 1, dtype=np.float64) ** -1.2
+        idx = rng.choice(N, size=E, p=p / p.sum())
+        if kind == "sorted zipf":
+            idx = np.sort(idx)
+        elif kind == "hub in sorted":
+            idx = np.sort(rng.integers(0, N, size=E))
+            idx[rng.random(E) < 0.4] = N // 3
+    index1 = torch.from_numpy(idx)
+    index = index1.view(1, E, 1).expand(B, E, K)
+    L = capi.lib()
+    need = L.ts_scatter_workspace_bytes(capi._i(B), capi._i(E), capi._i(K), capi._i(N), capi.DTYPE[dtype],
+                                        capi.REDUCE[reduce])
+    assert need == (256 if src.element_size() == 4 else 0)   # 4-byte elements only
+    for out_given in (False, True):
+        if out_given:
+            prev = random_values(rng, (B, N, K), dtype, ties=True)
+            want = prev.clone()
+            _, want_arg = oracle.scatter(src, index, 1, want, None, reduce)
+            out = prev.clone().to(DEV)
+        else:
+            want, want_arg = oracle.scatter(src, index, 1, None, N, reduce)
+            out = torch.empty((B, N, K), dtype=dtype, device=DEV)
+        arg = torch.empty((B, N, K), dtype=torch.long, device=DEV)
+        ws = capi.scatter_with_workspace(src.to(DEV), index1.to(DEV), out, arg, B, E, K, N, 0, 1, 0,
+                                         capi.REDUCE[reduce], out_given)
+        torch.cuda.synchronize()
+        assert_exact(out, want)
+        assert_exact(arg, want_arg)
+        if need == 0:
+            continue
+        # the probe's decision, restated: 1024 evenly spaced entries, repeats of an output row and descents
+        pos = np.arange(1024, dtype=np.int64) * ((B * E) // 1024)
+        b, e = pos // E, pos % E
+        dup = 1024 - np.unique(b * N + idx[e]).size
+        desc = int(np.sum(((pos + 1) // E == b) & (idx[(pos + 1) % E] < idx[e])))
+        flag = int(ws[:4].view(torch.int32).item())
+        if not (220 < dup < 290 or 12 < desc < 20):   # away from the thresholds (256 repeats, 16 descents)
+            assert flag == int(dup >= 256 and desc >= 16), (kind, dup, desc, flag)
+    if need:
+        assert flag == {"sorted zipf": 0, "zipf": 1}.get(kind, flag)
+
+
 @pytest.mark.parametrize("shape,kind,dtype", product(
     [(1, 60000, 32, 300), (2, 40000, 16, 700), (1, 50000, 128, 90), (1, 20000, 64, 100000), (3, 9000, 256, 5),
      (1, 30000, 24, 500)],
