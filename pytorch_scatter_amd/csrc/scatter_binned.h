@@ -19,7 +19,7 @@ namespace ts {
 
 constexpr int kBinKeys = 8192;        // keys of the LDS table: 64 KB, two workgroups per CU
 constexpr int kBinBlock = 1024;
-constexpr int kBinMaxBuckets = 4096;  // LDS histogram of count / place
+constexpr int kBinMaxBuckets = 8192;  // LDS histogram of count / place
 constexpr int kBinChunk = 8192;       // entries per chunk of a bucket in reduce (fewer for inputs under 4 M entries)
 constexpr int kBinPlaceChunk = 16384;  // entries per workgroup in count / place: one batch of 16 per lane
 constexpr int kBinPlaceBlock = 1024;   // (measured slower: 256 lanes x 4 batches, 64 K entries per workgroup, 8 K)
