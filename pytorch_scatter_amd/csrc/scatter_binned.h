@@ -40,6 +40,8 @@ struct BinArgs {
   int *unsorted;           // sum only (else null): set to 1 by the count pass when the index is not sorted;
                            // a sorted index is left to the kernels that combine runs, and the passes after
                            // the count return at once
+  int sampled = 0;         // sum only: *unsorted was set before the count pass from a sample of the index
+                           // (bin_sample_kernel); then the count pass returns at once as well
 };
 
 struct BinPlan {
@@ -172,9 +174,29 @@ __device__ __forceinline__ int32_t bin_take(int32_t *counter, int32_t bucket) {
   return before;
 }
 
+// Does the index look sorted? Sums of a sorted (or nearly sorted) index are left to the kernels that combine
+// runs, and finding that out with the full count pass costs 60-150 us for 10 M entries. It is a question of speed
+// only (both paths are correct for any index), so a sample answers it: 1024 evenly spaced entries and their right
+// neighbours, *flag = 1 (not sorted) if at least 1/64 of the pairs descend.
+static __global__ __launch_bounds__(kBinBlock) void bin_sample_kernel(ScatterArgs a, int *flag) {
+  __shared__ int s_desc;
+  if (threadIdx.x == 0) s_desc = 0;
+  __syncthreads();
+  const int64_t n = a.B * a.E;  // the host launches this only with n >= 2 * kBinBlock
+  const int64_t be = (int64_t)threadIdx.x * (n / kBinBlock);
+  const int64_t b = be / a.E, e = be - b * a.E;
+  const int64_t b1 = (be + 1) / a.E, e1 = be + 1 - b1 * a.E;
+  const int64_t idx = a.index[b * a.sb + e * a.se];
+  const int64_t nxt = a.index[b1 * a.sb + e1 * a.se];
+  if (b1 == b && nxt < idx) atomicAdd(&s_desc, 1);
+  __syncthreads();
+  if (threadIdx.x == 0) *flag = s_desc * 64 >= kBinBlock ? 1 : 0;
+}
+
 static __global__ __launch_bounds__(kBinPlaceBlock) void bin_count_kernel(ScatterArgs a, BinArgs p) {
   __shared__ int32_t s_hist[kBinMaxBuckets];
   __shared__ int s_hist_flag;
+  if (p.sampled && *p.unsorted == 0) return;
   for (int i = threadIdx.x; i < p.nb; i += kBinPlaceBlock) s_hist[i] = 0;
   if (threadIdx.x == 0) s_hist_flag = 0;
   __syncthreads();
@@ -183,7 +205,7 @@ static __global__ __launch_bounds__(kBinPlaceBlock) void bin_count_kernel(Scatte
   bool descent = false;
   for (int64_t b0 = lo; b0 < hi; b0 += kBinBatch) {
     int32_t bucket[kBinPer];
-    bin_buckets(a, p, b0, hi, bucket, nullptr, p.unsorted != nullptr ? &descent : nullptr);
+    bin_buckets(a, p, b0, hi, bucket, nullptr, p.unsorted != nullptr && !p.sampled ? &descent : nullptr);
 #pragma unroll
     for (int j = 0; j < kBinPer; ++j) bin_take(s_hist, bucket[j]);
   }
@@ -191,7 +213,7 @@ static __global__ __launch_bounds__(kBinPlaceBlock) void bin_count_kernel(Scatte
   // thousand wavefronts doing so one by one on the same address cost 100 us)
   if (__ballot(descent) != 0) s_hist_flag = 1;
   __syncthreads();
-  if (p.unsorted != nullptr && threadIdx.x == 0 && s_hist_flag != 0 &&
+  if (p.unsorted != nullptr && !p.sampled && threadIdx.x == 0 && s_hist_flag != 0 &&
       __hip_atomic_load(p.unsorted, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0)
     atomicOr(p.unsorted, 1);
   for (int i = threadIdx.x; i < p.nb; i += kBinPlaceBlock) {
@@ -206,6 +228,7 @@ static __global__ __launch_bounds__(kBinBlock) void bin_scan_kernel(BinArgs p) {
   constexpr int PER = kBinMaxBuckets / kBinBlock;
   __shared__ int64_t s_t[kBinBlock];
   __shared__ int64_t s_c[kBinBlock];
+  if (p.sampled && *p.unsorted == 0) return;
   int64_t t[PER], c[PER], sum_t = 0, sum_c = 0;
 #pragma unroll
   for (int j = 0; j < PER; ++j) {
@@ -557,9 +580,12 @@ void launch_binned_keys(const ScatterArgs &a, const BinArgs &plan, hipStream_t s
 // sum: count (with the test for a sorted index), scan, place, add. The caller launches its usual sum kernels
 // afterwards with skip_flag = p.unsorted: they run only if the index turned out to be sorted.
 template <typename T, int VEC>
-void launch_binned_add(const ScatterArgs &a, const BinArgs &p, int lshift, hipStream_t stream) {
+void launch_binned_add(const ScatterArgs &a, const BinArgs &plan, int lshift, hipStream_t stream) {
+  BinArgs p = plan;
+  p.sampled = a.B * a.E >= 2 * kBinBlock && !getenv("TS_BIN_NO_SAMPLE");  // env: tuning aid (sorted = no descent at all)
+  if (p.sampled) hipLaunchKernelGGL(bin_sample_kernel, dim3(1), dim3(kBinBlock), 0, stream, a, p.unsorted);
   hipLaunchKernelGGL(bin_clear_kernel, dim3((p.nb + kBlock - 1) / kBlock), dim3(kBlock), 0, stream, p.totals, p.nb,
-                     p.unsorted);
+                     p.sampled ? (int *)nullptr : p.unsorted);
   hipLaunchKernelGGL(bin_count_kernel, dim3((unsigned)p.n_place), dim3(kBinPlaceBlock), 0, stream, a, p);
   hipLaunchKernelGGL(bin_scan_kernel, dim3(1), dim3(kBinBlock), 0, stream, p);
   hipLaunchKernelGGL(bin_place_kernel, dim3((unsigned)p.n_place), dim3(kBinPlaceBlock), 0, stream, a, p);

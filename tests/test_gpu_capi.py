@@ -631,11 +631,14 @@ def test_scatter_minmax_skew_probe(capi, oracle, shape, kind, reduce, dtype, mon
     [torch.float32, torch.float64, torch.bfloat16, torch.float16, torch.int32, torch.int64, torch.int16]))
     + [((1, 20000, 64, 600000), "zipf", torch.float32), ((1, 20000, 64, 600000), "one descent", torch.int32)])  # 4688 buckets
 def test_scatter_sum_binned_variant(capi, oracle, shape, kind, dtype, monkeypatch):
-    """Sum with a workspace (forced on at these sizes): the first pass finds out whether the index is sorted;
+    """Sum with a workspace (forced on at these sizes): a sample of the index (or, with the sample switched
+    off as in the "one descent" cases, the count pass) finds out whether the index is sorted;
     if not, the entries are binned by bucket of output rows and added in LDS (double slots for floating
     types), else the usual kernels run. Exact for integers (int16 and K = 24 keep the path without
     workspace), within tolerance of the exact sum for floats, with and without previous content in out."""
     monkeypatch.setenv("TS_SCATTER_BINNED", "2")
+    if kind == "one descent":
+        monkeypatch.setenv("TS_BIN_NO_SAMPLE", "1")
     B, E, K, N = shape
     rng = np.random.default_rng(E + K + len(kind))
     p = np.arange(1, N + 1, dtype=np.float64) ** -1.2
