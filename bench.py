@@ -420,6 +420,12 @@ def main():
         table["X-zipf-unsorted-K8"] = bench_scatter_config(ts, wl, sz, dev, max(it // 2, 3), ["sum", "max"])
         sw32 = dataclasses.replace(wl.c4_scatter_minmax(32), name="X-zipf-unsorted-K32")
         table["X-zipf-unsorted-K32"] = bench_scatter_config(ts, wl, sw32, dev, max(it // 2, 3), ["sum"])
+        # few entries per output row (ten on average), unsorted: uniform index and the Zipf index from above
+        uni = torch.randint(0, 1_000_000, (wz.E,), generator=g)
+        su = wl.ScatterWorkload("X-uniform-deg10-K64", uni, 1_000_000, wz.E, 64, torch.float32)
+        table["X-uniform-deg10-K64"] = bench_scatter_config(ts, wl, su, dev, max(it // 2, 3), ["sum", "max"])
+        sz64 = wl.ScatterWorkload("X-zipf-unsorted-K64", zipf_index, 1_000_000, wz.E, 64, torch.float32)
+        table["X-zipf-unsorted-K64"] = bench_scatter_config(ts, wl, sz64, dev, max(it // 2, 3), ["sum", "max"])
         table["X-sorted-plan-C4-K32"] = bench_sorted_config(ts, wl, wl.c4_scatter_minmax(32), dev, max(it // 2, 3))
         ss = wl.ScatterWorkload("X-sorted-plan-C3-shuffled-K64", w3.index[torch.randperm(w3.E, generator=g)], w3.N, w3.E,
                                 64, torch.float32)
