@@ -19,7 +19,8 @@ namespace ts {
 
 constexpr int kBinKeys = 8192;        // keys of the LDS table: 64 KB, two workgroups per CU
 constexpr int kBinBlock = 1024;
-constexpr int kBinMaxBuckets = 8192;  // LDS histogram of count / place
+constexpr int kBinMaxBuckets = 16384;  // LDS histogram of count / place (their LDS is sized for 8192 or 16384 buckets)
+constexpr int kBinSmallCap = 8192;
 constexpr int kBinChunk = 8192;       // entries per chunk of a bucket in reduce (fewer for inputs under 4 M entries)
 constexpr int kBinPlaceChunk = 16384;  // entries per workgroup in count / place: one batch of 16 per lane
 constexpr int kBinPlaceBlock = 1024;   // (measured slower: 256 lanes x 4 batches, 64 K entries per workgroup, 8 K)
@@ -193,8 +194,9 @@ static __global__ __launch_bounds__(kBinBlock) void bin_sample_kernel(ScatterArg
   if (threadIdx.x == 0) *flag = s_desc * 64 >= kBinBlock ? 1 : 0;
 }
 
+template <int CAP>
 static __global__ __launch_bounds__(kBinPlaceBlock) void bin_count_kernel(ScatterArgs a, BinArgs p) {
-  __shared__ int32_t s_hist[kBinMaxBuckets];
+  __shared__ int32_t s_hist[CAP];
   __shared__ int s_hist_flag;
   if (p.sampled && *p.unsorted == 0) return;
   for (int i = threadIdx.x; i < p.nb; i += kBinPlaceBlock) s_hist[i] = 0;
@@ -283,9 +285,10 @@ static __global__ __launch_bounds__(kBinBlock) void bin_scan_kernel(BinArgs p) {
   }
 }
 
+template <int CAP>
 static __global__ __launch_bounds__(kBinPlaceBlock) void bin_place_kernel(ScatterArgs a, BinArgs p) {
-  __shared__ uint32_t s_base[kBinMaxBuckets];
-  __shared__ int32_t s_cnt[kBinMaxBuckets];
+  __shared__ uint32_t s_base[CAP];
+  __shared__ int32_t s_cnt[CAP];
   if (p.unsorted != nullptr && *p.unsorted == 0) return;
   for (int i = threadIdx.x; i < p.nb; i += kBinPlaceBlock) {
     const int32_t h = p.wg_hist[(int64_t)blockIdx.x * p.nb + i];
@@ -564,9 +567,15 @@ void launch_binned_keys(const ScatterArgs &a, const BinArgs &plan, hipStream_t s
   p.unsorted = nullptr;  // min / max take this path for sorted indices too
   hipLaunchKernelGGL(bin_clear_kernel, dim3((p.nb + kBlock - 1) / kBlock), dim3(kBlock), 0, stream, p.totals, p.nb,
                      (int *)nullptr);
-  hipLaunchKernelGGL(bin_count_kernel, dim3((unsigned)p.n_place), dim3(kBinPlaceBlock), 0, stream, a, p);
+  if (p.nb <= kBinSmallCap)
+    hipLaunchKernelGGL(bin_count_kernel<kBinSmallCap>, dim3((unsigned)p.n_place), dim3(kBinPlaceBlock), 0, stream, a, p);
+  else
+    hipLaunchKernelGGL(bin_count_kernel<kBinMaxBuckets>, dim3((unsigned)p.n_place), dim3(kBinPlaceBlock), 0, stream, a, p);
   hipLaunchKernelGGL(bin_scan_kernel, dim3(1), dim3(kBinBlock), 0, stream, p);
-  hipLaunchKernelGGL(bin_place_kernel, dim3((unsigned)p.n_place), dim3(kBinPlaceBlock), 0, stream, a, p);
+  if (p.nb <= kBinSmallCap)  // 64 KB of cursors, two workgroups per CU; above: 128 KB, one
+    hipLaunchKernelGGL(bin_place_kernel<kBinSmallCap>, dim3((unsigned)p.n_place), dim3(kBinPlaceBlock), 0, stream, a, p);
+  else
+    hipLaunchKernelGGL(bin_place_kernel<kBinMaxBuckets>, dim3((unsigned)p.n_place), dim3(kBinPlaceBlock), 0, stream, a, p);
   const int64_t kv = a.K / VEC;
   int lshift = 0;
   while (((int64_t)1 << lshift) < kv) ++lshift;
@@ -586,9 +595,15 @@ void launch_binned_add(const ScatterArgs &a, const BinArgs &plan, int lshift, hi
   if (p.sampled) hipLaunchKernelGGL(bin_sample_kernel, dim3(1), dim3(kBinBlock), 0, stream, a, p.unsorted);
   hipLaunchKernelGGL(bin_clear_kernel, dim3((p.nb + kBlock - 1) / kBlock), dim3(kBlock), 0, stream, p.totals, p.nb,
                      p.sampled ? (int *)nullptr : p.unsorted);
-  hipLaunchKernelGGL(bin_count_kernel, dim3((unsigned)p.n_place), dim3(kBinPlaceBlock), 0, stream, a, p);
+  if (p.nb <= kBinSmallCap)
+    hipLaunchKernelGGL(bin_count_kernel<kBinSmallCap>, dim3((unsigned)p.n_place), dim3(kBinPlaceBlock), 0, stream, a, p);
+  else
+    hipLaunchKernelGGL(bin_count_kernel<kBinMaxBuckets>, dim3((unsigned)p.n_place), dim3(kBinPlaceBlock), 0, stream, a, p);
   hipLaunchKernelGGL(bin_scan_kernel, dim3(1), dim3(kBinBlock), 0, stream, p);
-  hipLaunchKernelGGL(bin_place_kernel, dim3((unsigned)p.n_place), dim3(kBinPlaceBlock), 0, stream, a, p);
+  if (p.nb <= kBinSmallCap)  // 64 KB of cursors, two workgroups per CU; above: 128 KB, one
+    hipLaunchKernelGGL(bin_place_kernel<kBinSmallCap>, dim3((unsigned)p.n_place), dim3(kBinPlaceBlock), 0, stream, a, p);
+  else
+    hipLaunchKernelGGL(bin_place_kernel<kBinMaxBuckets>, dim3((unsigned)p.n_place), dim3(kBinPlaceBlock), 0, stream, a, p);
   hipLaunchKernelGGL((bin_add_wave_kernel<T, VEC>), dim3((unsigned)p.max_wgs), dim3(kBinBlock), 0, stream, a, p, lshift);
 }
 

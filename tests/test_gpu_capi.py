@@ -531,7 +531,8 @@ def test_scatter_minmax_lds_cached_variant(capi, oracle, shape, reduce, dtype, m
     [(1, 60000, 32, 300), (2, 40000, 16, 700), (1, 50000, 128, 90), (1, 30000, 24, 5000), (1, 20000, 64, 100000),
      (3, 9000, 512, 5), (1, 70000, 17, 40)],
     ["min", "max"], [torch.float32, torch.bfloat16, torch.int32, torch.int8]))
-    + [((1, 20000, 64, 600000), "max", torch.float32), ((1, 20000, 64, 600000), "min", torch.int32)])  # 4688 buckets
+    + [((1, 20000, 64, 600000), "max", torch.float32), ((1, 20000, 64, 600000), "min", torch.int32),  # 4688 buckets
+       ((1, 20000, 128, 540000), "max", torch.float32)])  # 8438 buckets
 def test_scatter_minmax_binned_variant(capi, oracle, shape, reduce, dtype, monkeypatch):
     """min / max with a workspace: entries binned by bucket of output rows and reduced in LDS (forced on at
     these sizes), skewed index with heavy ties, with and without previous content in out. Rows under 64 bytes
@@ -629,7 +630,8 @@ def test_scatter_minmax_skew_probe(capi, oracle, shape, kind, reduce, dtype, mon
      (1, 30000, 24, 500)],
     ["zipf", "sorted", "one descent"],
     [torch.float32, torch.float64, torch.bfloat16, torch.float16, torch.int32, torch.int64, torch.int16]))
-    + [((1, 20000, 64, 600000), "zipf", torch.float32), ((1, 20000, 64, 600000), "one descent", torch.int32)])  # 4688 buckets
+    + [((1, 20000, 64, 600000), "zipf", torch.float32), ((1, 20000, 64, 600000), "one descent", torch.int32),  # 4688 buckets
+       ((1, 20000, 128, 540000), "zipf", torch.int32)])  # 8438 buckets
 def test_scatter_sum_binned_variant(capi, oracle, shape, kind, dtype, monkeypatch):
     """Sum with a workspace (forced on at these sizes): a sample of the index (or, with the sample switched
     off as in the "one descent" cases, the count pass) finds out whether the index is sorted;
