@@ -76,6 +76,20 @@ int ts_segment_csr(const void *src, const int64_t *indptr, void *out,
                    int64_t indptr_batch_stride, int dtype, int reduce,
                    void *workspace, size_t workspace_bytes, ts_stream_t stream);
 
+/* ts_segment_csr without a workspace argument and without any allocation, for callers that cannot
+ * allocate device memory (code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc). It has no counterpart in the reference. Same kernels and same results as ts_segment_csr;
+ * the partial results of rows that cross a tile boundary go to a device array of
+ * TS_STATIC_SCRATCH_BYTES that the library holds on every GPU it runs on until the process ends.
+ * Inputs whose ts_segment_csr_workspace_bytes() exceeds that size return TS_ERR_WORKSPACE and launch
+ * nothing. All calls on one GPU share the array: calls that overlap in time on one GPU (two streams,
+ * two threads) race; calls on one stream, one after the other, are safe. */
+#define TS_STATIC_SCRATCH_BYTES (8u << 20)
+int ts_segment_csr_static(const void *src, const int64_t *indptr, void *out,
+                          int64_t *arg_out, int64_t B, int64_t N, int64_t E, int64_t K,
+                          int64_t indptr_batch_stride, int dtype, int reduce,
+                          ts_stream_t stream);
+
 /* ------------------------------------------------------------- gather_csr
  * out[b, e, :] = src[b, n, :] for e in [indptr[b, n], indptr[b, n+1])
  * Replaces gather_csr_cuda, csrc/cuda/segment_csr_cuda.cu:219-281 (kernels

@@ -22,7 +22,7 @@ DTYPE = {torch.float32: 0, torch.float64: 1, torch.float16: 2, torch.bfloat16: 3
 
 EXPORTS = (
     "ts_error_string", "ts_hip_version",
-    "ts_segment_csr_workspace_bytes", "ts_segment_csr", "ts_gather_csr",
+    "ts_segment_csr_workspace_bytes", "ts_segment_csr", "ts_segment_csr_static", "ts_gather_csr",
     "ts_segment_mean_csr_backward",
     "ts_segment_coo_workspace_bytes", "ts_segment_coo", "ts_gather_coo",
     "ts_segment_mean_coo_backward",
@@ -99,6 +99,18 @@ def segment_csr(src, indptr, out, arg_out, B, N, E, K, indptr_batch_stride, redu
                                 _i(indptr_batch_stride), DTYPE[out.dtype], reduce, _p(ws),
                                 ctypes.c_size_t(nbytes), _stream(out)))
     return ws
+
+
+STATIC_SCRATCH_BYTES = 8 << 20  # TS_STATIC_SCRATCH_BYTES of include/ts_hip.h
+
+
+def segment_csr_static(src, indptr, out, arg_out, B, N, E, K, indptr_batch_stride, reduce: int):
+    """ts_segment_csr_static: the same reduction with the library's own device array as scratch; nothing is
+    allocated here or in the library. Raises TsError (workspace) for inputs beyond the array's size."""
+    _dev(src, indptr, out, arg_out)
+    with torch.cuda.device(out.device):
+        _check(lib().ts_segment_csr_static(_p(src), _p(indptr), _p(out), _p(arg_out), _i(B), _i(N), _i(E), _i(K),
+                                           _i(indptr_batch_stride), DTYPE[out.dtype], reduce, _stream(out)))
 
 
 def gather_csr(src, indptr, out, B, N, E, K, indptr_batch_stride):

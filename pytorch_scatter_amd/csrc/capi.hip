@@ -238,6 +238,45 @@ int ts_segment_mean_csr_backward(const void *grad_out, const int64_t *indptr, vo
   return dispatch_csr_gather(dtype, a, p, B, true, static_cast<hipStream_t>(stream));
 }
 
+// ---- ts_segment_csr for callers that cannot allocate: the partial results of rows that cross tiles
+// live in a file-scope device array instead of a caller's workspace. Every GPU holds its own copy
+// of the array at its own address; the address is looked up once per device, with that device current.
+constexpr size_t kStaticScratchBytes = (size_t)TS_STATIC_SCRATCH_BYTES;
+constexpr int kStaticScratchDevices = 64;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+static std::atomic<void *> g_scratch_ptr[kStaticScratchDevices];
+
+static int static_scratch_ptr(void **out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kStaticScratchDevices) return TS_ERR_LAUNCH;
+  void *p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (p == nullptr) {
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || p == nullptr) return TS_ERR_LAUNCH;
+    g_scratch_ptr[dev].store(p, std::memory_order_release);
+  }
+  *out = p;
+  return TS_OK;
+}
+
+int ts_segment_csr_static(const void *src, const int64_t *indptr, void *out, int64_t *arg_out, int64_t B,
+                          int64_t N, int64_t E, int64_t K, int64_t indptr_batch_stride, int dtype, int reduce,
+                          ts_stream_t stream) {
+  if (!valid_dtype(dtype) || !sizes_ok(B, N, E, K)) return TS_ERR_BAD_ARG;
+  if (reduce != TS_SUM && reduce != TS_MEAN && reduce != TS_MIN && reduce != TS_MAX) return TS_ERR_UNSUPPORTED;
+  if (B * N * K == 0) return TS_OK;
+  if (!indptr || !out || (E * K > 0 && !src)) return TS_ERR_BAD_ARG;
+  if ((reduce == TS_MIN || reduce == TS_MAX) && !arg_out) return TS_ERR_BAD_ARG;
+  // the array is fixed in size: larger inputs must bring a workspace (ts_segment_csr)
+  if (csr_workspace_max(B, N, E, K, dtype, reduce) > kStaticScratchBytes) return TS_ERR_WORKSPACE;
+  void *ws = nullptr;
+  const int rc = static_scratch_ptr(&ws);
+  if (rc != TS_OK) return rc;
+  // Nothing in the array has to start at zero: the carry flags of a call hold that call's nonce, and
+  // the second kernel only reads what the first one wrote in the same call.
+  return run_csr_reduce(src, indptr, out, arg_out, nullptr, B, N, E, K, indptr_batch_stride, dtype, reduce, 0, ws,
+                        kStaticScratchBytes, static_cast<hipStream_t>(stream));
+}
+
 size_t ts_segment_csr_permuted_workspace_bytes(int64_t B, int64_t N, int64_t E, int64_t K, int dtype, int reduce) {
   if (!valid_dtype(dtype) || !sizes_ok(B, N, E, K)) return 0;
   const bool wa = reduce == TS_MIN || reduce == TS_MAX;
