@@ -6,6 +6,7 @@
 
 #include <atomic>
 #include <chrono>
+#include <type_traits>
 
 #include "csr_reduce.h"
 #include "csr_gather.h"
@@ -77,10 +78,26 @@ int dispatch_group_softmax(int dtype, const GroupArgs &g, int mode, int vec, hip
   }
 }
 
-// The reduction keeps edge positions in 32 bits inside a tile.
+// The reductions keep edge positions in 32 bits inside a tile. B is only bounded by the 64-bit element
+// offsets: kernels that put the batch into a grid dimension are launched in slices (for_batch_slices).
 inline bool sizes_ok(int64_t B, int64_t N, int64_t E, int64_t K) {
   return B >= 0 && N >= 0 && E >= 0 && K >= 0 && E < 0x7FFFFFFFll && N < 0x7FFFFFFFll &&
-         B <= 65535 && K < ((int64_t)1 << 40);
+         B < 0x7FFFFFFFll && K < ((int64_t)1 << 40);
+}
+
+// grid.y / grid.z hold at most 65535 workgroups: batches beyond that take further launches on the
+// same stream. fn(first batch, number of batches) -> status.
+constexpr int64_t kMaxGridBatches = 65535;
+template <typename F> int for_batch_slices(int64_t B, F fn) {
+  for (int64_t b0 = 0; b0 < B; b0 += kMaxGridBatches) {
+    const int rc = fn(b0, B - b0 < kMaxGridBatches ? B - b0 : kMaxGridBatches);
+    if (rc != TS_OK) return rc;
+  }
+  return TS_OK;
+}
+template <typename P> inline P *offset_bytes(P *p, int64_t bytes) {
+  typedef typename std::conditional<std::is_const<P>::value, const char, char>::type C;
+  return p == nullptr ? nullptr : reinterpret_cast<P *>(reinterpret_cast<C *>(p) + bytes);
 }
 
 int env_int(const char *name, int fallback) {
@@ -114,10 +131,10 @@ size_t csr_workspace_max(int64_t B, int64_t N, int64_t E, int64_t K, int dtype, 
   return w1 > w0 ? w1 : w0;
 }
 
-int run_csr_reduce(const void *src, const int64_t *indptr, void *out, int64_t *arg_out, void *count_out,
-                   int64_t B, int64_t N, int64_t E, int64_t K, int64_t indptr_batch_stride, int dtype,
-                   int reduce, int accumulate, void *ws, size_t ws_bytes, hipStream_t stream,
-                   const int32_t *perm = nullptr, int64_t perm_batch_stride = 0, bool *perm_args_done = nullptr) {
+int run_csr_reduce_slice(const void *src, const int64_t *indptr, void *out, int64_t *arg_out, void *count_out,
+                         int64_t B, int64_t N, int64_t E, int64_t K, int64_t indptr_batch_stride, int dtype,
+                         int reduce, int accumulate, void *ws, size_t ws_bytes, hipStream_t stream,
+                         const int32_t *perm, int64_t perm_batch_stride, bool want_perm_args, bool *perm_args_done) {
   const bool al = aligned16(src) && aligned16(out);
   // permuted rows always take the wide kernel (the narrow one stages consecutive entries)
   const CsrPlan p = csr_plan(N, E, K, kElemBytes[dtype], al, false, reduce == TS_MIN || reduce == TS_MAX,
@@ -152,9 +169,64 @@ int run_csr_reduce(const void *src, const int64_t *indptr, void *out, int64_t *a
   // in src's order right away;
   // when the output is large: the lookup at every row end makes the wavefront wait, a pass over [N, K]
   // afterwards moves 20 bytes per element (C4, 3.2 M elements: 13 us as a pass, +17 us fused; 68 M: 334 vs 150 us)
-  a.perm_args = perm != nullptr && (a.lookback || p.nblk <= 1) && B * N * K >= ((int64_t)8 << 20);
+  a.perm_args = perm != nullptr && (a.lookback || p.nblk <= 1) && want_perm_args;
   if (perm_args_done) *perm_args_done = a.perm_args != 0;
+  if (p.ychunks > kMaxGridBatches) return TS_ERR_UNSUPPORTED;
   return dispatch_csr_reduce(dtype, a, p, B, reduce, stream);
+}
+
+int run_csr_reduce(const void *src, const int64_t *indptr, void *out, int64_t *arg_out, void *count_out,
+                   int64_t B, int64_t N, int64_t E, int64_t K, int64_t indptr_batch_stride, int dtype,
+                   int reduce, int accumulate, void *ws, size_t ws_bytes, hipStream_t stream,
+                   const int32_t *perm = nullptr, int64_t perm_batch_stride = 0, bool *perm_args_done = nullptr) {
+  const int64_t s = kElemBytes[dtype];
+  const bool want_perm_args = B * N * K >= ((int64_t)8 << 20);
+  // every slice reuses the workspace: the launches follow each other on one stream
+  return for_batch_slices(B, [&](int64_t b0, int64_t nb) {
+    return run_csr_reduce_slice(offset_bytes(src, b0 * E * K * s), indptr + b0 * indptr_batch_stride,
+                                offset_bytes(out, b0 * N * K * s), arg_out ? arg_out + b0 * N * K : nullptr,
+                                offset_bytes(count_out, b0 * N * s), nb, N, E, K, indptr_batch_stride, dtype, reduce,
+                                accumulate, ws, ws_bytes, stream, perm ? perm + b0 * perm_batch_stride : nullptr,
+                                perm_batch_stride, want_perm_args, perm_args_done);
+  });
+}
+
+int run_csr_gather(int dtype, const CsrGatherArgs &args, const CsrPlan &p, int64_t B, bool divide, hipStream_t s) {
+  if (p.ychunks > kMaxGridBatches) return TS_ERR_UNSUPPORTED;
+  const int64_t sz = kElemBytes[dtype];
+  return for_batch_slices(B, [&](int64_t b0, int64_t nb) {
+    CsrGatherArgs a = args;
+    a.src = offset_bytes(args.src, b0 * args.N * args.K * sz);
+    a.indptr = args.indptr + b0 * args.indptr_batch_stride;
+    a.out = offset_bytes(args.out, b0 * args.E * args.K * sz);
+    return dispatch_csr_gather(dtype, a, p, nb, divide, s);
+  });
+}
+
+int run_coo_gather(int dtype, const CooGatherArgs &args, const CooGatherPlan &p, int64_t B, bool divide,
+                   hipStream_t s) {
+  if (p.ychunks > kMaxGridBatches) return TS_ERR_UNSUPPORTED;
+  const int64_t sz = kElemBytes[dtype];
+  return for_batch_slices(B, [&](int64_t b0, int64_t nb) {
+    CooGatherArgs a = args;
+    a.src = offset_bytes(args.src, b0 * args.N * args.K * sz);
+    a.index = args.index + b0 * args.index_batch_stride;
+    a.count = offset_bytes(args.count, b0 * args.N * sz);
+    a.out = offset_bytes(args.out, b0 * args.E * args.K * sz);
+    return dispatch_coo_gather(dtype, a, p, nb, divide, s);
+  });
+}
+
+// sorted index [B, E] -> row pointers [B, N + 1] (contiguous)
+int run_coo_to_indptr(const int64_t *index, int64_t *ptr, int64_t B, int64_t E, int64_t N, int64_t index_batch_stride,
+                      hipStream_t s) {
+  const int64_t per_block = (int64_t)kBlock * kCooPtrPerThread;
+  return for_batch_slices(B, [&](int64_t b0, int64_t nb) {
+    dim3 grid((unsigned)((E + 1 + per_block - 1) / per_block), (unsigned)nb);
+    hipLaunchKernelGGL(coo_to_indptr_kernel, grid, dim3(kBlock), 0, s, index + b0 * index_batch_stride,
+                       ptr + b0 * (N + 1), N, E, index_batch_stride);
+    return hipGetLastError() == hipSuccess ? (int)TS_OK : (int)TS_ERR_LAUNCH;
+  });
 }
 
 }  // namespace
@@ -212,7 +284,7 @@ int ts_gather_csr(const void *src, const int64_t *indptr, void *out, int64_t B, 
   a.BI = p.BI;
   a.ipw = p.ipw;
   a.nblk = p.nblk;
-  return dispatch_csr_gather(dtype, a, p, B, false, static_cast<hipStream_t>(stream));
+  return run_csr_gather(dtype, a, p, B, false, static_cast<hipStream_t>(stream));
 }
 
 int ts_segment_mean_csr_backward(const void *grad_out, const int64_t *indptr, void *grad_in, int64_t B,
@@ -235,7 +307,7 @@ int ts_segment_mean_csr_backward(const void *grad_out, const int64_t *indptr, vo
   a.BI = p.BI;
   a.ipw = p.ipw;
   a.nblk = p.nblk;
-  return dispatch_csr_gather(dtype, a, p, B, true, static_cast<hipStream_t>(stream));
+  return run_csr_gather(dtype, a, p, B, true, static_cast<hipStream_t>(stream));
 }
 
 // ---- ts_segment_csr for callers that cannot allocate: the partial results of rows that cross tiles
@@ -321,10 +393,8 @@ int ts_segment_coo(const void *src, const int64_t *index, void *out, void *arg_o
   if (!workspace || workspace_bytes < ptr_bytes) return TS_ERR_WORKSPACE;
   hipStream_t s = static_cast<hipStream_t>(stream);
   int64_t *ptr = static_cast<int64_t *>(workspace);
-  const int64_t per_block = (int64_t)kBlock * kCooPtrPerThread;
-  dim3 grid((unsigned)((E + 1 + per_block - 1) / per_block), (unsigned)B);
-  hipLaunchKernelGGL(coo_to_indptr_kernel, grid, dim3(kBlock), 0, s, index, ptr, N, E, index_batch_stride);
-  if (hipGetLastError() != hipSuccess) return TS_ERR_LAUNCH;
+  const int rc = run_coo_to_indptr(index, ptr, B, E, N, index_batch_stride, s);
+  if (rc != TS_OK) return rc;
   return run_csr_reduce(src, ptr, out, static_cast<int64_t *>(arg_out), count_out, B, N, E, K, N + 1, dtype,
                         reduce, out_given ? 1 : 0, static_cast<char *>(workspace) + ptr_bytes,
                         workspace_bytes - ptr_bytes, s);
@@ -347,7 +417,7 @@ int ts_gather_coo(const void *src, const int64_t *index, void *out, int64_t B, i
   a.index_batch_stride = index_batch_stride;
   a.G = p.G;
   a.epw = p.epw;
-  return dispatch_coo_gather(dtype, a, p, B, false, static_cast<hipStream_t>(stream));
+  return run_coo_gather(dtype, a, p, B, false, static_cast<hipStream_t>(stream));
 }
 
 int ts_segment_mean_coo_backward(const void *grad_out, const int64_t *index, const void *count,
@@ -369,7 +439,7 @@ int ts_segment_mean_coo_backward(const void *grad_out, const int64_t *index, con
   a.index_batch_stride = index_batch_stride;
   a.G = p.G;
   a.epw = p.epw;
-  return dispatch_coo_gather(dtype, a, p, B, true, static_cast<hipStream_t>(stream));
+  return run_coo_gather(dtype, a, p, B, true, static_cast<hipStream_t>(stream));
 }
 
 size_t ts_scatter_workspace_bytes(int64_t B, int64_t E, int64_t K, int64_t N, int dtype, int reduce) {
@@ -673,11 +743,7 @@ int ts_index_to_indptr(const int64_t *index, int64_t *indptr, int64_t B, int64_t
   if (B < 0 || E < 0 || N < 0) return TS_ERR_BAD_ARG;
   if (B == 0) return TS_OK;
   if (!indptr || (E > 0 && !index)) return TS_ERR_BAD_ARG;
-  const int64_t per_block = (int64_t)kBlock * kCooPtrPerThread;
-  dim3 grid((unsigned)((E + 1 + per_block - 1) / per_block), (unsigned)B);
-  hipLaunchKernelGGL(coo_to_indptr_kernel, grid, dim3(kBlock), 0, static_cast<hipStream_t>(stream), index, indptr, N,
-                     E, index_batch_stride);
-  return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
+  return run_coo_to_indptr(index, indptr, B, E, N, index_batch_stride, static_cast<hipStream_t>(stream));
 }
 
 size_t ts_indptr_to_index_workspace_bytes(int64_t B, int64_t N) {

@@ -149,17 +149,23 @@ __global__ __launch_bounds__(kBlock) void csr_gather_small_kernel(CsrGatherArgs 
   __syncthreads();
   const int rmax = nload - 2;  // last local row whose end is known; i0 + rmax <= N - 1
   if (rmax < 0) return;
+  // entries in front of indptr[0] or behind indptr[N] belong to no row and are left as they are
+  const int64_t w0 = ptr[0] - j0, w1 = ptr[a.N] - j0;
+  const int e_lo = w0 < 0 ? 0 : (w0 > ne ? ne : (int)w0);
+  const int e_hi = w1 < 0 ? 0 : (w1 > ne ? ne : (int)w1);
+  if (e_hi <= e_lo) return;
+  const int64_t fbase = j0 * K;  // element offset of the tile's first entry: entry numbers below are relative to it
 
   if (!VROW) {
     // Rows of 1-3 elements: a 16-byte granule of out covers several entries. Its first entry's row comes
     // from a binary search of the tile's row pointers (about ten LDS reads), the following entries
     // advance from there; no per-entry row table, no barriers.
-    const int64_t f0 = j0 * K, f1 = (j0 + ne) * K;
+    const int64_t f0 = (j0 + e_lo) * K, f1 = (j0 + e_hi) * K;
     const int64_t g0 = f0 / VE, g1 = (f1 + VE - 1) / VE;
     for (int64_t g = g0 + tid; g < g1; g += kBlock) {
       const int64_t fb = g * VE > f0 ? g * VE : f0;
       const int64_t fe = (g + 1) * VE < f1 ? (g + 1) * VE : f1;
-      const unsigned rel = (unsigned)(fb - f0);  // 32-bit arithmetic relative to the tile (f0 is a row start)
+      const unsigned rel = (unsigned)(fb - fbase);  // 32-bit arithmetic relative to the tile
       int e = (int)(rel / (unsigned)K);          // entry, relative to the tile
       int k = (int)(rel - (unsigned)e * (unsigned)K);
       int lo = 0, hi = rmax;  // the last row that starts at or before e (rows without entries share a start)
@@ -231,8 +237,9 @@ __global__ __launch_bounds__(kBlock) void csr_gather_small_kernel(CsrGatherArgs 
   __syncthreads();
 
   // elements of out_b this tile owns, cut into 16-byte granules of the whole buffer
-  const int64_t f0 = j0 * K, f1 = (j0 + ne) * K;
+  const int64_t f0 = (j0 + e_lo) * K, f1 = (j0 + e_hi) * K;
   const int64_t g0 = f0 / VE, g1 = (f1 + VE - 1) / VE;
+  const int64_t gbase = fbase / VE;  // rows are whole granules here
   if (VROW) {
     const int kv = K / VE;  // granules per row
     constexpr int U = 4;  // independent row loads in flight per lane
@@ -242,7 +249,7 @@ __global__ __launch_bounds__(kBlock) void csr_gather_small_kernel(CsrGatherArgs 
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         const int64_t g = gb + (int64_t)u * kBlock < g1 ? gb + (int64_t)u * kBlock : gb;
-        const unsigned gl = (unsigned)(g - g0);  // 32-bit arithmetic relative to the tile (f0 is a row start)
+        const unsigned gl = (unsigned)(g - gbase);  // 32-bit arithmetic relative to the tile
         const int e = (int)(gl / (unsigned)kv);
         const int c = (int)(gl - (unsigned)e * (unsigned)kv);
         row[u] = s_row[e];

@@ -254,8 +254,11 @@ __global__ __launch_bounds__(kBlock, (csr_reduce_min_blocks<T, VEC, REDUCE, PERM
   dw1 = dw1 < tile_items ? dw1 : tile_items;
   const int ri0 = merge_search_lds(s_ptr, nr, ne, dw0);
   const int ri1 = merge_search_lds(s_ptr, nr, ne, dw1);
-  const int je0 = dw0 - ri0;
+  int je0 = dw0 - ri0;
   const int je1 = dw1 - ri1;
+  // Entries in front of the first row pointer (indptr[0] > 0) belong to no row. Only row 0 can begin
+  // behind a worker's first entry: every other row begins where the row before it ended.
+  if (i0 + ri0 == 0 && s_ptr[0] > je0) je0 = s_ptr[0] < je1 ? s_ptr[0] : je1;
 
   auto row_end = [&](int r) -> int32_t { return s_ptr[r + 1]; };  // r + 1 <= nload + 1: a sentinel at the latest
 

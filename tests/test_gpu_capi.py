@@ -993,3 +993,136 @@ def test_error_codes(capi):
         capi.segment_csr(x, ptr, x, None, 1, 2, 4, 4, 0, capi.MUL)
     with pytest.raises(capi.TsError, match="device"):
         capi.gather_csr(x.cpu(), ptr, x, 1, 2, 4, 4, 0)
+
+
+# ---- row pointers that do not start at 0 or do not end at E: entries outside [indptr[0], indptr[N]) belong to
+# no row (csrc/cuda/segment_csr_cuda.cu:30-33 reduces [indptr[n], indptr[n+1]) only)
+WINDOW_CASES = [
+    # kind, rows, K, entries in front of the first row, entries behind the last row
+    ("zipf", 2000, 64, 37, 11), ("hub", 900, 64, 5000, 0), ("short", 300, 1, 3, 9), ("zipf", 2500, 4, 700, 1),
+    ("hub", 500, 128, 1, 2500), ("long", 9, 8, 30000, 5), ("short", 50, 200, 9000, 9000), ("hub", 300, 16, 2, 2),
+]
+
+
+def make_window(case, seed):
+    kind, n, K, front, back = case
+    rng, indptr, _ = make_csr(kind, seed, n)
+    if kind != "short":
+        indptr = indptr.clone()
+        # the first rows empty too: row 0 is not the one that begins behind the entries in front
+        indptr[1:3] = 0
+    return rng, indptr + front, int(indptr[-1]) + front + back
+
+
+@pytest.mark.parametrize("case,reduce,dtype", product(
+    WINDOW_CASES, ["sum", "mean", "min", "max"], [torch.float32, torch.bfloat16]))
+def test_segment_csr_window_of_entries(capi, oracle, case, reduce, dtype):
+    n, K = case[1], case[2]
+    rng, indptr, E = make_window(case, 300 + WINDOW_CASES.index(case))
+    src = values(rng, (E, K), dtype, reduce)
+    want, want_arg = oracle.segment_csr(src, indptr, None, reduce)
+    out = torch.full((n, K), 7, dtype=dtype, device=DEV)
+    arg = torch.full((n, K), -1, dtype=torch.long, device=DEV) if reduce in ("min", "max") else None
+    capi.segment_csr(src.to(DEV), indptr.to(DEV), out, arg, 1, n, E, K, 0, capi.REDUCE[reduce])
+    torch.cuda.synchronize()
+    if reduce in ("min", "max"):
+        assert_exact(out, want, "values")
+        assert_exact(arg, want_arg, "arg")
+    else:
+        scale = float(oracle.segment_csr(src.abs().double(), indptr, None, "sum")[0].max())
+        assert_close(out, want, scale, dtype, "values")
+
+
+@pytest.mark.parametrize("case,dtype", product(WINDOW_CASES, [torch.float32, torch.bfloat16]))
+def test_gather_csr_and_mean_backward_window_of_entries(capi, oracle, case, dtype):
+    """Positions of the output outside [indptr[0], indptr[N]) are left as they were."""
+    n, K = case[1], case[2]
+    rng, indptr, E = make_window(case, 400 + WINDOW_CASES.index(case))
+    src = random_values(rng, (n, K), dtype, ties=False)
+    lo, hi = int(indptr[0]), int(indptr[-1])
+    want = torch.full((E, K), 3, dtype=dtype)
+    want[lo:hi] = oracle.gather_csr(src, indptr - lo)
+    out = torch.full((E, K), 3, dtype=dtype, device=DEV)
+    capi.gather_csr(src.to(DEV), indptr.to(DEV), out, 1, n, E, K, 0)
+    torch.cuda.synchronize()
+    assert_exact(out, want)
+    want[lo:hi] = oracle.segment_mean_csr_backward(src, indptr - lo, (hi - lo, K))
+    out.fill_(3)
+    capi.segment_mean_csr_backward(src.to(DEV), indptr.to(DEV), out, 1, n, E, K, 0)
+    torch.cuda.synchronize()
+    assert_exact(out, want)
+
+
+@pytest.mark.parametrize("reduce", ["sum", "mean", "max"])
+def test_segment_csr_batched_window_of_entries(capi, oracle, reduce):
+    rng = np.random.default_rng(77)
+    B, n, K, E = 3, 400, 32, 9000
+    ptrs = []
+    for b in range(B):
+        deg = rng.multinomial(E - 40 * (b + 1), np.ones(n) / n)
+        ptrs.append(np.concatenate([[0], np.cumsum(deg)]) + 13 * (b + 1))
+    indptr = torch.from_numpy(np.stack(ptrs).astype(np.int64))
+    src = values(rng, (B, E, K), torch.float32, reduce)
+    want, want_arg = oracle.segment_csr(src, indptr, None, reduce)
+    out = torch.empty((B, n, K), dtype=torch.float32, device=DEV)
+    arg = torch.empty((B, n, K), dtype=torch.long, device=DEV) if reduce == "max" else None
+    capi.segment_csr(src.to(DEV), indptr.to(DEV), out, arg, B, n, E, K, n + 1, capi.REDUCE[reduce])
+    torch.cuda.synchronize()
+    if reduce == "max":
+        assert_exact(out, want)
+        assert_exact(arg, want_arg)
+    else:
+        assert_close(out, want, float(src.abs().sum(1).max()), torch.float32)
+
+
+# ---- more batch rows than a grid dimension holds (65535): the reference has no such limit
+# (csrc/cuda/segment_csr_cuda.cu:144-160 puts the batch into the flat thread index)
+@pytest.mark.parametrize("reduce,K", product(["sum", "mean", "max"], [1, 8]))
+def test_segment_csr_and_gathers_with_70000_batch_rows(capi, oracle, reduce, K):
+    rng = np.random.default_rng(78)
+    B, n, E = 70000, 3, 7
+    deg = rng.multinomial(E, np.ones(n) / n, size=B)
+    indptr = torch.from_numpy(np.concatenate([np.zeros((B, 1), np.int64), np.cumsum(deg, 1)], 1).astype(np.int64))
+    src = values(rng, (B, E, K), torch.float32, reduce)
+    want, want_arg = oracle.segment_csr(src, indptr, None, reduce)
+    out = torch.empty((B, n, K), dtype=torch.float32, device=DEV)
+    arg = torch.empty((B, n, K), dtype=torch.long, device=DEV) if reduce == "max" else None
+    dptr = indptr.to(DEV)
+    capi.segment_csr(src.to(DEV), dptr, out, arg, B, n, E, K, n + 1, capi.REDUCE[reduce])
+    torch.cuda.synchronize()
+    if reduce == "max":
+        assert_exact(out, want)
+        assert_exact(arg, want_arg)
+    else:
+        assert_close(out, want, float(src.abs().sum(1).max()), torch.float32)
+    if reduce == "sum":
+        # the gathers and the index-keyed reduction over the same batches
+        back = torch.empty((B, E, K), dtype=torch.float32, device=DEV)
+        capi.gather_csr(out, dptr, back, B, n, E, K, n + 1)
+        assert_exact(back, oracle.gather_csr(out.cpu(), indptr))
+        index = torch.from_numpy(np.stack([np.repeat(np.arange(n), d) for d in deg]).astype(np.int64))
+        capi.gather_coo(out, index.to(DEV), back, B, n, E, K, E)
+        assert_exact(back, oracle.gather_coo(out.cpu(), index))
+        out2 = torch.empty_like(out)
+        capi.segment_coo(src.to(DEV), index.to(DEV), out2, None, None, B, n, E, K, E, capi.SUM, False)
+        torch.cuda.synchronize()
+        assert_close(out2, want, float(src.abs().sum(1).max()), torch.float32)
+
+
+@pytest.mark.parametrize("reduce", ["sum", "max"])
+def test_scatter_with_70000_batch_rows(capi, oracle, reduce):
+    """scatter along the last dimension of a [70000, 16] tensor (the reference's default dim = -1)."""
+    rng = np.random.default_rng(79)
+    B, E, N = 70000, 16, 5
+    src = values(rng, (B, E), torch.float32, reduce)
+    index = torch.from_numpy(rng.integers(0, N, size=(B, E)).astype(np.int64))
+    want, want_arg = oracle.scatter(src, index, 1, None, N, reduce)
+    out = torch.empty((B, N), dtype=torch.float32, device=DEV)
+    arg = torch.empty((B, N), dtype=torch.long, device=DEV) if reduce == "max" else None
+    capi.scatter(src.to(DEV), index.to(DEV), out, arg, B, E, 1, N, E, 1, 0, capi.REDUCE[reduce], False)
+    torch.cuda.synchronize()
+    if reduce == "max":
+        assert_exact(out, want)
+        assert_exact(arg, want_arg)
+    else:
+        assert_close(out, want, float(src.abs().sum(1).max()), torch.float32)

@@ -440,3 +440,66 @@ def test_scatter_mean_counts_from_the_index(ts, oracle):
     ts.scatter_mean(src, index.to(DEV), 0, None, 25).backward(grad.to(DEV))
     count = torch.bincount(index, minlength=25).clamp(min=1).double()
     assert torch.allclose(src.grad.cpu(), (grad / count.view(-1, 1))[index], rtol=1e-12)
+
+
+@pytest.mark.parametrize("reduce", ["sum", "mean", "min", "max"])
+def test_segment_csr_row_pointers_that_start_behind_zero(ts, reduce):
+    """indptr[0] > 0 and indptr[-1] < E: only [indptr[n], indptr[n+1]) is reduced
+    (csrc/cuda/segment_csr_cuda.cu:30-33); forward and backward against the oracle."""
+    import ts_oracle
+    rng = np.random.default_rng(91)
+    n, K, front, back = 700, 64, 41, 17
+    deg = np.minimum(rng.zipf(1.7, size=n), 3000)
+    indptr = torch.from_numpy(np.concatenate([[0], np.cumsum(deg)]).astype(np.int64)) + front
+    E = int(indptr[-1]) + back
+    src = random_values(rng, (E, K), torch.float32, ties=reduce in ("min", "max"))
+    want, want_arg = ts_oracle.segment_csr(src, indptr, None, reduce)
+    x = src.to(DEV).requires_grad_()
+    got = ts.segment_csr(x, indptr.to(DEV), None, reduce)
+    if reduce in ("min", "max"):
+        assert torch.equal(got.detach().cpu(), want)
+    else:
+        scale = float(ts_oracle.segment_csr(src.abs(), indptr, None, "sum")[0].max())
+        assert bool(((got.detach().cpu() - want).abs() <= 1e-5 * want.abs() + 1e-5 * scale).all())
+    g = torch.from_numpy(rng.standard_normal((n, K)).astype(np.float32))
+    got.backward(g.to(DEV))
+    grad = x.grad.cpu()
+    # entries outside the window take no part; the reference's sum / mean backward gathers into torch::empty
+    # (csrc/segment_csr.cpp:70-78, 94-111) and so defines the gradient inside the window only
+    inner = indptr - front
+    if reduce == "sum":
+        assert torch.equal(grad[front:E - back], ts_oracle.gather_csr(g, inner))
+    elif reduce == "mean":
+        assert torch.equal(grad[front:E - back], ts_oracle.segment_mean_csr_backward(g, inner, (E - front - back, K)))
+    else:
+        assert torch.equal(grad, ts_oracle.arg_backward(g, want_arg, (E, K), 0))
+
+
+@pytest.mark.parametrize("reduce", ["sum", "mean", "max"])
+def test_scatter_along_the_last_dim_of_100000_rows(ts, reduce):
+    """More leading rows than a grid dimension holds: src [100000, 16], dim = -1 (the reference's default)."""
+    import ts_oracle
+    rng = np.random.default_rng(92)
+    src = random_values(rng, (100000, 16), torch.float32, ties=reduce == "max")
+    index = torch.from_numpy(rng.integers(0, 6, size=(100000, 16)).astype(np.int64))
+    want = ts_oracle.op_scatter(src, index, -1, None, 6, reduce)
+    got = ts.scatter(src.to(DEV), index.to(DEV), -1, None, 6, reduce)
+    if reduce == "max":
+        assert torch.equal(got.cpu(), want[0])
+        arg = ts.scatter_max(src.to(DEV), index.to(DEV), -1, None, 6)[1]
+        assert torch.equal(arg.cpu(), ts_oracle.scatter(src, index, 1, None, 6, "max")[1])
+    else:
+        assert bool(((got.cpu() - want).abs() <= 1e-5 * want.abs() + 1e-5 * float(src.abs().sum(1).max())).all())
+
+
+def test_segment_csr_with_100000_leading_rows(ts):
+    import ts_oracle
+    rng = np.random.default_rng(93)
+    B, n, E, K = 100000, 2, 5, 4
+    cut = rng.integers(0, E + 1, size=B)
+    indptr = torch.from_numpy(np.stack([np.zeros(B, np.int64), cut, np.full(B, E)], 1).astype(np.int64))
+    src = random_values(rng, (B, E, K), torch.float32, ties=True)
+    got, arg = ts.segment_max_csr(src.to(DEV), indptr.to(DEV))
+    want, want_arg = ts_oracle.segment_csr(src, indptr, None, "max")
+    assert torch.equal(got.cpu(), want) and torch.equal(arg.cpu(), want_arg)
+    assert torch.equal(ts.gather_csr(got, indptr.to(DEV)).cpu(), ts_oracle.gather_csr(want, indptr))
