@@ -67,8 +67,20 @@ int64_t ts_hip_version(void);
  * indptr row is shared by all batches).
  *
  * workspace: ts_segment_csr_workspace_bytes() bytes of device scratch for the
- * partial results of rows that cross a tile boundary (may be 0 -> NULL ok).
+ * partial results of rows that cross a tile boundary.
+ *
+ * Status word: the uint64 at workspace + ts_segment_csr_workspace_bytes() -
+ * TS_STATUS_BYTES (for ts_segment_coo and ts_segment_csr_permuted: the same
+ * offset from the end of what their own *_workspace_bytes() report). Every call
+ * sets it to 0 when it starts. A row that crosses tiles is finished by the
+ * tile in which it ends, which waits (bounded) for the partial results of the
+ * tiles before it; if that wait runs out -- row pointers that are not
+ * monotone, an index that is not sorted, or a tile that did not run for
+ * seconds -- the row is written as empty (0, arg = E; left untouched with
+ * out_given) and bit 0 of the word is set. The caller may read the word after
+ * the stream has finished; 0 = every row complete.
  */
+#define TS_STATUS_BYTES 256
 size_t ts_segment_csr_workspace_bytes(int64_t B, int64_t N, int64_t E, int64_t K,
                                       int dtype, int reduce);
 int ts_segment_csr(const void *src, const int64_t *indptr, void *out,

@@ -85,6 +85,24 @@ def _dev(*ts):
             raise TsError("ts_hip: all buffers must be device (HIP) tensors")
 
 
+STATUS_BYTES = 256  # TS_STATUS_BYTES of include/ts_hip.h
+# Set (TS_CHECK_STATUS=1, as the GPU tests do): the segment wrappers below wait for the stream and raise if the
+# call's status word is not 0, i.e. if a row was given up by the look-back.
+CHECK_STATUS = os.environ.get("TS_CHECK_STATUS") == "1"
+
+
+def status_word(ws: torch.Tensor, nbytes: int) -> int:
+    """The status word of a segment reduction that used `ws` (waits for the device)."""
+    return int(ws[nbytes - STATUS_BYTES:nbytes - STATUS_BYTES + 8].view(torch.int64).item())
+
+
+def _check_status(ws, nbytes, B, N, K):
+    if CHECK_STATUS and nbytes >= STATUS_BYTES and B * N * K > 0:
+        word = status_word(ws, nbytes)
+        if word != 0:
+            raise TsError(f"ts_hip: segment reduction left status word {word}: a row was given up")
+
+
 def hip_version() -> int:
     return int(lib().ts_hip_version())
 
@@ -98,6 +116,7 @@ def segment_csr(src, indptr, out, arg_out, B, N, E, K, indptr_batch_stride, redu
         _check(L.ts_segment_csr(_p(src), _p(indptr), _p(out), _p(arg_out), _i(B), _i(N), _i(E), _i(K),
                                 _i(indptr_batch_stride), DTYPE[out.dtype], reduce, _p(ws),
                                 ctypes.c_size_t(nbytes), _stream(out)))
+    _check_status(ws, nbytes, B, N, K)
     return ws
 
 
@@ -138,6 +157,7 @@ def segment_coo(src, index, out, arg_out, count_out, B, N, E, K, index_batch_str
         _check(L.ts_segment_coo(_p(src), _p(index), _p(out), _p(arg_out), _p(count_out), _i(B), _i(N),
                                 _i(E), _i(K), _i(index_batch_stride), DTYPE[out.dtype], reduce,
                                 int(out_given), _p(ws), ctypes.c_size_t(nbytes), _stream(out)))
+    _check_status(ws, nbytes, B, N, K)
     return ws
 
 
@@ -298,4 +318,5 @@ def segment_csr_permuted(src, perm, indptr, out, arg_out, B, N, E, K, perm_batch
         _check(L.ts_segment_csr_permuted(_p(src), _p(perm), _p(indptr), _p(out), _p(arg_out), _i(B), _i(N), _i(E),
                                          _i(K), _i(perm_batch_stride), _i(indptr_batch_stride), DTYPE[out.dtype],
                                          reduce, _p(ws), ctypes.c_size_t(nbytes), _stream(out)))
+    _check_status(ws, nbytes, B, N, K)
     return ws

@@ -124,17 +124,23 @@ CsrWs csr_workspace(const CsrPlan &p, int64_t B, int64_t K, int dtype, int reduc
 
 // Workspace for either plan: buffers that are not 16-byte aligned take one element per lane,
 // which changes the tile size and with it the number of partial results.
-size_t csr_workspace_max(int64_t B, int64_t N, int64_t E, int64_t K, int dtype, int reduce) {
+// The last kStatusBytes of what the *_workspace_bytes functions report hold the call's status word.
+constexpr size_t kStatusBytes = 256;
+size_t csr_workspace_max(int64_t B, int64_t N, int64_t E, int64_t K, int dtype, int reduce, bool allow_small = true) {
   const bool wa = reduce == TS_MIN || reduce == TS_MAX;
-  const size_t w1 = csr_workspace(csr_plan(N, E, K, kElemBytes[dtype], true, false, wa), B, K, dtype, reduce).total;
-  const size_t w0 = csr_workspace(csr_plan(N, E, K, kElemBytes[dtype], false, false, wa), B, K, dtype, reduce).total;
-  return w1 > w0 ? w1 : w0;
+  const size_t w1 = csr_workspace(csr_plan(N, E, K, kElemBytes[dtype], true, false, wa, allow_small), B, K, dtype, reduce).total;
+  const size_t w0 = csr_workspace(csr_plan(N, E, K, kElemBytes[dtype], false, false, wa, allow_small), B, K, dtype, reduce).total;
+  return (w1 > w0 ? w1 : w0) + kStatusBytes;
+}
+inline unsigned long long *status_word(void *ws, size_t reported_bytes) {
+  return reinterpret_cast<unsigned long long *>(static_cast<char *>(ws) + reported_bytes - kStatusBytes);
 }
 
 int run_csr_reduce_slice(const void *src, const int64_t *indptr, void *out, int64_t *arg_out, void *count_out,
                          int64_t B, int64_t N, int64_t E, int64_t K, int64_t indptr_batch_stride, int dtype,
                          int reduce, int accumulate, void *ws, size_t ws_bytes, hipStream_t stream,
-                         const int32_t *perm, int64_t perm_batch_stride, bool want_perm_args, bool *perm_args_done) {
+                         const int32_t *perm, int64_t perm_batch_stride, bool want_perm_args, bool *perm_args_done,
+                         unsigned long long *status, bool status_reset) {
   const bool al = aligned16(src) && aligned16(out);
   // permuted rows always take the wide kernel (the narrow one stages consecutive entries)
   const CsrPlan p = csr_plan(N, E, K, kElemBytes[dtype], al, false, reduce == TS_MIN || reduce == TS_MAX,
@@ -163,6 +169,9 @@ int run_csr_reduce_slice(const void *src, const int64_t *indptr, void *out, int6
   // four words of workspace per tile give every column chunk its flag; else by the second kernel
   a.lookback = !p.small && kAccBytes[dtype] >= 4 && p.ychunks <= 4 && p.nblk > 1 && env_int("TS_CSR_LOOKBACK", 1);
   a.nonce = next_nonce();
+  a.status = status;
+  a.status_reset = status_reset ? 1 : 0;
+  a.carry_spin = env_int("TS_CSR_SPIN", kCarrySpin);  // test aid: -1 makes every look-back give up at once
   a.perm = perm;
   a.perm_batch_stride = perm_batch_stride;
   // every row is finished inside the first kernel unless the second one runs: then the positions can leave it
@@ -177,8 +186,9 @@ int run_csr_reduce_slice(const void *src, const int64_t *indptr, void *out, int6
 
 int run_csr_reduce(const void *src, const int64_t *indptr, void *out, int64_t *arg_out, void *count_out,
                    int64_t B, int64_t N, int64_t E, int64_t K, int64_t indptr_batch_stride, int dtype,
-                   int reduce, int accumulate, void *ws, size_t ws_bytes, hipStream_t stream,
-                   const int32_t *perm = nullptr, int64_t perm_batch_stride = 0, bool *perm_args_done = nullptr) {
+                   int reduce, int accumulate, void *ws, size_t ws_bytes, unsigned long long *status,
+                   hipStream_t stream, const int32_t *perm = nullptr, int64_t perm_batch_stride = 0,
+                   bool *perm_args_done = nullptr) {
   const int64_t s = kElemBytes[dtype];
   const bool want_perm_args = B * N * K >= ((int64_t)8 << 20);
   // every slice reuses the workspace: the launches follow each other on one stream
@@ -187,7 +197,7 @@ int run_csr_reduce(const void *src, const int64_t *indptr, void *out, int64_t *a
                                 offset_bytes(out, b0 * N * K * s), arg_out ? arg_out + b0 * N * K : nullptr,
                                 offset_bytes(count_out, b0 * N * s), nb, N, E, K, indptr_batch_stride, dtype, reduce,
                                 accumulate, ws, ws_bytes, stream, perm ? perm + b0 * perm_batch_stride : nullptr,
-                                perm_batch_stride, want_perm_args, perm_args_done);
+                                perm_batch_stride, want_perm_args, perm_args_done, status, b0 == 0);
   });
 }
 
@@ -262,8 +272,10 @@ int ts_segment_csr(const void *src, const int64_t *indptr, void *out, int64_t *a
   if (B * N * K == 0) return TS_OK;
   if (!indptr || !out || (E * K > 0 && !src)) return TS_ERR_BAD_ARG;
   if ((reduce == TS_MIN || reduce == TS_MAX) && !arg_out) return TS_ERR_BAD_ARG;
-  return run_csr_reduce(src, indptr, out, arg_out, nullptr, B, N, E, K, indptr_batch_stride, dtype,
-                        reduce, 0, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
+  const size_t need = csr_workspace_max(B, N, E, K, dtype, reduce);
+  if (!workspace || workspace_bytes < need) return TS_ERR_WORKSPACE;
+  return run_csr_reduce(src, indptr, out, arg_out, nullptr, B, N, E, K, indptr_batch_stride, dtype, reduce, 0,
+                        workspace, need - kStatusBytes, status_word(workspace, need), static_cast<hipStream_t>(stream));
 }
 
 int ts_gather_csr(const void *src, const int64_t *indptr, void *out, int64_t B, int64_t N, int64_t E,
@@ -339,22 +351,20 @@ int ts_segment_csr_static(const void *src, const int64_t *indptr, void *out, int
   if (!indptr || !out || (E * K > 0 && !src)) return TS_ERR_BAD_ARG;
   if ((reduce == TS_MIN || reduce == TS_MAX) && !arg_out) return TS_ERR_BAD_ARG;
   // the array is fixed in size: larger inputs must bring a workspace (ts_segment_csr)
-  if (csr_workspace_max(B, N, E, K, dtype, reduce) > kStaticScratchBytes) return TS_ERR_WORKSPACE;
+  const size_t need = csr_workspace_max(B, N, E, K, dtype, reduce);
+  if (need > kStaticScratchBytes) return TS_ERR_WORKSPACE;
   void *ws = nullptr;
   const int rc = static_scratch_ptr(&ws);
   if (rc != TS_OK) return rc;
   // Nothing in the array has to start at zero: the carry flags of a call hold that call's nonce, and
   // the second kernel only reads what the first one wrote in the same call.
   return run_csr_reduce(src, indptr, out, arg_out, nullptr, B, N, E, K, indptr_batch_stride, dtype, reduce, 0, ws,
-                        kStaticScratchBytes, static_cast<hipStream_t>(stream));
+                        need - kStatusBytes, status_word(ws, need), static_cast<hipStream_t>(stream));
 }
 
 size_t ts_segment_csr_permuted_workspace_bytes(int64_t B, int64_t N, int64_t E, int64_t K, int dtype, int reduce) {
   if (!valid_dtype(dtype) || !sizes_ok(B, N, E, K)) return 0;
-  const bool wa = reduce == TS_MIN || reduce == TS_MAX;
-  const size_t w1 = csr_workspace(csr_plan(N, E, K, kElemBytes[dtype], true, false, wa, false), B, K, dtype, reduce).total;
-  const size_t w0 = csr_workspace(csr_plan(N, E, K, kElemBytes[dtype], false, false, wa, false), B, K, dtype, reduce).total;
-  return w1 > w0 ? w1 : w0;
+  return csr_workspace_max(B, N, E, K, dtype, reduce, false);
 }
 
 int ts_segment_csr_permuted(const void *src, const int32_t *perm, const int64_t *indptr, void *out,
@@ -369,8 +379,11 @@ int ts_segment_csr_permuted(const void *src, const int32_t *perm, const int64_t 
   if ((reduce == TS_MIN || reduce == TS_MAX) && !arg_out) return TS_ERR_BAD_ARG;
   hipStream_t s = static_cast<hipStream_t>(stream);
   bool args_done = false;
+  const size_t need = csr_workspace_max(B, N, E, K, dtype, reduce, false);
+  if (!workspace || workspace_bytes < need) return TS_ERR_WORKSPACE;
   const int rc = run_csr_reduce(src, indptr, out, arg_out, nullptr, B, N, E, K, indptr_batch_stride, dtype, reduce,
-                                0, workspace, workspace_bytes, s, perm, perm_batch_stride, &args_done);
+                                0, workspace, need - kStatusBytes, status_word(workspace, need), s, perm,
+                                perm_batch_stride, &args_done);
   if (rc != TS_OK || (reduce != TS_MIN && reduce != TS_MAX) || args_done) return rc;
   return dispatch_sorted_args(dtype, out, arg_out, perm, B, N * K, E, perm_batch_stride, reduce == TS_MAX, s);
 }
@@ -390,14 +403,15 @@ int ts_segment_coo(const void *src, const int64_t *index, void *out, void *arg_o
   if (!out || (E > 0 && (!index || (K > 0 && !src)))) return TS_ERR_BAD_ARG;
   if ((reduce == TS_MIN || reduce == TS_MAX) && !arg_out) return TS_ERR_BAD_ARG;
   const size_t ptr_bytes = ((size_t)B * (N + 1) * 8 + 255) & ~(size_t)255;
-  if (!workspace || workspace_bytes < ptr_bytes) return TS_ERR_WORKSPACE;
+  const size_t need = ptr_bytes + csr_workspace_max(B, N, E, K, dtype, reduce);
+  if (!workspace || workspace_bytes < need) return TS_ERR_WORKSPACE;
   hipStream_t s = static_cast<hipStream_t>(stream);
   int64_t *ptr = static_cast<int64_t *>(workspace);
   const int rc = run_coo_to_indptr(index, ptr, B, E, N, index_batch_stride, s);
   if (rc != TS_OK) return rc;
   return run_csr_reduce(src, ptr, out, static_cast<int64_t *>(arg_out), count_out, B, N, E, K, N + 1, dtype,
                         reduce, out_given ? 1 : 0, static_cast<char *>(workspace) + ptr_bytes,
-                        workspace_bytes - ptr_bytes, s);
+                        need - ptr_bytes - kStatusBytes, status_word(workspace, need), s);
 }
 
 int ts_gather_coo(const void *src, const int64_t *index, void *out, int64_t B, int64_t N, int64_t E,

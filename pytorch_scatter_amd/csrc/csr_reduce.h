@@ -8,9 +8,15 @@
 // in registers and writes every row that starts and ends inside its range
 // straight to `out`. A row that crosses a worker boundary leaves partials in
 // LDS which the workgroup combines in edge order; a row that crosses a
-// workgroup boundary leaves partials in the global workspace, combined in tile
-// order by a small second kernel. The result is independent of scheduling: no
-// atomics, no spinning.
+// workgroup boundary leaves partials (carries) in the global workspace. The tile in
+// which such a row ends collects the carries of the tiles before it in tile order
+// (look-back, carry_* below: memory-side atomics, nonce-tagged flags, a bounded wait);
+// 8- and 16-bit accumulators, more than four column chunks and the narrow-row kernel
+// leave the combination to a small second kernel instead. Either way the order of the
+// combination is fixed by the tiling, so the result is independent of scheduling.
+// If the bounded wait runs out (row pointers that are not monotone, or a producer tile
+// that did not run for seconds) the row is written as empty (0, arg = E) and a sticky
+// status word in the workspace is set; a clean call leaves that word at 0.
 //
 // Semantics follow the reference CPU loop (csrc/cpu/segment_csr_cpu.cpp:54-88):
 // accumulate in float for 16-bit floats, strict compare so the first index
@@ -57,7 +63,13 @@ struct CsrReduceArgs {
   int64_t perm_batch_stride;
   int perm_args;      // min / max with perm: the kernel itself writes positions in src's order and applies
                       // scatter's rule for slots that never beat the initial value (no pass over arg_out after it)
+  // status word of the call (device memory, may be null): set to 0 by the first tile when status_reset is set,
+  // or-ed with kStatusGaveUp by a tile whose look-back ran out of polls
+  unsigned long long *status;
+  int status_reset;
+  int carry_spin;     // polls per batch of carry flags before the look-back gives up; < 0: give up without polling
 };
+constexpr unsigned long long kStatusGaveUp = 1;
 
 // ---- rows that cross tiles, finished without a second kernel ---------------------------------
 // The tile in which such a row ends walks back over the tiles before it. A tile whose last row is
@@ -68,12 +80,13 @@ struct CsrReduceArgs {
 // release fence per workgroup was measured and made the kernel 4x slower). The flag is written
 // after the wavefront has received the returns of its carry writes, i.e. after they were performed.
 // Tiles only ever wait for tiles with a smaller index, which the dispatcher started earlier, and
-// publishing never waits, so the walk cannot deadlock; it is bounded all the same and gives up on an
-// indptr that is not monotone. A flag holds the call's nonce, so stale workspace content never
+// publishing never waits, so the walk cannot deadlock; it is bounded all the same: when the polls run out
+// (an indptr that is not monotone never publishes what the walk waits for) the row is written as empty and
+// the call's status word is set. A flag holds the call's nonce, so stale workspace content never
 // matches, and its reader clears it, so a replay of a captured launch (same nonce, same workspace)
 // starts clean.
 constexpr uint64_t kCarryTail = 1, kCarryPass = 2;
-constexpr int kCarrySpin = 1 << 20;
+constexpr int kCarrySpin = 1 << 20;  // default of CsrReduceArgs::carry_spin
 
 template <typename A> struct CarryBits { typedef uint32_t type; };
 template <> struct CarryBits<double> { typedef uint64_t type; };
@@ -220,6 +233,8 @@ __global__ __launch_bounds__(kBlock, (csr_reduce_min_blocks<T, VEC, REDUCE, PERM
     const int64_t i = merge_search_wave(ptr, a.N, a.E, wave == 0 ? d0 : d1);
     if ((tid & (kWave - 1)) == 0) s_cut[wave] = i;
   }
+  if (a.status_reset && a.status != nullptr && tid == 0 && (blockIdx.x | blockIdx.y | blockIdx.z) == 0)
+    __hip_atomic_exchange(a.status, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   __syncthreads();
   const int64_t i0 = s_cut[0], i1 = s_cut[1];
   const int64_t j0 = d0 - i0;
@@ -404,7 +419,8 @@ __global__ __launch_bounds__(kBlock, (csr_reduce_min_blocks<T, VEC, REDUCE, PERM
   // of tiles costs a few memory round trips per batch, not per tile.
   // (start, stride): the tiles start, start - stride, ... down to first_tile; one worker walking alone takes
   // (blockIdx.x - 1, 1), the workers of a workgroup that share a long walk take every W-th tile each.
-  auto walk_back = [&](int64_t first_tile, int64_t start, int64_t stride) {
+  // false: the wait for a carry ran out; the status word is set and the caller writes the row as empty
+  auto walk_back = [&](int64_t first_tile, int64_t start, int64_t stride) -> bool {
     if constexpr (kCarryOk) {
     constexpr int PF = VEC <= 4 ? 4 : 2;
     A *vals_b = static_cast<A *>(a.ws_vals) + (b * a.nblk) * 2 * a.K;
@@ -417,8 +433,8 @@ __global__ __launch_bounds__(kBlock, (csr_reduce_min_blocks<T, VEC, REDUCE, PERM
       bool ready[PF];
 #pragma unroll
       for (int q = 0; q < PF; ++q) ready[q] = q >= n;
-      int spin = kCarrySpin;
-      while (true) {
+      int spin = a.carry_spin;
+      while (spin >= 0) {
         uint64_t f[PF];
 #pragma unroll
         for (int q = 0; q < PF; ++q)
@@ -433,7 +449,11 @@ __global__ __launch_bounds__(kBlock, (csr_reduce_min_blocks<T, VEC, REDUCE, PERM
         if (all || --spin <= 0) break;
         __builtin_amdgcn_s_sleep(4);
       }
-      if (spin <= 0) return;  // indptr not monotone: these carries will never be published
+      if (spin <= 0) {  // e.g. indptr not monotone: these carries will never be published
+        if (lg == 0 && a.status != nullptr)
+          __hip_atomic_fetch_or(a.status, kStatusGaveUp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        return false;
+      }
       asm volatile("" ::: "memory");
       A early[PF][VEC];
       int32_t early_arg[PF][VEC];
@@ -471,6 +491,7 @@ __global__ __launch_bounds__(kBlock, (csr_reduce_min_blocks<T, VEC, REDUCE, PERM
       }
     }
     }
+    return true;
   };
 
   auto absorb_head = [&](int ww) {
@@ -537,9 +558,14 @@ __global__ __launch_bounds__(kBlock, (csr_reduce_min_blocks<T, VEC, REDUCE, PERM
             for (int v = 0; v < VEC; ++v) { my_tail_val[v] = acc[v]; if (kArg) my_tail_arg[v] = arg[v]; }
             if (lg == 0) s_cut[0] = first_tile;
           } else {
-            walk_back(first_tile, (int64_t)blockIdx.x - 1, 1);
+            const bool ok = walk_back(first_tile, (int64_t)blockIdx.x - 1, 1);
+            if (!ok) {
+#pragma unroll
+              for (int v = 0; v < VEC; ++v) acc[v] = acc_init<A, REDUCE>();  // the row is written as empty
+            }
             finalize_row<T, VEC, REDUCE, ACCUM, PERM>(a, out_b, arg_b, count_b, i0 + row, col, lg, acc, arg,
-                                                      (int64_t)s_ptr[row + 1] - (int64_t)s_ptr[row], col_ok, arg_perm);
+                                                      ok ? (int64_t)s_ptr[row + 1] - (int64_t)s_ptr[row] : 0, col_ok,
+                                                      arg_perm);
           }
         } else {
           publish_carry(kCarryPass);
@@ -571,13 +597,15 @@ __global__ __launch_bounds__(kBlock, (csr_reduce_min_blocks<T, VEC, REDUCE, PERM
     if (first_tile < 0) return;
 #pragma unroll
     for (int v = 0; v < VEC; ++v) { acc[v] = acc_init<A, REDUCE>(); arg[v] = INT32_MAX; }
-    walk_back(first_tile, (int64_t)blockIdx.x - 1 - w, W);
+    const bool ok = walk_back(first_tile, (int64_t)blockIdx.x - 1 - w, W);
     A *part_val = s_val + (size_t)w * CW + lg * VEC;  // the head slots: read for the last time before the barrier
     int32_t *part_arg = s_arg + (kArg ? (size_t)w * CW + lg * VEC : 0);
 #pragma unroll
     for (int v = 0; v < VEC; ++v) { part_val[v] = acc[v]; if (kArg) part_arg[v] = arg[v]; }
+    if (!ok && lg == 0) s_head_closes[0] = -1;  // read before the first barrier for the last time; now: a walk failed
     __syncthreads();
     if (w != 0) return;
+    const bool all_ok = s_head_closes[0] != -1;
 #pragma unroll
     for (int v = 0; v < VEC; ++v) { acc[v] = my_tail_val[v]; if (kArg) arg[v] = my_tail_arg[v]; }
     for (int ww = 0; ww < W; ++ww) {
@@ -595,8 +623,13 @@ __global__ __launch_bounds__(kBlock, (csr_reduce_min_blocks<T, VEC, REDUCE, PERM
       }
     }
     const int row = s_head_row[0];
+    if (!all_ok) {
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) acc[v] = acc_init<A, REDUCE>();  // the row is written as empty
+    }
     finalize_row<T, VEC, REDUCE, ACCUM, PERM>(a, out_b, arg_b, count_b, i0 + row, col, lg, acc, arg,
-                                              (int64_t)s_ptr[row + 1] - (int64_t)s_ptr[row], col_ok, arg_perm);
+                                              all_ok ? (int64_t)s_ptr[row + 1] - (int64_t)s_ptr[row] : 0, col_ok,
+                                              arg_perm);
   }
 }
 

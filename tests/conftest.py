@@ -9,6 +9,10 @@ for p in (ROOT, os.path.join(ROOT, "oracle")):
         sys.path.insert(0, p)
 
 
+# every segment reduction that goes through pytorch_scatter_amd.capi also checks its status word
+os.environ.setdefault("TS_CHECK_STATUS", "1")
+
+
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
 

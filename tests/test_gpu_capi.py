@@ -1126,3 +1126,32 @@ def test_scatter_with_70000_batch_rows(capi, oracle, reduce):
         assert_exact(arg, want_arg)
     else:
         assert_close(out, want, float(src.abs().sum(1).max()), torch.float32)
+
+
+def test_segment_csr_status_word_reports_rows_that_were_given_up(capi, oracle, monkeypatch):
+    """The wait of the look-back is bounded. With the bound forced to "never wait" from the host (TS_CSR_SPIN=-1)
+    every row that crosses a tile is given up: the kernels still finish normally, the status word is set, those
+    rows read as empty (0, arg = E) and every other row is correct. Without the override the word stays 0
+    (checked on every call of the other tests, see conftest)."""
+    rng, indptr, index = make_csr("hub", 55, 900)
+    n, K, E = 900, 64, index.numel()
+    src = values(rng, (E, K), torch.float32, "max")
+    want, want_arg = oracle.segment_csr(src, indptr, None, "max")
+    out = torch.empty((n, K), device=DEV)
+    arg = torch.empty((n, K), dtype=torch.long, device=DEV)
+    nbytes = capi.lib().ts_segment_csr_workspace_bytes(capi._i(1), capi._i(n), capi._i(E), capi._i(K), 0, capi.MAX)
+    monkeypatch.setattr(capi, "CHECK_STATUS", False)
+    monkeypatch.setenv("TS_CSR_SPIN", "-1")
+    ws = capi.segment_csr(src.to(DEV), indptr.to(DEV), out, arg, 1, n, E, K, 0, capi.MAX)
+    assert capi.status_word(ws, nbytes) == 1
+    got, got_arg = out.cpu(), arg.cpu()
+    deg = indptr[1:] - indptr[:-1]
+    given_up = (got_arg == E).all(1) & (deg > 0)
+    assert int(given_up.sum()) >= 1 and bool((got[given_up] == 0).all())
+    assert bool((deg[given_up] >= 2).all())  # a row must have two entries to cross a tile
+    assert torch.equal(got[~given_up], want[~given_up]) and torch.equal(got_arg[~given_up], want_arg[~given_up])
+    monkeypatch.delenv("TS_CSR_SPIN")
+    ws = capi.segment_csr(src.to(DEV), indptr.to(DEV), out, arg, 1, n, E, K, 0, capi.MAX)
+    assert capi.status_word(ws, nbytes) == 0
+    assert_exact(out, want)
+    assert_exact(arg, want_arg)
