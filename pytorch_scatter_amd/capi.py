@@ -26,7 +26,7 @@ EXPORTS = (
     "ts_segment_mean_csr_backward",
     "ts_segment_coo_workspace_bytes", "ts_segment_coo", "ts_gather_coo",
     "ts_segment_mean_coo_backward",
-    "ts_scatter", "ts_scatter_workspace_bytes", "ts_scatter_with_workspace", "ts_scatter_count", "ts_divide_by_count", "ts_arg_backward",
+    "ts_scatter", "ts_scatter_workspace_bytes", "ts_scatter_workspace_zero_bytes", "ts_scatter_with_workspace", "ts_scatter_count", "ts_divide_by_count", "ts_arg_backward",
     "ts_group_softmax_workspace_bytes", "ts_group_softmax", "ts_group_softmax_backward",
     "ts_group_logsumexp", "ts_group_logsumexp_backward",
     "ts_group_std", "ts_group_std_backward",
@@ -57,6 +57,7 @@ def lib() -> ctypes.CDLL:
         _lib.ts_group_softmax_workspace_bytes.restype = ctypes.c_size_t
         _lib.ts_indptr_to_index_workspace_bytes.restype = ctypes.c_size_t
         _lib.ts_scatter_workspace_bytes.restype = ctypes.c_size_t
+        _lib.ts_scatter_workspace_zero_bytes.restype = ctypes.c_size_t
         _lib.ts_sort_index_workspace_bytes.restype = ctypes.c_size_t
         _lib.ts_segment_csr_permuted_workspace_bytes.restype = ctypes.c_size_t
     return _lib
@@ -184,11 +185,14 @@ def scatter(src, index, out, arg_out, B, E, K, N, sb, se, sk, reduce: int, out_g
                                 _stream(out)))
 
 
-def scatter_with_workspace(src, index, out, arg_out, B, E, K, N, sb, se, sk, reduce: int, out_given: bool):
+def scatter_with_workspace(src, index, out, arg_out, B, E, K, N, sb, se, sk, reduce: int, out_given: bool, ws=None):
     _dev(src, index, out, arg_out)
     L = lib()
     nbytes = L.ts_scatter_workspace_bytes(_i(B), _i(E), _i(K), _i(N), DTYPE[out.dtype], reduce)
-    ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=out.device)
+    nzero = L.ts_scatter_workspace_zero_bytes(_i(B), _i(E), _i(K), _i(N), DTYPE[out.dtype], reduce)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=out.device)
+        ws[:nzero].zero_()  # the part that has to read as zero; the call leaves it zero for the next one
     with torch.cuda.device(out.device):
         _check(L.ts_scatter_with_workspace(_p(src), _p(index), _p(out), _p(arg_out), _i(B), _i(E), _i(K), _i(N),
                                            _i(sb), _i(se), _i(sk), DTYPE[out.dtype], reduce, int(out_given),

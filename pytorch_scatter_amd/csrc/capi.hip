@@ -461,6 +461,10 @@ size_t ts_scatter_workspace_bytes(int64_t B, int64_t E, int64_t K, int64_t N, in
   const bool any_size = env_int("TS_SCATTER_BINNED", 1) == 2;
   if (reduce == TS_MIN || reduce == TS_MAX) {
     if (kElemBytes[dtype] > 4) return 0;  // 64-bit elements do not use packed keys
+    if (env_int("TS_SCATTER_LDS_K1", 1) && env_int("TS_SCATTER_LDS", 1)) {
+      const size_t k1 = k1_plan(B, E, K, N, kElemBytes[dtype], nullptr, 0, env_int("TS_SCATTER_LDS", 1) == 2).bytes;
+      if (k1 != 0) return k1;
+    }
     const size_t binned = bin_plan(B, E, K, N, kElemBytes[dtype], nullptr, 0, any_size).bytes;
     if (binned != 0) return binned;
     // one flag for the sample of the index that picks the kernel when few entries meet in an output row
@@ -470,6 +474,13 @@ size_t ts_scatter_workspace_bytes(int64_t B, int64_t E, int64_t K, int64_t N, in
   if (reduce == TS_SUM && kAccBytes[dtype] >= 4)  // table slots: int32 for int32, 8 bytes for the other types
     return bin_plan(B, E, K, N, kElemBytes[dtype], nullptr, 0, any_size, dtype == TS_I32 ? 4 : 8).bytes;
   return 0;
+}
+
+size_t ts_scatter_workspace_zero_bytes(int64_t B, int64_t E, int64_t K, int64_t N, int dtype, int reduce) {
+  if (!valid_dtype(dtype) || !sizes_ok(B, N, E, K)) return 0;
+  if ((reduce != TS_MIN && reduce != TS_MAX) || kElemBytes[dtype] > 4) return 0;
+  if (!env_int("TS_SCATTER_LDS_K1", 1) || !env_int("TS_SCATTER_LDS", 1)) return 0;
+  return k1_plan(B, E, K, N, kElemBytes[dtype], nullptr, 0, env_int("TS_SCATTER_LDS", 1) == 2).zero_bytes;
 }
 
 int ts_scatter(const void *src, const int64_t *index, void *out, int64_t *arg_out, int64_t B, int64_t E,

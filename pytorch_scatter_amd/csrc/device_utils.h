@@ -123,6 +123,16 @@ template <typename A, int REDUCE> __device__ __forceinline__ A acc_init() {
   return (A)0;
 }
 
+// A read of a 32-bit word of LDS that may change under the reader (tags, the value half of a packed key): not
+// kept in a register across uses, and not a `volatile` access, which the compiler leaves in the generic address
+// space (a flat load) and follows with a wait for every load the wavefront has in flight.
+__device__ __forceinline__ uint32_t lds_peek(const uint32_t *p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+}
+__device__ __forceinline__ int32_t lds_peek(const int32_t *p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+}
+
 // ---- 16-byte vectors of VEC elements
 template <typename T, int VEC> struct alignas(sizeof(T) * VEC) Vec { T v[VEC]; };
 

@@ -1063,10 +1063,10 @@ __global__ __launch_bounds__(kLdsBlock, (TAGS <= 256 ? 4 : 1)) void scatter_key_
             uint64_t *p = &s_keys[row * K + k0];
             // cheap filter on the value half only (one 32-bit LDS read per element): an entry whose
             // value key is below the cached one cannot win; ties and improvements take the 64-bit atomic
-            const volatile uint32_t *hi = reinterpret_cast<const volatile uint32_t *>(p) + 1;
+            const uint32_t *hi = reinterpret_cast<const uint32_t *>(p) + 1;
 #pragma unroll
             for (int v = 0; v < VEC; ++v)
-              if ((uint32_t)(key[u][v] >> 32) >= hi[2 * v] && key[u][v] != 0)
+              if ((uint32_t)(key[u][v] >> 32) >= lds_peek(hi + 2 * v) && key[u][v] != 0)
                 __hip_atomic_fetch_max(p + v, key[u][v], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
           } else {
             miss_node[u] = node;
@@ -1232,7 +1232,7 @@ __global__ __launch_bounds__(kLdsBlockK1) void scatter_key_lds_k1_kernel(Scatter
       }
       if (tag == node[u]) {
         // value half first (one 32-bit LDS read): an entry below the cached value cannot win
-        const uint32_t cur_hi = reinterpret_cast<const volatile uint32_t *>(&s_keys[row])[1];
+        const uint32_t cur_hi = lds_peek(reinterpret_cast<const uint32_t *>(&s_keys[row]) + 1);
         if ((uint32_t)(key[u] >> 32) >= cur_hi)
           __hip_atomic_fetch_max(&s_keys[row], key[u], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
       } else {
@@ -1417,6 +1417,7 @@ __global__ __launch_bounds__(kBlock) void scatter_arg_wide_kernel(ScatterArgs a)
 
 }  // namespace ts
 #include "scatter_binned.h"
+#include "scatter_k1.h"
 namespace ts {
 
 // ---- elementwise helpers --------------------------------------------------------
@@ -1622,6 +1623,21 @@ int launch_scatter_v(const ScatterArgs &args, int reduce, hipStream_t stream) {
       const int64_t epb = lds_chunk_edges(a.lds_epb, a.K, n_edges);
       const unsigned g_lds = (unsigned)((n_edges + epb - 1) / epb);
       const unsigned g_key = scatter_grid(n_edges, a.K / VEC, kBlock, 4);
+      if constexpr (sizeof(T) == 4) {
+        // one value per entry, a workspace whose key table reads as zero: per-workgroup tables handed over in slabs
+        // instead of atomics, misses filtered by a pipelined read (scatter_k1.h)
+        if (a.lds_cache && a.lds_k1 && !a.out_given && a.K == 1 && a.B == 1 && a.se == 1 && a.bin_ws != nullptr &&
+            ((reinterpret_cast<uintptr_t>(a.src) | reinterpret_cast<uintptr_t>(a.index)) & 15) == 0) {
+          const K1Plan kp = k1_plan(a.B, a.E, a.K, a.N, (int)sizeof(T), a.bin_ws, a.bin_ws_bytes, a.lds_cache == 2);
+          if (kp.ok) {
+            if (is_max)
+              launch_scatter_k1<T, true>(a, kp, stream);
+            else
+              launch_scatter_k1<T, false>(a, kp, stream);
+            return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
+          }
+        }
+      }
       if ((a.lds_cache || a.bin_any_size) && a.sk == 0 && a.B * a.N < 0x7FFFFFFFll && a.bin_ws != nullptr &&
           a.K % VEC == 0 && n_src > 0) {
         // large inputs of wide rows with a workspace: entries binned by bucket of output rows, no table misses.

@@ -374,10 +374,10 @@ __global__ __launch_bounds__(kBinBlock) void bin_reduce_kernel(ScatterArgs a, Bi
         make_keys<T, VEC, IS_MAX>(x[u], e, key);
         uint64_t *row = &s_keys[(int)(ent[u] >> 32) * KP + k0];
         // filter on the value half (one 32-bit LDS read per element): below the cached key cannot win
-        const volatile uint32_t *hi32 = reinterpret_cast<const volatile uint32_t *>(row) + 1;
+        const uint32_t *hi32 = reinterpret_cast<const uint32_t *>(row) + 1;
 #pragma unroll
         for (int v = 0; v < VEC; ++v)
-          if (key[v] != 0 && (uint32_t)(key[v] >> 32) >= hi32[2 * v])
+          if (key[v] != 0 && (uint32_t)(key[v] >> 32) >= lds_peek(hi32 + 2 * v))
             __hip_atomic_fetch_max(row + v, key[v], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
       }
     }
@@ -438,10 +438,10 @@ __global__ __launch_bounds__(kBinBlock) void bin_reduce_wave_kernel(ScatterArgs 
           uint64_t key[VEC];
           make_keys<T, VEC, IS_MAX>(x[u], e, key);
           uint64_t *row = &s_keys[(int)e_row[u] * KP + k0];
-          const volatile uint32_t *hi32 = reinterpret_cast<const volatile uint32_t *>(row) + 1;
+          const uint32_t *hi32 = reinterpret_cast<const uint32_t *>(row) + 1;
 #pragma unroll
           for (int v = 0; v < VEC; ++v)
-            if (key[v] != 0 && (uint32_t)(key[v] >> 32) >= hi32[2 * v])
+            if (key[v] != 0 && (uint32_t)(key[v] >> 32) >= lds_peek(hi32 + 2 * v))
               __hip_atomic_fetch_max(row + v, key[v], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
         }
       }

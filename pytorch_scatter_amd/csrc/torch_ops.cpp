@@ -11,6 +11,9 @@
 #include <c10/core/DeviceGuard.h>
 #include <c10/hip/HIPStream.h>
 
+#include <map>
+#include <mutex>
+
 #include "../../include/ts_hip.h"
 
 namespace {
@@ -94,6 +97,35 @@ Tensor workspace(size_t bytes, const Tensor &like) {
   return at::empty({static_cast<int64_t>(bytes > 0 ? bytes : 1)}, like.options().dtype(at::kByte));
 }
 
+// A workspace whose first `zero_bytes` bytes must read as zero when a call starts and are left zero by it
+// (ts_scatter_workspace_zero_bytes): kept from call to call, one per device and stream, cleared when allocated.
+struct KeptWorkspaces {
+  std::mutex mu;
+  std::map<std::pair<int, void *>, Tensor> kept;
+};
+KeptWorkspaces &kept_workspaces() {
+  static KeptWorkspaces *k = new KeptWorkspaces();  // never destroyed: no frees after the runtime has shut down
+  return *k;
+}
+Tensor kept_workspace(size_t bytes, size_t zero_bytes, const Tensor &like, void *stream) {
+  KeptWorkspaces &k = kept_workspaces();
+  std::lock_guard<std::mutex> lock(k.mu);
+  const auto key = std::make_pair((int)like.get_device(), stream);
+  auto it = k.kept.find(key);
+  if (it == k.kept.end() || it->second.numel() < (int64_t)bytes) {
+    Tensor t = workspace(bytes, like);
+    t.narrow(0, 0, (int64_t)zero_bytes).zero_();
+    k.kept[key] = t;
+    return t;
+  }
+  return it->second;
+}
+void drop_kept_workspace(const Tensor &like, void *stream) {  // after a failed call its content is unknown
+  KeptWorkspaces &k = kept_workspaces();
+  std::lock_guard<std::mutex> lock(k.mu);
+  k.kept.erase(std::make_pair((int)like.get_device(), stream));
+}
+
 // csrc/scatter.cpp:25-33
 Tensor broadcast(Tensor src, const Tensor &other, int64_t dim) {
   if (src.dim() == 1)
@@ -175,14 +207,19 @@ std::tuple<Tensor, OptTensor> scatter_hip(Tensor src, Tensor index, int64_t dim,
   }
   // min / max of large inputs with wide rows can use scratch memory (entries binned by bucket of output rows)
   const size_t ws_bytes = sk.value() == 0 ? ts_scatter_workspace_bytes(B, E, K, N, dtype_code(src), reduce) : 0;
+  const size_t ws_zero = ws_bytes > 0 ? ts_scatter_workspace_zero_bytes(B, E, K, N, dtype_code(src), reduce) : 0;
   Tensor ws;
-  if (ws_bytes > 0) ws = workspace(ws_bytes, src);
-  check_status(ts_scatter_with_workspace(src.data_ptr(), index.data_ptr<int64_t>(), out.data_ptr(),
-                                         minmax ? arg_out.value().data_ptr<int64_t>() : nullptr, B, E, K, N,
-                                         sb.value(), se, sk.value(), dtype_code(src), reduce,
-                                         optional_out.has_value() ? 1 : 0, ws_bytes > 0 ? ws.data_ptr() : nullptr,
-                                         ws_bytes, stream_of(src)),
-               "scatter");
+  if (ws_zero > 0)
+    ws = kept_workspace(ws_bytes, ws_zero, src, stream_of(src));
+  else if (ws_bytes > 0)
+    ws = workspace(ws_bytes, src);
+  const int rc = ts_scatter_with_workspace(src.data_ptr(), index.data_ptr<int64_t>(), out.data_ptr(),
+                                           minmax ? arg_out.value().data_ptr<int64_t>() : nullptr, B, E, K, N,
+                                           sb.value(), se, sk.value(), dtype_code(src), reduce,
+                                           optional_out.has_value() ? 1 : 0, ws_bytes > 0 ? ws.data_ptr() : nullptr,
+                                           ws_bytes, stream_of(src));
+  if (rc != TS_OK && ws_zero > 0) drop_kept_workspace(src, stream_of(src));
+  check_status(rc, "scatter");
   return std::make_tuple(out, arg_out);
 }
 

@@ -1155,3 +1155,62 @@ def test_segment_csr_status_word_reports_rows_that_were_given_up(capi, oracle, m
     assert capi.status_word(ws, nbytes) == 0
     assert_exact(out, want)
     assert_exact(arg, want_arg)
+
+
+K1_CASES = [
+    # E, N, index: one value per entry through the workspace path (per-workgroup tables handed over in slabs)
+    (30001, 500, "zipf"), (50003, 20000, "zipf"), (20002, 300000, "uniform"), (9000, 7, "zipf"),
+    (40000, 9000, "uniform"), (3, 10, "uniform"), (70000, 100000, "zipf"),
+]
+
+
+@pytest.mark.parametrize("case,reduce,dtype", product(K1_CASES, ["min", "max"], [torch.float32, torch.int32]))
+def test_scatter_minmax_one_value_per_entry_with_workspace(capi, oracle, case, reduce, dtype, monkeypatch):
+    """Forced on at a small size. Heavy ties, NaN / infinite / lowest() values, indices outside [0, N), a number of
+    entries that is no multiple of four, output rows that share a table row (N > 8192), a uniform index (every
+    entry misses the table and goes through the queue). The same workspace serves two calls in a row: the key
+    table in its first bytes has to come back as zeros."""
+    monkeypatch.setenv("TS_SCATTER_LDS", "2")
+    E, N, kind = case
+    rng = np.random.default_rng(E + N)
+    src = random_values(rng, (1, E, 1), dtype, ties=True)
+    if kind == "zipf":
+        p = np.arange(1, N + 1, dtype=np.float64) ** -1.2
+        index = rng.choice(N, size=E, p=p / p.sum())
+        index = (index * 7919) % N  # hot rows spread over the id space
+    else:
+        index = rng.integers(0, N, size=E)
+    index = torch.from_numpy(index.astype(np.int64))
+    if E > 100:
+        index[5] = -1
+        index[77] = N
+        if dtype.is_floating_point:
+            src[0, 11, 0] = float("nan")
+            src[0, 13, 0] = float("-inf") if reduce == "max" else float("inf")
+            lim = torch.finfo(dtype).min if reduce == "max" else torch.finfo(dtype).max
+        else:
+            lim = torch.iinfo(dtype).min if reduce == "max" else torch.iinfo(dtype).max
+        src[0, 17, 0] = lim  # does not beat the initial value: counts as no entry
+        index[17] = N - 1
+        index[index == N - 1] = N - 1
+    valid = (index >= 0) & (index < N)
+    want, want_arg = oracle.scatter(src[:, valid], index[valid].view(1, -1, 1), 1, None, N, reduce)
+    # positions of the oracle are those of the filtered input: map them back
+    pos = torch.nonzero(valid).flatten()
+    keep = want_arg < pos.numel()
+    want_arg = torch.where(keep, pos[want_arg.clamp(max=max(pos.numel() - 1, 0))], torch.full_like(want_arg, E))
+    nbytes = capi.lib().ts_scatter_workspace_bytes(capi._i(1), capi._i(E), capi._i(1), capi._i(N), capi.DTYPE[dtype],
+                                                  capi.REDUCE[reduce])
+    nzero = capi.lib().ts_scatter_workspace_zero_bytes(capi._i(1), capi._i(E), capi._i(1), capi._i(N),
+                                                      capi.DTYPE[dtype], capi.REDUCE[reduce])
+    assert nbytes > nzero >= N * 8
+    ws = None
+    for rep in range(2):
+        out = torch.full((1, N, 1), 5, dtype=dtype, device=DEV)
+        arg = torch.full((1, N, 1), -3, dtype=torch.long, device=DEV)
+        ws = capi.scatter_with_workspace(src.to(DEV), index.to(DEV), out, arg, 1, E, 1, N, 0, 1, 0,
+                                         capi.REDUCE[reduce], False, ws)
+        torch.cuda.synchronize()
+        assert_exact(out, want, f"values rep={rep}")
+        assert_exact(arg, want_arg, f"arg rep={rep}")
+        assert bool((ws[:nzero] == 0).all()), "the key table is handed back as zeros"
