@@ -465,7 +465,7 @@ size_t ts_scatter_workspace_bytes(int64_t B, int64_t E, int64_t K, int64_t N, in
       const size_t k1 = k1_plan(B, E, K, N, kElemBytes[dtype], nullptr, 0, env_int("TS_SCATTER_LDS", 1) == 2).bytes;
       if (k1 != 0) return k1;
     }
-    const size_t binned = bin_plan(B, E, K, N, kElemBytes[dtype], nullptr, 0, any_size).bytes;
+    const size_t binned = bin_plan(B, E, K, N, kElemBytes[dtype], nullptr, 0, any_size, 8, true).bytes;
     if (binned != 0) return binned;
     // one flag for the sample of the index that picks the kernel when few entries meet in an output row
     const int probe = env_int("TS_SCATTER_SKEW", 1);

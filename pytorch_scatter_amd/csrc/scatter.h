@@ -1643,17 +1643,13 @@ int launch_scatter_v(const ScatterArgs &args, int reduce, hipStream_t stream) {
         // large inputs of wide rows with a workspace: entries binned by bucket of output rows, no table misses.
         // Also for an index with few entries per output row (10 M entries onto 1 M rows, uniform / Zipf(1.2) /
         // sorted index: K = 16 894 / 784 / 537 -> 565 / 452 / 357 us, K = 32 1618 / 1169 / 662 -> 757 / 645 / 614 us)
-        const BinPlan bp = bin_plan(a.B, a.E, a.K, a.N, (int)sizeof(T), a.bin_ws, a.bin_ws_bytes, a.bin_any_size != 0);
+        const BinPlan bp = bin_plan(a.B, a.E, a.K, a.N, (int)sizeof(T), a.bin_ws, a.bin_ws_bytes, a.bin_any_size != 0, 8,
+                                    true);
         if (bp.ok) {
-          if (is_max) {
-            hipLaunchKernelGGL((scatter_key_init_kernel<T, true>), dim3(g_out), dim3(kBlock), 0, stream, a);
+          if (is_max)
             launch_binned_keys<T, VEC, true>(a, bp.p, stream);
-            hipLaunchKernelGGL((scatter_key_final_kernel<T, true>), dim3(g_out), dim3(kBlock), 0, stream, a);
-          } else {
-            hipLaunchKernelGGL((scatter_key_init_kernel<T, false>), dim3(g_out), dim3(kBlock), 0, stream, a);
+          else
             launch_binned_keys<T, VEC, false>(a, bp.p, stream);
-            hipLaunchKernelGGL((scatter_key_final_kernel<T, false>), dim3(g_out), dim3(kBlock), 0, stream, a);
-          }
           return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
         }
       }

@@ -38,6 +38,11 @@ struct BinArgs {
   int32_t *wg_bucket;      // [max_wgs] bucket of a reducing workgroup, -1: none
   int32_t *wg_hist;        // [n_place][nb]
   uint64_t *binned;        // [B * E] (row in bucket << 32) | entry number
+  int32_t *slab_start;     // min / max: [nb + 1] first slab of a bucket that is reduced in more than one chunk
+  uint64_t *slabs;         // min / max: [slab][K << rshift] the tables of those chunks
+  int32_t *comb_list;      // min / max: buckets that the combining kernel finishes (not exactly one chunk), then
+  int32_t *comb_count;     //            how many
+
   int *unsorted;           // sum only (else null): set to 1 by the count pass when the index is not sorted;
                            // a sorted index is left to the kernels that combine runs, and the passes after
                            // the count return at once
@@ -53,7 +58,7 @@ struct BinPlan {
 
 // slot_bytes: size of a table slot (8: packed keys of min / max, 4 or 8: accumulators of a sum)
 inline BinPlan bin_plan(int64_t B, int64_t E, int64_t K, int64_t N, int elem_bytes, void *ws, size_t ws_bytes,
-                        bool any_size = false, int slot_bytes = 8) {
+                        bool any_size = false, int slot_bytes = 8, bool slabs = false) {
   BinPlan r;
   r.ok = false;
   r.bytes = 0;
@@ -77,6 +82,7 @@ inline BinPlan bin_plan(int64_t B, int64_t E, int64_t K, int64_t N, int elem_byt
   // 8 K entries take it about 200 us whatever the input, which is fine once there are a few workgroups per CU
   // (4 M entries and more) and far too long for a smaller input. Those get shorter chunks: about 512 workgroups.
   int64_t chunk = kBinChunk;
+  if (const char *env = getenv("TS_BIN_CHUNK")) chunk = atoi(env);  // tuning aid
   if (n_edges < (int64_t)512 * kBinChunk) {
     chunk = (n_edges / 512 + 63) & ~(int64_t)63;
     if (chunk < 1024) chunk = 1024;
@@ -89,6 +95,10 @@ inline BinPlan bin_plan(int64_t B, int64_t E, int64_t K, int64_t N, int elem_byt
   const size_t o_tot = take((size_t)nb * 8), o_cur = take((size_t)nb * 8), o_st = take((size_t)(nb + 1) * 8);
   const size_t o_cs = take((size_t)(nb + 1) * 4), o_wb = take((size_t)p.max_wgs * 4);
   const size_t o_wh = take((size_t)p.n_place * nb * 4), o_bin = take((size_t)n_edges * 8), o_flag = take(256);
+  // A bucket with m >= 2 chunks holds more than (m - 1) * chunk entries: at most 2 * n_edges / chunk slabs in all.
+  const int64_t n_slabs = slabs ? 2 * (n_edges / chunk) + 2 : 0;
+  const size_t o_ss = take(slabs ? (size_t)(nb + 1) * 4 : 0), o_cl = take(slabs ? (size_t)(nb + 1) * 4 : 0);
+  const size_t o_sl = take((size_t)n_slabs * ((size_t)K << rshift) * 8);
   r.bytes = off;
   if (ws == nullptr || ws_bytes < off || (reinterpret_cast<uintptr_t>(ws) & 15) != 0) return r;
   char *base = static_cast<char *>(ws);
@@ -100,6 +110,10 @@ inline BinPlan bin_plan(int64_t B, int64_t E, int64_t K, int64_t N, int elem_byt
   p.wg_hist = reinterpret_cast<int32_t *>(base + o_wh);
   p.binned = reinterpret_cast<uint64_t *>(base + o_bin);
   p.unsorted = reinterpret_cast<int *>(base + o_flag);  // callers that do not want the check set it to null
+  p.slab_start = slabs ? reinterpret_cast<int32_t *>(base + o_ss) : nullptr;
+  p.comb_list = slabs ? reinterpret_cast<int32_t *>(base + o_cl) : nullptr;
+  p.comb_count = slabs ? p.comb_list + nb : nullptr;
+  p.slabs = slabs ? reinterpret_cast<uint64_t *>(base + o_sl) : nullptr;
   r.ok = true;
   return r;
 }
@@ -230,29 +244,45 @@ static __global__ __launch_bounds__(kBinBlock) void bin_scan_kernel(BinArgs p) {
   constexpr int PER = kBinMaxBuckets / kBinBlock;
   __shared__ int64_t s_t[kBinBlock];
   __shared__ int64_t s_c[kBinBlock];
+  __shared__ int32_t s_m[kBinBlock];  // slabs: chunks of buckets with more than one
+  __shared__ int32_t s_l[kBinBlock];  // buckets for the combining kernel: those without exactly one chunk
   if (p.sampled && *p.unsorted == 0) return;
-  int64_t t[PER], c[PER], sum_t = 0, sum_c = 0;
+  // a bucket holds fewer than 2^32 entries (the plan refuses larger inputs): 32-bit counts and divisions
+  uint32_t t[PER], c[PER];
+  int64_t sum_t = 0, sum_c = 0;
+  int32_t sum_m = 0, sum_l = 0;
 #pragma unroll
   for (int j = 0; j < PER; ++j) {
     const int i = threadIdx.x * PER + j;
-    t[j] = i < p.nb ? (int64_t)p.totals[i] : 0;
-    c[j] = (t[j] + p.chunk - 1) / p.chunk;
+    t[j] = i < p.nb ? (uint32_t)p.totals[i] : 0u;
+    c[j] = t[j] / (uint32_t)p.chunk + (t[j] % (uint32_t)p.chunk != 0 ? 1u : 0u);
     sum_t += t[j];
     sum_c += c[j];
+    sum_m += c[j] > 1 ? (int32_t)c[j] : 0;
+    sum_l += (i < p.nb && c[j] != 1) ? 1 : 0;
   }
   s_t[threadIdx.x] = sum_t;
   s_c[threadIdx.x] = sum_c;
+  s_m[threadIdx.x] = sum_m;
+  s_l[threadIdx.x] = sum_l;
   __syncthreads();
   for (int d = 1; d < kBinBlock; d <<= 1) {  // inclusive scan over the threads
     int64_t vt = 0, vc = 0;
-    if ((int)threadIdx.x >= d) { vt = s_t[threadIdx.x - d]; vc = s_c[threadIdx.x - d]; }
+    int32_t vm = 0, vl = 0;
+    if ((int)threadIdx.x >= d) {
+      vt = s_t[threadIdx.x - d]; vc = s_c[threadIdx.x - d]; vm = s_m[threadIdx.x - d]; vl = s_l[threadIdx.x - d];
+    }
     __syncthreads();
     s_t[threadIdx.x] += vt;
     s_c[threadIdx.x] += vc;
+    s_m[threadIdx.x] += vm;
+    s_l[threadIdx.x] += vl;
     __syncthreads();
   }
   int64_t run_t = s_t[threadIdx.x] - sum_t, run_c = s_c[threadIdx.x] - sum_c;
+  int32_t run_m = s_m[threadIdx.x] - sum_m, run_l = s_l[threadIdx.x] - sum_l;
   const int64_t all_c = s_c[kBinBlock - 1];
+  if (p.comb_count != nullptr && threadIdx.x == 0) *p.comb_count = s_l[kBinBlock - 1];
 #pragma unroll
   for (int j = 0; j < PER; ++j) {
     const int i = threadIdx.x * PER + j;
@@ -260,10 +290,16 @@ static __global__ __launch_bounds__(kBinBlock) void bin_scan_kernel(BinArgs p) {
       p.starts[i] = run_t;
       p.cursor[i] = (unsigned long long)run_t;
       p.chunk_start[i] = (int32_t)run_c;
+      if (p.slab_start != nullptr) {
+        p.slab_start[i] = run_m;
+        if (c[j] != 1) p.comb_list[run_l] = i;
+      }
     }
     if (i == p.nb) { p.starts[i] = run_t; p.chunk_start[i] = (int32_t)run_c; }
     run_t += t[j];
     run_c += c[j];
+    run_m += c[j] > 1 ? (int32_t)c[j] : 0;
+    run_l += (i < p.nb && c[j] != 1) ? 1 : 0;
   }
   if (threadIdx.x == kBinBlock - 1 && p.nb == kBinMaxBuckets) {
     p.starts[p.nb] = run_t;
@@ -311,26 +347,103 @@ static __global__ __launch_bounds__(kBinPlaceBlock) void bin_place_kernel(Scatte
   }
 }
 
-// The table of one chunk (rows K + 1 keys apart) -> the table in memory: a read first, an atomic only for a key
-// that improves on what is there.
+// One finished packed key -> out / arg_out (element i of [B, N, K]): what scatter_key_init_kernel and
+// scatter_key_final_kernel do for the kernels that keep their keys in arg_out. key == 0: no entry.
+template <typename T, bool IS_MAX>
+__device__ __forceinline__ void bin_emit(const ScatterArgs &a, int64_t i, uint64_t key) {
+  T *out = static_cast<T *>(a.out);
+  const uint32_t kv = (uint32_t)(key >> 32);
+  bool has = key != 0;
+  if (a.out_given) {
+    // an entry has to beat the previous content strictly; a NaN in out is never beaten
+    const T prev = out[i];
+    uint32_t pk = Key<T>::enc(prev);
+    if (!IS_MAX) pk = ~pk;
+    has = has && !Key<T>::is_nan(prev) && kv > pk;
+    if (!has) {
+      a.arg_out[i] = a.E;
+      return;
+    }
+  } else {
+    // a value that does not beat the initial value of the reduction counts as no entry
+    uint32_t lim = Key<T>::enc(IS_MAX ? ElemLim<T>::lowest() : ElemLim<T>::max());
+    if (!IS_MAX) lim = ~lim;
+    has = has && kv > lim;
+    if (!has) {
+      out[i] = zero_elem<T>();
+      a.arg_out[i] = a.E;
+      return;
+    }
+  }
+  const int64_t e = (int64_t)(0xFFFFFFFEu - (uint32_t)key);
+  const uint32_t k = IS_MAX ? kv : ~kv;
+  T val = Key<T>::dec(k);
+  if (Key<T>::kFloat && k == 0x80000000u) {
+    // a zero: fetch it from src to keep the sign bit of the winning entry
+    const int64_t bn = i / a.K;
+    val = static_cast<const T *>(a.src)[((bn / a.N) * a.E + e) * a.K + (i - bn * a.K)];
+  }
+  out[i] = val;
+  a.arg_out[i] = e;
+}
+
+// The table of one chunk (rows K + 1 keys apart) leaves the workgroup without atomics: a bucket that is
+// reduced in one chunk goes straight to out / arg_out; the chunks of a larger bucket store their tables in
+// slabs of the workspace, which bin_combine_kernel puts together. (Writing the tables into one table of keys
+// in memory with a read and an atomic per key took 56 of 300 us for 10 M entries of 32 floats: 13 M atomics,
+// most of them on the 8192 keys of the bucket that holds the hubs.)
+template <typename T, bool IS_MAX>
 __device__ __forceinline__ void bin_flush_keys(const ScatterArgs &a, const BinArgs &p, int bucket,
                                                const uint64_t *s_keys) {
   const int K = (int)a.K;
-  uint64_t *gkeys = reinterpret_cast<uint64_t *>(a.arg_out) + ((int64_t)bucket << p.rshift) * a.K;
-  const int64_t limit = (a.B * a.N - ((int64_t)bucket << p.rshift)) * a.K;  // keys of rows that exist
+  const int64_t first = ((int64_t)bucket << p.rshift) * a.K;   // first element of the bucket in [B * N, K]
+  const int64_t limit = a.B * a.N * a.K - first;                // elements of rows that exist
   const int table = K << p.rshift;
-  for (int i0 = threadIdx.x; i0 < table; i0 += kBinBlock * 4) {
-    uint64_t key[4], cur[4];
+  const int chunks = p.chunk_start[bucket + 1] - p.chunk_start[bucket];
+  if (chunks == 1) {
+    for (int i = threadIdx.x; i < table && i < limit; i += kBinBlock) bin_emit<T, IS_MAX>(a, first + i, s_keys[i + i / K]);
+  } else {
+    uint64_t *slab = p.slabs + ((int64_t)p.slab_start[bucket] + ((int64_t)blockIdx.x - p.chunk_start[bucket])) * table;
+    for (int i = threadIdx.x; i < table; i += kBinBlock) slab[i] = s_keys[i + i / K];  // row i / K starts i / K keys later
+  }
+}
+
+// Buckets that were not reduced in exactly one chunk: the maximum over the slabs of their chunks (none: a bucket
+// without entries), element by element, to out / arg_out. A workgroup takes kCombPos neighbouring keys of one
+// bucket; its wavefronts share the slabs, sixteen loads in flight each, and meet in LDS.
+constexpr int kCombPos = 64;
+template <typename T, bool IS_MAX>
+__global__ __launch_bounds__(kBinBlock) void bin_combine_kernel(ScatterArgs a, BinArgs p) {
+  constexpr int W = kBinBlock / kWave;
+  __shared__ uint64_t s_part[W][kCombPos];
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  const int table = (int)a.K << p.rshift;
+  const int parts = (table + kCombPos - 1) / kCombPos;
+  const int n_list = *p.comb_count;
+  for (int64_t item = blockIdx.x; item < (int64_t)n_list * parts; item += gridDim.x) {
+    const int bucket = p.comb_list[item / parts];
+    const int pos = (int)(item % parts) * kCombPos + lane;
+    const int c0 = p.slab_start[bucket];
+    const int m = p.chunk_start[bucket + 1] - p.chunk_start[bucket];
+    const uint64_t *slab = p.slabs + (int64_t)c0 * table + (pos < table ? pos : 0);
+    uint64_t best = 0;
+    constexpr int U = 16;  // loads in flight per lane: the slabs of a bucket with a thousand chunks in four round trips
+    for (int s0 = wave; s0 < m; s0 += W * U) {
+      uint64_t k[U];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int i = i0 + j * kBinBlock;
-      key[j] = (i < table && i < limit) ? s_keys[i + i / K] : 0;  // row i / K starts i / K keys later
-      if (key[j] != 0) cur[j] = gkeys[i];
+      for (int u = 0; u < U; ++u) k[u] = slab[(int64_t)(s0 + u * W < m ? s0 + u * W : s0) * table];
+#pragma unroll
+      for (int u = 0; u < U; ++u) best = k[u] > best ? k[u] : best;
     }
+    s_part[wave][lane] = best;
+    __syncthreads();
+    if (wave == 0) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
-      if (key[j] != 0 && key[j] > cur[j])
-        __hip_atomic_fetch_max(gkeys + i0 + j * kBinBlock, key[j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      for (int w2 = 1; w2 < W; ++w2) best = s_part[w2][lane] > best ? s_part[w2][lane] : best;
+      const int64_t first = ((int64_t)bucket << p.rshift) * a.K;
+      if (pos < table && first + pos < a.B * a.N * a.K) bin_emit<T, IS_MAX>(a, first + pos, best);
+    }
+    __syncthreads();
   }
 }
 
@@ -383,7 +496,7 @@ __global__ __launch_bounds__(kBinBlock) void bin_reduce_kernel(ScatterArgs a, Bi
     }
   }
   __syncthreads();
-  bin_flush_keys(a, p, bucket, s_keys);
+  bin_flush_keys<T, IS_MAX>(a, p, bucket, s_keys);
 }
 
 // The same reduction for rows held by a power-of-two number of lanes (<= 64): a wavefront reads 64 entry words
@@ -448,7 +561,7 @@ __global__ __launch_bounds__(kBinBlock) void bin_reduce_wave_kernel(ScatterArgs 
     }
   }
   __syncthreads();
-  bin_flush_keys(a, p, bucket, s_keys);
+  bin_flush_keys<T, IS_MAX>(a, p, bucket, s_keys);
 }
 
 static __global__ __launch_bounds__(kBlock) void bin_clear_kernel(unsigned long long *totals, int n, int *flag) {
@@ -560,7 +673,7 @@ __global__ __launch_bounds__(kBinBlock) void bin_add_wave_kernel(ScatterArgs a, 
   }
 }
 
-// the passes between scatter_key_init_kernel and scatter_key_final_kernel
+// min / max through the buckets: every element of out / arg_out is written by the reducing or the combining kernel
 template <typename T, int VEC, bool IS_MAX>
 void launch_binned_keys(const ScatterArgs &a, const BinArgs &plan, hipStream_t stream) {
   BinArgs p = plan;
@@ -584,6 +697,7 @@ void launch_binned_keys(const ScatterArgs &a, const BinArgs &plan, hipStream_t s
                        p, lshift);
   else
     hipLaunchKernelGGL((bin_reduce_kernel<T, VEC, IS_MAX>), dim3((unsigned)p.max_wgs), dim3(kBinBlock), 0, stream, a, p);
+  hipLaunchKernelGGL((bin_combine_kernel<T, IS_MAX>), dim3(2048), dim3(kBinBlock), 0, stream, a, p);
 }
 
 // sum: count (with the test for a sorted index), scan, place, add. The caller launches its usual sum kernels
