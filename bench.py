@@ -44,6 +44,12 @@ def parse_args():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--probe-scatter", action="store_true",
                     help="launch sequence for the L2 / atomic counters of the scatter kernels (see probe_scatter)")
+    ap.add_argument("--probe-ceilings", action="store_true",
+                    help="plain read / write / copy / mixed streams over several GiB: what the memory system of this "
+                         "device sustains (the ceilings the kernels are held against), nothing else is run")
+    ap.add_argument("--sweep-thresholds", action="store_true",
+                    help="time scatter sum / max just either side of every size threshold of the dispatcher and "
+                         "flag neighbours that differ by more than 1.5x")
     ap.add_argument("--probe", action="store_true",
                     help="counter-collection mode for rocprofv3 --pmc: a few launches of the dominant kernels "
                          "next to copies of known size, nothing timed")
@@ -66,6 +72,27 @@ def event_time(fn, iters, warm=3):
     return a.elapsed_time(b) * 1e-3 / iters
 
 
+def cold_time(fn, iters):
+    """Median seconds of a call that finds nothing of its inputs in a cache: 1 GiB is written between the
+    launches (the memory-side cache holds 256 MB), each launch timed on its own."""
+    import torch
+    flush = torch.empty(1 << 30, dtype=torch.uint8, device="cuda")
+    ts_ = []
+    for _ in range(max(iters, 5)):
+        flush.zero_()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        fn()
+        b.record()
+        torch.cuda.synchronize()
+        ts_.append(a.elapsed_time(b) * 1e-3)
+    del flush
+    return sorted(ts_)[len(ts_) // 2]
+
+
+CACHE_BYTES = 256 << 20  # inputs below this size stay in the memory-side cache from launch to launch
+
+
 def gbs(nbytes, seconds):
     return nbytes / seconds / 1e9
 
@@ -76,7 +103,26 @@ def entry(nbytes, seconds, elems):
             "Gelem_per_s": round(elems / seconds / 1e9, 2), "MB": round(nbytes / 1e6, 1)}
 
 
-def bench_csr_config(ts, wl, w, dev, iters, ops, uniform=False):
+# kernels behind every op of the table (the first one dominates), for the per-op roofline entries
+KERNELS = {
+    "segment_csr_sum": ["ts::csr_reduce_kernel"], "segment_csr_mean": ["ts::csr_reduce_kernel"],
+    "segment_csr_max": ["ts::csr_reduce_kernel"], "segment_coo_max": ["ts::csr_reduce_kernel", "ts::coo_to_indptr_kernel"],
+    "segment_coo_sum": ["ts::csr_reduce_kernel", "ts::coo_to_indptr_kernel"],
+    "gather_csr": ["ts::csr_gather_kernel"], "gather_coo": ["ts::coo_gather_kernel"],
+    "segment_csr_mean_backward": ["ts::csr_gather_kernel<DIV>"],
+}
+
+
+def with_roofline(e, kernels):
+    """The table entry of an op plus its roofline: every kernel of the op is HBM-bound, the time is that of
+    the whole launch sequence of the op (HIP events around back-to-back calls)."""
+    e = dict(e)
+    e["roofline"] = {"bound": "hbm", "kernels": kernels, "achieved": e["GBps"], "peak": PEAK_GBS, "unit": "GB/s",
+                     "frac": round(e["GBps"] / PEAK_GBS, 4), "algorithmic_bytes": int(e["MB"] * 1e6), "us": e["us"]}
+    return e
+
+
+def bench_csr_config(ts, wl, w, dev, iters, ops, uniform=False, cold=False):
     """segment / gather ops of one CSR-shaped workload through the operators."""
     import torch
     s = torch.empty(0, dtype=w.dtype).element_size()
@@ -112,6 +158,17 @@ def bench_csr_config(ts, wl, w, dev, iters, ops, uniform=False):
                 from pytorch_scatter_amd import capi
                 t = event_time(lambda: capi.segment_mean_csr_backward(out, indptr, src, 1, w.N, w.E, w.K, 0), iters)
                 res[op] = entry(wl.bytes_gather(w.E, w.N, w.K, s), t, EK)
+            res[op] = with_roofline(res[op], KERNELS.get(op, []))
+        if cold and w.E * w.K * s < CACHE_BYTES:
+            # small enough to sit in the memory-side cache between launches: also the time from HBM
+            for op in ops:
+                if op in ("segment_csr_sum", "segment_csr_mean"):
+                    r = op.rsplit("_", 1)[1]
+                    t = cold_time(lambda: ts.segment_csr(src, indptr, out, r), max(iters // 2, 5))
+                    res[op + "_cold"] = entry(wl.bytes_segment(w.E, w.N, w.K, s), t, EK)
+                elif op == "gather_csr":
+                    t = cold_time(lambda: ts.gather_csr(out, indptr, src), max(iters // 2, 5))
+                    res[op + "_cold"] = entry(wl.bytes_gather(w.E, w.N, w.K, s), t, EK)
     del src, out
     torch.cuda.empty_cache()
     return res
@@ -127,26 +184,18 @@ def bench_scatter_config(ts, wl, w, dev, iters, reduces):
             if r == "sum":
                 t = event_time(lambda: ts.scatter_sum(src, index, 0, None, w.N), iters)
                 res["scatter_sum"] = entry(wl.bytes_scatter(w.E, w.N, w.K, 4), t, w.E * w.K)
-                if w.E * w.K * 4 < (256 << 20):
-                    # small enough to sit in the 256 MB memory-side cache between launches: also report the
-                    # cold time (1 GiB written between the launches, each launch timed on its own, median)
-                    flush = torch.empty(1 << 30, dtype=torch.uint8, device=src.device)
-                    ts_ = []
-                    for _ in range(max(iters // 2, 5)):
-                        flush.zero_()
-                        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                        a.record()
-                        ts.scatter_sum(src, index, 0, None, w.N)
-                        b.record()
-                        torch.cuda.synchronize()
-                        ts_.append(a.elapsed_time(b) * 1e-3)
-                    del flush
-                    res["scatter_sum_cold"] = entry(wl.bytes_scatter(w.E, w.N, w.K, 4), sorted(ts_)[len(ts_) // 2],
-                                                    w.E * w.K)
+                if w.E * w.K * 4 < CACHE_BYTES:
+                    t = cold_time(lambda: ts.scatter_sum(src, index, 0, None, w.N), max(iters // 2, 5))
+                    res["scatter_sum_cold"] = entry(wl.bytes_scatter(w.E, w.N, w.K, 4), t, w.E * w.K)
             else:
                 fn = ts.scatter_max if r == "max" else ts.scatter_min
                 t = event_time(lambda: fn(src, index, 0, None, w.N), iters)
                 res["scatter_" + r] = entry(wl.bytes_scatter(w.E, w.N, w.K, 4, True), t, w.E * w.K)
+                if w.E * w.K * 4 < CACHE_BYTES:
+                    t = cold_time(lambda: fn(src, index, 0, None, w.N), max(iters // 2, 5))
+                    res["scatter_" + r + "_cold"] = entry(wl.bytes_scatter(w.E, w.N, w.K, 4, True), t, w.E * w.K)
+            key = "scatter_" + r
+            res[key] = with_roofline(res[key], ["ts::scatter_* (see profiles/bench_kernel_trace_stats.txt)"])
     del src
     torch.cuda.empty_cache()
     return res
@@ -252,6 +301,156 @@ def cpu_baseline(wl, w):
                       f"segment_csr sum + mean + gather_csr, {dt * 1e3:.1f} ms per pass"}
 
 
+def cpu_baselines_other(wl):
+    """The reference's CPU kernels (oracle/_ref, else the C oracle) on the scatter / segment_coo configurations, one
+    thread: C1 in full (the configuration BASELINE.json names "on CPU reference"), C4 with one value per entry
+    in full, C3 on a slice of 1/16 of its segments (the full input is 4.6 GB)."""
+    import torch
+    torch.set_num_threads(1)
+    ref_path = os.path.join(ROOT, "oracle", "_ref", "libts_ref_cpu.so")
+    ops, kind = None, "port"
+    if os.path.exists(ref_path):
+        try:
+            torch.ops.load_library(ref_path)
+            ops, kind = torch.ops.ts_ref, "reference"
+        except Exception:
+            ops = None
+    import ts_oracle
+
+    def scatter(src, index, N, reduce):
+        idx = index.view(-1, 1).expand_as(src)
+        if ops is not None:
+            return ops.scatter(src, idx, 0, None, N, reduce)
+        return ts_oracle.scatter(src, idx, 0, None, N, reduce)
+
+    def segment_coo(src, index, N, reduce):
+        if ops is not None:
+            return ops.segment_coo(src, index, None, N, reduce)
+        return ts_oracle.segment_coo(src, index, None, N, reduce)
+
+    def timed(fn, reps):
+        fn()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            fn()
+        return (time.perf_counter() - t0) / reps
+
+    out = {}
+    g = torch.Generator().manual_seed(0)
+    w1 = wl.c1_scatter_sum()
+    src = torch.randn((w1.E, w1.K), generator=g)
+    dt = timed(lambda: scatter(src, w1.index, w1.N, "sum"), 20)
+    out["C1"] = {"value": round(gbs(wl.bytes_scatter(w1.E, w1.N, w1.K, 4), dt), 3), "unit": "GB/s", "cores": 1,
+                 "kind": kind, "host_cores_available": os.cpu_count(),
+                 "sample": f"full C1 (scatter sum, E={w1.E}, N={w1.N}, K={w1.K}, fp32), 20 passes, {dt * 1e3:.2f} ms per pass"}
+    w4 = wl.c4_scatter_minmax(1)
+    src = torch.randn((w4.E, 1), generator=g)
+    dt = timed(lambda: scatter(src, w4.index, w4.N, "max"), 3)
+    out["C4-K1"] = {"value": round(gbs(wl.bytes_scatter(w4.E, w4.N, 1, 4, True), dt), 3), "unit": "GB/s", "cores": 1,
+                    "kind": kind, "host_cores_available": os.cpu_count(),
+                    "sample": f"full C4 with one value per entry (scatter max + arg, E={w4.E}, N={w4.N}), 3 passes, "
+                              f"{dt * 1e3:.1f} ms per pass"}
+    w3 = wl.c3_segment_coo(scale=1.0 / 16)
+    src = torch.rand((w3.E, w3.K), generator=g) * 2 - 1
+    dt = timed(lambda: segment_coo(src, w3.index, w3.N, "max"), 3)
+    out["C3"] = {"value": round(gbs(wl.bytes_segment(w3.E, w3.N, w3.K, 4, True, coo=True), dt), 3), "unit": "GB/s",
+                 "cores": 1, "kind": kind, "host_cores_available": os.cpu_count(),
+                 "sample": f"1/16 of C3 (segment_coo max + arg, E={w3.E}, N={w3.N}, K={w3.K}, fp32), 3 passes, "
+                           f"{dt * 1e3:.1f} ms per pass"}
+    return out
+
+
+def measured_traffic():
+    """HBM bytes per launch of the headline kernel as the tracked counter profile states them (a line
+    `traffic_bytes_per_launch: <number>` in profiles/csr_reduce_pmc_traffic.txt), or None."""
+    import re
+    try:
+        text = open(os.path.join(ROOT, "profiles", "csr_reduce_pmc_traffic.txt")).read()
+    except OSError:
+        return None
+    m = re.search(r"traffic_bytes_per_launch:\s*([0-9.eE+]+)", text)
+    return float(m.group(1)) if m else None
+
+
+def probe_ceilings():
+    """Plain streams through libts_probe.so (pytorch_scatter_amd/csrc/probe.hip): read, write, copy and reads mixed
+    with writes 3:1 and 26:1, over GiB-sized buffers, HIP events around 10 launches each."""
+    import ctypes
+    import torch
+    lib = ctypes.CDLL(os.path.join(ROOT, "pytorch_scatter_amd", "libts_probe.so"))
+    lib.ts_probe_stream.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
+    dev = torch.device("cuda:0")
+    a = torch.empty(6 << 30, dtype=torch.uint8, device=dev)
+    b = torch.empty(4 << 30, dtype=torch.uint8, device=dev)
+    a.fill_(1)
+    b.fill_(2)
+    stream = torch.cuda.current_stream().cuda_stream
+    rows = []
+    for name, mode, wbytes in (("read only (non-temporal 16-byte loads)", 0, 4 << 30), ("write only", 1, 4 << 30),
+                               ("copy 1:1", 2, 3 << 30), ("read 3 : write 1", 4, 2 << 30),
+                               ("read 26 : write 1", 27, 224 << 20)):
+        rd = 0 if mode == 1 else (wbytes if mode == 0 else (mode - 1) * wbytes)
+        wr = 0 if mode == 0 else wbytes
+        t = event_time(lambda: lib.ts_probe_stream(mode, a.data_ptr(), b.data_ptr(), wbytes, stream), 10, warm=2)
+        rows.append({"stream": name, "read_GB": round(rd / 1e9, 2), "written_GB": round(wr / 1e9, 2),
+                     "us": round(t * 1e6, 1), "GBps": round((rd + wr) / t / 1e9, 1),
+                     "pct_of_peak": round(100 * (rd + wr) / t / 1e9 / PEAK_GBS, 1)})
+    t = event_time(lambda: b[:3 << 30].copy_(a[:3 << 30]), 10, warm=2)
+    rows.append({"stream": "torch copy_ 1:1", "read_GB": 3.22, "written_GB": 3.22, "us": round(t * 1e6, 1),
+                 "GBps": round(2 * (3 << 30) / t / 1e9, 1), "pct_of_peak": round(100 * 2 * (3 << 30) / t / 1e9 / PEAK_GBS, 1)})
+    for r in rows:
+        print(f"{r['stream']:42s} read {r['read_GB']:6.2f} GB  written {r['written_GB']:6.2f} GB  {r['us']:9.1f} us  "
+              f"{r['GBps']:7.1f} GB/s  {r['pct_of_peak']:5.1f} % of 8 TB/s", file=sys.stderr)
+    print(json.dumps({"probe": "ceilings", "rows": rows}))
+
+
+def sweep_thresholds():
+    """scatter sum / max through the operators at sizes just either side of every size threshold of the dispatcher
+    (pytorch_scatter_amd/csrc/scatter.h, scatter_binned.h, scatter_k1.h): neighbours that differ by more than 1.5x in time
+    per entry are flagged. Index: Zipf(1.2) over N rows, shuffled."""
+    import numpy as np
+    import torch
+    import pytorch_scatter_amd as ts
+    dev = torch.device("cuda:0")
+    rng = np.random.default_rng(0)
+
+    def zipf_index(E, N):
+        p = np.arange(1, N + 1, dtype=np.float64) ** -1.2
+        return torch.from_numpy(rng.choice(N, size=E, p=p / p.sum()).astype(np.int64)).to(dev)
+
+    # (what, K, N, sizes in entries around the threshold)
+    M = 1 << 20
+    cases = [
+        ("sum: LDS table from 2^17 elements (contended index)", "sum", 16, 1000, [M // 128 - 1024, M // 128 + 1024]),
+        ("sum: LDS table from 2^22 elements (any index, K < 32)", "sum", 8, 1_000_000, [M // 2 - 8192, M // 2 + 8192]),
+        ("sum: buckets of output rows from 64 MB (K = 32)", "sum", 32, 100_000, [M // 2 - 16384, M // 2 + 16384]),
+        ("max: LDS table from 2^20 elements (contended index)", "max", 8, 1000, [M // 8 - 4096, M // 8 + 4096]),
+        ("max: one value per entry, slabs from 2^23 entries", "max", 1, 100_000, [8 * M - 65536, 8 * M + 65536]),
+        ("max: buckets of output rows from 16 MB (K = 32)", "max", 32, 100_000, [M // 8 - 8192, M // 8 + 8192]),
+        ("max: sample of the index from 2^23 elements (K = 8)", "max", 8, 1_000_000, [M - 65536, M + 65536]),
+    ]
+    rows, flagged = [], 0
+    with torch.no_grad():
+        for what, reduce, K, N, sizes in cases:
+            per_entry = []
+            for E in sizes:
+                index = zipf_index(E, N)
+                src = torch.randn((E, K), device=dev)
+                fn = ts.scatter_sum if reduce == "sum" else ts.scatter_max
+                t = event_time(lambda: fn(src, index, 0, None, N), 10)
+                per_entry.append(t / E)
+                rows.append({"threshold": what, "E": E, "K": K, "N": N, "us": round(t * 1e6, 1),
+                             "ns_per_entry": round(t / E * 1e9, 4)})
+                del src, index
+            ratio = max(per_entry) / min(per_entry)
+            rows[-1]["ratio_across_threshold"] = round(ratio, 2)
+            rows[-1]["cliff"] = ratio > 1.5
+            flagged += ratio > 1.5
+    for r in rows:
+        print(r, file=sys.stderr)
+    print(json.dumps({"probe": "thresholds", "cliffs": flagged, "rows": rows}))
+
+
 def probe():
     """Launch sequence for `rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE -- python3 bench.py --probe`:
     1. torch copy of 1 GiB (plain loads/stores, known size: calibrates the counters);
@@ -332,6 +531,10 @@ def probe_scatter():
 
 def main():
     args = parse_args()
+    if args.probe_ceilings:
+        return probe_ceilings()
+    if args.sweep_thresholds:
+        return sweep_thresholds()
     if args.probe:
         return probe()
     if args.probe_scatter:
@@ -374,8 +577,8 @@ def main():
         t_kernel = event_time(lambda: ts.segment_csr(src, indptr, out, "sum"), max(args.steps, 20))
     kernel_bytes = wl.bytes_segment(w2.E, w2.N, w2.K, 4)
     # HBM bytes per launch of this kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, calibrated against
-    # copies of known size (profiles/csr_reduce_pmc_traffic.txt): 107.7 MB read + 26.9 MB written
-    traffic = 134.6e6
+    # copies of known size: read from the tracked profile, null if that file does not state it
+    traffic = measured_traffic()
     roofline = {"bound": "hbm", "kernel": "ts::csr_reduce_kernel<float, 4, SUM>",
                 "achieved": round(gbs(kernel_bytes, t_kernel), 1), "peak": PEAK_GBS, "unit": "GB/s",
                 "frac": round(gbs(kernel_bytes, t_kernel) / PEAK_GBS, 4), "traffic": traffic,
@@ -390,10 +593,11 @@ def main():
     if "C1" in want:
         table["C1"] = bench_scatter_config(ts, wl, wl.c1_scatter_sum(), dev, it, ["sum"])
     if "C2" in want:
-        table["C2"] = bench_csr_config(ts, wl, w2, dev, it, ["segment_csr_sum", "segment_csr_mean", "gather_csr"])
+        table["C2"] = bench_csr_config(ts, wl, w2, dev, it, ["segment_csr_sum", "segment_csr_mean", "gather_csr"],
+                                       cold=True)
     if "C2m" in want:
         table["C2-mean16"] = bench_csr_config(ts, wl, wl.c2_segment_csr(mean16=True), dev, it,
-                                              ["segment_csr_sum", "segment_csr_mean", "gather_csr"])
+                                              ["segment_csr_sum", "segment_csr_mean", "gather_csr"], cold=True)
     if "C3" in want:
         table["C3"] = bench_csr_config(ts, wl, wl.c3_segment_coo(), dev, it, ["segment_coo_max"], uniform=True)
     if "C4" in want:
@@ -436,6 +640,7 @@ def main():
                                                  "gather_csr", "gather_coo"], uniform=True)
 
     cpu = None if args.no_cpu else cpu_baseline(wl, w2)
+    cpu_other = None if args.no_cpu else cpu_baselines_other(wl)
 
     line = {
         "metric": "effective HBM GB/s, segment_csr sum + mean + gather_csr (BASELINE config C2), 1 MI355X",
@@ -452,6 +657,7 @@ def main():
                    "api": "torch.ops.torch_scatter.* (eager, out= preallocated)"},
         "roofline": roofline,
         "cpu_baseline": cpu,
+        "cpu_baselines_other_configs": cpu_other,
         "configs": table,
     }
     print(json.dumps(line))

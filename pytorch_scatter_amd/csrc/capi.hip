@@ -553,7 +553,7 @@ int ts_scatter_count(const int64_t *index, float *count, int64_t B, int64_t E, i
     a.precheck = 1;
     a.lds_cache = env_int("TS_SCATTER_LDS", 1);
     a.lds_epb = env_int("TS_SCATTER_EPB", 0);
-    const bool contended = a.lds_cache == 2 || (a.lds_cache == 1 && B * E >= ((int64_t)1 << 20) && B * E >= 32 * B * N);
+    const bool contended = a.lds_cache == 2 || (a.lds_cache == 1 && B * E >= ((int64_t)1 << 17) && B * E >= 32 * B * N);
     if (contended && B * N < 0x7FFFFFFFll) {
       const int64_t epb = per_cu_chunk_edges(a.lds_epb, B * E, 16384, 131072);
       hipLaunchKernelGGL(scatter_add_lds_kernel<float>, dim3((unsigned)((B * E + epb - 1) / epb)), dim3(kLdsAddBlock), 0,

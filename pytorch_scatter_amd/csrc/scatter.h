@@ -222,7 +222,7 @@ struct ScatterArgs {
 // and the launch that returns at once cost 10-20 us), fewer than 32 entries per output row on average.
 inline bool skew_probe_shape(int64_t B, int64_t E, int64_t K, int64_t N, int elem_bytes, bool any_size) {
   return elem_bytes == 4 && K > 1 && K <= 256 && B * E >= 8192 &&
-         (any_size || (B * E * K >= ((int64_t)1 << 25) && E < 32 * N));
+         (any_size || (B * E * K >= ((int64_t)1 << 23) && E < 32 * N));
 }
 
 // ---- thread -> (edge, column) mapping shared by the scatter kernels ------------
@@ -1529,9 +1529,9 @@ int launch_scatter_v(const ScatterArgs &args, int reduce, hipStream_t stream) {
           // pooling layer, takes 450 us there and 940 us through the table; an unsorted one has the workspace path)
           const bool use_lds = a.lds_cache && a.sk == 0 && tn >= 64 && a.B * a.N < 0x7FFFFFFFll &&
                                (a.lds_cache == 2 ||
-                                (n_src >= ((int64_t)1 << 20) &&
+                                (n_src >= ((int64_t)1 << 17) &&
                                  (n_edges >= 32 * a.B * a.N ? (a.K < 32 || n_src * (int64_t)sizeof(T) < (int64_t)300000000)
-                                                            : (a.K < 32 && n_src >= ((int64_t)1 << 23)))));
+                                                            : (a.K < 32 && n_src >= ((int64_t)1 << 22)))));
           if (use_lds) {
             const int64_t epb = per_cu_chunk_edges(a.lds_epb, n_edges, 16384 / a.K > 256 ? 16384 / a.K : 256,
                                                    131072 / a.K > 2048 ? 131072 / a.K : 2048);

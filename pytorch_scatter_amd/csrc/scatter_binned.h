@@ -65,7 +65,10 @@ inline BinPlan bin_plan(int64_t B, int64_t E, int64_t K, int64_t N, int elem_byt
   const int64_t n_edges = B * E, rows = B * N;
   // rows of 64 bytes and more, inputs from 128 MB (below, the five extra launches cost more than the misses:
   // 64 MB of 128-byte rows, Zipf index: 65 us without, 79 us with; 154 MB of 512-byte rows: 348 against 115 us)
-  if (K * elem_bytes < 64 || K > kBinKeys / 16 || (!any_size && n_edges * K * elem_bytes < ((int64_t)128 << 20)) ||
+  // min / max (slabs) from 16 MB, sums from 64 MB (measured crossovers, Zipf(1.2) and uniform index onto 100 k rows of
+  // 32 floats: max 87 / 70 us without and 72 / 64 us with the buckets at 16 MB; sum 154 / 72 us and 81 / 91 us at 64 MB)
+  const int64_t min_bytes = slabs ? ((int64_t)16 << 20) : ((int64_t)64 << 20);
+  if (K * elem_bytes < 64 || K > kBinKeys / 16 || (!any_size && n_edges * K * elem_bytes < min_bytes) ||
       n_edges >= 0xFFFFFFFEll || rows >= 0x7FFFFFFFll || rows < 1)
     return r;
   const int64_t slots = (int64_t)kBinKeys * 8 / slot_bytes;
@@ -86,6 +89,10 @@ inline BinPlan bin_plan(int64_t B, int64_t E, int64_t K, int64_t N, int elem_byt
   if (n_edges < (int64_t)512 * kBinChunk) {
     chunk = (n_edges / 512 + 63) & ~(int64_t)63;
     if (chunk < 1024) chunk = 1024;
+    // a bucket of average size in one chunk: a bucket cut into several chunks hands a whole table per chunk to the
+    // combining kernel, whatever the chunk's size (524 k entries over 391 buckets in chunks of 1024: 324 us, 50 MB of slabs)
+    const int64_t twice_avg = (2 * n_edges / nb + 63) & ~(int64_t)63;
+    if (slabs && chunk < twice_avg) chunk = twice_avg < kBinChunk ? twice_avg : kBinChunk;
   }
   p.chunk = (int)chunk;
   p.max_wgs = n_edges / chunk + nb + 1;
