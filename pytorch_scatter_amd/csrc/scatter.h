@@ -1519,10 +1519,13 @@ int launch_scatter_v(const ScatterArgs &args, int reduce, hipStream_t stream) {
           // many entries per output slot: reduce in LDS first (see scatter_add_lds_kernel)
           int tn = 1;
           while ((int64_t)tn * 2 * a.K <= kLdsAcc && tn * 2 <= kLdsAccRows) tn *= 2;
-          // Rows under 32 columns: from 1 M elements on for a contended index, from 8 M elements on whatever the
-          // number of entries per output row (200 k x 16 floats onto 10 k rows are 4 us faster without the table). A
-          // skewed index gains a lot even at ten entries per row (10 M entries of a Zipf(1.2) index onto 1 M
-          // rows: K = 1 924 -> 135 us, K = 8 424 -> 239 us), a uniform one loses nothing (493 -> 483, 522 -> 494 us).
+          // Rows under 32 columns: for a contended index (32 and more entries per output row) from 2^17 elements on;
+          // for any other index from 2^18 entries or 2^22 elements on. Measured crossovers (us, run kernel / table):
+          // Zipf(1.2) index onto 1 M rows, K = 8: 65 k entries 211 / 20, 262 k 357 / 23, 1 M 424 / 40 -- every entry
+          // of a hub is an atomic on one address, 10 ns each; the same sizes under a uniform index 14 / 21, 27 / 26,
+          // 79 / 63; 200 k x 16 floats onto 10 k rows (uniform) 16.4 / 21.4, 400 k x 16: 39 / 30. Below these sizes
+          // the table costs a uniform index 5-7 us and a skewed one is left to the run kernel (known cliff: up to
+          // 20x for 65 k - 262 k entries under a heavy-tailed index).
           // Rows of 32 and more columns: for a contended index, the table up to 300 MB of input (1 M entries onto 3000 nodes, K = 32:
           // 70 / 58 / 106 us for a Zipf / sorted / uniform index against 275 / 174 / 126 us through the run kernel),
           // the run kernel with its hot rows above (9-10 M entries: a sorted index, such as the batch vector of a
@@ -1531,7 +1534,8 @@ int launch_scatter_v(const ScatterArgs &args, int reduce, hipStream_t stream) {
                                (a.lds_cache == 2 ||
                                 (n_src >= ((int64_t)1 << 17) &&
                                  (n_edges >= 32 * a.B * a.N ? (a.K < 32 || n_src * (int64_t)sizeof(T) < (int64_t)300000000)
-                                                            : (a.K < 32 && n_src >= ((int64_t)1 << 22)))));
+                                                            : (a.K < 32 && (n_src >= ((int64_t)1 << 22) ||
+                                                                            n_edges >= ((int64_t)1 << 18))))));
           if (use_lds) {
             const int64_t epb = per_cu_chunk_edges(a.lds_epb, n_edges, 16384 / a.K > 256 ? 16384 / a.K : 256,
                                                    131072 / a.K > 2048 ? 131072 / a.K : 2048);
