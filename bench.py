@@ -47,6 +47,8 @@ def parse_args():
     ap.add_argument("--probe-ceilings", action="store_true",
                     help="plain read / write / copy / mixed streams over several GiB: what the memory system of this "
                          "device sustains (the ceilings the kernels are held against), nothing else is run")
+    ap.add_argument("--probe-atomics", action="store_true",
+                    help="rate of device-scope 64-bit atomics on scattered and on neighbouring addresses")
     ap.add_argument("--sweep-thresholds", action="store_true",
                     help="time scatter sum / max just either side of every size threshold of the dispatcher and "
                          "flag neighbours that differ by more than 1.5x")
@@ -404,6 +406,31 @@ def probe_ceilings():
     print(json.dumps({"probe": "ceilings", "rows": rows}))
 
 
+def probe_atomics():
+    """Rate of device-scope 64-bit atomics (libts_probe.so): scattered addresses (one transaction per lane) and
+    neighbouring addresses shared by all workgroups (a table written back by every workgroup at once)."""
+    import ctypes
+    import torch
+    lib = ctypes.CDLL(os.path.join(ROOT, "pytorch_scatter_amd", "libts_probe.so"))
+    lib.ts_probe_atomics.restype = ctypes.c_longlong
+    lib.ts_probe_atomics.argtypes = [ctypes.c_void_p, ctypes.c_uint, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
+    dev = torch.device("cuda:0")
+    table = torch.zeros(1 << 20, dtype=torch.int64, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    rows = []
+    for name, slots, iters, pattern in (("scattered, 100 k slots, 1 M atomics", 100_000, 4, 0),
+                                        ("scattered, 100 k slots, 4 M atomics", 100_000, 16, 0),
+                                        ("scattered, 1 M slots, 4 M atomics", 1_000_000, 16, 0),
+                                        ("4096 neighbouring slots from each of 256 workgroups", 4096, 1, 1),
+                                        ("8192 neighbouring slots from each of 256 workgroups", 8192, 1, 1)):
+        n = lib.ts_probe_atomics(table.data_ptr(), slots, iters, pattern, stream)
+        t = event_time(lambda: lib.ts_probe_atomics(table.data_ptr(), slots, iters, pattern, stream), 10, warm=2)
+        rows.append({"pattern": name, "atomics": n, "us": round(t * 1e6, 1), "G_atomics_per_s": round(n / t / 1e9, 1)})
+    for r in rows:
+        print(f"{r['pattern']:56s} {r['atomics']:9d} atomics {r['us']:8.1f} us {r['G_atomics_per_s']:7.1f} G/s", file=sys.stderr)
+    print(json.dumps({"probe": "atomics", "rows": rows}))
+
+
 def sweep_thresholds():
     """scatter sum / max through the operators at sizes just either side of every size threshold of the dispatcher
     (pytorch_scatter_amd/csrc/scatter.h, scatter_binned.h, scatter_k1.h): neighbours that differ by more than 1.5x in time
@@ -533,6 +560,8 @@ def main():
     args = parse_args()
     if args.probe_ceilings:
         return probe_ceilings()
+    if args.probe_atomics:
+        return probe_atomics()
     if args.sweep_thresholds:
         return sweep_thresholds()
     if args.probe:

@@ -64,9 +64,38 @@ __global__ __launch_bounds__(kThreads) void mix_kernel(const u4 *__restrict__ p,
     }
   }
 }
+__device__ __forceinline__ uint32_t hash32(uint32_t x) {
+  x ^= x >> 16; x *= 0x7feb352dU; x ^= x >> 15; x *= 0x846ca68bU; x ^= x >> 16;
+  return x;
+}
+// 64-bit atomic max, device scope, without return. pattern 0: every lane its own pseudo-random slot of `slots`
+// (one transaction per lane); pattern 1: lane i of every workgroup -> slots i, i + 1024, ... below `slots`
+// (neighbouring lanes neighbouring addresses, every workgroup the same addresses: a table written back)
+__global__ __launch_bounds__(1024) void atomic_kernel(unsigned long long *tab, uint32_t slots, int iters, int pattern) {
+  const uint32_t t = blockIdx.x * 1024 + threadIdx.x;
+  if (pattern == 0) {
+    for (int it = 0; it < iters; ++it) {
+      const uint32_t h = hash32(t * 7919u + it * 104729u);
+      __hip_atomic_fetch_max(tab + h % slots, (unsigned long long)h << 20, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  } else {
+    for (uint32_t i = threadIdx.x; i < slots; i += 1024)
+      __hip_atomic_fetch_max(tab + i, (unsigned long long)hash32(blockIdx.x * 7919u + i) << 20, __ATOMIC_RELAXED,
+                             __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
 }  // namespace
 
 extern "C" {
+// 256 workgroups of 1024 lanes issue atomics on a table of `slots` 8-byte slots (see atomic_kernel); returns the
+// number of atomics of the launch, or -1 on a launch error.
+long long ts_probe_atomics(void *table, unsigned slots, int iters, int pattern, void *stream) {
+  hipLaunchKernelGGL(atomic_kernel, dim3(256), dim3(1024), 0, static_cast<hipStream_t>(stream),
+                     static_cast<unsigned long long *>(table), slots, iters, pattern);
+  if (hipGetLastError() != hipSuccess) return -1;
+  return pattern == 0 ? 256ll * 1024 * iters : 256ll * slots;
+}
+
 // mode 0: read `bytes` from a.  1: write `bytes` to b.  2..: read (mode - 1) * bytes from a and write `bytes` to b
 // (2 = copy). a must hold max(1, mode - 1) * bytes, b `bytes`; both 16-byte aligned. Returns 0 or 1 (launch error).
 int ts_probe_stream(int mode, const void *a, void *b, size_t bytes, void *stream) {
