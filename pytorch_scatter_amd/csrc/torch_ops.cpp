@@ -14,6 +14,7 @@
 #include <map>
 #include <mutex>
 
+#include "../../include/torchscatter/scatter.h"
 #include "../../include/ts_hip.h"
 
 namespace {
@@ -989,7 +990,13 @@ template <int REDUCE> struct SortedScatterFn : public torch::autograd::Function<
   }
 };
 
+}  // namespace
+
 // ------------------------------------------------------- registered functions
+// Exported with the names and signatures of the C++ API header (include/torchscatter/scatter.h).
+using torch::Tensor;
+using OptTensor = std::optional<Tensor>;
+using OptInt = std::optional<int64_t>;
 Tensor scatter_sum(Tensor src, Tensor index, int64_t dim, OptTensor out, OptInt dim_size) {
   return ScatterFn<TS_SUM>::apply(src, index, dim, out, dim_size)[0];
 }
@@ -1039,6 +1046,10 @@ std::tuple<Tensor, Tensor> segment_max_coo(Tensor src, Tensor index, OptTensor o
   return std::make_tuple(r[0], r[1]);
 }
 Tensor gather_coo(Tensor src, Tensor index, OptTensor out) { return GatherCooFn::apply(src, index, out)[0]; }
+
+int64_t scatter::cuda_version() noexcept { return ts_hip_version(); }
+
+namespace {
 
 Tensor scatter_softmax(Tensor src, Tensor index, int64_t dim, OptInt dim_size, bool log_space, double eps) {
   TORCH_CHECK(src.is_floating_point(), log_space ? "`scatter_log_softmax`" : "`scatter_softmax`",
