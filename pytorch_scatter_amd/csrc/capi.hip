@@ -472,7 +472,7 @@ size_t ts_scatter_workspace_bytes(int64_t B, int64_t E, int64_t K, int64_t N, in
     return probe && skew_probe_shape(B, E, K, N, kElemBytes[dtype], probe == 2) ? 256 : 0;
   }
   if (reduce == TS_SUM && kAccBytes[dtype] >= 4)  // table slots: int32 for int32, 8 bytes for the other types
-    return bin_plan(B, E, K, N, kElemBytes[dtype], nullptr, 0, any_size, dtype == TS_I32 ? 4 : 8).bytes;
+    return bin_plan(B, E, K, N, kElemBytes[dtype], nullptr, 0, any_size, dtype == TS_I32 ? 4 : 8, false, true).bytes;
   return 0;
 }
 

@@ -1497,16 +1497,12 @@ int launch_scatter_v(const ScatterArgs &args, int reduce, hipStream_t stream) {
       // the first pass), the entries are binned by bucket of output rows and summed in LDS (scatter_binned.h);
       // the kernels launched below then return at once. A sorted index stays with them: they combine its runs.
       if constexpr (BinSlotOk<T>::value) {
-        const int64_t kv = a.K / VEC;
-        int lshift = 0;
-        while (((int64_t)1 << lshift) < kv) ++lshift;
-        if (((int64_t)1 << lshift) == kv && kv <= kWave) {
-          const BinPlan bp = bin_plan(a.B, a.E, a.K, a.N, (int)sizeof(T), a.bin_ws, a.bin_ws_bytes, a.bin_any_size != 0,
-                                      (int)sizeof(typename BinSlot<T>::type));
-          if (bp.ok) {
-            launch_binned_add<T, VEC>(a, bp.p, lshift, stream);
-            a.skip_flag = bp.p.unsorted;
-          }
+        const BinPlan bp = bin_plan(a.B, a.E, a.K, a.N, (int)sizeof(T), a.bin_ws, a.bin_ws_bytes, a.bin_any_size != 0,
+                                    (int)sizeof(typename BinSlot<T>::type), false, true);
+        const int lshift = bp.ok ? bin_lane_shift(bp.p, VEC) : -1;
+        if (lshift >= 0) {
+          launch_binned_add<T, VEC>(a, bp.p, lshift, stream);
+          a.skip_flag = bp.p.unsorted;
         }
       }
     }
@@ -1649,7 +1645,7 @@ int launch_scatter_v(const ScatterArgs &args, int reduce, hipStream_t stream) {
         // sorted index: K = 16 894 / 784 / 537 -> 565 / 452 / 357 us, K = 32 1618 / 1169 / 662 -> 757 / 645 / 614 us)
         const BinPlan bp = bin_plan(a.B, a.E, a.K, a.N, (int)sizeof(T), a.bin_ws, a.bin_ws_bytes, a.bin_any_size != 0, 8,
                                     true);
-        if (bp.ok) {
+        if (bp.ok && (bp.p.slices == 1 || bin_lane_shift(bp.p, VEC) >= 0)) {
           if (is_max)
             launch_binned_keys<T, VEC, true>(a, bp.p, stream);
           else

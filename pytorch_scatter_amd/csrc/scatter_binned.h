@@ -23,10 +23,14 @@ constexpr int kBinMaxBuckets = 16384;  // LDS histogram of count / place (their 
 constexpr int kBinSmallCap = 8192;
 constexpr int kBinChunk = 8192;       // entries per chunk of a bucket in reduce (fewer for inputs under 4 M entries)
 constexpr int kBinPlaceChunk = 16384;  // entries per workgroup in count / place: one batch of 16 per lane
+constexpr int kCombPos = 64;          // combining kernel: keys per step of a bucket of many chunks,
+constexpr int kCombFew = 32;          // many: more than this
 constexpr int kBinPlaceBlock = 1024;   // (measured slower: 256 lanes x 4 batches, 64 K entries per workgroup, 8 K)
 
 struct BinArgs {
   int rshift;              // log2 of the rows per bucket
+  int kc;                  // columns of a row that one reducing workgroup holds in LDS (K when slices == 1)
+  int slices;              // K / kc: reducing workgroups per chunk, each on its own columns of the same entries
   int chunk;               // entries per reducing workgroup
   int nb;                  // buckets
   int64_t n_place;         // workgroups of count / place
@@ -40,8 +44,9 @@ struct BinArgs {
   uint64_t *binned;        // [B * E] (row in bucket << 32) | entry number
   int32_t *slab_start;     // min / max: [nb + 1] first slab of a bucket that is reduced in more than one chunk
   uint64_t *slabs;         // min / max: [slab][K << rshift] the tables of those chunks
-  int32_t *comb_list;      // min / max: buckets that the combining kernel finishes (not exactly one chunk), then
-  int32_t *comb_count;     //            how many
+  int32_t *comb_list;      // min / max: buckets that the combining kernel finishes (not exactly one chunk): those of
+                           //            up to kCombFew chunks from the front, those of more from slot nb - 1 down
+  int32_t *comb_count;     //            how many of either
 
   int *unsorted;           // sum only (else null): set to 1 by the count pass when the index is not sorted;
                            // a sorted index is left to the kernels that combine runs, and the passes after
@@ -57,8 +62,9 @@ struct BinPlan {
 };
 
 // slot_bytes: size of a table slot (8: packed keys of min / max, 4 or 8: accumulators of a sum)
+// slabs: min / max (workspace for the tables of chunks); whole_pow2: see below
 inline BinPlan bin_plan(int64_t B, int64_t E, int64_t K, int64_t N, int elem_bytes, void *ws, size_t ws_bytes,
-                        bool any_size = false, int slot_bytes = 8, bool slabs = false) {
+                        bool any_size = false, int slot_bytes = 8, bool slabs = false, bool whole_pow2 = false) {
   BinPlan r;
   r.ok = false;
   r.bytes = 0;
@@ -68,17 +74,43 @@ inline BinPlan bin_plan(int64_t B, int64_t E, int64_t K, int64_t N, int elem_byt
   // min / max (slabs) from 16 MB, sums from 64 MB (measured crossovers, Zipf(1.2) and uniform index onto 100 k rows of
   // 32 floats: max 87 / 70 us without and 72 / 64 us with the buckets at 16 MB; sum 154 / 72 us and 81 / 91 us at 64 MB)
   const int64_t min_bytes = slabs ? ((int64_t)16 << 20) : ((int64_t)64 << 20);
-  if (K * elem_bytes < 64 || K > kBinKeys / 16 || (!any_size && n_edges * K * elem_bytes < min_bytes) ||
+  if (K * elem_bytes < 64 || (!any_size && n_edges * K * elem_bytes < min_bytes) ||
       n_edges >= 0xFFFFFFFEll || rows >= 0x7FFFFFFFll || rows < 1)
     return r;
   const int64_t slots = (int64_t)kBinKeys * 8 / slot_bytes;
-  int rshift = 0;
-  while (((int64_t)2 << rshift) * K <= slots) ++rshift;
-  if (((int64_t)1 << rshift) > slots / 16) return r;  // the padding holds one slot per row
+  // The LDS table holds R rows of kc columns, R * kc = slots. Rows that are too wide for a bucket count within
+  // the histograms of count / place (K = 128 floats onto 1.5 M rows: 64 rows per bucket, 23 k buckets) are cut
+  // into slices of kc columns: a bucket keeps more rows, and K / kc workgroups reduce each of its chunks, every
+  // one on its own columns of the same entries. Slices are 1024 ... 64 bytes wide, the widest that fits.
+  auto shift_for = [&](int64_t kc) {
+    int rs = 0;
+    while (((int64_t)2 << rs) * kc <= slots) ++rs;
+    return rs;
+  };
+  auto fits = [&](int64_t kc) {
+    const int rs = shift_for(kc);
+    return kc <= kBinKeys / 16 && ((int64_t)1 << rs) <= slots / 16 &&  // the padding holds one slot per row
+           ((rows + ((int64_t)1 << rs) - 1) >> rs) <= kBinMaxBuckets;
+  };
+  // whole_pow2 (sums, which have the wavefront kernel only): a row is kept whole only if 1 ... 64 lanes with 16 bytes
+  // each hold it, a power of two of them
+  const int64_t lanes = K * elem_bytes / 16;
+  const bool whole_ok = !whole_pow2 || (K * elem_bytes % 16 == 0 && lanes <= 64 && (lanes & (lanes - 1)) == 0);
+  int64_t kc = K;
+  if (!whole_ok || !fits(K)) {
+    kc = 0;
+    for (int64_t bytes = 1024; bytes >= 64 && kc == 0; bytes >>= 1) {
+      const int64_t c = bytes / elem_bytes;
+      if (c < K && K % c == 0 && fits(c)) kc = c;
+    }
+    if (kc == 0) return r;
+  }
+  const int rshift = shift_for(kc);
   const int64_t nb = (rows + ((int64_t)1 << rshift) - 1) >> rshift;
-  if (nb > kBinMaxBuckets) return r;
   BinArgs &p = r.p;
   p.rshift = rshift;
+  p.kc = (int)kc;
+  p.slices = (int)(K / kc);
   p.nb = (int)nb;
   p.n_place = (n_edges + kBinPlaceChunk - 1) / kBinPlaceChunk;
   // A reducing workgroup walks its chunk in steps of a few rows per lane group, each step a memory latency:
@@ -104,7 +136,7 @@ inline BinPlan bin_plan(int64_t B, int64_t E, int64_t K, int64_t N, int elem_byt
   const size_t o_wh = take((size_t)p.n_place * nb * 4), o_bin = take((size_t)n_edges * 8), o_flag = take(256);
   // A bucket with m >= 2 chunks holds more than (m - 1) * chunk entries: at most 2 * n_edges / chunk slabs in all.
   const int64_t n_slabs = slabs ? 2 * (n_edges / chunk) + 2 : 0;
-  const size_t o_ss = take(slabs ? (size_t)(nb + 1) * 4 : 0), o_cl = take(slabs ? (size_t)(nb + 1) * 4 : 0);
+  const size_t o_ss = take(slabs ? (size_t)(nb + 1) * 4 : 0), o_cl = take(slabs ? (size_t)(nb + 2) * 4 : 0);
   const size_t o_sl = take((size_t)n_slabs * ((size_t)K << rshift) * 8);
   r.bytes = off;
   if (ws == nullptr || ws_bytes < off || (reinterpret_cast<uintptr_t>(ws) & 15) != 0) return r;
@@ -252,12 +284,13 @@ static __global__ __launch_bounds__(kBinBlock) void bin_scan_kernel(BinArgs p) {
   __shared__ int64_t s_t[kBinBlock];
   __shared__ int64_t s_c[kBinBlock];
   __shared__ int32_t s_m[kBinBlock];  // slabs: chunks of buckets with more than one
-  __shared__ int32_t s_l[kBinBlock];  // buckets for the combining kernel: those without exactly one chunk
+  __shared__ int32_t s_l[kBinBlock];  // buckets for the combining kernel: those without exactly one chunk,
+  __shared__ int32_t s_g[kBinBlock];  // of which more than kCombFew chunks
   if (p.sampled && *p.unsorted == 0) return;
   // a bucket holds fewer than 2^32 entries (the plan refuses larger inputs): 32-bit counts and divisions
   uint32_t t[PER], c[PER];
   int64_t sum_t = 0, sum_c = 0;
-  int32_t sum_m = 0, sum_l = 0;
+  int32_t sum_m = 0, sum_l = 0, sum_g = 0;
 #pragma unroll
   for (int j = 0; j < PER; ++j) {
     const int i = threadIdx.x * PER + j;
@@ -266,8 +299,10 @@ static __global__ __launch_bounds__(kBinBlock) void bin_scan_kernel(BinArgs p) {
     sum_t += t[j];
     sum_c += c[j];
     sum_m += c[j] > 1 ? (int32_t)c[j] : 0;
-    sum_l += (i < p.nb && c[j] != 1) ? 1 : 0;
+    sum_l += (i < p.nb && c[j] != 1 && c[j] <= (uint32_t)kCombFew) ? 1 : 0;
+    sum_g += c[j] > (uint32_t)kCombFew ? 1 : 0;
   }
+  s_g[threadIdx.x] = sum_g;
   s_t[threadIdx.x] = sum_t;
   s_c[threadIdx.x] = sum_c;
   s_m[threadIdx.x] = sum_m;
@@ -275,21 +310,26 @@ static __global__ __launch_bounds__(kBinBlock) void bin_scan_kernel(BinArgs p) {
   __syncthreads();
   for (int d = 1; d < kBinBlock; d <<= 1) {  // inclusive scan over the threads
     int64_t vt = 0, vc = 0;
-    int32_t vm = 0, vl = 0;
+    int32_t vm = 0, vl = 0, vg = 0;
     if ((int)threadIdx.x >= d) {
       vt = s_t[threadIdx.x - d]; vc = s_c[threadIdx.x - d]; vm = s_m[threadIdx.x - d]; vl = s_l[threadIdx.x - d];
+      vg = s_g[threadIdx.x - d];
     }
     __syncthreads();
     s_t[threadIdx.x] += vt;
     s_c[threadIdx.x] += vc;
     s_m[threadIdx.x] += vm;
     s_l[threadIdx.x] += vl;
+    s_g[threadIdx.x] += vg;
     __syncthreads();
   }
   int64_t run_t = s_t[threadIdx.x] - sum_t, run_c = s_c[threadIdx.x] - sum_c;
-  int32_t run_m = s_m[threadIdx.x] - sum_m, run_l = s_l[threadIdx.x] - sum_l;
+  int32_t run_m = s_m[threadIdx.x] - sum_m, run_l = s_l[threadIdx.x] - sum_l, run_g = s_g[threadIdx.x] - sum_g;
   const int64_t all_c = s_c[kBinBlock - 1];
-  if (p.comb_count != nullptr && threadIdx.x == 0) *p.comb_count = s_l[kBinBlock - 1];
+  if (p.comb_count != nullptr && threadIdx.x == 0) {
+    p.comb_count[0] = s_l[kBinBlock - 1];
+    p.comb_count[1] = s_g[kBinBlock - 1];
+  }
 #pragma unroll
   for (int j = 0; j < PER; ++j) {
     const int i = threadIdx.x * PER + j;
@@ -299,14 +339,18 @@ static __global__ __launch_bounds__(kBinBlock) void bin_scan_kernel(BinArgs p) {
       p.chunk_start[i] = (int32_t)run_c;
       if (p.slab_start != nullptr) {
         p.slab_start[i] = run_m;
-        if (c[j] != 1) p.comb_list[run_l] = i;
+        if (c[j] > (uint32_t)kCombFew)
+          p.comb_list[p.nb - 1 - run_g] = i;
+        else if (c[j] != 1)
+          p.comb_list[run_l] = i;
       }
     }
     if (i == p.nb) { p.starts[i] = run_t; p.chunk_start[i] = (int32_t)run_c; }
     run_t += t[j];
     run_c += c[j];
     run_m += c[j] > 1 ? (int32_t)c[j] : 0;
-    run_l += (i < p.nb && c[j] != 1) ? 1 : 0;
+    run_l += (i < p.nb && c[j] != 1 && c[j] <= (uint32_t)kCombFew) ? 1 : 0;
+    run_g += c[j] > (uint32_t)kCombFew ? 1 : 0;
   }
   if (threadIdx.x == kBinBlock - 1 && p.nb == kBinMaxBuckets) {
     p.starts[p.nb] = run_t;
@@ -400,39 +444,50 @@ __device__ __forceinline__ void bin_emit(const ScatterArgs &a, int64_t i, uint64
 // in memory with a read and an atomic per key took 56 of 300 us for 10 M entries of 32 floats: 13 M atomics,
 // most of them on the 8192 keys of the bucket that holds the hubs.)
 template <typename T, bool IS_MAX>
-__device__ __forceinline__ void bin_flush_keys(const ScatterArgs &a, const BinArgs &p, int bucket,
+__device__ __forceinline__ void bin_flush_keys(const ScatterArgs &a, const BinArgs &p, int bucket, int wg, int slice,
                                                const uint64_t *s_keys) {
-  const int K = (int)a.K;
+  const int K = (int)a.K, kc = p.kc;
+  const int c0 = slice * kc;                                    // first column of this workgroup's slice
   const int64_t first = ((int64_t)bucket << p.rshift) * a.K;   // first element of the bucket in [B * N, K]
-  const int64_t limit = a.B * a.N * a.K - first;                // elements of rows that exist
-  const int table = K << p.rshift;
+  const int64_t rows_left = a.B * a.N - ((int64_t)bucket << p.rshift);  // rows that exist
+  const int table = kc << p.rshift;
   const int chunks = p.chunk_start[bucket + 1] - p.chunk_start[bucket];
   if (chunks == 1) {
-    for (int i = threadIdx.x; i < table && i < limit; i += kBinBlock) bin_emit<T, IS_MAX>(a, first + i, s_keys[i + i / K]);
+    for (int i = threadIdx.x; i < table; i += kBinBlock) {
+      const int row = i / kc;
+      if (row < rows_left) bin_emit<T, IS_MAX>(a, first + (int64_t)row * K + c0 + (i - row * kc), s_keys[i + row]);
+    }
   } else {
-    uint64_t *slab = p.slabs + ((int64_t)p.slab_start[bucket] + ((int64_t)blockIdx.x - p.chunk_start[bucket])) * table;
-    for (int i = threadIdx.x; i < table; i += kBinBlock) slab[i] = s_keys[i + i / K];  // row i / K starts i / K keys later
+    uint64_t *slab = p.slabs + ((int64_t)p.slab_start[bucket] + (wg - p.chunk_start[bucket])) * ((int64_t)K << p.rshift);
+    for (int i = threadIdx.x; i < table; i += kBinBlock) {
+      const int row = i / kc;
+      slab[row * K + c0 + (i - row * kc)] = s_keys[i + row];  // row `row` of the table starts `row` keys later
+    }
   }
 }
 
 // Buckets that were not reduced in exactly one chunk: the maximum over the slabs of their chunks (none: a bucket
-// without entries), element by element, to out / arg_out. A workgroup takes kCombPos neighbouring keys of one
-// bucket; its wavefronts share the slabs, sixteen loads in flight each, and meet in LDS.
-constexpr int kCombPos = 64;
+// without entries), element by element, to out / arg_out. A workgroup takes 1024 neighbouring keys of one bucket.
+// A bucket of few chunks (an index with many entries per output row everywhere: 2-4 chunks in every bucket) gives
+// every lane one key and walks the slabs in order; a bucket of many chunks (the one that holds the hubs of a skewed
+// index: a thousand slabs) is taken 64 keys at a time, the wavefronts share the slabs, sixteen loads in flight
+// each, and meet in LDS.
 template <typename T, bool IS_MAX>
 __global__ __launch_bounds__(kBinBlock) void bin_combine_kernel(ScatterArgs a, BinArgs p) {
   constexpr int W = kBinBlock / kWave;
   __shared__ uint64_t s_part[W][kCombPos];
   const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
   const int table = (int)a.K << p.rshift;
+  const int n_few = p.comb_count[0], n_many = p.comb_count[1];
+  const int64_t total = a.B * a.N * a.K;
+  // buckets of many chunks first (the long items), 64 keys per workgroup and step
   const int parts = (table + kCombPos - 1) / kCombPos;
-  const int n_list = *p.comb_count;
-  for (int64_t item = blockIdx.x; item < (int64_t)n_list * parts; item += gridDim.x) {
-    const int bucket = p.comb_list[item / parts];
-    const int pos = (int)(item % parts) * kCombPos + lane;
-    const int c0 = p.slab_start[bucket];
+  for (int64_t item = blockIdx.x; item < (int64_t)n_many * parts; item += gridDim.x) {
+    const int bucket = p.comb_list[p.nb - 1 - (int)(item / parts)];
     const int m = p.chunk_start[bucket + 1] - p.chunk_start[bucket];
-    const uint64_t *slab = p.slabs + (int64_t)c0 * table + (pos < table ? pos : 0);
+    const int pos = (int)(item % parts) * kCombPos + lane;
+    const int64_t first = ((int64_t)bucket << p.rshift) * a.K;
+    const uint64_t *slab = p.slabs + (int64_t)p.slab_start[bucket] * table + (pos < table ? pos : 0);
     uint64_t best = 0;
     constexpr int U = 16;  // loads in flight per lane: the slabs of a bucket with a thousand chunks in four round trips
     for (int s0 = wave; s0 < m; s0 += W * U) {
@@ -447,10 +502,29 @@ __global__ __launch_bounds__(kBinBlock) void bin_combine_kernel(ScatterArgs a, B
     if (wave == 0) {
 #pragma unroll
       for (int w2 = 1; w2 < W; ++w2) best = s_part[w2][lane] > best ? s_part[w2][lane] : best;
-      const int64_t first = ((int64_t)bucket << p.rshift) * a.K;
-      if (pos < table && first + pos < a.B * a.N * a.K) bin_emit<T, IS_MAX>(a, first + pos, best);
+      if (pos < table && first + pos < total) bin_emit<T, IS_MAX>(a, first + pos, best);
     }
     __syncthreads();
+  }
+  // buckets of few chunks, 1024 keys per workgroup and step
+  const int blocks = (table + kBinBlock - 1) / kBinBlock;
+  for (int64_t item = blockIdx.x; item < (int64_t)n_few * blocks; item += gridDim.x) {
+    const int bucket = p.comb_list[item / blocks];
+    const int m = p.chunk_start[bucket + 1] - p.chunk_start[bucket];
+    const int pos = (int)(item % blocks) * kBinBlock + (int)threadIdx.x;
+    const int64_t first = ((int64_t)bucket << p.rshift) * a.K;
+    if (pos >= table || first + pos >= total) continue;
+    const uint64_t *slab = p.slabs + (int64_t)p.slab_start[bucket] * table + pos;
+    constexpr int U = 8;
+    uint64_t best = 0;
+    for (int s0 = 0; s0 < m; s0 += U) {
+      uint64_t k[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) k[u] = slab[(int64_t)(s0 + u < m ? s0 + u : s0) * table];
+#pragma unroll
+      for (int u = 0; u < U; ++u) best = k[u] > best ? k[u] : best;
+    }
+    bin_emit<T, IS_MAX>(a, first + pos, best);
   }
 }
 
@@ -503,7 +577,7 @@ __global__ __launch_bounds__(kBinBlock) void bin_reduce_kernel(ScatterArgs a, Bi
     }
   }
   __syncthreads();
-  bin_flush_keys<T, IS_MAX>(a, p, bucket, s_keys);
+  bin_flush_keys<T, IS_MAX>(a, p, bucket, (int)blockIdx.x, 0, s_keys);
 }
 
 // The same reduction for rows held by a power-of-two number of lanes (<= 64): a wavefront reads 64 entry words
@@ -513,22 +587,23 @@ template <typename T, int VEC, bool IS_MAX>
 __global__ __launch_bounds__(kBinBlock) void bin_reduce_wave_kernel(ScatterArgs a, BinArgs p, int lshift) {
   constexpr int U = 4;  // eight rows in flight per lane: 90 VGPRs, one workgroup per CU, no gain
   __shared__ uint64_t s_keys[kBinKeys + kBinKeys / 16];  // rows K + 1 keys apart (LDS banks, see above)
-  const int bucket = p.wg_bucket[blockIdx.x];
+  const int wg = (int)(blockIdx.x / (unsigned)p.slices), slice = (int)(blockIdx.x - (unsigned)wg * p.slices);
+  const int bucket = p.wg_bucket[wg];
   if (bucket < 0) return;
-  const int K = (int)a.K;
-  const int KP = K + 1;
+  const int KP = p.kc + 1;
   const int rows = 1 << p.rshift;
   for (int i = threadIdx.x; i < rows * KP; i += kBinBlock) s_keys[i] = 0;
   __syncthreads();
 
   const T *src = static_cast<const T *>(a.src);
-  const int64_t lo = p.starts[bucket] + ((int64_t)blockIdx.x - p.chunk_start[bucket]) * p.chunk;
+  const int64_t lo = p.starts[bucket] + ((int64_t)wg - p.chunk_start[bucket]) * p.chunk;
   int64_t hi = lo + p.chunk;
   if (hi > p.starts[bucket + 1]) hi = p.starts[bucket + 1];
   const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
   const int g = lane >> lshift;                 // lane group: one entry at a time
   const int gpw = kWave >> lshift;              // lane groups per wavefront
-  const int k0 = (lane & ((1 << lshift) - 1)) * VEC;
+  const int k0 = (lane & ((1 << lshift) - 1)) * VEC;         // column inside the slice
+  const int ksrc = slice * p.kc + k0;                        // column of the row
   constexpr int64_t kStride = (int64_t)(kBinBlock / kWave) * kWave;  // entries per pass of the workgroup
   if (lo < hi) {
     int64_t base = lo + (int64_t)wave * kWave;
@@ -548,7 +623,7 @@ __global__ __launch_bounds__(kBinBlock) void bin_reduce_wave_kernel(ScatterArgs 
           const int from = i < n ? i : n - 1;
           e_ent[u] = (uint32_t)__shfl((int)ent_lo, from);
           e_row[u] = (uint32_t)__shfl((int)ent_hi, from);
-          x[u] = load_vec_stream<T, VEC>(src + (int64_t)e_ent[u] * a.K + k0);
+          x[u] = load_vec_stream<T, VEC>(src + (int64_t)e_ent[u] * a.K + ksrc);
         }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
@@ -568,7 +643,7 @@ __global__ __launch_bounds__(kBinBlock) void bin_reduce_wave_kernel(ScatterArgs 
     }
   }
   __syncthreads();
-  bin_flush_keys<T, IS_MAX>(a, p, bucket, s_keys);
+  bin_flush_keys<T, IS_MAX>(a, p, bucket, wg, slice, s_keys);
 }
 
 static __global__ __launch_bounds__(kBlock) void bin_clear_kernel(unsigned long long *totals, int n, int *flag) {
@@ -595,22 +670,24 @@ __global__ __launch_bounds__(kBinBlock) void bin_add_wave_kernel(ScatterArgs a, 
   constexpr int kSlots = (kBinKeys + kBinKeys / 16) * 8 / (int)sizeof(A);
   __shared__ A s_acc[kSlots];  // rows K + 1 slots apart (LDS banks)
   if (p.unsorted != nullptr && *p.unsorted == 0) return;
-  const int bucket = p.wg_bucket[blockIdx.x];
+  const int wg = (int)(blockIdx.x / (unsigned)p.slices), slice = (int)(blockIdx.x - (unsigned)wg * p.slices);
+  const int bucket = p.wg_bucket[wg];
   if (bucket < 0) return;
-  const int K = (int)a.K;
-  const int KP = K + 1;
+  const int K = (int)a.K, kc = p.kc;
+  const int KP = kc + 1;
   const int rows = 1 << p.rshift;
   for (int i = threadIdx.x; i < rows * KP; i += kBinBlock) s_acc[i] = (A)0;
   __syncthreads();
 
   const T *src = static_cast<const T *>(a.src);
-  const int64_t lo = p.starts[bucket] + ((int64_t)blockIdx.x - p.chunk_start[bucket]) * p.chunk;
+  const int64_t lo = p.starts[bucket] + ((int64_t)wg - p.chunk_start[bucket]) * p.chunk;
   int64_t hi = lo + p.chunk;
   if (hi > p.starts[bucket + 1]) hi = p.starts[bucket + 1];
   const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
   const int g = lane >> lshift;
   const int gpw = kWave >> lshift;
-  const int k0 = (lane & ((1 << lshift) - 1)) * VEC;
+  const int k0 = (lane & ((1 << lshift) - 1)) * VEC;  // column inside the slice
+  const int c0 = slice * kc;                          // first column of the slice
   constexpr int64_t kStride = (int64_t)(kBinBlock / kWave) * kWave;
   if (lo < hi) {
     int64_t base = lo + (int64_t)wave * kWave;
@@ -630,7 +707,7 @@ __global__ __launch_bounds__(kBinBlock) void bin_add_wave_kernel(ScatterArgs a, 
           const int from = i < n ? i : n - 1;
           const uint32_t e_ent = (uint32_t)__shfl((int)ent_lo, from);
           e_row[u] = (uint32_t)__shfl((int)ent_hi, from);
-          x[u] = load_vec_stream<T, VEC>(src + (int64_t)e_ent * a.K + k0);
+          x[u] = load_vec_stream<T, VEC>(src + (int64_t)e_ent * a.K + c0 + k0);
         }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
@@ -644,40 +721,56 @@ __global__ __launch_bounds__(kBinBlock) void bin_add_wave_kernel(ScatterArgs a, 
     }
   }
   __syncthreads();
-  T *out = static_cast<T *>(a.out) + ((int64_t)bucket << p.rshift) * a.K;
-  const int64_t limit = (a.B * a.N - ((int64_t)bucket << p.rshift)) * a.K;  // elements of rows that exist
-  const int table = K << p.rshift;
+  T *out = static_cast<T *>(a.out) + ((int64_t)bucket << p.rshift) * a.K + c0;
+  const int64_t rows_left = a.B * a.N - ((int64_t)bucket << p.rshift);  // rows that exist
+  const int table = kc << p.rshift;
   if constexpr (sizeof(T) == 2) {
-    // two neighbouring columns per packed atomic (K is even here: whole 16-byte vectors per lane)
+    // two neighbouring columns per packed atomic (kc is even here: whole 16-byte vectors per lane)
     if ((reinterpret_cast<uintptr_t>(a.out) & 3) == 0) {
-      for (int i = 2 * threadIdx.x; i < table && i < limit; i += 2 * kBinBlock) {
-        const A v0 = s_acc[i + i / K], v1 = s_acc[i + 1 + (i + 1) / K];
+      for (int i = 2 * threadIdx.x; i < table; i += 2 * kBinBlock) {
+        const int row = i / kc;
+        if (row >= rows_left) break;
+        const A v0 = s_acc[i + row], v1 = s_acc[i + 1 + row];
         if (v0 == (A)0 && v1 == (A)0) continue;
+        T *dst = out + (int64_t)row * K + (i - row * kc);
         if constexpr (__is_same(T, bf16_t)) {
           typedef short v2s __attribute__((ext_vector_type(2)));
           v2s pk;
           pk.x = (short)float_to_bf16((float)v0).x;
           pk.y = (short)float_to_bf16((float)v1).x;
-          __builtin_amdgcn_global_atomic_fadd_v2bf16(reinterpret_cast<v2s *>(out + i), pk);
+          __builtin_amdgcn_global_atomic_fadd_v2bf16(reinterpret_cast<v2s *>(dst), pk);
         } else {
           typedef _Float16 v2h __attribute__((ext_vector_type(2)));
           v2h pk;
           pk.x = (_Float16)(float)v0;
           pk.y = (_Float16)(float)v1;
-          __builtin_amdgcn_global_atomic_fadd_v2f16(reinterpret_cast<v2h *>(out + i), pk);
+          __builtin_amdgcn_global_atomic_fadd_v2f16(reinterpret_cast<v2h *>(dst), pk);
         }
       }
       return;
     }
   }
-  for (int i = threadIdx.x; i < table && i < limit; i += kBinBlock) {
-    const A v = s_acc[i + i / K];
+  for (int i = threadIdx.x; i < table; i += kBinBlock) {
+    const int row = i / kc;
+    if (row >= rows_left) break;
+    const A v = s_acc[i + row];
     if (v == (A)0) continue;
+    T *dst = out + (int64_t)row * K + (i - row * kc);
     if constexpr (sizeof(T) == 2)  // no compare-and-swap loop: hundreds of chunks of a hub bucket meet here
-      atomic_add_half<T>(out + i, from_acc<T>((F)v), static_cast<T *>(a.out), static_cast<T *>(a.out) + a.B * a.N * a.K);
+      atomic_add_half<T>(dst, from_acc<T>((F)v), static_cast<T *>(a.out), static_cast<T *>(a.out) + a.B * a.N * a.K);
     else
-      atomic_add_elem<T>(out + i, from_acc<T>((F)v));
+      atomic_add_elem<T>(dst, from_acc<T>((F)v));
   }
+}
+
+// log2 of the lanes that hold the kc columns of a slice, VEC columns each: the wavefront kernels want a power of
+// two up to 64. -1: no such number (then only bin_reduce_kernel can take the plan, and only without slices).
+inline int bin_lane_shift(const BinArgs &p, int vec) {
+  if (p.kc % vec != 0) return -1;
+  const int kv = p.kc / vec;
+  int lshift = 0;
+  while ((1 << lshift) < kv) ++lshift;
+  return ((1 << lshift) == kv && kv <= kWave) ? lshift : -1;
 }
 
 // min / max through the buckets: every element of out / arg_out is written by the reducing or the combining kernel
@@ -696,12 +789,10 @@ void launch_binned_keys(const ScatterArgs &a, const BinArgs &plan, hipStream_t s
     hipLaunchKernelGGL(bin_place_kernel<kBinSmallCap>, dim3((unsigned)p.n_place), dim3(kBinPlaceBlock), 0, stream, a, p);
   else
     hipLaunchKernelGGL(bin_place_kernel<kBinMaxBuckets>, dim3((unsigned)p.n_place), dim3(kBinPlaceBlock), 0, stream, a, p);
-  const int64_t kv = a.K / VEC;
-  int lshift = 0;
-  while (((int64_t)1 << lshift) < kv) ++lshift;
-  if (((int64_t)1 << lshift) == kv && kv <= kWave && !getenv("TS_BIN_NO_WAVE"))  // env: tuning aid
-    hipLaunchKernelGGL((bin_reduce_wave_kernel<T, VEC, IS_MAX>), dim3((unsigned)p.max_wgs), dim3(kBinBlock), 0, stream, a,
-                       p, lshift);
+  const int lshift = bin_lane_shift(p, VEC);
+  if (lshift >= 0 && (p.slices > 1 || !getenv("TS_BIN_NO_WAVE")))  // env: tuning aid
+    hipLaunchKernelGGL((bin_reduce_wave_kernel<T, VEC, IS_MAX>), dim3((unsigned)(p.max_wgs * p.slices)), dim3(kBinBlock), 0,
+                       stream, a, p, lshift);
   else
     hipLaunchKernelGGL((bin_reduce_kernel<T, VEC, IS_MAX>), dim3((unsigned)p.max_wgs), dim3(kBinBlock), 0, stream, a, p);
   hipLaunchKernelGGL((bin_combine_kernel<T, IS_MAX>), dim3(2048), dim3(kBinBlock), 0, stream, a, p);
@@ -725,7 +816,8 @@ void launch_binned_add(const ScatterArgs &a, const BinArgs &plan, int lshift, hi
     hipLaunchKernelGGL(bin_place_kernel<kBinSmallCap>, dim3((unsigned)p.n_place), dim3(kBinPlaceBlock), 0, stream, a, p);
   else
     hipLaunchKernelGGL(bin_place_kernel<kBinMaxBuckets>, dim3((unsigned)p.n_place), dim3(kBinPlaceBlock), 0, stream, a, p);
-  hipLaunchKernelGGL((bin_add_wave_kernel<T, VEC>), dim3((unsigned)p.max_wgs), dim3(kBinBlock), 0, stream, a, p, lshift);
+  hipLaunchKernelGGL((bin_add_wave_kernel<T, VEC>), dim3((unsigned)(p.max_wgs * p.slices)), dim3(kBinBlock), 0, stream, a, p,
+                     lshift);
 }
 
 }  // namespace ts

@@ -529,10 +529,13 @@ def test_scatter_minmax_lds_cached_variant(capi, oracle, shape, reduce, dtype, m
 
 @pytest.mark.parametrize("shape,reduce,dtype", list(product(
     [(1, 60000, 32, 300), (2, 40000, 16, 700), (1, 50000, 128, 90), (1, 30000, 24, 5000), (1, 20000, 64, 100000),
-     (3, 9000, 512, 5), (1, 70000, 17, 40)],
+     (3, 9000, 512, 5), (1, 70000, 17, 40),
+     (1, 8000, 1024, 50), (2, 5000, 768, 33)],   # rows wider than a table row: reduced in slices of columns
     ["min", "max"], [torch.float32, torch.bfloat16, torch.int32, torch.int8]))
     + [((1, 20000, 64, 600000), "max", torch.float32), ((1, 20000, 64, 600000), "min", torch.int32),  # 4688 buckets
-       ((1, 20000, 128, 540000), "max", torch.float32)])  # 8438 buckets
+       ((1, 20000, 128, 540000), "max", torch.float32),  # 8438 buckets
+       # too many buckets of whole rows (16 875): four slices of 128 columns, 4219 buckets
+       ((1, 20000, 512, 270000), "max", torch.float32), ((1, 20000, 512, 270000), "min", torch.bfloat16)])
 def test_scatter_minmax_binned_variant(capi, oracle, shape, reduce, dtype, monkeypatch):
     """min / max with a workspace: entries binned by bucket of output rows and reduced in LDS (forced on at
     these sizes), skewed index with heavy ties, with and without previous content in out. Rows under 64 bytes
@@ -563,7 +566,7 @@ def test_scatter_minmax_binned_variant(capi, oracle, shape, reduce, dtype, monke
     L = capi.lib()
     need = L.ts_scatter_workspace_bytes(capi._i(B), capi._i(E), capi._i(K), capi._i(N), capi.DTYPE[dtype],
                                         capi.REDUCE[reduce])
-    assert (need > 0) == (K * src.element_size() >= 64 and K <= 512)
+    assert (need > 0) == (K * src.element_size() >= 64)
     assert L.ts_scatter_workspace_bytes(capi._i(B), capi._i(E), capi._i(K), capi._i(N), capi.DTYPE[dtype], capi.MUL) == 0
 
 
@@ -627,11 +630,13 @@ def test_scatter_minmax_skew_probe(capi, oracle, shape, kind, reduce, dtype, mon
 
 @pytest.mark.parametrize("shape,kind,dtype", list(product(
     [(1, 60000, 32, 300), (2, 40000, 16, 700), (1, 50000, 128, 90), (1, 20000, 64, 100000), (3, 9000, 256, 5),
-     (1, 30000, 24, 500)],
+     (1, 30000, 24, 500),
+     (1, 8000, 1024, 50), (2, 5000, 96, 330)],   # reduced in slices of columns (96: no power of two of lanes)
     ["zipf", "sorted", "one descent"],
     [torch.float32, torch.float64, torch.bfloat16, torch.float16, torch.int32, torch.int64, torch.int16]))
     + [((1, 20000, 64, 600000), "zipf", torch.float32), ((1, 20000, 64, 600000), "one descent", torch.int32),  # 4688 buckets
-       ((1, 20000, 128, 540000), "zipf", torch.int32)])  # 8438 buckets
+       ((1, 20000, 128, 540000), "zipf", torch.int32),  # 8438 buckets
+       ((1, 20000, 512, 270000), "zipf", torch.float32)])  # four slices of 128 columns, 4219 buckets
 def test_scatter_sum_binned_variant(capi, oracle, shape, kind, dtype, monkeypatch):
     """Sum with a workspace (forced on at these sizes): a sample of the index (or, with the sample switched
     off as in the "one descent" cases, the count pass) finds out whether the index is sorted;
