@@ -445,7 +445,7 @@ def sweep_thresholds():
         p = np.arange(1, N + 1, dtype=np.float64) ** -1.2
         return torch.from_numpy(rng.choice(N, size=E, p=p / p.sum()).astype(np.int64)).to(dev)
 
-    # (what, K, N, sizes in entries around the threshold)
+    # (what, K, N, sizes in entries around the threshold); N a list: 2 M entries, output rows around the threshold
     M = 1 << 20
     cases = [
         ("sum: LDS table from 2^17 elements (contended index)", "sum", 16, 1000, [M // 128 - 1024, M // 128 + 1024]),
@@ -455,12 +455,15 @@ def sweep_thresholds():
         ("max: one value per entry, slabs from 2^23 entries", "max", 1, 100_000, [8 * M - 65536, 8 * M + 65536]),
         ("max: buckets of output rows from 16 MB (K = 32)", "max", 32, 100_000, [M // 8 - 8192, M // 8 + 8192]),
         ("max: sample of the index from 2^23 elements (K = 8)", "max", 8, 1_000_000, [M - 65536, M + 65536]),
+        ("sum: rows in slices of columns above 16384 buckets (K = 128)", "sum", 128, [M - 8192, M + 8192], None),
+        ("max: rows in slices of columns above 16384 buckets (K = 128)", "max", 128, [M - 8192, M + 8192], None),
     ]
     rows, flagged = [], 0
     with torch.no_grad():
         for what, reduce, K, N, sizes in cases:
             per_entry = []
-            for E in sizes:
+            points = [(E, N) for E in sizes] if sizes is not None else [(2 * M, n) for n in N]
+            for E, N in points:
                 index = zipf_index(E, N)
                 src = torch.randn((E, K), device=dev)
                 fn = ts.scatter_sum if reduce == "sum" else ts.scatter_max
