@@ -74,6 +74,40 @@ def event_time(fn, iters, warm=3):
     return a.elapsed_time(b) * 1e-3 / iters
 
 
+def graph_time(fn, iters):
+    """Average seconds per call when `iters` calls in a row are captured in one HIP graph (a caller that captures a
+    whole step: no launch gaps between the kernels), the graph replayed four times between two events; None if the
+    call cannot be captured. (A graph of one call alone is slower than eager launches: 28 against 17 us for the
+    small scatter, the cost of starting a graph.)"""
+    import torch
+    try:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(3):
+                fn()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for _ in range(iters):
+                fn()
+        graph.replay()
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(4):
+            graph.replay()
+        b.record()
+        torch.cuda.synchronize()
+        t = a.elapsed_time(b) * 1e-3 / (4 * iters)
+        del graph
+        return t
+    except Exception as e:  # noqa: BLE001 -- a bench row, not a test
+        print(f"[bench] graph capture failed: {e}", file=sys.stderr)
+        return None
+
+
 def cold_time(fn, iters):
     """Median seconds of a call that finds nothing of its inputs in a cache: 1 GiB is written between the
     launches (the memory-side cache holds 256 MB), each launch timed on its own."""
@@ -171,6 +205,17 @@ def bench_csr_config(ts, wl, w, dev, iters, ops, uniform=False, cold=False):
                 elif op == "gather_csr":
                     t = cold_time(lambda: ts.gather_csr(out, indptr, src), max(iters // 2, 5))
                     res[op + "_cold"] = entry(wl.bytes_gather(w.E, w.N, w.K, s), t, EK)
+            # and the same calls replayed from a HIP graph: what a caller with a launch-bound loop gets
+            for op in ops:
+                if op in ("segment_csr_sum", "segment_csr_mean"):
+                    r = op.rsplit("_", 1)[1]
+                    t = graph_time(lambda: ts.segment_csr(src, indptr, out, r), iters)
+                    if t is not None:
+                        res[op + "_graph_replay"] = entry(wl.bytes_segment(w.E, w.N, w.K, s), t, EK)
+                elif op == "gather_csr":
+                    t = graph_time(lambda: ts.gather_csr(out, indptr, src), iters)
+                    if t is not None:
+                        res[op + "_graph_replay"] = entry(wl.bytes_gather(w.E, w.N, w.K, s), t, EK)
     del src, out
     torch.cuda.empty_cache()
     return res
@@ -189,6 +234,10 @@ def bench_scatter_config(ts, wl, w, dev, iters, reduces):
                 if w.E * w.K * 4 < CACHE_BYTES:
                     t = cold_time(lambda: ts.scatter_sum(src, index, 0, None, w.N), max(iters // 2, 5))
                     res["scatter_sum_cold"] = entry(wl.bytes_scatter(w.E, w.N, w.K, 4), t, w.E * w.K)
+                if w.E * w.K * 4 < (64 << 20):   # launch-bound sizes: the same call replayed from a HIP graph
+                    t = graph_time(lambda: ts.scatter_sum(src, index, 0, None, w.N), iters)
+                    if t is not None:
+                        res["scatter_sum_graph_replay"] = entry(wl.bytes_scatter(w.E, w.N, w.K, 4), t, w.E * w.K)
             else:
                 fn = ts.scatter_max if r == "max" else ts.scatter_min
                 t = event_time(lambda: fn(src, index, 0, None, w.N), iters)
