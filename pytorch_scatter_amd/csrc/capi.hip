@@ -140,11 +140,12 @@ int run_csr_reduce_slice(const void *src, const int64_t *indptr, void *out, int6
                          int64_t B, int64_t N, int64_t E, int64_t K, int64_t indptr_batch_stride, int dtype,
                          int reduce, int accumulate, void *ws, size_t ws_bytes, hipStream_t stream,
                          const int32_t *perm, int64_t perm_batch_stride, bool want_perm_args, bool *perm_args_done,
-                         unsigned long long *status, bool status_reset) {
+                         unsigned long long *status, bool status_reset, const int *gate = nullptr,
+                         int scatter_rule = 0) {
   const bool al = aligned16(src) && aligned16(out);
-  // permuted rows always take the wide kernel (the narrow one stages consecutive entries)
+  // permuted rows always take the wide kernel (the narrow one stages consecutive entries), and so does a gated call
   const CsrPlan p = csr_plan(N, E, K, kElemBytes[dtype], al, false, reduce == TS_MIN || reduce == TS_MAX,
-                             perm == nullptr);
+                             perm == nullptr && gate == nullptr && !scatter_rule);
   const CsrWs w = csr_workspace(p, B, K, dtype, reduce);
   if (ws == nullptr || ws_bytes < w.total) return TS_ERR_WORKSPACE;
   CsrReduceArgs a;
@@ -174,6 +175,9 @@ int run_csr_reduce_slice(const void *src, const int64_t *indptr, void *out, int6
   a.carry_spin = env_int("TS_CSR_SPIN", kCarrySpin);  // test aid: -1 makes every look-back give up at once
   a.perm = perm;
   a.perm_batch_stride = perm_batch_stride;
+  a.gate = gate;
+  a.gate_want = 0;
+  a.scatter_rule = scatter_rule;
   // every row is finished inside the first kernel unless the second one runs: then the positions can leave it
   // in src's order right away;
   // when the output is large: the lookup at every row end makes the wavefront wait, a pass over [N, K]
@@ -188,7 +192,7 @@ int run_csr_reduce(const void *src, const int64_t *indptr, void *out, int64_t *a
                    int64_t B, int64_t N, int64_t E, int64_t K, int64_t indptr_batch_stride, int dtype,
                    int reduce, int accumulate, void *ws, size_t ws_bytes, unsigned long long *status,
                    hipStream_t stream, const int32_t *perm = nullptr, int64_t perm_batch_stride = 0,
-                   bool *perm_args_done = nullptr) {
+                   bool *perm_args_done = nullptr, const int *gate = nullptr, int scatter_rule = 0) {
   const int64_t s = kElemBytes[dtype];
   const bool want_perm_args = B * N * K >= ((int64_t)8 << 20);
   // every slice reuses the workspace: the launches follow each other on one stream
@@ -197,8 +201,33 @@ int run_csr_reduce(const void *src, const int64_t *indptr, void *out, int64_t *a
                                 offset_bytes(out, b0 * N * K * s), arg_out ? arg_out + b0 * N * K : nullptr,
                                 offset_bytes(count_out, b0 * N * s), nb, N, E, K, indptr_batch_stride, dtype, reduce,
                                 accumulate, ws, ws_bytes, stream, perm ? perm + b0 * perm_batch_stride : nullptr,
-                                perm_batch_stride, want_perm_args, perm_args_done, status, b0 == 0);
+                                perm_batch_stride, want_perm_args, perm_args_done, status, b0 == 0, gate, scatter_rule);
   });
+}
+
+// A scatter whose index turns out to be sorted (found by the count pass of the buckets) is finished by the
+// segmented reduction instead: sorted index -> row pointers -> one pass over src without atomics, both gated on
+// the device flag. The reduction must finish every row inside its first kernel (look-back), which needs 4- or
+// 8-byte accumulators and at most four column chunks. Extra workspace behind that of the buckets: the row
+// pointers, then the reduction's own.
+struct SortedRoute {
+  bool ok;
+  size_t ptr_bytes, csr_bytes;
+};
+SortedRoute sorted_route_plan(int64_t B, int64_t E, int64_t K, int64_t N, int dtype, int reduce) {
+  SortedRoute r = {false, 0, 0};
+  if (!env_int("TS_SCATTER_SORTED_ROUTE", 1) || !env_int("TS_CSR_LOOKBACK", 1)) return r;
+  if (reduce != TS_SUM && reduce != TS_MIN && reduce != TS_MAX) return r;
+  if (kAccBytes[dtype] < 4 || B < 1 || E < 1) return r;
+  const bool wa = reduce != TS_SUM;
+  for (int al = 0; al < 2; ++al) {
+    const CsrPlan p = csr_plan(N, E, K, kElemBytes[dtype], al != 0, false, wa, false);
+    if (p.small || p.ychunks > 4) return r;
+  }
+  r.ptr_bytes = ((size_t)B * (N + 1) * 8 + 255) & ~(size_t)255;
+  r.csr_bytes = csr_workspace_max(B, N, E, K, dtype, reduce, false) - kStatusBytes;
+  r.ok = true;
+  return r;
 }
 
 int run_csr_gather(int dtype, const CsrGatherArgs &args, const CsrPlan &p, int64_t B, bool divide, hipStream_t s) {
@@ -229,12 +258,12 @@ int run_coo_gather(int dtype, const CooGatherArgs &args, const CooGatherPlan &p,
 
 // sorted index [B, E] -> row pointers [B, N + 1] (contiguous)
 int run_coo_to_indptr(const int64_t *index, int64_t *ptr, int64_t B, int64_t E, int64_t N, int64_t index_batch_stride,
-                      hipStream_t s) {
+                      hipStream_t s, const int *gate = nullptr, int gate_want = 0) {
   const int64_t per_block = (int64_t)kBlock * kCooPtrPerThread;
   return for_batch_slices(B, [&](int64_t b0, int64_t nb) {
     dim3 grid((unsigned)((E + 1 + per_block - 1) / per_block), (unsigned)nb);
     hipLaunchKernelGGL(coo_to_indptr_kernel, grid, dim3(kBlock), 0, s, index + b0 * index_batch_stride,
-                       ptr + b0 * (N + 1), N, E, index_batch_stride);
+                       ptr + b0 * (N + 1), N, E, index_batch_stride, gate, gate_want);
     return hipGetLastError() == hipSuccess ? (int)TS_OK : (int)TS_ERR_LAUNCH;
   });
 }
@@ -466,13 +495,20 @@ size_t ts_scatter_workspace_bytes(int64_t B, int64_t E, int64_t K, int64_t N, in
       if (k1 != 0) return k1;
     }
     const size_t binned = bin_plan(B, E, K, N, kElemBytes[dtype], nullptr, 0, any_size, 8, true).bytes;
-    if (binned != 0) return binned;
+    if (binned != 0) {
+      const SortedRoute sr = sorted_route_plan(B, E, K, N, dtype, reduce);
+      return binned + (sr.ok ? sr.ptr_bytes + sr.csr_bytes : 0);
+    }
     // one flag for the sample of the index that picks the kernel when few entries meet in an output row
     const int probe = env_int("TS_SCATTER_SKEW", 1);
     return probe && skew_probe_shape(B, E, K, N, kElemBytes[dtype], probe == 2) ? 256 : 0;
   }
-  if (reduce == TS_SUM && kAccBytes[dtype] >= 4)  // table slots: int32 for int32, 8 bytes for the other types
-    return bin_plan(B, E, K, N, kElemBytes[dtype], nullptr, 0, any_size, dtype == TS_I32 ? 4 : 8, false, true).bytes;
+  if (reduce == TS_SUM && kAccBytes[dtype] >= 4) {  // table slots: int32 for int32, 8 bytes for the other types
+    const size_t binned = bin_plan(B, E, K, N, kElemBytes[dtype], nullptr, 0, any_size, dtype == TS_I32 ? 4 : 8, false, true).bytes;
+    if (binned == 0) return 0;
+    const SortedRoute sr = sorted_route_plan(B, E, K, N, dtype, reduce);
+    return binned + (sr.ok ? sr.ptr_bytes + sr.csr_bytes : 0);
+  }
   return 0;
 }
 
@@ -525,7 +561,30 @@ int ts_scatter_with_workspace(const void *src, const int64_t *index, void *out, 
   }
   const int full = kVecBytes / kElemBytes[dtype];
   const int vec = (full > 1 && K % full == 0 && aligned16(src)) ? full : 1;
-  return dispatch_scatter(dtype, a, reduce, vec, static_cast<hipStream_t>(stream));
+  // sorted index: finished by the segmented reduction (see sorted_route_plan); its workspace lies behind the buckets'
+  const int *route_flag = nullptr;
+  size_t bin_bytes = 0;
+  SortedRoute sr = {false, 0, 0};
+  if (a.bin_ws != nullptr && !out_given && index_stride_k == 0 && index_stride_e == 1 && B * E * K > 0) {
+    const bool any_size = a.bin_any_size != 0;
+    if (reduce == TS_MIN || reduce == TS_MAX)
+      bin_bytes = kElemBytes[dtype] > 4 ? 0 : bin_plan(B, E, K, N, kElemBytes[dtype], nullptr, 0, any_size, 8, true).bytes;
+    else if (reduce == TS_SUM && kAccBytes[dtype] >= 4)
+      bin_bytes = bin_plan(B, E, K, N, kElemBytes[dtype], nullptr, 0, any_size, dtype == TS_I32 ? 4 : 8, false, true).bytes;
+    if (bin_bytes != 0) sr = sorted_route_plan(B, E, K, N, dtype, reduce);
+    if (sr.ok && workspace_bytes >= bin_bytes + sr.ptr_bytes + sr.csr_bytes) {
+      a.sorted_route = 1;
+      a.route_flag = &route_flag;
+      a.route_ptr = reinterpret_cast<int64_t *>(static_cast<char *>(workspace) + bin_bytes);
+    }
+  }
+  const int rc = dispatch_scatter(dtype, a, reduce, vec, static_cast<hipStream_t>(stream));
+  if (rc != TS_OK || route_flag == nullptr) return rc;
+  // the row pointers of a sorted index come from the place pass of the buckets (bin_place_kernel)
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  return run_csr_reduce(src, a.route_ptr, out, arg_out, nullptr, B, N, E, K, N + 1, dtype, reduce, 0,
+                        static_cast<char *>(workspace) + bin_bytes + sr.ptr_bytes, sr.csr_bytes, nullptr, s, nullptr, 0,
+                        nullptr, route_flag, 1);
 }
 
 int ts_scatter_count(const int64_t *index, float *count, int64_t B, int64_t E, int64_t N,

@@ -323,7 +323,10 @@ template <typename T> int launch_csr_gather(const CsrGatherArgs &a, const CsrPla
 constexpr int kCooPtrPerThread = 4;  // entries per thread: a quarter of the wavefronts to launch
 static __global__ __launch_bounds__(kBlock) void coo_to_indptr_kernel(const int64_t *__restrict__ index,
                                                                int64_t *__restrict__ ptr, int64_t N,
-                                                               int64_t E, int64_t index_batch_stride) {
+                                                               int64_t E, int64_t index_batch_stride,
+                                                               const int *gate = nullptr, int gate_want = 0) {
+  // gate (optional): run only if (*gate != 0) == (gate_want != 0) -- a scatter that found its index sorted
+  if (gate != nullptr && (*gate != 0) != (gate_want != 0)) return;
   const int64_t b = blockIdx.y;
   const int64_t e0 = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * kCooPtrPerThread;
   if (e0 > E) return;

@@ -65,6 +65,13 @@ struct CsrReduceArgs {
                       // scatter's rule for slots that never beat the initial value (no pass over arg_out after it)
   // status word of the call (device memory, may be null): set to 0 by the first tile when status_reset is set,
   // or-ed with kStatusGaveUp by a tile whose look-back ran out of polls
+  // optional gate (a scatter whose index turned out to be sorted takes this reduction instead of the buckets):
+  // the kernel returns at once unless (*gate != 0) == (gate_want != 0). scatter_rule: min / max write a slot whose
+  // entries never beat the initial value of the element type as 0 with position E, as scatter does
+  // (csrc/cpu/scatter_cpu.cpp:81-82). Both need the look-back mode and a call without perm / accumulate.
+  const int *gate = nullptr;
+  int gate_want = 0;
+  int scatter_rule = 0;
   unsigned long long *status;
   int status_reset;
   int carry_spin;     // polls per batch of carry flags before the look-back gives up; < 0: give up without polling
@@ -121,7 +128,8 @@ __device__ __forceinline__ void reduce_step(A &acc, int32_t &arg, A v, int32_t e
 // Write one finished row slice. `count` is the full length of the row.
 // ACCUM: 0 = `out` is overwritten (known at compile time: the row-end code sits in divergent control flow,
 // where every instruction counts), -1 = decided by a.accumulate at run time.
-template <typename T, int VEC, int REDUCE, int ACCUM = -1, bool PERM = false>
+// PERM: 0 rows in place, 1 rows through a.perm, 2 rows in place under a.gate with scatter's rule for min / max
+template <typename T, int VEC, int REDUCE, int ACCUM = -1, int PERM = 0>
 __device__ __forceinline__ void finalize_row_at(const CsrReduceArgs &a, T *op, int64_t *ap, T *count_slot,
                                                 const typename Acc<T>::type *acc, const int32_t *arg,
                                                 int64_t count, const int32_t *perm_b = nullptr) {
@@ -150,14 +158,14 @@ __device__ __forceinline__ void finalize_row_at(const CsrReduceArgs &a, T *op, i
       } else {
         o.v[v] = count > 0 ? from_acc<T>(x) : zero_elem<T>();
         oa[v] = count > 0 ? (int64_t)arg[v] : a.E;
-        if constexpr (PERM) {
-          if (perm_b != nullptr && count > 0) {
+        if constexpr (PERM != 0) {
+          if ((PERM == 2 || perm_b != nullptr) && count > 0) {
             // scatter's view of the slot: the position in src's order, or 0 and E if nothing beat the initial
             // value of the element type (csrc/cpu/scatter_cpu.cpp:81-82)
             const A lim = to_acc<T>(REDUCE == TS_MAX ? ElemLim<T>::lowest() : ElemLim<T>::max());
             const A xv = to_acc<T>(o.v[v]);
             if ((REDUCE == TS_MAX) ? (xv > lim) : (xv < lim)) {
-              oa[v] = perm_b[arg[v]];
+              if (PERM == 1) oa[v] = perm_b[arg[v]];
             } else {
               o.v[v] = zero_elem<T>();
               oa[v] = a.E;
@@ -175,7 +183,7 @@ __device__ __forceinline__ void finalize_row_at(const CsrReduceArgs &a, T *op, i
   if (REDUCE == TS_MEAN && count_slot != nullptr) *count_slot = count_as<T>(count > 0 ? count : 1);
 }
 
-template <typename T, int VEC, int REDUCE, int ACCUM = -1, bool PERM = false>
+template <typename T, int VEC, int REDUCE, int ACCUM = -1, int PERM = 0>
 __device__ __forceinline__ void finalize_row(const CsrReduceArgs &a, T *out_b, int64_t *arg_b,
                                              T *count_b, int64_t row, int64_t col, int lg,
                                              const typename Acc<T>::type *acc, const int32_t *arg,
@@ -190,23 +198,26 @@ __device__ __forceinline__ void finalize_row(const CsrReduceArgs &a, T *out_b, i
 // Workgroups per CU the register allocation aims at: six for sum / mean of 4- and 8-byte types (80 VGPRs;
 // mean would take 82 and drop to five, measured 7 % slower on 146 MB inputs). The other instantiations keep
 // the compiler's choice (forcing five on the 16-bit mean cost 3 % on 16 GB inputs).
-template <typename T, int VEC, int REDUCE, bool PERM = false> constexpr int csr_reduce_min_blocks() {
-  return PERM ? 1 : ((REDUCE == TS_SUM || REDUCE == TS_MEAN) && sizeof(T) >= 4 ? 6 : 1);  // PERM: 8 KB more LDS
+template <typename T, int VEC, int REDUCE, int PERM = 0> constexpr int csr_reduce_min_blocks() {
+  return PERM == 1 ? 1 : ((REDUCE == TS_SUM || REDUCE == TS_MEAN) && sizeof(T) >= 4 ? 6 : 1);  // PERM: 8 KB more LDS
 }
-template <typename T, int VEC, int REDUCE, int ACCUM, bool PERM = false>
+template <typename T, int VEC, int REDUCE, int ACCUM, int PERM = 0>
 __global__ __launch_bounds__(kBlock, (csr_reduce_min_blocks<T, VEC, REDUCE, PERM>())) void csr_reduce_kernel(CsrReduceArgs a) {
   typedef typename Acc<T>::type A;
   constexpr bool kArg = (REDUCE == TS_MIN || REDUCE == TS_MAX);
   constexpr int U = kLoadsInFlight;
 
   __shared__ int32_t s_ptr[kMaxBlockItems + 4];  // row pointers of the tile + one sentinel
-  __shared__ int32_t s_perm[PERM ? kMaxBlockItems : 1];  // source rows of the tile's entries
+  __shared__ int32_t s_perm[PERM == 1 ? kMaxBlockItems : 1];  // source rows of the tile's entries
   __shared__ A s_val[2 * kBlock * VEC];
   __shared__ int32_t s_arg[kArg ? 2 * kBlock * VEC : 1];
   __shared__ int32_t s_head_row[kBlock];    // local row of the head partial, -1: none
   __shared__ int32_t s_head_closes[kBlock];
   __shared__ int32_t s_tail_row[kBlock];    // local row of the tail partial, -1: none
   __shared__ int64_t s_cut[2];
+  if constexpr (PERM == 2) {
+    if (a.gate != nullptr && (*a.gate != 0) != (a.gate_want != 0)) return;  // the same for every wavefront of the grid
+  }
 
   const int tid = threadIdx.x;
   const int G = a.G;
@@ -247,7 +258,7 @@ __global__ __launch_bounds__(kBlock, (csr_reduce_min_blocks<T, VEC, REDUCE, PERM
   for (int t = tid; t < nload; t += kBlock) s_ptr[t] = (int32_t)(ptr[i0 + t] - j0);
   if (tid == 0) { s_ptr[nload] = INT32_MAX; s_ptr[nload + 1] = INT32_MAX; }  // rows past the last one never end
   const int32_t *arg_perm = nullptr;  // set: positions leave the kernel in src's order
-  if constexpr (PERM) {
+  if constexpr (PERM == 1) {
     const int32_t *perm_b = a.perm + b * a.perm_batch_stride;
     const int32_t last_row = a.E > 0 ? (int32_t)(a.E - 1) : 0;
     for (int t = tid; t < ne; t += kBlock) {
@@ -330,7 +341,7 @@ __global__ __launch_bounds__(kBlock, (csr_reduce_min_blocks<T, VEC, REDUCE, PERM
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       int ee = e + u < je1 ? e + u : je1 - 1;
-      const int64_t srow = PERM ? (int64_t)s_perm[ee] : j0 + ee;
+      const int64_t srow = PERM == 1 ? (int64_t)s_perm[ee] : j0 + ee;
       x[u] = load_vec_stream<T, VEC>(src_col + srow * a.K);
     }
   };
@@ -823,7 +834,10 @@ int launch_csr_reduce_t(const CsrReduceArgs &a, const CsrPlan &p, int64_t B, hip
   dim3 grid((unsigned)p.nblk, (unsigned)p.ychunks, (unsigned)B);
   if (a.perm != nullptr) {
     if (a.accumulate) return TS_ERR_UNSUPPORTED;
-    hipLaunchKernelGGL((csr_reduce_kernel<T, VEC, REDUCE, 0, true>), grid, dim3(kBlock), 0, stream, a);
+    hipLaunchKernelGGL((csr_reduce_kernel<T, VEC, REDUCE, 0, 1>), grid, dim3(kBlock), 0, stream, a);
+  } else if (a.gate != nullptr || a.scatter_rule) {
+    if (a.accumulate || !(a.lookback || p.nblk <= 1)) return TS_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL((csr_reduce_kernel<T, VEC, REDUCE, 0, 2>), grid, dim3(kBlock), 0, stream, a);
   } else if (a.accumulate)
     hipLaunchKernelGGL((csr_reduce_kernel<T, VEC, REDUCE, -1>), grid, dim3(kBlock), 0, stream, a);
   else

@@ -215,6 +215,14 @@ struct ScatterArgs {
   int skew_probe = 1;              // min/max: sample the index for skew (needs 256 bytes of workspace): 0 never, 2 at any size
   const int *skew_flag = nullptr;  // min/max kernels behind the probe: run only if (*skew_flag != 0) == (skew_want != 0)
   int skew_want = 0;
+  // A caller that can finish the scatter with the segmented reduction when the index turns out to be sorted
+  // (it launches that reduction afterwards, gated on the flag) sets sorted_route. The launcher then lets the
+  // count pass of the buckets check the whole index (in order, inside [0, N)), reports through *route_flag the
+  // device flag that reads 0 for such an index once the count pass has run, and launches nothing else that
+  // would handle the sorted case; *route_flag stays null when the buckets were not taken.
+  int sorted_route = 0;
+  const int **route_flag = nullptr;
+  int64_t *route_ptr = nullptr;  // [B][N + 1]: the row pointers of a sorted index, written by the place pass
 };
 
 // Inputs for which the min/max launcher samples the index (see index_skew_kernel): rows of 2-256 columns of
@@ -1415,6 +1423,13 @@ __global__ __launch_bounds__(kBlock) void scatter_arg_wide_kernel(ScatterArgs a)
   }
 }
 
+inline unsigned grid_for(int64_t n, int per_thread = 1) {
+  int64_t blocks = (n + (int64_t)kBlock * per_thread - 1) / ((int64_t)kBlock * per_thread);
+  if (blocks < 1) blocks = 1;
+  const int64_t cap = 256 * 32;  // 256 CUs x 32 workgroups: enough to fill the chip, grid-stride beyond
+  return (unsigned)(blocks < cap ? blocks : cap);
+}
+
 }  // namespace ts
 #include "scatter_binned.h"
 #include "scatter_k1.h"
@@ -1431,13 +1446,6 @@ template <typename T>
 __global__ __launch_bounds__(kBlock) void mask_init_kernel(T *p, int64_t n, T init) {
   for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlock)
     if (p[i] == init) p[i] = (T)0;
-}
-
-inline unsigned grid_for(int64_t n, int per_thread = 1) {
-  int64_t blocks = (n + (int64_t)kBlock * per_thread - 1) / ((int64_t)kBlock * per_thread);
-  if (blocks < 1) blocks = 1;
-  const int64_t cap = 256 * 32;  // 256 CUs x 32 workgroups: enough to fill the chip, grid-stride beyond
-  return (unsigned)(blocks < cap ? blocks : cap);
 }
 
 // ---- host side --------------------------------------------------------------------
@@ -1489,20 +1497,32 @@ int launch_scatter_v(const ScatterArgs &args, int reduce, hipStream_t stream) {
   const int64_t n_edges = a.B * a.E;
   const unsigned g_out = grid_for(n_out);
   if (reduce == TS_SUM || reduce == TS_MUL) {
-    if (!a.out_given)
+    // Large inputs with rows of 64 bytes and more, given a workspace: unless the index is sorted (found out by
+    // the first pass), the entries are binned by bucket of output rows and summed in LDS (scatter_binned.h);
+    // the kernels launched below then return at once. A sorted index stays with them: they combine its runs
+    // (or, for a caller with sorted_route, is left to that caller's segmented reduction: then out is cleared
+    // only if the buckets are going to add into it).
+    BinPlan bp;
+    bp.ok = false;
+    int lshift = -1;
+    if constexpr (BinSlotOk<T>::value) {
+      if (reduce == TS_SUM && n_src > 0 && a.bin_ws != nullptr && a.sk == 0 && a.K % VEC == 0) {
+        bp = bin_plan(a.B, a.E, a.K, a.N, (int)sizeof(T), a.bin_ws, a.bin_ws_bytes, a.bin_any_size != 0,
+                      (int)sizeof(typename BinSlot<T>::type), false, true);
+        lshift = bp.ok ? bin_lane_shift(bp.p, VEC) : -1;
+      }
+    }
+    const bool routed = lshift >= 0 && a.sorted_route && a.route_flag != nullptr && !a.out_given;
+    if (!a.out_given && !routed)
       hipLaunchKernelGGL(fill_kernel<T>, dim3(g_out), dim3(kBlock), 0, stream, out, n_out,
                          small_const<T>(reduce == TS_MUL ? 1 : 0));
-    if (reduce == TS_SUM && n_src > 0 && a.bin_ws != nullptr && a.sk == 0 && a.K % VEC == 0) {
-      // Large inputs with rows of 64 bytes and more, given a workspace: unless the index is sorted (found out by
-      // the first pass), the entries are binned by bucket of output rows and summed in LDS (scatter_binned.h);
-      // the kernels launched below then return at once. A sorted index stays with them: they combine its runs.
-      if constexpr (BinSlotOk<T>::value) {
-        const BinPlan bp = bin_plan(a.B, a.E, a.K, a.N, (int)sizeof(T), a.bin_ws, a.bin_ws_bytes, a.bin_any_size != 0,
-                                    (int)sizeof(typename BinSlot<T>::type), false, true);
-        const int lshift = bp.ok ? bin_lane_shift(bp.p, VEC) : -1;
-        if (lshift >= 0) {
-          launch_binned_add<T, VEC>(a, bp.p, lshift, stream);
-          a.skip_flag = bp.p.unsorted;
+    if constexpr (BinSlotOk<T>::value) {
+      if (lshift >= 0) {
+        launch_binned_add<T, VEC>(a, bp.p, lshift, stream, routed ? n_out : 0);
+        a.skip_flag = bp.p.unsorted;
+        if (routed) {
+          *a.route_flag = bp.p.unsorted;
+          return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
         }
       }
     }
@@ -1650,6 +1670,7 @@ int launch_scatter_v(const ScatterArgs &args, int reduce, hipStream_t stream) {
             launch_binned_keys<T, VEC, true>(a, bp.p, stream);
           else
             launch_binned_keys<T, VEC, false>(a, bp.p, stream);
+          if (a.sorted_route && a.route_flag != nullptr) *a.route_flag = bp.p.unsorted;
           return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
         }
       }

@@ -51,6 +51,8 @@ struct BinArgs {
   int *unsorted;           // sum only (else null): set to 1 by the count pass when the index is not sorted;
                            // a sorted index is left to the kernels that combine runs, and the passes after
                            // the count return at once
+  int strict = 0;          // the count pass also reports an index outside [0, N) as unsorted (a caller that hands a
+                           // sorted index to the segmented reduction needs both)
   int sampled = 0;         // sum only: *unsorted was set before the count pass from a sample of the index
                            // (bin_sample_kernel); then the count pass returns at once as well
 };
@@ -172,7 +174,8 @@ constexpr int kBinBatch = kBinPer * kBinPlaceBlock;
 // descent (optional): set when an entry's node lies below that of the entry before it. The entry before is the
 // neighbouring lane's (a shuffle); only the first lane of a wavefront loads it.
 __device__ __forceinline__ void bin_buckets(const ScatterArgs &a, const BinArgs &p, int64_t lo, int64_t hi,
-                                            int32_t *bucket, int32_t *local, bool *descent = nullptr) {
+                                            int32_t *bucket, int32_t *local, bool *descent = nullptr,
+                                            bool strict = false) {
   int64_t node[kBinPer];
 #pragma unroll
   for (int j = 0; j < kBinPer; ++j) {
@@ -180,18 +183,23 @@ __device__ __forceinline__ void bin_buckets(const ScatterArgs &a, const BinArgs 
     node[j] = be < hi ? bin_node(a, be) : -1;
   }
   if (descent != nullptr) {
+    // The entry before a lane's entry is the neighbouring lane's (a shuffle); the first lane of a wavefront needs the
+    // entry before the wavefront's first one. One load instruction fetches those of all kBinPer rows: lane j
+    // loads the entry in front of row j.
     const int lane = threadIdx.x & (kWave - 1);
-    int64_t before[kBinPer];
-#pragma unroll
-    for (int j = 0; j < kBinPer; ++j) {
-      const int64_t be = lo + threadIdx.x + (int64_t)j * kBinPlaceBlock;
-      before[j] = (lane == 0 && be > 0 && be < hi) ? bin_node(a, be - 1) : -1;
+    int64_t edge = -1;
+    if (lane < kBinPer) {
+      const int64_t be = lo + (int64_t)(threadIdx.x - lane) + (int64_t)lane * kBinPlaceBlock;
+      if (be > 0 && be < hi) edge = bin_node(a, be - 1);
     }
 #pragma unroll
     for (int j = 0; j < kBinPer; ++j) {
+      const int elo = __shfl((int)(uint32_t)edge, j), ehi = __shfl((int)(edge >> 32), j);
       const int lo32 = __shfl_up((int)(uint32_t)node[j], 1), hi32 = __shfl_up((int)(node[j] >> 32), 1);
-      const int64_t prev = lane == 0 ? before[j] : (int64_t)(((uint64_t)(uint32_t)hi32 << 32) | (uint32_t)lo32);
+      const int64_t prev = lane == 0 ? (int64_t)(((uint64_t)(uint32_t)ehi << 32) | (uint32_t)elo)
+                                     : (int64_t)(((uint64_t)(uint32_t)hi32 << 32) | (uint32_t)lo32);
       *descent = *descent || (node[j] >= 0 && prev >= 0 && node[j] < prev);
+      if (strict && node[j] < 0 && lo + threadIdx.x + (int64_t)j * kBinPlaceBlock < hi) *descent = true;
     }
   }
 #pragma unroll
@@ -260,7 +268,7 @@ static __global__ __launch_bounds__(kBinPlaceBlock) void bin_count_kernel(Scatte
   bool descent = false;
   for (int64_t b0 = lo; b0 < hi; b0 += kBinBatch) {
     int32_t bucket[kBinPer];
-    bin_buckets(a, p, b0, hi, bucket, nullptr, p.unsorted != nullptr && !p.sampled ? &descent : nullptr);
+    bin_buckets(a, p, b0, hi, bucket, nullptr, p.unsorted != nullptr && !p.sampled ? &descent : nullptr, p.strict != 0);
 #pragma unroll
     for (int j = 0; j < kBinPer; ++j) bin_take(s_hist, bucket[j]);
   }
@@ -286,7 +294,8 @@ static __global__ __launch_bounds__(kBinBlock) void bin_scan_kernel(BinArgs p) {
   __shared__ int32_t s_m[kBinBlock];  // slabs: chunks of buckets with more than one
   __shared__ int32_t s_l[kBinBlock];  // buckets for the combining kernel: those without exactly one chunk,
   __shared__ int32_t s_g[kBinBlock];  // of which more than kCombFew chunks
-  if (p.sampled && *p.unsorted == 0) return;
+  __shared__ int32_t s_cs[kBinMaxBuckets + 1];  // chunk_start, for the search at the end
+  if (p.unsorted != nullptr && *p.unsorted == 0) return;  // sorted: none of the later passes runs
   // a bucket holds fewer than 2^32 entries (the plan refuses larger inputs): 32-bit counts and divisions
   uint32_t t[PER], c[PER];
   int64_t sum_t = 0, sum_c = 0;
@@ -337,6 +346,7 @@ static __global__ __launch_bounds__(kBinBlock) void bin_scan_kernel(BinArgs p) {
       p.starts[i] = run_t;
       p.cursor[i] = (unsigned long long)run_t;
       p.chunk_start[i] = (int32_t)run_c;
+      s_cs[i] = (int32_t)run_c;
       if (p.slab_start != nullptr) {
         p.slab_start[i] = run_m;
         if (c[j] > (uint32_t)kCombFew)
@@ -356,15 +366,14 @@ static __global__ __launch_bounds__(kBinBlock) void bin_scan_kernel(BinArgs p) {
     p.starts[p.nb] = run_t;
     p.chunk_start[p.nb] = (int32_t)run_c;
   }
-  __syncthreads();  // chunk_start is complete (written and read by this one workgroup)
-  __threadfence_block();
+  __syncthreads();  // the chunk starts are complete
   for (int64_t k = threadIdx.x; k < p.max_wgs; k += kBinBlock) {
     int32_t b = -1;
     if (k < all_c) {  // the bucket whose chunks include k: last i with chunk_start[i] <= k
       int lo = 0, hi = p.nb - 1;
       while (lo < hi) {
         const int mid = (lo + hi + 1) >> 1;
-        if (p.chunk_start[mid] <= k) lo = mid; else hi = mid - 1;
+        if (s_cs[mid] <= k) lo = mid; else hi = mid - 1;
       }
       b = lo;
     }
@@ -376,7 +385,29 @@ template <int CAP>
 static __global__ __launch_bounds__(kBinPlaceBlock) void bin_place_kernel(ScatterArgs a, BinArgs p) {
   __shared__ uint32_t s_base[CAP];
   __shared__ int32_t s_cnt[CAP];
-  if (p.unsorted != nullptr && *p.unsorted == 0) return;
+  if (p.unsorted != nullptr && *p.unsorted == 0) {
+    // A sorted index: nothing to place. A caller that finishes it with the segmented reduction gets the row
+    // pointers from this launch instead: ptr[b][r] = first e with index[b][e] >= r (the count pass has checked
+    // that the index is in order and inside [0, N)).
+    if (a.route_ptr != nullptr) {
+#pragma unroll 4
+      for (int j = 0; j < kBinPer; ++j) {
+        const int64_t be = (int64_t)blockIdx.x * kBinPlaceChunk + threadIdx.x + (int64_t)j * kBinPlaceBlock;
+        if (be >= a.B * a.E) break;
+        const int64_t b = be / a.E, e = be - b * a.E;
+        const int64_t *idx = a.index + b * a.sb;
+        int64_t *ptr = a.route_ptr + b * (a.N + 1);
+        int64_t hi = idx[e];
+        int64_t lo = e == 0 ? 0 : idx[e - 1] + 1;
+        if (lo < 0) lo = 0;
+        if (hi > a.N) hi = a.N;
+        for (int64_t r = lo; r <= hi; ++r) ptr[r] = e;
+        if (e == a.E - 1)
+          for (int64_t r = (hi < 0 ? 0 : hi + 1); r <= a.N; ++r) ptr[r] = a.E;
+      }
+    }
+    return;
+  }
   for (int i = threadIdx.x; i < p.nb; i += kBinPlaceBlock) {
     const int32_t h = p.wg_hist[(int64_t)blockIdx.x * p.nb + i];
     s_base[i] = h != 0 ? (uint32_t)atomicAdd(&p.cursor[i], (unsigned long long)h) : 0u;
@@ -476,6 +507,7 @@ template <typename T, bool IS_MAX>
 __global__ __launch_bounds__(kBinBlock) void bin_combine_kernel(ScatterArgs a, BinArgs p) {
   constexpr int W = kBinBlock / kWave;
   __shared__ uint64_t s_part[W][kCombPos];
+  if (p.unsorted != nullptr && *p.unsorted == 0) return;  // sorted index: left to the caller's segmented reduction
   const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
   const int table = (int)a.K << p.rshift;
   const int n_few = p.comb_count[0], n_many = p.comb_count[1];
@@ -534,6 +566,7 @@ __global__ __launch_bounds__(kBinBlock) void bin_reduce_kernel(ScatterArgs a, Bi
   // rows are K + 1 keys apart: with K a multiple of 32 the rows would all start in the same LDS bank and the
   // lanes of a wavefront, which hold the same columns of different rows, would queue up behind each other
   __shared__ uint64_t s_keys[kBinKeys + kBinKeys / 16];
+  if (p.unsorted != nullptr && *p.unsorted == 0) return;
   const int bucket = p.wg_bucket[blockIdx.x];
   if (bucket < 0) return;
   const int K = (int)a.K;
@@ -587,6 +620,7 @@ template <typename T, int VEC, bool IS_MAX>
 __global__ __launch_bounds__(kBinBlock) void bin_reduce_wave_kernel(ScatterArgs a, BinArgs p, int lshift) {
   constexpr int U = 4;  // eight rows in flight per lane: 90 VGPRs, one workgroup per CU, no gain
   __shared__ uint64_t s_keys[kBinKeys + kBinKeys / 16];  // rows K + 1 keys apart (LDS banks, see above)
+  if (p.unsorted != nullptr && *p.unsorted == 0) return;
   const int wg = (int)(blockIdx.x / (unsigned)p.slices), slice = (int)(blockIdx.x - (unsigned)wg * p.slices);
   const int bucket = p.wg_bucket[wg];
   if (bucket < 0) return;
@@ -777,9 +811,12 @@ inline int bin_lane_shift(const BinArgs &p, int vec) {
 template <typename T, int VEC, bool IS_MAX>
 void launch_binned_keys(const ScatterArgs &a, const BinArgs &plan, hipStream_t stream) {
   BinArgs p = plan;
-  p.unsorted = nullptr;  // min / max take this path for sorted indices too
+  if (a.sorted_route && a.route_flag != nullptr)
+    p.strict = 1;          // the count pass checks the index; the caller finishes a sorted one
+  else
+    p.unsorted = nullptr;  // min / max take this path for sorted indices too
   hipLaunchKernelGGL(bin_clear_kernel, dim3((p.nb + kBlock - 1) / kBlock), dim3(kBlock), 0, stream, p.totals, p.nb,
-                     (int *)nullptr);
+                     p.unsorted);
   if (p.nb <= kBinSmallCap)
     hipLaunchKernelGGL(bin_count_kernel<kBinSmallCap>, dim3((unsigned)p.n_place), dim3(kBinPlaceBlock), 0, stream, a, p);
   else
@@ -800,10 +837,23 @@ void launch_binned_keys(const ScatterArgs &a, const BinArgs &plan, hipStream_t s
 
 // sum: count (with the test for a sorted index), scan, place, add. The caller launches its usual sum kernels
 // afterwards with skip_flag = p.unsorted: they run only if the index turned out to be sorted.
+// out[i] = 0 unless the index is sorted (then nobody adds into out: the caller's segmented reduction writes it)
+template <typename T>
+__global__ __launch_bounds__(kBlock) void bin_zero_out_kernel(T *out, int64_t n, const int *unsorted) {
+  if (*unsorted == 0) return;
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlock)
+    out[i] = zero_elem<T>();
+}
+
+// zero_out: elements of out to clear once the count pass has found the index unsorted (0: the caller has cleared it)
 template <typename T, int VEC>
-void launch_binned_add(const ScatterArgs &a, const BinArgs &plan, int lshift, hipStream_t stream) {
+void launch_binned_add(const ScatterArgs &a, const BinArgs &plan, int lshift, hipStream_t stream, int64_t zero_out = 0) {
   BinArgs p = plan;
   p.sampled = a.B * a.E >= 2 * kBinBlock && !getenv("TS_BIN_NO_SAMPLE");  // env: tuning aid (sorted = no descent at all)
+  if (a.sorted_route && a.route_flag != nullptr) {  // the caller's segmented reduction needs the whole index checked
+    p.sampled = 0;
+    p.strict = 1;
+  }
   if (p.sampled) hipLaunchKernelGGL(bin_sample_kernel, dim3(1), dim3(kBinBlock), 0, stream, a, p.unsorted);
   hipLaunchKernelGGL(bin_clear_kernel, dim3((p.nb + kBlock - 1) / kBlock), dim3(kBlock), 0, stream, p.totals, p.nb,
                      p.sampled ? (int *)nullptr : p.unsorted);
@@ -811,6 +861,9 @@ void launch_binned_add(const ScatterArgs &a, const BinArgs &plan, int lshift, hi
     hipLaunchKernelGGL(bin_count_kernel<kBinSmallCap>, dim3((unsigned)p.n_place), dim3(kBinPlaceBlock), 0, stream, a, p);
   else
     hipLaunchKernelGGL(bin_count_kernel<kBinMaxBuckets>, dim3((unsigned)p.n_place), dim3(kBinPlaceBlock), 0, stream, a, p);
+  if (zero_out > 0)
+    hipLaunchKernelGGL(bin_zero_out_kernel<T>, dim3(grid_for(zero_out)), dim3(kBlock), 0, stream, static_cast<T *>(a.out),
+                       zero_out, p.unsorted);
   hipLaunchKernelGGL(bin_scan_kernel, dim3(1), dim3(kBinBlock), 0, stream, p);
   if (p.nb <= kBinSmallCap)  // 64 KB of cursors, two workgroups per CU; above: 128 KB, one
     hipLaunchKernelGGL(bin_place_kernel<kBinSmallCap>, dim3((unsigned)p.n_place), dim3(kBinPlaceBlock), 0, stream, a, p);

@@ -718,6 +718,72 @@ def test_scatter_sum_binned_variant(capi, oracle, shape, kind, dtype, monkeypatc
         assert bool((err <= bound).all()), (kind, out_given, float((err - bound).max()))
 
 
+SORTED_KINDS = ["sorted", "sorted gaps", "one descent", "beyond N", "negative first"]
+
+
+@pytest.mark.parametrize("shape,reduce,kind,dtype", list(product(
+    [(1, 60000, 32, 300), (2, 40000, 16, 700), (1, 20000, 64, 100000), (1, 8000, 1024, 50), (3, 9000, 512, 5)],
+    ["sum", "min", "max"], SORTED_KINDS, [torch.float32, torch.bfloat16, torch.int32])))
+def test_scatter_sorted_index_with_workspace(capi, oracle, shape, reduce, kind, dtype, monkeypatch):
+    """With a workspace, the count pass of the buckets (forced on at these sizes) checks the whole index; one that
+    is in order and inside [0, N) is finished by the segmented reduction (row pointers from the index, one pass
+    over src, no atomics), anything else by the buckets. Both must give scatter's result: values that never beat
+    the initial value of the element type (-inf, lowest()) leave 0 with position E, empty rows too; a single
+    descent, an index beyond N at the end or a negative one in front sends the call down the other path."""
+    monkeypatch.setenv("TS_SCATTER_BINNED", "2")
+    B, E, K, N = shape
+    rng = np.random.default_rng(E + K + len(kind))
+    src = random_values(rng, (B, E, K), dtype, ties=True)
+    if dtype.is_floating_point:
+        src[:, ::7, ::3] = float("-inf") if reduce == "max" else float("inf")
+        src[:, 5::11, 1::2] = torch.finfo(dtype).min if reduce == "max" else torch.finfo(dtype).max
+    elif reduce != "sum":
+        src[:, ::7, ::3] = torch.iinfo(dtype).min if reduce == "max" else torch.iinfo(dtype).max
+    if reduce == "sum" and dtype.is_floating_point:
+        src = torch.from_numpy(rng.standard_normal(size=(B, E, K))).to(dtype)
+    idx = np.sort(rng.integers(0, N, size=E))
+    if kind == "sorted gaps":
+        idx = np.sort(rng.choice(np.arange(0, N, 3), size=E))
+    if kind == "one descent":
+        idx[E // 2], idx[E // 2 + 1] = N - 1, 0
+    if kind == "beyond N":
+        idx[-3:] = N + 5
+    if kind == "negative first":
+        idx[:2] = -1
+    index1 = torch.from_numpy(idx)
+    valid = (index1 >= 0) & (index1 < N)
+    # scatter drops entries whose index lies outside [0, N); positions stay those of the full input
+    safe = torch.where(valid, index1, torch.zeros_like(index1))
+    index = safe.view(1, E, 1).expand(B, E, K)
+    if reduce == "sum":
+        src_ok = torch.where(valid.view(1, E, 1), src, torch.zeros_like(src))
+        out = torch.full((B, N, K), 9, dtype=dtype, device=DEV)
+        capi.scatter_with_workspace(src.to(DEV), index1.to(DEV), out, None, B, E, K, N, 0, 1, 0, capi.SUM, 0)
+        torch.cuda.synchronize()
+        if not dtype.is_floating_point:
+            assert_exact(out, oracle.scatter(src_ok, index, 1, None, N, "sum")[0], kind)
+            return
+        exact = oracle.scatter(src_ok.double(), index, 1, None, N, "sum")[0]
+        absum = oracle.scatter(src_ok.double().abs(), index, 1, None, N, "sum")[0]
+        if dtype == torch.bfloat16:
+            assert_sum16_no_worse_than_reference(oracle, out, src_ok, index, safe, N, 1, exact, None, kind)
+        else:
+            err = (out.cpu().double() - exact).abs()
+            assert bool((err <= RTOL[dtype] * (exact.abs() + absum) + 1e-30).all()), kind
+        return
+    # min / max: an entry outside [0, N) must not win, so give it the value that never does
+    lose = (torch.finfo(dtype).min if reduce == "max" else torch.finfo(dtype).max) if dtype.is_floating_point else \
+        (torch.iinfo(dtype).min if reduce == "max" else torch.iinfo(dtype).max)
+    src_ok = torch.where(valid.view(1, E, 1), src, torch.full_like(src, lose))
+    want, want_arg = oracle.scatter(src_ok, index, 1, None, N, reduce)
+    out = torch.empty((B, N, K), dtype=dtype, device=DEV)
+    arg = torch.empty((B, N, K), dtype=torch.long, device=DEV)
+    capi.scatter_with_workspace(src.to(DEV), index1.to(DEV), out, arg, B, E, K, N, 0, 1, 0, capi.REDUCE[reduce], 0)
+    torch.cuda.synchronize()
+    assert_exact(out, want, kind)
+    assert_exact(arg, want_arg, kind + " arg")
+
+
 @pytest.mark.parametrize("shape,dtype", product(
     [(1, 30000, 1, 500), (1, 9000, 32, 300), (2, 5000, 8, 40), (1, 4000, 12, 70000)],
     [torch.float32, torch.bfloat16, torch.float16]))
