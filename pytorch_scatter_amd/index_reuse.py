@@ -12,7 +12,18 @@ no atomics, the same bits on every call. The cache keeps a reference to every
 index it has seen, so an address cannot come back with other contents, and an
 in-place change of an index bumps its version counter and with it the key.
 Sums of 16-bit floats accumulate in fp32 on this path (``scatter`` adds in the
-element type).
+element type), so a result can change in its last bits between the first calls
+(atomic kernels) and the later ones (plan).
+
+Caveats. The key is an identity, not a checksum. Writes that do not bump the
+version counter leave a stale plan behind, and every later call silently uses
+the old permutation: ``index.data.copy_(...)``, in-place updates through a
+``detach()``-ed alias, writes through a raw pointer or a DLPack capsule, custom
+operators that take ``data_ptr()``. After such a write call
+:func:`disable_index_reuse` (and enable again), use a fresh tensor, or pass an
+explicit :class:`~pytorch_scatter_amd.index_format.SortedIndex` to
+``scatter_sorted``. The cache holds strong references to at most ``max_plans``
+index tensors; their device memory stays allocated while they are cached.
 """
 import os
 from collections import OrderedDict
