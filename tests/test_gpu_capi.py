@@ -784,6 +784,43 @@ def test_scatter_sorted_index_with_workspace(capi, oracle, shape, reduce, kind, 
     assert_exact(arg, want_arg, kind + " arg")
 
 
+@pytest.mark.parametrize("reduce,dtype", product(["sum", "max"], [torch.float32, torch.float64, torch.int32]))
+def test_scatter_sorted_index_per_batch_rows(capi, oracle, reduce, dtype, monkeypatch):
+    """A batched index [B, E] whose rows are sorted one by one (different rows per batch, stride E): in order as a
+    whole for the count pass of the buckets, row pointers per batch for the segmented reduction. The second batch
+    row of the last case has one descent: the whole call then goes through the buckets."""
+    monkeypatch.setenv("TS_SCATTER_BINNED", "2")
+    B, E, K, N = 3, 30000, 32, 900
+    rng = np.random.default_rng(K + len(reduce))
+    for descent in (False, True):
+        idx = np.sort(rng.integers(0, N, size=(B, E)), axis=1)
+        if descent:
+            idx[1, E // 3], idx[1, E // 3 + 1] = N - 1, 0
+        index2 = torch.from_numpy(idx)
+        index = index2.view(B, E, 1).expand(B, E, K)
+        if dtype.is_floating_point and reduce == "sum":
+            src = torch.from_numpy(rng.standard_normal(size=(B, E, K))).to(dtype)
+        else:
+            src = random_values(rng, (B, E, K), dtype, ties=True)
+        out = torch.full((B, N, K), 9, dtype=dtype, device=DEV)
+        arg = torch.empty((B, N, K), dtype=torch.long, device=DEV) if reduce == "max" else None
+        if dtype == torch.float64 and reduce == "max":
+            continue  # 64-bit elements keep the two-pass kernels (no packed keys, no workspace)
+        capi.scatter_with_workspace(src.to(DEV), index2.to(DEV), out, arg, B, E, K, N, E, 1, 0, capi.REDUCE[reduce], 0)
+        torch.cuda.synchronize()
+        want, want_arg = oracle.scatter(src, index, 1, None, N, reduce)
+        if reduce == "max":
+            assert_exact(out, want, f"descent={descent}")
+            assert_exact(arg, want_arg, f"descent={descent} arg")
+        elif not dtype.is_floating_point:
+            assert_exact(out, want, f"descent={descent}")
+        else:
+            exact = oracle.scatter(src.double(), index, 1, None, N, "sum")[0]
+            absum = oracle.scatter(src.double().abs(), index, 1, None, N, "sum")[0]
+            err = (out.cpu().double() - exact).abs()
+            assert bool((err <= RTOL[dtype] * (exact.abs() + absum) + 1e-30).all()), descent
+
+
 @pytest.mark.parametrize("shape,dtype", product(
     [(1, 30000, 1, 500), (1, 9000, 32, 300), (2, 5000, 8, 40), (1, 4000, 12, 70000)],
     [torch.float32, torch.bfloat16, torch.float16]))

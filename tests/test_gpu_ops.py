@@ -503,3 +503,44 @@ def test_segment_csr_with_100000_leading_rows(ts):
     want, want_arg = ts_oracle.segment_csr(src, indptr, None, "max")
     assert torch.equal(got.cpu(), want) and torch.equal(arg.cpu(), want_arg)
     assert torch.equal(ts.gather_csr(got, indptr.to(DEV)).cpu(), ts_oracle.gather_csr(want, indptr))
+
+
+@pytest.mark.parametrize("reduce", ["sum", "mean", "min", "max"])
+def test_scatter_large_sorted_index_through_the_operators(ts, oracle, reduce):
+    """77 MB of 128-byte rows under a sorted index with gaps: above the sizes from which the operators hand the
+    scatter kernels a workspace, where the count pass of the buckets finds the index in order and the segmented
+    reduction finishes the call. Same results as the oracle (sums in another order of additions), -inf entries
+    and empty rows included, and the backward through arg / the index. The same index with two entries swapped
+    goes through the buckets and gives the same values."""
+    g = torch.Generator().manual_seed(11)
+    E, K, N = 600_000, 32, 20_000
+    index = torch.sort(torch.randint(0, N // 2, (E,), generator=g) * 2)[0]
+    src = torch.randint(-8, 9, (E, K), generator=g).float()
+    src[::13, ::5] = float("-inf") if reduce == "max" else (float("inf") if reduce == "min" else 1.0)
+    want = oracle.op_scatter(src, index, 0, None, N, reduce)
+    for swapped in (False, True):
+        idx = index.clone()
+        s = src
+        if swapped:
+            # the two entries change places together with their rows: the same scatter, no longer in order
+            i, j = E // 2, E // 2 + 40
+            perm = torch.arange(E)
+            perm[i], perm[j] = j, i
+            idx, s = index[perm], src[perm]
+        x = s.to(DEV).requires_grad_(reduce in ("sum", "mean"))
+        got = getattr(ts, "scatter_" + reduce)(x, idx.to(DEV), 0, None, N)
+        if reduce in ("min", "max"):
+            assert torch.equal(got[0].cpu(), want[0]), swapped
+            if not swapped:
+                assert torch.equal(got[1].cpu(), want[1])
+            else:  # positions follow the entries that changed places
+                ref = want[1].clone()
+                ref[want[1] == i], ref[want[1] == j] = j, i
+                assert torch.equal(got[1].cpu(), ref)
+        else:
+            assert torch.allclose(got.detach().cpu(), want, rtol=1e-5, atol=1e-4), swapped
+            grad = torch.randn(N, K, generator=g)
+            got.backward(grad.to(DEV))
+            count = torch.bincount(idx, minlength=N).clamp(min=1).float().view(-1, 1)
+            expect = (grad / count if reduce == "mean" else grad)[idx]
+            assert torch.allclose(x.grad.cpu(), expect, rtol=1e-6, atol=1e-7)
