@@ -852,7 +852,14 @@ inline RunGrid run_grid(int64_t n_edges, int64_t kc, int c, int lane_bytes) {
   while ((1 << g.lshift) < kc && g.lshift < 6) ++g.lshift;
   const int L = 1 << g.lshift, epr = kWave >> g.lshift;
   g.hot_rlog = -1;
-  if (c > 0 && n_edges >= ((int64_t)1 << 18) && !getenv("TS_SCATTER_NO_HOT")) {  // env: tuning aid
+  // The table from 2^18 entries on; for rows of 128 bytes and more from 2^15. Below, a hub serialises the atomics of
+  // its row (Zipf(1.2) index, 32 k - 262 k entries of 32 / 64 floats: 120 - 1040 us without the table, 42 - 270 us
+  // with it), while a uniform index pays the tag look-ups (+10-18 %, 3-7 us at these sizes). Narrower rows keep 2^18:
+  // 200 k entries of 16 floats under a uniform index 16.4 us without, 22.7 us with the table (536 against 159 us
+  // under the Zipf index: the known cliff of small skewed sums of narrow rows).
+  int64_t hot_min = run_is_serial(g.lshift, lane_bytes) ? (int64_t)1 << 15 : (int64_t)1 << 18;
+  if (const char *env = getenv("TS_SCATTER_HOT_MIN")) hot_min = atoll(env);  // tuning aid
+  if (c > 0 && n_edges >= hot_min && !getenv("TS_SCATTER_NO_HOT")) {  // env: tuning aid
     int cshift = 0;
     while ((1 << cshift) < c) ++cshift;
     g.hot_rlog = hot_rows_log(g.lshift + cshift);
