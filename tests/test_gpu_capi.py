@@ -821,6 +821,72 @@ def test_scatter_sorted_index_per_batch_rows(capi, oracle, reduce, dtype, monkey
             assert bool((err <= RTOL[dtype] * (exact.abs() + absum) + 1e-30).all()), descent
 
 
+@pytest.mark.parametrize("seed", [1, 2, 3])
+def test_scatter_with_workspace_agrees_with_plain_scatter_on_random_shapes(capi, seed, monkeypatch):
+    """Forty random calls per seed (1-3 batches, 4-1024 columns, 1 - 1.2 M output rows, seven element types, uniform /
+    Zipf / sorted / sorted with entries outside [0, N) / one descent / three distinct values, with and without a
+    given out), buckets forced on: min / max with a workspace (buckets, column slices, slabs, the segmented
+    reduction for a sorted index) give the bits of the call without workspace; floating sums stay within
+    4 * min(n, 128) half-ulp roundings of the exact sum."""
+    monkeypatch.setenv("TS_SCATTER_BINNED", "2")
+    rng = np.random.default_rng(seed)
+    dtypes = [torch.float32, torch.bfloat16, torch.float16, torch.int32, torch.int16, torch.int8, torch.uint8]
+    for case in range(40):
+        dtype = dtypes[rng.integers(len(dtypes))]
+        reduce = ["sum", "min", "max"][rng.integers(3)]
+        B = int(rng.choice([1, 1, 1, 2, 3]))
+        K = int(rng.choice([4, 8, 16, 24, 32, 48, 64, 96, 128, 256, 384, 512, 1024]))
+        E = int(rng.integers(1, 60000))
+        N = int(rng.choice([1, 7, 300, 5000, 70000, 300000, 1200000]))
+        N = min(N, max(int(3e8 // (B * K)), 1))
+        E = min(E, max(int(3e8 // (B * K)), 1))
+        kind = ["uniform", "zipf", "sorted", "sorted-oor", "one-descent", "few-values"][rng.integers(6)]
+        if kind == "zipf":
+            idx = np.minimum(rng.zipf(1.3, size=E) - 1, N - 1)
+        elif kind == "few-values":
+            idx = rng.integers(0, min(N, 3), size=E)
+        else:
+            idx = rng.integers(0, N, size=E)
+        if kind.startswith("sorted") or kind == "one-descent":
+            idx = np.sort(idx)
+        if kind == "sorted-oor" and E > 3:
+            idx[-2:] = N + 3
+            idx[0] = -5
+        if kind == "one-descent" and E > 4:
+            idx[E // 2], idx[E // 2 + 1] = N - 1, 0
+        index = torch.from_numpy(idx.astype(np.int64)).to(DEV)
+        what = (case, dtype, reduce, B, E, K, N, kind)
+        if dtype.is_floating_point and reduce == "sum":
+            src = torch.from_numpy(rng.standard_normal(size=(B, E, K))).to(dtype).to(DEV)
+        else:
+            v = rng.integers(-8, 9, size=(B, E, K))
+            src = torch.from_numpy(np.abs(v) if dtype == torch.uint8 else v).to(dtype).to(DEV)
+            if dtype.is_floating_point:
+                src[:, ::5, ::3] = float("-inf") if reduce == "max" else float("inf")
+        out_given = bool(rng.integers(2)) and reduce != "sum"
+        prev = torch.from_numpy(rng.integers(-3, 4, size=(B, N, K))).to(dtype).to(DEV) if out_given else None
+        res = []
+        for fn in (capi.scatter, capi.scatter_with_workspace):
+            out = prev.clone() if out_given else torch.full((B, N, K), 9, dtype=dtype, device=DEV)
+            arg = torch.full((B, N, K), -7, dtype=torch.long, device=DEV) if reduce != "sum" else None
+            fn(src, index, out, arg, B, E, K, N, 0, 1, 0, capi.REDUCE[reduce], out_given)
+            torch.cuda.synchronize()
+            res.append((out, arg))
+        (o0, a0), (o1, a1) = res
+        if reduce == "sum" and dtype.is_floating_point:
+            valid = (index >= 0) & (index < N)
+            vi = index[valid]
+            exact = torch.zeros((B, N, K), dtype=torch.double, device=DEV).index_add_(1, vi, src[:, valid].double())
+            sq = torch.zeros((B, N, K), dtype=torch.double, device=DEV).index_add_(1, vi, src[:, valid].double() ** 2)
+            n_row = torch.bincount(vi, minlength=N).double().clamp(min=1, max=128).view(1, N, 1)
+            u = {torch.float32: 2.0 ** -24, torch.bfloat16: 2.0 ** -9, torch.float16: 2.0 ** -12}[dtype]
+            bound = u * 4 * n_row * torch.maximum(exact.abs(), sq.sqrt()) + 1e-30
+            assert bool(((o1.double() - exact).abs() <= bound).all()), what
+        else:
+            assert torch.equal(o0, o1), what
+            assert a0 is None or torch.equal(a0, a1), what
+
+
 @pytest.mark.parametrize("shape,dtype", product(
     [(1, 30000, 1, 500), (1, 9000, 32, 300), (2, 5000, 8, 40), (1, 4000, 12, 70000)],
     [torch.float32, torch.bfloat16, torch.float16]))
