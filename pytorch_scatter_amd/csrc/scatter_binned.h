@@ -171,10 +171,10 @@ constexpr int kBinPer = 16;  // entries per lane and batch in count / place (all
 constexpr int kBinBatch = kBinPer * kBinPlaceBlock;
 
 // buckets of the kBinPer entries of a lane, all index loads in flight at once; -1: no bucket
-// descent (optional): set when an entry's node lies below that of the entry before it. The entry before is the
+// check: descent is set when an entry's node lies below that of the entry before it. The entry before is the
 // neighbouring lane's (a shuffle); only the first lane of a wavefront loads it.
 __device__ __forceinline__ void bin_buckets(const ScatterArgs &a, const BinArgs &p, int64_t lo, int64_t hi,
-                                            int32_t *bucket, int32_t *local, bool *descent = nullptr,
+                                            int32_t *bucket, int32_t *local, bool check, bool &descent,
                                             bool strict = false) {
   int64_t node[kBinPer];
 #pragma unroll
@@ -182,7 +182,7 @@ __device__ __forceinline__ void bin_buckets(const ScatterArgs &a, const BinArgs 
     const int64_t be = lo + threadIdx.x + (int64_t)j * kBinPlaceBlock;
     node[j] = be < hi ? bin_node(a, be) : -1;
   }
-  if (descent != nullptr) {
+  if (check) {
     // The entry before a lane's entry is the neighbouring lane's (a shuffle); the first lane of a wavefront needs the
     // entry before the wavefront's first one. One load instruction fetches those of all kBinPer rows: lane j
     // loads the entry in front of row j.
@@ -198,8 +198,8 @@ __device__ __forceinline__ void bin_buckets(const ScatterArgs &a, const BinArgs 
       const int lo32 = __shfl_up((int)(uint32_t)node[j], 1), hi32 = __shfl_up((int)(node[j] >> 32), 1);
       const int64_t prev = lane == 0 ? (int64_t)(((uint64_t)(uint32_t)ehi << 32) | (uint32_t)elo)
                                      : (int64_t)(((uint64_t)(uint32_t)hi32 << 32) | (uint32_t)lo32);
-      *descent = *descent || (node[j] >= 0 && prev >= 0 && node[j] < prev);
-      if (strict && node[j] < 0 && lo + threadIdx.x + (int64_t)j * kBinPlaceBlock < hi) *descent = true;
+      descent = descent || (node[j] >= 0 && prev >= 0 && node[j] < prev);
+      if (strict && node[j] < 0 && lo + threadIdx.x + (int64_t)j * kBinPlaceBlock < hi) descent = true;
     }
   }
 #pragma unroll
@@ -255,8 +255,10 @@ static __global__ __launch_bounds__(kBinBlock) void bin_sample_kernel(ScatterArg
   if (threadIdx.x == 0) *flag = s_desc * 64 >= kBinBlock ? 1 : 0;
 }
 
+// 72 scalar registers at most: with 92 (the two argument structs) a SIMD holds seven of these wavefronts instead of
+// eight, which is one 1024-lane workgroup per CU instead of two (SPI_RA_SGPR_SIMD_FULL was the stall; 52 -> 44 us)
 template <int CAP>
-static __global__ __launch_bounds__(kBinPlaceBlock) void bin_count_kernel(ScatterArgs a, BinArgs p) {
+static __global__ __launch_bounds__(kBinPlaceBlock) __attribute__((amdgpu_num_sgpr(72))) void bin_count_kernel(ScatterArgs a, BinArgs p) {
   __shared__ int32_t s_hist[CAP];
   __shared__ int s_hist_flag;
   if (p.sampled && *p.unsorted == 0) return;
@@ -268,7 +270,7 @@ static __global__ __launch_bounds__(kBinPlaceBlock) void bin_count_kernel(Scatte
   bool descent = false;
   for (int64_t b0 = lo; b0 < hi; b0 += kBinBatch) {
     int32_t bucket[kBinPer];
-    bin_buckets(a, p, b0, hi, bucket, nullptr, p.unsorted != nullptr && !p.sampled ? &descent : nullptr, p.strict != 0);
+    bin_buckets(a, p, b0, hi, bucket, nullptr, p.unsorted != nullptr && !p.sampled, descent, p.strict != 0);
 #pragma unroll
     for (int j = 0; j < kBinPer; ++j) bin_take(s_hist, bucket[j]);
   }
@@ -424,7 +426,8 @@ static __global__ __launch_bounds__(kBinPlaceBlock) void bin_place_kernel(Scatte
   const int64_t hi = lo + kBinPlaceChunk < a.B * a.E ? lo + kBinPlaceChunk : a.B * a.E;
   for (int64_t b0 = lo; b0 < hi; b0 += kBinBatch) {
     int32_t bucket[kBinPer], local[kBinPer];
-    bin_buckets(a, p, b0, hi, bucket, local);
+    bool unused = false;
+    bin_buckets(a, p, b0, hi, bucket, local, false, unused);
 #pragma unroll
     for (int j = 0; j < kBinPer; ++j) {
       const int32_t rank = bin_take(s_cnt, bucket[j]);
