@@ -5,9 +5,11 @@
 // entries are first binned by bucket of R consecutive output rows, R * K keys = 64 KB of LDS, so that a
 // workgroup which reduces (a chunk of) one bucket holds every row it can meet: no misses, no tags, and the
 // only traffic besides the stream is the table written back once per chunk.
-//   count  : per workgroup, a histogram of its entries over the buckets (LDS), added to the bucket totals
+//   count  : at most 512 workgroups with equal shares of the index, each a histogram over the buckets in LDS that
+//            it adds to the bucket totals (also: is the index in order?)
 //   scan   : bucket starts, chunks per bucket, the (bucket, chunk) of every reducing workgroup
-//   place  : every entry -> (row inside its bucket, entry number) at its bucket's next free slot (8 bytes)
+//   place  : a workgroup per tile of the index: its own histogram again, one atomic per bucket reserves the tile's
+//            run of slots, every entry -> (row inside its bucket, entry number) in its run (8 bytes)
 //   reduce : a workgroup per chunk of a bucket: rows of src by entry number, packed keys into the LDS table,
 //            table -> global table with a read before each atomic
 // The order inside a bucket is whatever the placement gives; the packed keys carry the positions, so the result
@@ -22,7 +24,7 @@ constexpr int kBinBlock = 1024;
 constexpr int kBinMaxBuckets = 16384;  // LDS histogram of count / place (their LDS is sized for 8192 or 16384 buckets)
 constexpr int kBinSmallCap = 8192;
 constexpr int kBinChunk = 8192;       // entries per chunk of a bucket in reduce (fewer for inputs under 4 M entries)
-constexpr int kBinPlaceChunk = 16384;  // entries per workgroup in count / place: one batch of 16 per lane
+constexpr int kBinPlaceChunk = 16384;  // most entries per workgroup in place: one batch of 16 per lane
 constexpr int kCombPos = 64;          // combining kernel: keys per step of a bucket of many chunks,
 constexpr int kCombFew = 32;          // many: more than this
 constexpr int kBinPlaceBlock = 1024;   // (measured slower: 256 lanes x 4 batches, 64 K entries per workgroup, 8 K)
@@ -33,14 +35,14 @@ struct BinArgs {
   int slices;              // K / kc: reducing workgroups per chunk, each on its own columns of the same entries
   int chunk;               // entries per reducing workgroup
   int nb;                  // buckets
-  int64_t n_place;         // workgroups of count / place
+  int place_tile;          // entries per workgroup of place: a multiple of 1024, one batch at most
+  int64_t n_place;         // workgroups of place
   int64_t max_wgs;         // workgroups of reduce (upper bound of the chunks)
   unsigned long long *totals;  // [nb] entries per bucket
   unsigned long long *cursor;  // [nb] next free slot
   int64_t *starts;         // [nb + 1]
   int32_t *chunk_start;    // [nb + 1]
   int32_t *wg_bucket;      // [max_wgs] bucket of a reducing workgroup, -1: none
-  int32_t *wg_hist;        // [n_place][nb]
   uint64_t *binned;        // [B * E] (row in bucket << 32) | entry number
   int32_t *slab_start;     // min / max: [nb + 1] first slab of a bucket that is reduced in more than one chunk
   uint64_t *slabs;         // min / max: [slab][K << rshift] the tables of those chunks
@@ -114,7 +116,19 @@ inline BinPlan bin_plan(int64_t B, int64_t E, int64_t K, int64_t N, int elem_byt
   p.kc = (int)kc;
   p.slices = (int)(K / kc);
   p.nb = (int)nb;
-  p.n_place = (n_edges + kBinPlaceChunk - 1) / kBinPlaceChunk;
+  // Place: a workgroup holds its tile in registers (up to 16 entries per lane). Two workgroups fit a CU, so the
+  // tiles are sized for a whole number of rounds of 512 workgroups (10 M entries in tiles of 16384: 611 workgroups,
+  // a round of 512 and a round of 99 that takes as long).
+  {
+    const int64_t rounds = (n_edges + (int64_t)512 * kBinPlaceChunk - 1) / ((int64_t)512 * kBinPlaceChunk);
+    int64_t tile = (((n_edges + 512 * rounds - 1) / (512 * rounds)) + kBinPlaceBlock - 1) & ~(int64_t)(kBinPlaceBlock - 1);
+    if (const char *env = getenv("TS_BIN_PLACE_TILE")) tile = atoi(env);  // tuning aid
+    if (tile < kBinPlaceBlock) tile = kBinPlaceBlock;
+    if (tile > kBinPlaceChunk) tile = kBinPlaceChunk;
+    tile &= ~(int64_t)(kBinPlaceBlock - 1);
+    p.place_tile = (int)tile;
+    p.n_place = (n_edges + tile - 1) / tile;
+  }
   // A reducing workgroup walks its chunk in steps of a few rows per lane group, each step a memory latency:
   // 8 K entries take it about 200 us whatever the input, which is fine once there are a few workgroups per CU
   // (4 M entries and more) and far too long for a smaller input. Those get shorter chunks: about 512 workgroups.
@@ -135,7 +149,7 @@ inline BinPlan bin_plan(int64_t B, int64_t E, int64_t K, int64_t N, int elem_byt
   auto take = [&](size_t bytes) { const size_t o = off; off += up(bytes); return o; };
   const size_t o_tot = take((size_t)nb * 8), o_cur = take((size_t)nb * 8), o_st = take((size_t)(nb + 1) * 8);
   const size_t o_cs = take((size_t)(nb + 1) * 4), o_wb = take((size_t)p.max_wgs * 4);
-  const size_t o_wh = take((size_t)p.n_place * nb * 4), o_bin = take((size_t)n_edges * 8), o_flag = take(256);
+  const size_t o_bin = take((size_t)n_edges * 8), o_flag = take(256);
   // A bucket with m >= 2 chunks holds more than (m - 1) * chunk entries: at most 2 * n_edges / chunk slabs in all.
   const int64_t n_slabs = slabs ? 2 * (n_edges / chunk) + 2 : 0;
   const size_t o_ss = take(slabs ? (size_t)(nb + 1) * 4 : 0), o_cl = take(slabs ? (size_t)(nb + 2) * 4 : 0);
@@ -148,7 +162,6 @@ inline BinPlan bin_plan(int64_t B, int64_t E, int64_t K, int64_t N, int elem_byt
   p.starts = reinterpret_cast<int64_t *>(base + o_st);
   p.chunk_start = reinterpret_cast<int32_t *>(base + o_cs);
   p.wg_bucket = reinterpret_cast<int32_t *>(base + o_wb);
-  p.wg_hist = reinterpret_cast<int32_t *>(base + o_wh);
   p.binned = reinterpret_cast<uint64_t *>(base + o_bin);
   p.unsorted = reinterpret_cast<int *>(base + o_flag);  // callers that do not want the check set it to null
   p.slab_start = slabs ? reinterpret_cast<int32_t *>(base + o_ss) : nullptr;
@@ -255,8 +268,15 @@ static __global__ __launch_bounds__(kBinBlock) void bin_sample_kernel(ScatterArg
   if (threadIdx.x == 0) *flag = s_desc * 64 >= kBinBlock ? 1 : 0;
 }
 
+// Count pass: entries per bucket (and, for callers that ask, whether the index is in order and inside [0, N)).
+// At most two workgroups per CU, each with an equal share of the entries, which it walks in batches of four
+// entries per lane with the loads of the next batch in flight while this one is counted (a workgroup per 16384
+// entries ran in rounds: 611 workgroups = 512 + 99, every one loading, then counting, then writing: 44 us).
 // 72 scalar registers at most: with 92 (the two argument structs) a SIMD holds seven of these wavefronts instead of
-// eight, which is one 1024-lane workgroup per CU instead of two (SPI_RA_SGPR_SIMD_FULL was the stall; 52 -> 44 us)
+// eight, which is one 1024-lane workgroup per CU instead of two (SPI_RA_SGPR_SIMD_FULL was the stall counter).
+constexpr int kBinCountPer = 4;
+constexpr int kBinCountBatch = kBinCountPer * kBinPlaceBlock;
+constexpr int kBinCountGroups = 512;
 template <int CAP>
 static __global__ __launch_bounds__(kBinPlaceBlock) __attribute__((amdgpu_num_sgpr(72))) void bin_count_kernel(ScatterArgs a, BinArgs p) {
   __shared__ int32_t s_hist[CAP];
@@ -265,25 +285,58 @@ static __global__ __launch_bounds__(kBinPlaceBlock) __attribute__((amdgpu_num_sg
   for (int i = threadIdx.x; i < p.nb; i += kBinPlaceBlock) s_hist[i] = 0;
   if (threadIdx.x == 0) s_hist_flag = 0;
   __syncthreads();
-  const int64_t lo = (int64_t)blockIdx.x * kBinPlaceChunk;
-  const int64_t hi = lo + kBinPlaceChunk < a.B * a.E ? lo + kBinPlaceChunk : a.B * a.E;
-  bool descent = false;
-  for (int64_t b0 = lo; b0 < hi; b0 += kBinBatch) {
-    int32_t bucket[kBinPer];
-    bin_buckets(a, p, b0, hi, bucket, nullptr, p.unsorted != nullptr && !p.sampled, descent, p.strict != 0);
+  const int64_t n = a.B * a.E;
+  const int64_t per = (n + gridDim.x - 1) / gridDim.x;
+  const int64_t lo = (int64_t)blockIdx.x * per;
+  const int64_t hi = lo + per < n ? lo + per : n;
+  const bool check = p.unsorted != nullptr && !p.sampled;
+  const bool strict = p.strict != 0;
+  const int lane = threadIdx.x & (kWave - 1);
+  int64_t node[kBinCountPer], next[kBinCountPer];
+  auto load = [&](int64_t b0, int64_t *x) {
 #pragma unroll
-    for (int j = 0; j < kBinPer; ++j) bin_take(s_hist, bucket[j]);
+    for (int j = 0; j < kBinCountPer; ++j) {
+      const int64_t be = b0 + threadIdx.x + (int64_t)j * kBinPlaceBlock;
+      x[j] = be < hi ? bin_node(a, be) : -1;
+    }
+  };
+  bool descent = false;
+  if (lo < hi) load(lo, node);
+  for (int64_t b0 = lo; b0 < hi; b0 += kBinCountBatch) {
+    load(b0 + kBinCountBatch, next);  // unconditional: past the end every lane gets -1 without a load
+    if (check) {
+      // The entry before a lane's entry is the neighbouring lane's (a shuffle); the first lane of a wavefront needs
+      // the entry before the wavefront's first one: lane j loads it for row j (one load instruction for all rows).
+      int64_t edge = -1;
+      if (lane < kBinCountPer) {
+        const int64_t be = b0 + (int64_t)(threadIdx.x - lane) + (int64_t)lane * kBinPlaceBlock;
+        if (be > 0 && be < hi) edge = bin_node(a, be - 1);
+      }
+#pragma unroll
+      for (int j = 0; j < kBinCountPer; ++j) {
+        const int elo = __shfl((int)(uint32_t)edge, j), ehi = __shfl((int)(edge >> 32), j);
+        const int lo32 = __shfl_up((int)(uint32_t)node[j], 1), hi32 = __shfl_up((int)(node[j] >> 32), 1);
+        const int64_t prev = lane == 0 ? (int64_t)(((uint64_t)(uint32_t)ehi << 32) | (uint32_t)elo)
+                                       : (int64_t)(((uint64_t)(uint32_t)hi32 << 32) | (uint32_t)lo32);
+        descent = descent || (node[j] >= 0 && prev >= 0 && node[j] < prev);
+        if (strict && node[j] < 0 && b0 + threadIdx.x + (int64_t)j * kBinPlaceBlock < hi) descent = true;
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < kBinCountPer; ++j) {
+      bin_take(s_hist, node[j] >= 0 ? (int32_t)(node[j] >> p.rshift) : -1);
+      node[j] = next[j];
+    }
   }
   // one flag for the whole launch: a workgroup that saw a descent sets it unless it reads as set already (ten
   // thousand wavefronts doing so one by one on the same address cost 100 us)
   if (__ballot(descent) != 0) s_hist_flag = 1;
   __syncthreads();
-  if (p.unsorted != nullptr && !p.sampled && threadIdx.x == 0 && s_hist_flag != 0 &&
+  if (check && threadIdx.x == 0 && s_hist_flag != 0 &&
       __hip_atomic_load(p.unsorted, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0)
     atomicOr(p.unsorted, 1);
   for (int i = threadIdx.x; i < p.nb; i += kBinPlaceBlock) {
     const int32_t h = s_hist[i];
-    p.wg_hist[(int64_t)blockIdx.x * p.nb + i] = h;
     if (h != 0) atomicAdd(&p.totals[i], (unsigned long long)h);
   }
 }
@@ -400,7 +453,8 @@ static __global__ __launch_bounds__(kBinPlaceBlock) void bin_place_kernel(Scatte
     if (a.route_ptr != nullptr) {
 #pragma unroll 4
       for (int j = 0; j < kBinPer; ++j) {
-        const int64_t be = (int64_t)blockIdx.x * kBinPlaceChunk + threadIdx.x + (int64_t)j * kBinPlaceBlock;
+        if (j * kBinPlaceBlock >= p.place_tile) break;
+        const int64_t be = (int64_t)blockIdx.x * p.place_tile + threadIdx.x + (int64_t)j * kBinPlaceBlock;
         if (be >= a.B * a.E) break;
         const int64_t b = be / a.E, e = be - b * a.E;
         const int64_t *idx = a.index + b * a.sb;
@@ -416,27 +470,31 @@ static __global__ __launch_bounds__(kBinPlaceBlock) void bin_place_kernel(Scatte
     }
     return;
   }
+  for (int i = threadIdx.x; i < p.nb; i += kBinPlaceBlock) s_cnt[i] = 0;
+  __syncthreads();
+  // the workgroup's tile (one batch at most, held in registers): rank inside the workgroup per bucket, then one
+  // atomic per bucket that occurs reserves the workgroup's run, then the words go out
+  const int64_t lo = (int64_t)blockIdx.x * p.place_tile;
+  const int64_t hi = lo + p.place_tile < a.B * a.E ? lo + p.place_tile : a.B * a.E;
+  int32_t bucket[kBinPer], local[kBinPer], rank[kBinPer];
+  bool unused = false;
+  bin_buckets(a, p, lo, hi, bucket, local, false, unused);
+#pragma unroll
+  for (int j = 0; j < kBinPer; ++j) rank[j] = bin_take(s_cnt, bucket[j]);
+  __syncthreads();
   for (int i = threadIdx.x; i < p.nb; i += kBinPlaceBlock) {
-    const int32_t h = p.wg_hist[(int64_t)blockIdx.x * p.nb + i];
-    s_base[i] = h != 0 ? (uint32_t)atomicAdd(&p.cursor[i], (unsigned long long)h) : 0u;
-    s_cnt[i] = 0;
+    const int32_t h = s_cnt[i];
+    if (h != 0) s_base[i] = (uint32_t)atomicAdd(&p.cursor[i], (unsigned long long)h);
   }
   __syncthreads();
-  const int64_t lo = (int64_t)blockIdx.x * kBinPlaceChunk;
-  const int64_t hi = lo + kBinPlaceChunk < a.B * a.E ? lo + kBinPlaceChunk : a.B * a.E;
-  for (int64_t b0 = lo; b0 < hi; b0 += kBinBatch) {
-    int32_t bucket[kBinPer], local[kBinPer];
-    bool unused = false;
-    bin_buckets(a, p, b0, hi, bucket, local, false, unused);
 #pragma unroll
-    for (int j = 0; j < kBinPer; ++j) {
-      const int32_t rank = bin_take(s_cnt, bucket[j]);
-      if (bucket[j] < 0) continue;
-      const int64_t be = b0 + threadIdx.x + (int64_t)j * kBinPlaceBlock;
-      p.binned[s_base[bucket[j]] + (uint32_t)rank] = ((uint64_t)(uint32_t)local[j] << 32) | (uint32_t)be;
-    }
+  for (int j = 0; j < kBinPer; ++j) {
+    if (bucket[j] < 0) continue;
+    const int64_t be = lo + threadIdx.x + (int64_t)j * kBinPlaceBlock;
+    p.binned[s_base[bucket[j]] + (uint32_t)rank[j]] = ((uint64_t)(uint32_t)local[j] << 32) | (uint32_t)be;
   }
 }
+static_assert(kBinPlaceChunk == kBinBatch, "the place pass holds a workgroup's entries in registers: one batch");
 
 // One finished packed key -> out / arg_out (element i of [B, N, K]): what scatter_key_init_kernel and
 // scatter_key_final_kernel do for the kernels that keep their keys in arg_out. key == 0: no entry.
@@ -806,6 +864,17 @@ __global__ __launch_bounds__(kBinBlock) void bin_add_wave_kernel(ScatterArgs a, 
   }
 }
 
+// the count pass: equal shares of the entries for at most kBinCountGroups workgroups
+inline void launch_bin_count(const ScatterArgs &a, const BinArgs &p, hipStream_t stream) {
+  int64_t groups = (a.B * a.E + kBinCountBatch - 1) / kBinCountBatch;
+  if (groups > kBinCountGroups) groups = kBinCountGroups;
+  if (groups < 1) groups = 1;
+  if (p.nb <= kBinSmallCap)
+    hipLaunchKernelGGL(bin_count_kernel<kBinSmallCap>, dim3((unsigned)groups), dim3(kBinPlaceBlock), 0, stream, a, p);
+  else
+    hipLaunchKernelGGL(bin_count_kernel<kBinMaxBuckets>, dim3((unsigned)groups), dim3(kBinPlaceBlock), 0, stream, a, p);
+}
+
 // log2 of the lanes that hold the kc columns of a slice, VEC columns each: the wavefront kernels want a power of
 // two up to 64. -1: no such number (then only bin_reduce_kernel can take the plan, and only without slices).
 inline int bin_lane_shift(const BinArgs &p, int vec) {
@@ -826,10 +895,7 @@ void launch_binned_keys(const ScatterArgs &a, const BinArgs &plan, hipStream_t s
     p.unsorted = nullptr;  // min / max take this path for sorted indices too
   hipLaunchKernelGGL(bin_clear_kernel, dim3((p.nb + kBlock - 1) / kBlock), dim3(kBlock), 0, stream, p.totals, p.nb,
                      p.unsorted);
-  if (p.nb <= kBinSmallCap)
-    hipLaunchKernelGGL(bin_count_kernel<kBinSmallCap>, dim3((unsigned)p.n_place), dim3(kBinPlaceBlock), 0, stream, a, p);
-  else
-    hipLaunchKernelGGL(bin_count_kernel<kBinMaxBuckets>, dim3((unsigned)p.n_place), dim3(kBinPlaceBlock), 0, stream, a, p);
+  launch_bin_count(a, p, stream);
   hipLaunchKernelGGL(bin_scan_kernel, dim3(1), dim3(kBinBlock), 0, stream, p);
   if (p.nb <= kBinSmallCap)  // 64 KB of cursors, two workgroups per CU; above: 128 KB, one
     hipLaunchKernelGGL(bin_place_kernel<kBinSmallCap>, dim3((unsigned)p.n_place), dim3(kBinPlaceBlock), 0, stream, a, p);
@@ -866,10 +932,7 @@ void launch_binned_add(const ScatterArgs &a, const BinArgs &plan, int lshift, hi
   if (p.sampled) hipLaunchKernelGGL(bin_sample_kernel, dim3(1), dim3(kBinBlock), 0, stream, a, p.unsorted);
   hipLaunchKernelGGL(bin_clear_kernel, dim3((p.nb + kBlock - 1) / kBlock), dim3(kBlock), 0, stream, p.totals, p.nb,
                      p.sampled ? (int *)nullptr : p.unsorted);
-  if (p.nb <= kBinSmallCap)
-    hipLaunchKernelGGL(bin_count_kernel<kBinSmallCap>, dim3((unsigned)p.n_place), dim3(kBinPlaceBlock), 0, stream, a, p);
-  else
-    hipLaunchKernelGGL(bin_count_kernel<kBinMaxBuckets>, dim3((unsigned)p.n_place), dim3(kBinPlaceBlock), 0, stream, a, p);
+  launch_bin_count(a, p, stream);
   if (zero_out > 0)
     hipLaunchKernelGGL(bin_zero_out_kernel<T>, dim3(grid_for(zero_out)), dim3(kBlock), 0, stream, static_cast<T *>(a.out),
                        zero_out, p.unsorted);
