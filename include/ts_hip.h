@@ -238,11 +238,18 @@ int ts_arg_backward(const void *grad_out, const int64_t *arg, void *grad_in,
  *   m = group max, s = group sum of exp(src - m)
  *   log_space == 0:  out = exp(src - m) / s
  *   log_space != 0:  out = (src - m) - log(s + eps)
- * Replaces, in three passes over src, the op sequences of
- * torch_scatter/composite/softmax.py:16-29 and :45-59 (scatter_max, gather,
- * sub, exp, scatter_sum, gather, div); the reference has no single launcher
- * for it. Floating types only. Entries whose index lies outside [0, N) belong
- * to no group and yield 0. The backward call takes the forward result:
+ * Replaces the op sequences of torch_scatter/composite/softmax.py:16-29 and
+ * :45-59 (scatter_max, gather, sub, exp, scatter_sum, gather, div); the
+ * reference has no single launcher for it. Three passes over src for an index
+ * in any order. An index that is in order along E, with rows of up to 128
+ * bytes and from 16 MB of input on (32 MB backward), takes one pass: tiles of
+ * entries are finished in LDS, every tile checks the order of its part of the
+ * index, and the three passes run behind them only if a tile found a descent
+ * (the word at workspace + ts_group_softmax_workspace_bytes() - 256 is then
+ * 1, else 0). That path
+ * multiplies by the reciprocal of the group sum (fp32 / fp64: within 1 ulp of
+ * the quotient). Floating types only. Entries whose index lies outside [0, N)
+ * belong to no group and yield 0. The backward call takes the forward result:
  *   log_space == 0:  grad_in = result * (grad_out - S),  S = group sum of result * grad_out
  *   log_space != 0:  grad_in = grad_out - exp(result) * G,  G = group sum of grad_out
  * workspace: ts_group_softmax_workspace_bytes() bytes of device scratch,

@@ -663,7 +663,7 @@ int run_group_softmax(const void *src, const void *grad, const int64_t *index, v
   g.index = index;
   g.out = out;
   g.gmax = workspace;
-  g.gsum = static_cast<char *>(workspace) + need / 2;
+  g.gsum = static_cast<char *>(workspace) + group_three_pass_bytes(B, N, K, kElemBytes[dtype]) / 2;
   g.B = B;
   g.E = E;
   g.K = K;
@@ -677,6 +677,8 @@ int run_group_softmax(const void *src, const void *grad, const int64_t *index, v
   g.total = nullptr;
   g.count = nullptr;
   g.unbiased = 0;
+  g.ws_bytes = group_three_pass_bytes(B, N, K, kElemBytes[dtype]);
+  g.flag = reinterpret_cast<int *>(static_cast<char *>(workspace) + g.ws_bytes);
   const int full = kVecBytes / kElemBytes[dtype];
   const bool al = aligned16(src) && aligned16(out) && (!grad || aligned16(grad));
   const int vec = (full > 1 && K % full == 0 && al) ? full : 1;
@@ -721,7 +723,7 @@ int ts_group_logsumexp(const void *src, const int64_t *index, void *out, int64_t
   g.index = index;
   g.out = out;
   g.gmax = workspace;
-  g.gsum = static_cast<char *>(workspace) + need / 2;
+  g.gsum = static_cast<char *>(workspace) + group_three_pass_bytes(B, N, K, kElemBytes[dtype]) / 2;
   g.B = B;
   g.E = E;
   g.K = K;
@@ -776,7 +778,7 @@ int ts_group_std(const void *src, const int64_t *index, const void *total, const
   g.index = index;
   g.out = out;
   g.gmax = workspace;
-  g.gsum = static_cast<char *>(workspace) + need / 2;
+  g.gsum = static_cast<char *>(workspace) + group_three_pass_bytes(B, N, K, kElemBytes[dtype]) / 2;
   g.total = total;
   g.count = count;
   g.unbiased = unbiased ? 1 : 0;

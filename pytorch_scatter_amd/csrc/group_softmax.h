@@ -55,6 +55,8 @@ __device__ __forceinline__ double exp_acc(double v) { return exp(v); }
 __device__ __forceinline__ float log_acc(float v) { return logf(v); }
 __device__ __forceinline__ double log_acc(double v) { return log(v); }
 __device__ __forceinline__ float sqrt_acc(float v) { return sqrtf(v); }
+__device__ __forceinline__ float max_acc(float a, float b) { return fmaxf(a, b); }
+__device__ __forceinline__ double max_acc(double a, double b) { return fmax(a, b); }
 __device__ __forceinline__ double sqrt_acc(double v) { return sqrt(v); }
 
 // a value of the accumulate type as the element type would hold it
@@ -87,6 +89,9 @@ struct GroupArgs {
   const void *total;      // [B, N, K]: std, the group sums of src in the element type
   const float *count;     // [B, N]: std, entries per group
   int unbiased;           // std: divide by count - 1
+  const int *gate = nullptr;  // the three passes of softmax run only if *gate != 0 (null: always)
+  int *flag = nullptr;        // softmax: a word behind the workspace of the three passes, for the one-pass kernels
+  size_t ws_bytes = 0;        //          bytes of that workspace (gmax is its start)
 };
 
 // std: the group mean as the reference forms it (composite/std.py:27-31: sum / clamp(count, 1), in the
@@ -107,16 +112,21 @@ template <typename T> __device__ __forceinline__ typename Acc<T>::type group_div
 }
 
 inline size_t group_align(size_t v) { return (v + 255) / 256 * 256; }
-// bytes of workspace: keys and sums, each [B, N, K] in 8 bytes at most
-inline size_t group_workspace_bytes(int64_t B, int64_t N, int64_t K, int elem_bytes) {
+// bytes of workspace: keys and sums, each [B, N, K] in 8 bytes at most, and behind them the word that tells
+// the one-pass kernels (group_fused.h) and the three passes apart
+inline size_t group_three_pass_bytes(int64_t B, int64_t N, int64_t K, int elem_bytes) {
   const size_t acc = elem_bytes == 8 ? 8 : 4;
   return 2 * group_align((size_t)(B * N * K) * acc);
+}
+inline size_t group_workspace_bytes(int64_t B, int64_t N, int64_t K, int elem_bytes) {
+  return group_three_pass_bytes(B, N, K, elem_bytes) + 256;
 }
 
 template <typename T>
 __global__ __launch_bounds__(kBlock) void group_init_kernel(GroupArgs g, int with_max) {
   typedef typename Acc<T>::type F;
   typedef typename OrdKey<F>::bits KB;
+  if (g.gate != nullptr && *g.gate == 0) return;
   const int64_t n = g.B * g.N * g.K;
   KB *gmax = static_cast<KB *>(g.gmax);
   F *gsum = static_cast<F *>(g.gsum);
@@ -163,6 +173,7 @@ __global__ __launch_bounds__(kBlock) void group_max_run_kernel(ScatterArgs a, Gr
                                                                int rows_per_wave) {
   typedef typename GroupMaxRun<T, C>::A A;
   __shared__ A s_stage[kBlock / kWave][kWave * C];
+  if (g.gate != nullptr && *g.gate == 0) return;
   GroupMaxRun<T, C> p;
   p.src = static_cast<const T *>(g.src);
   p.gmax = static_cast<A *>(g.gmax);
@@ -258,6 +269,7 @@ __global__ __launch_bounds__(kBlock) void group_sum_run_kernel(ScatterArgs a, Gr
   __shared__ A s_stage[kBlock / kWave][kWave * C];
   __shared__ typename HotSlot<A>::type s_hot[kHotAcc];
   __shared__ uint32_t s_tags[kHotRowsMax];
+  if (g.gate != nullptr && *g.gate == 0) return;
   GroupSumRun<T, C, MODE> p;
   p.src = static_cast<const T *>(g.src);
   p.grad = static_cast<const T *>(g.grad);
@@ -278,6 +290,7 @@ template <typename T, int VEC, int MODE>
 __global__ __launch_bounds__(kBlock) void group_finish_kernel(GroupArgs g) {
   typedef typename Acc<T>::type F;
   constexpr int U = 4;
+  if (g.gate != nullptr && *g.gate == 0) return;
   const T *src = static_cast<const T *>(g.src);
   const T *grad = static_cast<const T *>(g.grad);
   const F *gsum = static_cast<const F *>(g.gsum);
@@ -407,6 +420,10 @@ __global__ __launch_bounds__(kBlock) void group_std_finish_kernel(GroupArgs g) {
   }
 }
 
+}  // namespace ts
+#include "group_fused.h"
+namespace ts {
+
 // ---- host side
 inline ScatterArgs group_index_args(const GroupArgs &g) {
   ScatterArgs a = {};
@@ -422,12 +439,24 @@ inline ScatterArgs group_index_args(const GroupArgs &g) {
 }
 
 template <typename T, int VEC, int MODE>
-int launch_group_softmax_m(const GroupArgs &g, hipStream_t stream) {
+int launch_group_softmax_m(const GroupArgs &g_in, hipStream_t stream) {
   constexpr bool kForward = MODE == GS_SOFTMAX || MODE == GS_LOG_SOFTMAX;
+  GroupArgs g = g_in;
   const int64_t n_edges = g.B * g.E;
   if (g.B * g.N >= 0x7FFFFFFFll) return TS_ERR_UNSUPPORTED;
   const RunGrid rg = run_grid(n_edges, g.K / VEC, VEC, VEC * (int)sizeof(T));
   if (!rg.ok) return TS_ERR_UNSUPPORTED;
+  // An index that looks sorted goes through the one-pass kernels first; the three passes below then run only
+  // if those found a descent. TS_GROUP_FUSED: 0 never, 2 at any size and whatever the index looks like.
+  int fused_mode = 1;
+  if (const char *env = getenv("TS_GROUP_FUSED")) fused_mode = atoi(env);
+  FusedArgs f;
+  if (fused_mode != 0 && g.flag != nullptr &&
+      group_fused_plan(g, MODE, (int)sizeof(T), g.gmax, g.ws_bytes, fused_mode == 2, f)) {
+    const int rc = launch_group_fused<T, VEC, MODE>(g, f, fused_mode == 2, stream);
+    if (rc != TS_OK) return rc;
+    g.gate = f.flag;
+  }
   const ScatterArgs a = group_index_args(g);
   const dim3 gd(rg.blocks, rg.ychunks);
   hipLaunchKernelGGL(group_init_kernel<T>, dim3(grid_for(g.B * g.N * g.K)), dim3(kBlock), 0, stream, g,

@@ -63,40 +63,162 @@ def forward_bound(dtype, want64, z64, log_space):
     return e * (4.0 + z64.abs()) * want64.abs() + (2.0 ** -23 if dtype == torch.float16 else 1e-30)
 
 
+def check_against_oracle(capi, oracle, src, grad, index1, shape, dtype):
+    B, E, K, N = shape
+    index = index1.view(1, E, 1).expand(B, E, K)
+    exact = dtype in (torch.float32, torch.float64)
+    ref_src = src if exact else src.double()
+    inside = (index >= 0) & (index < N)
+    safe = index.clamp(0, N - 1)
+    if bool(inside.all()):
+        group_max = oracle.scatter(ref_src, index, 1, None, N, "max")[0]
+    else:  # entries outside [0, N) belong to no group: keep them out of the reference, expect 0 for them
+        low = torch.finfo(ref_src.dtype).min
+        group_max = oracle.scatter(torch.where(inside, ref_src, torch.full_like(ref_src, low)), safe, 1, None, N, "max")[0]
+    z64 = (ref_src - group_max.gather(1, safe)).double()
+    for log_space in (False, True):
+        out = torch.empty((B, E, K), dtype=dtype, device=DEV)
+        capi.group_softmax(src.to(DEV), index1.to(DEV), out, B, E, K, N, 0, 1, log_space)
+        torch.cuda.synchronize()
+        if bool(inside.all()):
+            want = (oracle.scatter_log_softmax(ref_src, index, 1, 1e-12, N) if log_space
+                    else oracle.scatter_softmax(ref_src, index, 1, N)).double()
+        else:
+            keep = inside[0, :, 0]
+            part = (oracle.scatter_log_softmax(ref_src[:, keep], index[:, keep], 1, 1e-12, N) if log_space
+                    else oracle.scatter_softmax(ref_src[:, keep], index[:, keep], 1, N)).double()
+            want = torch.zeros((B, E, K), dtype=torch.float64)
+            want[:, keep] = part
+        err = (out.cpu().double() - want).abs()
+        bound = forward_bound(dtype, want, z64, log_space)
+        assert bool((err <= bound).all()), (log_space, float((err - bound).max()))
+        assert float(out.cpu().double()[~inside].abs().max() if bool((~inside).any()) else 0.0) == 0.0
+
+        grad_in = torch.empty((B, E, K), dtype=dtype, device=DEV)
+        capi.group_softmax_backward(out, grad.to(DEV), index1.to(DEV), grad_in, B, E, K, N, 0, 1, log_space)
+        torch.cuda.synchronize()
+        y64, g64 = out.cpu().double(), grad.double()
+        keep = inside[0, :, 0]
+        want_g = torch.zeros((B, E, K), dtype=torch.float64)
+        want_g[:, keep] = oracle.scatter_softmax_backward(y64[:, keep], g64[:, keep], index[:, keep], 1, N, log_space)
+        terms = (g64.abs() if log_space else (y64 * g64).abs())
+        spread = oracle.scatter(terms * inside, safe, 1, None, N, "sum")[0].gather(1, safe)
+        scale = g64.abs() + y64.exp() * spread if log_space else y64.abs() * (g64.abs() + spread)
+        e = EPS_T[dtype]
+        gerr = (grad_in.cpu().double() - want_g).abs()
+        gbound = 8 * e * scale + (2.0 ** -23 if dtype == torch.float16 else 1e-30)  # fp16 subnormals
+        assert bool((gerr[:, keep] <= gbound[:, keep]).all()), ("backward", log_space, float((gerr - gbound).max()))
+        assert float(grad_in.cpu().double()[~inside].abs().max() if bool((~inside).any()) else 0.0) == 0.0
+
+
 @pytest.mark.parametrize("shape,kind,dtype", product(SHAPES, ["random", "sorted", "hub"], DTYPES))
 def test_forward_and_backward_capi(capi, oracle, shape, kind, dtype):
     B, E, K, N = shape
     rng = np.random.default_rng(E * 13 + K)
     src = torch.from_numpy(rng.standard_normal(size=(B, E, K)) * 3).to(dtype)
     grad = torch.from_numpy(rng.standard_normal(size=(B, E, K))).to(dtype)
-    index1 = make_index(kind, rng, E, N)
-    index = index1.view(1, E, 1).expand(B, E, K)
-    exact = dtype in (torch.float32, torch.float64)
-    ref_src = src if exact else src.double()
-    group_max = oracle.scatter(ref_src, index, 1, None, N, "max")[0]
-    z64 = (ref_src - group_max.gather(1, index)).double()
-    for log_space in (False, True):
-        out = torch.empty((B, E, K), dtype=dtype, device=DEV)
-        capi.group_softmax(src.to(DEV), index1.to(DEV), out, B, E, K, N, 0, 1, log_space)
-        torch.cuda.synchronize()
-        want = (oracle.scatter_log_softmax(ref_src, index, 1, 1e-12, N) if log_space
-                else oracle.scatter_softmax(ref_src, index, 1, N)).double()
-        err = (out.cpu().double() - want).abs()
-        bound = forward_bound(dtype, want, z64, log_space)
-        assert bool((err <= bound).all()), (log_space, float((err - bound).max()))
+    check_against_oracle(capi, oracle, src, grad, make_index(kind, rng, E, N), shape, dtype)
 
-        grad_in = torch.empty((B, E, K), dtype=dtype, device=DEV)
-        capi.group_softmax_backward(out, grad.to(DEV), index1.to(DEV), grad_in, B, E, K, N, 0, 1, log_space)
+
+# The one-pass kernels for an index that is in order (group_fused.h) take over from 16 / 32 MB of input; the
+# environment switches them on at any size and sets their tile, so that small inputs reach every part of them:
+# runs inside a tile, runs that cross one border or fill whole tiles, short / medium / long runs, entries outside
+# [0, N) at either end, an index that is not in order (the tiles notice and the three passes redo the work).
+FUSED_SHAPES = [
+    # B, E, K, N
+    (1, 5000, 1, 600), (1, 5000, 1, 3), (2, 3000, 4, 50), (1, 2000, 8, 300), (1, 2000, 8, 2), (1, 1500, 3, 40),
+    (1, 900, 32, 20), (3, 400, 16, 7), (1, 257, 2, 300), (1, 4099, 8, 1), (1, 2, 4, 5),
+]
+
+
+def fused_index(kind, rng, E, N):
+    if kind == "skewed":  # a few long runs among many short ones
+        idx = np.sort(np.concatenate([rng.integers(0, N, size=E - E // 2), np.full(E // 2, N // 2)]))
+    elif kind == "outside":  # sorted, with entries below 0 in front and from N on at the end
+        idx = np.sort(rng.integers(-max(N // 8, 1), N + max(N // 8, 1), size=E))
+    elif kind == "one_descent":
+        idx = np.sort(rng.integers(0, N, size=E))
+        idx[E // 2:] = np.sort(rng.integers(0, N, size=E - E // 2))
+    else:
+        idx = np.sort(rng.integers(0, N, size=E))
+    return torch.from_numpy(idx)
+
+
+@pytest.mark.parametrize("shape,kind,dtype",
+                         product(FUSED_SHAPES, ["sorted", "skewed", "outside", "one_descent"], DTYPES))
+@pytest.mark.parametrize("tile", [256, 0])
+def test_one_pass_kernels_capi(capi, oracle, monkeypatch, shape, kind, dtype, tile):
+    B, E, K, N = shape
+    monkeypatch.setenv("TS_GROUP_FUSED", "2")
+    if tile:
+        monkeypatch.setenv("TS_GROUP_TILE", str(tile))
+    rng = np.random.default_rng(E * 7 + K + N)
+    src = torch.from_numpy(rng.standard_normal(size=(B, E, K)) * 3).to(dtype)
+    grad = torch.from_numpy(rng.standard_normal(size=(B, E, K))).to(dtype)
+    check_against_oracle(capi, oracle, src, grad, fused_index(kind, rng, E, N), shape, dtype)
+
+
+def test_one_pass_kernels_leave_their_verdict(capi, monkeypatch):
+    """The word behind the workspace of the three passes says whether the tiles found the index in order: 1 after
+    one descent (the three passes then ran), 0 for a sorted index (they returned at once)."""
+    monkeypatch.setenv("TS_GROUP_FUSED", "2")
+    monkeypatch.setenv("TS_GROUP_TILE", "256")
+    rng = np.random.default_rng(3)
+    B, E, K, N = 1, 3000, 4, 200
+    src = torch.from_numpy(rng.standard_normal(size=(B, E, K))).float().to(DEV)
+    for kind, verdict in (("one_descent", 1), ("sorted", 0), ("one_descent", 1)):
+        index = fused_index(kind, rng, E, N).to(DEV)
+        out = torch.empty_like(src)
+        ws = capi.group_softmax(src, index, out, B, E, K, N, 0, 1, False)
         torch.cuda.synchronize()
-        y64, g64 = out.cpu().double(), grad.double()
-        want_g = oracle.scatter_softmax_backward(y64, g64, index, 1, N, log_space)
-        terms = (g64.abs() if log_space else (y64 * g64).abs())
-        spread = oracle.scatter(terms, index, 1, None, N, "sum")[0].gather(1, index)
-        scale = g64.abs() + y64.exp() * spread if log_space else y64.abs() * (g64.abs() + spread)
-        e = EPS_T[dtype]
-        gerr = (grad_in.cpu().double() - want_g).abs()
-        gbound = 8 * e * scale + (2.0 ** -23 if dtype == torch.float16 else 1e-30)  # fp16 subnormals
-        assert bool((gerr <= gbound).all()), ("backward", log_space, float((gerr - gbound).max()))
+        assert int(ws[-256:-252].cpu().view(torch.int32)[0]) == verdict, kind
+
+
+def test_one_pass_kernels_special_values(capi, oracle, monkeypatch):
+    """The cases of test_special_values_capi in order, in tiles of 256 entries with the groups repeated so that
+    runs of -inf, a NaN and an empty group meet tile borders."""
+    monkeypatch.setenv("TS_GROUP_FUSED", "2")
+    monkeypatch.setenv("TS_GROUP_TILE", "256")
+    vals = [[0.2, 0.2], [0.0, -2.1, 3.2], [7.0], [], [-1.0, float("-inf")], [float("-inf")] * 2,
+            [1.0, float("nan"), 2.0], []]
+    reps = 90
+    src = torch.tensor([v for _ in range(reps) for grp in vals for v in grp])
+    index = torch.tensor([r * len(vals) + g for r in range(reps) for g, grp in enumerate(vals) for _ in grp])
+    E, N = src.numel(), reps * len(vals)
+    for log_space in (False, True):
+        out = torch.empty(E, device=DEV)
+        capi.group_softmax(src.to(DEV), index.to(DEV), out, 1, E, 1, N, 0, 1, log_space)
+        torch.cuda.synchronize()
+        want = (oracle.scatter_log_softmax(src, index, 0, 1e-12, N) if log_space
+                else oracle.scatter_softmax(src, index, 0, dim_size=N))
+        assert torch.allclose(out.cpu(), want, rtol=1e-5, atol=1e-7, equal_nan=True), log_space
+
+
+@pytest.mark.parametrize("dtype,K", [(torch.float32, 8), (torch.bfloat16, 16), (torch.float32, 1)])
+def test_one_pass_kernels_take_large_sorted_inputs(capi, monkeypatch, dtype, K):
+    """At its default settings the library sends a sorted index of this size through the one-pass kernels;
+    the three passes (switched on by the environment) give the reference result."""
+    E, N = (1 << 21) + 77, 250_000
+    if K == 1:
+        E *= 4
+    g = torch.Generator().manual_seed(5)
+    index = torch.sort(torch.randint(0, N, (E,), generator=g)).values.to(DEV)
+    src = (torch.randn((1, E, K), generator=g) * 3).to(dtype).to(DEV)
+    grad = torch.randn((1, E, K), generator=g).to(dtype).to(DEV)
+    res = {}
+    for mode in ("0", "1"):
+        monkeypatch.setenv("TS_GROUP_FUSED", mode)
+        for log_space in (False, True):
+            out, gin = torch.empty_like(src), torch.empty_like(src)
+            capi.group_softmax(src, index, out, 1, E, K, N, 0, 1, log_space)
+            capi.group_softmax_backward(out, grad, index, gin, 1, E, K, N, 0, 1, log_space)
+            res[mode, log_space] = (out.double(), gin.double())
+    torch.cuda.synchronize()
+    e = EPS_T[dtype]
+    for log_space in (False, True):
+        a, b = res["0", log_space], res["1", log_space]
+        assert bool(((a[0] - b[0]).abs() <= 16 * e * (1.0 + a[0].abs())).all())
+        assert bool(((a[1] - b[1]).abs() <= 64 * e * (1.0 + a[1].abs())).all())
 
 
 def test_special_values_capi(capi, oracle):
