@@ -18,7 +18,7 @@
 
 namespace ts {
 
-constexpr int kFusedMaxTile = 4096;   // entries per tile at most (run starts are 16-bit words with a flag bit)
+constexpr int kFusedMaxTile = 2048;   // entries per tile at most (run starts are 16-bit words with a flag bit)
 constexpr int kFusedShortRun = 12;    // runs of up to this many entries inside a tile: one lane per (run, columns)
 constexpr int kFusedGroup = 8;        // longer ones: eight lanes, and a wavefront from kFusedGroup * kFusedShortRun entries on
 constexpr int kFusedRowBytes = 128;   // widest row the tiles are built for
@@ -134,39 +134,57 @@ __device__ __forceinline__ void fused_absorb(typename OrdKey<typename Acc<T>::ty
 __device__ __forceinline__ float fast_rcp(float v) { return __builtin_amdgcn_rcpf(v); }
 __device__ __forceinline__ double fast_rcp(double v) { return 1.0 / v; }
 
-// The EPL neighbouring entries of a lane, from local entry e0 on: which of them begin a run (bit i of headmask),
-// whether that run's index lies outside [0, N) (badmask), whether an entry lies below the one before it. All index
-// loads are issued before `between` runs (the caller's stores of the staged tile, which wait for the tile's loads).
+// Which entries of the tile begin a run, and whether that run's index lies outside [0, N). The index is loaded
+// coalesced (lane tid takes entries tid, tid + 256, ...: with one value per entry the index is two thirds of the
+// bytes); an entry's predecessor comes from the neighbouring lane, for the first lane of a wavefront from memory.
+// The flags go through LDS (a byte per entry) so that afterwards every lane holds those of its EPL neighbouring
+// entries e0 .. e0 + EPL - 1 as bit masks. All index loads are issued before `between` runs (the caller's stores
+// of the staged tile, which wait for the tile's loads). Ends with the workgroup in step (barrier).
 template <int EPL, typename Between>
-__device__ __forceinline__ void fused_find_runs(const int64_t *idx, int64_t se, int64_t j0, int e0, int ne, int64_t E,
-                                                int64_t N, Between &&between, uint32_t &headmask, uint32_t &badmask,
-                                                bool &descent, bool &enters, bool &leaves) {
-  int64_t id[EPL];
+__device__ __forceinline__ void fused_find_runs(const int64_t *idx, int64_t se, int64_t j0, int tid, int ne, int64_t E,
+                                                int64_t N, uint8_t *s_flag, Between &&between, uint32_t &headmask,
+                                                uint32_t &badmask, bool &descent, bool &enters, bool &leaves) {
+  const int lane = tid & (kWave - 1);
+  int64_t id[EPL], edge[EPL];
 #pragma unroll
-  for (int i = 0; i < EPL; ++i) id[i] = e0 + i < ne ? idx[(j0 + e0 + i) * se] : 0;
-  int64_t prev = 0, next = 0;
-  bool have_prev = false, have_next = false;
-  if (e0 < ne && j0 + e0 > 0) {
-    prev = idx[(j0 + e0 - 1) * se];
-    have_prev = true;
+  for (int q = 0; q < EPL; ++q) {
+    const int e = tid + q * kBlock;
+    id[q] = e < ne ? idx[(j0 + e) * se] : 0;
   }
-  if (e0 <= ne - 1 && ne - 1 < e0 + EPL && j0 + ne < E) {  // the lane that holds the tile's last entry
-    next = idx[(j0 + ne) * se];
-    have_next = true;
+#pragma unroll
+  for (int q = 0; q < EPL; ++q) {
+    const int e = tid + q * kBlock;
+    edge[q] = (lane == 0 && e < ne && j0 + e > 0) ? idx[(j0 + e - 1) * se] : 0;
   }
+  const int e_last = ne - 1;
+  const bool owns_last = (e_last & (kBlock - 1)) == tid;
+  int64_t next = 0;
+  const bool have_next = owns_last && j0 + ne < E;
+  if (have_next) next = idx[(j0 + ne) * se];
   between();
-  if (e0 == 0 && have_prev && id[0] == prev) enters = true;
+#pragma unroll
+  for (int q = 0; q < EPL; ++q) {
+    const int e = tid + q * kBlock;
+    const int lo32 = __shfl_up((int)(uint32_t)id[q], 1), hi32 = __shfl_up((int)(id[q] >> 32), 1);
+    const int64_t prev = lane == 0 ? edge[q] : (int64_t)(((uint64_t)(uint32_t)hi32 << 32) | (uint32_t)lo32);
+    if (e < ne) {
+      const bool have_prev = j0 + e > 0;
+      const bool head = e == 0 || id[q] != prev;
+      const bool bad = head && (id[q] < 0 || id[q] >= N);
+      if (have_prev && id[q] < prev) descent = true;
+      if (e == 0 && have_prev && id[q] == prev) enters = true;
+      if (e == e_last && have_next && next == id[q]) leaves = true;
+      s_flag[e] = (uint8_t)((head ? 1 : 0) | (bad ? 2 : 0));
+    }
+  }
+  __syncthreads();
+  const int e0 = tid * EPL;
 #pragma unroll
   for (int i = 0; i < EPL; ++i) {
     if (e0 + i < ne) {
-      if (e0 + i == 0 || id[i] != prev) {
-        headmask |= 1u << i;
-        if (id[i] < 0 || id[i] >= N) badmask |= 1u << i;
-      }
-      if (have_prev && id[i] < prev) descent = true;
-      prev = id[i];
-      have_prev = true;
-      if (e0 + i == ne - 1 && have_next && next == id[i]) leaves = true;
+      const uint32_t fl = s_flag[e0 + i];
+      headmask |= (fl & 1u) << i;
+      badmask |= (fl >> 1 & 1u) << i;
     }
   }
 }
@@ -218,6 +236,7 @@ __global__ __launch_bounds__(kBlock, 4) void group_fused_kernel(GroupArgs g, Fus
   // ---- runs: a lane looks at epl neighbouring entries
   const int64_t *idx = g.index + b * g.sb;
   const int e0 = tid * f.epl;
+  uint8_t *s_flag = reinterpret_cast<uint8_t *>(s_start);  // read by all lanes before the run starts are written
   uint32_t headmask = 0, badmask = 0;
   bool descent = false, lane_enters = false, lane_leaves = false;
   auto stage_to_lds = [&]() {
@@ -229,11 +248,10 @@ __global__ __launch_bounds__(kBlock, 4) void group_fused_kernel(GroupArgs g, Fus
     }
   };
   switch (f.epl) {
-  case 1: fused_find_runs<1>(idx, g.se, j0, e0, ne, g.E, g.N, stage_to_lds, headmask, badmask, descent, lane_enters, lane_leaves); break;
-  case 2: fused_find_runs<2>(idx, g.se, j0, e0, ne, g.E, g.N, stage_to_lds, headmask, badmask, descent, lane_enters, lane_leaves); break;
-  case 4: fused_find_runs<4>(idx, g.se, j0, e0, ne, g.E, g.N, stage_to_lds, headmask, badmask, descent, lane_enters, lane_leaves); break;
-  case 8: fused_find_runs<8>(idx, g.se, j0, e0, ne, g.E, g.N, stage_to_lds, headmask, badmask, descent, lane_enters, lane_leaves); break;
-  default: fused_find_runs<16>(idx, g.se, j0, e0, ne, g.E, g.N, stage_to_lds, headmask, badmask, descent, lane_enters, lane_leaves); break;
+  case 1: fused_find_runs<1>(idx, g.se, j0, tid, ne, g.E, g.N, s_flag, stage_to_lds, headmask, badmask, descent, lane_enters, lane_leaves); break;
+  case 2: fused_find_runs<2>(idx, g.se, j0, tid, ne, g.E, g.N, s_flag, stage_to_lds, headmask, badmask, descent, lane_enters, lane_leaves); break;
+  case 4: fused_find_runs<4>(idx, g.se, j0, tid, ne, g.E, g.N, s_flag, stage_to_lds, headmask, badmask, descent, lane_enters, lane_leaves); break;
+  default: fused_find_runs<8>(idx, g.se, j0, tid, ne, g.E, g.N, s_flag, stage_to_lds, headmask, badmask, descent, lane_enters, lane_leaves); break;
   }
   if (lane_enters) s_info[0] = 1;
   if (lane_leaves) s_info[1] = 1;
