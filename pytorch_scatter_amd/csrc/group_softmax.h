@@ -11,7 +11,9 @@
 //   log_softmax  out = (src - m) - log(s + eps)[index[i]]       (composite/softmax.py:45-59)
 //
 // The reference runs this as two scatters, two gathers and four elementwise
-// passes. Here it is three passes over src: group maxima as order-preserving
+// passes. An index that is in order takes the one-pass tiles of group_fused.h;
+// any other index (and whatever those tiles decline) takes the kernels of this
+// file, three passes over src: group maxima as order-preserving
 // integer keys (atomic max), group sums in the accumulate type (atomic add),
 // and the elementwise finish that recomputes e from src. The first two reuse
 // the wavefront pre-reduction of runs of equal neighbouring indices, so a
