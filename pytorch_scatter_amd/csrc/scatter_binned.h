@@ -24,7 +24,7 @@ constexpr int kBinBlock = 1024;
 constexpr int kBinMaxBuckets = 16384;  // LDS histogram of count / place (their LDS is sized for 8192 or 16384 buckets)
 constexpr int kBinSmallCap = 8192;
 constexpr int kBinChunk = 8192;       // entries per chunk of a bucket in reduce (fewer for inputs under 4 M entries)
-constexpr int kBinPlaceChunk = 16384;  // most entries per workgroup in place: one batch of 16 per lane
+constexpr int kBinPlaceChunk = 10240;  // most entries per workgroup in place: one batch of 10 per lane
 constexpr int kCombPos = 64;          // combining kernel: keys per step of a bucket of many chunks,
 constexpr int kCombFew = 32;          // many: more than this
 constexpr int kBinPlaceBlock = 1024;   // (measured slower: 256 lanes x 4 batches, 64 K entries per workgroup, 8 K)
@@ -180,7 +180,8 @@ __device__ __forceinline__ int64_t bin_node(const ScatterArgs &a, int64_t be) {
   return (idx >= 0 && idx < a.N) ? b * a.N + idx : -1;
 }
 
-constexpr int kBinPer = 16;  // entries per lane and batch in count / place (all index loads of a batch in flight)
+constexpr int kBinPer = 10;  // entries per lane in place (all index loads in flight; three words per entry stay in
+                             // registers: with 16 the kernel needs 91 VGPRs, which is one workgroup per CU instead of two)
 constexpr int kBinBatch = kBinPer * kBinPlaceBlock;
 
 // buckets of the kBinPer entries of a lane, all index loads in flight at once; -1: no bucket
