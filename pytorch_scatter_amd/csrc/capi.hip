@@ -663,7 +663,10 @@ int run_group_softmax(const void *src, const void *grad, const int64_t *index, v
   g.index = index;
   g.out = out;
   g.gmax = workspace;
-  g.gsum = static_cast<char *>(workspace) + group_three_pass_bytes(B, N, K, kElemBytes[dtype]) / 2;
+  // forward: a group's keys and sums side by side (the finish reads both with one line); backward: sums only
+  const bool with_keys = mode == GS_SOFTMAX || mode == GS_LOG_SOFTMAX;
+  g.gs = with_keys ? 2 * K : K;
+  g.gsum = static_cast<char *>(workspace) + (with_keys ? (size_t)K * (kElemBytes[dtype] == 8 ? 8 : 4) : 0);
   g.B = B;
   g.E = E;
   g.K = K;
@@ -723,7 +726,8 @@ int ts_group_logsumexp(const void *src, const int64_t *index, void *out, int64_t
   g.index = index;
   g.out = out;
   g.gmax = workspace;
-  g.gsum = static_cast<char *>(workspace) + group_three_pass_bytes(B, N, K, kElemBytes[dtype]) / 2;
+  g.gs = 2 * K;  // a group's keys and sums side by side
+  g.gsum = static_cast<char *>(workspace) + (size_t)K * (kElemBytes[dtype] == 8 ? 8 : 4);
   g.B = B;
   g.E = E;
   g.K = K;
@@ -778,7 +782,8 @@ int ts_group_std(const void *src, const int64_t *index, const void *total, const
   g.index = index;
   g.out = out;
   g.gmax = workspace;
-  g.gsum = static_cast<char *>(workspace) + group_three_pass_bytes(B, N, K, kElemBytes[dtype]) / 2;
+  g.gs = K;  // sums only
+  g.gsum = workspace;
   g.total = total;
   g.count = count;
   g.unbiased = unbiased ? 1 : 0;

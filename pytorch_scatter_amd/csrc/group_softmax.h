@@ -80,8 +80,9 @@ struct GroupArgs {
   const void *grad;      // [B, E, K]: backward only, gradient of the result
   const int64_t *index;  // index[b * sb + e * se]
   void *out;             // [B, E, K]
-  void *gmax;            // [B, N, K] keys of the group maxima (forward)
-  void *gsum;            // [B, N, K] group sums in the accumulate type
+  void *gmax;            // [B, N, 2, K]: the keys of a group's maxima (forward) in [.., 0, :],
+  void *gsum;            // its sums in the accumulate type in [.., 1, :] (gsum = gmax + K words)
+  int64_t gs;            // words from one group to the next: 2K like that, or K when only the sums are used (then gsum = gmax)
   int64_t B, E, K, N;
   int64_t sb, se;
   double eps;
@@ -129,13 +130,17 @@ __global__ __launch_bounds__(kBlock) void group_init_kernel(GroupArgs g, int wit
   typedef typename Acc<T>::type F;
   typedef typename OrdKey<F>::bits KB;
   if (g.gate != nullptr && *g.gate == 0) return;
-  const int64_t n = g.B * g.N * g.K;
-  KB *gmax = static_cast<KB *>(g.gmax);
-  F *gsum = static_cast<F *>(g.gsum);
+  // a group's K keys and K sums lie side by side (one 64-byte line for eight floats): slot (node, k) of the keys
+  // is word node * 2K + k from gmax on, of the sums the same from gsum = gmax + K on
+  const int64_t n = g.B * g.N * g.gs;
+  KB *keys = static_cast<KB *>(g.gmax);
+  F *sums = reinterpret_cast<F *>(g.gmax);
   const KB empty = g.from_neg_inf ? OrdKey<F>::enc(-INFINITY) : group_empty_key<T>();
   for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlock) {
-    if (with_max) gmax[i] = empty;
-    gsum[i] = (F)0;
+    if (g.gs == g.K || ((i / g.K) & 1) != 0)
+      sums[i] = (F)0;
+    else if (with_max)
+      keys[i] = empty;
   }
 }
 
@@ -149,7 +154,7 @@ template <typename T, int C_> struct GroupMaxRun {
   static constexpr int U = 4;
   const T *src;
   A *gmax;
-  int64_t K;
+  int64_t K, gs;
   __device__ A identity() const { return (A)0; }
   __device__ void load(int64_t e, int64_t, int64_t col, int, A *x) const {
     const Vec<T, C> r = load_vec_stream<T, C>(src + e * K + col);
@@ -165,7 +170,7 @@ template <typename T, int C_> struct GroupMaxRun {
   bool check = true;
   __device__ void begin_row(int heads, int entries) { check = heads * 2 > entries; }
   __device__ void emit(int node, int64_t col, const A *x) const {
-    A *p = gmax + (int64_t)node * K + col;
+    A *p = gmax + (int64_t)node * gs + col;
     if (!check || x[0] > *p) __hip_atomic_fetch_max(p, x[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
 };
@@ -180,6 +185,7 @@ __global__ __launch_bounds__(kBlock) void group_max_run_kernel(ScatterArgs a, Gr
   p.src = static_cast<const T *>(g.src);
   p.gmax = static_cast<A *>(g.gmax);
   p.K = g.K;
+  p.gs = g.gs;
   run_wave<SERIAL>(a, lshift, rows_per_wave, p, s_stage[threadIdx.x / kWave]);
 }
 
@@ -211,7 +217,7 @@ template <typename T, int C_, int MODE> struct GroupSumRun : HotState<typename A
   A *gsum;
   const T *total;
   const float *count;
-  int64_t K;
+  int64_t K, gs;
   __device__ A identity() const { return (A)0; }
   __device__ void load(int64_t e, int64_t, int64_t col, int node, A *x) const {
     if constexpr (MODE == GS_SOFTMAX || MODE == GS_LOG_SOFTMAX || MODE == GS_LSE) {
@@ -222,7 +228,7 @@ template <typename T, int C_, int MODE> struct GroupSumRun : HotState<typename A
         return;
       }
       A m[C];
-      group_shift<T, C, MODE == GS_LSE>(gmax, (int64_t)node * K + col, m);
+      group_shift<T, C, MODE == GS_LSE>(gmax, (int64_t)node * gs + col, m);
 #pragma unroll
       for (int c = 0; c < C; ++c) {
         A z = round_elem<T>(to_acc<T>(r.v[c]) - m[c]);
@@ -260,7 +266,7 @@ template <typename T, int C_, int MODE> struct GroupSumRun : HotState<typename A
     to_memory(node, col, x);
   }
   __device__ void to_memory(int node, int64_t col, const A *x) const {
-    atomic_add_elem<A>(gsum + (int64_t)node * K + col, x[0]);
+    atomic_add_elem<A>(gsum + (int64_t)node * gs + col, x[0]);
   }
 };
 
@@ -280,6 +286,7 @@ __global__ __launch_bounds__(kBlock) void group_sum_run_kernel(ScatterArgs a, Gr
   p.total = static_cast<const T *>(g.total);
   p.count = g.count;
   p.K = g.K;
+  p.gs = g.gs;
   p.hot_init(s_hot, s_tags, hot_rlog, lshift + LogC<C>::value);
   run_wave<SERIAL>(a, lshift, rows_per_wave, p, s_stage[threadIdx.x / kWave]);
   p.hot.template flush<1>([&](int node, int j, const A *x) {
@@ -358,9 +365,10 @@ __global__ __launch_bounds__(kBlock) void group_finish_kernel(GroupArgs g) {
           store_vec_stream<T, VEC>(out + be * g.K + k0, r);
           continue;
         }
-        const Vec<F, VEC> s = load_vec<F, VEC>(gsum + slot);
+        const int64_t wslot = (bb[u] * g.N + idx[u]) * g.gs + k0;  // keys and sums of a group side by side
+        const Vec<F, VEC> s = load_vec<F, VEC>(gsum + wslot);
         F mx[VEC];
-        if (MODE == GS_SOFTMAX || MODE == GS_LOG_SOFTMAX) group_shift<T, VEC>(g.gmax, slot, mx);
+        if (MODE == GS_SOFTMAX || MODE == GS_LOG_SOFTMAX) group_shift<T, VEC>(g.gmax, wslot, mx);
 #pragma unroll
         for (int v = 0; v < VEC; ++v) {
           const F xv = to_acc<T>(x[u].v[v]);
@@ -400,8 +408,9 @@ __global__ __launch_bounds__(kBlock) void group_lse_finish_kernel(GroupArgs g) {
   T *out = static_cast<T *>(g.out);
   const F eps = (F)g.eps;
   for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlock) {
-    const F m = OrdKey<F>::dec(gmax[i]);
-    const F l = round_elem<T>(log_acc(round_elem<T>(round_elem<T>(gsum[i]) + eps)));
+    const int64_t node = i / g.K, w = node * g.gs + (i - node * g.K);
+    const F m = OrdKey<F>::dec(gmax[w]);
+    const F l = round_elem<T>(log_acc(round_elem<T>(round_elem<T>(gsum[w]) + eps)));
     F o = round_elem<T>(l + m);
     if (o != o || o == -INFINITY) o = (F)0;
     if (o == INFINITY) o = to_acc<T>(ElemLim<T>::max());
@@ -418,7 +427,8 @@ __global__ __launch_bounds__(kBlock) void group_std_finish_kernel(GroupArgs g) {
   T *out = static_cast<T *>(g.out);
   for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlock) {
     const F div = group_divisor<T>(g.count[i / g.K], g.unbiased);
-    out[i] = from_acc<T>(sqrt_acc(round_elem<T>(round_elem<T>(gsum[i]) / div)));
+    const int64_t node = i / g.K;
+    out[i] = from_acc<T>(sqrt_acc(round_elem<T>(round_elem<T>(gsum[node * g.gs + (i - node * g.K)]) / div)));
   }
 }
 
