@@ -505,7 +505,12 @@ size_t ts_scatter_workspace_bytes(int64_t B, int64_t E, int64_t K, int64_t N, in
   }
   if (reduce == TS_SUM && kAccBytes[dtype] >= 4) {  // table slots: int32 for int32, 8 bytes for the other types
     const size_t binned = bin_plan(B, E, K, N, kElemBytes[dtype], nullptr, 0, any_size, dtype == TS_I32 ? 4 : 8, false, true).bytes;
-    if (binned == 0) return 0;
+    if (binned == 0) {
+      // one word for the sample of the index that keeps a sorted one away from the table kernel
+      const bool table = is_float_dtype(dtype) && kElemBytes[dtype] <= 4 && env_int("TS_SCATTER_LDS", 1) == 1 &&
+                         sum_table_by_size(B, E, K, N, kElemBytes[dtype]);
+      return table ? 256 : 0;
+    }
     const SortedRoute sr = sorted_route_plan(B, E, K, N, dtype, reduce);
     return binned + (sr.ok ? sr.ptr_bytes + sr.csr_bytes : 0);
   }
@@ -578,6 +583,8 @@ int ts_scatter_with_workspace(const void *src, const int64_t *index, void *out, 
       a.route_ptr = reinterpret_cast<int64_t *>(static_cast<char *>(workspace) + bin_bytes);
     }
   }
+  if (reduce == TS_SUM && bin_bytes == 0 && workspace != nullptr && workspace_bytes >= 256 && aligned16(workspace))
+    a.order_ws = static_cast<int *>(workspace);
   const int rc = dispatch_scatter(dtype, a, reduce, vec, static_cast<hipStream_t>(stream));
   if (rc != TS_OK || route_flag == nullptr) return rc;
   // the row pointers of a sorted index come from the place pass of the buckets (bin_place_kernel)

@@ -212,6 +212,8 @@ struct ScatterArgs {
   size_t bin_ws_bytes = 0;
   int bin_any_size = 0;    // tuning aid / tests: also for inputs below the size from which it pays
   const int *skip_flag = nullptr;  // sum kernels: leave at once if *skip_flag != 0 (the binned pass did the work)
+  int skip_inverse = 0;            // ... if *skip_flag == 0 instead
+  int *order_ws = nullptr;         // sum of narrow rows: a word of scratch for the sample of the index that picks the kernel
   int skew_probe = 1;              // min/max: sample the index for skew (needs 256 bytes of workspace): 0 never, 2 at any size
   const int *skew_flag = nullptr;  // min/max kernels behind the probe: run only if (*skew_flag != 0) == (skew_want != 0)
   int skew_want = 0;
@@ -1305,7 +1307,7 @@ constexpr int kLdsAddBlock = 1024;    // one table per 16 wavefronts: every work
 template <typename T>
 __global__ __launch_bounds__(kLdsAddBlock) void scatter_add_lds_kernel(ScatterArgs a, int tn_mask, int64_t epb) {
   constexpr int U = 4;
-  if (a.skip_flag != nullptr && *a.skip_flag != 0) return;
+  if (a.skip_flag != nullptr && (*a.skip_flag != 0) != (a.skip_inverse != 0)) return;
   // double slots: ds_add_f32 loses its rate when many lanes meet on one address (a hub, or a sorted index whose
   // neighbouring entries share a row), ds_add_f64 does not (Zipf(1.2) index, K = 8: 391 -> 263 us; sorted: 476 -> 177 us)
   typedef double LdsAcc;
@@ -1495,6 +1497,14 @@ inline unsigned scatter_grid(int64_t n_edges, int64_t kv, int block, int U) {
   return (unsigned)(blocks < cap ? blocks : cap);
 }
 
+// sizes from which a floating-point sum goes through the LDS table kernel (the crossovers are with its use below)
+inline bool sum_table_by_size(int64_t B, int64_t E, int64_t K, int64_t N, int elem_bytes) {
+  const int64_t n_edges = B * E, n_src = n_edges * K;
+  if (n_src < ((int64_t)1 << 17)) return false;
+  if (n_edges >= 32 * B * N) return K < 32 || n_src * elem_bytes < (int64_t)300000000;
+  return K < 32 && (n_src >= ((int64_t)1 << 22) || n_edges >= ((int64_t)1 << 18));
+}
+
 template <typename T, int VEC>
 int launch_scatter_v(const ScatterArgs &args, int reduce, hipStream_t stream) {
   ScatterArgs a = args;
@@ -1554,17 +1564,26 @@ int launch_scatter_v(const ScatterArgs &args, int reduce, hipStream_t stream) {
           // the run kernel with its hot rows above (9-10 M entries: a sorted index, such as the batch vector of a
           // pooling layer, takes 450 us there and 940 us through the table; an unsorted one has the workspace path)
           const bool use_lds = a.lds_cache && a.sk == 0 && tn >= 64 && a.B * a.N < 0x7FFFFFFFll &&
-                               (a.lds_cache == 2 ||
-                                (n_src >= ((int64_t)1 << 17) &&
-                                 (n_edges >= 32 * a.B * a.N ? (a.K < 32 || n_src * (int64_t)sizeof(T) < (int64_t)300000000)
-                                                            : (a.K < 32 && (n_src >= ((int64_t)1 << 22) ||
-                                                                            n_edges >= ((int64_t)1 << 18))))));
+                               (a.lds_cache == 2 || sum_table_by_size(a.B, a.E, a.K, a.N, (int)sizeof(T)));
           if (use_lds) {
+            // The table is for an index in no particular order. One that is sorted does better through the run
+            // kernel below (9 M entries of the graph of C3, sorted: K = 8 343 against 156 us, K = 4 152 / 96,
+            // K = 1 60 / 44; shuffled: 448 / 463), so with a word of scratch a sample of the index decides on the
+            // device: the table returns at once if the index looks sorted, the run kernel if not.
+            const bool sampled = a.lds_cache != 2 && a.order_ws != nullptr && a.skip_flag == nullptr && a.run_reduce &&
+                                 n_edges >= 2 * kBinBlock;
+            ScatterArgs t = a;
+            if (sampled) {
+              hipLaunchKernelGGL(bin_sample_kernel, dim3(1), dim3(kBinBlock), 0, stream, a, a.order_ws);
+              t.skip_flag = a.order_ws;
+              t.skip_inverse = 1;
+              a.skip_flag = a.order_ws;
+            }
             const int64_t epb = per_cu_chunk_edges(a.lds_epb, n_edges, 16384 / a.K > 256 ? 16384 / a.K : 256,
                                                    131072 / a.K > 2048 ? 131072 / a.K : 2048);
             hipLaunchKernelGGL(scatter_add_lds_kernel<T>, dim3((unsigned)((n_edges + epb - 1) / epb)),
-                               dim3(kLdsAddBlock), 0, stream, a, tn - 1, epb);
-            return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
+                               dim3(kLdsAddBlock), 0, stream, t, tn - 1, epb);
+            if (!sampled) return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
           }
         }
         {

@@ -919,6 +919,49 @@ def test_scatter_sum_lds_aggregated_variant(capi, oracle, shape, dtype, monkeypa
     assert torch.equal(cnt.cpu(), torch.bincount(index1, minlength=N).float())
 
 
+@pytest.mark.parametrize("shape,kind,dtype", product(
+    [(1, 300000, 8, 40000), (1, 400000, 1, 90000), (2, 140000, 4, 9000), (1, 270000, 12, 30000)],
+    ["sorted", "shuffled", "zipf"], [torch.float32, torch.bfloat16]))
+def test_scatter_sum_narrow_rows_sample_picks_the_kernel(capi, oracle, shape, kind, dtype):
+    """Sums of narrow rows at sizes that the accumulator table takes: with 256 bytes of workspace a sample of the
+    index sends a sorted index to the run kernel instead (word 0 of the workspace: 0) and any other to the table
+    (1). Either way the sum is the oracle's, with and without previous content in out."""
+    B, E, K, N = shape
+    rng = np.random.default_rng(E + K)
+    src = torch.from_numpy(rng.standard_normal(size=(B, E, K))).to(dtype)
+    if kind == "zipf":
+        p = np.arange(1, N + 1, dtype=np.float64) ** -1.2
+        idx = rng.choice(N, size=E, p=p / p.sum())
+    else:
+        idx = rng.integers(0, N, size=E)
+        if kind == "sorted":
+            idx = np.sort(idx)
+    index1 = torch.from_numpy(idx)
+    index = index1.view(1, E, 1).expand(B, E, K)
+    L = capi.lib()
+    need = L.ts_scatter_workspace_bytes(capi._i(B), capi._i(E), capi._i(K), capi._i(N), capi.DTYPE[dtype], capi.SUM)
+    assert need == 256
+    exact = oracle.scatter(src.double(), index, 1, None, N, "sum")[0]
+    absum = oracle.scatter(src.double().abs(), index, 1, None, N, "sum")[0]
+    for out_given in (False, True):
+        prev = torch.from_numpy(rng.standard_normal(size=(B, N, K))).to(dtype)
+        out = prev.clone().to(DEV) if out_given else torch.empty((B, N, K), dtype=dtype, device=DEV)
+        ws = capi.scatter_with_workspace(src.to(DEV), index1.to(DEV), out, None, B, E, K, N, 0, 1, 0, capi.SUM,
+                                         out_given)
+        torch.cuda.synchronize()
+        assert int(ws[:4].view(torch.int32).item()) == (0 if kind == "sorted" else 1), kind
+        want = exact + (prev.double() if out_given else 0)
+        rtol = 1e-5 if dtype == torch.float32 else 1e-2
+        err = (out.cpu().double() - want).abs()
+        bound = rtol * want.abs() + rtol * (absum + (prev.double().abs() if out_given else 0)).clamp(min=1e-30)
+        assert bool((err <= bound).all()), float((err - bound).max())
+        plain = prev.clone().to(DEV) if out_given else torch.empty((B, N, K), dtype=dtype, device=DEV)
+        capi.scatter(src.to(DEV), index1.to(DEV), plain, None, B, E, K, N, 0, 1, 0, capi.SUM, out_given)
+        torch.cuda.synchronize()
+        perr = (plain.cpu().double() - want).abs()
+        assert bool((perr <= bound).all()), "without workspace"
+
+
 RUN_SHAPES = [
     # B, E, K, N
     (1, 5000, 1, 600), (1, 3000, 2, 40), (1, 2000, 3, 300), (2, 1500, 5, 64), (1, 4000, 16, 500),
