@@ -52,6 +52,9 @@ def parse_args():
     ap.add_argument("--sweep-thresholds", action="store_true",
                     help="time scatter sum / max just either side of every size threshold of the dispatcher and "
                          "flag neighbours that differ by more than 1.5x")
+    ap.add_argument("--sweep-orders", action="store_true",
+                    help="scatter sum / max for one shape under a sorted, a shuffled and a skewed index, fp32 and bf16; "
+                         "flags a sorted index that is slower than a shuffled one and 16-bit types far behind fp32")
     ap.add_argument("--probe", action="store_true",
                     help="counter-collection mode for rocprofv3 --pmc: a few launches of the dominant kernels "
                          "next to copies of known size, nothing timed")
@@ -530,6 +533,44 @@ def sweep_thresholds():
     print(json.dumps({"probe": "thresholds", "cliffs": flagged, "rows": rows}))
 
 
+def sweep_orders():
+    """scatter sum / max through the operators for the same shape under a sorted, a shuffled and a Zipf(1.2) index,
+    fp32 and bf16: the thresholds of the dispatcher are sizes, and a kernel picked by size can be the wrong one for
+    the order of the index or for the element type (found that way: the accumulator table for narrow rows was
+    twice as slow as the run kernel under a sorted index, and 30-300x slower for 16-bit floats under any other).
+    Flags: a sorted index more than 1.5x slower than the same index shuffled; bf16 more than 8x slower than fp32."""
+    import numpy as np
+    import torch
+    import pytorch_scatter_amd as ts
+    dev = torch.device("cuda:0")
+    rng = np.random.default_rng(0)
+    rows, flagged = [], 0
+    with torch.no_grad():
+        for E, N in ((4_000_000, 400_000), (4_000_000, 4_000), (500_000, 50_000)):
+            uni = rng.integers(0, N, size=E)
+            p = np.arange(1, N + 1, dtype=np.float64) ** -1.2
+            zipf = rng.choice(N, size=E, p=p / p.sum())
+            orders = {"sorted": np.sort(uni), "shuffled": uni, "zipf": zipf}
+            index = {k: torch.from_numpy(v.astype(np.int64)).to(dev) for k, v in orders.items()}
+            for K in (1, 8, 32):
+                t = {}
+                for dtype in (torch.float32, torch.bfloat16):
+                    src = torch.randn((E, K), device=dev).to(dtype)
+                    for order, idx in index.items():
+                        for reduce, fn in (("sum", ts.scatter_sum), ("max", ts.scatter_max)):
+                            t[dtype, order, reduce] = event_time(lambda: fn(src, idx, 0, None, N), 5)
+                    del src
+                for (dtype, order, reduce), v in t.items():
+                    slow_sorted = order == "sorted" and v > 1.5 * t[dtype, "shuffled", reduce]
+                    slow_16 = dtype == torch.bfloat16 and v > 8 * t[torch.float32, order, reduce]
+                    rows.append({"E": E, "N": N, "K": K, "dtype": str(dtype)[6:], "order": order, "reduce": reduce,
+                                 "us": round(v * 1e6, 1), "flag": bool(slow_sorted or slow_16)})
+                    flagged += bool(slow_sorted or slow_16)
+    for r in rows:
+        print(r, file=sys.stderr)
+    print(json.dumps({"probe": "orders", "flagged": flagged, "rows": rows}))
+
+
 def probe():
     """Launch sequence for `rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE -- python3 bench.py --probe`:
     1. torch copy of 1 GiB (plain loads/stores, known size: calibrates the counters);
@@ -616,6 +657,8 @@ def main():
         return probe_atomics()
     if args.sweep_thresholds:
         return sweep_thresholds()
+    if args.sweep_orders:
+        return sweep_orders()
     if args.probe:
         return probe()
     if args.probe_scatter:
