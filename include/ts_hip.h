@@ -179,6 +179,12 @@ int ts_segment_mean_coo_backward(const void *grad_out, const int64_t *index,
  *   out_given != 0: accumulate into out; arg_out (MIN/MAX) is fully written:
  *                   E where no entry strictly beat the previous content.
  * Ties keep the smallest e (the CPU rule, csrc/cpu/reducer.h:63-67).
+ * SUM of 8- and 16-bit integers, and MUL of any type, have no hardware atomic: they loop on a compare-and-swap
+ * of the word around the element, as the reference does (csrc/cuda/atomics.cuh), and that loop slows down with
+ * the square of the entries that meet in one output row. For such sums a caller widens to int32 first (the
+ * operator library does: the wrap-around of an int32 sum agrees with the narrow type's modulo 2^8 / 2^16);
+ * products combine inside the wavefront before the loop (one value per entry, 30 % of 100 k entries on one
+ * row: 418 -> 2 ms; eight values per entry: 554 -> 115 ms).
  * The index element of (b, e, k) is index[b*sb + e*se + k*sk]; a 1-D index
  * broadcast along dim is sb = 0, se = 1, sk = 0.
  */

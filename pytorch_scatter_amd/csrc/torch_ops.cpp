@@ -164,6 +164,21 @@ std::tuple<Tensor, OptTensor> scatter_hip(Tensor src, Tensor index, int64_t dim,
   for (int64_t i = 0; i < index.dim() - 1; i++) check_input(src.size(i) >= index.size(i));
   TORCH_CHECK(index.scalar_type() == at::kLong, "index must be int64");
 
+  // 8- and 16-bit integers have no atomic add: ts_scatter adds them with a compare-and-swap loop on the 32-bit
+  // word around the element, and the cost of that loop grows with the square of the entries that meet in one row
+  // (100 k entries, 30 % of them on one row: 0.3 - 0.7 s; int32: 0.3 ms). Their sums run in int32 instead, whose
+  // wrap-around agrees with that of the narrow type modulo 2^8 / 2^16, and are cast back (also faster without
+  // any contention: 2.25 M entries in random order, one int8 each: 458 against 97 us).
+  const auto st = src.scalar_type();
+  if (reduce == TS_SUM && (st == at::kChar || st == at::kByte || st == at::kShort) && src.numel() > 0) {
+    OptTensor wide_out;
+    if (optional_out.has_value()) wide_out = optional_out.value().to(at::kInt);
+    Tensor narrow = std::get<0>(scatter_hip(src.to(at::kInt), index, dim, wide_out, dim_size, reduce)).to(st);
+    if (!optional_out.has_value()) return std::make_tuple(narrow, OptTensor());
+    optional_out.value().copy_(narrow);
+    return std::make_tuple(optional_out.value(), OptTensor());
+  }
+
   src = src.contiguous();
   Tensor out;
   if (optional_out.has_value()) {

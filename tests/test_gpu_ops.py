@@ -544,3 +544,48 @@ def test_scatter_large_sorted_index_through_the_operators(ts, oracle, reduce):
             count = torch.bincount(idx, minlength=N).clamp(min=1).float().view(-1, 1)
             expect = (grad / count if reduce == "mean" else grad)[idx]
             assert torch.allclose(x.grad.cpu(), expect, rtol=1e-6, atol=1e-7)
+
+
+@pytest.mark.parametrize("dtype,K", product([torch.int8, torch.uint8, torch.int16], [1, 6]))
+def test_scatter_sum_of_narrow_integers_under_a_hub(ts, dtype, K):
+    """8- and 16-bit integer sums run in int32 and are cast back: the result wraps like the narrow type's own
+    arithmetic (what the reference's atomAdd on these types gives), also on top of previous content in `out`,
+    and a row that takes a third of the entries does not take longer than the rest."""
+    g = torch.Generator().manual_seed(3)
+    E, N = 60000, 500
+    index = torch.where(torch.rand(E, generator=g) < 0.3, torch.tensor(7), torch.randint(0, N, (E,), generator=g))
+    src = torch.randint(0, 100, (E, K), generator=g).to(dtype)
+    prev = torch.randint(0, 50, (N, K), generator=g).to(dtype)
+    want = torch.zeros((N, K), dtype=torch.int64).index_add_(0, index, src.long())
+    got = ts.scatter(src.to(DEV), index.to(DEV), 0, None, N, "sum")
+    assert got.dtype == dtype and torch.equal(got.cpu(), want.to(dtype))
+    out = prev.clone().to(DEV)
+    res = ts.scatter(src.to(DEV), index.to(DEV), 0, out, None, "sum")
+    assert res.data_ptr() == out.data_ptr()
+    assert torch.equal(out.cpu(), (want + prev.long()).to(dtype))
+    mean = ts.scatter(src.to(DEV), index.to(DEV), 0, None, N, "mean")
+    count = torch.bincount(index, minlength=N).clamp(min=1).to(dtype).view(N, 1)
+    assert torch.equal(mean.cpu(), torch.div(want.to(dtype), count, rounding_mode="floor"))
+
+
+@pytest.mark.parametrize("dtype,K", product([torch.float32, torch.float64, torch.int32], [1, 5]))
+def test_scatter_mul_under_a_hub(ts, dtype, K):
+    """Products of a row that takes a third of the entries: the lanes of a wavefront combine before the
+    compare-and-swap; the result is the product whatever the order."""
+    g = torch.Generator().manual_seed(4)
+    E, N = 30000, 300
+    index = torch.where(torch.rand(E, generator=g) < 0.3, torch.tensor(11), torch.randint(0, N, (E,), generator=g))
+    if dtype == torch.int32:
+        src = torch.where(torch.rand((E, K), generator=g) < 0.01, 3, 1).to(dtype) * \
+            torch.where(torch.rand((E, K), generator=g) < 0.5, 1, -1).to(dtype)
+    else:
+        src = (torch.rand((E, K), generator=g, dtype=torch.float64) * 0.02 + 0.99).to(dtype)
+    got = ts.scatter(src.to(DEV), index.to(DEV), 0, None, N, "mul").cpu()
+    want = torch.ones((N, K), dtype=torch.float64)
+    want = want.scatter_reduce(0, index.view(E, 1).expand(E, K), src.double(), "prod")
+    if dtype == torch.int32:
+        wrapped = torch.ones((N, K), dtype=torch.int64).scatter_reduce(
+            0, index.view(E, 1).expand(E, K), src.long(), "prod")  # at most 3^k: fits 64 bits for these inputs
+        assert torch.equal(got.long(), wrapped.to(torch.int32).long())
+    else:
+        assert torch.allclose(got.double(), want, rtol=1e-4 if dtype == torch.float32 else 1e-11)
