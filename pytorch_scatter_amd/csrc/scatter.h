@@ -1348,6 +1348,11 @@ constexpr int kLdsAcc = 8192;         // accumulators of the table (64 KB of dou
 constexpr int kLdsAccRows = 4096;     // 16 KB of tags
 constexpr int kLdsAddBlock = 1024;    // one table per 16 wavefronts: every workgroup adds its table to out once
 
+// slot of the accumulator table: double for the floating types, the element's own width for int32 / int64
+template <typename T> struct TableSlot { typedef double type; };
+template <> struct TableSlot<int32_t> { typedef int32_t type; };
+template <> struct TableSlot<int64_t> { typedef long long type; };
+
 // What leaves the table for `out` (rows that missed it, and the table itself at the end). The rows of a hub are
 // in every workgroup's table, so thousands of workgroups add to the same elements: 16-bit floats go through the
 // packed-pair add of the hardware, not through a compare-and-swap loop (4 M entries of 8 bf16 under a Zipf(1.2)
@@ -1363,9 +1368,10 @@ template <typename T>
 __global__ __launch_bounds__(kLdsAddBlock) void scatter_add_lds_kernel(ScatterArgs a, int tn_mask, int64_t epb) {
   constexpr int U = 4;
   if (a.skip_flag != nullptr && (*a.skip_flag != 0) != (a.skip_inverse != 0)) return;
-  // double slots: ds_add_f32 loses its rate when many lanes meet on one address (a hub, or a sorted index whose
-  // neighbouring entries share a row), ds_add_f64 does not (Zipf(1.2) index, K = 8: 391 -> 263 us; sorted: 476 -> 177 us)
-  typedef double LdsAcc;
+  // double slots for the floating types: ds_add_f32 loses its rate when many lanes meet on one address (a hub, or a
+  // sorted index whose neighbouring entries share a row), ds_add_f64 does not (Zipf(1.2) index, K = 8: 391 -> 263 us;
+  // sorted: 476 -> 177 us). Integers keep their own width (their sums wrap, which a double cannot follow).
+  typedef typename TableSlot<T>::type LdsAcc;
   __shared__ LdsAcc s_acc[kLdsAcc];
   __shared__ int32_t s_tags[kLdsAccRows];
   const int K = (int)a.K;
@@ -1385,13 +1391,13 @@ __global__ __launch_bounds__(kLdsAddBlock) void scatter_add_lds_kernel(ScatterAr
   if (m.active) {
     for (int64_t be0 = be_lo + m.el; be0 < be_hi; be0 += (int64_t)m.epp * U) {
       for (int k = m.cl; k < K; k += m.L) {
-        float x[U];
+        LdsAcc x[U];
         int64_t idx[U], bb[U], ee[U];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
           const int64_t be = be0 + (int64_t)u * m.epp;
           split_edge(be < be_hi ? be : be0, a.B, a.E, bb[u], ee[u]);
-          x[u] = src ? (float)to_acc<T>(src[(bb[u] * a.E + ee[u]) * a.K + k]) : 1.0f;
+          x[u] = src ? (LdsAcc)to_acc<T>(src[(bb[u] * a.E + ee[u]) * a.K + k]) : (LdsAcc)1;
           idx[u] = a.index[bb[u] * a.sb + ee[u] * a.se];
         }
 #pragma unroll
@@ -1406,7 +1412,7 @@ __global__ __launch_bounds__(kLdsAddBlock) void scatter_add_lds_kernel(ScatterAr
             tag = old == -1 ? node : old;
           }
           if (tag == node)
-            __hip_atomic_fetch_add(&s_acc[row * K + k], (LdsAcc)x[u], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            __hip_atomic_fetch_add(&s_acc[row * K + k], x[u], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
           else
             table_add_out<T>(out + (int64_t)node * a.K + k, from_acc<T>((typename Acc<T>::type)x[u]), out, out_end);
         }
@@ -1427,8 +1433,8 @@ __global__ __launch_bounds__(kLdsAddBlock) void scatter_add_lds_kernel(ScatterAr
     }
   }
   for (int i = threadIdx.x; i < tn * K; i += kLdsAddBlock) {
-    const float v = (float)s_acc[i];
-    if (v == 0.0f) continue;
+    const LdsAcc v = s_acc[i];
+    if (v == (LdsAcc)0) continue;
     const int row = i / K;
     table_add_out<T>(out + (int64_t)s_tags[row] * a.K + (i - row * K), from_acc<T>((typename Acc<T>::type)v), out, out_end);
   }
@@ -1496,7 +1502,9 @@ __global__ __launch_bounds__(kBlock) void scatter_arg_wide_kernel(ScatterArgs a)
     const int64_t idx = a.index[b * a.sb + e * a.se + k * a.sk];
     if (idx < 0 || idx >= a.N) continue;
     const int64_t o = (b * a.N + idx) * a.K + k;
-    if (src[i] == out[o]) __hip_atomic_fetch_min(a.arg_out + o, e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    // the position only ever goes down: read it first (among many equal values nearly every entry is too late)
+    if (src[i] == out[o] && e < __hip_atomic_load(a.arg_out + o, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))
+      __hip_atomic_fetch_min(a.arg_out + o, e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
 }
 
@@ -1616,7 +1624,8 @@ int launch_scatter_v(const ScatterArgs &args, int reduce, hipStream_t stream) {
       // (4 lines per instruction for fp32 instead of 16 with 4 elements per lane)
       const unsigned g = scatter_grid(n_edges, a.K, kBlock, 4);
       if (reduce == TS_SUM) {
-        if constexpr (__is_same(T, float) || __is_same(T, bf16_t) || __is_same(T, f16_t)) {
+        if constexpr (__is_same(T, float) || __is_same(T, bf16_t) || __is_same(T, f16_t) || __is_same(T, double) ||
+                      __is_same(T, int32_t) || __is_same(T, int64_t)) {
           // many entries per output slot: reduce in LDS first (see scatter_add_lds_kernel)
           int tn = 1;
           while ((int64_t)tn * 2 * a.K <= kLdsAcc && tn * 2 <= kLdsAccRows) tn *= 2;
