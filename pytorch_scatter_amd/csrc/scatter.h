@@ -1471,6 +1471,25 @@ __global__ __launch_bounds__(kBlock) void scatter_key_final_kernel(ScatterArgs a
 }
 
 // ---- two-pass min/max for 64-bit element types --------------------------------
+// First pass: the value, by compare-and-swap. A slot that an entry strictly improves gets kArgOpen into its arg_out
+// (filled with E before): the second pass looks for positions only there, so a slot in which no entry beat the
+// initial or previous content keeps E even if an entry equals that content.
+constexpr int64_t kArgOpen = INT64_MAX;
+template <typename T, bool IS_MAX> __device__ __forceinline__ bool wide_improve(T *slot, T val) {
+  static_assert(sizeof(T) == 8, "");
+  uint64_t *word = reinterpret_cast<uint64_t *>(slot);
+  uint64_t old = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  uint64_t desired;
+  __builtin_memcpy(&desired, &val, 8);
+  while (true) {
+    T cur;
+    __builtin_memcpy(&cur, &old, 8);
+    if (!(IS_MAX ? val > cur : val < cur)) return false;
+    if (__hip_atomic_compare_exchange_strong(word, &old, desired, __ATOMIC_RELAXED, __ATOMIC_RELAXED,
+                                             __HIP_MEMORY_SCOPE_AGENT))
+      return true;
+  }
+}
 template <typename T, bool IS_MAX>
 __global__ __launch_bounds__(kBlock) void scatter_minmax_wide_kernel(ScatterArgs a) {
   const T *src = static_cast<const T *>(a.src);
@@ -1484,11 +1503,95 @@ __global__ __launch_bounds__(kBlock) void scatter_minmax_wide_kernel(ScatterArgs
     const int64_t idx = a.index[b * a.sb + e * a.se + k * a.sk];
     if (idx < 0 || idx >= a.N) continue;
     const T val = src[i];
-    atomic_rmw<T>(out + (b * a.N + idx) * a.K + k, [val](T cur) {
-      return IS_MAX ? (val > cur ? val : cur) : (val < cur ? val : cur);
-    });
+    const int64_t o = (b * a.N + idx) * a.K + k;
+    if (wide_improve<T, IS_MAX>(out + o, val)) a.arg_out[o] = kArgOpen;
   }
 }
+// order-preserving 64-bit keys of the 64-bit element types; 0 stands for "no entry" in the table below
+template <typename T> struct WideKey;
+template <> struct WideKey<int64_t> {
+  __device__ static uint64_t enc(int64_t v) { return (uint64_t)v ^ 0x8000000000000000ull; }
+  __device__ static int64_t dec(uint64_t k) { return (int64_t)(k ^ 0x8000000000000000ull); }
+  __device__ static bool is_nan(int64_t) { return false; }
+};
+template <> struct WideKey<double> {
+  __device__ static uint64_t enc(double v) {
+    uint64_t u = (uint64_t)__double_as_longlong(v);
+    if (u == 0x8000000000000000ull) u = 0;  // -0.0 and +0.0 compare equal
+    return (u >> 63) ? ~u : (u | 0x8000000000000000ull);
+  }
+  __device__ static double dec(uint64_t k) {
+    return __longlong_as_double((long long)((k >> 63) ? (k & 0x7FFFFFFFFFFFFFFFull) : ~k));
+  }
+  __device__ static bool is_nan(double v) { return v != v; }
+};
+
+// First pass of min / max for 64-bit elements when many entries meet in an output slot: the compare-and-swap
+// loop of scatter_minmax_wide_kernel starts with a read that is coherent across the XCDs, and those reads queue
+// up at the memory side when they fall on few lines (16.7 M entries onto 64 k slots: 4.4 ms, 3.8 G entries/s).
+// Here a workgroup keeps a table of keys in LDS for the rows it meets (tags as in scatter_add_lds_kernel) and
+// sends every touched slot to memory once, at the end; rows that miss the table go the old way.
+template <typename T, bool IS_MAX>
+__global__ __launch_bounds__(kLdsAddBlock) void scatter_minmax_wide_lds_kernel(ScatterArgs a, int tn_mask, int64_t epb) {
+  constexpr int U = 4;
+  __shared__ unsigned long long s_key[kLdsAcc];
+  __shared__ int32_t s_tags[kLdsAccRows];
+  const int K = (int)a.K;
+  const int tn = tn_mask + 1;
+  for (int i = threadIdx.x; i < tn * K; i += kLdsAddBlock) s_key[i] = 0;
+  for (int i = threadIdx.x; i < tn; i += kLdsAddBlock) s_tags[i] = -1;
+  __syncthreads();
+  const T *src = static_cast<const T *>(a.src);
+  T *out = static_cast<T *>(a.out);
+  const EdgeLanes m = edge_lanes(K, kLdsAddBlock);
+  const int64_t be_lo = (int64_t)blockIdx.x * epb;
+  int64_t be_hi = be_lo + epb;
+  if (be_hi > a.B * a.E) be_hi = a.B * a.E;
+  auto to_memory = [&](int64_t o, T val) {
+    if (wide_improve<T, IS_MAX>(out + o, val)) a.arg_out[o] = kArgOpen;
+  };
+  if (m.active) {
+    for (int64_t be0 = be_lo + m.el; be0 < be_hi; be0 += (int64_t)m.epp * U) {
+      for (int k = m.cl; k < K; k += m.L) {
+        T x[U];
+        int64_t idx[U], bb[U], ee[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const int64_t be = be0 + (int64_t)u * m.epp;
+          split_edge(be < be_hi ? be : be0, a.B, a.E, bb[u], ee[u]);
+          x[u] = src[(bb[u] * a.E + ee[u]) * a.K + k];
+          idx[u] = a.index[bb[u] * a.sb + ee[u] * a.se];
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          if (be0 + (int64_t)u * m.epp >= be_hi) continue;
+          if (idx[u] < 0 || idx[u] >= a.N || WideKey<T>::is_nan(x[u])) continue;  // a NaN never wins
+          const int node = (int)(bb[u] * a.N + idx[u]);
+          const int row = node & tn_mask;
+          int tag = s_tags[row];
+          if (tag == -1) {
+            const int old = atomicCAS(&s_tags[row], -1, node);
+            tag = old == -1 ? node : old;
+          }
+          const uint64_t enc = WideKey<T>::enc(x[u]);
+          const unsigned long long key = IS_MAX ? enc : ~enc;
+          if (tag == node && key != 0)
+            __hip_atomic_fetch_max(&s_key[row * K + k], key, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+          else
+            to_memory((int64_t)node * a.K + k, x[u]);
+        }
+      }
+    }
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < tn * K; i += kLdsAddBlock) {
+    const unsigned long long key = s_key[i];
+    if (key == 0) continue;
+    const int row = i / K;
+    to_memory((int64_t)s_tags[row] * a.K + (i - row * K), WideKey<T>::dec(IS_MAX ? key : ~key));
+  }
+}
+
 template <typename T>
 __global__ __launch_bounds__(kBlock) void scatter_arg_wide_kernel(ScatterArgs a) {
   const T *src = static_cast<const T *>(a.src);
@@ -1502,9 +1605,11 @@ __global__ __launch_bounds__(kBlock) void scatter_arg_wide_kernel(ScatterArgs a)
     const int64_t idx = a.index[b * a.sb + e * a.se + k * a.sk];
     if (idx < 0 || idx >= a.N) continue;
     const int64_t o = (b * a.N + idx) * a.K + k;
-    // the position only ever goes down: read it first (among many equal values nearly every entry is too late)
-    if (src[i] == out[o] && e < __hip_atomic_load(a.arg_out + o, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))
-      __hip_atomic_fetch_min(a.arg_out + o, e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (src[i] != out[o]) continue;
+    // only slots that the first pass improved (no longer E); the position only ever goes down, so read it first
+    // (among many equal values nearly every entry is too late)
+    const int64_t seen = __hip_atomic_load(a.arg_out + o, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (seen != a.E && e < seen) __hip_atomic_fetch_min(a.arg_out + o, e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
 }
 
@@ -1715,10 +1820,24 @@ int launch_scatter_v(const ScatterArgs &args, int reduce, hipStream_t stream) {
         hipLaunchKernelGGL(fill_kernel<T>, dim3(g_out), dim3(kBlock), 0, stream, out, n_out, init);
       hipLaunchKernelGGL(fill_kernel<int64_t>, dim3(g_out), dim3(kBlock), 0, stream, a.arg_out, n_out, a.E);
       if (n_src > 0) {
-        if (is_max)
+        // several entries per output slot: keys meet in LDS first (scatter_minmax_wide_lds_kernel)
+        int tn = 1;
+        while ((int64_t)tn * 2 * a.K <= kLdsAcc && tn * 2 <= kLdsAccRows) tn *= 2;
+        const bool table = a.lds_cache && a.sk == 0 && tn >= 16 && a.B * a.N < 0x7FFFFFFFll &&
+                           (a.lds_cache == 2 || (n_edges >= ((int64_t)1 << 17) && n_edges >= 4 * a.B * a.N));
+        if (table) {
+          const int64_t epb = per_cu_chunk_edges(a.lds_epb, n_edges, 16384 / a.K > 256 ? 16384 / a.K : 256,
+                                                 131072 / a.K > 2048 ? 131072 / a.K : 2048);
+          const dim3 gt((unsigned)((n_edges + epb - 1) / epb));
+          if (is_max)
+            hipLaunchKernelGGL((scatter_minmax_wide_lds_kernel<T, true>), gt, dim3(kLdsAddBlock), 0, stream, a, tn - 1, epb);
+          else
+            hipLaunchKernelGGL((scatter_minmax_wide_lds_kernel<T, false>), gt, dim3(kLdsAddBlock), 0, stream, a, tn - 1, epb);
+        } else if (is_max) {
           hipLaunchKernelGGL((scatter_minmax_wide_kernel<T, true>), dim3(g_src), dim3(kBlock), 0, stream, a);
-        else
+        } else {
           hipLaunchKernelGGL((scatter_minmax_wide_kernel<T, false>), dim3(g_src), dim3(kBlock), 0, stream, a);
+        }
       }
       if (!a.out_given)
         hipLaunchKernelGGL(mask_init_kernel<T>, dim3(g_out), dim3(kBlock), 0, stream, out, n_out, init);

@@ -532,15 +532,26 @@ def test_scatter(capi, oracle, shape, reduce, dtype):
 
 @pytest.mark.parametrize("shape,reduce,dtype", product(
     [(1, 30000, 1, 500), (1, 9000, 32, 300), (2, 5000, 8, 40), (1, 4000, 12, 70000)],
-    ["min", "max"], [torch.float32, torch.bfloat16, torch.int32]))
+    ["min", "max"], [torch.float32, torch.bfloat16, torch.int32, torch.int64, torch.float64]))
 def test_scatter_minmax_lds_cached_variant(capi, oracle, shape, reduce, dtype, monkeypatch):
     """The workgroup-private table variant (forced on, with a small chunk so that
-    several workgroups meet on the same slots), skewed index with heavy ties."""
+    several workgroups meet on the same slots), skewed index with heavy ties. 64-bit types: the table of keys
+    in front of their compare-and-swap pass."""
     monkeypatch.setenv("TS_SCATTER_LDS", "2")
     monkeypatch.setenv("TS_SCATTER_EPB", "700")
     B, E, K, N = shape
     rng = np.random.default_rng(E + K)
     src = random_values(rng, (B, E, K), dtype, ties=True)
+    if dtype == torch.float64:  # the values that the keys fold or skip
+        flat = src.view(-1)
+        flat[::97] = float("nan")
+        flat[5::89] = -0.0
+        flat[7::83] = float("-inf")
+        flat[11::79] = float("inf")
+    elif dtype == torch.int64:  # the ends of the range map to the keys that stand for "no entry"
+        flat = src.view(-1)
+        flat[::97] = torch.iinfo(torch.int64).min
+        flat[5::89] = torch.iinfo(torch.int64).max
     p = np.arange(1, N + 1, dtype=np.float64) ** -1.2
     index1 = torch.from_numpy(rng.choice(N, size=E, p=p / p.sum()))
     index = index1.view(1, E, 1).expand(B, E, K)
