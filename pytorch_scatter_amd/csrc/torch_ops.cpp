@@ -555,10 +555,13 @@ template <int REDUCE> struct ScatterFn : public torch::autograd::Function<Scatte
         const int64_t B = prod(src.sizes(), 0, dim), E = src.size(dim), N = out.size(dim);
         const int64_t K = prod(src.sizes(), dim + 1, src.dim());
         const BatchedIndex bi = batched_index(old_index);
-        Tensor count_f = at::empty({B * N}, src.options().dtype(at::kFloat));
-        check_status(ts_scatter_count(bi.t.data_ptr<int64_t>(), count_f.data_ptr<float>(), B, E, N, bi.batch_stride, 1,
+        // one index row shared by every batch row (an expanded view): counted once and repeated
+        const int64_t Bc = (bi.batch_stride == 0 && B > 1) ? 1 : B;
+        Tensor count_f = at::empty({Bc * N}, src.options().dtype(at::kFloat));
+        check_status(ts_scatter_count(bi.t.data_ptr<int64_t>(), count_f.data_ptr<float>(), Bc, E, N, bi.batch_stride, 1,
                                       stream_of(src)),
                      "scatter_mean count");
+        if (Bc != B) count_f = count_f.view({1, N}).expand({B, N}).contiguous().view({B * N});
         Tensor out_c = out.contiguous();
         check_status(ts_divide_by_count(out_c.data_ptr(), count_f.data_ptr<float>(), B, N, K, dtype_code(out_c),
                                         stream_of(src)),

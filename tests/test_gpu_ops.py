@@ -589,3 +589,24 @@ def test_scatter_mul_under_a_hub(ts, dtype, K):
         assert torch.equal(got.long(), wrapped.to(torch.int32).long())
     else:
         assert torch.allclose(got.double(), want, rtol=1e-4 if dtype == torch.float32 else 1e-11)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.int64])
+def test_scatter_mean_with_one_index_row_for_every_batch_row(ts, dtype):
+    """An index row expanded over the batch rows (stride 0) is counted once; the result is that of the same index
+    written out per batch row, forward and backward."""
+    g = torch.Generator().manual_seed(8)
+    B, E, N = 37, 500, 23
+    row = torch.randint(0, N - 2, (E,), generator=g)
+    src = torch.randn((B, E), generator=g).mul(10).to(dtype)
+    shared = row.view(1, E).expand(B, E)
+    a = ts.scatter(src.to(DEV), shared.to(DEV).expand(B, E), 1, None, N, "mean")
+    b = ts.scatter(src.to(DEV), shared.contiguous().to(DEV), 1, None, N, "mean")
+    # float sums come from atomics in whatever order; the counts, and with them the integer means, are exact
+    assert torch.allclose(a, b, rtol=1e-5, atol=1e-5) if dtype.is_floating_point else torch.equal(a, b)
+    if dtype.is_floating_point:
+        x = src.to(DEV).requires_grad_(True)
+        y = ts.scatter(x, row.to(DEV).view(1, E).expand(B, E), 1, None, N, "mean")
+        (gx,) = torch.autograd.grad(y, x, torch.ones_like(y))
+        count = torch.bincount(row, minlength=N).clamp(min=1).float()
+        assert torch.allclose(gx.cpu(), (1.0 / count)[row].view(1, E).expand(B, E))
