@@ -1391,13 +1391,13 @@ __global__ __launch_bounds__(kLdsAddBlock) void scatter_add_lds_kernel(ScatterAr
   if (m.active) {
     for (int64_t be0 = be_lo + m.el; be0 < be_hi; be0 += (int64_t)m.epp * U) {
       for (int k = m.cl; k < K; k += m.L) {
-        LdsAcc x[U];
+        typename Acc<T>::type x[U];  // widened for the table only where it is added (doubles here cost 30 % of the kernel)
         int64_t idx[U], bb[U], ee[U];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
           const int64_t be = be0 + (int64_t)u * m.epp;
           split_edge(be < be_hi ? be : be0, a.B, a.E, bb[u], ee[u]);
-          x[u] = src ? (LdsAcc)to_acc<T>(src[(bb[u] * a.E + ee[u]) * a.K + k]) : (LdsAcc)1;
+          x[u] = src ? to_acc<T>(src[(bb[u] * a.E + ee[u]) * a.K + k]) : (typename Acc<T>::type)1;
           idx[u] = a.index[bb[u] * a.sb + ee[u] * a.se];
         }
 #pragma unroll
@@ -1412,9 +1412,9 @@ __global__ __launch_bounds__(kLdsAddBlock) void scatter_add_lds_kernel(ScatterAr
             tag = old == -1 ? node : old;
           }
           if (tag == node)
-            __hip_atomic_fetch_add(&s_acc[row * K + k], x[u], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            __hip_atomic_fetch_add(&s_acc[row * K + k], (LdsAcc)x[u], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
           else
-            table_add_out<T>(out + (int64_t)node * a.K + k, from_acc<T>((typename Acc<T>::type)x[u]), out, out_end);
+            table_add_out<T>(out + (int64_t)node * a.K + k, from_acc<T>(x[u]), out, out_end);
         }
       }
     }
