@@ -502,10 +502,16 @@ def sweep_thresholds():
     cases = [
         ("sum: LDS table from 2^17 elements (contended index)", "sum", 16, 1000, [M // 128 - 1024, M // 128 + 1024]),
         ("sum: LDS table from 2^22 elements (any index, K < 32)", "sum", 8, 1_000_000, [M // 2 - 8192, M // 2 + 8192]),
+        ("sum: LDS table from 2^22 elements (any index, K = 32)", "sum", 32, 100_000, [M // 8 - 8192, M // 8 + 8192]),
         ("sum: buckets of output rows from 64 MB (K = 32)", "sum", 32, 100_000, [M // 2 - 16384, M // 2 + 16384]),
         ("max: LDS table from 2^20 elements (contended index)", "max", 8, 1000, [M // 8 - 4096, M // 8 + 4096]),
         ("max: one value per entry, slabs from 2^23 entries", "max", 1, 100_000, [8 * M - 65536, 8 * M + 65536]),
-        ("max: buckets of output rows from 16 MB (K = 32)", "max", 32, 100_000, [M // 8 - 8192, M // 8 + 8192]),
+        ("max: buckets of output rows from 24 MB (K = 32, keys of 25 MB)", "max", 32, 100_000,
+         [3 * M // 16 - 8192, 3 * M // 16 + 8192]),
+        ("max: buckets of output rows from 64 MB (K = 32, keys of 2.5 MB)", "max", 32, 10_000,
+         [M // 2 - 16384, M // 2 + 16384]),
+        ("max: parts of 4 / 8 / 16 entries by the number of wavefronts (K = 32)", "max", 32, 100_000,
+         [M // 8 - 8192, M // 8 + 8192]),
         ("max: sample of the index from 2^23 elements (K = 8)", "max", 8, 1_000_000, [M - 65536, M + 65536]),
         ("sum: rows in slices of columns above 16384 buckets (K = 128)", "sum", 128, [M - 8192, M + 8192], None),
         ("max: rows in slices of columns above 16384 buckets (K = 128)", "max", 128, [M - 8192, M + 8192], None),

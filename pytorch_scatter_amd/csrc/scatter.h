@@ -902,7 +902,8 @@ inline RunGrid run_grid(int64_t n_edges, int64_t kc, int c, int lane_bytes) {
   // its row (Zipf(1.2) index, 32 k - 262 k entries of 32 / 64 floats: 120 - 1040 us without the table, 42 - 270 us
   // with it), while a uniform index pays the tag look-ups (+10-18 %, 3-7 us at these sizes). Narrower rows keep 2^18:
   // 200 k entries of 16 floats under a uniform index 16.4 us without, 22.7 us with the table (536 against 159 us
-  // under the Zipf index: the known cliff of small skewed sums of narrow rows).
+  // under the Zipf index). These sizes now matter for the element types and strided indices that
+  // scatter_add_lds_kernel does not take (see sum_table_by_size).
   int64_t hot_min = run_is_serial(g.lshift, lane_bytes) ? (int64_t)1 << 15 : (int64_t)1 << 18;
   if (const char *env = getenv("TS_SCATTER_HOT_MIN")) hot_min = atoll(env);  // tuning aid
   if (c > 0 && n_edges >= hot_min && !getenv("TS_SCATTER_NO_HOT")) {  // env: tuning aid
@@ -917,13 +918,20 @@ inline RunGrid run_grid(int64_t n_edges, int64_t kc, int c, int lane_bytes) {
   // a slot only combines what lies inside its own part: keep the parts at 16 entries or more -- but not for small
   // inputs, where a part is a chain of dependent reads and atomics and 16 of them are the whole call (min / max
   // of 8192 entries of 32 floats: 42 us with parts of 16, 15 us with parts of 4; sums 11 us either way)
+  // Sums keep 16 from 2^17 entries on (a sorted index combines more per part: 262 k entries of 32 floats 24 us with
+  // parts of 16, 35 us with parts of 4); min / max have nothing to combine before the keys and want 16 k wavefronts
+  // first (131 k / 262 k entries of 32 floats onto 100 k rows: 71 / 85 us with parts of 16, 48 / 72 us with 4 / 8).
+  const int64_t ychunks = (kc + L - 1) / L;
   if (serial && !getenv("TS_RUN_RPW")) {
-    const int floor_rpw = n_edges < ((int64_t)1 << 17) ? 4 : 16;
+    int floor_rpw = n_edges < ((int64_t)1 << 17) ? 4 : 16;
+    if (c == 0) {
+      const int64_t wave_rows = (n_edges + epr - 1) / epr * ychunks;
+      floor_rpw = wave_rows >= 16 * 16384 ? 16 : wave_rows >= 8 * 16384 ? 8 : 4;
+    }
     if (g.rpw < floor_rpw) g.rpw = floor_rpw;
   }
   const int64_t waves = (n_edges + (int64_t)g.rpw * epr - 1) / ((int64_t)g.rpw * epr);
   const int64_t blocks = (waves + kBlock / kWave - 1) / (kBlock / kWave);
-  const int64_t ychunks = (kc + L - 1) / L;
   g.ok = blocks < 0x7FFFFFFFll && ychunks <= 65535;
   g.blocks = (unsigned)blocks;
   g.ychunks = (unsigned)ychunks;
@@ -1636,6 +1644,40 @@ __global__ __launch_bounds__(kBlock) void fill_kernel(T *p, int64_t n, T value) 
   for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlock)
     p[i] = value;
 }
+// The fill of a sum whose kernel is picked by a sample of the index: the first workgroup also takes the sample
+// of bin_sample_kernel (the same entries and the same verdict in *flag), which saves that kernel's launch and
+// hides its loads behind the fill (5-7 us of a 25 us call).
+template <typename T>
+__global__ __launch_bounds__(kBlock) void fill_sample_kernel(T *p, int64_t n, T value, ScatterArgs a, int *flag) {
+  __shared__ int s_desc;
+  constexpr int PER = kBinBlock / kBlock;
+  int desc = 0;
+  if (blockIdx.x == 0) {
+    if (threadIdx.x == 0) s_desc = 0;
+    const int64_t ne = a.B * a.E;  // the host asks for a sample only with ne >= 2 * kBinBlock
+    int64_t idx[PER], nxt[PER];
+    bool same[PER];
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      const int64_t be = (int64_t)(threadIdx.x * PER + j) * (ne / kBinBlock);
+      const int64_t b = be / a.E, e = be - b * a.E;
+      const int64_t b1 = (be + 1) / a.E, e1 = be + 1 - b1 * a.E;
+      idx[j] = a.index[b * a.sb + e * a.se];
+      nxt[j] = a.index[b1 * a.sb + e1 * a.se];
+      same[j] = b1 == b;
+    }
+#pragma unroll
+    for (int j = 0; j < PER; ++j) desc += same[j] && nxt[j] < idx[j] ? 1 : 0;
+  }
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlock)
+    p[i] = value;
+  if (blockIdx.x == 0) {
+    __syncthreads();
+    if (desc) atomicAdd(&s_desc, desc);
+    __syncthreads();
+    if (threadIdx.x == 0) *flag = s_desc * 64 >= kBinBlock ? 1 : 0;
+  }
+}
 // out[out == init] = 0 (csrc/cuda/scatter_cuda.cu:126-127)
 template <typename T>
 __global__ __launch_bounds__(kBlock) void mask_init_kernel(T *p, int64_t n, T init) {
@@ -1683,13 +1725,30 @@ inline unsigned scatter_grid(int64_t n_edges, int64_t kv, int block, int U) {
   return (unsigned)(blocks < cap ? blocks : cap);
 }
 
-// sizes from which a floating-point sum goes through the LDS table kernel (the crossovers are with its use below)
+// Sizes from which a sum goes through the LDS table kernel (scatter_add_lds_kernel). The table is the kernel
+// that a skewed index cannot hurt: a hub's entries meet in LDS, where the run kernel sends each of them to one
+// address in memory, 10 ns apiece (Zipf(1.2) index, us run kernel / table: 16 k entries of 32 floats 56 / 11,
+// 65 k entries 143 / 14, 200 k entries of 16 floats 479 / 27, 131 k single values 268 / 11). With chunks sized
+// for one workgroup per CU it costs a uniform or sorted index nothing where the call is bound by its two launches
+// (up to 2^19 elements: 10.4-11.5 us either way), 1-4 us at 2^21 elements (200 k x 16 floats onto 10 k rows:
+// 16.2 / 19.9 us), and from 2^23 elements it is level or ahead. So, for 4-byte elements: from 2^17 elements, rows
+// above 64 columns (a table of 64 rows) from 2^20. Other element types keep the sizes measured for them: a
+// contended index (32 and more entries per output row) from 2^17 elements, narrow rows from 2^18 entries or 2^22
+// elements; 2-byte elements are flushed with packed adds and lose through the table under an uncontended index
+// (16 MB of 32 bf16 per entry: 17 -> 50 us). Rows of 32 and more columns stay under 300 MB of input (9-10 M entries:
+// a sorted index takes 450 us through the run kernel with its hot rows and 940 us through the table; an unsorted
+// one has the workspace path).
 inline bool sum_table_by_size(int64_t B, int64_t E, int64_t K, int64_t N, int elem_bytes) {
   const int64_t n_edges = B * E, n_src = n_edges * K;
   if (n_src < ((int64_t)1 << 17)) return false;
-  if (n_edges >= 32 * B * N) return K < 32 || n_src * elem_bytes < (int64_t)300000000;
+  if (K >= 32 && n_src * elem_bytes >= (int64_t)300000000) return false;
+  if (n_edges >= 32 * B * N) return true;
+  if (elem_bytes == 4) return K <= 64 || n_src >= ((int64_t)1 << 20);
   return K < 32 && (n_src >= ((int64_t)1 << 22) || n_edges >= ((int64_t)1 << 18));
 }
+// entries per workgroup of that kernel at least: 2048 elements, 64 entries (8192 entries of 32 floats: 17.4 us in
+// chunks of 512, 10.6 us in chunks of 64; the chunk of a larger input is its share of one workgroup per CU)
+inline int64_t sum_table_min_chunk(int64_t K) { return 2048 / K > 64 ? 2048 / K : 64; }
 
 template <typename T, int VEC>
 int launch_scatter_v(const ScatterArgs &args, int reduce, hipStream_t stream) {
@@ -1716,9 +1775,34 @@ int launch_scatter_v(const ScatterArgs &args, int reduce, hipStream_t stream) {
       }
     }
     const bool routed = lshift >= 0 && a.sorted_route && a.route_flag != nullptr && !a.out_given;
-    if (!a.out_given && !routed)
-      hipLaunchKernelGGL(fill_kernel<T>, dim3(g_out), dim3(kBlock), 0, stream, out, n_out,
-                         small_const<T>(reduce == TS_MUL ? 1 : 0));
+    // sums that go through the LDS table (scatter_add_lds_kernel; the sizes and crossovers are with its launch
+    // below), and whether a sample of the index picks between it and the run kernel
+    bool use_lds = false, sampled = false;
+    int tn = 1;
+    if constexpr (__is_same(T, float) || __is_same(T, bf16_t) || __is_same(T, f16_t) || __is_same(T, double) ||
+                  __is_same(T, int32_t) || __is_same(T, int64_t)) {
+      if (reduce == TS_SUM && n_src > 0) {
+        while ((int64_t)tn * 2 * a.K <= kLdsAcc && tn * 2 <= kLdsAccRows) tn *= 2;
+        // (behind the buckets only an index in order arrives here: that one has the table only if contended)
+        const bool by_size = sum_table_by_size(a.B, a.E, a.K, a.N, (int)sizeof(T)) &&
+                             (lshift < 0 || n_edges >= 32 * a.B * a.N);
+        use_lds = a.lds_cache && a.sk == 0 && tn >= 64 && a.B * a.N < 0x7FFFFFFFll && (a.lds_cache == 2 || by_size);
+        // (a sample of the index: from 2^23 elements, where a sorted index does better through the run kernel;
+        // below, the table is level with it and the launch that returns at once would cost 2-4 us)
+        sampled = use_lds && a.lds_cache != 2 && a.order_ws != nullptr && a.skip_flag == nullptr && lshift < 0 &&
+                  a.run_reduce && n_edges >= 2 * kBinBlock && n_src >= ((int64_t)1 << 23);
+      }
+    }
+    if (!a.out_given && !routed) {
+      if (sampled)
+        hipLaunchKernelGGL(fill_sample_kernel<T>, dim3(g_out), dim3(kBlock), 0, stream, out, n_out, small_const<T>(0),
+                           a, a.order_ws);
+      else
+        hipLaunchKernelGGL(fill_kernel<T>, dim3(g_out), dim3(kBlock), 0, stream, out, n_out,
+                           small_const<T>(reduce == TS_MUL ? 1 : 0));
+    } else if (sampled) {
+      hipLaunchKernelGGL(bin_sample_kernel, dim3(1), dim3(kBinBlock), 0, stream, a, a.order_ws);
+    }
     if constexpr (BinSlotOk<T>::value) {
       if (lshift >= 0) {
         launch_binned_add<T, VEC>(a, bp.p, lshift, stream, routed ? n_out : 0);
@@ -1737,36 +1821,20 @@ int launch_scatter_v(const ScatterArgs &args, int reduce, hipStream_t stream) {
         if constexpr (__is_same(T, float) || __is_same(T, bf16_t) || __is_same(T, f16_t) || __is_same(T, double) ||
                       __is_same(T, int32_t) || __is_same(T, int64_t)) {
           // many entries per output slot: reduce in LDS first (see scatter_add_lds_kernel)
-          int tn = 1;
-          while ((int64_t)tn * 2 * a.K <= kLdsAcc && tn * 2 <= kLdsAccRows) tn *= 2;
-          // Rows under 32 columns: for a contended index (32 and more entries per output row) from 2^17 elements on;
-          // for any other index from 2^18 entries or 2^22 elements on. Measured crossovers (us, run kernel / table):
-          // Zipf(1.2) index onto 1 M rows, K = 8: 65 k entries 211 / 20, 262 k 357 / 23, 1 M 424 / 40 -- every entry
-          // of a hub is an atomic on one address, 10 ns each; the same sizes under a uniform index 14 / 21, 27 / 26,
-          // 79 / 63; 200 k x 16 floats onto 10 k rows (uniform) 16.4 / 21.4, 400 k x 16: 39 / 30. Below these sizes
-          // the table costs a uniform index 5-7 us and a skewed one is left to the run kernel (known cliff: up to
-          // 20x for 65 k - 262 k entries under a heavy-tailed index).
-          // Rows of 32 and more columns: for a contended index, the table up to 300 MB of input (1 M entries onto 3000 nodes, K = 32:
-          // 70 / 58 / 106 us for a Zipf / sorted / uniform index against 275 / 174 / 126 us through the run kernel),
-          // the run kernel with its hot rows above (9-10 M entries: a sorted index, such as the batch vector of a
-          // pooling layer, takes 450 us there and 940 us through the table; an unsorted one has the workspace path)
-          const bool use_lds = a.lds_cache && a.sk == 0 && tn >= 64 && a.B * a.N < 0x7FFFFFFFll &&
-                               (a.lds_cache == 2 || sum_table_by_size(a.B, a.E, a.K, a.N, (int)sizeof(T)));
+          // (sizes: sum_table_by_size)
           if (use_lds) {
             // The table is for an index in no particular order. One that is sorted does better through the run
             // kernel below (9 M entries of the graph of C3, sorted: K = 8 343 against 156 us, K = 4 152 / 96,
             // K = 1 60 / 44; shuffled: 448 / 463), so with a word of scratch a sample of the index decides on the
             // device: the table returns at once if the index looks sorted, the run kernel if not.
-            const bool sampled = a.lds_cache != 2 && a.order_ws != nullptr && a.skip_flag == nullptr && a.run_reduce &&
-                                 n_edges >= 2 * kBinBlock;
+            // (the sample was taken with the fill of out above)
             ScatterArgs t = a;
             if (sampled) {
-              hipLaunchKernelGGL(bin_sample_kernel, dim3(1), dim3(kBinBlock), 0, stream, a, a.order_ws);
               t.skip_flag = a.order_ws;
               t.skip_inverse = 1;
               a.skip_flag = a.order_ws;
             }
-            const int64_t epb = per_cu_chunk_edges(a.lds_epb, n_edges, 16384 / a.K > 256 ? 16384 / a.K : 256,
+            const int64_t epb = per_cu_chunk_edges(a.lds_epb, n_edges, sum_table_min_chunk(a.K),
                                                    131072 / a.K > 2048 ? 131072 / a.K : 2048);
             hipLaunchKernelGGL(scatter_add_lds_kernel<T>, dim3((unsigned)((n_edges + epb - 1) / epb)),
                                dim3(kLdsAddBlock), 0, stream, t, tn - 1, epb);

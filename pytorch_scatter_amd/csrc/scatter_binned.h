@@ -73,12 +73,23 @@ inline BinPlan bin_plan(int64_t B, int64_t E, int64_t K, int64_t N, int elem_byt
   r.ok = false;
   r.bytes = 0;
   const int64_t n_edges = B * E, rows = B * N;
-  // rows of 64 bytes and more, inputs from 128 MB (below, the five extra launches cost more than the misses:
-  // 64 MB of 128-byte rows, Zipf index: 65 us without, 79 us with; 154 MB of 512-byte rows: 348 against 115 us)
-  // min / max (slabs) from 16 MB, sums from 64 MB (measured crossovers, Zipf(1.2) and uniform index onto 100 k rows of
-  // 32 floats: max 87 / 70 us without and 72 / 64 us with the buckets at 16 MB; sum 154 / 72 us and 81 / 91 us at 64 MB)
-  const int64_t min_bytes = slabs ? ((int64_t)16 << 20) : ((int64_t)64 << 20);
+  // Rows of 64 bytes and more. Sums from 64 MB of input (below, the five extra launches cost more than the misses:
+  // Zipf(1.2) / uniform index onto 100 k rows of 32 floats, 64 MB: 72 / 91 us with the buckets, and the table of
+  // scatter_add_lds_kernel takes the sizes below), and with two entries per output row: every bucket is flushed
+  // whatever it received (96 MB / 256 MB of 32 ... 128 floats per entry onto 1 M rows, uniform index: 155 / 224,
+  // 237 / 332, 379 / 513 us with the buckets, 104 / 248, 126 / 274, 175 / 314 us without).
+  // min / max: the other path fills a table of 8-byte keys as large as out and walks it once more at the end, so
+  // the crossover moves with that table (uniform index, us without / with the buckets):
+  //   keys of 2.5 MB (10 k rows of 32 floats):  16 MB 30 / 57, 48 MB 90 / 92, 64 MB 98 / 96
+  //   keys of 10 - 25 MB:                        16 MB 39 / 54 and 48 / 49, 24 MB 56 / 55 and 65 / 52, 48 MB 93 / 60
+  //   keys of 256 MB and 1 GB (1 M rows):        4 MB 159 / 122 and 777 / 562, 64 MB 256 / 184 and 842 / 514
+  // (a Zipf(1.2) index gains earlier: keys of 25 MB, 8 MB of input: 64 / 49 us)
+  const int64_t key_bytes = rows * K * 8;
+  const int64_t minmax_bytes = key_bytes >= ((int64_t)256 << 20) ? ((int64_t)1 << 20)
+                               : key_bytes >= ((int64_t)8 << 20) ? ((int64_t)24 << 20) : ((int64_t)64 << 20);
+  const int64_t min_bytes = slabs ? minmax_bytes : ((int64_t)64 << 20);
   if (K * elem_bytes < 64 || (!any_size && n_edges * K * elem_bytes < min_bytes) ||
+      (!any_size && !slabs && n_edges < 2 * rows) ||
       n_edges >= 0xFFFFFFFEll || rows >= 0x7FFFFFFFll || rows < 1)
     return r;
   const int64_t slots = (int64_t)kBinKeys * 8 / slot_bytes;
