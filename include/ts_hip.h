@@ -199,9 +199,9 @@ int ts_scatter(const void *src, const int64_t *index, void *out,
  * is not sorted, first bin the entries by bucket of output rows (8 bytes per entry) and reduce every
  * bucket in LDS: no atomics on the table in memory except one write-back per chunk. MIN / MAX of
  * other large inputs of 4-byte elements with few entries per output row ask for 256 bytes: one flag,
- * written by a sample of the index, that picks the kernel for a skewed or an even index; so do SUMs of
- * floating-point rows under 64 bytes at the sizes that go through the accumulator table in LDS (there the
- * sample keeps a sorted index with the kernel that combines its runs: about twice as fast). MIN / MAX: same
+ * written by a sample of the index, that picks the kernel for a skewed or an even index; so do SUMs
+ * at the sizes that go through the accumulator table in LDS (from 2^23 elements on the sample keeps a
+ * sorted index with the kernel that combines its runs: about twice as fast). MIN / MAX: same
  * results as ts_scatter; SUM: the same sum in another order of additions. No counterpart in the reference
  * (scatter_cuda allocates nothing beyond its outputs, csrc/cuda/scatter_cuda.cu:54-138). */
 size_t ts_scatter_workspace_bytes(int64_t B, int64_t E, int64_t K, int64_t N,
