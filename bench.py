@@ -500,9 +500,11 @@ def sweep_thresholds():
     # (what, K, N, sizes in entries around the threshold); N a list: 2 M entries, output rows around the threshold
     M = 1 << 20
     cases = [
-        ("sum: LDS table from 2^17 elements (K = 16)", "sum", 16, 1000, [M // 128 - 1024, M // 128 + 1024]),
-        ("sum: LDS table from 2^20 elements for rows above 64 columns (K = 128)", "sum", 128, 100_000,
-         [M // 128 - 512, M // 128 + 512]),
+        ("sum: LDS table from 2^16 elements (K = 16)", "sum", 16, 1000, [M // 256 - 512, M // 256 + 512]),
+        ("sum: LDS table from 2^18 elements for rows of 33-64 columns (K = 64)", "sum", 64, 100_000,
+         [M // 256 - 256, M // 256 + 256]),
+        ("sum: LDS table from 2^19 elements for rows above 64 columns (K = 128)", "sum", 128, 100_000,
+         [M // 256 - 256, M // 256 + 256]),
         ("sum: sample of the index from 2^23 elements (K = 8)", "sum", 8, 1_000_000, [M - 65536, M + 65536]),
         ("sum: buckets of output rows from 64 MB (K = 32)", "sum", 32, 100_000, [M // 2 - 16384, M // 2 + 16384]),
         ("max: LDS table from 2^20 elements (contended index)", "max", 8, 1000, [M // 8 - 4096, M // 8 + 4096]),

@@ -623,7 +623,7 @@ int ts_scatter_count(const int64_t *index, float *count, int64_t B, int64_t E, i
     // costs an atomic on one address per entry: 4 M entries under a Zipf(1.2) index 1.3 ms against 0.08 ms)
     const bool contended = a.lds_cache == 2 || (a.lds_cache == 1 && sum_table_by_size(B, E, 1, N, 4));
     if (contended && B * N < 0x7FFFFFFFll) {
-      const int64_t epb = per_cu_chunk_edges(a.lds_epb, B * E, sum_table_min_chunk(1), 131072);
+      const int64_t epb = per_cu_chunk_edges(a.lds_epb, B * E, sum_table_min_chunk(1, 4), 131072);
       hipLaunchKernelGGL(scatter_add_lds_kernel<float>, dim3((unsigned)((B * E + epb - 1) / epb)), dim3(kLdsAddBlock), 0,
                          s, a, kLdsAccRows - 1, epb);
     } else if (env_int("TS_SCATTER_RUNS", 1) && B * N < 0x7FFFFFFFll) {

@@ -1731,8 +1731,12 @@ inline unsigned scatter_grid(int64_t n_edges, int64_t kv, int block, int U) {
 // 65 k entries 143 / 14, 200 k entries of 16 floats 479 / 27, 131 k single values 268 / 11). With chunks sized
 // for one workgroup per CU it costs a uniform or sorted index nothing where the call is bound by its two launches
 // (up to 2^19 elements: 10.4-11.5 us either way), 1-4 us at 2^21 elements (200 k x 16 floats onto 10 k rows:
-// 16.2 / 19.9 us), and from 2^23 elements it is level or ahead. So, for 4-byte elements: from 2^17 elements, rows
-// above 64 columns (a table of 64 rows) from 2^20. Other element types keep the sizes measured for them: a
+// 16.2 / 19.9 us), and from 2^23 elements it is level or ahead. Its write-back is a phase of its own after the
+// entries, which shows where the atomics miss the L2 (+1 us on the smallest calls, +4 us for rows of 64 floats onto
+// 100 k rows), so the smallest inputs stay with the run kernel for as long as a hub costs less than that: 4-byte
+// elements go through the table from 2^16 elements, rows of 33-64 columns from 2^18, wider ones (a table of 64
+// rows: 4096 entries of 128 floats onto 100 k rows, uniform 13.6 / 18.9 us, Zipf 37 / 19 us) from 2^19.
+// Other element types keep the sizes measured for them: a
 // contended index (32 and more entries per output row) from 2^17 elements, narrow rows from 2^18 entries or 2^22
 // elements; 2-byte elements are flushed with packed adds and lose through the table under an uncontended index
 // (16 MB of 32 bf16 per entry: 17 -> 50 us). Rows of 32 and more columns stay under 300 MB of input (9-10 M entries:
@@ -1740,15 +1744,23 @@ inline unsigned scatter_grid(int64_t n_edges, int64_t kv, int block, int U) {
 // one has the workspace path).
 inline bool sum_table_by_size(int64_t B, int64_t E, int64_t K, int64_t N, int elem_bytes) {
   const int64_t n_edges = B * E, n_src = n_edges * K;
-  if (n_src < ((int64_t)1 << 17)) return false;
+  if (n_src < ((int64_t)1 << 16)) return false;
   if (K >= 32 && n_src * elem_bytes >= (int64_t)300000000) return false;
+  if (elem_bytes == 4 && n_src >= ((int64_t)1 << (K <= 32 ? 16 : K <= 64 ? 18 : 19))) return true;
+  if (n_src < ((int64_t)1 << 17)) return false;
   if (n_edges >= 32 * B * N) return true;
-  if (elem_bytes == 4) return K <= 64 || n_src >= ((int64_t)1 << 20);
+  if (elem_bytes == 4) return false;
   return K < 32 && (n_src >= ((int64_t)1 << 22) || n_edges >= ((int64_t)1 << 18));
 }
 // entries per workgroup of that kernel at least: 2048 elements, 64 entries (8192 entries of 32 floats: 17.4 us in
 // chunks of 512, 10.6 us in chunks of 64; the chunk of a larger input is its share of one workgroup per CU)
-inline int64_t sum_table_min_chunk(int64_t K) { return 2048 / K > 64 ? 2048 / K : 64; }
+// 2-byte elements keep chunks of 16384 elements: every partial sum that leaves the table is rounded to the element
+// type, and with one entry per row and chunk nothing has been combined in fp32 before that (300 k single bf16 values
+// onto 5000 rows: RMS error 0.105 in chunks of 2048, 0.074 for the reference's entry-by-entry adds, less in large chunks).
+inline int64_t sum_table_min_chunk(int64_t K, int elem_bytes) {
+  if (elem_bytes == 2) return 16384 / K > 256 ? 16384 / K : 256;
+  return 2048 / K > 64 ? 2048 / K : 64;
+}
 
 template <typename T, int VEC>
 int launch_scatter_v(const ScatterArgs &args, int reduce, hipStream_t stream) {
@@ -1834,7 +1846,7 @@ int launch_scatter_v(const ScatterArgs &args, int reduce, hipStream_t stream) {
               t.skip_inverse = 1;
               a.skip_flag = a.order_ws;
             }
-            const int64_t epb = per_cu_chunk_edges(a.lds_epb, n_edges, sum_table_min_chunk(a.K),
+            const int64_t epb = per_cu_chunk_edges(a.lds_epb, n_edges, sum_table_min_chunk(a.K, (int)sizeof(T)),
                                                    131072 / a.K > 2048 ? 131072 / a.K : 2048);
             hipLaunchKernelGGL(scatter_add_lds_kernel<T>, dim3((unsigned)((n_edges + epb - 1) / epb)),
                                dim3(kLdsAddBlock), 0, stream, t, tn - 1, epb);

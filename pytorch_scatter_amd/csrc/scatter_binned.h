@@ -77,7 +77,9 @@ inline BinPlan bin_plan(int64_t B, int64_t E, int64_t K, int64_t N, int elem_byt
   // Zipf(1.2) / uniform index onto 100 k rows of 32 floats, 64 MB: 72 / 91 us with the buckets, and the table of
   // scatter_add_lds_kernel takes the sizes below), and with two entries per output row: every bucket is flushed
   // whatever it received (96 MB / 256 MB of 32 ... 128 floats per entry onto 1 M rows, uniform index: 155 / 224,
-  // 237 / 332, 379 / 513 us with the buckets, 104 / 248, 126 / 274, 175 / 314 us without).
+  // 237 / 332, 379 / 513 us with the buckets, 104 / 248, 126 / 274, 175 / 314 us without) -- up to 300 MB, where the
+  // table of scatter_add_lds_kernel stops taking wide rows and the buckets are the path that a hub cannot hurt
+  // (1 GB of 128 floats per entry, one entry per row, Zipf(1.2): 607 us with the buckets, 1226 us without).
   // min / max: the other path fills a table of 8-byte keys as large as out and walks it once more at the end, so
   // the crossover moves with that table (uniform index, us without / with the buckets):
   //   keys of 2.5 MB (10 k rows of 32 floats):  16 MB 30 / 57, 48 MB 90 / 92, 64 MB 98 / 96
@@ -89,7 +91,7 @@ inline BinPlan bin_plan(int64_t B, int64_t E, int64_t K, int64_t N, int elem_byt
                                : key_bytes >= ((int64_t)8 << 20) ? ((int64_t)24 << 20) : ((int64_t)64 << 20);
   const int64_t min_bytes = slabs ? minmax_bytes : ((int64_t)64 << 20);
   if (K * elem_bytes < 64 || (!any_size && n_edges * K * elem_bytes < min_bytes) ||
-      (!any_size && !slabs && n_edges < 2 * rows) ||
+      (!any_size && !slabs && n_edges < 2 * rows && n_edges * K * elem_bytes < (int64_t)300000000) ||
       n_edges >= 0xFFFFFFFEll || rows >= 0x7FFFFFFFll || rows < 1)
     return r;
   const int64_t slots = (int64_t)kBinKeys * 8 / slot_bytes;

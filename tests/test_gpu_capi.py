@@ -970,7 +970,9 @@ def test_scatter_sum_narrow_rows_sample_picks_the_kernel(capi, oracle, shape, ki
         if by_sample:
             assert int(ws[:4].view(torch.int32).item()) == (0 if kind == "sorted" else 1), kind
         want = exact + (prev.double() if out_given else 0)
-        rtol = 1e-5 if dtype == torch.float32 else 1e-2
+        # bf16: every add into out rounds to 8 bits, as the reference's atomicAdd does (60 adds at magnitude 16 were
+        # seen at 0.95e-2 of this bound's scale)
+        rtol = 1e-5 if dtype == torch.float32 else 2e-2
         err = (out.cpu().double() - want).abs()
         bound = rtol * want.abs() + rtol * (absum + (prev.double().abs() if out_given else 0)).clamp(min=1e-30)
         assert bool((err <= bound).all()), float((err - bound).max())
