@@ -327,25 +327,29 @@ static __global__ __launch_bounds__(kBlock) void coo_to_indptr_kernel(const int6
                                                                const int *gate = nullptr, int gate_want = 0) {
   // gate (optional): run only if (*gate != 0) == (gate_want != 0) -- a scatter that found its index sorted
   if (gate != nullptr && (*gate != 0) != (gate_want != 0)) return;
+  __shared__ GapList s_gaps;
+  if (threadIdx.x == 0) s_gaps.n = 0;
+  __syncthreads();
   const int64_t b = blockIdx.y;
   const int64_t e0 = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * kCooPtrPerThread;
-  if (e0 > E) return;
   const int64_t *idx = index + b * index_batch_stride;
   int64_t *p = ptr + b * (N + 1);
   int64_t v[kCooPtrPerThread + 1];
-  v[0] = e0 == 0 ? -1 : idx[e0 - 1];
+  v[0] = e0 == 0 || e0 > E ? -1 : idx[e0 - 1];
 #pragma unroll
   for (int i = 0; i < kCooPtrPerThread; ++i) v[i + 1] = e0 + i < E ? idx[e0 + i] : N;
 #pragma unroll
-  for (int i = 0; i < kCooPtrPerThread; ++i) {
+  for (int i = 0; i < kCooPtrPerThread; ++i) {  // (no lane leaves early: the wavefront writes long ranges together)
     const int64_t e = e0 + i;
-    if (e > E) break;
     int64_t lo = v[i] + 1;
     int64_t hi = e == E ? N : v[i + 1];
     if (lo < 0) lo = 0;
     if (hi > N) hi = N;
-    for (int64_t r = lo; r <= hi; ++r) p[r] = e;
+    if (e > E) hi = lo - 1;
+    gap_rows(p, lo, hi, e, s_gaps);
   }
+  __syncthreads();
+  gap_rows_finish(p, s_gaps);
 }
 
 }  // namespace ts

@@ -20,12 +20,17 @@ static __global__ __launch_bounds__(kBlock) void index_keys_kernel(const int64_t
 // (keys[e-1], keys[e]], thread E the rows after the last key
 static __global__ __launch_bounds__(kBlock) void keys_to_indptr_kernel(const uint32_t *__restrict__ keys,
                                                                      int64_t *__restrict__ ptr, int64_t N, int64_t E) {
+  __shared__ GapList s_gaps;
+  if (threadIdx.x == 0) s_gaps.n = 0;
+  __syncthreads();
   const int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  if (e > E) return;
-  int64_t lo = e == 0 ? 0 : (int64_t)keys[e - 1] + 1;
-  int64_t hi = e == E ? N : (int64_t)keys[e];
+  int64_t lo = e == 0 || e > E ? 0 : (int64_t)keys[e - 1] + 1;
+  int64_t hi = e >= E ? N : (int64_t)keys[e];
   if (hi > N) hi = N;
-  for (int64_t r = lo; r <= hi; ++r) ptr[r] = e;
+  if (e > E) hi = lo - 1;
+  gap_rows(ptr, lo, hi, e, s_gaps);  // (no lane leaves early: the wavefront writes long ranges together)
+  __syncthreads();
+  gap_rows_finish(ptr, s_gaps);
 }
 
 static __global__ __launch_bounds__(kBlock) void row_numbers_kernel(int64_t *__restrict__ p, int64_t total, int64_t N) {

@@ -465,21 +465,32 @@ static __global__ __launch_bounds__(kBinPlaceBlock) void bin_place_kernel(Scatte
     // pointers from this launch instead: ptr[b][r] = first e with index[b][e] >= r (the count pass has checked
     // that the index is in order and inside [0, N)).
     if (a.route_ptr != nullptr) {
-#pragma unroll 4
+      // (long ranges of rows without entries are written by the wavefront or the workgroup: gap_rows; the
+      // workgroup's tile may span two batches, whose pointers differ, so the list is emptied after every round)
+      __shared__ GapList s_gaps;
       for (int j = 0; j < kBinPer; ++j) {
-        if (j * kBinPlaceBlock >= p.place_tile) break;
+        if (j * kBinPlaceBlock >= p.place_tile) break;  // uniform
+        if (threadIdx.x == 0) s_gaps.n = 0;
+        __syncthreads();
         const int64_t be = (int64_t)blockIdx.x * p.place_tile + threadIdx.x + (int64_t)j * kBinPlaceBlock;
-        if (be >= a.B * a.E) break;
-        const int64_t b = be / a.E, e = be - b * a.E;
+        const bool live = be < a.B * a.E;
+        const int64_t b = live ? be / a.E : 0, e = live ? be - b * a.E : 0;
         const int64_t *idx = a.index + b * a.sb;
-        int64_t *ptr = a.route_ptr + b * (a.N + 1);
-        int64_t hi = idx[e];
+        int64_t hi = live ? idx[e] : -1;
         int64_t lo = e == 0 ? 0 : idx[e - 1] + 1;
         if (lo < 0) lo = 0;
         if (hi > a.N) hi = a.N;
-        for (int64_t r = lo; r <= hi; ++r) ptr[r] = e;
-        if (e == a.E - 1)
-          for (int64_t r = (hi < 0 ? 0 : hi + 1); r <= a.N; ++r) ptr[r] = a.E;
+        if (!live) hi = lo - 1;
+        // the ranges of one round are written through pointers relative to batch 0: lanes of one wavefront may
+        // belong to two batches
+        const int64_t off = b * (a.N + 1);
+        gap_rows(a.route_ptr, off + lo, off + hi, e, s_gaps);
+        const bool last = live && e == a.E - 1;
+        const int64_t tl = hi < 0 ? 0 : hi + 1;
+        gap_rows(a.route_ptr, off + tl, last ? off + a.N : off + tl - 1, a.E, s_gaps);
+        __syncthreads();
+        gap_rows_finish(a.route_ptr, s_gaps);
+        __syncthreads();
       }
     }
     return;

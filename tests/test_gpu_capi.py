@@ -398,6 +398,61 @@ def test_segment_coo(capi, oracle, case, reduce, dtype):
             assert_exact(cnt, want2)
 
 
+GAP_KINDS = ["one_row", "empty_tail", "empty_head", "two_hubs", "every_3000th"]
+
+
+def gap_index(kind, rng, E, N):
+    """Sorted indices that leave long ranges of output rows without entries."""
+    if kind == "one_row":
+        return np.full(E, N // 2)
+    if kind == "empty_tail":
+        return np.sort(rng.integers(0, max(N // 100, 1), size=E))
+    if kind == "empty_head":
+        return np.sort(rng.integers(N - max(N // 100, 1), N, size=E))
+    if kind == "two_hubs":
+        return np.sort(np.where(rng.random(E) < 0.5, 17, N - 9))
+    return np.sort(rng.integers(0, N // 3000 + 1, size=E) * 3000 % N)
+
+
+@pytest.mark.parametrize("kind,shape,reduce", product(
+    GAP_KINDS, [(1, 5000, 3, 50_000), (2, 700, 8, 9000), (1, 300, 1, 300_000), (3, 9, 2, 70_000)], ["sum", "max"]))
+def test_segment_coo_long_ranges_of_empty_rows(capi, oracle, kind, shape, reduce):
+    """Row pointers of a sorted index whose entries leave thousands of neighbouring rows empty: the rows between
+    two entries are written by the lane that owns the later entry when they are few, by its wavefront or
+    workgroup when they are many (gap_rows in device_utils.h). Results as the oracle's, batches included."""
+    B, E, K, N = shape
+    rng = np.random.default_rng(E + N)
+    idx = np.stack([gap_index(kind, rng, E, N) for _ in range(B)])
+    index = torch.from_numpy(idx)
+    src = values(rng, (B, E, K), torch.float32, reduce)
+    want, want2 = oracle.segment_coo(src, index, None, N, reduce)
+    out = torch.full((B, N, K), 7, dtype=torch.float32, device=DEV)
+    arg = torch.full((B, N, K), -1, dtype=torch.long, device=DEV) if reduce == "max" else None
+    capi.segment_coo(src.to(DEV), index.to(DEV), out, arg, None, B, N, E, K, E, capi.REDUCE[reduce], False)
+    torch.cuda.synchronize()
+    if reduce == "max":
+        assert_exact(out, want)
+        assert_exact(arg, want2)
+    else:
+        assert torch.allclose(out.cpu(), want, rtol=1e-4, atol=1e-3)
+
+
+@pytest.mark.parametrize("kind", GAP_KINDS)
+def test_sort_index_long_ranges_of_empty_rows(capi, kind):
+    """The row pointers that ts_sort_index writes next to its permutation, for indices that leave long ranges of
+    rows empty: ptr[r] = number of entries below row r."""
+    E, N = 6000, 200_000
+    rng = np.random.default_rng(5)
+    idx = rng.permutation(gap_index(kind, rng, E, N))
+    perm = torch.empty(E, dtype=torch.int32, device=DEV)
+    ptr = torch.full((N + 1,), -5, dtype=torch.long, device=DEV)
+    capi.sort_index(torch.from_numpy(idx).to(DEV), perm, ptr, E, N)
+    torch.cuda.synchronize()
+    want = np.concatenate([[0], np.cumsum(np.bincount(idx, minlength=N))])
+    assert np.array_equal(ptr.cpu().numpy(), want)
+    assert np.array_equal(np.sort(idx, kind="stable"), idx[perm.cpu().numpy()])
+
+
 @pytest.mark.parametrize("reduce,dtype,K", product(["sum", "mean", "min", "max"], [torch.float32, torch.bfloat16],
                                                    [16, 2]))
 def test_segment_coo_out_given(capi, oracle, reduce, dtype, K):
