@@ -259,11 +259,16 @@ int run_coo_gather(int dtype, const CooGatherArgs &args, const CooGatherPlan &p,
 // sorted index [B, E] -> row pointers [B, N + 1] (contiguous)
 int run_coo_to_indptr(const int64_t *index, int64_t *ptr, int64_t B, int64_t E, int64_t N, int64_t index_batch_stride,
                       hipStream_t s, const int *gate = nullptr, int gate_want = 0) {
-  const int64_t per_block = (int64_t)kBlock * kCooPtrPerThread;
+  const int per = E < ((int64_t)1 << 20) ? 1 : kCooPtrPerThread;
+  const int64_t per_block = (int64_t)kBlock * per;
   return for_batch_slices(B, [&](int64_t b0, int64_t nb) {
     dim3 grid((unsigned)((E + 1 + per_block - 1) / per_block), (unsigned)nb);
-    hipLaunchKernelGGL(coo_to_indptr_kernel, grid, dim3(kBlock), 0, s, index + b0 * index_batch_stride,
-                       ptr + b0 * (N + 1), N, E, index_batch_stride, gate, gate_want);
+    if (per == 1)
+      hipLaunchKernelGGL(coo_to_indptr_kernel<1>, grid, dim3(kBlock), 0, s, index + b0 * index_batch_stride,
+                         ptr + b0 * (N + 1), N, E, index_batch_stride, gate, gate_want);
+    else
+      hipLaunchKernelGGL(coo_to_indptr_kernel<kCooPtrPerThread>, grid, dim3(kBlock), 0, s,
+                         index + b0 * index_batch_stride, ptr + b0 * (N + 1), N, E, index_batch_stride, gate, gate_want);
     return hipGetLastError() == hipSuccess ? (int)TS_OK : (int)TS_ERR_LAUNCH;
   });
 }

@@ -184,7 +184,25 @@ __global__ __launch_bounds__(kBlock) void csr_gather_small_kernel(CsrGatherArgs 
           if (++k == K) {
             k = 0;
             ++e;
-            while (row < rmax && s_ptr[row + 1] <= e) ++row;
+            if (row < rmax && s_ptr[row + 1] <= e) {
+              // the next row that has entries may lie thousands of rows on (the sparse end of a sorted index:
+              // walking there a row at a time took 80 us for 20 k entries over 50 k rows): gallop, then bisect
+              int lo = row + 1, hi = rmax + 1, step = 1;  // s_ptr[lo] <= e; hi: first row known to start behind e
+              while (lo + step <= rmax) {
+                if (s_ptr[lo + step] <= e) {
+                  lo += step;
+                  step <<= 1;
+                } else {
+                  hi = lo + step;
+                  break;
+                }
+              }
+              while (hi - lo > 1) {
+                const int mid = (lo + hi) >> 1;
+                if (s_ptr[mid] <= e) lo = mid; else hi = mid;
+              }
+              row = lo;
+            }
           }
         }
       }
@@ -320,7 +338,11 @@ template <typename T> int launch_csr_gather(const CsrGatherArgs &a, const CsrPla
 // the rows (index[e-1], index[e]]; thread E owns the rows after the last index.
 // Values outside [0, N) are clamped so that a malformed index cannot make the
 // reduction read or write out of bounds.
-constexpr int kCooPtrPerThread = 4;  // entries per thread: a quarter of the wavefronts to launch
+// entries per thread: 4 for a large index (a quarter of the wavefronts to launch), 1 below 2^20 entries, where the
+// launch is cheap either way and the rows of a sparse stretch of the index then spread over four times as many
+// wavefronts (20 k entries of a sorted Zipf index over 50 k rows: the last thousand entries own 45 k rows)
+constexpr int kCooPtrPerThread = 4;
+template <int PER>
 static __global__ __launch_bounds__(kBlock) void coo_to_indptr_kernel(const int64_t *__restrict__ index,
                                                                int64_t *__restrict__ ptr, int64_t N,
                                                                int64_t E, int64_t index_batch_stride,
@@ -331,15 +353,15 @@ static __global__ __launch_bounds__(kBlock) void coo_to_indptr_kernel(const int6
   if (threadIdx.x == 0) s_gaps.n = 0;
   __syncthreads();
   const int64_t b = blockIdx.y;
-  const int64_t e0 = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * kCooPtrPerThread;
+  const int64_t e0 = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * PER;
   const int64_t *idx = index + b * index_batch_stride;
   int64_t *p = ptr + b * (N + 1);
-  int64_t v[kCooPtrPerThread + 1];
+  int64_t v[PER + 1];
   v[0] = e0 == 0 || e0 > E ? -1 : idx[e0 - 1];
 #pragma unroll
-  for (int i = 0; i < kCooPtrPerThread; ++i) v[i + 1] = e0 + i < E ? idx[e0 + i] : N;
+  for (int i = 0; i < PER; ++i) v[i + 1] = e0 + i < E ? idx[e0 + i] : N;
 #pragma unroll
-  for (int i = 0; i < kCooPtrPerThread; ++i) {  // (no lane leaves early: the wavefront writes long ranges together)
+  for (int i = 0; i < PER; ++i) {  // (no lane leaves early: the wavefront writes long ranges together)
     const int64_t e = e0 + i;
     int64_t lo = v[i] + 1;
     int64_t hi = e == E ? N : v[i + 1];
