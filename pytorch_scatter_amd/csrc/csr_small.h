@@ -202,6 +202,18 @@ __global__ __launch_bounds__(kBlock) void csr_reduce_fixup_wave_kernel(CsrReduce
   const A *vals = static_cast<const A *>(a.ws_vals) + (b * a.nblk) * 2 * a.K;
   const int32_t *args = kArg ? a.ws_args + (b * a.nblk) * 2 * a.K : nullptr;
 
+  // a chain of more than kLongChain tiles (one row that holds most of a large input: 4 M entries of 16 floats in
+  // one row pass through 15 k tiles, 220 us for one wavefront) is shared by the wavefronts of the workgroup; the
+  // tiles of a workgroup number fewer than that, so at most one such chain begins in them
+  constexpr int kLongChain = 512;
+  constexpr int WV = kBlock / kWave;
+  __shared__ long long s_chain[3];  // t, last, first thread of the group that owns the row
+  __shared__ int s_nchain;
+  __shared__ A s_pv[WV][16];
+  __shared__ int32_t s_pa[WV][16];
+  if (threadIdx.x == 0) s_nchain = 0;
+  __syncthreads();
+
   auto absorb = [&](A &x, int32_t &xa, A y, int32_t ya) {
     if (kArg) {
       const bool better = (REDUCE == TS_MIN ? y < x : y > x) || (y == x && ya < xa);
@@ -224,8 +236,15 @@ __global__ __launch_bounds__(kBlock) void csr_reduce_fixup_wave_kernel(CsrReduce
   if (!has || last >= a.nblk) last = has ? a.nblk - 1 : tc;
   if (has && last > t) absorb(acc, arg, next_val, next_arg);
 
+  bool shared_chain = false;
+  if (has && last - t - 1 > kLongChain && lg == 0 && atomicAdd(&s_nchain, 1) == 0) {
+    s_chain[0] = t;
+    s_chain[1] = last;
+    s_chain[2] = threadIdx.x;
+    shared_chain = true;
+  }
   // chains that go on beyond the next tile: the whole wavefront works on one at a time
-  uint64_t pending = __ballot(has && last > t + 1 && lg == 0);
+  uint64_t pending = __ballot(has && last > t + 1 && lg == 0 && !shared_chain);
   while (pending != 0) {
     const int leader = __ffsll((unsigned long long)pending) - 1;
     pending &= pending - 1;
@@ -256,6 +275,42 @@ __global__ __launch_bounds__(kBlock) void csr_reduce_fixup_wave_kernel(CsrReduce
     const A total = __shfl(part, lg);
     const int32_t total_arg = __shfl(part_arg, lg);
     if (j == leader / G) absorb(acc, arg, total, total_arg);
+  }
+  __syncthreads();
+  if (s_nchain > 0) {  // uniform: the long chain, every wavefront a share of its tiles
+    const int64_t t_s = s_chain[0], last_s = s_chain[1];
+    const int owner = (int)s_chain[2];
+    const int wv = threadIdx.x / kWave;
+    A part = acc_init<A, REDUCE>();
+    int32_t part_arg = 0x7FFFFFFF;
+    const int64_t stride = (int64_t)WV * S;
+    for (int64_t t0 = t_s + 2 + wv * S + j; t0 <= last_s; t0 += stride * PF) {
+      A hv[PF];
+      int32_t ha[PF];
+#pragma unroll
+      for (int q = 0; q < PF; ++q) {
+        const int64_t tt = t0 + (int64_t)q * stride <= last_s ? t0 + (int64_t)q * stride : last_s;
+        hv[q] = vals[(tt * 2) * a.K + c];
+        ha[q] = kArg ? args[(tt * 2) * a.K + c] : 0;
+      }
+#pragma unroll
+      for (int q = 0; q < PF; ++q) {
+        if (t0 + (int64_t)q * stride <= last_s) absorb(part, part_arg, hv[q], ha[q]);
+      }
+    }
+    for (int off = S / 2; off >= 1; off >>= 1) {
+      const A o = __shfl_down(part, off * G);
+      const int32_t oa = __shfl_down(part_arg, off * G);
+      absorb(part, part_arg, o, oa);
+    }
+    if (j == 0) {
+      s_pv[wv][lg] = part;
+      s_pa[wv][lg] = part_arg;
+    }
+    __syncthreads();
+    if ((int)threadIdx.x >= owner && (int)threadIdx.x < owner + G) {
+      for (int w2 = 0; w2 < WV; ++w2) absorb(acc, arg, s_pv[w2][lg], s_pa[w2][lg]);
+    }
   }
   if (has) {
     T *out_b = static_cast<T *>(a.out) + b * a.N * a.K;

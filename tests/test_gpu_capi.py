@@ -398,6 +398,35 @@ def test_segment_coo(capi, oracle, case, reduce, dtype):
             assert_exact(cnt, want2)
 
 
+@pytest.mark.parametrize("K,E,reduce,dtype", [
+    (16, 400_000, "sum", torch.float32), (16, 400_000, "max", torch.float32), (16, 400_000, "mean", torch.float32),
+    (1, 2_400_000, "sum", torch.float32), (1, 2_400_000, "min", torch.float32), (4, 700_000, "max", torch.float32),
+    (16, 600_000, "max", torch.bfloat16), (3, 900_000, "sum", torch.int32), (2, 1_300_000, "max", torch.int64)])
+def test_segment_csr_one_row_through_hundreds_of_tiles(capi, oracle, K, E, reduce, dtype):
+    """Narrow rows, one segment that holds nearly all entries and so passes through more than 512 tiles of the
+    first kernel: its chain of partial results is combined by all wavefronts of a workgroup of the second kernel.
+    A few short segments either side of it, and a second long one behind it that stays with one wavefront."""
+    rng = np.random.default_rng(K + E)
+    deg = np.concatenate([rng.integers(0, 5, size=40), [E], rng.integers(0, 5, size=30), [E // 40],
+                          rng.integers(0, 3, size=20)])
+    n = deg.size
+    indptr = torch.from_numpy(np.concatenate([[0], np.cumsum(deg)]).astype(np.int64))
+    total = int(indptr[-1])
+    src = values(rng, (total, K), dtype, reduce)
+    want, want2 = oracle.segment_csr(src, indptr, None, reduce)
+    out = torch.full((n, K), 7, dtype=dtype, device=DEV)
+    arg = torch.full((n, K), -1, dtype=torch.long, device=DEV) if reduce in ("min", "max") else None
+    capi.segment_csr(src.to(DEV), indptr.to(DEV), out, arg, 1, n, total, K, 0, capi.REDUCE[reduce])
+    torch.cuda.synchronize()
+    if reduce in ("min", "max") or not dtype.is_floating_point:
+        assert_exact(out, want)
+        if arg is not None:
+            assert_exact(arg, want2)
+    else:
+        scale = float(oracle.segment_csr(src.abs().double(), indptr, None, "sum")[0].max())
+        assert_close(out, want, scale, dtype)
+
+
 GAP_KINDS = ["one_row", "empty_tail", "empty_head", "two_hubs", "every_3000th"]
 
 
