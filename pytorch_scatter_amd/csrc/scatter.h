@@ -1377,7 +1377,31 @@ template <typename T> __device__ __forceinline__ void table_add_out(T *p, T v, c
     atomic_add_elem<T>(p, v);
 }
 
-template <typename T>
+// the table's slot *= v: LDS has no atomic product, so a compare-and-swap loop on the slot's bits (an LDS round trip
+// per try, and only the lanes of one workgroup meet there)
+template <typename L> __device__ __forceinline__ void lds_slot_mul(L *slot, L v) {
+  typedef typename std::conditional<sizeof(L) == 8, uint64_t, uint32_t>::type U;
+  static_assert(sizeof(L) == sizeof(U), "");
+  U *word = reinterpret_cast<U *>(slot);
+  U old = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+  while (true) {
+    L cur;
+    __builtin_memcpy(&cur, &old, sizeof(L));
+    const L nv = cur * v;
+    U desired;
+    __builtin_memcpy(&desired, &nv, sizeof(L));
+    if (desired == old) return;
+    if (__hip_atomic_compare_exchange_strong(word, &old, desired, __ATOMIC_RELAXED, __ATOMIC_RELAXED,
+                                             __HIP_MEMORY_SCOPE_WORKGROUP))
+      return;
+  }
+}
+
+// MUL = true: the same table for products (slots start at 1 and are multiplied into out). A product has no
+// hardware atomic at all, so every entry that reaches memory is a compare-and-swap loop whose time grows with
+// the square of the entries that meet in one element (1 M entries of 8 floats, 30 % of them on one row: 89 ms
+// through scatter_atomic_kernel); here a row's entries meet in LDS and memory sees one factor per row and workgroup.
+template <typename T, bool MUL = false>
 __global__ __launch_bounds__(kLdsAddBlock) void scatter_add_lds_kernel(ScatterArgs a, int tn_mask, int64_t epb) {
   constexpr int U = 4;
   if (a.skip_flag != nullptr && (*a.skip_flag != 0) != (a.skip_inverse != 0)) return;
@@ -1389,7 +1413,7 @@ __global__ __launch_bounds__(kLdsAddBlock) void scatter_add_lds_kernel(ScatterAr
   __shared__ int32_t s_tags[kLdsAccRows];
   const int K = (int)a.K;
   const int tn = tn_mask + 1;
-  for (int i = threadIdx.x; i < tn * K; i += kLdsAddBlock) s_acc[i] = (LdsAcc)0;
+  for (int i = threadIdx.x; i < tn * K; i += kLdsAddBlock) s_acc[i] = (LdsAcc)(MUL ? 1 : 0);
   for (int i = threadIdx.x; i < tn; i += kLdsAddBlock) s_tags[i] = -1;
   __syncthreads();
 
@@ -1424,15 +1448,33 @@ __global__ __launch_bounds__(kLdsAddBlock) void scatter_add_lds_kernel(ScatterAr
             const int old = atomicCAS(&s_tags[row], -1, node);
             tag = old == -1 ? node : old;
           }
-          if (tag == node)
+          if (MUL) {
+            if (tag == node) {
+              lds_slot_mul<LdsAcc>(&s_acc[row * K + k], (LdsAcc)x[u]);
+            } else {
+              const T f = from_acc<T>(x[u]);
+              atomic_rmw<T>(out + (int64_t)node * a.K + k, [f](T cur) { return mul_elem<T>(cur, f); });
+            }
+          } else if (tag == node) {
             __hip_atomic_fetch_add(&s_acc[row * K + k], (LdsAcc)x[u], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-          else
+          } else {
             table_add_out<T>(out + (int64_t)node * a.K + k, from_acc<T>(x[u]), out, out_end);
+          }
         }
       }
     }
   }
   __syncthreads();
+  if constexpr (MUL) {
+    for (int i = threadIdx.x; i < tn * K; i += kLdsAddBlock) {
+      const LdsAcc v = s_acc[i];
+      if (v == (LdsAcc)1) continue;
+      const int row = i / K;
+      const T f = from_acc<T>((typename Acc<T>::type)v);
+      atomic_rmw<T>(out + (int64_t)s_tags[row] * a.K + (i - row * K), [f](T cur) { return mul_elem<T>(cur, f); });
+    }
+    return;
+  }
   if constexpr (__is_same(T, bf16_t) || __is_same(T, f16_t)) {
     // two neighbouring columns per packed add when the rows allow it
     if ((K & 1) == 0 && (reinterpret_cast<uintptr_t>(out) & 3) == 0) {
@@ -1893,6 +1935,20 @@ int launch_scatter_v(const ScatterArgs &args, int reduce, hipStream_t stream) {
         }
         hipLaunchKernelGGL((scatter_atomic_kernel<T, 1, TS_SUM>), dim3(g), dim3(kBlock), 0, stream, a);
       } else {
+        // products of the types that the accumulator table takes, one index per row: through the table from 2^16
+        // elements on (below, the call is its launches)
+        if constexpr (__is_same(T, float) || __is_same(T, bf16_t) || __is_same(T, f16_t) || __is_same(T, double) ||
+                      __is_same(T, int32_t) || __is_same(T, int64_t)) {
+          int tm = 1;
+          while ((int64_t)tm * 2 * a.K <= kLdsAcc && tm * 2 <= kLdsAccRows) tm *= 2;
+          if (a.lds_cache && a.sk == 0 && tm >= 64 && a.B * a.N < 0x7FFFFFFFll && n_src >= ((int64_t)1 << 16)) {
+            const int64_t epb = per_cu_chunk_edges(a.lds_epb, n_edges, sum_table_min_chunk(a.K, 4),
+                                                   131072 / a.K > 2048 ? 131072 / a.K : 2048);
+            hipLaunchKernelGGL((scatter_add_lds_kernel<T, true>), dim3((unsigned)((n_edges + epb - 1) / epb)),
+                               dim3(kLdsAddBlock), 0, stream, a, tm - 1, epb);
+            return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
+          }
+        }
         hipLaunchKernelGGL((scatter_atomic_kernel<T, 1, TS_MUL>), dim3(g), dim3(kBlock), 0, stream, a);
       }
     }
