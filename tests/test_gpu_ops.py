@@ -568,27 +568,36 @@ def test_scatter_sum_of_narrow_integers_under_a_hub(ts, dtype, K):
     assert torch.equal(mean.cpu(), torch.div(want.to(dtype), count, rounding_mode="floor"))
 
 
-@pytest.mark.parametrize("dtype,K", product([torch.float32, torch.float64, torch.int32], [1, 5]))
-def test_scatter_mul_under_a_hub(ts, dtype, K):
-    """Products of a row that takes a third of the entries: the lanes of a wavefront combine before the
-    compare-and-swap; the result is the product whatever the order."""
+@pytest.mark.parametrize("dtype,K,E", product([torch.float32, torch.float64, torch.int32, torch.int64], [1, 5, 100],
+                                              [30000, 200_000]))
+def test_scatter_mul_under_a_hub(ts, dtype, K, E):
+    """Products of a row that takes a third of the entries: below 2^16 elements the lanes of a wavefront combine
+    before the compare-and-swap in memory, above the factors of a row meet in the table in LDS; the result is the
+    product whatever the order."""
     g = torch.Generator().manual_seed(4)
-    E, N = 30000, 300
+    N = 300
+    if E * K > 4_000_000:
+        pytest.skip("covered by the smaller input")
     index = torch.where(torch.rand(E, generator=g) < 0.3, torch.tensor(11), torch.randint(0, N, (E,), generator=g))
-    if dtype == torch.int32:
-        src = torch.where(torch.rand((E, K), generator=g) < 0.01, 3, 1).to(dtype) * \
+    integer = not dtype.is_floating_point
+    if integer:
+        # a factor of 3 now and then (at most 3^39 per row: fits 64 bits), signs at random
+        src = torch.where(torch.rand((E, K), generator=g) < 0.01 * 30000 / E, 3, 1).to(dtype) * \
             torch.where(torch.rand((E, K), generator=g) < 0.5, 1, -1).to(dtype)
     else:
-        src = (torch.rand((E, K), generator=g, dtype=torch.float64) * 0.02 + 0.99).to(dtype)
-    got = ts.scatter(src.to(DEV), index.to(DEV), 0, None, N, "mul").cpu()
-    want = torch.ones((N, K), dtype=torch.float64)
-    want = want.scatter_reduce(0, index.view(E, 1).expand(E, K), src.double(), "prod")
-    if dtype == torch.int32:
-        wrapped = torch.ones((N, K), dtype=torch.int64).scatter_reduce(
-            0, index.view(E, 1).expand(E, K), src.long(), "prod")  # at most 3^k: fits 64 bits for these inputs
-        assert torch.equal(got.long(), wrapped.to(torch.int32).long())
-    else:
-        assert torch.allclose(got.double(), want, rtol=1e-4 if dtype == torch.float32 else 1e-11)
+        src = (torch.rand((E, K), generator=g, dtype=torch.float64) * (600.0 / E) + (1 - 300.0 / E)).to(dtype)
+    for out_given in (False, True):
+        prev = torch.where(torch.rand((N, K), generator=g) < 0.5, 2, -1).to(dtype)
+        out = prev.clone().to(DEV) if out_given else None
+        got = ts.scatter(src.to(DEV), index.to(DEV), 0, out, None if out_given else N, "mul").cpu()
+        start = prev.double() if out_given else torch.ones((N, K), dtype=torch.float64)
+        want = start.scatter_reduce(0, index.view(E, 1).expand(E, K), src.double(), "prod")
+        if integer:
+            start64 = prev.long() if out_given else torch.ones((N, K), dtype=torch.int64)
+            wrapped = start64.scatter_reduce(0, index.view(E, 1).expand(E, K), src.long(), "prod")
+            assert torch.equal(got.long(), wrapped.to(dtype).long())
+        else:
+            assert torch.allclose(got.double(), want, rtol=1e-4 if dtype == torch.float32 else 1e-11)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.int64])
