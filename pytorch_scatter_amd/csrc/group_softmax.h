@@ -294,6 +294,104 @@ __global__ __launch_bounds__(kBlock) void group_sum_run_kernel(ScatterArgs a, Gr
   });
 }
 
+// The same pass through a workgroup's accumulator table (the design of scatter_add_lds_kernel in scatter.h): the
+// terms of a group meet in LDS and reach gsum once per group and workgroup. The run kernel above sends every term
+// of an unsorted index to memory, and the terms of a hub group to one address, 7 ns apiece: 1 M single values, 30 %
+// of them in one group: 2.0 ms for this pass (100 k x 8: 0.34 ms); its hot rows do not catch such a group.
+template <typename T, int MODE>
+__global__ __launch_bounds__(kLdsAddBlock) void group_sum_lds_kernel(ScatterArgs a, GroupArgs g, int tn_mask, int64_t epb) {
+  typedef typename Acc<T>::type A;
+  typedef double LdsAcc;
+  constexpr int U = 4;
+  __shared__ LdsAcc s_acc[kLdsAcc];
+  __shared__ int32_t s_tags[kLdsAccRows];
+  if (g.gate != nullptr && *g.gate == 0) return;
+  GroupSumRun<T, 1, MODE> p;
+  p.src = static_cast<const T *>(g.src);
+  p.grad = static_cast<const T *>(g.grad);
+  p.gmax = g.gmax;
+  p.gsum = static_cast<A *>(g.gsum);
+  p.total = static_cast<const T *>(g.total);
+  p.count = g.count;
+  p.K = g.K;
+  p.gs = g.gs;
+  const int K = (int)g.K;
+  const int tn = tn_mask + 1;
+  for (int i = threadIdx.x; i < tn * K; i += kLdsAddBlock) s_acc[i] = 0.0;
+  for (int i = threadIdx.x; i < tn; i += kLdsAddBlock) s_tags[i] = -1;
+  __syncthreads();
+  const EdgeLanes m = edge_lanes(K, kLdsAddBlock);
+  const int64_t be_lo = (int64_t)blockIdx.x * epb;
+  int64_t be_hi = be_lo + epb;
+  if (be_hi > a.B * a.E) be_hi = a.B * a.E;
+  if (m.active) {
+    for (int64_t be0 = be_lo + m.el; be0 < be_hi; be0 += (int64_t)m.epp * U) {
+      for (int k = m.cl; k < K; k += m.L) {
+        A x[U];
+        int node[U];
+        int64_t bec[U], pos[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const int64_t be = be0 + (int64_t)u * m.epp;
+          bec[u] = be < be_hi ? be : be0;
+          int64_t b;
+          split_edge(bec[u], a.B, a.E, b, pos[u]);
+          const int64_t idx = a.index[b * a.sb + pos[u] * a.se];
+          node[u] = (be < be_hi && idx >= 0 && idx < a.N) ? (int)(b * a.N + idx) : -1;
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) p.load(bec[u], pos[u], k, node[u], &x[u]);
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          if (node[u] < 0) continue;
+          const int row = node[u] & tn_mask;
+          int tag = s_tags[row];
+          if (tag == -1) {
+            const int old = atomicCAS(&s_tags[row], -1, node[u]);
+            tag = old == -1 ? node[u] : old;
+          }
+          if (tag == node[u])
+            __hip_atomic_fetch_add(&s_acc[row * K + k], (LdsAcc)x[u], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+          else
+            p.to_memory(node[u], k, &x[u]);
+        }
+      }
+    }
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < tn * K; i += kLdsAddBlock) {
+    const LdsAcc v = s_acc[i];
+    if (v == 0.0) continue;
+    const int row = i / K;
+    const A out = (A)v;
+    p.to_memory(s_tags[row], i - row * K, &out);
+  }
+}
+// sizes from which the pass goes through the table: 2^16 terms, rows of up to 128 columns (64 table rows), group
+// numbers that fit 31 bits; entries per workgroup as for the sums of scatter (sum_table_min_chunk)
+inline bool group_sum_table_ok(const GroupArgs &g, int elem_bytes, bool one_pass_modes, int *tn_out) {
+  int tn = 1;
+  while ((int64_t)tn * 2 * g.K <= kLdsAcc && tn * 2 <= kLdsAccRows) tn *= 2;
+  *tn_out = tn;
+  if (const char *env = getenv("TS_GROUP_TABLE")) {  // tuning aid: 0 keeps the run kernel
+    if (atoi(env) == 0) return false;
+  }
+  // From 2^23 terms on only where a sorted index never gets here (softmax and its backward with rows of up to 128
+  // bytes: the one-pass kernels take it): a large sorted index needs one atomic per run through the run kernel and
+  // loses through the table (scatter_std of 9 M entries of 8 floats, sorted: 436 -> 703 us; unsorted 1401 -> 1448).
+  const int64_t n_src = g.B * g.E * g.K;
+  return tn >= 64 && g.B * g.N < 0x7FFFFFFFll && n_src >= ((int64_t)1 << 16) &&
+         (n_src < ((int64_t)1 << 23) || (one_pass_modes && g.K * elem_bytes <= 128));
+}
+template <typename T, int MODE>
+void launch_group_sum_lds(const ScatterArgs &a, const GroupArgs &g, int tn, hipStream_t stream) {
+  const int64_t n_edges = g.B * g.E;
+  const int64_t epb = per_cu_chunk_edges(0, n_edges, sum_table_min_chunk(g.K, 4),
+                                         131072 / g.K > 2048 ? 131072 / g.K : 2048);
+  hipLaunchKernelGGL((group_sum_lds_kernel<T, MODE>), dim3((unsigned)((n_edges + epb - 1) / epb)), dim3(kLdsAddBlock), 0,
+                     stream, a, g, tn - 1, epb);
+}
+
 // ---- pass 3: the elementwise finish
 template <typename T, int VEC, int MODE>
 __global__ __launch_bounds__(kBlock) void group_finish_kernel(GroupArgs g) {
@@ -476,8 +574,12 @@ int launch_group_softmax_m(const GroupArgs &g_in, hipStream_t stream) {
   if (kForward)
     TS_LAUNCH_RUN(rg.serial, (group_max_run_kernel<T, VEC, true>), (group_max_run_kernel<T, VEC, false>), gd, stream, a, g,
                   rg.lshift, rg.rpw);
-  TS_LAUNCH_RUN(rg.serial, (group_sum_run_kernel<T, VEC, MODE, true>), (group_sum_run_kernel<T, VEC, MODE, false>), gd,
-                stream, a, g, rg.lshift, rg.rpw, rg.hot_rlog);
+  int tn = 1;
+  if (group_sum_table_ok(g, (int)sizeof(T), true, &tn))
+    launch_group_sum_lds<T, MODE>(a, g, tn, stream);
+  else
+    TS_LAUNCH_RUN(rg.serial, (group_sum_run_kernel<T, VEC, MODE, true>), (group_sum_run_kernel<T, VEC, MODE, false>), gd,
+                  stream, a, g, rg.lshift, rg.rpw, rg.hot_rlog);
   hipLaunchKernelGGL((group_finish_kernel<T, VEC, MODE>), dim3(scatter_grid(n_edges, g.K / VEC, kBlock, 4)),
                      dim3(kBlock), 0, stream, g);
   return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
@@ -500,8 +602,12 @@ int launch_group_lse_v(const GroupArgs &g, bool backward, hipStream_t stream) {
   hipLaunchKernelGGL(group_init_kernel<T>, dim3(g_out), dim3(kBlock), 0, stream, g, 1);
   TS_LAUNCH_RUN(rg.serial, (group_max_run_kernel<T, VEC, true>), (group_max_run_kernel<T, VEC, false>), gd, stream, a, g,
                 rg.lshift, rg.rpw);
-  TS_LAUNCH_RUN(rg.serial, (group_sum_run_kernel<T, VEC, GS_LSE, true>), (group_sum_run_kernel<T, VEC, GS_LSE, false>), gd,
-                stream, a, g, rg.lshift, rg.rpw, rg.hot_rlog);
+  int tn = 1;
+  if (group_sum_table_ok(g, (int)sizeof(T), false, &tn))
+    launch_group_sum_lds<T, GS_LSE>(a, g, tn, stream);
+  else
+    TS_LAUNCH_RUN(rg.serial, (group_sum_run_kernel<T, VEC, GS_LSE, true>), (group_sum_run_kernel<T, VEC, GS_LSE, false>), gd,
+                  stream, a, g, rg.lshift, rg.rpw, rg.hot_rlog);
   hipLaunchKernelGGL(group_lse_finish_kernel<T>, dim3(g_out), dim3(kBlock), 0, stream, g);
   return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
 }
@@ -521,7 +627,10 @@ int launch_group_std_v(const GroupArgs &g, bool backward, hipStream_t stream) {
   const dim3 gd(rg.blocks, rg.ychunks);
   const unsigned g_out = grid_for(g.B * g.N * g.K);
   hipLaunchKernelGGL(group_init_kernel<T>, dim3(g_out), dim3(kBlock), 0, stream, g, 0);
-  if (n_edges > 0)
+  int tn = 1;
+  if (n_edges > 0 && group_sum_table_ok(g, (int)sizeof(T), false, &tn))
+    launch_group_sum_lds<T, GS_STD>(a, g, tn, stream);
+  else if (n_edges > 0)
     TS_LAUNCH_RUN(rg.serial, (group_sum_run_kernel<T, VEC, GS_STD, true>), (group_sum_run_kernel<T, VEC, GS_STD, false>), gd,
                   stream, a, g, rg.lshift, rg.rpw, rg.hot_rlog);
   hipLaunchKernelGGL(group_std_finish_kernel<T>, dim3(g_out), dim3(kBlock), 0, stream, g);
