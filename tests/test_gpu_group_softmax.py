@@ -24,6 +24,8 @@ SHAPES = [
     # B, E, K, N
     (1, 5000, 1, 300), (2, 3000, 4, 50), (1, 2000, 8, 100), (1, 1500, 3, 40), (1, 900, 64, 20),
     (1, 700, 130, 9), (3, 400, 16, 7), (1, 1, 1, 1), (1, 257, 2, 300),
+    # 2^16 terms and more, rows of up to 128 columns: the group sums go through the accumulator table
+    (1, 70_000, 1, 3000), (2, 6000, 8, 500), (1, 1200, 64, 90), (1, 600, 128, 40),
 ]
 
 
@@ -53,9 +55,9 @@ def make_index(kind, rng, E, N):
     return torch.from_numpy(idx)
 
 
-def forward_bound(dtype, want64, z64, log_space):
+def forward_bound(dtype, want64, z64, log_space, exact=True):
     e = EPS_T[dtype]
-    if dtype in (torch.float32, torch.float64):
+    if dtype in (torch.float32, torch.float64) and exact:
         return e * want64.abs() + e * (1.0 if log_space else 1e-30)
     if log_space:
         return e * (4.0 + want64.abs() + z64.abs())
@@ -66,7 +68,10 @@ def forward_bound(dtype, want64, z64, log_space):
 def check_against_oracle(capi, oracle, src, grad, index1, shape, dtype):
     B, E, K, N = shape
     index = index1.view(1, E, 1).expand(B, E, K)
-    exact = dtype in (torch.float32, torch.float64)
+    # fp32 / fp64 against the oracle's sequence in the same type -- for groups of up to a few thousand entries: the
+    # fp32 sum of a group of 35 000 terms in entry order is itself 1e-5 away from the exact one, so the large
+    # shapes are checked against the oracle in fp64, like the 16-bit types
+    exact = dtype in (torch.float32, torch.float64) and E <= 10_000
     ref_src = src if exact else src.double()
     inside = (index >= 0) & (index < N)
     safe = index.clamp(0, N - 1)
@@ -90,7 +95,7 @@ def check_against_oracle(capi, oracle, src, grad, index1, shape, dtype):
             want = torch.zeros((B, E, K), dtype=torch.float64)
             want[:, keep] = part
         err = (out.cpu().double() - want).abs()
-        bound = forward_bound(dtype, want, z64, log_space)
+        bound = forward_bound(dtype, want, z64, log_space, exact)
         assert bool((err <= bound).all()), (log_space, float((err - bound).max()))
         assert float(out.cpu().double()[~inside].abs().max() if bool((~inside).any()) else 0.0) == 0.0
 
@@ -401,6 +406,8 @@ STD_SHAPES = [
     # B, E, K, N
     (1, 5000, 1, 600), (2, 3000, 4, 300), (1, 2000, 8, 250), (1, 1500, 3, 200), (1, 900, 64, 100),
     (1, 700, 130, 80), (3, 400, 16, 50), (1, 1, 1, 1), (1, 257, 2, 300),
+    # 2^16 terms and more, rows of up to 128 columns: the group sums go through the accumulator table
+    (1, 70_000, 1, 3000), (2, 6000, 8, 500), (1, 1200, 64, 90), (1, 600, 128, 40),
 ]
 
 
@@ -455,6 +462,8 @@ def test_std_forward_and_backward_capi(capi, oracle, shape, kind, dtype, unbiase
     scale = (grad.double().abs() / std64.clamp_min(1e-300)).gather(1, index)
     cnt = cnt_n.gather(1, index)
     gbound = (8 if exact else 16) * e * (want_g.abs() + scale * mean_abs.gather(1, index) / cnt)
+    if dtype == torch.float16:
+        gbound = gbound + 2.0 ** -24  # gradients below 2^-14 are subnormal in fp16: absolute spacing 2^-24
     gerr = (got_g - want_g).abs()
     assert bool((gerr[live] <= gbound[live]).all()), float((gerr[live] - gbound[live]).max())
 
