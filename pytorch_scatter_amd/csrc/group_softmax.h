@@ -367,21 +367,94 @@ __global__ __launch_bounds__(kLdsAddBlock) void group_sum_lds_kernel(ScatterArgs
     p.to_memory(s_tags[row], i - row * K, &out);
   }
 }
+// Pass 1 the same way: the keys of a group meet in LDS (an atomic max there) and each workgroup sends one key per
+// group it met to gmax. Under a hub the run kernel reads and raises one address from every wavefront: 1 M single
+// values, 30 % of them in one group: 100-320 us for this pass.
+template <typename T>
+__global__ __launch_bounds__(kLdsAddBlock) void group_max_lds_kernel(ScatterArgs a, GroupArgs g, int tn_mask, int64_t epb) {
+  typedef typename GroupMaxRun<T, 1>::A KB;
+  constexpr int U = 4;
+  __shared__ KB s_keys[kLdsAcc];
+  __shared__ int32_t s_tags[kLdsAccRows];
+  if (g.gate != nullptr && *g.gate == 0) return;
+  GroupMaxRun<T, 1> p;
+  p.src = static_cast<const T *>(g.src);
+  p.gmax = static_cast<KB *>(g.gmax);
+  p.K = g.K;
+  p.gs = g.gs;
+  const int K = (int)g.K;
+  const int tn = tn_mask + 1;
+  for (int i = threadIdx.x; i < tn * K; i += kLdsAddBlock) s_keys[i] = (KB)0;
+  for (int i = threadIdx.x; i < tn; i += kLdsAddBlock) s_tags[i] = -1;
+  __syncthreads();
+  const EdgeLanes m = edge_lanes(K, kLdsAddBlock);
+  const int64_t be_lo = (int64_t)blockIdx.x * epb;
+  int64_t be_hi = be_lo + epb;
+  if (be_hi > a.B * a.E) be_hi = a.B * a.E;
+  if (m.active) {
+    for (int64_t be0 = be_lo + m.el; be0 < be_hi; be0 += (int64_t)m.epp * U) {
+      for (int k = m.cl; k < K; k += m.L) {
+        KB x[U];
+        int node[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const int64_t be = be0 + (int64_t)u * m.epp;
+          const int64_t bec = be < be_hi ? be : be0;
+          int64_t b, pos;
+          split_edge(bec, a.B, a.E, b, pos);
+          const int64_t idx = a.index[b * a.sb + pos * a.se];
+          node[u] = (be < be_hi && idx >= 0 && idx < a.N) ? (int)(b * a.N + idx) : -1;
+          p.load(bec, pos, k, node[u], &x[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          if (node[u] < 0 || x[u] == (KB)0) continue;  // 0: a NaN, which never wins
+          const int row = node[u] & tn_mask;
+          int tag = s_tags[row];
+          if (tag == -1) {
+            const int old = atomicCAS(&s_tags[row], -1, node[u]);
+            tag = old == -1 ? node[u] : old;
+          }
+          if (tag == node[u])
+            __hip_atomic_fetch_max(&s_keys[row * K + k], x[u], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+          else
+            p.emit(node[u], k, &x[u]);
+        }
+      }
+    }
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < tn * K; i += kLdsAddBlock) {
+    const KB v = s_keys[i];
+    if (v == (KB)0) continue;
+    const int row = i / K;
+    p.emit(s_tags[row], i - row * K, &v);
+  }
+}
+template <typename T>
+void launch_group_max_lds(const ScatterArgs &a, const GroupArgs &g, int tn, hipStream_t stream) {
+  const int64_t n_edges = g.B * g.E;
+  const int64_t epb = per_cu_chunk_edges(0, n_edges, sum_table_min_chunk(g.K, 4),
+                                         131072 / g.K > 2048 ? 131072 / g.K : 2048);
+  hipLaunchKernelGGL(group_max_lds_kernel<T>, dim3((unsigned)((n_edges + epb - 1) / epb)), dim3(kLdsAddBlock), 0, stream,
+                     a, g, tn - 1, epb);
+}
+
 // sizes from which the pass goes through the table: 2^16 terms, rows of up to 128 columns (64 table rows), group
 // numbers that fit 31 bits; entries per workgroup as for the sums of scatter (sum_table_min_chunk)
-inline bool group_sum_table_ok(const GroupArgs &g, int elem_bytes, bool one_pass_modes, int *tn_out) {
+inline bool group_sum_table_ok(const GroupArgs &g, int *tn_out) {
   int tn = 1;
   while ((int64_t)tn * 2 * g.K <= kLdsAcc && tn * 2 <= kLdsAccRows) tn *= 2;
   *tn_out = tn;
   if (const char *env = getenv("TS_GROUP_TABLE")) {  // tuning aid: 0 keeps the run kernel
     if (atoi(env) == 0) return false;
   }
-  // From 2^23 terms on only where a sorted index never gets here (softmax and its backward with rows of up to 128
-  // bytes: the one-pass kernels take it): a large sorted index needs one atomic per run through the run kernel and
-  // loses through the table (scatter_std of 9 M entries of 8 floats, sorted: 436 -> 703 us; unsorted 1401 -> 1448).
+  // Up to 2^23 terms. Beyond, the run kernels are ahead on the index of a graph (9 M entries of 8 floats of a real
+  // graph in random order: softmax 1182 us, 1339 us with both passes through the table; scatter_std of the same
+  // entries in order 436 -> 703 us), and their hot rows do hold a hub at that size (10 M x 8 with a 20 % hub: no
+  // extra cost).
   const int64_t n_src = g.B * g.E * g.K;
-  return tn >= 64 && g.B * g.N < 0x7FFFFFFFll && n_src >= ((int64_t)1 << 16) &&
-         (n_src < ((int64_t)1 << 23) || (one_pass_modes && g.K * elem_bytes <= 128));
+  return tn >= 64 && g.B * g.N < 0x7FFFFFFFll && n_src >= ((int64_t)1 << 16) && n_src < ((int64_t)1 << 23);
 }
 template <typename T, int MODE>
 void launch_group_sum_lds(const ScatterArgs &a, const GroupArgs &g, int tn, hipStream_t stream) {
@@ -571,11 +644,14 @@ int launch_group_softmax_m(const GroupArgs &g_in, hipStream_t stream) {
   const dim3 gd(rg.blocks, rg.ychunks);
   hipLaunchKernelGGL(group_init_kernel<T>, dim3(grid_for(g.B * g.N * g.K)), dim3(kBlock), 0, stream, g,
                      kForward ? 1 : 0);
-  if (kForward)
+  int tn = 1;
+  const bool table = group_sum_table_ok(g, &tn);
+  if (kForward && table)
+    launch_group_max_lds<T>(a, g, tn, stream);
+  else if (kForward)
     TS_LAUNCH_RUN(rg.serial, (group_max_run_kernel<T, VEC, true>), (group_max_run_kernel<T, VEC, false>), gd, stream, a, g,
                   rg.lshift, rg.rpw);
-  int tn = 1;
-  if (group_sum_table_ok(g, (int)sizeof(T), true, &tn))
+  if (table)
     launch_group_sum_lds<T, MODE>(a, g, tn, stream);
   else
     TS_LAUNCH_RUN(rg.serial, (group_sum_run_kernel<T, VEC, MODE, true>), (group_sum_run_kernel<T, VEC, MODE, false>), gd,
@@ -600,10 +676,14 @@ int launch_group_lse_v(const GroupArgs &g, bool backward, hipStream_t stream) {
   const dim3 gd(rg.blocks, rg.ychunks);
   const unsigned g_out = grid_for(g.B * g.N * g.K);
   hipLaunchKernelGGL(group_init_kernel<T>, dim3(g_out), dim3(kBlock), 0, stream, g, 1);
-  TS_LAUNCH_RUN(rg.serial, (group_max_run_kernel<T, VEC, true>), (group_max_run_kernel<T, VEC, false>), gd, stream, a, g,
-                rg.lshift, rg.rpw);
   int tn = 1;
-  if (group_sum_table_ok(g, (int)sizeof(T), false, &tn))
+  const bool table = group_sum_table_ok(g, &tn);
+  if (table)
+    launch_group_max_lds<T>(a, g, tn, stream);
+  else
+    TS_LAUNCH_RUN(rg.serial, (group_max_run_kernel<T, VEC, true>), (group_max_run_kernel<T, VEC, false>), gd, stream, a, g,
+                  rg.lshift, rg.rpw);
+  if (table)
     launch_group_sum_lds<T, GS_LSE>(a, g, tn, stream);
   else
     TS_LAUNCH_RUN(rg.serial, (group_sum_run_kernel<T, VEC, GS_LSE, true>), (group_sum_run_kernel<T, VEC, GS_LSE, false>), gd,
@@ -628,7 +708,7 @@ int launch_group_std_v(const GroupArgs &g, bool backward, hipStream_t stream) {
   const unsigned g_out = grid_for(g.B * g.N * g.K);
   hipLaunchKernelGGL(group_init_kernel<T>, dim3(g_out), dim3(kBlock), 0, stream, g, 0);
   int tn = 1;
-  if (n_edges > 0 && group_sum_table_ok(g, (int)sizeof(T), false, &tn))
+  if (n_edges > 0 && group_sum_table_ok(g, &tn))
     launch_group_sum_lds<T, GS_STD>(a, g, tn, stream);
   else if (n_edges > 0)
     TS_LAUNCH_RUN(rg.serial, (group_sum_run_kernel<T, VEC, GS_STD, true>), (group_sum_run_kernel<T, VEC, GS_STD, false>), gd,
