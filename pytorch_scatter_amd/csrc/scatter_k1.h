@@ -61,7 +61,7 @@ inline K1Plan k1_plan(int64_t B, int64_t E, int64_t K, int64_t N, int elem_bytes
                       bool any_size) {
   K1Plan p = {};
   if (B != 1 || K != 1 || elem_bytes != 4 || E < 1 || N < 1 || E >= 0xFFFFFFFEll ||
-      N > (int64_t)kK1PerRow * kK1Rows || (!any_size && E < ((int64_t)1 << 23)))
+      N > (int64_t)kK1PerRow * kK1Rows || (!any_size && E < ((int64_t)1 << 14)))
     return p;
   int64_t G = (E + kK1Batch - 1) / kK1Batch;
   if (G > kK1Groups) G = kK1Groups;
