@@ -813,7 +813,7 @@ def test_scatter_sum_binned_variant(capi, oracle, shape, kind, dtype, monkeypatc
         assert bool((err <= bound).all()), (kind, out_given, float((err - bound).max()))
 
 
-SORTED_KINDS = ["sorted", "sorted gaps", "one descent", "beyond N", "negative first"]
+SORTED_KINDS = ["sorted", "sorted gaps", "one descent", "beyond N", "negative first", "empty tail", "one row"]
 
 
 @pytest.mark.parametrize("shape,reduce,kind,dtype", list(product(
@@ -841,6 +841,10 @@ def test_scatter_sorted_index_with_workspace(capi, oracle, shape, reduce, kind, 
         idx = np.sort(rng.choice(np.arange(0, N, 3), size=E))
     if kind == "one descent":
         idx[E // 2], idx[E // 2 + 1] = N - 1, 0
+    if kind == "empty tail":  # long ranges of rows without entries: written by a wavefront or the workgroup
+        idx = np.sort(rng.integers(0, max(N // 100, 1), size=E))
+    if kind == "one row":
+        idx = np.full(E, N // 2)
     if kind == "beyond N":
         idx[-3:] = N + 5
     if kind == "negative first":
