@@ -209,8 +209,10 @@ int ts_scatter(const void *src, const int64_t *index, void *out,
  * (scatter_cuda allocates nothing beyond its outputs, csrc/cuda/scatter_cuda.cu:54-138). */
 size_t ts_scatter_workspace_bytes(int64_t B, int64_t E, int64_t K, int64_t N,
                                   int dtype, int reduce);
-/* MIN / MAX of one 4-byte value per entry (K == 1, B == 1, large E, N <= 262144) keep their table of packed
- * keys in the first ts_scatter_workspace_zero_bytes() bytes of the workspace instead of in arg_out. Those bytes
+/* MIN / MAX of one 4-byte value per entry (K == 1, B == 1, E >= 16384, N <= 524288) keep their table of packed
+ * keys in the first ts_scatter_workspace_zero_bytes() bytes of the workspace instead of in arg_out. That part has
+ * one size (4 MiB) for every such call, whatever N, so a workspace kept across calls with different N stays
+ * valid: everything a call writes behind it (its slabs) is never read as zero by a later call. Those bytes
  * must read as zero when ts_scatter_with_workspace starts, and the call puts them back to zero before it ends:
  * a caller that keeps its workspace from call to call (one per stream) clears it once and never pays for an
  * initial fill again; a caller that takes fresh memory for every call clears that part first

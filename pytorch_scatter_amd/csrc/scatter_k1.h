@@ -69,7 +69,10 @@ inline K1Plan k1_plan(int64_t B, int64_t E, int64_t K, int64_t N, int elem_bytes
   p.J = (int)((N + kK1Rows - 1) / kK1Rows);
   p.epb = ((E + G - 1) / G + 3) & ~(int64_t)3;
   auto up = [](size_t x) { return (x + 255) & ~(size_t)255; };
-  const size_t o_keys = up((size_t)N * 8), o_tags = o_keys + up((size_t)G * kK1Rows * 8);
+  // The key table takes the room of the largest N this plan serves, whatever N is: a workspace kept from call
+  // to call then has the same zero-on-entry part for every call, and the slabs of one call never land in what a
+  // later call with more output rows reads as its (zero) key table.
+  const size_t o_keys = up((size_t)kK1PerRow * kK1Rows * 8), o_tags = o_keys + up((size_t)G * kK1Rows * 8);
   p.zero_bytes = o_keys;
   p.bytes = o_tags + up((size_t)G * kK1Rows * 4);
   if (ws == nullptr || ws_bytes < p.bytes || (reinterpret_cast<uintptr_t>(ws) & 15) != 0) return p;

@@ -1570,3 +1570,35 @@ def test_scatter_minmax_one_value_per_entry_with_workspace(capi, oracle, case, r
         assert_exact(out, want, f"values rep={rep}")
         assert_exact(arg, want_arg, f"arg rep={rep}")
         assert bool((ws[:nzero] == 0).all()), "the key table is handed back as zeros"
+
+
+@pytest.mark.parametrize("reduce", ["min", "max"])
+def test_scatter_k1_workspace_kept_across_calls_with_different_row_counts(capi, oracle, reduce):
+    """One workspace, cleared once, reused for calls whose N goes up and down: the zero-on-entry part has one
+    size for every N, so the slabs of a call with few rows never sit where a later call keeps its keys."""
+    rng = np.random.default_rng(5)
+    E = 200_000
+    sizes = [100_000, 50_000, 100_000, 300, 524_288, 100_000]
+    L = capi.lib()
+    nbytes = max(L.ts_scatter_workspace_bytes(capi._i(1), capi._i(E), capi._i(1), capi._i(N), capi.DTYPE[torch.float32],
+                                              capi.REDUCE[reduce]) for N in sizes)
+    zeros = {L.ts_scatter_workspace_zero_bytes(capi._i(1), capi._i(E), capi._i(1), capi._i(N), capi.DTYPE[torch.float32],
+                                               capi.REDUCE[reduce]) for N in sizes}
+    assert len(zeros) == 1 and min(zeros) >= max(sizes) * 8, zeros
+    nzero = zeros.pop()
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=DEV)
+    ws[nzero:] = 0xA5          # whatever earlier calls may have left behind the key table
+    ws[:nzero].zero_()
+    for step, N in enumerate(sizes):
+        src = torch.from_numpy(rng.integers(-50, 51, size=(1, E, 1)).astype(np.float32))
+        index = torch.from_numpy(rng.integers(0, N, size=E).astype(np.int64))
+        want, want_arg = oracle.scatter(src, index.view(1, -1, 1), 1, None, N, reduce)
+        out = torch.empty((1, N, 1), dtype=torch.float32, device=DEV)
+        arg = torch.empty((1, N, 1), dtype=torch.long, device=DEV)
+        ws2 = capi.scatter_with_workspace(src.to(DEV), index.to(DEV), out, arg, 1, E, 1, N, 0, 1, 0,
+                                          capi.REDUCE[reduce], False, ws)
+        assert ws2.data_ptr() == ws.data_ptr()
+        torch.cuda.synchronize()
+        assert_exact(out, want, f"values step={step} N={N}")
+        assert_exact(arg, want_arg, f"arg step={step} N={N}")
+        assert bool((ws[:nzero] == 0).all()), "the key table is handed back as zeros"

@@ -619,3 +619,19 @@ def test_scatter_mean_with_one_index_row_for_every_batch_row(ts, dtype):
         (gx,) = torch.autograd.grad(y, x, torch.ones_like(y))
         count = torch.bincount(row, minlength=N).clamp(min=1).float()
         assert torch.allclose(gx.cpu(), (1.0 / count)[row].view(1, E).expand(B, E))
+
+
+@pytest.mark.parametrize("reduce", ["min", "max"])
+def test_scatter_of_single_values_with_a_changing_number_of_output_rows(ts, oracle, reduce):
+    """Mini-batches with a varying node count on one stream: the operator keeps one workspace per stream for
+    min / max of one 4-byte value per entry, and what a call with few output rows leaves behind its key table
+    must not be read as keys by a later call with more output rows."""
+    rng = np.random.default_rng(11)
+    E = 300_000
+    for step, N in enumerate([100_000, 50_000, 100_000, 7, 524_288, 50_001, 100_000]):
+        src = torch.from_numpy(rng.integers(-50, 51, size=E).astype(np.float32))
+        index = torch.from_numpy(rng.integers(0, N, size=E).astype(np.int64))
+        got, arg = getattr(ts, "scatter_" + reduce)(src.to(DEV), index.to(DEV), 0, None, N)
+        want, want_arg = oracle.scatter(src, index, 0, None, N, reduce)
+        assert torch.equal(got.cpu(), want), f"values step={step} N={N}"
+        assert torch.equal(arg.cpu(), want_arg), f"arg step={step} N={N}"
