@@ -3,21 +3,30 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--configs C1,C2,...]
 
-Headline (`value`): configuration C2 of BASELINE.json -- segment_csr sum,
-segment_csr mean and gather_csr of the result back to the edges, 100000
-segments with Zipf(2.0) degrees, fp32 [E, 64] -- as effective HBM GB/s:
-algorithmic bytes (every input and output tensor counted once) divided by the
-wall time of K steps, inputs resident in HBM, called through the registered
-operators (torch.ops.torch_scatter.*). One step = the three ops once.
+Headline (`value`): configuration C5 of BASELINE.json, the largest one and the
+only one whose tensors do not fit the 256 MB memory-side cache -- N = 2.4 M
+nodes, E = 62.4 M edges (out-degree Zipf(1.8), mean 26), bf16 features
+[., 128]. One step = gather_csr (node -> edge) + segment_csr mean (edge ->
+node) + the backward of that mean, through the registered operators
+(torch.ops.torch_scatter.*; the backward through autograd). Reported as
+effective HBM GB/s: algorithmic bytes (every input and output tensor counted
+once, 3 x 16.6 GB) divided by the wall time of K steps, inputs resident in HBM.
 
 The same JSON line carries
-  roofline      the dominant kernel of the headline (the CSR reduction), timed
-                with HIP events on the launch stream, against the 8 TB/s peak;
+  roofline      the dominant kernel of the step (the CSR reduction of the mean,
+                ts::csr_reduce_kernel<bf16, 8, MEAN>), timed with HIP events on
+                the launch stream, against the 8 TB/s peak; `traffic` = HBM bytes
+                per launch from the tracked counter profile;
   cpu_baseline  the reference's CPU kernels (oracle/_ref, else the C oracle)
-                timed on the host for the same workload, one thread;
+                timed on the host on a 1/4-scale slice of the same workload,
+                one thread;
   configs       effective GB/s of every op of configurations C1..C5, timed the
-                same way (events around back-to-back launches); the X-* rows are
-                extra shapes (sorted index given to scatter, one value per entry).
+                same way (events around back-to-back launches; inputs under
+                256 MB also cold, with 1 GiB written between launches); the X-*
+                rows are extra shapes (sorted index given to scatter, one value
+                per entry, fused composites).
+
+Hardware probes and dispatcher sweeps: python3 -m benchmark.hw_probes.
 """
 import argparse
 import json
@@ -36,28 +45,12 @@ PEAK_GBS = 8000.0  # MI355X HBM3E
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--configs", default="C1,C2,C2m,C3,C4,C5,X",
-                    help="comma list of side configurations to time (C2 is always run)")
+                    help="comma list of side configurations to time (the C5 headline is always run)")
     ap.add_argument("--iters", type=int, default=20, help="launches per op in the per-config table")
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
-    ap.add_argument("--probe-scatter", action="store_true",
-                    help="launch sequence for the L2 / atomic counters of the scatter kernels (see probe_scatter)")
-    ap.add_argument("--probe-ceilings", action="store_true",
-                    help="plain read / write / copy / mixed streams over several GiB: what the memory system of this "
-                         "device sustains (the ceilings the kernels are held against), nothing else is run")
-    ap.add_argument("--probe-atomics", action="store_true",
-                    help="rate of device-scope 64-bit atomics on scattered and on neighbouring addresses")
-    ap.add_argument("--sweep-thresholds", action="store_true",
-                    help="time scatter sum / max just either side of every size threshold of the dispatcher and "
-                         "flag neighbours that differ by more than 1.5x")
-    ap.add_argument("--sweep-orders", action="store_true",
-                    help="scatter sum / max for one shape under a sorted, a shuffled and a skewed index, fp32 and bf16; "
-                         "flags a sorted index that is slower than a shuffled one and 16-bit types far behind fp32")
-    ap.add_argument("--probe", action="store_true",
-                    help="counter-collection mode for rocprofv3 --pmc: a few launches of the dominant kernels "
-                         "next to copies of known size, nothing timed")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
     return ap.parse_args()
 
 
@@ -310,65 +303,75 @@ def bench_softmax_config(ts, wl, w, dev, iters, K):
     return res
 
 
-def cpu_baseline(wl, w):
-    """The same three ops of C2 on the host, single thread: the reference's own
-    CPU kernels when oracle/_ref is built, else the C restatement."""
+def load_ref_ops():
+    """The reference's own CPU kernels (oracle/_ref) as torch.ops.ts_ref, or None when they are not built."""
+    import torch
+    ref_path = os.path.join(ROOT, "oracle", "_ref", "libts_ref_cpu.so")
+    if not os.path.exists(ref_path):
+        return None
+    try:
+        torch.ops.load_library(ref_path)
+        return torch.ops.ts_ref
+    except Exception:  # built against another torch: the C restatement serves instead
+        return None
+
+
+def cpu_baseline(wl, scale=1.0 / 4):
+    """The three ops of the C5 step on the host, single thread, on a slice of the workload (the same
+    generator with N scaled down: same degree distribution, same cap rule, bf16): the reference's own CPU kernels
+    when oracle/_ref is built, else the C restatement. The backward follows csrc/segment_csr.cpp:93-109: gather
+    of the gradient, gather of the counts, one division."""
     import torch
     torch.set_num_threads(1)
+    w = wl.c5_gnn(scale)
     g = torch.Generator().manual_seed(0)
-    src = torch.randn((w.E, w.K), generator=g, dtype=torch.float32)
-    out = torch.empty((w.N, w.K), dtype=torch.float32)
-    back = torch.empty_like(src)
-    kind = "port"
-    ref_path = os.path.join(ROOT, "oracle", "_ref", "libts_ref_cpu.so")
-    run = None
-    if os.path.exists(ref_path):
-        try:
-            torch.ops.load_library(ref_path)
-            ops = torch.ops.ts_ref
-
-            def run():
-                ops.segment_csr(src, w.indptr, out, "sum")
-                ops.segment_csr(src, w.indptr, out, "mean")
-                ops.gather_csr(out, w.indptr, back)
-            run()
-            kind = "reference"
-        except Exception:  # library built against another torch: fall back to the port
-            run = None
-    if run is None:
+    x = torch.randn((w.N, w.K), generator=g).to(w.dtype)
+    src = torch.empty((w.E, w.K), dtype=w.dtype)
+    for s0 in range(0, w.E, 1 << 20):
+        src[s0:s0 + (1 << 20)] = torch.randn((min(1 << 20, w.E - s0), w.K), generator=g).to(w.dtype)
+    grad = torch.randn((w.N, w.K), generator=g).to(w.dtype)
+    out = torch.empty((w.N, w.K), dtype=w.dtype)
+    msg = torch.empty_like(src)
+    count = (w.indptr[1:] - w.indptr[:-1]).to(w.dtype)
+    ops = load_ref_ops()
+    kind = "reference" if ops is not None else "port"
+    if ops is not None:
+        def run():
+            ops.gather_csr(x, w.indptr, msg)
+            ops.segment_csr(src, w.indptr, out, "mean")
+            ops.gather_csr(grad, w.indptr, msg)
+            msg.true_divide_(ops.gather_csr(count, w.indptr, None).unsqueeze(-1))
+    else:
         import ts_oracle
 
         def run():
-            ts_oracle.segment_csr(src, w.indptr, out, "sum")
+            ts_oracle.gather_csr(x, w.indptr, msg)
             ts_oracle.segment_csr(src, w.indptr, out, "mean")
-            ts_oracle.gather_csr(out, w.indptr, back)
-        run()
-    reps = 5
+            ts_oracle.gather_csr(grad, w.indptr, msg)
+            msg.true_divide_(ts_oracle.gather_csr(count, w.indptr, None).unsqueeze(-1))
+    run()
+    reps = 4
     t0 = time.perf_counter()
     for _ in range(reps):
         run()
     dt = (time.perf_counter() - t0) / reps
-    nbytes = 2 * wl.bytes_segment(w.E, w.N, w.K, 4) + wl.bytes_gather(w.E, w.N, w.K, 4)
+    s = 2
+    nbytes = 2 * wl.bytes_gather(w.E, w.N, w.K, s) + wl.bytes_segment(w.E, w.N, w.K, s)
     return {"value": round(gbs(nbytes, dt), 3), "unit": "GB/s", "cores": 1, "kind": kind,
             "host_cores_available": os.cpu_count(),
-            "sample": f"full C2 workload (E={w.E}, N={w.N}, K={w.K}, fp32), {reps} passes of "
-                      f"segment_csr sum + mean + gather_csr, {dt * 1e3:.1f} ms per pass"}
+            "sample": f"1/{round(1 / scale)} slice of C5 (N={w.N}, E={w.E}, K={w.K}, bf16: the same generator with "
+                      f"the node count scaled), {reps} passes of gather_csr + segment_csr mean + mean backward "
+                      f"(gather, gather of counts, divide), {dt * 1e3:.0f} ms per pass"}
 
 
 def cpu_baselines_other(wl):
-    """The reference's CPU kernels (oracle/_ref, else the C oracle) on the scatter / segment_coo configurations, one
-    thread: C1 in full (the configuration BASELINE.json names "on CPU reference"), C4 with one value per entry
-    in full, C3 on a slice of 1/16 of its segments (the full input is 4.6 GB)."""
+    """The reference's CPU kernels (oracle/_ref, else the C oracle) on the other configurations, one thread: C1 in
+    full (the configuration BASELINE.json names "on CPU reference"), C2 in full, C4 with one value per entry in
+    full, C3 on a slice of 1/16 of its segments (the full input is 4.6 GB)."""
     import torch
     torch.set_num_threads(1)
-    ref_path = os.path.join(ROOT, "oracle", "_ref", "libts_ref_cpu.so")
-    ops, kind = None, "port"
-    if os.path.exists(ref_path):
-        try:
-            torch.ops.load_library(ref_path)
-            ops, kind = torch.ops.ts_ref, "reference"
-        except Exception:
-            ops = None
+    ops = load_ref_ops()
+    kind = "reference" if ops is not None else "port"
     import ts_oracle
 
     def scatter(src, index, N, reduce):
@@ -404,6 +407,19 @@ def cpu_baselines_other(wl):
                     "kind": kind, "host_cores_available": os.cpu_count(),
                     "sample": f"full C4 with one value per entry (scatter max + arg, E={w4.E}, N={w4.N}), 3 passes, "
                               f"{dt * 1e3:.1f} ms per pass"}
+    w2 = wl.c2_segment_csr()
+    src = torch.randn((w2.E, w2.K), generator=g)
+    o2, b2 = torch.empty((w2.N, w2.K)), torch.empty((w2.E, w2.K))
+
+    def c2_step():
+        for r in ("sum", "mean"):
+            (ops.segment_csr if ops is not None else ts_oracle.segment_csr)(src, w2.indptr, o2, r)
+        (ops.gather_csr if ops is not None else ts_oracle.gather_csr)(o2, w2.indptr, b2)
+    dt = timed(c2_step, 5)
+    out["C2"] = {"value": round(gbs(2 * wl.bytes_segment(w2.E, w2.N, w2.K, 4) + wl.bytes_gather(w2.E, w2.N, w2.K, 4), dt), 3),
+                 "unit": "GB/s", "cores": 1, "kind": kind, "host_cores_available": os.cpu_count(),
+                 "sample": f"full C2 (segment_csr sum + mean + gather_csr, E={w2.E}, N={w2.N}, K={w2.K}, fp32), 5 passes, "
+                           f"{dt * 1e3:.1f} ms per pass"}
     w3 = wl.c3_segment_coo(scale=1.0 / 16)
     src = torch.rand((w3.E, w3.K), generator=g) * 2 - 1
     dt = timed(lambda: segment_coo(src, w3.index, w3.N, "max"), 3)
@@ -414,264 +430,20 @@ def cpu_baselines_other(wl):
     return out
 
 
-def measured_traffic():
-    """HBM bytes per launch of the headline kernel as the tracked counter profile states them (a line
-    `traffic_bytes_per_launch: <number>` in profiles/csr_reduce_pmc_traffic.txt), or None."""
+def measured_traffic(key):
+    """HBM bytes per launch of a kernel as the tracked counter profile states them (a line
+    `<key>: <number>` in profiles/csr_reduce_pmc_traffic.txt), or None."""
     import re
     try:
         text = open(os.path.join(ROOT, "profiles", "csr_reduce_pmc_traffic.txt")).read()
     except OSError:
         return None
-    m = re.search(r"traffic_bytes_per_launch:\s*([0-9.eE+]+)", text)
+    m = re.search(r"^" + re.escape(key) + r":\s*([0-9.eE+]+)", text, re.M)
     return float(m.group(1)) if m else None
-
-
-def probe_ceilings():
-    """Plain streams through libts_probe.so (pytorch_scatter_amd/csrc/probe.hip): read, write, copy and reads mixed
-    with writes 3:1 and 26:1, over GiB-sized buffers, HIP events around 10 launches each."""
-    import ctypes
-    import torch
-    lib = ctypes.CDLL(os.path.join(ROOT, "pytorch_scatter_amd", "libts_probe.so"))
-    lib.ts_probe_stream.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
-    dev = torch.device("cuda:0")
-    a = torch.empty(6 << 30, dtype=torch.uint8, device=dev)
-    b = torch.empty(4 << 30, dtype=torch.uint8, device=dev)
-    a.fill_(1)
-    b.fill_(2)
-    stream = torch.cuda.current_stream().cuda_stream
-    rows = []
-    for name, mode, wbytes in (("read only (non-temporal 16-byte loads)", 0, 4 << 30), ("write only", 1, 4 << 30),
-                               ("copy 1:1", 2, 3 << 30), ("read 3 : write 1", 4, 2 << 30),
-                               ("read 26 : write 1", 27, 224 << 20)):
-        rd = 0 if mode == 1 else (wbytes if mode == 0 else (mode - 1) * wbytes)
-        wr = 0 if mode == 0 else wbytes
-        t = event_time(lambda: lib.ts_probe_stream(mode, a.data_ptr(), b.data_ptr(), wbytes, stream), 10, warm=2)
-        rows.append({"stream": name, "read_GB": round(rd / 1e9, 2), "written_GB": round(wr / 1e9, 2),
-                     "us": round(t * 1e6, 1), "GBps": round((rd + wr) / t / 1e9, 1),
-                     "pct_of_peak": round(100 * (rd + wr) / t / 1e9 / PEAK_GBS, 1)})
-    t = event_time(lambda: b[:3 << 30].copy_(a[:3 << 30]), 10, warm=2)
-    rows.append({"stream": "torch copy_ 1:1", "read_GB": 3.22, "written_GB": 3.22, "us": round(t * 1e6, 1),
-                 "GBps": round(2 * (3 << 30) / t / 1e9, 1), "pct_of_peak": round(100 * 2 * (3 << 30) / t / 1e9 / PEAK_GBS, 1)})
-    for r in rows:
-        print(f"{r['stream']:42s} read {r['read_GB']:6.2f} GB  written {r['written_GB']:6.2f} GB  {r['us']:9.1f} us  "
-              f"{r['GBps']:7.1f} GB/s  {r['pct_of_peak']:5.1f} % of 8 TB/s", file=sys.stderr)
-    print(json.dumps({"probe": "ceilings", "rows": rows}))
-
-
-def probe_atomics():
-    """Rate of device-scope 64-bit atomics (libts_probe.so): scattered addresses (one transaction per lane) and
-    neighbouring addresses shared by all workgroups (a table written back by every workgroup at once)."""
-    import ctypes
-    import torch
-    lib = ctypes.CDLL(os.path.join(ROOT, "pytorch_scatter_amd", "libts_probe.so"))
-    lib.ts_probe_atomics.restype = ctypes.c_longlong
-    lib.ts_probe_atomics.argtypes = [ctypes.c_void_p, ctypes.c_uint, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
-    dev = torch.device("cuda:0")
-    table = torch.zeros(1 << 20, dtype=torch.int64, device=dev)
-    stream = torch.cuda.current_stream().cuda_stream
-    rows = []
-    for name, slots, iters, pattern in (("scattered, 100 k slots, 1 M atomics", 100_000, 4, 0),
-                                        ("scattered, 100 k slots, 4 M atomics", 100_000, 16, 0),
-                                        ("scattered, 1 M slots, 4 M atomics", 1_000_000, 16, 0),
-                                        ("4096 neighbouring slots from each of 256 workgroups", 4096, 1, 1),
-                                        ("8192 neighbouring slots from each of 256 workgroups", 8192, 1, 1)):
-        n = lib.ts_probe_atomics(table.data_ptr(), slots, iters, pattern, stream)
-        t = event_time(lambda: lib.ts_probe_atomics(table.data_ptr(), slots, iters, pattern, stream), 10, warm=2)
-        rows.append({"pattern": name, "atomics": n, "us": round(t * 1e6, 1), "G_atomics_per_s": round(n / t / 1e9, 1)})
-    for r in rows:
-        print(f"{r['pattern']:56s} {r['atomics']:9d} atomics {r['us']:8.1f} us {r['G_atomics_per_s']:7.1f} G/s", file=sys.stderr)
-    print(json.dumps({"probe": "atomics", "rows": rows}))
-
-
-def sweep_thresholds():
-    """scatter sum / max through the operators at sizes just either side of every size threshold of the dispatcher
-    (pytorch_scatter_amd/csrc/scatter.h, scatter_binned.h, scatter_k1.h): neighbours that differ by more than 1.5x in time
-    per entry are flagged. Index: Zipf(1.2) over N rows, shuffled."""
-    import numpy as np
-    import torch
-    import pytorch_scatter_amd as ts
-    dev = torch.device("cuda:0")
-    rng = np.random.default_rng(0)
-
-    def zipf_index(E, N):
-        p = np.arange(1, N + 1, dtype=np.float64) ** -1.2
-        return torch.from_numpy(rng.choice(N, size=E, p=p / p.sum()).astype(np.int64)).to(dev)
-
-    # (what, K, N, sizes in entries around the threshold); N a list: 2 M entries, output rows around the threshold
-    M = 1 << 20
-    cases = [
-        ("sum: LDS table from 2^16 elements (K = 16)", "sum", 16, 1000, [M // 256 - 512, M // 256 + 512]),
-        ("sum: LDS table from 2^18 elements for rows of 33-64 columns (K = 64)", "sum", 64, 100_000,
-         [M // 256 - 256, M // 256 + 256]),
-        ("sum: LDS table from 2^19 elements for rows above 64 columns (K = 128)", "sum", 128, 100_000,
-         [M // 256 - 256, M // 256 + 256]),
-        ("sum: sample of the index from 2^23 elements (K = 8)", "sum", 8, 1_000_000, [M - 65536, M + 65536]),
-        ("sum: buckets of output rows from 64 MB (K = 32)", "sum", 32, 100_000, [M // 2 - 16384, M // 2 + 16384]),
-        ("max: LDS table from 2^20 elements (contended index)", "max", 8, 1000, [M // 8 - 4096, M // 8 + 4096]),
-        ("max: one value per entry, slabs from 2^14 entries", "max", 1, 100_000, [M // 64 - 1024, M // 64 + 1024]),
-        ("max: buckets of output rows from 24 MB (K = 32, keys of 25 MB)", "max", 32, 100_000,
-         [3 * M // 16 - 8192, 3 * M // 16 + 8192]),
-        ("max: buckets of output rows from 64 MB (K = 32, keys of 2.5 MB)", "max", 32, 10_000,
-         [M // 2 - 16384, M // 2 + 16384]),
-        ("max: parts of 4 / 8 / 16 entries by the number of wavefronts (K = 32)", "max", 32, 100_000,
-         [M // 8 - 8192, M // 8 + 8192]),
-        ("max: sample of the index from 2^23 elements (K = 8)", "max", 8, 1_000_000, [M - 65536, M + 65536]),
-        ("sum: rows in slices of columns above 16384 buckets (K = 128)", "sum", 128, [M - 8192, M + 8192], None),
-        ("max: rows in slices of columns above 16384 buckets (K = 128)", "max", 128, [M - 8192, M + 8192], None),
-    ]
-    rows, flagged = [], 0
-    with torch.no_grad():
-        for what, reduce, K, N, sizes in cases:
-            per_entry = []
-            points = [(E, N) for E in sizes] if sizes is not None else [(2 * M, n) for n in N]
-            for E, N in points:
-                index = zipf_index(E, N)
-                src = torch.randn((E, K), device=dev)
-                fn = ts.scatter_sum if reduce == "sum" else ts.scatter_max
-                t = event_time(lambda: fn(src, index, 0, None, N), 10)
-                per_entry.append(t / E)
-                rows.append({"threshold": what, "E": E, "K": K, "N": N, "us": round(t * 1e6, 1),
-                             "ns_per_entry": round(t / E * 1e9, 4)})
-                del src, index
-            ratio = max(per_entry) / min(per_entry)
-            rows[-1]["ratio_across_threshold"] = round(ratio, 2)
-            rows[-1]["cliff"] = ratio > 1.5
-            flagged += ratio > 1.5
-    for r in rows:
-        print(r, file=sys.stderr)
-    print(json.dumps({"probe": "thresholds", "cliffs": flagged, "rows": rows}))
-
-
-def sweep_orders():
-    """scatter sum / max through the operators for the same shape under a sorted, a shuffled and a Zipf(1.2) index,
-    fp32 and bf16: the thresholds of the dispatcher are sizes, and a kernel picked by size can be the wrong one for
-    the order of the index or for the element type (found that way: the accumulator table for narrow rows was
-    twice as slow as the run kernel under a sorted index, and 30-300x slower for 16-bit floats under any other).
-    Flags: a sorted index more than 1.5x slower than the same index shuffled; bf16 more than 8x slower than fp32."""
-    import numpy as np
-    import torch
-    import pytorch_scatter_amd as ts
-    dev = torch.device("cuda:0")
-    rng = np.random.default_rng(0)
-    rows, flagged = [], 0
-    with torch.no_grad():
-        for E, N in ((4_000_000, 400_000), (4_000_000, 4_000), (500_000, 50_000)):
-            uni = rng.integers(0, N, size=E)
-            p = np.arange(1, N + 1, dtype=np.float64) ** -1.2
-            zipf = rng.choice(N, size=E, p=p / p.sum())
-            orders = {"sorted": np.sort(uni), "shuffled": uni, "zipf": zipf}
-            index = {k: torch.from_numpy(v.astype(np.int64)).to(dev) for k, v in orders.items()}
-            for K in (1, 8, 32):
-                t = {}
-                for dtype in (torch.float32, torch.bfloat16):
-                    src = torch.randn((E, K), device=dev).to(dtype)
-                    for order, idx in index.items():
-                        for reduce, fn in (("sum", ts.scatter_sum), ("max", ts.scatter_max)):
-                            t[dtype, order, reduce] = event_time(lambda: fn(src, idx, 0, None, N), 5)
-                    del src
-                for (dtype, order, reduce), v in t.items():
-                    slow_sorted = order == "sorted" and v > 1.5 * t[dtype, "shuffled", reduce]
-                    slow_16 = dtype == torch.bfloat16 and v > 8 * t[torch.float32, order, reduce]
-                    rows.append({"E": E, "N": N, "K": K, "dtype": str(dtype)[6:], "order": order, "reduce": reduce,
-                                 "us": round(v * 1e6, 1), "flag": bool(slow_sorted or slow_16)})
-                    flagged += bool(slow_sorted or slow_16)
-    for r in rows:
-        print(r, file=sys.stderr)
-    print(json.dumps({"probe": "orders", "flagged": flagged, "rows": rows}))
-
-
-def probe():
-    """Launch sequence for `rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE -- python3 bench.py --probe`:
-    1. torch copy of 1 GiB (plain loads/stores, known size: calibrates the counters);
-    2. segment_csr sum with one entry per segment over 1 GiB of fp32 [4Mi, 64]: a copy through the
-       reduction kernel itself (same non-temporal loads), known size;
-    3. C2 segment_csr sum x3, C5 segment_csr mean x2, C5 gather_csr x2."""
-    import torch
-    import pytorch_scatter_amd as ts
-    from pytorch_scatter_amd import workloads as wl
-    dev = torch.device("cuda:0")
-    a = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
-    b = torch.empty_like(a)
-    b.copy_(a)
-    n = 1 << 22
-    x = torch.ones((n, 64), dtype=torch.float32, device=dev)
-    ident = torch.arange(n + 1, device=dev)
-    y = torch.empty_like(x)
-    with torch.no_grad():
-        ts.segment_csr(x, ident, y, "sum")
-        del a, b, x, y
-        w2 = wl.c2_segment_csr()
-        src = wl.edge_values(w2, dev)
-        out = torch.empty((w2.N, w2.K), dtype=torch.float32, device=dev)
-        for _ in range(3):
-            ts.segment_csr(src, w2.indptr.to(dev), out, "sum")
-        del src, out
-        w5 = wl.c5_gnn()
-        src = wl.edge_values(w5, dev)
-        out = torch.empty((w5.N, w5.K), dtype=torch.bfloat16, device=dev)
-        ip = w5.indptr.to(dev)
-        for _ in range(2):
-            ts.segment_csr(src, ip, out, "mean")
-        for _ in range(2):
-            ts.gather_csr(out, ip, src)
-    torch.cuda.synchronize()
-    print(json.dumps({"probe": "done", "copy_bytes": 1 << 30, "identity_rows": n, "C2": [w2.N, w2.E, w2.K],
-                      "C5": [w5.N, w5.E, w5.K]}))
-
-
-def probe_scatter():
-    """Launch sequence for `rocprofv3 --pmc TCC_HIT_sum TCC_MISS_sum TCC_ATOMIC_sum -- python3 bench.py
-    --probe-scatter`: C1 scatter sum x3, C4 scatter max with K = 1 and K = 32 x2 each (K = 32 also as a sum and
-    through an index sorted once, x2 each), scatter sum and max over the sorted index of C3 with K = 64 x2 each."""
-    import torch
-    import pytorch_scatter_amd as ts
-    from pytorch_scatter_amd import workloads as wl
-    dev = torch.device("cuda:0")
-    done = {}
-    with torch.no_grad():
-        w1 = wl.c1_scatter_sum()
-        src, index = wl.scatter_values(w1, dev), w1.index.to(dev)
-        for _ in range(3):
-            ts.scatter_sum(src, index, 0, None, w1.N)
-        done["C1"] = [w1.N, w1.E, w1.K]
-        for K in (1, 32):
-            w4 = wl.c4_scatter_minmax(K)
-            src, index = wl.scatter_values(w4, dev), w4.index.to(dev)
-            for _ in range(2):
-                ts.scatter_max(src, index, 0, None, w4.N)
-            done[f"C4-K{K}"] = [w4.N, w4.E, w4.K]
-            if K == 32:  # the same scatter as a sum, and through an index sorted once
-                for _ in range(2):
-                    ts.scatter_sum(src, index, 0, None, w4.N)
-                plan = ts.SortedIndex(index, w4.N)
-                for _ in range(2):
-                    ts.scatter_sorted(src, plan, 0, "max")
-        w3 = wl.c3_segment_coo()
-        index = w3.index.to(dev)
-        src = torch.randn((w3.E, 64), device=dev)
-        for _ in range(2):
-            ts.scatter_sum(src, index, 0, None, w3.N)
-        for _ in range(2):
-            ts.scatter_max(src, index, 0, None, w3.N)
-        done["X-sorted-K64"] = [w3.N, w3.E, 64]
-    torch.cuda.synchronize()
-    print(json.dumps({"probe": "scatter done", **done}))
 
 
 def main():
     args = parse_args()
-    if args.probe_ceilings:
-        return probe_ceilings()
-    if args.probe_atomics:
-        return probe_atomics()
-    if args.sweep_thresholds:
-        return sweep_thresholds()
-    if args.sweep_orders:
-        return sweep_orders()
-    if args.probe:
-        return probe()
-    if args.probe_scatter:
-        return probe_scatter()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU; every box of this run has a single MI355X, "
               "so --gpus above 1 is not supported (segment / gather ops would shard by node range "
@@ -684,40 +456,49 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
 
-    # ---------------- headline: C2 through the registered operators
-    w2 = wl.c2_segment_csr()
-    src = wl.edge_values(w2, dev)
-    indptr = w2.indptr.to(dev)
-    out = torch.empty((w2.N, w2.K), dtype=torch.float32, device=dev)
-    back = torch.empty_like(src)
-    step_bytes = 2 * wl.bytes_segment(w2.E, w2.N, w2.K, 4) + wl.bytes_gather(w2.E, w2.N, w2.K, 4)
+    # ---------------- headline: C5 through the registered operators (HBM-resident: 16.6 GB per op)
+    w5 = wl.c5_gnn()
+    indptr = w5.indptr.to(dev)
+    g = torch.Generator(device=dev).manual_seed(1)
+    x = torch.randn((w5.N, w5.K), generator=g, device=dev).to(w5.dtype)          # node features
+    grad_out = torch.randn((w5.N, w5.K), generator=g, device=dev).to(w5.dtype)   # gradient of the mean
+    src = wl.edge_values(w5, dev).requires_grad_(True)                           # edge features
+    msg = torch.empty((w5.E, w5.K), dtype=w5.dtype, device=dev)                  # node -> edge messages
+    out = torch.empty((w5.N, w5.K), dtype=w5.dtype, device=dev)
+    op_bytes = {"gather_csr": wl.bytes_gather(w5.E, w5.N, w5.K, 2),
+                "segment_csr_mean": wl.bytes_segment(w5.E, w5.N, w5.K, 2),
+                "segment_csr_mean_backward": wl.bytes_gather(w5.E, w5.N, w5.K, 2)}
+    step_bytes = sum(op_bytes.values())
 
     def step():
-        ts.segment_csr(src, indptr, out, "sum")
-        ts.segment_csr(src, indptr, out, "mean")
-        ts.gather_csr(out, indptr, back)
+        with torch.no_grad():
+            ts.gather_csr(x, indptr, msg)
+        y = ts.segment_csr(src, indptr, None, "mean")
+        (gin,) = torch.autograd.grad(y, src, grad_out)   # the fused gather-and-divide kernel, 16 GB written
+        return gin
 
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / args.steps
+    # dominant kernel: the CSR reduction of the mean (one launch per call), HIP events on the launch stream
     with torch.no_grad():
-        for _ in range(args.warmup):
-            step()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(args.steps):
-            step()
-        torch.cuda.synchronize()
-        dt = (time.perf_counter() - t0) / args.steps
-        # dominant kernel: the CSR reduction (segment_csr sum), HIP events on the launch stream
-        t_kernel = event_time(lambda: ts.segment_csr(src, indptr, out, "sum"), max(args.steps, 20))
-    kernel_bytes = wl.bytes_segment(w2.E, w2.N, w2.K, 4)
-    # HBM bytes per launch of this kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, calibrated against
-    # copies of known size: read from the tracked profile, null if that file does not state it
-    traffic = measured_traffic()
-    roofline = {"bound": "hbm", "kernel": "ts::csr_reduce_kernel<float, 4, SUM>",
+        t_kernel = event_time(lambda: ts.segment_csr(src, indptr, out, "mean"), max(args.steps, 10))
+    kernel_bytes = op_bytes["segment_csr_mean"]
+    # HBM bytes per launch of this kernel from rocprofv3 --pmc (memory-side read / write requests by size):
+    # read from the tracked profile, null if that file does not state it
+    traffic = measured_traffic("traffic_bytes_per_launch_c5_mean")
+    roofline = {"bound": "hbm", "kernel": "ts::csr_reduce_kernel<bf16, 8, MEAN> (segment_csr mean of C5)",
                 "achieved": round(gbs(kernel_bytes, t_kernel), 1), "peak": PEAK_GBS, "unit": "GB/s",
                 "frac": round(gbs(kernel_bytes, t_kernel) / PEAK_GBS, 4), "traffic": traffic,
-                "algorithmic_bytes_per_launch": kernel_bytes, "us_per_launch": round(t_kernel * 1e6, 2)}
-    del src, back, out
+                "algorithmic_bytes_per_launch": kernel_bytes, "us_per_launch": round(t_kernel * 1e6, 1)}
+    del src, msg, out, x, grad_out
     torch.cuda.empty_cache()
+    w2 = wl.c2_segment_csr()
 
     # ---------------- side table: every configuration
     want = set(args.configs.split(",")) if args.configs else set()
@@ -772,22 +553,24 @@ def main():
                                                 ["segment_csr_sum", "segment_csr_max", "segment_coo_sum",
                                                  "gather_csr", "gather_coo"], uniform=True)
 
-    cpu = None if args.no_cpu else cpu_baseline(wl, w2)
+    cpu = None if args.no_cpu else cpu_baseline(wl)
     cpu_other = None if args.no_cpu else cpu_baselines_other(wl)
 
     line = {
-        "metric": "effective HBM GB/s, segment_csr sum + mean + gather_csr (BASELINE config C2), 1 MI355X",
+        "metric": "effective HBM GB/s, gather_csr + segment_csr mean + mean backward (BASELINE config C5), 1 MI355X",
         "value": round(gbs(step_bytes, dt), 1),
         "unit": "GB/s",
         "pct_of_8TBps_peak": round(100 * gbs(step_bytes, dt) / PEAK_GBS, 1),
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(dt * 1e3, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "C2: segment_csr sum+mean, gather_csr; 100000 segments, degrees "
-                               "clip(Zipf(2.0),1,512), src fp32 [E,64], numpy default_rng(0)",
-                   "N": w2.N, "E": w2.E, "K": w2.K, "algorithmic_bytes_per_step": step_bytes,
-                   "api": "torch.ops.torch_scatter.* (eager, out= preallocated)"},
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "C5: gather_csr (node->edge) + segment_csr mean (edge->node) + mean backward; "
+                               "N=2.4M nodes, out-degree Zipf(1.8) capped for mean 26, features bf16 [., 128], "
+                               "numpy default_rng(0)",
+                   "N": w5.N, "E": w5.E, "K": w5.K, "algorithmic_bytes_per_step": step_bytes,
+                   "algorithmic_bytes_per_op": op_bytes,
+                   "api": "torch.ops.torch_scatter.* (eager; backward through autograd)"},
         "roofline": roofline,
         "cpu_baseline": cpu,
         "cpu_baselines_other_configs": cpu_other,

@@ -34,6 +34,11 @@ constexpr int kMaxBlockItems = 2048;  // rows + edges per workgroup tile
 #ifndef TS_CSR_U
 #define TS_CSR_U 4
 #endif
+#ifndef TS_CSR_BLOCK
+#define TS_CSR_BLOCK 256
+#endif
+constexpr int kCsrBlock = TS_CSR_BLOCK;  // lanes per workgroup of csr_reduce_kernel
+constexpr int kCsrMaxItems = kMaxBlockItems * kCsrBlock / 256;  // rows + edges per tile of csr_reduce_kernel
 constexpr int kSharedWalkMin = 32;  // tiles a row must have passed through before the workgroup shares the walk
 constexpr int kLoadsInFlight = TS_CSR_U;  // U: 16-byte loads per lane per batch (two batches in flight)
 
@@ -202,18 +207,18 @@ template <typename T, int VEC, int REDUCE, int PERM = 0> constexpr int csr_reduc
   return PERM == 1 ? 1 : ((REDUCE == TS_SUM || REDUCE == TS_MEAN) && sizeof(T) >= 4 ? 6 : 1);  // PERM: 8 KB more LDS
 }
 template <typename T, int VEC, int REDUCE, int ACCUM, int PERM = 0>
-__global__ __launch_bounds__(kBlock, (csr_reduce_min_blocks<T, VEC, REDUCE, PERM>())) void csr_reduce_kernel(CsrReduceArgs a) {
+__global__ __launch_bounds__(kCsrBlock, (csr_reduce_min_blocks<T, VEC, REDUCE, PERM>())) void csr_reduce_kernel(CsrReduceArgs a) {
   typedef typename Acc<T>::type A;
   constexpr bool kArg = (REDUCE == TS_MIN || REDUCE == TS_MAX);
   constexpr int U = kLoadsInFlight;
 
-  __shared__ int32_t s_ptr[kMaxBlockItems + 4];  // row pointers of the tile + one sentinel
-  __shared__ int32_t s_perm[PERM == 1 ? kMaxBlockItems : 1];  // source rows of the tile's entries
-  __shared__ A s_val[2 * kBlock * VEC];
-  __shared__ int32_t s_arg[kArg ? 2 * kBlock * VEC : 1];
-  __shared__ int32_t s_head_row[kBlock];    // local row of the head partial, -1: none
-  __shared__ int32_t s_head_closes[kBlock];
-  __shared__ int32_t s_tail_row[kBlock];    // local row of the tail partial, -1: none
+  __shared__ int32_t s_ptr[kCsrMaxItems + 4];  // row pointers of the tile + one sentinel
+  __shared__ int32_t s_perm[PERM == 1 ? kCsrMaxItems : 1];  // source rows of the tile's entries
+  __shared__ A s_val[2 * kCsrBlock * VEC];
+  __shared__ int32_t s_arg[kArg ? 2 * kCsrBlock * VEC : 1];
+  __shared__ int32_t s_head_row[kCsrBlock];    // local row of the head partial, -1: none
+  __shared__ int32_t s_head_closes[kCsrBlock];
+  __shared__ int32_t s_tail_row[kCsrBlock];    // local row of the tail partial, -1: none
   __shared__ int64_t s_cut[2];
   if constexpr (PERM == 2) {
     if (a.gate != nullptr && (*a.gate != 0) != (a.gate_want != 0)) return;  // the same for every wavefront of the grid
@@ -221,7 +226,7 @@ __global__ __launch_bounds__(kBlock, (csr_reduce_min_blocks<T, VEC, REDUCE, PERM
 
   const int tid = threadIdx.x;
   const int G = a.G;
-  const int W = kBlock / G;
+  const int W = kCsrBlock / G;
   const int w = tid / G;
   const int lg = tid - w * G;
   const int CW = G * VEC;
@@ -240,9 +245,14 @@ __global__ __launch_bounds__(kBlock, (csr_reduce_min_blocks<T, VEC, REDUCE, PERM
   const int64_t d0 = (int64_t)blockIdx.x * a.BI;
   const int64_t d1 = d0 + a.BI < total ? d0 + a.BI : total;
   const int wave = tid / kWave;
-  if (wave < 2) {
-    const int64_t i = merge_search_wave(ptr, a.N, a.E, wave == 0 ? d0 : d1);
-    if ((tid & (kWave - 1)) == 0) s_cut[wave] = i;
+  if constexpr (kCsrBlock >= 2 * kWave) {
+    if (wave < 2) {
+      const int64_t i = merge_search_wave(ptr, a.N, a.E, wave == 0 ? d0 : d1);
+      if ((tid & (kWave - 1)) == 0) s_cut[wave] = i;
+    }
+  } else {
+    const int64_t ia = merge_search_wave(ptr, a.N, a.E, d0), ib = merge_search_wave(ptr, a.N, a.E, d1);
+    if (tid == 0) { s_cut[0] = ia; s_cut[1] = ib; }
   }
   if (a.status_reset && a.status != nullptr && tid == 0 && (blockIdx.x | blockIdx.y | blockIdx.z) == 0)
     __hip_atomic_exchange(a.status, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -255,13 +265,13 @@ __global__ __launch_bounds__(kBlock, (csr_reduce_min_blocks<T, VEC, REDUCE, PERM
   // ---- row pointers of the tile into LDS, relative to the tile's first edge
   const int64_t last = i1 + 1 < a.N ? i1 + 1 : a.N;
   const int nload = (int)(last - i0) + 1;  // ptr[i0 .. last]
-  for (int t = tid; t < nload; t += kBlock) s_ptr[t] = (int32_t)(ptr[i0 + t] - j0);
+  for (int t = tid; t < nload; t += kCsrBlock) s_ptr[t] = (int32_t)(ptr[i0 + t] - j0);
   if (tid == 0) { s_ptr[nload] = INT32_MAX; s_ptr[nload + 1] = INT32_MAX; }  // rows past the last one never end
   const int32_t *arg_perm = nullptr;  // set: positions leave the kernel in src's order
   if constexpr (PERM == 1) {
     const int32_t *perm_b = a.perm + b * a.perm_batch_stride;
     const int32_t last_row = a.E > 0 ? (int32_t)(a.E - 1) : 0;
-    for (int t = tid; t < ne; t += kBlock) {
+    for (int t = tid; t < ne; t += kCsrBlock) {
       const int32_t r = perm_b[j0 + t];
       s_perm[t] = r < 0 ? 0 : (r > last_row ? last_row : r);  // a malformed perm must not read outside src
     }
@@ -298,9 +308,9 @@ __global__ __launch_bounds__(kBlock, (csr_reduce_min_blocks<T, VEC, REDUCE, PERM
   const bool head_open = has_work && (i0 + ri0 < a.N) && (s_ptr[ri0] < je0);
 
   A *my_head_val = s_val + (size_t)w * CW + lg * VEC;
-  A *my_tail_val = s_val + (size_t)kBlock * VEC + (size_t)w * CW + lg * VEC;
+  A *my_tail_val = s_val + (size_t)kCsrBlock * VEC + (size_t)w * CW + lg * VEC;
   int32_t *my_head_arg = s_arg + (kArg ? (size_t)w * CW + lg * VEC : 0);
-  int32_t *my_tail_arg = s_arg + (kArg ? (size_t)kBlock * VEC + (size_t)w * CW + lg * VEC : 0);
+  int32_t *my_tail_arg = s_arg + (kArg ? (size_t)kCsrBlock * VEC + (size_t)w * CW + lg * VEC : 0);
 
   int r = ri0;
   T *op_row = out_b + (i0 + r) * a.K + (col_ok ? col : 0);
@@ -793,8 +803,8 @@ inline CsrPlan csr_plan(int64_t N, int64_t E, int64_t K, int elem_bytes, bool al
   p.G = G;
   p.ychunks = (int)((K + (int64_t)G * p.vec - 1) / ((int64_t)G * p.vec));
   const int64_t items = N + E;
-  const int W = kBlock / G;
-  const int cap = kMaxBlockItems / W;  // LDS holds the row pointers of one tile
+  const int W = (expand ? kBlock : kCsrBlock) / G;
+  const int cap = (expand ? kMaxBlockItems : kCsrMaxItems) / W;  // LDS holds the row pointers of one tile
   // Items per worker, from sweeps on 146 MB / 366 MB / 6 GB / 16 GB inputs (the curve is flat within 1-2 %
   // except for a few sharp optima): reductions 24 below 1 M items (more, shorter workgroups: the kernel is
   // latency bound there), 72 up to 32 M, 64 above; the write-bound expansion likes short ranges at every size
@@ -834,14 +844,14 @@ int launch_csr_reduce_t(const CsrReduceArgs &a, const CsrPlan &p, int64_t B, hip
   dim3 grid((unsigned)p.nblk, (unsigned)p.ychunks, (unsigned)B);
   if (a.perm != nullptr) {
     if (a.accumulate) return TS_ERR_UNSUPPORTED;
-    hipLaunchKernelGGL((csr_reduce_kernel<T, VEC, REDUCE, 0, 1>), grid, dim3(kBlock), 0, stream, a);
+    hipLaunchKernelGGL((csr_reduce_kernel<T, VEC, REDUCE, 0, 1>), grid, dim3(kCsrBlock), 0, stream, a);
   } else if (a.gate != nullptr || a.scatter_rule) {
     if (a.accumulate || !(a.lookback || p.nblk <= 1)) return TS_ERR_UNSUPPORTED;
-    hipLaunchKernelGGL((csr_reduce_kernel<T, VEC, REDUCE, 0, 2>), grid, dim3(kBlock), 0, stream, a);
+    hipLaunchKernelGGL((csr_reduce_kernel<T, VEC, REDUCE, 0, 2>), grid, dim3(kCsrBlock), 0, stream, a);
   } else if (a.accumulate)
-    hipLaunchKernelGGL((csr_reduce_kernel<T, VEC, REDUCE, -1>), grid, dim3(kBlock), 0, stream, a);
+    hipLaunchKernelGGL((csr_reduce_kernel<T, VEC, REDUCE, -1>), grid, dim3(kCsrBlock), 0, stream, a);
   else
-    hipLaunchKernelGGL((csr_reduce_kernel<T, VEC, REDUCE, 0>), grid, dim3(kBlock), 0, stream, a);
+    hipLaunchKernelGGL((csr_reduce_kernel<T, VEC, REDUCE, 0>), grid, dim3(kCsrBlock), 0, stream, a);
   if (p.nblk > 1 && !a.lookback) {  // a single tile has no rows that cross tiles
     const int W = kBlock / p.G;
     dim3 grid2((unsigned)((p.nblk + W - 1) / W), (unsigned)p.ychunks, (unsigned)B);
