@@ -226,15 +226,17 @@ int ts_scatter_with_workspace(const void *src, const int64_t *index, void *out,
                               int dtype, int reduce, int out_given, void *workspace,
                               size_t workspace_bytes, ts_stream_t stream);
 
-/* count[b, index[b*sb + e*se]] += 1 as float32, count pre-zeroed by the call.
- * The count half of ScatterMean::forward, csrc/scatter.cpp:131-137. */
-int ts_scatter_count(const int64_t *index, float *count, int64_t B, int64_t E,
+/* count[b, index[b*sb + e*se]] += 1 as int32 (exact for any group size below 2^31), count pre-zeroed by the
+ * call. The count half of ScatterMean::forward, csrc/scatter.cpp:131-137, which sums ones in the element
+ * type: equal wherever that sum is exact (any size for int32 / int64 / double), and exact beyond 2^24 entries
+ * per group in float and 2^8 / 2^11 in bf16 / half, where a running total of ones in the element type stalls. */
+int ts_scatter_count(const int64_t *index, int32_t *count, int64_t B, int64_t E,
                      int64_t N, int64_t index_stride_b, int64_t index_stride_e,
                      ts_stream_t stream);
 
 /* out[b, n, k] = out[b, n, k] / (T)max(count[b, n], 1): true division for
  * floating types, floor division for integers (csrc/scatter.cpp:138-141). */
-int ts_divide_by_count(void *out, const float *count, int64_t B, int64_t N,
+int ts_divide_by_count(void *out, const int32_t *count, int64_t B, int64_t N,
                        int64_t K, int dtype, ts_stream_t stream);
 
 /* Backward of every min/max flavour (csrc/scatter.cpp:184-196,
@@ -304,7 +306,7 @@ int ts_group_logsumexp_backward(const void *src, const int64_t *index,
 
 /* Standard deviation over the entries that share an index, one index per row, given the group sums
  * `total` ([B, N, K], element type: ts_scatter with SUM) and the entries per group `count` ([B, N]
- * float: ts_scatter_count):
+ * int32: ts_scatter_count):
  *   mean = total / max(count, 1);  out = sqrt(sum_group (src - mean)^2 / (d + 1e-6)),
  *   d = max(count - 1, 1) if unbiased else max(count, 1).
  * Replaces the second half of torch_scatter/composite/std.py:8-41 (gather of the mean, sub, mul,
@@ -313,12 +315,12 @@ int ts_group_logsumexp_backward(const void *src, const int64_t *index,
  * Workspace as for ts_group_softmax. Floating types only.
  */
 int ts_group_std(const void *src, const int64_t *index, const void *total,
-                 const float *count, void *out, int64_t B, int64_t E, int64_t K,
+                 const int32_t *count, void *out, int64_t B, int64_t E, int64_t K,
                  int64_t N, int64_t index_stride_b, int64_t index_stride_e,
                  int dtype, int unbiased, void *workspace, size_t workspace_bytes,
                  ts_stream_t stream);
 int ts_group_std_backward(const void *src, const int64_t *index,
-                          const void *total, const float *count,
+                          const void *total, const int32_t *count,
                           const void *out, const void *grad_out, void *grad_in,
                           int64_t B, int64_t E, int64_t K, int64_t N,
                           int64_t index_stride_b, int64_t index_stride_e,

@@ -56,7 +56,7 @@ int dispatch_coo_gather(int dtype, const CooGatherArgs &a, const CooGatherPlan &
 int dispatch_scatter(int dtype, const ScatterArgs &a, int reduce, int vec, hipStream_t s) {
   TS_DISPATCH(dtype, launch_scatter<T>(a, reduce, vec, s))
 }
-int dispatch_divide(int dtype, void *out, const float *count, int64_t rows, int64_t K, hipStream_t s) {
+int dispatch_divide(int dtype, void *out, const int32_t *count, int64_t rows, int64_t K, hipStream_t s) {
   TS_DISPATCH(dtype, launch_divide_by_count<T>(out, count, rows, K, s))
 }
 int dispatch_sorted_args(int dtype, void *out, int64_t *arg, const int32_t *perm, int64_t B, int64_t per_batch,
@@ -599,13 +599,13 @@ int ts_scatter_with_workspace(const void *src, const int64_t *index, void *out, 
                         nullptr, route_flag, 1);
 }
 
-int ts_scatter_count(const int64_t *index, float *count, int64_t B, int64_t E, int64_t N,
+int ts_scatter_count(const int64_t *index, int32_t *count, int64_t B, int64_t E, int64_t N,
                      int64_t index_stride_b, int64_t index_stride_e, ts_stream_t stream) {
   if (B < 0 || E < 0 || N < 0) return TS_ERR_BAD_ARG;
   if (B * N == 0) return TS_OK;
   if (!count || (B * E > 0 && !index)) return TS_ERR_BAD_ARG;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  hipLaunchKernelGGL(fill_kernel<float>, dim3(grid_for(B * N)), dim3(kBlock), 0, s, count, B * N, 0.0f);
+  hipLaunchKernelGGL(fill_kernel<int32_t>, dim3(grid_for(B * N)), dim3(kBlock), 0, s, count, B * N, (int32_t)0);
   if (B * E > 0) {
     // a sum of ones with K = 1: same kernels as scatter sum (src == nullptr adds 1.0 per entry)
     ScatterArgs a;
@@ -629,12 +629,12 @@ int ts_scatter_count(const int64_t *index, float *count, int64_t B, int64_t E, i
     const bool contended = a.lds_cache == 2 || (a.lds_cache == 1 && sum_table_by_size(B, E, 1, N, 4));
     if (contended && B * N < 0x7FFFFFFFll) {
       const int64_t epb = per_cu_chunk_edges(a.lds_epb, B * E, sum_table_min_chunk(1, 4), 131072);
-      hipLaunchKernelGGL(scatter_add_lds_kernel<float>, dim3((unsigned)((B * E + epb - 1) / epb)), dim3(kLdsAddBlock), 0,
+      hipLaunchKernelGGL(scatter_add_lds_kernel<int32_t>, dim3((unsigned)((B * E + epb - 1) / epb)), dim3(kLdsAddBlock), 0,
                          s, a, kLdsAccRows - 1, epb);
     } else if (env_int("TS_SCATTER_RUNS", 1) && B * N < 0x7FFFFFFFll) {
       // runs of equal neighbouring indices (sorted input) are counted in the wavefront first
       const RunGrid g = run_grid(B * E, 1, 1, 4);
-      launch_add_run<float, 1, 1>(a, g, s);
+      launch_add_run<int32_t, 1, 1>(a, g, s);
     } else {
       hipLaunchKernelGGL(scatter_count_kernel, dim3(grid_for(B * E)), dim3(kBlock), 0, s, index, count, B, E, N,
                          index_stride_b, index_stride_e);
@@ -643,7 +643,7 @@ int ts_scatter_count(const int64_t *index, float *count, int64_t B, int64_t E, i
   return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
 }
 
-int ts_divide_by_count(void *out, const float *count, int64_t B, int64_t N, int64_t K, int dtype,
+int ts_divide_by_count(void *out, const int32_t *count, int64_t B, int64_t N, int64_t K, int dtype,
                        ts_stream_t stream) {
   if (!valid_dtype(dtype) || B < 0 || N < 0 || K < 0) return TS_ERR_BAD_ARG;
   if (B * N * K == 0) return TS_OK;
@@ -781,7 +781,7 @@ int ts_group_logsumexp_backward(const void *src, const int64_t *index, const voi
   return dispatch_group_softmax(dtype, g, GS_LSE_BWD, vec, static_cast<hipStream_t>(stream));
 }
 
-int ts_group_std(const void *src, const int64_t *index, const void *total, const float *count, void *out, int64_t B,
+int ts_group_std(const void *src, const int64_t *index, const void *total, const int32_t *count, void *out, int64_t B,
                  int64_t E, int64_t K, int64_t N, int64_t index_stride_b, int64_t index_stride_e, int dtype,
                  int unbiased, void *workspace, size_t workspace_bytes, ts_stream_t stream) {
   if (!valid_dtype(dtype) || !sizes_ok(B, N, E, K)) return TS_ERR_BAD_ARG;
@@ -812,7 +812,7 @@ int ts_group_std(const void *src, const int64_t *index, const void *total, const
   return dispatch_group_softmax(dtype, g, GS_STD, vec, static_cast<hipStream_t>(stream));
 }
 
-int ts_group_std_backward(const void *src, const int64_t *index, const void *total, const float *count,
+int ts_group_std_backward(const void *src, const int64_t *index, const void *total, const int32_t *count,
                           const void *out, const void *grad_out, void *grad_in, int64_t B, int64_t E, int64_t K,
                           int64_t N, int64_t index_stride_b, int64_t index_stride_e, int dtype, int unbiased,
                           ts_stream_t stream) {

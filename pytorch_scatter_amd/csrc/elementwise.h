@@ -7,9 +7,9 @@
 
 namespace ts {
 
-// count[b, index[b, e]] += 1 (float32; exact up to 2^24 entries per slot)
+// count[b, index[b, e]] += 1 (int32: exact)
 static __global__ __launch_bounds__(kBlock) void scatter_count_kernel(const int64_t *__restrict__ index,
-                                                               float *__restrict__ count, int64_t B,
+                                                               int32_t *__restrict__ count, int64_t B,
                                                                int64_t E, int64_t N, int64_t sb, int64_t se) {
   const int64_t n = B * E;
   for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlock) {
@@ -17,7 +17,7 @@ static __global__ __launch_bounds__(kBlock) void scatter_count_kernel(const int6
     const int64_t e = i - b * E;
     const int64_t idx = index[b * sb + e * se];
     if (idx < 0 || idx >= N) continue;
-    unsafeAtomicAdd(count + b * N + idx, 1.0f);
+    atomicAdd(count + b * N + idx, 1);
   }
 }
 
@@ -31,12 +31,12 @@ template <> struct IsFloatElem<f16_t> { static constexpr bool value = true; };
 // integers (csrc/scatter.cpp:138-141)
 template <typename T>
 __global__ __launch_bounds__(kBlock) void divide_by_count_kernel(T *__restrict__ out,
-                                                                 const float *__restrict__ count,
+                                                                 const int32_t *__restrict__ count,
                                                                  int64_t rows, int64_t K) {
   const int64_t n = rows * K;
   for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlock) {
-    const float cf = count[i / K];
-    const int64_t c = cf < 1.0f ? 1 : (int64_t)cf;
+    const int32_t ci = count[i / K];
+    const int64_t c = ci < 1 ? 1 : (int64_t)ci;
     if constexpr (IsFloatElem<T>::value) {
       out[i] = div_elem<T>(out[i], count_as<T>(c));
     } else {
@@ -96,7 +96,7 @@ __global__ __launch_bounds__(kBlock) void sorted_args_kernel(T *__restrict__ out
 
 template <typename T> int launch_sorted_args(void *out, int64_t *arg, const int32_t *perm, int64_t B, int64_t per_batch,
                                              int64_t E, int64_t perm_batch_stride, bool is_max, hipStream_t stream);
-template <typename T> int launch_divide_by_count(void *out, const float *count, int64_t rows, int64_t K,
+template <typename T> int launch_divide_by_count(void *out, const int32_t *count, int64_t rows, int64_t K,
                                                  hipStream_t stream);
 template <typename T> int launch_arg_backward(const void *grad_out, const int64_t *arg, void *grad_in,
                                               int64_t B, int64_t N, int64_t E, int64_t K,
@@ -117,7 +117,7 @@ template <typename T> int launch_arg_backward(const void *grad_out, const int64_
                          perm_batch_stride);                                                       \
     return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;                                \
   }                                                                                                \
-  template <> int launch_divide_by_count<T>(void *out, const float *count, int64_t rows, int64_t K, \
+  template <> int launch_divide_by_count<T>(void *out, const int32_t *count, int64_t rows, int64_t K, \
                                             hipStream_t stream) {                                  \
     if (rows * K > 0)                                                                              \
       hipLaunchKernelGGL(divide_by_count_kernel<T>, dim3(grid_for(rows * K)), dim3(kBlock), 0,     \

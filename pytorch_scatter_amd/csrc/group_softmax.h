@@ -90,7 +90,7 @@ struct GroupArgs {
   const void *node_grad;  // [B, N, K]: logsumexp backward, its gradient
   int from_neg_inf;       // the group maximum starts from -inf (logsumexp) instead of lowest() (softmax)
   const void *total;      // [B, N, K]: std, the group sums of src in the element type
-  const float *count;     // [B, N]: std, entries per group
+  const int32_t *count;   // [B, N]: std, entries per group (exact)
   int unbiased;           // std: divide by count - 1
   const int *gate = nullptr;  // the three passes of softmax run only if *gate != 0 (null: always)
   int *flag = nullptr;        // softmax: a word behind the workspace of the three passes, for the one-pass kernels
@@ -99,14 +99,14 @@ struct GroupArgs {
 
 // std: the group mean as the reference forms it (composite/std.py:27-31: sum / clamp(count, 1), in the
 // element type) and the divisor of the squared deviations (:36-38: count or clamp(count - 1, 1), plus 1e-6)
-template <typename T> __device__ __forceinline__ typename Acc<T>::type group_mean(T total, float count) {
+template <typename T> __device__ __forceinline__ typename Acc<T>::type group_mean(T total, int32_t count) {
   typedef typename Acc<T>::type F;
-  const F c = round_elem<T>((F)(count < 1.0f ? 1.0f : count));
+  const F c = round_elem<T>((F)(count < 1 ? 1 : count));
   return round_elem<T>(to_acc<T>(total) / c);
 }
-template <typename T> __device__ __forceinline__ typename Acc<T>::type group_divisor(float count, int unbiased) {
+template <typename T> __device__ __forceinline__ typename Acc<T>::type group_divisor(int32_t count, int unbiased) {
   typedef typename Acc<T>::type F;
-  F c = round_elem<T>((F)(count < 1.0f ? 1.0f : count));
+  F c = round_elem<T>((F)(count < 1 ? 1 : count));
   if (unbiased) {
     c = round_elem<T>(c - (F)1);
     if (c < (F)1) c = (F)1;
@@ -216,7 +216,7 @@ template <typename T, int C_, int MODE> struct GroupSumRun : HotState<typename A
   const void *gmax;
   A *gsum;
   const T *total;
-  const float *count;
+  const int32_t *count;
   int64_t K, gs;
   __device__ A identity() const { return (A)0; }
   __device__ void load(int64_t e, int64_t, int64_t col, int node, A *x) const {
@@ -243,7 +243,7 @@ template <typename T, int C_, int MODE> struct GroupSumRun : HotState<typename A
         return;
       }
       const Vec<T, C> tot = load_vec<T, C>(total + (int64_t)node * K + col);
-      const float cnt = count[node];
+      const int32_t cnt = count[node];
 #pragma unroll
       for (int c = 0; c < C; ++c) {
         const A d = round_elem<T>(to_acc<T>(r.v[c]) - group_mean<T>(tot.v[c], cnt));
@@ -513,7 +513,7 @@ __global__ __launch_bounds__(kBlock) void group_finish_kernel(GroupArgs g) {
           const Vec<T, VEC> o = load_vec<T, VEC>(static_cast<const T *>(g.node_out) + slot);
           const Vec<T, VEC> go = load_vec<T, VEC>(static_cast<const T *>(g.node_grad) + slot);
           const Vec<T, VEC> tot = load_vec<T, VEC>(static_cast<const T *>(g.total) + slot);
-          const float cnt = g.count[bb[u] * g.N + idx[u]];
+          const int32_t cnt = g.count[bb[u] * g.N + idx[u]];
           const F div = group_divisor<T>(cnt, g.unbiased);
 #pragma unroll
           for (int v = 0; v < VEC; ++v) {

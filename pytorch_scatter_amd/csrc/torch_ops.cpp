@@ -548,7 +548,7 @@ template <int REDUCE> struct ScatterFn : public torch::autograd::Function<Scatte
     if (REDUCE == TS_MEAN) {
       // count over the index as given (csrc/scatter.cpp:131-141). One index per row (a 1-D index along
       // dim 0, or an index shaped like src's leading dims): the entries are counted straight from the
-      // index (no tensor of ones; fp32 counts) and one kernel clamps, casts and divides.
+      // index (no tensor of ones; exact int32 counts) and one kernel clamps, casts and divides.
       bool per_row = old_index.dim() == dim + 1 && src.numel() > 0 && out.numel() > 0 && old_index.size(dim) == src.size(dim);
       for (int64_t i = 0; per_row && i < dim; i++) per_row = old_index.size(i) == src.size(i);
       if (per_row) {
@@ -557,13 +557,13 @@ template <int REDUCE> struct ScatterFn : public torch::autograd::Function<Scatte
         const BatchedIndex bi = batched_index(old_index);
         // one index row shared by every batch row (an expanded view): counted once and repeated
         const int64_t Bc = (bi.batch_stride == 0 && B > 1) ? 1 : B;
-        Tensor count_f = at::empty({Bc * N}, src.options().dtype(at::kFloat));
-        check_status(ts_scatter_count(bi.t.data_ptr<int64_t>(), count_f.data_ptr<float>(), Bc, E, N, bi.batch_stride, 1,
+        Tensor count_f = at::empty({Bc * N}, src.options().dtype(at::kInt));
+        check_status(ts_scatter_count(bi.t.data_ptr<int64_t>(), count_f.data_ptr<int32_t>(), Bc, E, N, bi.batch_stride, 1,
                                       stream_of(src)),
                      "scatter_mean count");
         if (Bc != B) count_f = count_f.view({1, N}).expand({B, N}).contiguous().view({B * N});
         Tensor out_c = out.contiguous();
-        check_status(ts_divide_by_count(out_c.data_ptr(), count_f.data_ptr<float>(), B, N, K, dtype_code(out_c),
+        check_status(ts_divide_by_count(out_c.data_ptr(), count_f.data_ptr<int32_t>(), B, N, K, dtype_code(out_c),
                                         stream_of(src)),
                      "scatter_mean divide");
         if (!out_c.is_same(out)) out.copy_(out_c);
@@ -841,13 +841,13 @@ struct GroupStdFn : public torch::autograd::Function<GroupStdFn> {
     src = src.contiguous();
     const GroupLayout l = group_layout(src, index, dim);
     Tensor total = std::get<0>(scatter_hip(src, index, dim, std::nullopt, N, TS_SUM)).contiguous();
-    Tensor count = at::empty({l.B * N}, src.options().dtype(at::kFloat));
-    check_status(ts_scatter_count(index.data_ptr<int64_t>(), count.data_ptr<float>(), l.B, l.E, N, l.sb, l.se,
+    Tensor count = at::empty({l.B * N}, src.options().dtype(at::kInt));
+    check_status(ts_scatter_count(index.data_ptr<int64_t>(), count.data_ptr<int32_t>(), l.B, l.E, N, l.sb, l.se,
                                   stream_of(src)),
                  "scatter_std count");
     Tensor out = at::empty_like(total);
     Tensor ws = workspace(ts_group_softmax_workspace_bytes(l.B, N, l.K, dtype_code(src)), src);
-    check_status(ts_group_std(src.data_ptr(), index.data_ptr<int64_t>(), total.data_ptr(), count.data_ptr<float>(),
+    check_status(ts_group_std(src.data_ptr(), index.data_ptr<int64_t>(), total.data_ptr(), count.data_ptr<int32_t>(),
                               out.data_ptr(), l.B, l.E, l.K, N, l.sb, l.se, dtype_code(src), unbiased ? 1 : 0,
                               ws.data_ptr(), static_cast<size_t>(ws.numel()), stream_of(src)),
                  "scatter_std");
@@ -867,7 +867,7 @@ struct GroupStdFn : public torch::autograd::Function<GroupStdFn> {
     const GroupLayout l = group_layout(src, index, dim);
     Tensor grad_in = at::empty_like(src);
     check_status(ts_group_std_backward(src.data_ptr(), index.data_ptr<int64_t>(), total.data_ptr(),
-                                       count.data_ptr<float>(), out.data_ptr(), grad_out.data_ptr(),
+                                       count.data_ptr<int32_t>(), out.data_ptr(), grad_out.data_ptr(),
                                        grad_in.data_ptr(), l.B, l.E, l.K, out.size(dim), l.sb, l.se, dtype_code(src),
                                        unbiased ? 1 : 0, stream_of(src)),
                  "scatter_std backward");

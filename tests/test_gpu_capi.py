@@ -1012,10 +1012,10 @@ def test_scatter_sum_lds_aggregated_variant(capi, oracle, shape, dtype, monkeypa
         err = (out.cpu().double() - want).abs()
         bound = rtol * want.abs() + rtol * (absum + (prev.double().abs() if out_given else 0)).clamp(min=1e-30)
         assert bool((err <= bound).all()), float((err - bound).max())
-    cnt = torch.empty((N,), dtype=torch.float32, device=DEV)
+    cnt = torch.empty((N,), dtype=torch.int32, device=DEV)
     capi.scatter_count(index1.to(DEV), cnt, 1, E, N, 0, 1)
     torch.cuda.synchronize()
-    assert torch.equal(cnt.cpu(), torch.bincount(index1, minlength=N).float())
+    assert torch.equal(cnt.cpu(), torch.bincount(index1, minlength=N).int())
 
 
 @pytest.mark.parametrize("shape,kind,dtype", product(
@@ -1133,10 +1133,10 @@ def test_scatter_sum_runs_of_equal_indices(capi, oracle, shape, kind, dtype):
                 cnt = oracle.scatter(torch.ones(B, E, K, dtype=torch.double), index, 1, None, N, "sum")[0]
                 bound = bound + 2.0 ** -8 * cnt * absum
             assert bool((err <= bound).all()), (kind, out_given, float((err - bound).max()))
-    cnt = torch.empty((N,), dtype=torch.float32, device=DEV)
+    cnt = torch.empty((N,), dtype=torch.int32, device=DEV)
     capi.scatter_count(index1.to(DEV), cnt, 1, E, N, 0, 1)
     torch.cuda.synchronize()
-    assert torch.equal(cnt.cpu(), torch.bincount(index1, minlength=N).float())
+    assert torch.equal(cnt.cpu(), torch.bincount(index1, minlength=N).int())
 
 
 @pytest.mark.parametrize("shape,kind,reduce,dtype", product(
@@ -1223,10 +1223,10 @@ def test_scatter_sum_hot_rows(capi, oracle, K, kind, dtype):
         err = (out.cpu().double() - want).abs()
         bound = rtol * want.abs() + rtol * (absum + (prev.double().abs() if out_given else 0)).clamp(min=1e-30)
         assert bool((err <= bound).all()), (kind, out_given, float((err - bound).max()))
-    cnt = torch.empty((N,), dtype=torch.float32, device=DEV)
+    cnt = torch.empty((N,), dtype=torch.int32, device=DEV)
     capi.scatter_count(index1.to(DEV), cnt, 1, E, N, 0, 1)
     torch.cuda.synchronize()
-    assert torch.equal(cnt.cpu(), torch.bincount(index1, minlength=N).float())
+    assert torch.equal(cnt.cpu(), torch.bincount(index1, minlength=N).int())
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
@@ -1268,11 +1268,11 @@ def test_scatter_sum_plain_atomic_kernel_still_covered(capi, oracle, monkeypatch
     want = oracle.scatter(src, index1.view(1, E, 1).expand(B, E, K), 1, None, N, "sum")[0]
     out = torch.empty((B, N, K), dtype=torch.int32, device=DEV)
     capi.scatter(src.to(DEV), index1.to(DEV), out, None, B, E, K, N, 0, 1, 0, capi.SUM, False)
-    cnt = torch.empty((N,), dtype=torch.float32, device=DEV)
+    cnt = torch.empty((N,), dtype=torch.int32, device=DEV)
     capi.scatter_count(index1.to(DEV), cnt, 1, E, N, 0, 1)
     torch.cuda.synchronize()
     assert_exact(out, want)
-    assert torch.equal(cnt.cpu(), torch.bincount(index1, minlength=N).float())
+    assert torch.equal(cnt.cpu(), torch.bincount(index1, minlength=N).int())
 
 
 @pytest.mark.parametrize("reduce,dtype", product(["sum", "min", "max"], [torch.float32, torch.float64, torch.int64]))
@@ -1310,7 +1310,7 @@ def test_scatter_mean_pieces(capi, oracle):
         index1 = torch.from_numpy(rng.integers(0, N - 2, size=E))
         want = oracle.op_scatter(src, index1, 1, None, N, "mean")
         out = torch.empty((B, N, K), dtype=dtype, device=DEV)
-        cnt = torch.empty((N,), dtype=torch.float32, device=DEV)
+        cnt = torch.empty((N,), dtype=torch.int32, device=DEV)
         capi.scatter(src.to(DEV), index1.to(DEV), out, None, B, E, K, N, 0, 1, 0, capi.SUM, False)
         capi.scatter_count(index1.to(DEV), cnt, 1, E, N, 0, 1)
         for b in range(B):
@@ -1602,3 +1602,28 @@ def test_scatter_k1_workspace_kept_across_calls_with_different_row_counts(capi, 
         assert_exact(out, want, f"values step={step} N={N}")
         assert_exact(arg, want_arg, f"arg step={step} N={N}")
         assert bool((ws[:nzero] == 0).all()), "the key table is handed back as zeros"
+
+
+@pytest.mark.parametrize("dtype", [torch.int32, torch.float64, torch.float32])
+def test_scatter_mean_of_a_group_with_more_than_2_pow_24_entries(capi, oracle, dtype):
+    """One group of 2^24 + 3 entries, one value per entry: the count of scatter mean is an exact integer (a count
+    of ones in fp32 would stop at 2^24), as the reference's count in int32 / double is (csrc/scatter.cpp:131-141).
+    float32: the reference's own count of ones in fp32 stalls at 2^24; here the exact count is rounded once."""
+    E, N = (1 << 24) + 3, 3
+    index = torch.zeros(E, dtype=torch.long)
+    index[5] = 2                      # one entry elsewhere; row 1 stays empty
+    src = torch.ones((1, E, 1), dtype=dtype)
+    src[0, 7, 0] = 9
+    cnt = torch.empty((N,), dtype=torch.int32, device=DEV)
+    capi.scatter_count(index.to(DEV), cnt, 1, E, N, 0, 1)
+    assert cnt.tolist() == [E - 1, 0, 1]
+    out = torch.empty((1, N, 1), dtype=dtype, device=DEV)
+    capi.scatter(src.to(DEV), index.to(DEV), out, None, 1, E, 1, N, 0, 1, 0, capi.SUM, False)
+    capi.divide_by_count(out, cnt, 1, N, 1)
+    torch.cuda.synchronize()
+    if dtype == torch.float32:
+        want = torch.tensor([float(np.float32(np.float32(E - 1 + 8) / np.float32(E - 1))), 0.0, 1.0]).view(1, N, 1)
+        assert torch.allclose(out.cpu(), want, rtol=1e-6, atol=0)
+    else:
+        want = oracle.op_scatter(src, index.view(1, E, 1), 1, None, N, "mean")
+        assert_exact(out, want)

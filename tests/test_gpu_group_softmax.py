@@ -430,7 +430,7 @@ def test_std_forward_and_backward_capi(capi, oracle, shape, kind, dtype, unbiase
     src_d, idx_d = src.to(DEV), index1.to(DEV)
     total = torch.empty((B, N, K), dtype=dtype, device=DEV)
     capi.scatter(src_d, idx_d, total, None, B, E, K, N, 0, 1, 0, capi.SUM, False)
-    count = torch.empty((B, N), dtype=torch.float32, device=DEV)
+    count = torch.empty((B, N), dtype=torch.int32, device=DEV)
     capi.scatter_count(idx_d, count, B, E, N, 0, 1)
     out = torch.empty((B, N, K), dtype=dtype, device=DEV)
     capi.group_std(src_d, idx_d, total, count, out, B, E, K, N, 0, 1, unbiased)
