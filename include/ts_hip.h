@@ -69,18 +69,27 @@ int64_t ts_hip_version(void);
  * workspace: ts_segment_csr_workspace_bytes() bytes of device scratch for the
  * partial results of rows that cross a tile boundary.
  *
- * Status word: the uint64 at workspace + ts_segment_csr_workspace_bytes() -
+ * Status words: two uint64 at workspace + ts_segment_csr_workspace_bytes() -
  * TS_STATUS_BYTES (for ts_segment_coo and ts_segment_csr_permuted: the same
- * offset from the end of what their own *_workspace_bytes() report). Every call
- * sets it to 0 when it starts. A row that crosses tiles is finished by the
- * tile in which it ends, which waits (bounded) for the partial results of the
- * tiles before it; if that wait runs out -- row pointers that are not
- * monotone, an index that is not sorted, or a tile that did not run for
- * seconds -- the row is written as empty (0, arg = E; left untouched with
- * out_given) and bit 0 of the word is set. The caller may read the word after
- * the stream has finished; 0 = every row complete.
+ * offset from the end of what their own *_workspace_bytes() report). Every
+ * call writes a tag of its own (never 0) into word 0. A row that crosses tiles
+ * is finished by the tile in which it ends, which waits (bounded) for the
+ * partial results of the tiles before it; if that wait runs out -- row
+ * pointers that are not monotone, an index that is not sorted, or a tile that
+ * did not run for seconds -- the row is written as empty (0, arg = E; left
+ * untouched with out_given) and the call's tag is written into word 1. After
+ * the stream has finished, word 1 == word 0 means that the latest call gave at
+ * least one row up (ts_status_gave_up below); anything else: every row is
+ * complete. Neither write has to happen before the other, and what an earlier
+ * call left in word 1 never equals a later call's tag. Nothing in the library
+ * reads the words back: a caller that cannot vouch for its row pointers must
+ * (16 bytes, device to host). The torch operators do so after every segment
+ * call when the environment variable TS_CHECK_STATUS is set to 1, and raise.
  */
 #define TS_STATUS_BYTES 256
+/* words: a host copy of the two status words; 1 if the latest call gave a row up, else 0. Host arithmetic only:
+ * no device call. No counterpart in the reference, whose kernels neither wait nor report. */
+int ts_status_gave_up(const unsigned long long *words);
 size_t ts_segment_csr_workspace_bytes(int64_t B, int64_t N, int64_t E, int64_t K,
                                       int dtype, int reduce);
 int ts_segment_csr(const void *src, const int64_t *indptr, void *out,
@@ -212,7 +221,11 @@ size_t ts_scatter_workspace_bytes(int64_t B, int64_t E, int64_t K, int64_t N,
 /* MIN / MAX of one 4-byte value per entry (K == 1, B == 1, E >= 16384, N <= 524288) keep their table of packed
  * keys in the first ts_scatter_workspace_zero_bytes() bytes of the workspace instead of in arg_out. That part has
  * one size (4 MiB) for every such call, whatever N, so a workspace kept across calls with different N stays
- * valid: everything a call writes behind it (its slabs) is never read as zero by a later call. Those bytes
+ * valid: everything a call writes behind it (its slabs) is never read as zero by a later call. The last
+ * TS_STATUS_BYTES of that part are not keys but one uint64 that the call sets to 1, and nobody resets, if one
+ * of the two bounded waits inside the kernel ran out (a lane waiting about a second for room in a queue in
+ * LDS): then entries were lost and the result is not to be trusted; the caller clears the word with the rest
+ * of the part. The torch operators read it after such a call when TS_CHECK_STATUS=1 is set. Those bytes
  * must read as zero when ts_scatter_with_workspace starts, and the call puts them back to zero before it ends:
  * a caller that keeps its workspace from call to call (one per stream) clears it once and never pays for an
  * initial fill again; a caller that takes fresh memory for every call clears that part first

@@ -21,7 +21,7 @@ DTYPE = {torch.float32: 0, torch.float64: 1, torch.float16: 2, torch.bfloat16: 3
          torch.int32: 4, torch.int64: 5, torch.int16: 6, torch.int8: 7, torch.uint8: 8}
 
 EXPORTS = (
-    "ts_error_string", "ts_hip_version",
+    "ts_error_string", "ts_hip_version", "ts_status_gave_up",
     "ts_segment_csr_workspace_bytes", "ts_segment_csr", "ts_segment_csr_static", "ts_gather_csr",
     "ts_segment_mean_csr_backward",
     "ts_segment_coo_workspace_bytes", "ts_segment_coo", "ts_gather_coo",
@@ -93,8 +93,10 @@ CHECK_STATUS = os.environ.get("TS_CHECK_STATUS") == "1"
 
 
 def status_word(ws: torch.Tensor, nbytes: int) -> int:
-    """The status word of a segment reduction that used `ws` (waits for the device)."""
-    return int(ws[nbytes - STATUS_BYTES:nbytes - STATUS_BYTES + 8].view(torch.int64).item())
+    """1 if the latest segment reduction that used `ws` gave a row up, else 0 (waits for the device): the two
+    status words hold the tag of the latest call and the tag of the latest call that gave a row up."""
+    call, gave_up = ws[nbytes - STATUS_BYTES:nbytes - STATUS_BYTES + 16].view(torch.int64).tolist()
+    return int(call != 0 and gave_up == call)
 
 
 def _check_status(ws, nbytes, B, N, K):
@@ -197,6 +199,10 @@ def scatter_with_workspace(src, index, out, arg_out, B, E, K, N, sb, se, sk, red
         _check(L.ts_scatter_with_workspace(_p(src), _p(index), _p(out), _p(arg_out), _i(B), _i(E), _i(K), _i(N),
                                            _i(sb), _i(se), _i(sk), DTYPE[out.dtype], reduce, int(out_given),
                                            _p(ws) if nbytes else None, ctypes.c_size_t(nbytes), _stream(out)))
+    if CHECK_STATUS and nzero >= STATUS_BYTES:
+        # min / max of single values: the word behind the key table is set when a bounded wait in the kernel ran out
+        if int(ws[nzero - STATUS_BYTES:nzero - STATUS_BYTES + 8].view(torch.int64).item()) != 0:
+            raise TsError("ts_hip: scatter min / max lost entries: a bounded wait inside the kernel ran out")
     return ws
 
 

@@ -140,8 +140,8 @@ int run_csr_reduce_slice(const void *src, const int64_t *indptr, void *out, int6
                          int64_t B, int64_t N, int64_t E, int64_t K, int64_t indptr_batch_stride, int dtype,
                          int reduce, int accumulate, void *ws, size_t ws_bytes, hipStream_t stream,
                          const int32_t *perm, int64_t perm_batch_stride, bool want_perm_args, bool *perm_args_done,
-                         unsigned long long *status, bool status_reset, const int *gate = nullptr,
-                         int scatter_rule = 0) {
+                         unsigned long long *status, bool status_reset, uint64_t status_nonce,
+                         const int *gate = nullptr, int scatter_rule = 0) {
   const bool al = aligned16(src) && aligned16(out);
   // permuted rows always take the wide kernel (the narrow one stages consecutive entries), and so does a gated call
   const CsrPlan p = csr_plan(N, E, K, kElemBytes[dtype], al, false, reduce == TS_MIN || reduce == TS_MAX,
@@ -172,6 +172,7 @@ int run_csr_reduce_slice(const void *src, const int64_t *indptr, void *out, int6
   a.nonce = next_nonce();
   a.status = status;
   a.status_reset = status_reset ? 1 : 0;
+  a.status_nonce = status_nonce;
   a.carry_spin = env_int("TS_CSR_SPIN", kCarrySpin);  // test aid: -1 makes every look-back give up at once
   a.perm = perm;
   a.perm_batch_stride = perm_batch_stride;
@@ -195,13 +196,15 @@ int run_csr_reduce(const void *src, const int64_t *indptr, void *out, int64_t *a
                    bool *perm_args_done = nullptr, const int *gate = nullptr, int scatter_rule = 0) {
   const int64_t s = kElemBytes[dtype];
   const bool want_perm_args = B * N * K >= ((int64_t)8 << 20);
+  const uint64_t status_nonce = next_nonce();  // one for all slices: the status words describe the whole call
   // every slice reuses the workspace: the launches follow each other on one stream
   return for_batch_slices(B, [&](int64_t b0, int64_t nb) {
     return run_csr_reduce_slice(offset_bytes(src, b0 * E * K * s), indptr + b0 * indptr_batch_stride,
                                 offset_bytes(out, b0 * N * K * s), arg_out ? arg_out + b0 * N * K : nullptr,
                                 offset_bytes(count_out, b0 * N * s), nb, N, E, K, indptr_batch_stride, dtype, reduce,
                                 accumulate, ws, ws_bytes, stream, perm ? perm + b0 * perm_batch_stride : nullptr,
-                                perm_batch_stride, want_perm_args, perm_args_done, status, b0 == 0, gate, scatter_rule);
+                                perm_batch_stride, want_perm_args, perm_args_done, status, b0 == 0, status_nonce, gate,
+                                scatter_rule);
   });
 }
 
@@ -276,6 +279,10 @@ int run_coo_to_indptr(const int64_t *index, int64_t *ptr, int64_t B, int64_t E, 
 }  // namespace
 
 extern "C" {
+
+int ts_status_gave_up(const unsigned long long *words) {
+  return words != nullptr && words[0] != 0 && words[1] == words[0];
+}
 
 const char *ts_error_string(int status) {
   switch (status) {

@@ -15,8 +15,8 @@
 // leave the combination to a small second kernel instead. Either way the order of the
 // combination is fixed by the tiling, so the result is independent of scheduling.
 // If the bounded wait runs out (row pointers that are not monotone, or a producer tile
-// that did not run for seconds) the row is written as empty (0, arg = E) and a sticky
-// status word in the workspace is set; a clean call leaves that word at 0.
+// that did not run for seconds) the row is written as empty (0, arg = E) and the call's
+// nonce is left in the second status word of the workspace (see CsrReduceArgs::status).
 //
 // Semantics follow the reference CPU loop (csrc/cpu/segment_csr_cpu.cpp:54-88):
 // accumulate in float for 16-bit floats, strict compare so the first index
@@ -68,8 +68,11 @@ struct CsrReduceArgs {
   int64_t perm_batch_stride;
   int perm_args;      // min / max with perm: the kernel itself writes positions in src's order and applies
                       // scatter's rule for slots that never beat the initial value (no pass over arg_out after it)
-  // status word of the call (device memory, may be null): set to 0 by the first tile when status_reset is set,
-  // or-ed with kStatusGaveUp by a tile whose look-back ran out of polls
+  // status words of the call (device memory, two 64-bit words, may be null): word 0 receives status_nonce from
+  // the first tile when status_reset is set ("the latest call"), word 1 receives status_nonce from a tile whose
+  // look-back ran out of polls ("the latest call that gave a row up"). The call gave a row up iff the two are
+  // equal afterwards: no write has to be ordered against another one, and a word left by an earlier call
+  // never matches.
   // optional gate (a scatter whose index turned out to be sorted takes this reduction instead of the buckets):
   // the kernel returns at once unless (*gate != 0) == (gate_want != 0). scatter_rule: min / max write a slot whose
   // entries never beat the initial value of the element type as 0 with position E, as scatter does
@@ -79,9 +82,9 @@ struct CsrReduceArgs {
   int scatter_rule = 0;
   unsigned long long *status;
   int status_reset;
+  uint64_t status_nonce;  // never 0; the same for every slice of one call
   int carry_spin;     // polls per batch of carry flags before the look-back gives up; < 0: give up without polling
 };
-constexpr unsigned long long kStatusGaveUp = 1;
 
 // ---- rows that cross tiles, finished without a second kernel ---------------------------------
 // The tile in which such a row ends walks back over the tiles before it. A tile whose last row is
@@ -255,7 +258,7 @@ __global__ __launch_bounds__(kCsrBlock, (csr_reduce_min_blocks<T, VEC, REDUCE, P
     if (tid == 0) { s_cut[0] = ia; s_cut[1] = ib; }
   }
   if (a.status_reset && a.status != nullptr && tid == 0 && (blockIdx.x | blockIdx.y | blockIdx.z) == 0)
-    __hip_atomic_exchange(a.status, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_exchange(a.status, (unsigned long long)a.status_nonce, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   __syncthreads();
   const int64_t i0 = s_cut[0], i1 = s_cut[1];
   const int64_t j0 = d0 - i0;
@@ -472,7 +475,8 @@ __global__ __launch_bounds__(kCsrBlock, (csr_reduce_min_blocks<T, VEC, REDUCE, P
       }
       if (spin <= 0) {  // e.g. indptr not monotone: these carries will never be published
         if (lg == 0 && a.status != nullptr)
-          __hip_atomic_fetch_or(a.status, kStatusGaveUp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          __hip_atomic_exchange(a.status + 1, (unsigned long long)a.status_nonce, __ATOMIC_RELAXED,
+                                __HIP_MEMORY_SCOPE_AGENT);
         return false;
       }
       asm volatile("" ::: "memory");

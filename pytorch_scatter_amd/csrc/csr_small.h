@@ -62,7 +62,7 @@ __global__ __launch_bounds__(kBlock) void csr_reduce_small_kernel(CsrReduceArgs 
   }
   if (tid == 0) s_nlong = 0;
   if (a.status_reset && a.status != nullptr && tid == 0 && (blockIdx.x | blockIdx.z) == 0)
-    __hip_atomic_exchange(a.status, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // this kernel never waits
+    __hip_atomic_exchange(a.status, (unsigned long long)a.status_nonce, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // this kernel never waits
   __syncthreads();
   const int64_t i0 = s_cut[0], i1 = s_cut[1];
   const int64_t j0 = d0 - i0;

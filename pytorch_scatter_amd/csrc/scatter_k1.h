@@ -24,6 +24,9 @@
 //    for each of the output rows that map to these table rows, and writes out / arg_out directly.
 // The key table must read as zero when the call starts and is put back to zero by the final kernel, so a
 // caller that reuses its workspace pays for no initial fill: two launches in all.
+// Both waits in the main kernel are bounded (a producer waiting for room in its queue, a consumer waiting for
+// its producers): if one of them ever runs out, entries are lost, and the kernel says so in a word behind the key
+// table (K1Plan::fail), which stays set until the caller clears it.
 //
 // Keys are those of scatter.h: order(value) << 32 | (0xFFFFFFFE - position), larger wins, so equal values
 // keep the smallest position (csrc/cpu/reducer.h:63-67). A value that does not beat the initial value of the
@@ -44,6 +47,7 @@ constexpr int kK1Groups = 256;    // workgroups of the main kernel: one per CU
 constexpr int kK1PerRow = 64;     // output rows that may share a table row: N <= kK1PerRow * kK1Rows
 constexpr int kK1FinalRows = 16;  // table rows per workgroup of the final kernel
 constexpr int kK1FinalBlock = 256;
+constexpr int kK1Spin = 1 << 24;  // polls of a producer that waits for room in its queue (about a second)
 
 struct K1Plan {
   bool ok;
@@ -53,6 +57,8 @@ struct K1Plan {
   size_t bytes;        // workspace
   size_t zero_bytes;   // its leading part that must be zero before the call and is zero after it
   uint64_t *gkeys;     // [N]
+  unsigned long long *fail;  // set (sticky) when a bounded wait of the main kernel ran out: entries were lost
+  int spin;            // polls of a producer that waits for room in its queue
   uint64_t *slab_keys; // [G][kK1Rows]
   int32_t *slab_tags;  // [G][kK1Rows]
 };
@@ -72,11 +78,15 @@ inline K1Plan k1_plan(int64_t B, int64_t E, int64_t K, int64_t N, int elem_bytes
   // The key table takes the room of the largest N this plan serves, whatever N is: a workspace kept from call
   // to call then has the same zero-on-entry part for every call, and the slabs of one call never land in what a
   // later call with more output rows reads as its (zero) key table.
-  const size_t o_keys = up((size_t)kK1PerRow * kK1Rows * 8), o_tags = o_keys + up((size_t)G * kK1Rows * 8);
-  p.zero_bytes = o_keys;
+  const size_t o_fail = up((size_t)kK1PerRow * kK1Rows * 8), o_keys = o_fail + 256;
+  const size_t o_tags = o_keys + up((size_t)G * kK1Rows * 8);
+  p.zero_bytes = o_keys;  // the key table and the word behind it
+  p.spin = kK1Spin;
+  if (const char *env = getenv("TS_K1_SPIN")) p.spin = atoi(env);  // test aid: 0 = a producer never waits
   p.bytes = o_tags + up((size_t)G * kK1Rows * 4);
   if (ws == nullptr || ws_bytes < p.bytes || (reinterpret_cast<uintptr_t>(ws) & 15) != 0) return p;
   p.gkeys = static_cast<uint64_t *>(ws);
+  p.fail = reinterpret_cast<unsigned long long *>(static_cast<char *>(ws) + o_fail);
   p.slab_keys = reinterpret_cast<uint64_t *>(static_cast<char *>(ws) + o_keys);
   p.slab_tags = reinterpret_cast<int32_t *>(static_cast<char *>(ws) + o_tags);
   p.ok = true;
@@ -94,14 +104,14 @@ __global__ __launch_bounds__(kK1Block) void scatter_k1_main_kernel(ScatterArgs a
   __shared__ uint64_t s_qkey[kK1Queues][kK1QueueCap];
   __shared__ int32_t s_qnode[kK1Queues][kK1QueueCap];
   __shared__ int32_t s_tail[kK1Queues], s_head[kK1Queues];
-  __shared__ int32_t s_done;
+  __shared__ int32_t s_done, s_fail;
   for (int i = threadIdx.x; i < kK1Rows; i += kK1Block) {
     s_keys[i] = 0;
     s_tags[i] = -1;
   }
   for (int i = threadIdx.x; i < kK1Queues * kK1QueueCap; i += kK1Block) (&s_qnode[0][0])[i] = -1;
   if (threadIdx.x < kK1Queues) { s_tail[threadIdx.x] = 0; s_head[threadIdx.x] = 0; }
-  if (threadIdx.x == 0) s_done = 0;
+  if (threadIdx.x == 0) { s_done = 0; s_fail = 0; }
   __syncthreads();
 
   const T *src = static_cast<const T *>(a.src);
@@ -128,8 +138,10 @@ __global__ __launch_bounds__(kK1Block) void scatter_k1_main_kernel(ScatterArgs a
     auto push = [&](int node, uint64_t key) {
       const int slot = atomicAdd(&s_tail[q], 1);
       // the slot is free once the consumer has passed slot - cap; the consumer never waits for a producer
-      for (int spin = 0; slot - lds_peek(&s_head[q]) >= kK1QueueCap && spin < (1 << 24); ++spin)
-        __builtin_amdgcn_s_sleep(2);
+      int spin = 0;
+      for (; slot - lds_peek(&s_head[q]) >= kK1QueueCap && spin < p.spin; ++spin) __builtin_amdgcn_s_sleep(2);
+      // ran out: the store below overwrites an entry the consumer has not taken yet
+      if (slot - lds_peek(&s_head[q]) >= kK1QueueCap) s_fail = 1;
       s_qkey[q][slot & (kK1QueueCap - 1)] = key;
       __hip_atomic_store(&s_qnode[q][slot & (kK1QueueCap - 1)], node, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     };
@@ -192,8 +204,8 @@ __global__ __launch_bounds__(kK1Block) void scatter_k1_main_kernel(ScatterArgs a
   } else {
     // ---- the wavefronts that issue the atomics: one queue each, entries taken in order
     const int q = wave - kK1StreamWaves;
-    int head = 0;
-    for (int idle = 0; idle < (1 << 26);) {
+    int head = 0, idle = 0;
+    for (; idle < (1 << 26);) {
       const int at = (head + lane) & (kK1QueueCap - 1);
       const int node = lds_peek(&s_qnode[q][at]);
       const uint64_t ready = __ballot(node != -1);
@@ -212,8 +224,11 @@ __global__ __launch_bounds__(kK1Block) void scatter_k1_main_kernel(ScatterArgs a
       head += cnt;
       if (lane == 0) __hip_atomic_store(&s_head[q], head, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
+    if (idle >= (1 << 26)) s_fail = 1;  // left with entries still queued
   }
   __syncthreads();
+  if (threadIdx.x == 0 && s_fail != 0)
+    __hip_atomic_fetch_or(p.fail, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   uint64_t *sk = p.slab_keys + (int64_t)blockIdx.x * kK1Rows;
   int32_t *st = p.slab_tags + (int64_t)blockIdx.x * kK1Rows;
   for (int i = threadIdx.x; i < kK1Rows; i += kK1Block) {

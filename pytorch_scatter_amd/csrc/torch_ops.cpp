@@ -94,6 +94,26 @@ std::optional<int64_t> collapsed_stride(const Tensor &t, int64_t lo, int64_t hi)
   return have ? inner : 0;
 }
 
+// Opt-in check of a segment reduction's status words (TS_CHECK_STATUS=1 in the environment, read once): copies
+// the 16 bytes back, which waits for the stream, and raises if the call gave a row up (row pointers that are
+// not monotone, an index that is not sorted). Off by default: the operators never synchronise on their own.
+bool status_checks_on() {
+  static const bool on = [] {
+    const char *e = getenv("TS_CHECK_STATUS");
+    return e != nullptr && atoi(e) != 0;
+  }();
+  return on;
+}
+void maybe_check_status_words(const Tensor &ws, size_t ws_bytes, const char *what) {
+  if (!status_checks_on() || ws_bytes < TS_STATUS_BYTES || (size_t)ws.numel() < ws_bytes) return;
+  const Tensor words = ws.narrow(0, (int64_t)(ws_bytes - TS_STATUS_BYTES), 16).cpu();
+  unsigned long long w[2];
+  memcpy(w, words.data_ptr(), sizeof(w));
+  TORCH_CHECK(!ts_status_gave_up(w), "torch_scatter (", what,
+              "): a row that crosses tiles was given up and written as empty -- row pointers that are not "
+              "monotone or an index that is not sorted");
+}
+
 Tensor workspace(size_t bytes, const Tensor &like) {
   return at::empty({static_cast<int64_t>(bytes > 0 ? bytes : 1)}, like.options().dtype(at::kByte));
 }
@@ -236,6 +256,12 @@ std::tuple<Tensor, OptTensor> scatter_hip(Tensor src, Tensor index, int64_t dim,
                                            ws_bytes, stream_of(src));
   if (rc != TS_OK && ws_zero > 0) drop_kept_workspace(src, stream_of(src));
   check_status(rc, "scatter");
+  if (ws_zero >= TS_STATUS_BYTES && status_checks_on()) {
+    // min / max of single values: the word behind the key table says whether a bounded wait in the kernel ran out
+    const bool lost = ws.narrow(0, (int64_t)(ws_zero - TS_STATUS_BYTES), 8).cpu().view(at::kLong).item<int64_t>() != 0;
+    if (lost) drop_kept_workspace(src, stream_of(src));
+    TORCH_CHECK(!lost, "torch_scatter (scatter): a bounded wait inside the kernel ran out and entries were lost");
+  }
   return std::make_tuple(out, arg_out);
 }
 
@@ -299,6 +325,7 @@ std::tuple<Tensor, OptTensor> segment_csr_hip(Tensor src, Tensor indptr, OptTens
                               minmax ? arg_out.value().data_ptr<int64_t>() : nullptr, cs.B, N, E, K,
                               cs.batch_stride, dtype_code(src), reduce, ws.data_ptr(), ws_bytes, stream_of(src)),
                "segment_csr");
+  maybe_check_status_words(ws, ws_bytes, "segment_csr");
   return std::make_tuple(out, arg_out);
 }
 
@@ -424,6 +451,7 @@ std::tuple<Tensor, OptTensor> segment_coo_hip(Tensor src, Tensor index, OptTenso
                               cs.batch_stride, dtype_code(src), reduce, optional_out.has_value() ? 1 : 0,
                               ws.data_ptr(), ws_bytes, stream_of(src)),
                "segment_coo");
+  maybe_check_status_words(ws, ws_bytes, "segment_coo");
   return std::make_tuple(out, second);
 }
 
@@ -966,12 +994,14 @@ template <int REDUCE> struct SortedScatterFn : public torch::autograd::Function<
     Tensor out = at::empty(sizes, src.options());
     Tensor arg_out = kArg ? at::empty(sizes, index.options()) : Tensor();
     if (out.numel() > 0) {
-      Tensor ws = workspace(ts_segment_csr_permuted_workspace_bytes(B, N, E, K, dtype_code(src), reduce), src);
+      const size_t ws_bytes = ts_segment_csr_permuted_workspace_bytes(B, N, E, K, dtype_code(src), reduce);
+      Tensor ws = workspace(ws_bytes, src);
       check_status(ts_segment_csr_permuted(src.data_ptr(), perm.data_ptr<int32_t>(), indptr.data_ptr<int64_t>(),
                                            out.data_ptr(), kArg ? arg_out.data_ptr<int64_t>() : nullptr, B, N, E, K, 0,
                                            0, dtype_code(src), reduce, ws.data_ptr(),
                                            static_cast<size_t>(ws.numel()), stream_of(src)),
                    "scatter_sorted");
+      maybe_check_status_words(ws, ws_bytes, "scatter_sorted");
     }
     ctx->saved_data["dim"] = dim;
     ctx->saved_data["src_shape"] = src.sizes();

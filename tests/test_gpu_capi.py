@@ -1627,3 +1627,64 @@ def test_scatter_mean_of_a_group_with_more_than_2_pow_24_entries(capi, oracle, d
     else:
         want = oracle.op_scatter(src, index.view(1, E, 1), 1, None, N, "mean")
         assert_exact(out, want)
+
+
+@pytest.mark.parametrize("case,reduce", product([("hub", 900, 64), ("zipf", 3000, 64), ("long", 12, 64)],
+                                                ["sum", "mean", "min", "max"]))
+def test_segment_csr_two_launch_fallback(capi, oracle, case, reduce, monkeypatch):
+    """TS_CSR_LOOKBACK=0: rows that cross tiles are finished by the second kernel instead of the look-back inside
+    the first (the path 8- / 16-bit accumulators and rows of more than four column chunks always take, and the way
+    out for 4- / 8-byte accumulators should the look-back ever misbehave). fp32, 64 columns, every reduction, next
+    to the look-back run of the same input (sums may differ in the last bits: the second kernel adds the partial
+    sums of a row front to back, the look-back back to front)."""
+    kind, n, K = case
+    rng, indptr, index = make_csr(kind, 77, n)
+    E = index.numel()
+    src = values(rng, (E, K), torch.float32, reduce)
+    want, want_arg = oracle.segment_csr(src, indptr, None, reduce)
+    for lookback in ("0", "1"):
+        monkeypatch.setenv("TS_CSR_LOOKBACK", lookback)
+        out = torch.full((n, K), 7, dtype=torch.float32, device=DEV)
+        arg = torch.full((n, K), -1, dtype=torch.long, device=DEV) if reduce in ("min", "max") else None
+        capi.segment_csr(src.to(DEV), indptr.to(DEV), out, arg, 1, n, E, K, 0, capi.REDUCE[reduce])
+        torch.cuda.synchronize()
+        if reduce in ("min", "max"):
+            assert_exact(out, want, f"values lookback={lookback}")
+            assert_exact(arg, want_arg, f"arg lookback={lookback}")
+        else:
+            scale = float(oracle.segment_csr(src.abs().double(), indptr, None, "sum")[0].max())
+            assert_close(out, want, scale, torch.float32, f"values lookback={lookback}")
+
+
+@pytest.mark.parametrize("reduce", ["min", "max"])
+def test_scatter_k1_reports_a_wait_that_ran_out(capi, oracle, reduce, monkeypatch):
+    """The producers of the one-value-per-entry kernel wait (bounded) for room in a queue in LDS. With the bound
+    forced to "never wait" from the host (TS_K1_SPIN=0) a full queue loses entries: every kernel still exits
+    normally, and the word behind the key table says so -- a result is either exact or flagged. With the default
+    bound the same input is exact and the word stays 0."""
+    monkeypatch.setenv("TS_SCATTER_LDS", "2")
+    rng = np.random.default_rng(3)
+    E, N = 400_000, 300_000                       # a uniform index: nearly every entry goes through a queue
+    src = torch.from_numpy(rng.standard_normal((1, E, 1)).astype(np.float32))
+    index = torch.from_numpy(rng.integers(0, N, size=E).astype(np.int64))
+    want, want_arg = oracle.scatter(src, index.view(1, -1, 1), 1, None, N, reduce)
+    L = capi.lib()
+    nzero = L.ts_scatter_workspace_zero_bytes(capi._i(1), capi._i(E), capi._i(1), capi._i(N), capi.DTYPE[torch.float32],
+                                              capi.REDUCE[reduce])
+    assert nzero >= capi.STATUS_BYTES
+    monkeypatch.setattr(capi, "CHECK_STATUS", False)
+    for spin, must_be_clean in (("0", False), (None, True)):
+        if spin is None:
+            monkeypatch.delenv("TS_K1_SPIN")
+        else:
+            monkeypatch.setenv("TS_K1_SPIN", spin)
+        out = torch.empty((1, N, 1), dtype=torch.float32, device=DEV)
+        arg = torch.empty((1, N, 1), dtype=torch.long, device=DEV)
+        ws = capi.scatter_with_workspace(src.to(DEV), index.to(DEV), out, arg, 1, E, 1, N, 0, 1, 0,
+                                         capi.REDUCE[reduce], False, None)
+        torch.cuda.synchronize()
+        flagged = int(ws[nzero - capi.STATUS_BYTES:nzero - capi.STATUS_BYTES + 8].view(torch.int64).item()) != 0
+        exact = torch.equal(out.cpu(), want) and torch.equal(arg.cpu(), want_arg)
+        assert exact or flagged, "a result that lost entries must be flagged"
+        if must_be_clean:
+            assert exact and not flagged

@@ -635,3 +635,28 @@ def test_scatter_of_single_values_with_a_changing_number_of_output_rows(ts, orac
         want, want_arg = oracle.scatter(src, index, 0, None, N, reduce)
         assert torch.equal(got.cpu(), want), f"values step={step} N={N}"
         assert torch.equal(arg.cpu(), want_arg), f"arg step={step} N={N}"
+
+
+def test_operators_raise_when_a_row_was_given_up(ts):
+    """TS_CHECK_STATUS=1 (set for the whole test run): after a segment reduction the operators read the two status
+    words back and raise if a row that crosses tiles was given up. The give-up is forced from the host on
+    well-formed row pointers (TS_CSR_SPIN=-1: no tile waits for another, every kernel exits normally); without
+    the override the same call returns the sums."""
+    import os
+    K = 64
+    indptr = torch.tensor([0, 200, 5000, 9000], device=DEV)      # rows of thousands of entries cross tiles
+    src = torch.randn((9000, K), device=DEV)
+    old = os.environ.get("TS_CSR_SPIN")
+    os.environ["TS_CSR_SPIN"] = "-1"
+    try:
+        with pytest.raises(RuntimeError, match="given up"):
+            ts.segment_csr(src, indptr, None, "sum")
+        with pytest.raises(RuntimeError, match="given up"):
+            ts.segment_coo(src, torch.repeat_interleave(torch.arange(3, device=DEV), indptr[1:] - indptr[:-1]), None, 3, "sum")
+    finally:
+        if old is None:
+            del os.environ["TS_CSR_SPIN"]
+        else:
+            os.environ["TS_CSR_SPIN"] = old
+    out = ts.segment_csr(src, indptr, None, "sum")
+    assert torch.allclose(out[1], src[200:5000].double().sum(0).float(), rtol=1e-4, atol=1e-3)
