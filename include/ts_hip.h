@@ -239,6 +239,33 @@ int ts_scatter_with_workspace(const void *src, const int64_t *index, void *out,
                               int dtype, int reduce, int out_given, void *workspace,
                               size_t workspace_bytes, ts_stream_t stream);
 
+/* Which kernels the last ts_scatter / ts_scatter_with_workspace call of the calling thread launched: a host-side
+ * note for tests and tools (no device call, no synchronisation). Where two kernels are launched and a flag
+ * written on the device picks the one that does the work (a sample or a full check of the index), the name says
+ * both. No counterpart in the reference, which has one kernel per reduction (csrc/cuda/scatter_cuda.cu:13-56). */
+enum ts_scatter_route {
+  TS_ROUTE_NONE = 0,
+  TS_ROUTE_SUM_ATOMIC = 1,               /* one atomic per element (per packed pair for 16-bit floats) */
+  TS_ROUTE_SUM_RUNS = 2,                 /* runs of equal neighbouring indices combined in the wavefront, hot rows in LDS */
+  TS_ROUTE_SUM_TABLE = 3,                /* accumulator table in LDS per workgroup */
+  TS_ROUTE_SUM_TABLE_OR_RUNS = 4,        /* a sample of the index picks: table (unsorted) or runs (sorted) */
+  TS_ROUTE_SUM_BUCKETS_OR_RUNS = 5,      /* workspace: entries binned by bucket of output rows; a sorted-looking index: runs */
+  TS_ROUTE_SUM_BUCKETS_OR_SEGMENTED = 6, /* workspace: buckets; an index found sorted: the segmented reduction */
+  TS_ROUTE_MUL_ATOMIC = 7,
+  TS_ROUTE_MUL_TABLE = 8,
+  TS_ROUTE_MINMAX_ATOMIC = 9,            /* packed 64-bit keys, one atomic max per element */
+  TS_ROUTE_MINMAX_RUNS = 10,             /* runs combined in the wavefront first */
+  TS_ROUTE_MINMAX_RUNS_OR_TABLE = 11,    /* a sample of the index picks: runs (even / sorted) or key table in LDS (skewed) */
+  TS_ROUTE_MINMAX_TABLE = 12,            /* key table in LDS per workgroup */
+  TS_ROUTE_MINMAX_TABLE_K1 = 13,         /* the same for one value per entry */
+  TS_ROUTE_MINMAX_K1_SLABS = 14,         /* workspace, one value per entry: tables handed over in slabs */
+  TS_ROUTE_MINMAX_BUCKETS = 15,          /* workspace: entries binned by bucket of output rows */
+  TS_ROUTE_MINMAX_BUCKETS_OR_SEGMENTED = 16, /* the same; an index found sorted: the segmented reduction */
+  TS_ROUTE_MINMAX_64BIT = 17             /* 64-bit elements: value pass, then position pass */
+};
+int ts_scatter_last_route(void);
+const char *ts_scatter_route_name(int route);
+
 /* count[b, index[b*sb + e*se]] += 1 as int32 (exact for any group size below 2^31), count pre-zeroed by the
  * call. The count half of ScatterMean::forward, csrc/scatter.cpp:131-137, which sums ones in the element
  * type: equal wherever that sum is exact (any size for int32 / int64 / double), and exact beyond 2^24 entries

@@ -21,7 +21,7 @@ DTYPE = {torch.float32: 0, torch.float64: 1, torch.float16: 2, torch.bfloat16: 3
          torch.int32: 4, torch.int64: 5, torch.int16: 6, torch.int8: 7, torch.uint8: 8}
 
 EXPORTS = (
-    "ts_error_string", "ts_hip_version", "ts_status_gave_up",
+    "ts_error_string", "ts_hip_version", "ts_status_gave_up", "ts_scatter_last_route", "ts_scatter_route_name",
     "ts_segment_csr_workspace_bytes", "ts_segment_csr", "ts_segment_csr_static", "ts_gather_csr",
     "ts_segment_mean_csr_backward",
     "ts_segment_coo_workspace_bytes", "ts_segment_coo", "ts_gather_coo",
@@ -104,6 +104,13 @@ def _check_status(ws, nbytes, B, N, K):
         word = status_word(ws, nbytes)
         if word != 0:
             raise TsError(f"ts_hip: segment reduction left status word {word}: a row was given up")
+
+
+def scatter_last_route() -> str:
+    """Name of the kernels the last scatter call of this thread launched (ts_scatter_last_route)."""
+    L = lib()
+    L.ts_scatter_route_name.restype = ctypes.c_char_p
+    return L.ts_scatter_route_name(L.ts_scatter_last_route()).decode()
 
 
 def hip_version() -> int:

@@ -280,6 +280,21 @@ int run_coo_to_indptr(const int64_t *index, int64_t *ptr, int64_t B, int64_t E, 
 
 extern "C" {
 
+namespace {
+thread_local int g_scatter_route = TS_ROUTE_NONE;
+}
+void ts_note_scatter_route(int route) { g_scatter_route = route; }
+int ts_scatter_last_route(void) { return g_scatter_route; }
+const char *ts_scatter_route_name(int route) {
+  static const char *const names[] = {
+      "none", "sum: atomic", "sum: runs", "sum: table", "sum: table or runs (sample)", "sum: buckets or runs (sample)",
+      "sum: buckets or segmented reduction (index checked)", "mul: atomic", "mul: table", "min/max: atomic",
+      "min/max: runs", "min/max: runs or table (sample)", "min/max: table", "min/max: table, one value per entry",
+      "min/max: slabs, one value per entry", "min/max: buckets", "min/max: buckets or segmented reduction (index checked)",
+      "min/max: 64-bit elements, two passes"};
+  return route >= 0 && route < (int)(sizeof(names) / sizeof(names[0])) ? names[route] : "unknown";
+}
+
 int ts_status_gave_up(const unsigned long long *words) {
   return words != nullptr && words[0] != 0 && words[1] == words[0];
 }

@@ -37,6 +37,10 @@
 
 #include "device_utils.h"
 
+// Which kernels the last ts_scatter* call of this thread launched (TS_ROUTE_* of include/ts_hip.h; defined in
+// capi.hip): a host-side note for tests and tools, read back through ts_scatter_last_route().
+extern "C" void ts_note_scatter_route(int route);
+
 namespace ts {
 
 // ---------------------------------------------------------------- atomics
@@ -1859,6 +1863,7 @@ int launch_scatter_v(const ScatterArgs &args, int reduce, hipStream_t stream) {
     }
     if constexpr (BinSlotOk<T>::value) {
       if (lshift >= 0) {
+        ts_note_scatter_route(routed ? TS_ROUTE_SUM_BUCKETS_OR_SEGMENTED : TS_ROUTE_SUM_BUCKETS_OR_RUNS);
         launch_binned_add<T, VEC>(a, bp.p, lshift, stream, routed ? n_out : 0);
         a.skip_flag = bp.p.unsorted;
         if (routed) {
@@ -1890,6 +1895,7 @@ int launch_scatter_v(const ScatterArgs &args, int reduce, hipStream_t stream) {
             }
             const int64_t epb = per_cu_chunk_edges(a.lds_epb, n_edges, sum_table_min_chunk(a.K, (int)sizeof(T)),
                                                    131072 / a.K > 2048 ? 131072 / a.K : 2048);
+            ts_note_scatter_route(sampled ? TS_ROUTE_SUM_TABLE_OR_RUNS : TS_ROUTE_SUM_TABLE);
             hipLaunchKernelGGL(scatter_add_lds_kernel<T>, dim3((unsigned)((n_edges + epb - 1) / epb)),
                                dim3(kLdsAddBlock), 0, stream, t, tn - 1, epb);
             if (!sampled) return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
@@ -1905,6 +1911,7 @@ int launch_scatter_v(const ScatterArgs &args, int reduce, hipStream_t stream) {
             // rows that cannot be written word by word: one column per lane and atomic
             const RunGrid g = run_grid(n_edges, a.K, 1, (int)sizeof(T));
             if (g.ok) {
+              if (lshift < 0 && !use_lds) ts_note_scatter_route(TS_ROUTE_SUM_RUNS);
               launch_add_run<T, 1, 1>(a, g, stream);
               return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
             }
@@ -1917,6 +1924,7 @@ int launch_scatter_v(const ScatterArgs &args, int reduce, hipStream_t stream) {
             const RunGrid g = run_grid(n_edges, a.K / (wide ? C : CN), wide ? C : CN, (wide ? C : CN) * (int)sizeof(T));
             if (g.ok) {
               constexpr int EWD = sizeof(T) < 4 ? 4 / (int)sizeof(T) : 1;  // a whole 32-bit word per atomic
+              if (lshift < 0 && !use_lds) ts_note_scatter_route(TS_ROUTE_SUM_RUNS);
               if (wide)
                 launch_add_run<T, C, EWD>(a, g, stream);
               else
@@ -1928,11 +1936,13 @@ int launch_scatter_v(const ScatterArgs &args, int reduce, hipStream_t stream) {
         if constexpr (__is_same(T, bf16_t) || __is_same(T, f16_t)) {
           if (a.K % 2 == 0 && a.sk == 0 && (reinterpret_cast<uintptr_t>(a.out) & 3) == 0 &&
               (reinterpret_cast<uintptr_t>(a.src) & 3) == 0) {
+            ts_note_scatter_route(TS_ROUTE_SUM_ATOMIC);
             hipLaunchKernelGGL(scatter_add_pk16_kernel<T>, dim3(scatter_grid(n_edges, a.K / 2, kBlock, 1)),
                                dim3(kBlock), 0, stream, a);
             return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
           }
         }
+        ts_note_scatter_route(TS_ROUTE_SUM_ATOMIC);
         hipLaunchKernelGGL((scatter_atomic_kernel<T, 1, TS_SUM>), dim3(g), dim3(kBlock), 0, stream, a);
       } else {
         // products of the types that the accumulator table takes, one index per row: through the table from 2^16
@@ -1944,11 +1954,13 @@ int launch_scatter_v(const ScatterArgs &args, int reduce, hipStream_t stream) {
           if (a.lds_cache && a.sk == 0 && tm >= 64 && a.B * a.N < 0x7FFFFFFFll && n_src >= ((int64_t)1 << 16)) {
             const int64_t epb = per_cu_chunk_edges(a.lds_epb, n_edges, sum_table_min_chunk(a.K, 4),
                                                    131072 / a.K > 2048 ? 131072 / a.K : 2048);
+            ts_note_scatter_route(TS_ROUTE_MUL_TABLE);
             hipLaunchKernelGGL((scatter_add_lds_kernel<T, true>), dim3((unsigned)((n_edges + epb - 1) / epb)),
                                dim3(kLdsAddBlock), 0, stream, a, tm - 1, epb);
             return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
           }
         }
+        ts_note_scatter_route(TS_ROUTE_MUL_ATOMIC);
         hipLaunchKernelGGL((scatter_atomic_kernel<T, 1, TS_MUL>), dim3(g), dim3(kBlock), 0, stream, a);
       }
     }
@@ -1964,6 +1976,7 @@ int launch_scatter_v(const ScatterArgs &args, int reduce, hipStream_t stream) {
         // several entries per output slot: keys meet in LDS first (scatter_minmax_wide_lds_kernel)
         int tn = 1;
         while ((int64_t)tn * 2 * a.K <= kLdsAcc && tn * 2 <= kLdsAccRows) tn *= 2;
+        ts_note_scatter_route(TS_ROUTE_MINMAX_64BIT);
         const bool table = a.lds_cache && a.sk == 0 && tn >= 16 && a.B * a.N < 0x7FFFFFFFll &&
                            (a.lds_cache == 2 || (n_edges >= ((int64_t)1 << 17) && n_edges >= 4 * a.B * a.N));
         if (table) {
@@ -2013,6 +2026,7 @@ int launch_scatter_v(const ScatterArgs &args, int reduce, hipStream_t stream) {
             ((reinterpret_cast<uintptr_t>(a.src) | reinterpret_cast<uintptr_t>(a.index)) & 15) == 0) {
           const K1Plan kp = k1_plan(a.B, a.E, a.K, a.N, (int)sizeof(T), a.bin_ws, a.bin_ws_bytes, a.lds_cache == 2);
           if (kp.ok) {
+            ts_note_scatter_route(TS_ROUTE_MINMAX_K1_SLABS);
             if (is_max)
               launch_scatter_k1<T, true>(a, kp, stream);
             else
@@ -2029,6 +2043,8 @@ int launch_scatter_v(const ScatterArgs &args, int reduce, hipStream_t stream) {
         const BinPlan bp = bin_plan(a.B, a.E, a.K, a.N, (int)sizeof(T), a.bin_ws, a.bin_ws_bytes, a.bin_any_size != 0, 8,
                                     true);
         if (bp.ok && (bp.p.slices == 1 || bin_lane_shift(bp.p, VEC) >= 0)) {
+          ts_note_scatter_route(a.sorted_route && a.route_flag != nullptr ? TS_ROUTE_MINMAX_BUCKETS_OR_SEGMENTED
+                                                                          : TS_ROUTE_MINMAX_BUCKETS);
           if (is_max)
             launch_binned_keys<T, VEC, true>(a, bp.p, stream);
           else
@@ -2049,6 +2065,7 @@ int launch_scatter_v(const ScatterArgs &args, int reduce, hipStream_t stream) {
           const bool probe = a.skew_probe && a.lds_cache == 1 && a.K % VEC == 0 && a.bin_ws != nullptr &&
                              a.bin_ws_bytes >= 256 && ((uintptr_t)a.bin_ws & 3) == 0 &&
                              skew_probe_shape(a.B, a.E, a.K, a.N, (int)sizeof(T), a.skew_probe == 2);
+          ts_note_scatter_route(probe ? TS_ROUTE_MINMAX_RUNS_OR_TABLE : TS_ROUTE_MINMAX_RUNS);
           ScatterArgs ar = a, al = a;
           if (probe) {
             ar.skew_flag = al.skew_flag = static_cast<const int *>(a.bin_ws);
@@ -2083,6 +2100,7 @@ int launch_scatter_v(const ScatterArgs &args, int reduce, hipStream_t stream) {
         }
       }
       if (use_lds && a.K == 1 && n_src > 0 && a.lds_k1) {
+        ts_note_scatter_route(TS_ROUTE_MINMAX_TABLE_K1);
           const int64_t epb1 = per_cu_chunk_edges(a.lds_epb, n_edges, 16384, 131072);
         const unsigned g1 = (unsigned)((n_edges + epb1 - 1) / epb1);
         if (is_max) {
@@ -2096,6 +2114,7 @@ int launch_scatter_v(const ScatterArgs &args, int reduce, hipStream_t stream) {
         }
         return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
       }
+      ts_note_scatter_route(use_lds ? TS_ROUTE_MINMAX_TABLE : TS_ROUTE_MINMAX_ATOMIC);
       if (is_max) {
         hipLaunchKernelGGL((scatter_key_init_kernel<T, true>), dim3(g_out), dim3(kBlock), 0, stream, a);
         if (n_src > 0) {
