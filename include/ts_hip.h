@@ -263,6 +263,12 @@ enum ts_scatter_route {
   TS_ROUTE_MINMAX_BUCKETS_OR_SEGMENTED = 16, /* the same; an index found sorted: the segmented reduction */
   TS_ROUTE_MINMAX_64BIT = 17             /* 64-bit elements: value pass, then position pass */
 };
+/* Self-test of the fixed-pattern cross-lane helpers the kernels use (DPP row shifts, wave_shr:1,
+ * v_permlane16_swap / v_permlane32_swap: csrc/dpp.h): one wavefront applies each helper to x = 3 * lane + 1 and
+ * writes TS_LANE_OPS_ROWS rows of 64 int32 to out (device memory). tests/test_gpu_lane_ops.py holds the
+ * expected rows. No counterpart in the reference, whose kernels shuffle (csrc/cuda/utils.cuh:38-47). */
+#define TS_LANE_OPS_ROWS 17
+int ts_selftest_lane_ops(int32_t *out, ts_stream_t stream);
 int ts_scatter_last_route(void);
 const char *ts_scatter_route_name(int route);
 

@@ -21,7 +21,7 @@ DTYPE = {torch.float32: 0, torch.float64: 1, torch.float16: 2, torch.bfloat16: 3
          torch.int32: 4, torch.int64: 5, torch.int16: 6, torch.int8: 7, torch.uint8: 8}
 
 EXPORTS = (
-    "ts_error_string", "ts_hip_version", "ts_status_gave_up", "ts_scatter_last_route", "ts_scatter_route_name",
+    "ts_error_string", "ts_hip_version", "ts_status_gave_up", "ts_selftest_lane_ops", "ts_scatter_last_route", "ts_scatter_route_name",
     "ts_segment_csr_workspace_bytes", "ts_segment_csr", "ts_segment_csr_static", "ts_gather_csr",
     "ts_segment_mean_csr_backward",
     "ts_segment_coo_workspace_bytes", "ts_segment_coo", "ts_gather_coo",

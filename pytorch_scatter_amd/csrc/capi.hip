@@ -295,6 +295,39 @@ const char *ts_scatter_route_name(int route) {
   return route >= 0 && route < (int)(sizeof(names) / sizeof(names[0])) ? names[route] : "unknown";
 }
 
+namespace {
+// every fixed-pattern cross-lane helper of dpp.h applied to x = 3 * lane + 1, one row of 64 results each
+__global__ __launch_bounds__(kWave) void lane_ops_selftest_kernel(int32_t *out) {
+  const int lane = threadIdx.x;
+  const int x = 3 * lane + 1;
+  int row = 0;
+  out[64 * row++ + lane] = lane_up1(x);
+  out[64 * row++ + lane] = lane_xor<1>(x);
+  out[64 * row++ + lane] = lane_xor<2>(x);
+  out[64 * row++ + lane] = lane_xor<4>(x);
+  out[64 * row++ + lane] = lane_xor<8>(x);
+  out[64 * row++ + lane] = lane_xor<16>(x);
+  out[64 * row++ + lane] = lane_xor<32>(x);
+  out[64 * row++ + lane] = lane_down<1>(x);
+  out[64 * row++ + lane] = lane_down<2>(x);
+  out[64 * row++ + lane] = lane_down<4>(x);
+  out[64 * row++ + lane] = lane_down<8>(x);
+  out[64 * row++ + lane] = lane_down<16>(x);
+  out[64 * row++ + lane] = lane_down<32>(x);
+  out[64 * row++ + lane] = wave_inclusive_sum(x);
+  out[64 * row++ + lane] = (int)lane_up1_64(((int64_t)x << 32) | (uint32_t)(x + 7));
+  out[64 * row++ + lane] = (int)(lane_up1_64(((int64_t)x << 32) | (uint32_t)(x + 7)) >> 32);
+  float f = (float)x * 0.5f;
+  out[64 * row++ + lane] = (int)(lane_xor<16>(f) * 2.0f);
+}
+}  // namespace
+
+int ts_selftest_lane_ops(int32_t *out, ts_stream_t stream) {
+  if (!out) return TS_ERR_BAD_ARG;
+  hipLaunchKernelGGL(lane_ops_selftest_kernel, dim3(1), dim3(kWave), 0, static_cast<hipStream_t>(stream), out);
+  return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
+}
+
 int ts_status_gave_up(const unsigned long long *words) {
   return words != nullptr && words[0] != 0 && words[1] == words[0];
 }

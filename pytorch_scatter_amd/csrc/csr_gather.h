@@ -243,7 +243,7 @@ __global__ __launch_bounds__(kBlock) void csr_gather_small_kernel(CsrGatherArgs 
     __syncthreads();
     int m = 0;
     for (int w2 = 0; w2 < wave; ++w2) m = m > s_wtot[w2] ? m : s_wtot[w2];
-    const int up = __shfl_up(incl, 1);
+    const int up = lane_up1(incl);
     if (lane > 0) m = m > up ? m : up;
     for (int i = 0; i < chunk; ++i) {
       if (base + i < ne) {

@@ -143,10 +143,7 @@ __global__ __launch_bounds__(kBlock) void csr_reduce_small_kernel(CsrReduceArgs 
       int32_t arg = 0;
       for (int e = lo + lane; e < hi; e += kWave)
         reduce_step<A, REDUCE>(acc, arg, to_acc<T>(s_src[e * K + k]), (int32_t)(j0 + e));
-#pragma unroll
-      for (int off = kWave / 2; off >= 1; off >>= 1) {
-        const A oacc = __shfl_down(acc, off);
-        const int32_t oarg = __shfl_down(arg, off);
+      auto tree_step = [&](A oacc, int32_t oarg) {
         if (REDUCE == TS_SUM || REDUCE == TS_MEAN) {
           acc = acc + oacc;
         } else {
@@ -154,7 +151,15 @@ __global__ __launch_bounds__(kBlock) void csr_reduce_small_kernel(CsrReduceArgs 
           const bool better = (REDUCE == TS_MIN ? oacc < acc : oacc > acc) || (oacc == acc && oarg < arg);
           if (better) { acc = oacc; arg = oarg; }
         }
-      }
+      };
+      // lane i takes lane i + 32, 16, ... 1 (row shifts and row / half swaps in the vector ALU): lane 0 ends with
+      // the row's result
+      tree_step(lane_down_any<32>(acc), lane_down<32>(arg));
+      tree_step(lane_down_any<16>(acc), lane_down<16>(arg));
+      tree_step(lane_down_any<8>(acc), lane_down<8>(arg));
+      tree_step(lane_down_any<4>(acc), lane_down<4>(arg));
+      tree_step(lane_down_any<2>(acc), lane_down<2>(arg));
+      tree_step(lane_down_any<1>(acc), lane_down<1>(arg));
       if (lane == 0) deliver(r, k, kind, acc, arg);
     }
   }

@@ -6,6 +6,7 @@
 #include <stdint.h>
 
 #include "../../include/ts_hip.h"
+#include "dpp.h"
 
 namespace ts {
 

@@ -165,8 +165,8 @@ __device__ __forceinline__ void fused_find_runs(const int64_t *idx, int64_t se, 
 #pragma unroll
   for (int q = 0; q < EPL; ++q) {
     const int e = tid + q * kBlock;
-    const int lo32 = __shfl_up((int)(uint32_t)id[q], 1), hi32 = __shfl_up((int)(id[q] >> 32), 1);
-    const int64_t prev = lane == 0 ? edge[q] : (int64_t)(((uint64_t)(uint32_t)hi32 << 32) | (uint32_t)lo32);
+    const int64_t up = lane_up1_64(id[q]);  // by every lane, lane 0 included: its value is what lane 1 reads
+    const int64_t prev = lane == 0 ? edge[q] : up;
     if (e < ne) {
       const bool have_prev = j0 + e > 0;
       const bool head = e == 0 || id[q] != prev;
@@ -257,12 +257,7 @@ __global__ __launch_bounds__(kBlock, 4) void group_fused_kernel(GroupArgs g, Fus
   if (lane_leaves) s_info[1] = 1;
   if (badmask != 0) s_info[5] = 1;
   const int heads = __popc(headmask);
-  int incl = heads;
-#pragma unroll
-  for (int off = 1; off < kWave; off <<= 1) {
-    const int v = __shfl_up(incl, off);
-    if (lane >= off) incl += v;
-  }
+  const int incl = wave_inclusive_sum(heads);
   if (lane == kWave - 1) s_wsum[wave] = incl;
   if (__ballot(descent) != 0 && lane == 0) s_info[3] = 1;
   __syncthreads();
@@ -348,10 +343,8 @@ __global__ __launch_bounds__(kBlock, 4) void group_fused_kernel(GroupArgs g, Fus
 #pragma unroll
         for (int v = 0; v < CV; ++v) top[v] = max_acc(top[v], to_acc<T>(x.v[v]));
       }
-      for (int off = step / 2; off >= 1; off >>= 1) {
 #pragma unroll
-        for (int v = 0; v < CV; ++v) top[v] = max_acc(top[v], __shfl_xor(top[v], off));
-      }
+      for (int v = 0; v < CV; ++v) top[v] = group_butterfly(top[v], step, [](F p, F q) { return max_acc(p, q); });
       const bool frag_in = r == 0 && enters, frag_out = r == nruns - 1 && leaves;
       if ((frag_in || frag_out) && first == 0) {
 #pragma unroll
@@ -372,10 +365,8 @@ __global__ __launch_bounds__(kBlock, 4) void group_fused_kernel(GroupArgs g, Fus
 #pragma unroll
         for (int v = 0; v < CV; ++v) s[v] += to_acc<T>(x.v[v]);
       }
-      for (int off = step / 2; off >= 1; off >>= 1) {
 #pragma unroll
-        for (int v = 0; v < CV; ++v) s[v] += __shfl_xor(s[v], off);
-      }
+      for (int v = 0; v < CV; ++v) s[v] = group_butterfly(s[v], step, [](F p, F q) { return p + q; });
       const bool frag_in = r == 0 && enters, frag_out = r == nruns - 1 && leaves;
       if (frag_in || frag_out) {
         if (first == 0) {
@@ -474,10 +465,8 @@ __global__ __launch_bounds__(kBlock, 4) void group_fused_kernel(GroupArgs g, Fus
         for (int v = 0; v < CV; ++v)
           s[v] += MODE == GS_SOFTMAX_BWD ? to_acc<T>(y.v[v]) * to_acc<T>(gr.v[v]) : to_acc<T>(gr.v[v]);
       }
-      for (int off = step / 2; off >= 1; off >>= 1) {
 #pragma unroll
-        for (int v = 0; v < CV; ++v) s[v] += __shfl_xor(s[v], off);
-      }
+      for (int v = 0; v < CV; ++v) s[v] = group_butterfly(s[v], step, [](F p, F q) { return p + q; });
       if (frag_in || frag_out) {
         if (first == 0) {
 #pragma unroll

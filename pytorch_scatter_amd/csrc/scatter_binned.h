@@ -222,9 +222,8 @@ __device__ __forceinline__ void bin_buckets(const ScatterArgs &a, const BinArgs 
 #pragma unroll
     for (int j = 0; j < kBinPer; ++j) {
       const int elo = __shfl((int)(uint32_t)edge, j), ehi = __shfl((int)(edge >> 32), j);
-      const int lo32 = __shfl_up((int)(uint32_t)node[j], 1), hi32 = __shfl_up((int)(node[j] >> 32), 1);
-      const int64_t prev = lane == 0 ? (int64_t)(((uint64_t)(uint32_t)ehi << 32) | (uint32_t)elo)
-                                     : (int64_t)(((uint64_t)(uint32_t)hi32 << 32) | (uint32_t)lo32);
+      const int64_t up = lane_up1_64(node[j]);  // by every lane: lane 0's value is what lane 1 reads
+      const int64_t prev = lane == 0 ? (int64_t)(((uint64_t)(uint32_t)ehi << 32) | (uint32_t)elo) : up;
       descent = descent || (node[j] >= 0 && prev >= 0 && node[j] < prev);
       if (strict && node[j] < 0 && lo + threadIdx.x + (int64_t)j * kBinPlaceBlock < hi) descent = true;
     }
@@ -329,9 +328,8 @@ static __global__ __launch_bounds__(kBinPlaceBlock) __attribute__((amdgpu_num_sg
 #pragma unroll
       for (int j = 0; j < kBinCountPer; ++j) {
         const int elo = __shfl((int)(uint32_t)edge, j), ehi = __shfl((int)(edge >> 32), j);
-        const int lo32 = __shfl_up((int)(uint32_t)node[j], 1), hi32 = __shfl_up((int)(node[j] >> 32), 1);
-        const int64_t prev = lane == 0 ? (int64_t)(((uint64_t)(uint32_t)ehi << 32) | (uint32_t)elo)
-                                       : (int64_t)(((uint64_t)(uint32_t)hi32 << 32) | (uint32_t)lo32);
+        const int64_t up = lane_up1_64(node[j]);  // by every lane: lane 0's value is what lane 1 reads
+      const int64_t prev = lane == 0 ? (int64_t)(((uint64_t)(uint32_t)ehi << 32) | (uint32_t)elo) : up;
         descent = descent || (node[j] >= 0 && prev >= 0 && node[j] < prev);
         if (strict && node[j] < 0 && b0 + threadIdx.x + (int64_t)j * kBinPlaceBlock < hi) descent = true;
       }

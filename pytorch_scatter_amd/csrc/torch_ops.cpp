@@ -10,6 +10,7 @@
 
 #include <c10/core/DeviceGuard.h>
 #include <c10/hip/HIPStream.h>
+#include <hip/hip_runtime_api.h>
 
 #include <map>
 #include <mutex>
@@ -97,12 +98,16 @@ std::optional<int64_t> collapsed_stride(const Tensor &t, int64_t lo, int64_t hi)
 // Opt-in check of a segment reduction's status words (TS_CHECK_STATUS=1 in the environment, read once): copies
 // the 16 bytes back, which waits for the stream, and raises if the call gave a row up (row pointers that are
 // not monotone, an index that is not sorted). Off by default: the operators never synchronise on their own.
+// (never while the current stream is being captured into a graph: a copy to the host is not allowed there)
 bool status_checks_on() {
   static const bool on = [] {
     const char *e = getenv("TS_CHECK_STATUS");
     return e != nullptr && atoi(e) != 0;
   }();
-  return on;
+  if (!on) return false;
+  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(c10::hip::getCurrentHIPStream().stream(), &capture) != hipSuccess) return false;
+  return capture == hipStreamCaptureStatusNone;
 }
 void maybe_check_status_words(const Tensor &ws, size_t ws_bytes, const char *what) {
   if (!status_checks_on() || ws_bytes < TS_STATUS_BYTES || (size_t)ws.numel() < ws_bytes) return;
