@@ -280,6 +280,15 @@ int ts_scatter_count(const int64_t *index, int32_t *count, int64_t B, int64_t E,
                      int64_t N, int64_t index_stride_b, int64_t index_stride_e,
                      ts_stream_t stream);
 
+/* The same count with scratch memory (ts_scatter_count_workspace_bytes; 0 = no use for it): from 2 M entries on an
+ * unsorted index is binned by bucket of output rows (8 bytes per entry) and counted in LDS, as
+ * ts_scatter_with_workspace does for the sum of one value per entry. Same result. */
+size_t ts_scatter_count_workspace_bytes(int64_t B, int64_t E, int64_t N);
+int ts_scatter_count_with_workspace(const int64_t *index, int32_t *count, int64_t B,
+                                    int64_t E, int64_t N, int64_t index_stride_b,
+                                    int64_t index_stride_e, void *workspace,
+                                    size_t workspace_bytes, ts_stream_t stream);
+
 /* out[b, n, k] = out[b, n, k] / (T)max(count[b, n], 1): true division for
  * floating types, floor division for integers (csrc/scatter.cpp:138-141). */
 int ts_divide_by_count(void *out, const int32_t *count, int64_t B, int64_t N,

@@ -26,7 +26,7 @@ EXPORTS = (
     "ts_segment_mean_csr_backward",
     "ts_segment_coo_workspace_bytes", "ts_segment_coo", "ts_gather_coo",
     "ts_segment_mean_coo_backward",
-    "ts_scatter", "ts_scatter_workspace_bytes", "ts_scatter_workspace_zero_bytes", "ts_scatter_with_workspace", "ts_scatter_count", "ts_divide_by_count", "ts_arg_backward",
+    "ts_scatter", "ts_scatter_workspace_bytes", "ts_scatter_workspace_zero_bytes", "ts_scatter_with_workspace", "ts_scatter_count", "ts_scatter_count_workspace_bytes", "ts_scatter_count_with_workspace", "ts_divide_by_count", "ts_arg_backward",
     "ts_group_softmax_workspace_bytes", "ts_group_softmax", "ts_group_softmax_backward",
     "ts_group_logsumexp", "ts_group_logsumexp_backward",
     "ts_group_std", "ts_group_std_backward",
@@ -58,6 +58,7 @@ def lib() -> ctypes.CDLL:
         _lib.ts_indptr_to_index_workspace_bytes.restype = ctypes.c_size_t
         _lib.ts_scatter_workspace_bytes.restype = ctypes.c_size_t
         _lib.ts_scatter_workspace_zero_bytes.restype = ctypes.c_size_t
+        _lib.ts_scatter_count_workspace_bytes.restype = ctypes.c_size_t
         _lib.ts_sort_index_workspace_bytes.restype = ctypes.c_size_t
         _lib.ts_segment_csr_permuted_workspace_bytes.restype = ctypes.c_size_t
     return _lib
@@ -218,6 +219,17 @@ def scatter_count(index, count, B, E, N, sb, se):
     with torch.cuda.device(count.device):
         _check(lib().ts_scatter_count(_p(index), _p(count), _i(B), _i(E), _i(N), _i(sb), _i(se),
                                       _stream(count)))
+
+
+def scatter_count_with_workspace(index, count, B, E, N, sb, se):
+    _dev(index, count)
+    L = lib()
+    nbytes = L.ts_scatter_count_workspace_bytes(_i(B), _i(E), _i(N))
+    ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=count.device)
+    with torch.cuda.device(count.device):
+        _check(L.ts_scatter_count_with_workspace(_p(index), _p(count), _i(B), _i(E), _i(N), _i(sb), _i(se),
+                                                 _p(ws) if nbytes else None, ctypes.c_size_t(nbytes), _stream(count)))
+    return nbytes
 
 
 def divide_by_count(out, count, B, N, K):

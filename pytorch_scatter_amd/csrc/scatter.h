@@ -1830,6 +1830,13 @@ int launch_scatter_v(const ScatterArgs &args, int reduce, hipStream_t stream) {
         bp = bin_plan(a.B, a.E, a.K, a.N, (int)sizeof(T), a.bin_ws, a.bin_ws_bytes, a.bin_any_size != 0,
                       (int)sizeof(typename BinSlot<T>::type), false, true);
         lshift = bp.ok ? bin_lane_shift(bp.p, VEC) : -1;
+        if constexpr (sizeof(T) == 4 && VEC == 1) {
+          // one 4-byte value per entry: the value travels in the binned word (bin_plan_payload)
+          if (!bp.ok && a.K == 1 && a.lds_cache) {
+            bp = bin_plan_payload(a.B, a.E, a.K, a.N, (int)sizeof(T), a.bin_ws, a.bin_ws_bytes, a.bin_any_size != 0);
+            lshift = bp.ok ? 0 : -1;
+          }
+        }
       }
     }
     const bool routed = lshift >= 0 && a.sorted_route && a.route_flag != nullptr && !a.out_given;
@@ -1895,7 +1902,7 @@ int launch_scatter_v(const ScatterArgs &args, int reduce, hipStream_t stream) {
             }
             const int64_t epb = per_cu_chunk_edges(a.lds_epb, n_edges, sum_table_min_chunk(a.K, (int)sizeof(T)),
                                                    131072 / a.K > 2048 ? 131072 / a.K : 2048);
-            ts_note_scatter_route(sampled ? TS_ROUTE_SUM_TABLE_OR_RUNS : TS_ROUTE_SUM_TABLE);
+            if (lshift < 0) ts_note_scatter_route(sampled ? TS_ROUTE_SUM_TABLE_OR_RUNS : TS_ROUTE_SUM_TABLE);
             hipLaunchKernelGGL(scatter_add_lds_kernel<T>, dim3((unsigned)((n_edges + epb - 1) / epb)),
                                dim3(kLdsAddBlock), 0, stream, t, tn - 1, epb);
             if (!sampled) return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;

@@ -57,6 +57,8 @@ struct BinArgs {
                            // sorted index to the segmented reduction needs both)
   int sampled = 0;         // sum only: *unsorted was set before the count pass from a sample of the index
                            // (bin_sample_kernel); then the count pass returns at once as well
+  int payload = 0;         // sum of one 4-byte value per entry: the low half of a binned word holds the value's bits
+                           // instead of the entry number, so the reducing pass never goes back to src
 };
 
 struct BinPlan {
@@ -185,6 +187,75 @@ inline BinPlan bin_plan(int64_t B, int64_t E, int64_t K, int64_t N, int elem_byt
   return r;
 }
 
+// Sums of ONE 4-byte value per entry (K == 1: degrees, edge weights, attention scores) under an unsorted index.
+// The kernels without workspace pay one device atomic per entry that misses their LDS table (about 21 G entries/s
+// whatever is done: 46 M entries onto 1 M rows 2.2 ms). Here the value travels with its bucket: the place pass writes
+// (row in bucket, value) words, and the reducing pass streams the words of a bucket's chunk, adds them in an LDS
+// table of the bucket's rows and adds every touched row to out once per chunk. Traffic per entry: 8 bytes of index
+// twice, 4 of src, 8 written and 8 read again, against one scattered atomic. Buckets are small (64 ... 4096 rows,
+// at most a sixteenth of a chunk) so that the write-back stays below a sixteenth of the entries.
+inline BinPlan bin_plan_payload(int64_t B, int64_t E, int64_t K, int64_t N, int elem_bytes, void *ws, size_t ws_bytes,
+                                bool any_size = false) {
+  BinPlan r;
+  r.ok = false;
+  r.bytes = 0;
+  const int64_t n_edges = B * E, rows = B * N;
+  if (K != 1 || elem_bytes != 4 || n_edges >= 0xFFFFFFFEll || rows >= 0x7FFFFFFFll || rows < 1) return r;
+  if (!any_size && n_edges < ((int64_t)1 << 21)) return r;   // below: the table kernel's launches are the call
+  // chunk: entries per reducing workgroup, about 1024 workgroups, 2048 ... 65536 entries
+  int64_t chunk = (n_edges / 1024 + 1023) & ~(int64_t)1023;
+  if (chunk < 2048) chunk = 2048;
+  if (chunk > 65536) chunk = 65536;
+  if (const char *env = getenv("TS_BIN_CHUNK")) chunk = atoi(env) > 0 ? atoi(env) : chunk;  // tuning aid
+  // rows per bucket: as many as the table holds (4096). Fewer, larger buckets make the place pass cheaper (21 M entries:
+  // 256 rows 580 us, 1024 rows 494, 4096 rows 393 for the whole call), which outweighs the longer write-back per chunk.
+  int rshift = 12;
+  if (const char *env = getenv("TS_BIN_PAYLOAD_RSHIFT")) rshift = atoi(env);  // tuning aid
+  while (rshift < 12 && ((rows + ((int64_t)1 << rshift) - 1) >> rshift) > kBinMaxBuckets) ++rshift;
+  if (rshift > 12) rshift = 12;
+  const int64_t nb = (rows + ((int64_t)1 << rshift) - 1) >> rshift;
+  if (nb > kBinMaxBuckets) return r;                       // more output rows than 16384 buckets of 4096 hold
+  if (!any_size && n_edges < 2 * nb * 64) return r;        // nearly empty buckets: every one still costs its share
+  BinArgs &p = r.p;
+  p.rshift = rshift;
+  p.kc = 1;
+  p.slices = 1;
+  p.nb = (int)nb;
+  p.payload = 1;
+  {
+    const int64_t rounds = (n_edges + (int64_t)512 * kBinPlaceChunk - 1) / ((int64_t)512 * kBinPlaceChunk);
+    int64_t tile = (((n_edges + 512 * rounds - 1) / (512 * rounds)) + kBinPlaceBlock - 1) & ~(int64_t)(kBinPlaceBlock - 1);
+    if (tile < kBinPlaceBlock) tile = kBinPlaceBlock;
+    if (tile > kBinPlaceChunk) tile = kBinPlaceChunk;
+    p.place_tile = (int)tile;
+    p.n_place = (n_edges + tile - 1) / tile;
+  }
+  p.chunk = (int)chunk;
+  p.max_wgs = n_edges / chunk + nb + 1;
+  auto up = [](size_t x) { return (x + 255) & ~(size_t)255; };
+  size_t off = 0;
+  auto take = [&](size_t bytes) { const size_t o = off; off += up(bytes); return o; };
+  const size_t o_tot = take((size_t)nb * 8), o_cur = take((size_t)nb * 8), o_st = take((size_t)(nb + 1) * 8);
+  const size_t o_cs = take((size_t)(nb + 1) * 4), o_wb = take((size_t)p.max_wgs * 4);
+  const size_t o_bin = take((size_t)n_edges * 8), o_flag = take(256);
+  r.bytes = off;
+  if (ws == nullptr || ws_bytes < off || (reinterpret_cast<uintptr_t>(ws) & 15) != 0) return r;
+  char *base = static_cast<char *>(ws);
+  p.totals = reinterpret_cast<unsigned long long *>(base + o_tot);
+  p.cursor = reinterpret_cast<unsigned long long *>(base + o_cur);
+  p.starts = reinterpret_cast<int64_t *>(base + o_st);
+  p.chunk_start = reinterpret_cast<int32_t *>(base + o_cs);
+  p.wg_bucket = reinterpret_cast<int32_t *>(base + o_wb);
+  p.binned = reinterpret_cast<uint64_t *>(base + o_bin);
+  p.unsorted = reinterpret_cast<int *>(base + o_flag);
+  p.slab_start = nullptr;
+  p.comb_list = nullptr;
+  p.comb_count = nullptr;
+  p.slabs = nullptr;
+  r.ok = true;
+  return r;
+}
+
 // node (b * N + index) of entry be, -1 for an index outside [0, N)
 __device__ __forceinline__ int64_t bin_node(const ScatterArgs &a, int64_t be) {
   int64_t b = 0, e = be;
@@ -196,6 +267,14 @@ __device__ __forceinline__ int64_t bin_node(const ScatterArgs &a, int64_t be) {
 constexpr int kBinPer = 10;  // entries per lane in place (all index loads in flight; three words per entry stay in
                              // registers: with 16 the kernel needs 91 VGPRs, which is one workgroup per CU instead of two)
 constexpr int kBinBatch = kBinPer * kBinPlaceBlock;
+
+// total of the per-wavefront sums of a workgroup scan (valid entries of a tile)
+__device__ __forceinline__ int run_total(const int32_t *wsum) {
+  int t = 0;
+#pragma unroll
+  for (int w = 0; w < kBinPlaceBlock / kWave; ++w) t += wsum[w];
+  return t;
+}
 
 // buckets of the kBinPer entries of a lane, all index loads in flight at once; -1: no bucket
 // check: descent is set when an entry's node lies below that of the entry before it. The entry before is the
@@ -514,10 +593,83 @@ static __global__ __launch_bounds__(kBinPlaceBlock) void bin_place_kernel(Scatte
   for (int j = 0; j < kBinPer; ++j) {
     if (bucket[j] < 0) continue;
     const int64_t be = lo + threadIdx.x + (int64_t)j * kBinPlaceBlock;
-    p.binned[s_base[bucket[j]] + (uint32_t)rank[j]] = ((uint64_t)(uint32_t)local[j] << 32) | (uint32_t)be;
+    // (payload: one 4-byte value per entry, K == 1, so entry be of the flattened [B, E] is element be of src)
+    const uint32_t low = (p.payload && a.src != nullptr) ? static_cast<const uint32_t *>(a.src)[be]
+                                                         : (p.payload ? 1u : (uint32_t)be);  // no src: a count of ones
+    p.binned[s_base[bucket[j]] + (uint32_t)rank[j]] = ((uint64_t)(uint32_t)local[j] << 32) | low;
   }
 }
 static_assert(kBinPlaceChunk == kBinBatch, "the place pass holds a workgroup's entries in registers: one batch");
+
+// The place pass for (row in bucket, value) words under an index in no particular order. With every lane of a
+// wavefront bound for another bucket the 8-byte stores of bin_place_kernel each open a memory line of their own
+// (21 M entries of a uniform index over 358 buckets: 290 us, and 111 us with the same words stored in entry order).
+// Here the tile is sorted by bucket in LDS first -- the ranks give every entry its place behind the tile's
+// exclusive prefix over the buckets -- and written out in that order: neighbouring lanes, neighbouring words of one
+// bucket's run. A staged word carries its bucket in bits 44 and up (the row in the bucket needs 12 bits at most), so
+// the lane that writes it finds the run's base. Tiles of kBinSortTile entries, at most kBinSortBuckets buckets: 64 KB
+// of LDS, two workgroups per CU.
+constexpr int kBinSortTile = 6144;
+constexpr int kBinSortBuckets = 2048;
+static __global__ __launch_bounds__(kBinPlaceBlock) void bin_place_sorted_kernel(ScatterArgs a, BinArgs p) {
+  __shared__ uint64_t s_stage[kBinSortTile];
+  __shared__ int32_t s_cnt[kBinSortBuckets];   // counts, then the tile's exclusive prefix
+  __shared__ uint32_t s_base[kBinSortBuckets];  // first word of the tile's run in every bucket
+  __shared__ int32_t s_wsum[kBinPlaceBlock / kWave];
+  if (p.unsorted != nullptr && *p.unsorted == 0) return;
+  for (int i = threadIdx.x; i < p.nb; i += kBinPlaceBlock) s_cnt[i] = 0;
+  __syncthreads();
+  const int64_t lo = (int64_t)blockIdx.x * kBinSortTile;
+  const int64_t hi = lo + kBinSortTile < a.B * a.E ? lo + kBinSortTile : a.B * a.E;
+  int32_t bucket[kBinPer], local[kBinPer], rank[kBinPer];
+  bool unused = false;
+  bin_buckets(a, p, lo, hi, bucket, local, false, unused);
+#pragma unroll
+  for (int j = 0; j < kBinPer; ++j) rank[j] = bin_take(s_cnt, bucket[j]);
+  __syncthreads();
+  // reserve the tile's runs, then turn the counts into the tile's exclusive prefix: every lane owns `per`
+  // neighbouring buckets
+  const int per = (p.nb + kBinPlaceBlock - 1) / kBinPlaceBlock;
+  const int b0 = threadIdx.x * per;
+  int32_t mine = 0;
+  for (int j = 0; j < per; ++j) {
+    const int i = b0 + j;
+    if (i >= p.nb) break;
+    const int32_t h = s_cnt[i];
+    if (h != 0) s_base[i] = (uint32_t)atomicAdd(&p.cursor[i], (unsigned long long)h);
+    mine += h;
+  }
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  const int32_t incl = wave_inclusive_sum(mine);
+  if (lane == kWave - 1) s_wsum[wave] = incl;
+  __syncthreads();
+  int32_t run = incl - mine;
+  for (int w2 = 0; w2 < wave; ++w2) run += s_wsum[w2];
+  for (int j = 0; j < per; ++j) {
+    const int i = b0 + j;
+    if (i >= p.nb) break;
+    const int32_t h = s_cnt[i];
+    s_cnt[i] = run;
+    run += h;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int j = 0; j < kBinPer; ++j) {
+    if (bucket[j] < 0) continue;
+    const int64_t be = lo + threadIdx.x + (int64_t)j * kBinPlaceBlock;
+    const uint32_t low = (p.payload && a.src != nullptr) ? static_cast<const uint32_t *>(a.src)[be]
+                                                         : (p.payload ? 1u : (uint32_t)be);
+    s_stage[s_cnt[bucket[j]] + rank[j]] =
+        ((uint64_t)(uint32_t)bucket[j] << 44) | ((uint64_t)(uint32_t)local[j] << 32) | low;
+  }
+  __syncthreads();
+  const int total = run_total(s_wsum);  // the tile's entries with an index inside [0, N)
+  for (int pos = threadIdx.x; pos < total; pos += kBinPlaceBlock) {
+    const uint64_t w = s_stage[pos];
+    const uint32_t b = (uint32_t)(w >> 44);
+    p.binned[s_base[b] + (uint32_t)(pos - s_cnt[b])] = w & (((uint64_t)1 << 44) - 1);
+  }
+}
 
 // One finished packed key -> out / arg_out (element i of [B, N, K]): what scatter_key_init_kernel and
 // scatter_key_final_kernel do for the kernels that keep their keys in arg_out. key == 0: no entry.
@@ -887,6 +1039,65 @@ __global__ __launch_bounds__(kBinBlock) void bin_add_wave_kernel(ScatterArgs a, 
   }
 }
 
+// Sum of one 4-byte value per entry from (row in bucket, value) words: see bin_plan_payload. A workgroup streams
+// its chunk of a bucket with 16-byte loads (two words per lane, four loads in flight), adds into the bucket's table
+// in LDS (double slots for floats: ds_add_f64 keeps its rate when many lanes meet on one address, a hub row) and
+// adds every row it touched to out once.
+template <typename T>
+__global__ __launch_bounds__(kBinBlock) void bin_add_payload_kernel(ScatterArgs a, BinArgs p) {
+  static_assert(sizeof(T) == 4, "one 4-byte value per word");
+  typedef typename BinSlot<T>::type A;
+  typedef unsigned long long u64x2 __attribute__((ext_vector_type(2)));
+  constexpr int U = 4;
+  __shared__ A s_acc[4096];
+  if (p.unsorted != nullptr && *p.unsorted == 0) return;
+  const int wg = (int)blockIdx.x;
+  const int bucket = p.wg_bucket[wg];
+  if (bucket < 0) return;
+  const int rows = 1 << p.rshift;
+  for (int i = threadIdx.x; i < rows; i += kBinBlock) s_acc[i] = (A)0;
+  __syncthreads();
+  const int64_t lo = p.starts[bucket] + ((int64_t)wg - p.chunk_start[bucket]) * p.chunk;
+  int64_t hi = lo + p.chunk;
+  if (hi > p.starts[bucket + 1]) hi = p.starts[bucket + 1];
+  auto add = [&](unsigned long long w) {
+    T v;
+    const uint32_t bits = (uint32_t)w;
+    __builtin_memcpy(&v, &bits, 4);
+    __hip_atomic_fetch_add(&s_acc[(uint32_t)(w >> 32) & (uint32_t)(rows - 1)], (A)v, __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_WORKGROUP);
+  };
+  if (lo < hi) {
+    // words lo .. hi - 1; the 16-byte loads start at an even word
+    const int64_t first = lo & ~(int64_t)1;
+    const u64x2 *pairs = reinterpret_cast<const u64x2 *>(p.binned + first);
+    const int64_t n_pairs = (hi - first + 1) >> 1;  // the last pair may reach one word past hi: inside the array or its padding
+    for (int64_t base = 0; base < n_pairs; base += (int64_t)U * kBinBlock) {
+      u64x2 w[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int64_t i = base + (int64_t)u * kBinBlock + threadIdx.x;
+        w[u] = __builtin_nontemporal_load(pairs + (i < n_pairs ? i : n_pairs - 1));
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int64_t i = base + (int64_t)u * kBinBlock + threadIdx.x;
+        if (i >= n_pairs) continue;
+        const int64_t e0 = first + 2 * i;
+        if (e0 >= lo) add(w[u].x);
+        if (e0 + 1 < hi) add(w[u].y);
+      }
+    }
+  }
+  __syncthreads();
+  T *out = static_cast<T *>(a.out) + ((int64_t)bucket << p.rshift);
+  const int64_t rows_left = a.B * a.N - ((int64_t)bucket << p.rshift);  // rows that exist
+  for (int i = threadIdx.x; i < rows && i < rows_left; i += kBinBlock) {
+    const A v = s_acc[i];
+    if (v != (A)0) atomic_add_elem<T>(out + i, (T)v);
+  }
+}
+
 // the count pass: equal shares of the entries for at most kBinCountGroups workgroups
 inline void launch_bin_count(const ScatterArgs &a, const BinArgs &p, hipStream_t stream) {
   int64_t groups = (a.B * a.E + kBinCountBatch - 1) / kBinCountBatch;
@@ -960,10 +1171,19 @@ void launch_binned_add(const ScatterArgs &a, const BinArgs &plan, int lshift, hi
     hipLaunchKernelGGL(bin_zero_out_kernel<T>, dim3(grid_for(zero_out)), dim3(kBlock), 0, stream, static_cast<T *>(a.out),
                        zero_out, p.unsorted);
   hipLaunchKernelGGL(bin_scan_kernel, dim3(1), dim3(kBinBlock), 0, stream, p);
-  if (p.nb <= kBinSmallCap)  // 64 KB of cursors, two workgroups per CU; above: 128 KB, one
+  if (p.payload && p.nb <= kBinSortBuckets && !getenv("TS_BIN_NO_SORTED_PLACE"))  // env: tuning aid
+    hipLaunchKernelGGL(bin_place_sorted_kernel, dim3((unsigned)((a.B * a.E + kBinSortTile - 1) / kBinSortTile)),
+                       dim3(kBinPlaceBlock), 0, stream, a, p);
+  else if (p.nb <= kBinSmallCap)  // 64 KB of cursors, two workgroups per CU; above: 128 KB, one
     hipLaunchKernelGGL(bin_place_kernel<kBinSmallCap>, dim3((unsigned)p.n_place), dim3(kBinPlaceBlock), 0, stream, a, p);
   else
     hipLaunchKernelGGL(bin_place_kernel<kBinMaxBuckets>, dim3((unsigned)p.n_place), dim3(kBinPlaceBlock), 0, stream, a, p);
+  if constexpr (sizeof(T) == 4 && VEC == 1) {
+    if (p.payload) {
+      hipLaunchKernelGGL(bin_add_payload_kernel<T>, dim3((unsigned)p.max_wgs), dim3(kBinBlock), 0, stream, a, p);
+      return;
+    }
+  }
   hipLaunchKernelGGL((bin_add_wave_kernel<T, VEC>), dim3((unsigned)(p.max_wgs * p.slices)), dim3(kBinBlock), 0, stream, a, p,
                      lshift);
 }

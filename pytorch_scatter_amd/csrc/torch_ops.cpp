@@ -591,8 +591,11 @@ template <int REDUCE> struct ScatterFn : public torch::autograd::Function<Scatte
         // one index row shared by every batch row (an expanded view): counted once and repeated
         const int64_t Bc = (bi.batch_stride == 0 && B > 1) ? 1 : B;
         Tensor count_f = at::empty({Bc * N}, src.options().dtype(at::kInt));
-        check_status(ts_scatter_count(bi.t.data_ptr<int64_t>(), count_f.data_ptr<int32_t>(), Bc, E, N, bi.batch_stride, 1,
-                                      stream_of(src)),
+        const size_t cws_bytes = ts_scatter_count_workspace_bytes(Bc, E, N);
+        Tensor cws = workspace(cws_bytes, src);
+        check_status(ts_scatter_count_with_workspace(bi.t.data_ptr<int64_t>(), count_f.data_ptr<int32_t>(), Bc, E, N,
+                                                     bi.batch_stride, 1, cws_bytes > 0 ? cws.data_ptr() : nullptr,
+                                                     cws_bytes, stream_of(src)),
                      "scatter_mean count");
         if (Bc != B) count_f = count_f.view({1, N}).expand({B, N}).contiguous().view({B * N});
         Tensor out_c = out.contiguous();

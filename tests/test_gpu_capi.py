@@ -1688,3 +1688,74 @@ def test_scatter_k1_reports_a_wait_that_ran_out(capi, oracle, reduce, monkeypatc
         assert exact or flagged, "a result that lost entries must be flagged"
         if must_be_clean:
             assert exact and not flagged
+
+
+PAYLOAD_CASES = [
+    # B, E, N, index: sums and counts of one 4-byte value per entry through (row in bucket, value) words
+    (1, 30001, 500, "uniform"), (1, 50003, 20000, "zipf"), (1, 70000, 300000, "uniform"), (2, 9001, 7, "zipf"),
+    (3, 40000, 9000, "uniform"), (1, 3, 10, "uniform"), (1, 120000, 100000, "hub"), (1, 65536, 4096, "uniform"),
+    (1, 100000, 9_000_000, "uniform"),   # more buckets than the sorting place pass takes
+]
+
+
+@pytest.mark.parametrize("case,dtype,out_given", product(PAYLOAD_CASES, [torch.float32, torch.int32], [False, True]))
+def test_scatter_sum_of_single_values_through_buckets(capi, oracle, case, dtype, out_given, monkeypatch):
+    """Forced on at small sizes (TS_SCATTER_BINNED=2). Indices outside [0, N), a hub row, an odd number of entries,
+    several batch rows, `out` given (the sums are added on top), an output with more rows than entries."""
+    monkeypatch.setenv("TS_SCATTER_BINNED", "2")
+    B, E, N, kind = case
+    rng = np.random.default_rng(E + N)
+    if dtype.is_floating_point:
+        src = torch.from_numpy(rng.standard_normal(size=(B, E, 1)).astype(np.float32))
+    else:
+        src = torch.from_numpy(rng.integers(-1000, 1000, size=(B, E, 1)).astype(np.int32))
+    if kind == "zipf":
+        p = np.arange(1, N + 1, dtype=np.float64) ** -1.2
+        index = (rng.choice(N, size=(B, E), p=p / p.sum()) * 7919) % N
+    elif kind == "hub":
+        index = rng.integers(0, N, size=(B, E))
+        index[:, rng.random(E) < 0.4] = N // 3
+    else:
+        index = rng.integers(0, N, size=(B, E))
+    index = torch.from_numpy(index.astype(np.int64))
+    if E > 100:
+        index[0, 5] = -1
+        index[-1, 77] = N
+    valid = (index >= 0) & (index < N)
+    prev = torch.from_numpy(rng.integers(-5, 6, size=(B, N, 1))).to(dtype) if out_given else torch.zeros((B, N, 1), dtype=dtype)
+    want = prev.clone().double()
+    for b in range(B):
+        want[b, :, 0].index_add_(0, index[b][valid[b]], src[b, valid[b], 0].double())
+    nbytes = capi.lib().ts_scatter_workspace_bytes(capi._i(B), capi._i(E), capi._i(1), capi._i(N), capi.DTYPE[dtype], capi.SUM)
+    assert nbytes >= 8 * B * E, "the plan for single values asks for 8 bytes of scratch per entry"
+    out = prev.clone().to(DEV)
+    capi.scatter_with_workspace(src.to(DEV), index.to(DEV), out, None, B, E, 1, N, E, 1, 0, capi.SUM, out_given)
+    torch.cuda.synchronize()
+    assert capi.scatter_last_route() == "sum: buckets or runs (sample)"
+    if dtype.is_floating_point:
+        mags = torch.zeros((B, N, 1), dtype=torch.float64)
+        for b in range(B):
+            mags[b, :, 0].index_add_(0, index[b][valid[b]], src[b, valid[b], 0].double().abs())
+        err = (out.cpu().double() - want).abs()
+        assert bool((err <= 1e-5 * want.abs() + 1e-5 * mags.max()).all()), float(err.max())
+    else:
+        assert torch.equal(out.cpu().double(), want)
+    # the count of the same index
+    cnt = torch.empty((B, N), dtype=torch.int32, device=DEV)
+    used = capi.scatter_count_with_workspace(index.to(DEV), cnt, B, E, N, E, 1)
+    assert used >= 8 * B * E
+    want_cnt = torch.stack([torch.bincount(index[b][valid[b]], minlength=N) for b in range(B)]).int()
+    assert torch.equal(cnt.cpu(), want_cnt)
+
+
+def test_scatter_sum_of_single_values_sorted_index_keeps_the_run_kernels(capi, oracle, monkeypatch):
+    """A sorted index: the sample sends the call to the kernels that combine runs; the bucket passes return at once."""
+    monkeypatch.setenv("TS_SCATTER_BINNED", "2")
+    rng = np.random.default_rng(8)
+    E, N = 90_001, 5000
+    index = torch.from_numpy(np.sort(rng.integers(0, N, size=E)).astype(np.int64))
+    src = torch.from_numpy(rng.integers(-9, 10, size=(1, E, 1)).astype(np.float32))     # small integers: exact
+    want, _ = oracle.scatter(src, index.view(1, -1, 1), 1, None, N, "sum")
+    out = torch.zeros((1, N, 1), device=DEV)
+    capi.scatter_with_workspace(src.to(DEV), index.to(DEV), out, None, 1, E, 1, N, 0, 1, 0, capi.SUM, False)
+    assert_exact(out, want)
