@@ -261,7 +261,9 @@ enum ts_scatter_route {
   TS_ROUTE_MINMAX_K1_SLABS = 14,         /* workspace, one value per entry: tables handed over in slabs */
   TS_ROUTE_MINMAX_BUCKETS = 15,          /* workspace: entries binned by bucket of output rows */
   TS_ROUTE_MINMAX_BUCKETS_OR_SEGMENTED = 16, /* the same; an index found sorted: the segmented reduction */
-  TS_ROUTE_MINMAX_64BIT = 17             /* 64-bit elements: value pass, then position pass */
+  TS_ROUTE_MINMAX_64BIT = 17,            /* 64-bit elements: value pass, then position pass */
+  TS_ROUTE_SUM_VALUE_BUCKETS = 18        /* workspace, one 4-byte value per entry: the values travel in the binned words;
+                                            a sample of the index picks buckets (even), table (skewed) or runs (sorted) */
 };
 /* Self-test of the fixed-pattern cross-lane helpers the kernels use (DPP row shifts, wave_shr:1,
  * v_permlane16_swap / v_permlane32_swap: csrc/dpp.h): one wavefront applies each helper to x = 3 * lane + 1 and

@@ -291,7 +291,7 @@ const char *ts_scatter_route_name(int route) {
       "sum: buckets or segmented reduction (index checked)", "mul: atomic", "mul: table", "min/max: atomic",
       "min/max: runs", "min/max: runs or table (sample)", "min/max: table", "min/max: table, one value per entry",
       "min/max: slabs, one value per entry", "min/max: buckets", "min/max: buckets or segmented reduction (index checked)",
-      "min/max: 64-bit elements, two passes"};
+      "min/max: 64-bit elements, two passes", "sum: single values in buckets, table or runs (sample)"};
   return route >= 0 && route < (int)(sizeof(names) / sizeof(names[0])) ? names[route] : "unknown";
 }
 
@@ -699,6 +699,7 @@ int ts_scatter_count_with_workspace(const int64_t *index, int32_t *count, int64_
     a.precheck = 1;
     a.lds_cache = env_int("TS_SCATTER_LDS", 1);
     a.lds_epb = env_int("TS_SCATTER_EPB", 0);
+    bool binned = false, three_way = false;
     // A large count under an unsorted index, given scratch: the entries are binned by bucket of output rows like a sum
     // of one value per entry (bin_plan_payload; the "value" of an entry is 1) instead of one device atomic per entry
     // that misses the table. A sample of the index decides; the kernels below then run only for an index that looks sorted.
@@ -706,14 +707,30 @@ int ts_scatter_count_with_workspace(const int64_t *index, int32_t *count, int64_
         B * N < 0x7FFFFFFFll) {  // (the kernels behind it that can be told to stand back)
       const BinPlan bp = bin_plan_payload(B, E, 1, N, 4, workspace, workspace_bytes, env_int("TS_SCATTER_BINNED", 1) == 2);
       if (bp.ok) {
-        launch_binned_add<int32_t, 1>(a, bp.p, 0, s);
+        // the sample of the index gives one of three answers: sorted (the run kernel below), skewed (the table
+        // kernel below), even (the buckets); without the table kernel or the sample only the first and the last
+        three_way = a.lds_cache == 1 && sum_table_by_size(B, E, 1, N, 4) && B * E >= 2 * kBinBlock &&
+                    !getenv("TS_BIN_NO_SAMPLE");
+        launch_binned_add<int32_t, 1>(a, bp.p, 0, s, 0, three_way);
         a.skip_flag = bp.p.unsorted;
+        binned = true;
       }
     }
     // the sizes from which the sum of one float per entry goes through the accumulator table (a hub otherwise
     // costs an atomic on one address per entry: 4 M entries under a Zipf(1.2) index 1.3 ms against 0.08 ms)
     const bool contended = a.lds_cache == 2 || (a.lds_cache == 1 && sum_table_by_size(B, E, 1, N, 4));
-    if (contended && B * N < 0x7FFFFFFFll) {
+    if (binned) {
+      // behind the buckets: the table kernel for a skewed index (flag 2), the run kernel for a sorted one (flag 0)
+      if (three_way) {
+        ScatterArgs t = a;
+        t.skip_want = 2;
+        const int64_t epb = per_cu_chunk_edges(a.lds_epb, B * E, sum_table_min_chunk(1, 4), 131072);
+        hipLaunchKernelGGL(scatter_add_lds_kernel<int32_t>, dim3((unsigned)((B * E + epb - 1) / epb)), dim3(kLdsAddBlock),
+                           0, s, t, kLdsAccRows - 1, epb);
+      }
+      const RunGrid g = run_grid(B * E, 1, 1, 4);
+      launch_add_run<int32_t, 1, 1>(a, g, s);
+    } else if (contended && B * N < 0x7FFFFFFFll) {
       const int64_t epb = per_cu_chunk_edges(a.lds_epb, B * E, sum_table_min_chunk(1, 4), 131072);
       hipLaunchKernelGGL(scatter_add_lds_kernel<int32_t>, dim3((unsigned)((B * E + epb - 1) / epb)), dim3(kLdsAddBlock), 0,
                          s, a, kLdsAccRows - 1, epb);

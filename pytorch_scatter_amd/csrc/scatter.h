@@ -235,6 +235,7 @@ struct ScatterArgs {
   int bin_any_size = 0;    // tuning aid / tests: also for inputs below the size from which it pays
   const int *skip_flag = nullptr;  // sum kernels: leave at once if *skip_flag != 0 (the binned pass did the work)
   int skip_inverse = 0;            // ... if *skip_flag == 0 instead
+  int skip_want = -1;              // >= 0 (table kernel only): run only if *skip_flag == skip_want
   int *order_ws = nullptr;         // sum of narrow rows: a word of scratch for the sample of the index that picks the kernel
   int skew_probe = 1;              // min/max: sample the index for skew (needs 256 bytes of workspace): 0 never, 2 at any size
   const int *skew_flag = nullptr;  // min/max kernels behind the probe: run only if (*skew_flag != 0) == (skew_want != 0)
@@ -1408,7 +1409,11 @@ template <typename L> __device__ __forceinline__ void lds_slot_mul(L *slot, L v)
 template <typename T, bool MUL = false>
 __global__ __launch_bounds__(kLdsAddBlock) void scatter_add_lds_kernel(ScatterArgs a, int tn_mask, int64_t epb) {
   constexpr int U = 4;
-  if (a.skip_flag != nullptr && (*a.skip_flag != 0) != (a.skip_inverse != 0)) return;
+  if (a.skip_flag != nullptr && a.skip_want >= 0) {
+    if (*a.skip_flag != a.skip_want) return;
+  } else if (a.skip_flag != nullptr && (*a.skip_flag != 0) != (a.skip_inverse != 0)) {
+    return;
+  }
   // double slots for the floating types: ds_add_f32 loses its rate when many lanes meet on one address (a hub, or a
   // sorted index whose neighbouring entries share a row), ds_add_f64 does not (Zipf(1.2) index, K = 8: 391 -> 263 us;
   // sorted: 476 -> 177 us). Integers keep their own width (their sums wrap, which a double cannot follow).
@@ -1842,7 +1847,8 @@ int launch_scatter_v(const ScatterArgs &args, int reduce, hipStream_t stream) {
     const bool routed = lshift >= 0 && a.sorted_route && a.route_flag != nullptr && !a.out_given;
     // sums that go through the LDS table (scatter_add_lds_kernel; the sizes and crossovers are with its launch
     // below), and whether a sample of the index picks between it and the run kernel
-    bool use_lds = false, sampled = false;
+    bool use_lds = false, sampled = false, three_way = false;
+    const bool payload = lshift >= 0 && bp.p.payload != 0;
     int tn = 1;
     if constexpr (__is_same(T, float) || __is_same(T, bf16_t) || __is_same(T, f16_t) || __is_same(T, double) ||
                   __is_same(T, int32_t) || __is_same(T, int64_t)) {
@@ -1850,8 +1856,12 @@ int launch_scatter_v(const ScatterArgs &args, int reduce, hipStream_t stream) {
         while ((int64_t)tn * 2 * a.K <= kLdsAcc && tn * 2 <= kLdsAccRows) tn *= 2;
         // (behind the buckets only an index in order arrives here: that one has the table only if contended)
         const bool by_size = sum_table_by_size(a.B, a.E, a.K, a.N, (int)sizeof(T)) &&
-                             (lshift < 0 || n_edges >= 32 * a.B * a.N);
+                             (lshift < 0 || payload || n_edges >= 32 * a.B * a.N);
         use_lds = a.lds_cache && a.sk == 0 && tn >= 64 && a.B * a.N < 0x7FFFFFFFll && (a.lds_cache == 2 || by_size);
+        // single values through the buckets: the sample of the index gives one of three answers (sorted: the run
+        // kernel; skewed: the table kernel; even: the buckets), which needs the table kernel and the sample
+        three_way = payload && use_lds && n_edges >= 2 * kBinBlock && !getenv("TS_BIN_NO_SAMPLE");
+        if (payload && !three_way) use_lds = false;
         // (a sample of the index: from 2^23 elements, where a sorted index does better through the run kernel;
         // below, the table is level with it and the launch that returns at once would cost 2-4 us)
         sampled = use_lds && a.lds_cache != 2 && a.order_ws != nullptr && a.skip_flag == nullptr && lshift < 0 &&
@@ -1870,8 +1880,9 @@ int launch_scatter_v(const ScatterArgs &args, int reduce, hipStream_t stream) {
     }
     if constexpr (BinSlotOk<T>::value) {
       if (lshift >= 0) {
-        ts_note_scatter_route(routed ? TS_ROUTE_SUM_BUCKETS_OR_SEGMENTED : TS_ROUTE_SUM_BUCKETS_OR_RUNS);
-        launch_binned_add<T, VEC>(a, bp.p, lshift, stream, routed ? n_out : 0);
+        ts_note_scatter_route(payload ? TS_ROUTE_SUM_VALUE_BUCKETS : routed ? TS_ROUTE_SUM_BUCKETS_OR_SEGMENTED
+                                                                              : TS_ROUTE_SUM_BUCKETS_OR_RUNS);
+        launch_binned_add<T, VEC>(a, bp.p, lshift, stream, routed ? n_out : 0, three_way);
         a.skip_flag = bp.p.unsorted;
         if (routed) {
           *a.route_flag = bp.p.unsorted;
@@ -1900,12 +1911,13 @@ int launch_scatter_v(const ScatterArgs &args, int reduce, hipStream_t stream) {
               t.skip_inverse = 1;
               a.skip_flag = a.order_ws;
             }
+            if (three_way) t.skip_want = 2;  // (skip_flag is the buckets' flag: 2 = unsorted and skewed)
             const int64_t epb = per_cu_chunk_edges(a.lds_epb, n_edges, sum_table_min_chunk(a.K, (int)sizeof(T)),
                                                    131072 / a.K > 2048 ? 131072 / a.K : 2048);
             if (lshift < 0) ts_note_scatter_route(sampled ? TS_ROUTE_SUM_TABLE_OR_RUNS : TS_ROUTE_SUM_TABLE);
             hipLaunchKernelGGL(scatter_add_lds_kernel<T>, dim3((unsigned)((n_edges + epb - 1) / epb)),
                                dim3(kLdsAddBlock), 0, stream, t, tn - 1, epb);
-            if (!sampled) return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
+            if (!sampled && !three_way) return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
           }
         }
         {

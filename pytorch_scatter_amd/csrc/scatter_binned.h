@@ -50,7 +50,9 @@ struct BinArgs {
                            //            up to kCombFew chunks from the front, those of more from slot nb - 1 down
   int32_t *comb_count;     //            how many of either
 
-  int *unsorted;           // sum only (else null): set to 1 by the count pass when the index is not sorted;
+  int *unsorted;           // sum only (else null): 1 = the buckets take the call (set by the count pass or by a sample when
+                           // the index is not sorted); 0 = sorted, 2 = (single values only) unsorted but skewed: both
+                           // leave the call to other kernels, and every pass of the buckets returns at once;
                            // a sorted index is left to the kernels that combine runs, and the passes after
                            // the count return at once
   int strict = 0;          // the count pass also reports an index outside [0, N) as unsorted (a caller that hands a
@@ -201,7 +203,9 @@ inline BinPlan bin_plan_payload(int64_t B, int64_t E, int64_t K, int64_t N, int 
   r.bytes = 0;
   const int64_t n_edges = B * E, rows = B * N;
   if (K != 1 || elem_bytes != 4 || n_edges >= 0xFFFFFFFEll || rows >= 0x7FFFFFFFll || rows < 1) return r;
-  if (!any_size && n_edges < ((int64_t)1 << 21)) return r;   // below: the table kernel's launches are the call
+  // from 4 M entries: a uniform index gains from 2 M on (74 against 106 us), but a skewed one, which the sample hands
+  // to the table kernel, pays about 15 us for the launches that return at once (2.3 M entries: 51 against 36 us)
+  if (!any_size && n_edges < ((int64_t)1 << 22)) return r;
   // chunk: entries per reducing workgroup, about 1024 workgroups, 2048 ... 65536 entries
   int64_t chunk = (n_edges / 1024 + 1023) & ~(int64_t)1023;
   if (chunk < 2048) chunk = 2048;
@@ -360,6 +364,41 @@ static __global__ __launch_bounds__(kBinBlock) void bin_sample_kernel(ScatterArg
   if (threadIdx.x == 0) *flag = s_desc * 64 >= kBinBlock ? 1 : 0;
 }
 
+// The same sample for sums of single values, with a third answer. The buckets pay for an index that spreads evenly
+// over the output rows (8 M entries onto 1 M rows, uniform: 126 us against 409 us through the table kernel); under a
+// skewed index the table kernel's hot rows absorb most entries and it wins (Zipf(1.5): 56 against 165 us). So the
+// sample also counts how many of its 1024 entries name a row that an earlier one named (a hash set in LDS):
+// *flag = 0 sorted-looking, 2 not sorted and at least three quarters repeat (the table kernel), 1 else (buckets).
+// (Around two thirds -- a Zipf(1.2) index -- the two are level: 8-10 M entries onto 1 M rows 152-160 us through
+// the buckets and 106-195 us through the table, by where the hot rows lie; at 86 %, Zipf(1.5), the table takes 56 us.)
+static __global__ __launch_bounds__(kBinBlock) void bin_sample_skew_kernel(ScatterArgs a, int *flag) {
+  constexpr int kSlots = 2048;
+  __shared__ int s_set[kSlots];
+  __shared__ int s_desc, s_dup;
+  for (int i = threadIdx.x; i < kSlots; i += kBinBlock) s_set[i] = -1;
+  if (threadIdx.x == 0) { s_desc = 0; s_dup = 0; }
+  __syncthreads();
+  const int64_t n = a.B * a.E;  // the host launches this only with n >= 2 * kBinBlock
+  const int64_t be = (int64_t)threadIdx.x * (n / kBinBlock);
+  const int64_t b = be / a.E, e = be - b * a.E;
+  const int64_t b1 = (be + 1) / a.E, e1 = be + 1 - b1 * a.E;
+  const int64_t idx = a.index[b * a.sb + e * a.se];
+  const int64_t nxt = a.index[b1 * a.sb + e1 * a.se];
+  if (b1 == b && nxt < idx) atomicAdd(&s_desc, 1);
+  if (idx >= 0 && idx < a.N) {
+    const int node = (int)(b * a.N + idx);
+    unsigned h = ((unsigned)node * 2654435761u) >> 21;  // 11 bits
+    for (int probe = 0; probe < 16; ++probe) {
+      const int old = atomicCAS(&s_set[h], -1, node);
+      if (old == -1) break;
+      if (old == node) { atomicAdd(&s_dup, 1); break; }
+      h = (h + 1) & (kSlots - 1);
+    }
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) *flag = s_desc * 64 < kBinBlock ? 0 : (s_dup * 4 >= 3 * kBinBlock ? 2 : 1);
+}
+
 // Count pass: entries per bucket (and, for callers that ask, whether the index is in order and inside [0, N)).
 // At most two workgroups per CU, each with an equal share of the entries, which it walks in batches of four
 // entries per lane with the loads of the next batch in flight while this one is counted (a workgroup per 16384
@@ -373,7 +412,7 @@ template <int CAP>
 static __global__ __launch_bounds__(kBinPlaceBlock) __attribute__((amdgpu_num_sgpr(72))) void bin_count_kernel(ScatterArgs a, BinArgs p) {
   __shared__ int32_t s_hist[CAP];
   __shared__ int s_hist_flag;
-  if (p.sampled && *p.unsorted == 0) return;
+  if (p.sampled && *p.unsorted != 1) return;
   for (int i = threadIdx.x; i < p.nb; i += kBinPlaceBlock) s_hist[i] = 0;
   if (threadIdx.x == 0) s_hist_flag = 0;
   __syncthreads();
@@ -441,7 +480,7 @@ static __global__ __launch_bounds__(kBinBlock) void bin_scan_kernel(BinArgs p) {
   __shared__ int32_t s_l[kBinBlock];  // buckets for the combining kernel: those without exactly one chunk,
   __shared__ int32_t s_g[kBinBlock];  // of which more than kCombFew chunks
   __shared__ int32_t s_cs[kBinMaxBuckets + 1];  // chunk_start, for the search at the end
-  if (p.unsorted != nullptr && *p.unsorted == 0) return;  // sorted: none of the later passes runs
+  if (p.unsorted != nullptr && *p.unsorted != 1) return;  // sorted: none of the later passes runs
   // a bucket holds fewer than 2^32 entries (the plan refuses larger inputs): 32-bit counts and divisions
   // every lane owns `per` neighbouring buckets, no more than the bucket count asks for: the integer divisions below
   // are the kernel's time (sixteen per lane on one CU took 10 us whatever the number of buckets)
@@ -537,8 +576,8 @@ template <int CAP>
 static __global__ __launch_bounds__(kBinPlaceBlock) void bin_place_kernel(ScatterArgs a, BinArgs p) {
   __shared__ uint32_t s_base[CAP];
   __shared__ int32_t s_cnt[CAP];
-  if (p.unsorted != nullptr && *p.unsorted == 0) {
-    // A sorted index: nothing to place. A caller that finishes it with the segmented reduction gets the row
+  if (p.unsorted != nullptr && *p.unsorted != 1) {
+    // A sorted index (or, for single values, a skewed one that the table kernel takes): nothing to place. A caller that finishes it with the segmented reduction gets the row
     // pointers from this launch instead: ptr[b][r] = first e with index[b][e] >= r (the count pass has checked
     // that the index is in order and inside [0, N)).
     if (a.route_ptr != nullptr) {
@@ -616,7 +655,7 @@ static __global__ __launch_bounds__(kBinPlaceBlock) void bin_place_sorted_kernel
   __shared__ int32_t s_cnt[kBinSortBuckets];   // counts, then the tile's exclusive prefix
   __shared__ uint32_t s_base[kBinSortBuckets];  // first word of the tile's run in every bucket
   __shared__ int32_t s_wsum[kBinPlaceBlock / kWave];
-  if (p.unsorted != nullptr && *p.unsorted == 0) return;
+  if (p.unsorted != nullptr && *p.unsorted != 1) return;
   for (int i = threadIdx.x; i < p.nb; i += kBinPlaceBlock) s_cnt[i] = 0;
   __syncthreads();
   const int64_t lo = (int64_t)blockIdx.x * kBinSortTile;
@@ -749,7 +788,7 @@ template <typename T, bool IS_MAX>
 __global__ __launch_bounds__(kBinBlock) void bin_combine_kernel(ScatterArgs a, BinArgs p) {
   constexpr int W = kBinBlock / kWave;
   __shared__ uint64_t s_part[W][kCombPos];
-  if (p.unsorted != nullptr && *p.unsorted == 0) return;  // sorted index: left to the caller's segmented reduction
+  if (p.unsorted != nullptr && *p.unsorted != 1) return;  // sorted index: left to the caller's segmented reduction
   const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
   const int table = (int)a.K << p.rshift;
   const int n_few = p.comb_count[0], n_many = p.comb_count[1];
@@ -808,7 +847,7 @@ __global__ __launch_bounds__(kBinBlock) void bin_reduce_kernel(ScatterArgs a, Bi
   // rows are K + 1 keys apart: with K a multiple of 32 the rows would all start in the same LDS bank and the
   // lanes of a wavefront, which hold the same columns of different rows, would queue up behind each other
   __shared__ uint64_t s_keys[kBinKeys + kBinKeys / 16];
-  if (p.unsorted != nullptr && *p.unsorted == 0) return;
+  if (p.unsorted != nullptr && *p.unsorted != 1) return;
   const int bucket = p.wg_bucket[blockIdx.x];
   if (bucket < 0) return;
   const int K = (int)a.K;
@@ -862,7 +901,7 @@ template <typename T, int VEC, bool IS_MAX>
 __global__ __launch_bounds__(kBinBlock) void bin_reduce_wave_kernel(ScatterArgs a, BinArgs p, int lshift) {
   constexpr int U = 4;  // eight rows in flight per lane: 90 VGPRs, one workgroup per CU, no gain
   __shared__ uint64_t s_keys[kBinKeys + kBinKeys / 16];  // rows K + 1 keys apart (LDS banks, see above)
-  if (p.unsorted != nullptr && *p.unsorted == 0) return;
+  if (p.unsorted != nullptr && *p.unsorted != 1) return;
   const int wg = (int)(blockIdx.x / (unsigned)p.slices), slice = (int)(blockIdx.x - (unsigned)wg * p.slices);
   const int bucket = p.wg_bucket[wg];
   if (bucket < 0) return;
@@ -945,7 +984,7 @@ __global__ __launch_bounds__(kBinBlock) void bin_add_wave_kernel(ScatterArgs a, 
   constexpr int U = 4;
   constexpr int kSlots = (kBinKeys + kBinKeys / 16) * 8 / (int)sizeof(A);
   __shared__ A s_acc[kSlots];  // rows K + 1 slots apart (LDS banks)
-  if (p.unsorted != nullptr && *p.unsorted == 0) return;
+  if (p.unsorted != nullptr && *p.unsorted != 1) return;
   const int wg = (int)(blockIdx.x / (unsigned)p.slices), slice = (int)(blockIdx.x - (unsigned)wg * p.slices);
   const int bucket = p.wg_bucket[wg];
   if (bucket < 0) return;
@@ -1050,7 +1089,7 @@ __global__ __launch_bounds__(kBinBlock) void bin_add_payload_kernel(ScatterArgs 
   typedef unsigned long long u64x2 __attribute__((ext_vector_type(2)));
   constexpr int U = 4;
   __shared__ A s_acc[4096];
-  if (p.unsorted != nullptr && *p.unsorted == 0) return;
+  if (p.unsorted != nullptr && *p.unsorted != 1) return;
   const int wg = (int)blockIdx.x;
   const int bucket = p.wg_bucket[wg];
   if (bucket < 0) return;
@@ -1149,21 +1188,27 @@ void launch_binned_keys(const ScatterArgs &a, const BinArgs &plan, hipStream_t s
 // out[i] = 0 unless the index is sorted (then nobody adds into out: the caller's segmented reduction writes it)
 template <typename T>
 __global__ __launch_bounds__(kBlock) void bin_zero_out_kernel(T *out, int64_t n, const int *unsorted) {
-  if (*unsorted == 0) return;
+  if (*unsorted != 1) return;
   for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlock)
     out[i] = zero_elem<T>();
 }
 
 // zero_out: elements of out to clear once the count pass has found the index unsorted (0: the caller has cleared it)
+// three_way: the caller has the table kernel behind this launch for a skewed index (flag value 2, see
+// bin_sample_skew_kernel); needs the sample (no sorted_route, enough entries), else the answer stays 0 / 1
 template <typename T, int VEC>
-void launch_binned_add(const ScatterArgs &a, const BinArgs &plan, int lshift, hipStream_t stream, int64_t zero_out = 0) {
+void launch_binned_add(const ScatterArgs &a, const BinArgs &plan, int lshift, hipStream_t stream, int64_t zero_out = 0,
+                       bool three_way = false) {
   BinArgs p = plan;
   p.sampled = a.B * a.E >= 2 * kBinBlock && !getenv("TS_BIN_NO_SAMPLE");  // env: tuning aid (sorted = no descent at all)
   if (a.sorted_route && a.route_flag != nullptr) {  // the caller's segmented reduction needs the whole index checked
     p.sampled = 0;
     p.strict = 1;
   }
-  if (p.sampled) hipLaunchKernelGGL(bin_sample_kernel, dim3(1), dim3(kBinBlock), 0, stream, a, p.unsorted);
+  if (p.sampled && three_way)
+    hipLaunchKernelGGL(bin_sample_skew_kernel, dim3(1), dim3(kBinBlock), 0, stream, a, p.unsorted);
+  else if (p.sampled)
+    hipLaunchKernelGGL(bin_sample_kernel, dim3(1), dim3(kBinBlock), 0, stream, a, p.unsorted);
   hipLaunchKernelGGL(bin_clear_kernel, dim3((p.nb + kBlock - 1) / kBlock), dim3(kBlock), 0, stream, p.totals, p.nb,
                      p.sampled ? (int *)nullptr : p.unsorted);
   launch_bin_count(a, p, stream);

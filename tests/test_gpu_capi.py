@@ -1731,7 +1731,7 @@ def test_scatter_sum_of_single_values_through_buckets(capi, oracle, case, dtype,
     out = prev.clone().to(DEV)
     capi.scatter_with_workspace(src.to(DEV), index.to(DEV), out, None, B, E, 1, N, E, 1, 0, capi.SUM, out_given)
     torch.cuda.synchronize()
-    assert capi.scatter_last_route() == "sum: buckets or runs (sample)"
+    assert capi.scatter_last_route() == "sum: single values in buckets, table or runs (sample)"
     if dtype.is_floating_point:
         mags = torch.zeros((B, N, 1), dtype=torch.float64)
         for b in range(B):
