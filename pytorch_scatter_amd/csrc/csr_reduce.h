@@ -421,14 +421,24 @@ __global__ __launch_bounds__(kCsrBlock, (csr_reduce_min_blocks<T, VEC, REDUCE, P
 
   // look-back mode: this tile's carry slot is the second of its two partial slots
   uint64_t *carry_flags = reinterpret_cast<uint64_t *>(a.ws_meta) + (b * a.nblk) * 4 + blockIdx.y;
+  // Where element v of this lane's slice sits inside a carry row. The lanes of a worker hold VEC neighbouring
+  // columns each, so instruction v of a carry written column by column would touch G addresses VEC elements apart
+  // -- every 64-byte sector of the row VEC times over, and each of those atomics is a read-modify-write of a
+  // sector at the memory side (C5: 254 MB written next to 614 MB of output). With whole column chunks the
+  // carry row is stored transposed instead: instruction v covers G neighbouring elements. Reader and writer
+  // use the same rule; the layout is private to the look-back.
+  const bool carry_transposed = a.K % CW == 0;
+  auto carry_pos = [&](int v) -> int64_t {
+    return carry_transposed ? (int64_t)blockIdx.y * CW + (int64_t)v * G + lg : col + v;
+  };
   auto publish_carry = [&](uint64_t kind) {
     if constexpr (kCarryOk) {
     uint64_t sink = 0;
     if (col_ok) {
 #pragma unroll
       for (int v = 0; v < VEC; ++v) {
-        sink |= carry_put<A>(ws_val_blk + a.K + col + v, acc[v]);
-        if (kArg) sink |= carry_put<int32_t>(ws_arg_blk + a.K + col + v, arg[v]);
+        sink |= carry_put<A>(ws_val_blk + a.K + carry_pos(v), acc[v]);
+        if (kArg) sink |= carry_put<int32_t>(ws_arg_blk + a.K + carry_pos(v), arg[v]);
       }
     }
     asm volatile("" ::"v"(sink) : "memory");  // the returns are in: the carry is in memory
@@ -487,8 +497,9 @@ __global__ __launch_bounds__(kCsrBlock, (csr_reduce_min_blocks<T, VEC, REDUCE, P
         if (q < n) {
 #pragma unroll
           for (int v = 0; v < VEC; ++v) {
-            early[q][v] = carry_get<A>(vals_b + ((hi - q * stride) * 2 + 1) * a.K + c + v);
-            if (kArg) early_arg[q][v] = carry_get<int32_t>(args_b + ((hi - q * stride) * 2 + 1) * a.K + c + v);
+            const int64_t cp = col_ok ? carry_pos(v) : (int64_t)v;
+            early[q][v] = carry_get<A>(vals_b + ((hi - q * stride) * 2 + 1) * a.K + cp);
+            if (kArg) early_arg[q][v] = carry_get<int32_t>(args_b + ((hi - q * stride) * 2 + 1) * a.K + cp);
           }
         }
       }
