@@ -88,7 +88,7 @@ def ceiling_matrix():
     import torch
     lib = probe_lib()
     lib.ts_probe_matrix.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_size_t] + \
-        [ctypes.c_int] * 7 + [ctypes.c_void_p]
+        [ctypes.c_int] * 8 + [ctypes.c_void_p]
     dev = torch.device("cuda:0")
     heavy = 6 << 30
     ratio = 26
@@ -109,7 +109,7 @@ def ceiling_matrix():
                             for nt_load in ((1,) if not (burst == 4096 and depth == 8) else (1, 0)):
                                 grid = 256 * wg_per_cu
                                 fn = lambda: lib.ts_probe_matrix(a.data_ptr(), b.data_ptr(), units, burst, ratio, heavy_read,
-                                                                 depth, nt_load, nt_store, split, grid, stream)
+                                                                 depth, nt_load, nt_store, split, grid, 0, stream)
                                 assert fn() == 0
                                 t = event_time(fn, 3, warm=1)
                                 rows.append({"mix": "read 26 : write 1" if heavy_read else "read 1 : write 26",

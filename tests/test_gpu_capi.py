@@ -44,9 +44,9 @@ def assert_sum16_no_worse_than_reference(oracle, out, src, index, index1, N, dim
     entries, and a hub row far fewer. Checked two ways against the exact (fp64) sum:
       * in aggregate: the RMS error is not above that of the oracle run in the 16-bit type (the reference's
         arithmetic on the same input);
-      * element by element: at most 4 * min(n, 128) half-ulp roundings of a running total of the size
-        max(|exact|, sqrt(sum of squares)) (n: entries of the row) -- the envelope the reference's arithmetic
-        itself reaches on these inputs (measured up to 480 such units for it, up to 200 here)."""
+      * element by element: at most 4 * min(n, 100) half-ulp roundings of a running total of the size
+        max(|exact|, sqrt(sum of squares)) (n: entries of the row), i.e. never more than 400 such units: twice the
+        200 that the kernels reach on these inputs (the reference's own arithmetic reaches 480)."""
     dtype = src.dtype
     u = HALF_ULP[dtype]
     want = exact + (prev.double() if prev is not None else 0)
@@ -58,7 +58,7 @@ def assert_sum16_no_worse_than_reference(oracle, out, src, index, index1, N, dim
     scale = torch.maximum(want.abs(), sq.sqrt())
     shape = [1] * want.dim()
     shape[dim] = N
-    n_row = torch.bincount(index1, minlength=N).double().clamp(min=1, max=128).view(shape)
+    n_row = torch.bincount(index1, minlength=N).double().clamp(min=1, max=100).view(shape)
     err = (out.cpu().double() - want).abs()
     bound = u * 4 * n_row * scale + 1e-30
     assert bool((err <= bound).all()), (what, "element", float((err / bound).max()))
