@@ -304,7 +304,7 @@ __device__ __forceinline__ void bin_buckets(const ScatterArgs &a, const BinArgs 
     }
 #pragma unroll
     for (int j = 0; j < kBinPer; ++j) {
-      const int elo = __shfl((int)(uint32_t)edge, j), ehi = __shfl((int)(edge >> 32), j);
+      const int elo = __builtin_amdgcn_readlane((int)(uint32_t)edge, j), ehi = __builtin_amdgcn_readlane((int)(edge >> 32), j);
       const int64_t up = lane_up1_64(node[j]);  // by every lane: lane 0's value is what lane 1 reads
       const int64_t prev = lane == 0 ? (int64_t)(((uint64_t)(uint32_t)ehi << 32) | (uint32_t)elo) : up;
       descent = descent || (node[j] >= 0 && prev >= 0 && node[j] < prev);
@@ -323,21 +323,25 @@ __device__ __forceinline__ void bin_buckets(const ScatterArgs &a, const BinArgs 
 // of their leader (with a heavy-tailed index nearly all lanes: the bucket of the hubs, which would otherwise
 // queue up on one LDS address); whoever is left adds on its own.
 __device__ __forceinline__ int32_t bin_take(int32_t *counter, int32_t bucket) {
-  const int lane = threadIdx.x & (kWave - 1);
   int32_t before = 0;
   bool waiting = bucket >= 0;
 #pragma unroll
   for (int round = 0; round < 2; ++round) {
     const uint64_t todo = __ballot(waiting);
     if (todo == 0) break;
-    const int head = __ffsll((unsigned long long)todo) - 1;
-    const int32_t first = __shfl(bucket, head);
-    const uint64_t same = __ballot(waiting && bucket == first);
+    // head and first are the same for the whole wavefront: scalar registers, v_readlane instead of a shuffle
+    const int head = __builtin_ctzll((unsigned long long)todo);
+    const int32_t first = __builtin_amdgcn_readlane(bucket, head);
+    const bool with_head = waiting && bucket == first;
+    const uint64_t same = __ballot(with_head);
+    // lanes of `same` below this one (v_mbcnt): the head's is 0
+    const int32_t below = (int32_t)__builtin_amdgcn_mbcnt_hi((uint32_t)(same >> 32),
+                                                             __builtin_amdgcn_mbcnt_lo((uint32_t)same, 0u));
     int32_t base = 0;
-    if (lane == head) base = atomicAdd(&counter[first], __popcll(same));
-    base = __shfl(base, head);
-    if ((same >> lane) & 1) {
-      before = base + __popcll(same & (((uint64_t)1 << lane) - 1));
+    if (with_head && below == 0) base = atomicAdd(&counter[first], __popcll(same));
+    base = __builtin_amdgcn_readlane(base, head);
+    if (with_head) {
+      before = base + below;
       waiting = false;
     }
   }
@@ -445,7 +449,7 @@ static __global__ __launch_bounds__(kBinPlaceBlock) __attribute__((amdgpu_num_sg
       }
 #pragma unroll
       for (int j = 0; j < kBinCountPer; ++j) {
-        const int elo = __shfl((int)(uint32_t)edge, j), ehi = __shfl((int)(edge >> 32), j);
+        const int elo = __builtin_amdgcn_readlane((int)(uint32_t)edge, j), ehi = __builtin_amdgcn_readlane((int)(edge >> 32), j);
         const int64_t up = lane_up1_64(node[j]);  // by every lane: lane 0's value is what lane 1 reads
       const int64_t prev = lane == 0 ? (int64_t)(((uint64_t)(uint32_t)ehi << 32) | (uint32_t)elo) : up;
         descent = descent || (node[j] >= 0 && prev >= 0 && node[j] < prev);
