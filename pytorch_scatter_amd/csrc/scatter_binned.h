@@ -203,9 +203,10 @@ inline BinPlan bin_plan_payload(int64_t B, int64_t E, int64_t K, int64_t N, int 
   r.bytes = 0;
   const int64_t n_edges = B * E, rows = B * N;
   if (K != 1 || elem_bytes != 4 || n_edges >= 0xFFFFFFFEll || rows >= 0x7FFFFFFFll || rows < 1) return r;
-  // from 4 M entries: a uniform index gains from 2 M on (74 against 106 us), but a skewed one, which the sample hands
-  // to the table kernel, pays about 15 us for the launches that return at once (2.3 M entries: 51 against 36 us)
-  if (!any_size && n_edges < ((int64_t)1 << 22)) return r;
+  // from 2 M entries: an even index gains from there on (74 against 106 us; 2.3 M entries of a graph in random order
+  // 85 against 125 us); a skewed one, which the sample hands to the table kernel, pays about 15 us for the launches
+  // that return at once (2.3 M entries: 51 against 36 us)
+  if (!any_size && n_edges < ((int64_t)1 << 21)) return r;
   // chunk: entries per reducing workgroup, about 1024 workgroups, 2048 ... 65536 entries
   int64_t chunk = (n_edges / 1024 + 1023) & ~(int64_t)1023;
   if (chunk < 2048) chunk = 2048;

@@ -95,3 +95,20 @@ def test_route_narrow_rows_unsorted(env):
     assert capi.scatter_last_route() == "min/max: runs or table (sample)"
     _check_max(got, arg, src, index, 1_000_000)
     assert route_sum == "sum: table or runs (sample)"
+
+
+@pytest.mark.parametrize("E,route", [((1 << 21) + 4096, "sum: single values in buckets, table or runs (sample)"),
+                                     ((1 << 21) - 4096, "sum: table")])
+def test_route_single_values_either_side_of_the_value_buckets(env, E, route):
+    """One float per entry under an index in random order (the width-1 column of the benchmark table): value
+    buckets from 2^21 entries, the accumulator table below."""
+    ts, capi, _ = env
+    g = torch.Generator().manual_seed(E)
+    N = 270_000
+    index = torch.randint(0, N, (E,), generator=g).to(DEV)
+    src = torch.randn((E, 1), device=DEV)
+    got = ts.scatter_sum(src, index, 0, None, N)
+    assert capi.scatter_last_route() == route
+    _check_sum(got, src, index, N)
+    want = torch.zeros((N, 1), dtype=torch.float64, device=DEV).index_add_(0, index, src.double())
+    assert torch.allclose(got.double(), want, rtol=1e-5, atol=1e-4)
