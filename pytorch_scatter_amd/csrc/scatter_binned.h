@@ -374,8 +374,12 @@ static __global__ __launch_bounds__(kBinBlock) void bin_sample_kernel(ScatterArg
 // skewed index the table kernel's hot rows absorb most entries and it wins (Zipf(1.5): 56 against 165 us). So the
 // sample also counts how many of its 1024 entries name a row that an earlier one named (a hash set in LDS):
 // *flag = 0 sorted-looking, 2 not sorted and at least three quarters repeat (the table kernel), 1 else (buckets).
-// (Around two thirds -- a Zipf(1.2) index -- the two are level: 8-10 M entries onto 1 M rows 152-160 us through
-// the buckets and 106-195 us through the table, by where the hot rows lie; at 86 %, Zipf(1.5), the table takes 56 us.)
+// (Around two thirds -- a Zipf(1.2) index -- the two are level from 8 M entries: 8-10 M onto 1 M rows 152-160 us
+// through the buckets and 106-195 us through the table, by where the hot rows lie; at 86 %, Zipf(1.5), the table takes
+// 56 us. Below 8 M entries the table is sometimes ahead at two thirds -- Zipf(1.2), 64 % repeats, 2.2 / 4.3 M entries
+// onto 270 k rows: 51 / 89 us against 77 / 101 us through the buckets -- and sometimes far behind: the same onto 1 M
+// rows 141 / 79 us against 80 / 106 us. A bar of one half below 8 M entries was measured and lost more than it won, the
+// launches that return included; the buckets' time does not depend on where the hot rows lie.)
 static __global__ __launch_bounds__(kBinBlock) void bin_sample_skew_kernel(ScatterArgs a, int *flag) {
   constexpr int kSlots = 2048;
   __shared__ int s_set[kSlots];
