@@ -581,6 +581,37 @@ static __global__ __launch_bounds__(kBinBlock) void bin_scan_kernel(BinArgs p) {
   }
 }
 
+// ptr[b][r] = first e with index[b][e] >= r, from the entries [lo, hi) of the flattened index (which is in order and
+// inside [0, N)), in rounds of one entry per lane: what a place pass leaves for the segmented reduction that
+// finishes a sorted index
+__device__ __forceinline__ void bin_row_pointers(const ScatterArgs &a, int64_t lo, int64_t hi, GapList &s_gaps) {
+  // (long ranges of rows without entries are written by the wavefront or the workgroup: gap_rows; a round may span
+  // two batches, whose pointers differ, so the list is emptied after every round)
+  for (int64_t r0 = lo; r0 < hi; r0 += kBinPlaceBlock) {  // uniform
+    if (threadIdx.x == 0) s_gaps.n = 0;
+    __syncthreads();
+    const int64_t be = r0 + threadIdx.x;
+    const bool live = be < hi;
+    const int64_t b = live ? be / a.E : 0, e = live ? be - b * a.E : 0;
+    const int64_t *idx = a.index + b * a.sb;
+    int64_t top = live ? idx[e] : -1;
+    int64_t bot = e == 0 ? 0 : idx[e - 1] + 1;
+    if (bot < 0) bot = 0;
+    if (top > a.N) top = a.N;
+    if (!live) top = bot - 1;
+    // the ranges of one round are written through pointers relative to batch 0: lanes of one wavefront may
+    // belong to two batches
+    const int64_t off = b * (a.N + 1);
+    gap_rows(a.route_ptr, off + bot, off + top, e, s_gaps);
+    const bool last = live && e == a.E - 1;
+    const int64_t tl = top < 0 ? 0 : top + 1;
+    gap_rows(a.route_ptr, off + tl, last ? off + a.N : off + tl - 1, a.E, s_gaps);
+    __syncthreads();
+    gap_rows_finish(a.route_ptr, s_gaps);
+    __syncthreads();
+  }
+}
+
 template <int CAP>
 static __global__ __launch_bounds__(kBinPlaceBlock) void bin_place_kernel(ScatterArgs a, BinArgs p) {
   __shared__ uint32_t s_base[CAP];
@@ -590,33 +621,10 @@ static __global__ __launch_bounds__(kBinPlaceBlock) void bin_place_kernel(Scatte
     // pointers from this launch instead: ptr[b][r] = first e with index[b][e] >= r (the count pass has checked
     // that the index is in order and inside [0, N)).
     if (a.route_ptr != nullptr) {
-      // (long ranges of rows without entries are written by the wavefront or the workgroup: gap_rows; the
-      // workgroup's tile may span two batches, whose pointers differ, so the list is emptied after every round)
       __shared__ GapList s_gaps;
-      for (int j = 0; j < kBinPer; ++j) {
-        if (j * kBinPlaceBlock >= p.place_tile) break;  // uniform
-        if (threadIdx.x == 0) s_gaps.n = 0;
-        __syncthreads();
-        const int64_t be = (int64_t)blockIdx.x * p.place_tile + threadIdx.x + (int64_t)j * kBinPlaceBlock;
-        const bool live = be < a.B * a.E;
-        const int64_t b = live ? be / a.E : 0, e = live ? be - b * a.E : 0;
-        const int64_t *idx = a.index + b * a.sb;
-        int64_t hi = live ? idx[e] : -1;
-        int64_t lo = e == 0 ? 0 : idx[e - 1] + 1;
-        if (lo < 0) lo = 0;
-        if (hi > a.N) hi = a.N;
-        if (!live) hi = lo - 1;
-        // the ranges of one round are written through pointers relative to batch 0: lanes of one wavefront may
-        // belong to two batches
-        const int64_t off = b * (a.N + 1);
-        gap_rows(a.route_ptr, off + lo, off + hi, e, s_gaps);
-        const bool last = live && e == a.E - 1;
-        const int64_t tl = hi < 0 ? 0 : hi + 1;
-        gap_rows(a.route_ptr, off + tl, last ? off + a.N : off + tl - 1, a.E, s_gaps);
-        __syncthreads();
-        gap_rows_finish(a.route_ptr, s_gaps);
-        __syncthreads();
-      }
+      const int64_t lo = (int64_t)blockIdx.x * p.place_tile;
+      const int64_t hi = lo + p.place_tile < a.B * a.E ? lo + p.place_tile : a.B * a.E;
+      bin_row_pointers(a, lo, hi, s_gaps);
     }
     return;
   }
@@ -664,11 +672,18 @@ static __global__ __launch_bounds__(kBinPlaceBlock) void bin_place_sorted_kernel
   __shared__ int32_t s_cnt[kBinSortBuckets];   // counts, then the tile's exclusive prefix
   __shared__ uint32_t s_base[kBinSortBuckets];  // first word of the tile's run in every bucket
   __shared__ int32_t s_wsum[kBinPlaceBlock / kWave];
-  if (p.unsorted != nullptr && *p.unsorted != 1) return;
-  for (int i = threadIdx.x; i < p.nb; i += kBinPlaceBlock) s_cnt[i] = 0;
-  __syncthreads();
   const int64_t lo = (int64_t)blockIdx.x * kBinSortTile;
   const int64_t hi = lo + kBinSortTile < a.B * a.E ? lo + kBinSortTile : a.B * a.E;
+  if (p.unsorted != nullptr && *p.unsorted != 1) {
+    // nothing to place; a caller that finishes a sorted index with the segmented reduction gets its row pointers
+    if (a.route_ptr != nullptr) {
+      __shared__ GapList s_gaps;
+      bin_row_pointers(a, lo, hi, s_gaps);
+    }
+    return;
+  }
+  for (int i = threadIdx.x; i < p.nb; i += kBinPlaceBlock) s_cnt[i] = 0;
+  __syncthreads();
   int32_t bucket[kBinPer], local[kBinPer], rank[kBinPer];
   bool unused = false;
   bin_buckets(a, p, lo, hi, bucket, local, false, unused);
@@ -1146,6 +1161,14 @@ __global__ __launch_bounds__(kBinBlock) void bin_add_payload_kernel(ScatterArgs 
   }
 }
 
+// The place pass that sorts its tile in LDS first (bin_place_sorted_kernel) takes every plan it has room for (2048
+// buckets of up to 4096 rows): under an even index every 8-byte store of the plain pass is a line of its own (46 M
+// entries over 1860 buckets: 628 against 433 us); under a skewed one, whose runs are long either way, the two are
+// level (Zipf(1.2), 391 buckets: 64 against 65 us).
+inline bool bin_place_sorted_ok(const BinArgs &p) {
+  return p.nb <= kBinSortBuckets && p.rshift <= 12 && !getenv("TS_BIN_NO_SORTED_PLACE");  // env: tuning aid
+}
+
 // the count pass: equal shares of the entries for at most kBinCountGroups workgroups
 inline void launch_bin_count(const ScatterArgs &a, const BinArgs &p, hipStream_t stream) {
   int64_t groups = (a.B * a.E + kBinCountBatch - 1) / kBinCountBatch;
@@ -1179,7 +1202,10 @@ void launch_binned_keys(const ScatterArgs &a, const BinArgs &plan, hipStream_t s
                      p.unsorted);
   launch_bin_count(a, p, stream);
   hipLaunchKernelGGL(bin_scan_kernel, dim3(1), dim3(kBinBlock), 0, stream, p);
-  if (p.nb <= kBinSmallCap)  // 64 KB of cursors, two workgroups per CU; above: 128 KB, one
+  if (bin_place_sorted_ok(p))
+    hipLaunchKernelGGL(bin_place_sorted_kernel, dim3((unsigned)((a.B * a.E + kBinSortTile - 1) / kBinSortTile)),
+                       dim3(kBinPlaceBlock), 0, stream, a, p);
+  else if (p.nb <= kBinSmallCap)  // 64 KB of cursors, two workgroups per CU; above: 128 KB, one
     hipLaunchKernelGGL(bin_place_kernel<kBinSmallCap>, dim3((unsigned)p.n_place), dim3(kBinPlaceBlock), 0, stream, a, p);
   else
     hipLaunchKernelGGL(bin_place_kernel<kBinMaxBuckets>, dim3((unsigned)p.n_place), dim3(kBinPlaceBlock), 0, stream, a, p);
@@ -1225,7 +1251,7 @@ void launch_binned_add(const ScatterArgs &a, const BinArgs &plan, int lshift, hi
     hipLaunchKernelGGL(bin_zero_out_kernel<T>, dim3(grid_for(zero_out)), dim3(kBlock), 0, stream, static_cast<T *>(a.out),
                        zero_out, p.unsorted);
   hipLaunchKernelGGL(bin_scan_kernel, dim3(1), dim3(kBinBlock), 0, stream, p);
-  if (p.payload && p.nb <= kBinSortBuckets && !getenv("TS_BIN_NO_SORTED_PLACE"))  // env: tuning aid
+  if (bin_place_sorted_ok(p))
     hipLaunchKernelGGL(bin_place_sorted_kernel, dim3((unsigned)((a.B * a.E + kBinSortTile - 1) / kBinSortTile)),
                        dim3(kBinPlaceBlock), 0, stream, a, p);
   else if (p.nb <= kBinSmallCap)  // 64 KB of cursors, two workgroups per CU; above: 128 KB, one
