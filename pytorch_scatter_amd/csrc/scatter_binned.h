@@ -581,17 +581,18 @@ static __global__ __launch_bounds__(kBinBlock) void bin_scan_kernel(BinArgs p) {
   }
 }
 
-// ptr[b][r] = first e with index[b][e] >= r, from the entries [lo, hi) of the flattened index (which is in order and
-// inside [0, N)), in rounds of one entry per lane: what a place pass leaves for the segmented reduction that
+// ptr[b][r] = first e with index[b][e] >= r, from the `tile` entries at lo of the flattened index (which is in order
+// and inside [0, N)), in rounds of one entry per lane: what a place pass leaves for the segmented reduction that
 // finishes a sorted index
-__device__ __forceinline__ void bin_row_pointers(const ScatterArgs &a, int64_t lo, int64_t hi, GapList &s_gaps) {
+__device__ __forceinline__ void bin_row_pointers(const ScatterArgs &a, int64_t lo, int tile, GapList &s_gaps) {
   // (long ranges of rows without entries are written by the wavefront or the workgroup: gap_rows; a round may span
   // two batches, whose pointers differ, so the list is emptied after every round)
-  for (int64_t r0 = lo; r0 < hi; r0 += kBinPlaceBlock) {  // uniform
+  for (int j = 0; j < kBinPer; ++j) {
+    if (j * kBinPlaceBlock >= tile) break;  // uniform
     if (threadIdx.x == 0) s_gaps.n = 0;
     __syncthreads();
-    const int64_t be = r0 + threadIdx.x;
-    const bool live = be < hi;
+    const int64_t be = lo + threadIdx.x + (int64_t)j * kBinPlaceBlock;
+    const bool live = be < a.B * a.E;
     const int64_t b = live ? be / a.E : 0, e = live ? be - b * a.E : 0;
     const int64_t *idx = a.index + b * a.sb;
     int64_t top = live ? idx[e] : -1;
@@ -612,8 +613,11 @@ __device__ __forceinline__ void bin_row_pointers(const ScatterArgs &a, int64_t l
   }
 }
 
+// (eight wavefronts per SIMD, i.e. at most 64 vector registers: two workgroups per CU at CAP = 8192; left to itself
+// the compiler takes 66-71, which is one: Zipf(1.2), 391 buckets, 10 M entries 65 against 55 us)
 template <int CAP>
-static __global__ __launch_bounds__(kBinPlaceBlock) void bin_place_kernel(ScatterArgs a, BinArgs p) {
+static __global__ __launch_bounds__(kBinPlaceBlock) __attribute__((amdgpu_waves_per_eu(8, 8)))
+void bin_place_kernel(ScatterArgs a, BinArgs p) {
   __shared__ uint32_t s_base[CAP];
   __shared__ int32_t s_cnt[CAP];
   if (p.unsorted != nullptr && *p.unsorted != 1) {
@@ -622,9 +626,7 @@ static __global__ __launch_bounds__(kBinPlaceBlock) void bin_place_kernel(Scatte
     // that the index is in order and inside [0, N)).
     if (a.route_ptr != nullptr) {
       __shared__ GapList s_gaps;
-      const int64_t lo = (int64_t)blockIdx.x * p.place_tile;
-      const int64_t hi = lo + p.place_tile < a.B * a.E ? lo + p.place_tile : a.B * a.E;
-      bin_row_pointers(a, lo, hi, s_gaps);
+      bin_row_pointers(a, (int64_t)blockIdx.x * p.place_tile, p.place_tile, s_gaps);
     }
     return;
   }
@@ -667,7 +669,10 @@ static_assert(kBinPlaceChunk == kBinBatch, "the place pass holds a workgroup's e
 // of LDS, two workgroups per CU.
 constexpr int kBinSortTile = 6144;
 constexpr int kBinSortBuckets = 2048;
-static __global__ __launch_bounds__(kBinPlaceBlock) void bin_place_sorted_kernel(ScatterArgs a, BinArgs p) {
+// (eight wavefronts per SIMD = two workgroups per CU: the branch that writes row pointers would otherwise cost
+// the placing branch its registers, 70 instead of 60)
+static __global__ __launch_bounds__(kBinPlaceBlock) __attribute__((amdgpu_waves_per_eu(8, 8)))
+void bin_place_sorted_kernel(ScatterArgs a, BinArgs p) {
   __shared__ uint64_t s_stage[kBinSortTile];
   __shared__ int32_t s_cnt[kBinSortBuckets];   // counts, then the tile's exclusive prefix
   __shared__ uint32_t s_base[kBinSortBuckets];  // first word of the tile's run in every bucket
@@ -678,7 +683,7 @@ static __global__ __launch_bounds__(kBinPlaceBlock) void bin_place_sorted_kernel
     // nothing to place; a caller that finishes a sorted index with the segmented reduction gets its row pointers
     if (a.route_ptr != nullptr) {
       __shared__ GapList s_gaps;
-      bin_row_pointers(a, lo, hi, s_gaps);
+      bin_row_pointers(a, lo, kBinSortTile, s_gaps);
     }
     return;
   }
@@ -1161,12 +1166,16 @@ __global__ __launch_bounds__(kBinBlock) void bin_add_payload_kernel(ScatterArgs 
   }
 }
 
-// The place pass that sorts its tile in LDS first (bin_place_sorted_kernel) takes every plan it has room for (2048
-// buckets of up to 4096 rows): under an even index every 8-byte store of the plain pass is a line of its own (46 M
-// entries over 1860 buckets: 628 against 433 us); under a skewed one, whose runs are long either way, the two are
-// level (Zipf(1.2), 391 buckets: 64 against 65 us).
+// Which plans the place pass that sorts its tile in LDS first (bin_place_sorted_kernel) takes, of those it has room
+// for (2048 buckets of up to 4096 rows): value words always, entry words from 512 buckets on. Under an even index
+// every 8-byte store of the plain pass is a line of its own and the sorted pass wins at any number of buckets (10 M
+// entries over 391 / 977 buckets: 65 / 76 against 86 / 116 us; 46 M over 1860: 433 against 628 us); under a skewed
+// index, whose runs are long as they are, the plain pass does (Zipf(1.2), 391 buckets: 55 against 64 us). The host
+// does not know which it has; the heavy-tailed indices measured here come with few buckets. (Choosing per tile, from
+// the tile's largest bucket, was measured: both branches in one kernel spill and lose 10 us each.)
 inline bool bin_place_sorted_ok(const BinArgs &p) {
-  return p.nb <= kBinSortBuckets && p.rshift <= 12 && !getenv("TS_BIN_NO_SORTED_PLACE");  // env: tuning aid
+  return p.nb <= kBinSortBuckets && p.rshift <= 12 && (p.payload || p.nb >= 512) &&
+         !getenv("TS_BIN_NO_SORTED_PLACE");  // env: tuning aid
 }
 
 // the count pass: equal shares of the entries for at most kBinCountGroups workgroups
