@@ -658,6 +658,7 @@ def test_scatter_minmax_lds_cached_variant(capi, oracle, shape, reduce, dtype, m
 @pytest.mark.parametrize("shape,reduce,dtype", list(product(
     [(1, 60000, 32, 300), (2, 40000, 16, 700), (1, 50000, 128, 90), (1, 30000, 24, 5000), (1, 20000, 64, 100000),
      (3, 9000, 512, 5), (1, 70000, 17, 40),
+     (2, 30000, 64, 40000),   # 625 buckets over two batch rows: the place pass that sorts its tile in LDS
      (1, 8000, 1024, 50), (2, 5000, 768, 33)],   # rows wider than a table row: reduced in slices of columns
     ["min", "max"], [torch.float32, torch.bfloat16, torch.int32, torch.int8]))
     + [((1, 20000, 64, 600000), "max", torch.float32), ((1, 20000, 64, 600000), "min", torch.int32),  # 4688 buckets
@@ -758,7 +759,7 @@ def test_scatter_minmax_skew_probe(capi, oracle, shape, kind, reduce, dtype, mon
 
 @pytest.mark.parametrize("shape,kind,dtype", list(product(
     [(1, 60000, 32, 300), (2, 40000, 16, 700), (1, 50000, 128, 90), (1, 20000, 64, 100000), (3, 9000, 256, 5),
-     (1, 30000, 24, 500),
+     (1, 30000, 24, 500), (2, 30000, 64, 40000),
      (1, 8000, 1024, 50), (2, 5000, 96, 330)],   # reduced in slices of columns (96: no power of two of lanes)
     ["zipf", "sorted", "one descent"],
     [torch.float32, torch.float64, torch.bfloat16, torch.float16, torch.int32, torch.int64, torch.int16]))
