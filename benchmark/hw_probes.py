@@ -347,10 +347,51 @@ def counters_scatter():
     print(json.dumps({"probe": "scatter done", **done}))
 
 
+def lane_moves():
+    """The kernels whose fixed-pattern cross-lane steps run in the vector ALU (csrc/dpp.h): HIP-event times of ten
+    calls each on stderr, and, under `rocprofv3 --pmc SQ_INSTS_VALU SQ_INSTS_SALU SQ_INSTS_LDS SQ_WAVE_CYCLES
+    SQ_BUSY_CYCLES -- python3 -m benchmark.hw_probes --lane-moves`, their instruction counts per dispatch. Run
+    against a library built with -DTS_DPP_OFF (make -B EXTRA=-DTS_DPP_OFF, then make torch) it gives the same
+    kernels with every such step as a shuffle through LDS."""
+    import torch
+    import pytorch_scatter_amd as ts
+    from pytorch_scatter_amd import workloads as wl
+    dev = torch.device("cuda:0")
+    w3 = wl.c3_segment_coo()
+    index, indptr = w3.index.to(dev), w3.indptr.to(dev)
+    src8, g8 = torch.randn((w3.E, 8), device=dev), torch.randn((w3.E, 8), device=dev)
+    src1, out1 = torch.randn((w3.E, 1), device=dev), torch.empty((w3.N, 1), device=dev)
+    src64 = torch.randn((w3.E, 64), device=dev)
+    x = src8.clone().requires_grad_(True)
+    y = ts.scatter_softmax(x, index, 0, w3.N)
+    cases = {
+        "scatter_softmax forward, sorted index, K=8": lambda: ts.scatter_softmax(src8, index, 0, w3.N),
+        "scatter_softmax backward, sorted index, K=8": lambda: torch.autograd.grad(y, x, g8, retain_graph=True),
+        "segment_csr sum, K=1": lambda: ts.segment_csr(src1, indptr, out1, "sum"),
+        "segment_csr max, K=1": lambda: ts.segment_max_csr(src1, indptr),
+        "gather_csr, K=1": lambda: ts.gather_csr(out1, indptr, src1),
+        "scatter sum, sorted index, K=64": lambda: ts.scatter_sum(src64, index, 0, None, w3.N),
+        "scatter sum, sorted index, K=8": lambda: ts.scatter_sum(src8, index, 0, None, w3.N),
+    }
+    w4 = wl.c4_scatter_minmax(32)
+    s4, i4 = wl.scatter_values(w4, dev), w4.index.to(dev)
+    cases["C4 scatter max, K=32"] = lambda: ts.scatter_max(s4, i4, 0, None, w4.N)
+    rows = []
+    for name, fn in cases.items():
+        if "backward" in name:
+            t = event_time(fn, 10)
+        else:
+            with torch.no_grad():
+                t = event_time(fn, 10)
+        rows.append({"case": name, "us": round(t * 1e6, 1)})
+        print(f"{name:48s} {t * 1e6:9.1f} us", file=sys.stderr)
+    print(json.dumps({"probe": "lane moves", "rows": rows}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     for flag in ("--ceilings", "--ceiling-matrix", "--atomics", "--counters", "--counters-scatter",
-                 "--sweep-thresholds", "--sweep-orders"):
+                 "--sweep-thresholds", "--sweep-orders", "--lane-moves"):
         ap.add_argument(flag, action="store_true")
     args = ap.parse_args()
     if args.ceilings:
@@ -367,6 +408,8 @@ def main():
         return sweep_thresholds()
     if args.sweep_orders:
         return sweep_orders()
+    if args.lane_moves:
+        return lane_moves()
     ap.print_help()
 
 

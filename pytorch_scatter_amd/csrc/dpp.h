@@ -49,7 +49,13 @@ __device__ __forceinline__ T mov(T old, T x) {
 }  // namespace dpp
 
 // value of lane i - 1; lane 0 keeps its own (what __shfl_up(x, 1) returns)
-template <typename T> __device__ __forceinline__ T lane_up1(T x) { return dpp::mov<dpp::kWaveShr1>(x, x); }
+template <typename T> __device__ __forceinline__ T lane_up1(T x) {
+#if defined(TS_DPP_OFF)  // build switch for measurements: every helper of this file through the LDS crossbar again
+  return __shfl_up(x, 1);
+#else
+  return dpp::mov<dpp::kWaveShr1>(x, x);
+#endif
+}
 __device__ __forceinline__ int64_t lane_up1_64(int64_t x) {
   const int lo = lane_up1((int)(uint32_t)x), hi = lane_up1((int)(x >> 32));
   return (int64_t)(((uint64_t)(uint32_t)hi << 32) | (uint32_t)lo);
@@ -58,6 +64,9 @@ __device__ __forceinline__ int64_t lane_up1_64(int64_t x) {
 // value of lane i ^ OFF, OFF a power of two below 64 (what __shfl_xor(x, OFF) returns)
 template <int OFF, typename T> __device__ __forceinline__ T lane_xor(T x) {
   static_assert(OFF == 1 || OFF == 2 || OFF == 4 || OFF == 8 || OFF == 16 || OFF == 32, "power of two below 64");
+#if defined(TS_DPP_OFF)
+  return __shfl_xor(x, OFF);
+#endif
   if constexpr (OFF == 1) {
     return dpp::mov<dpp::kQuadXor1>(x, x);
   } else if constexpr (OFF == 2) {
@@ -84,6 +93,9 @@ template <int OFF, typename T> __device__ __forceinline__ T lane_xor(T x) {
 // an unspecified lane's value, which such a tree never uses
 template <int OFF, typename T> __device__ __forceinline__ T lane_down(T x) {
   static_assert(OFF == 1 || OFF == 2 || OFF == 4 || OFF == 8 || OFF == 16 || OFF == 32, "power of two below 64");
+#if defined(TS_DPP_OFF)
+  return __shfl_down(x, OFF);
+#endif
   if constexpr (OFF < 16) {
     return dpp::mov<dpp::kRowShl + OFF>(x, x);
   } else if constexpr (OFF == 16) {
@@ -137,6 +149,14 @@ template <typename T, typename Op> __device__ __forceinline__ T group_butterfly(
 // inclusive prefix sum over the 64 lanes of a wavefront (int32): four steps inside the rows, then lane 15 of rows 0
 // and 2 into rows 1 and 3, then lane 31 into rows 2 and 3
 __device__ __forceinline__ int wave_inclusive_sum(int x) {
+#if defined(TS_DPP_OFF)
+  const int lane = threadIdx.x & 63;
+  for (int d = 1; d < 64; d <<= 1) {
+    const int y = __shfl_up(x, d);
+    if (lane >= d) x += y;
+  }
+  return x;
+#endif
   x += __builtin_amdgcn_update_dpp(0, x, dpp::kRowShr + 1, 0xf, 0xf, true);
   x += __builtin_amdgcn_update_dpp(0, x, dpp::kRowShr + 2, 0xf, 0xf, true);
   x += __builtin_amdgcn_update_dpp(0, x, dpp::kRowShr + 4, 0xf, 0xf, true);
