@@ -388,10 +388,39 @@ def lane_moves():
     print(json.dumps({"probe": "lane moves", "rows": rows}))
 
 
+def value_buckets():
+    """Sums and means of one float per entry under an index in random order, at the sizes of the two large row
+    structures of the benchmark tables: this library against torch's scatter_add_ (HIP-event times on stderr); under
+    `rocprofv3 --kernel-trace --stats` the passes of the value buckets (count, scan, place, add) one by one."""
+    import torch
+    import pytorch_scatter_amd as ts
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(0)
+    rows = []
+    with torch.no_grad():
+        for name, N, E in (("StocF-1465-like", 1_465_137, 21_005_389), ("ldoor-like", 952_203, 46_522_475)):
+            index = torch.randint(0, N, (E,), generator=g).to(dev)
+            src = torch.randn((E, 1), device=dev)
+            out = torch.zeros((N, 1), device=dev)
+            idx2 = index.view(-1, 1)
+            t_sum = event_time(lambda: ts.scatter_sum(src, index, 0, None, N), 10)
+            t_mean = event_time(lambda: ts.scatter_mean(src, index, 0, None, N), 10)
+            t_torch = event_time(lambda: out.zero_().scatter_add_(0, idx2, src), 10)
+            want = torch.zeros((N, 1), dtype=torch.float64, device=dev).index_add_(0, index, src.double())
+            got = ts.scatter_sum(src, index, 0, None, N)
+            ok = bool(torch.allclose(got.double(), want, rtol=1e-5, atol=1e-4))
+            rows.append({"structure": name, "N": N, "E": E, "sum_us": round(t_sum * 1e6, 1), "mean_us": round(t_mean * 1e6, 1),
+                         "torch_scatter_add_us": round(t_torch * 1e6, 1), "sum_matches_fp64": ok})
+            print(f"{name:18s} N {N:8d} E {E:9d}  sum {t_sum * 1e6:8.1f} us  mean {t_mean * 1e6:8.1f} us  "
+                  f"torch scatter_add_ {t_torch * 1e6:8.1f} us  sum matches fp64 index_add_: {ok}", file=sys.stderr)
+            del index, src, out, idx2, want, got
+    print(json.dumps({"probe": "value buckets", "rows": rows}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     for flag in ("--ceilings", "--ceiling-matrix", "--atomics", "--counters", "--counters-scatter",
-                 "--sweep-thresholds", "--sweep-orders", "--lane-moves"):
+                 "--sweep-thresholds", "--sweep-orders", "--lane-moves", "--value-buckets"):
         ap.add_argument(flag, action="store_true")
     args = ap.parse_args()
     if args.ceilings:
@@ -410,6 +439,8 @@ def main():
         return sweep_orders()
     if args.lane_moves:
         return lane_moves()
+    if args.value_buckets:
+        return value_buckets()
     ap.print_help()
 
 
