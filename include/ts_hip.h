@@ -291,6 +291,19 @@ int ts_scatter_count_with_workspace(const int64_t *index, int32_t *count, int64_
                                     int64_t index_stride_e, void *workspace,
                                     size_t workspace_bytes, ts_stream_t stream);
 
+/* Sum and entries per output row in one call: the two halves of ScatterMean::forward, csrc/scatter.cpp:122-141,
+ * before its division, for one index per row (index[b * index_stride_b + e * index_stride_e]). out as
+ * ts_scatter_with_workspace(reduce = sum, index_stride_k = 0) leaves it, count as ts_scatter_count leaves it. When
+ * the sum goes through buckets of output rows (ts_scatter_sum_count_workspace_bytes() of scratch: wide rows from
+ * 64 MB, single 4-byte values from 2 M entries) the index is read and binned once for both: the adding pass keeps
+ * a table of counts beside its sums. Every other case is the two calls in a row. */
+size_t ts_scatter_sum_count_workspace_bytes(int64_t B, int64_t E, int64_t K, int64_t N, int dtype);
+int ts_scatter_sum_count_with_workspace(const void *src, const int64_t *index, void *out,
+                                        int32_t *count, int64_t B, int64_t E, int64_t K, int64_t N,
+                                        int64_t index_stride_b, int64_t index_stride_e,
+                                        int dtype, int out_given, void *workspace,
+                                        size_t workspace_bytes, ts_stream_t stream);
+
 /* out[b, n, k] = out[b, n, k] / (T)max(count[b, n], 1): true division for
  * floating types, floor division for integers (csrc/scatter.cpp:138-141). */
 int ts_divide_by_count(void *out, const int32_t *count, int64_t B, int64_t N,

@@ -26,7 +26,7 @@ EXPORTS = (
     "ts_segment_mean_csr_backward",
     "ts_segment_coo_workspace_bytes", "ts_segment_coo", "ts_gather_coo",
     "ts_segment_mean_coo_backward",
-    "ts_scatter", "ts_scatter_workspace_bytes", "ts_scatter_workspace_zero_bytes", "ts_scatter_with_workspace", "ts_scatter_count", "ts_scatter_count_workspace_bytes", "ts_scatter_count_with_workspace", "ts_divide_by_count", "ts_arg_backward",
+    "ts_scatter", "ts_scatter_workspace_bytes", "ts_scatter_workspace_zero_bytes", "ts_scatter_with_workspace", "ts_scatter_count", "ts_scatter_count_workspace_bytes", "ts_scatter_count_with_workspace", "ts_scatter_sum_count_workspace_bytes", "ts_scatter_sum_count_with_workspace", "ts_divide_by_count", "ts_arg_backward",
     "ts_group_softmax_workspace_bytes", "ts_group_softmax", "ts_group_softmax_backward",
     "ts_group_logsumexp", "ts_group_logsumexp_backward",
     "ts_group_std", "ts_group_std_backward",
@@ -59,6 +59,7 @@ def lib() -> ctypes.CDLL:
         _lib.ts_scatter_workspace_bytes.restype = ctypes.c_size_t
         _lib.ts_scatter_workspace_zero_bytes.restype = ctypes.c_size_t
         _lib.ts_scatter_count_workspace_bytes.restype = ctypes.c_size_t
+        _lib.ts_scatter_sum_count_workspace_bytes.restype = ctypes.c_size_t
         _lib.ts_sort_index_workspace_bytes.restype = ctypes.c_size_t
         _lib.ts_segment_csr_permuted_workspace_bytes.restype = ctypes.c_size_t
     return _lib
@@ -229,6 +230,19 @@ def scatter_count_with_workspace(index, count, B, E, N, sb, se):
     with torch.cuda.device(count.device):
         _check(L.ts_scatter_count_with_workspace(_p(index), _p(count), _i(B), _i(E), _i(N), _i(sb), _i(se),
                                                  _p(ws) if nbytes else None, ctypes.c_size_t(nbytes), _stream(count)))
+    return nbytes
+
+
+def scatter_sum_count_with_workspace(src, index, out, count, B, E, K, N, sb, se, out_given: bool):
+    """Sum and int32 count of the entries per output row in one call (ts_scatter_sum_count_with_workspace)."""
+    _dev(src, index, out, count)
+    L = lib()
+    nbytes = L.ts_scatter_sum_count_workspace_bytes(_i(B), _i(E), _i(K), _i(N), DTYPE[out.dtype])
+    ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=out.device)
+    with torch.cuda.device(out.device):
+        _check(L.ts_scatter_sum_count_with_workspace(_p(src), _p(index), _p(out), _p(count), _i(B), _i(E), _i(K), _i(N),
+                                                     _i(sb), _i(se), DTYPE[out.dtype], 1 if out_given else 0,
+                                                     _p(ws) if nbytes else None, ctypes.c_size_t(nbytes), _stream(out)))
     return nbytes
 
 

@@ -596,10 +596,13 @@ int ts_scatter(const void *src, const int64_t *index, void *out, int64_t *arg_ou
                                    index_stride_k, dtype, reduce, out_given, nullptr, 0, stream);
 }
 
-int ts_scatter_with_workspace(const void *src, const int64_t *index, void *out, int64_t *arg_out, int64_t B,
-                              int64_t E, int64_t K, int64_t N, int64_t index_stride_b, int64_t index_stride_e,
-                              int64_t index_stride_k, int dtype, int reduce, int out_given, void *workspace,
-                              size_t workspace_bytes, ts_stream_t stream) {
+}  // extern "C"
+namespace {
+// ts_scatter_with_workspace; count_out / count_flag: see ScatterArgs (a sum through the buckets that counts as well)
+int scatter_ws_impl(const void *src, const int64_t *index, void *out, int64_t *arg_out, int64_t B,
+                    int64_t E, int64_t K, int64_t N, int64_t index_stride_b, int64_t index_stride_e,
+                    int64_t index_stride_k, int dtype, int reduce, int out_given, void *workspace,
+                    size_t workspace_bytes, ts_stream_t stream, int32_t *count_out, const int **count_flag) {
   if (!valid_dtype(dtype) || !sizes_ok(B, N, E, K)) return TS_ERR_BAD_ARG;
   if (reduce != TS_SUM && reduce != TS_MUL && reduce != TS_MIN && reduce != TS_MAX) return TS_ERR_UNSUPPORTED;
   if (B * N * K == 0) return TS_OK;
@@ -618,6 +621,8 @@ int ts_scatter_with_workspace(const void *src, const int64_t *index, void *out, 
   a.se = index_stride_e;
   a.sk = index_stride_k;
   a.out_given = out_given ? 1 : 0;
+  a.count_out = count_out;
+  a.count_flag = count_flag;
   a.precheck = env_int("TS_SCATTER_PRECHECK", 1);   // tuning aids
   a.lds_cache = env_int("TS_SCATTER_LDS", 1);
   a.lds_epb = env_int("TS_SCATTER_EPB", 0);
@@ -661,6 +666,16 @@ int ts_scatter_with_workspace(const void *src, const int64_t *index, void *out, 
   return run_csr_reduce(src, a.route_ptr, out, arg_out, nullptr, B, N, E, K, N + 1, dtype, reduce, 0,
                         static_cast<char *>(workspace) + bin_bytes + sr.ptr_bytes, sr.csr_bytes, nullptr, s, nullptr, 0,
                         nullptr, route_flag, 1);
+}
+}  // namespace
+extern "C" {
+
+int ts_scatter_with_workspace(const void *src, const int64_t *index, void *out, int64_t *arg_out, int64_t B,
+                              int64_t E, int64_t K, int64_t N, int64_t index_stride_b, int64_t index_stride_e,
+                              int64_t index_stride_k, int dtype, int reduce, int out_given, void *workspace,
+                              size_t workspace_bytes, ts_stream_t stream) {
+  return scatter_ws_impl(src, index, out, arg_out, B, E, K, N, index_stride_b, index_stride_e, index_stride_k, dtype, reduce,
+                         out_given, workspace, workspace_bytes, stream, nullptr, nullptr);
 }
 
 size_t ts_scatter_count_workspace_bytes(int64_t B, int64_t E, int64_t N) {
@@ -743,6 +758,73 @@ int ts_scatter_count_with_workspace(const int64_t *index, int32_t *count, int64_
                          index_stride_b, index_stride_e);
     }
   }
+  return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
+}
+
+size_t ts_scatter_sum_count_workspace_bytes(int64_t B, int64_t E, int64_t K, int64_t N, int dtype) {
+  const size_t sum = ts_scatter_workspace_bytes(B, E, K, N, dtype, TS_SUM);
+  const size_t cnt = ts_scatter_count_workspace_bytes(B, E, N);
+  return sum > cnt ? sum : cnt;
+}
+
+int ts_scatter_sum_count_with_workspace(const void *src, const int64_t *index, void *out, int32_t *count, int64_t B,
+                                        int64_t E, int64_t K, int64_t N, int64_t index_stride_b,
+                                        int64_t index_stride_e, int dtype, int out_given, void *workspace,
+                                        size_t workspace_bytes, ts_stream_t stream) {
+  if (!valid_dtype(dtype) || !sizes_ok(B, N, E, K)) return TS_ERR_BAD_ARG;
+  if (B * N == 0) return TS_OK;
+  if (!count) return TS_ERR_BAD_ARG;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  // The sum. If it goes through the buckets, their adding pass counts as well (one pass over the index for both) and
+  // leaves the buckets' flag here: 1 = the buckets took the call.
+  const int *flag = nullptr;
+  bool may_fuse = B * E * K > 0 && workspace != nullptr && B * N < 0x7FFFFFFFll && env_int("TS_SCATTER_RUNS", 1) &&
+                  env_int("TS_SCATTER_LDS", 1) && env_int("TS_SCATTER_BINNED", 1);
+  if (may_fuse) {  // only where the sum has a plan for the buckets (else count is cleared by its own call below)
+    const bool any_size = env_int("TS_SCATTER_BINNED", 1) == 2;
+    bool planned = kAccBytes[dtype] >= 4 && bin_plan(B, E, K, N, kElemBytes[dtype], workspace, workspace_bytes, any_size,
+                                                     dtype == TS_I32 ? 4 : 8, false, true).ok;
+    if (!planned && K == 1 && kElemBytes[dtype] == 4)
+      planned = bin_plan_payload(B, E, 1, N, 4, workspace, workspace_bytes, any_size).ok;
+    may_fuse = planned;
+  }
+  if (may_fuse)
+    hipLaunchKernelGGL(fill_kernel<int32_t>, dim3(grid_for(B * N)), dim3(kBlock), 0, s, count, B * N, (int32_t)0);
+  const int rc = scatter_ws_impl(src, index, out, nullptr, B, E, K, N, index_stride_b, index_stride_e, 0, dtype, TS_SUM,
+                                 out_given, workspace, workspace_bytes, stream, may_fuse ? count : nullptr,
+                                 may_fuse ? &flag : nullptr);
+  if (rc != TS_OK) return rc;
+  if (flag == nullptr)  // another route: the count on its own (with its own fill)
+    return ts_scatter_count_with_workspace(index, count, B, E, N, index_stride_b, index_stride_e, workspace, workspace_bytes,
+                                           stream);
+  // the kernels behind the buckets, for the counts: the table for a skewed index (flag 2, single values only), runs for
+  // a sorted one (flag 0)
+  ScatterArgs c;
+  c.src = nullptr;
+  c.index = index;
+  c.out = count;
+  c.arg_out = nullptr;
+  c.B = B;
+  c.E = E;
+  c.K = 1;
+  c.N = N;
+  c.sb = index_stride_b;
+  c.se = index_stride_e;
+  c.sk = 0;
+  c.out_given = 1;
+  c.precheck = 1;
+  c.lds_cache = env_int("TS_SCATTER_LDS", 1);
+  c.lds_epb = env_int("TS_SCATTER_EPB", 0);
+  c.skip_flag = flag;
+  if (K == 1) {
+    ScatterArgs t = c;
+    t.skip_want = 2;
+    const int64_t epb = per_cu_chunk_edges(c.lds_epb, B * E, sum_table_min_chunk(1, 4), 131072);
+    hipLaunchKernelGGL(scatter_add_lds_kernel<int32_t>, dim3((unsigned)((B * E + epb - 1) / epb)), dim3(kLdsAddBlock), 0, s,
+                       t, kLdsAccRows - 1, epb);
+  }
+  const RunGrid g = run_grid(B * E, 1, 1, 4);
+  launch_add_run<int32_t, 1, 1>(c, g, s);
   return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
 }
 

@@ -236,6 +236,10 @@ struct ScatterArgs {
   const int *skip_flag = nullptr;  // sum kernels: leave at once if *skip_flag != 0 (the binned pass did the work)
   int skip_inverse = 0;            // ... if *skip_flag == 0 instead
   int skip_want = -1;              // >= 0 (table kernel only): run only if *skip_flag == skip_want
+  int32_t *count_out = nullptr;    // sum through the buckets: also count the entries of every output row into this
+                                   // zeroed [B * N] array ...
+  const int **count_flag = nullptr;  // ... and leave the buckets' flag here (still null afterwards: the call took another
+                                   // route and nothing was counted)
   int *order_ws = nullptr;         // sum of narrow rows: a word of scratch for the sample of the index that picks the kernel
   int skew_probe = 1;              // min/max: sample the index for skew (needs 256 bytes of workspace): 0 never, 2 at any size
   const int *skew_flag = nullptr;  // min/max kernels behind the probe: run only if (*skew_flag != 0) == (skew_want != 0)
@@ -1882,6 +1886,10 @@ int launch_scatter_v(const ScatterArgs &args, int reduce, hipStream_t stream) {
       if (lshift >= 0) {
         ts_note_scatter_route(payload ? TS_ROUTE_SUM_VALUE_BUCKETS : routed ? TS_ROUTE_SUM_BUCKETS_OR_SEGMENTED
                                                                               : TS_ROUTE_SUM_BUCKETS_OR_RUNS);
+        if (a.count_out != nullptr && a.count_flag != nullptr && (payload || bp.p.rshift <= kBinCountShift)) {
+          bp.p.count_out = a.count_out;
+          *a.count_flag = bp.p.unsorted;
+        }
         launch_binned_add<T, VEC>(a, bp.p, lshift, stream, routed ? n_out : 0, three_way);
         a.skip_flag = bp.p.unsorted;
         if (routed) {

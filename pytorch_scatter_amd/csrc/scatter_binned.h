@@ -27,6 +27,7 @@ constexpr int kBinChunk = 8192;       // entries per chunk of a bucket in reduce
 constexpr int kBinPlaceChunk = 10240;  // most entries per workgroup in place: one batch of 10 per lane
 constexpr int kCombPos = 64;          // combining kernel: keys per step of a bucket of many chunks,
 constexpr int kCombFew = 32;          // many: more than this
+constexpr int kBinCountShift = 10;   // rows per bucket (log2) up to which bin_add_wave_kernel can count entries per row as well
 constexpr int kBinPlaceBlock = 1024;   // (measured slower: 256 lanes x 4 batches, 64 K entries per workgroup, 8 K)
 
 struct BinArgs {
@@ -61,6 +62,8 @@ struct BinArgs {
                            // (bin_sample_kernel); then the count pass returns at once as well
   int payload = 0;         // sum of one 4-byte value per entry: the low half of a binned word holds the value's bits
                            // instead of the entry number, so the reducing pass never goes back to src
+  int32_t *count_out = nullptr;  // sums: the adding pass also counts the entries of every output row into this
+                           // [B * N] array (the divisor of a mean, from the same words); row buckets: rshift <= kBinCountShift
 };
 
 struct BinPlan {
@@ -1013,6 +1016,7 @@ __global__ __launch_bounds__(kBinBlock) void bin_add_wave_kernel(ScatterArgs a, 
   constexpr int U = 4;
   constexpr int kSlots = (kBinKeys + kBinKeys / 16) * 8 / (int)sizeof(A);
   __shared__ A s_acc[kSlots];  // rows K + 1 slots apart (LDS banks)
+  __shared__ int32_t s_num[1 << kBinCountShift];  // entries per row, for a caller that wants them (BinArgs::count_out)
   if (p.unsorted != nullptr && *p.unsorted != 1) return;
   const int wg = (int)(blockIdx.x / (unsigned)p.slices), slice = (int)(blockIdx.x - (unsigned)wg * p.slices);
   const int bucket = p.wg_bucket[wg];
@@ -1020,7 +1024,10 @@ __global__ __launch_bounds__(kBinBlock) void bin_add_wave_kernel(ScatterArgs a, 
   const int K = (int)a.K, kc = p.kc;
   const int KP = kc + 1;
   const int rows = 1 << p.rshift;
+  const bool counting = p.count_out != nullptr && slice == 0;  // the workgroups of one column slice count
   for (int i = threadIdx.x; i < rows * KP; i += kBinBlock) s_acc[i] = (A)0;
+  if (counting)
+    for (int i = threadIdx.x; i < rows; i += kBinBlock) s_num[i] = 0;
   __syncthreads();
 
   const T *src = static_cast<const T *>(a.src);
@@ -1060,6 +1067,8 @@ __global__ __launch_bounds__(kBinBlock) void bin_add_wave_kernel(ScatterArgs a, 
 #pragma unroll
           for (int v = 0; v < VEC; ++v)
             __hip_atomic_fetch_add(row + v, (A)to_acc<T>(x[u].v[v]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+          if (counting && k0 == 0)  // the lane with the row's first columns
+            __hip_atomic_fetch_add(&s_num[e_row[u]], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
         }
       }
     }
@@ -1068,6 +1077,12 @@ __global__ __launch_bounds__(kBinBlock) void bin_add_wave_kernel(ScatterArgs a, 
   T *out = static_cast<T *>(a.out) + ((int64_t)bucket << p.rshift) * a.K + c0;
   const int64_t rows_left = a.B * a.N - ((int64_t)bucket << p.rshift);  // rows that exist
   const int table = kc << p.rshift;
+  if (counting) {
+    for (int i = threadIdx.x; i < rows && i < rows_left; i += kBinBlock) {
+      const int32_t c = s_num[i];
+      if (c != 0) atomicAdd(p.count_out + ((int64_t)bucket << p.rshift) + i, c);
+    }
+  }
   if constexpr (sizeof(T) == 2) {
     // two neighbouring columns per packed atomic (kc is even here: whole 16-byte vectors per lane)
     if ((reinterpret_cast<uintptr_t>(a.out) & 3) == 0) {
@@ -1111,19 +1126,24 @@ __global__ __launch_bounds__(kBinBlock) void bin_add_wave_kernel(ScatterArgs a, 
 // its chunk of a bucket with 16-byte loads (two words per lane, four loads in flight), adds into the bucket's table
 // in LDS (double slots for floats: ds_add_f64 keeps its rate when many lanes meet on one address, a hub row) and
 // adds every row it touched to out once.
-template <typename T>
+// COUNT: the entries of every row are counted as well (BinArgs::count_out), in a second table.
+template <typename T, bool COUNT = false>
 __global__ __launch_bounds__(kBinBlock) void bin_add_payload_kernel(ScatterArgs a, BinArgs p) {
   static_assert(sizeof(T) == 4, "one 4-byte value per word");
   typedef typename BinSlot<T>::type A;
   typedef unsigned long long u64x2 __attribute__((ext_vector_type(2)));
   constexpr int U = 4;
   __shared__ A s_acc[4096];
+  __shared__ int32_t s_num[COUNT ? 4096 : 1];
   if (p.unsorted != nullptr && *p.unsorted != 1) return;
   const int wg = (int)blockIdx.x;
   const int bucket = p.wg_bucket[wg];
   if (bucket < 0) return;
   const int rows = 1 << p.rshift;
-  for (int i = threadIdx.x; i < rows; i += kBinBlock) s_acc[i] = (A)0;
+  for (int i = threadIdx.x; i < rows; i += kBinBlock) {
+    s_acc[i] = (A)0;
+    if (COUNT) s_num[i] = 0;
+  }
   __syncthreads();
   const int64_t lo = p.starts[bucket] + ((int64_t)wg - p.chunk_start[bucket]) * p.chunk;
   int64_t hi = lo + p.chunk;
@@ -1132,8 +1152,9 @@ __global__ __launch_bounds__(kBinBlock) void bin_add_payload_kernel(ScatterArgs 
     T v;
     const uint32_t bits = (uint32_t)w;
     __builtin_memcpy(&v, &bits, 4);
-    __hip_atomic_fetch_add(&s_acc[(uint32_t)(w >> 32) & (uint32_t)(rows - 1)], (A)v, __ATOMIC_RELAXED,
-                           __HIP_MEMORY_SCOPE_WORKGROUP);
+    const uint32_t row = (uint32_t)(w >> 32) & (uint32_t)(rows - 1);
+    __hip_atomic_fetch_add(&s_acc[row], (A)v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    if (COUNT) __hip_atomic_fetch_add(&s_num[row], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
   };
   if (lo < hi) {
     // words lo .. hi - 1; the 16-byte loads start at an even word
@@ -1163,6 +1184,10 @@ __global__ __launch_bounds__(kBinBlock) void bin_add_payload_kernel(ScatterArgs 
   for (int i = threadIdx.x; i < rows && i < rows_left; i += kBinBlock) {
     const A v = s_acc[i];
     if (v != (A)0) atomic_add_elem<T>(out + i, (T)v);
+    if (COUNT) {
+      const int32_t c = s_num[i];
+      if (c != 0) atomicAdd(p.count_out + ((int64_t)bucket << p.rshift) + i, c);
+    }
   }
 }
 
@@ -1269,7 +1294,10 @@ void launch_binned_add(const ScatterArgs &a, const BinArgs &plan, int lshift, hi
     hipLaunchKernelGGL(bin_place_kernel<kBinMaxBuckets>, dim3((unsigned)p.n_place), dim3(kBinPlaceBlock), 0, stream, a, p);
   if constexpr (sizeof(T) == 4 && VEC == 1) {
     if (p.payload) {
-      hipLaunchKernelGGL(bin_add_payload_kernel<T>, dim3((unsigned)p.max_wgs), dim3(kBinBlock), 0, stream, a, p);
+      if (p.count_out != nullptr)
+        hipLaunchKernelGGL((bin_add_payload_kernel<T, true>), dim3((unsigned)p.max_wgs), dim3(kBinBlock), 0, stream, a, p);
+      else
+        hipLaunchKernelGGL((bin_add_payload_kernel<T, false>), dim3((unsigned)p.max_wgs), dim3(kBinBlock), 0, stream, a, p);
       return;
     }
   }

@@ -178,8 +178,11 @@ BatchedIndex batched_index(const Tensor &idx) {
 
 // ------------------------------------------------------------------ scatter
 // host half of scatter_cuda (csrc/cuda/scatter_cuda.cu:58-138)
+// mean_count (sum only): if the call is a sum under one index per row, the entries of every output row are counted
+// in the same call (ts_scatter_sum_count_with_workspace) and the int32 counts [B * N]
+// are left here; else it stays undefined
 std::tuple<Tensor, OptTensor> scatter_hip(Tensor src, Tensor index, int64_t dim, OptTensor optional_out,
-                                          OptInt dim_size, int reduce) {
+                                          OptInt dim_size, int reduce, Tensor *mean_count = nullptr) {
   check_device(src, "src");
   check_device(index, "index");
   if (optional_out.has_value()) check_device(optional_out.value(), "out");
@@ -245,6 +248,18 @@ std::tuple<Tensor, OptTensor> scatter_hip(Tensor src, Tensor index, int64_t dim,
     sb = E * K;
     se = K;
     sk = 1;
+  }
+  if (mean_count != nullptr && reduce == TS_SUM && sk.value() == 0 && B * N < 0x7FFFFFFFll) {
+    const size_t cs_bytes = ts_scatter_sum_count_workspace_bytes(B, E, K, N, dtype_code(src));
+    Tensor cws = workspace(cs_bytes, src);
+    Tensor count = at::empty({B * N}, src.options().dtype(at::kInt));
+    check_status(ts_scatter_sum_count_with_workspace(src.data_ptr(), index.data_ptr<int64_t>(), out.data_ptr(),
+                                                     count.data_ptr<int32_t>(), B, E, K, N, sb.value(), se, dtype_code(src),
+                                                     optional_out.has_value() ? 1 : 0,
+                                                     cs_bytes > 0 ? cws.data_ptr() : nullptr, cs_bytes, stream_of(src)),
+                 "scatter (sum and count)");
+    *mean_count = count;
+    return std::make_tuple(out, OptTensor());
   }
   // min / max of large inputs with wide rows can use scratch memory (entries binned by bucket of output rows)
   const size_t ws_bytes = sk.value() == 0 ? ts_scatter_workspace_bytes(B, E, K, N, dtype_code(src), reduce) : 0;
@@ -567,7 +582,9 @@ template <int REDUCE> struct ScatterFn : public torch::autograd::Function<Scatte
     ctx->saved_data["src_shape"] = src.sizes();
     Variable old_index = index;
     index = broadcast(index, src, dim);
-    auto result = scatter_hip(src, index, dim, optional_out, dim_size, REDUCE == TS_MEAN ? TS_SUM : REDUCE);
+    Tensor fused_count;  // mean of single values: counted together with the sum
+    auto result = scatter_hip(src, index, dim, optional_out, dim_size, REDUCE == TS_MEAN ? TS_SUM : REDUCE,
+                              REDUCE == TS_MEAN ? &fused_count : nullptr);
     Variable out = std::get<0>(result);
     if (optional_out.has_value()) ctx->mark_dirty({optional_out.value()});
     if (REDUCE == TS_SUM) {
@@ -590,14 +607,19 @@ template <int REDUCE> struct ScatterFn : public torch::autograd::Function<Scatte
         const BatchedIndex bi = batched_index(old_index);
         // one index row shared by every batch row (an expanded view): counted once and repeated
         const int64_t Bc = (bi.batch_stride == 0 && B > 1) ? 1 : B;
-        Tensor count_f = at::empty({Bc * N}, src.options().dtype(at::kInt));
-        const size_t cws_bytes = ts_scatter_count_workspace_bytes(Bc, E, N);
-        Tensor cws = workspace(cws_bytes, src);
-        check_status(ts_scatter_count_with_workspace(bi.t.data_ptr<int64_t>(), count_f.data_ptr<int32_t>(), Bc, E, N,
-                                                     bi.batch_stride, 1, cws_bytes > 0 ? cws.data_ptr() : nullptr,
-                                                     cws_bytes, stream_of(src)),
-                     "scatter_mean count");
-        if (Bc != B) count_f = count_f.view({1, N}).expand({B, N}).contiguous().view({B * N});
+        Tensor count_f;
+        if (fused_count.defined() && fused_count.numel() == B * N) {
+          count_f = fused_count;
+        } else {
+          count_f = at::empty({Bc * N}, src.options().dtype(at::kInt));
+          const size_t cws_bytes = ts_scatter_count_workspace_bytes(Bc, E, N);
+          Tensor cws = workspace(cws_bytes, src);
+          check_status(ts_scatter_count_with_workspace(bi.t.data_ptr<int64_t>(), count_f.data_ptr<int32_t>(), Bc, E, N,
+                                                       bi.batch_stride, 1, cws_bytes > 0 ? cws.data_ptr() : nullptr,
+                                                       cws_bytes, stream_of(src)),
+                       "scatter_mean count");
+          if (Bc != B) count_f = count_f.view({1, N}).expand({B, N}).contiguous().view({B * N});
+        }
         Tensor out_c = out.contiguous();
         check_status(ts_divide_by_count(out_c.data_ptr(), count_f.data_ptr<int32_t>(), B, N, K, dtype_code(out_c),
                                         stream_of(src)),

@@ -1749,6 +1749,55 @@ def test_scatter_sum_of_single_values_through_buckets(capi, oracle, case, dtype,
     assert torch.equal(cnt.cpu(), want_cnt)
 
 
+@pytest.mark.parametrize("case,dtype,out_given,forced", product(
+    PAYLOAD_CASES + [(1, 90001, 5000, "sorted"), (1, 200000, 30000, "skewed")], [torch.float32, torch.int32], [False, True],
+    [True, False]))
+def test_scatter_sum_and_count_in_one_call(capi, case, dtype, out_given, forced, monkeypatch):
+    """ts_scatter_sum_count_with_workspace: sum and int32 count of one value per entry from one pass over the index when
+    the value buckets take the call (forced on at these sizes), the two separate calls otherwise (forced = False: these
+    sizes are below the buckets' threshold). A sorted index (run kernels behind the buckets) and a heavily skewed one
+    (table kernel behind the buckets) leave both results to the kernels behind the buckets."""
+    if forced:
+        monkeypatch.setenv("TS_SCATTER_BINNED", "2")
+    B, E, N, kind = case
+    rng = np.random.default_rng(E + N + 1)
+    if dtype.is_floating_point:
+        src = torch.from_numpy(rng.integers(-9, 10, size=(B, E, 1)).astype(np.float32))  # small integers: exact sums
+    else:
+        src = torch.from_numpy(rng.integers(-1000, 1000, size=(B, E, 1)).astype(np.int32))
+    if kind == "zipf":
+        p = np.arange(1, N + 1, dtype=np.float64) ** -1.2
+        index = (rng.choice(N, size=(B, E), p=p / p.sum()) * 7919) % N
+    elif kind == "skewed":
+        p = np.arange(1, N + 1, dtype=np.float64) ** -2.0
+        index = (rng.choice(N, size=(B, E), p=p / p.sum()) * 7919) % N
+    elif kind == "hub":
+        index = rng.integers(0, N, size=(B, E))
+        index[:, rng.random(E) < 0.4] = N // 3
+    elif kind == "sorted":
+        index = np.sort(rng.integers(0, N, size=(B, E)), axis=1)
+    else:
+        index = rng.integers(0, N, size=(B, E))
+    index = torch.from_numpy(index.astype(np.int64))
+    if E > 100 and kind != "sorted":
+        index[0, 5] = -1
+        index[-1, 77] = N
+    valid = (index >= 0) & (index < N)
+    prev = torch.from_numpy(rng.integers(-5, 6, size=(B, N, 1))).to(dtype) if out_given else torch.zeros((B, N, 1), dtype=dtype)
+    want = prev.clone().double()
+    for b in range(B):
+        want[b, :, 0].index_add_(0, index[b][valid[b]], src[b, valid[b], 0].double())
+    want_cnt = torch.stack([torch.bincount(index[b][valid[b]], minlength=N) for b in range(B)]).int()
+    out = prev.clone().to(DEV)
+    cnt = torch.full((B, N), -7, dtype=torch.int32, device=DEV)
+    used = capi.scatter_sum_count_with_workspace(src.to(DEV), index.to(DEV), out, cnt, B, E, 1, N, E, 1, out_given)
+    torch.cuda.synchronize()
+    if forced:
+        assert used >= 8 * B * E
+    assert torch.equal(out.cpu().double(), want)
+    assert torch.equal(cnt.cpu(), want_cnt)
+
+
 def test_scatter_sum_of_single_values_sorted_index_keeps_the_run_kernels(capi, oracle, monkeypatch):
     """A sorted index: the sample sends the call to the kernels that combine runs; the bucket passes return at once."""
     monkeypatch.setenv("TS_SCATTER_BINNED", "2")

@@ -660,3 +660,33 @@ def test_operators_raise_when_a_row_was_given_up(ts):
             os.environ["TS_CSR_SPIN"] = old
     out = ts.segment_csr(src, indptr, None, "sum")
     assert torch.allclose(out[1], src[200:5000].double().sum(0).float(), rtol=1e-4, atol=1e-3)
+
+
+@pytest.mark.parametrize("kind", ["uniform", "zipf", "sorted"])
+def test_scatter_mean_of_single_values_counts_with_the_sum(kind):
+    """scatter_mean of one float per entry at a size where the value buckets take the sum: sum and count come from
+    one call (torch_ops.cpp: scatter_hip with mean_count). Values, gradient, and an integer input."""
+    import pytorch_scatter_amd as ts
+    g = torch.Generator().manual_seed(5)
+    E, N = (1 << 21) + 1234, 300_000
+    if kind == "zipf":
+        w = torch.arange(1, N + 1, dtype=torch.float64) ** -1.1
+        index = torch.multinomial(w, E, replacement=True, generator=g)
+    else:
+        index = torch.randint(0, N, (E,), generator=g)
+    if kind == "sorted":
+        index = index.sort().values
+    index = index.to(DEV)
+    src = torch.randn((E,), generator=g).to(DEV).requires_grad_(True)
+    out = ts.scatter_mean(src, index, 0, None, N)
+    cnt = torch.bincount(index, minlength=N).clamp(min=1).double()
+    want = torch.zeros(N, dtype=torch.float64, device=DEV).index_add_(0, index, src.detach().double()) / cnt
+    mags = torch.zeros(N, dtype=torch.float64, device=DEV).index_add_(0, index, src.detach().double().abs()) / cnt
+    assert bool(((out.double() - want).abs() <= 1e-5 * (want.abs() + mags)).all())
+    grad_out = torch.randn((N,), generator=g).to(DEV)
+    (grad,) = torch.autograd.grad(out, src, grad_out)
+    assert torch.allclose(grad.double(), (grad_out.double() / cnt)[index], rtol=1e-6, atol=0)
+    isrc = torch.randint(-50, 50, (E,), generator=g, dtype=torch.int32).to(DEV)
+    iout = ts.scatter_mean(isrc, index, 0, None, N)
+    isum = torch.zeros(N, dtype=torch.int64, device=DEV).index_add_(0, index, isrc.long())
+    assert torch.equal(iout.long(), torch.div(isum, cnt.long(), rounding_mode="floor"))
