@@ -298,6 +298,10 @@ def bench_softmax_config(ts, wl, w, dev, iters, K):
         t = event_time(lambda: torch.autograd.grad(y, x, gn, retain_graph=True), iters)
         res[f"std_backward_{name}"] = entry(2 * w.E * K * 4 + w.E * 8, t, w.E * K)
         del x, y
+        # logsumexp: src and index read once, N*K result
+        with torch.no_grad():
+            t = event_time(lambda: ts.scatter_logsumexp(src, idx, 0, None, w.N), iters)
+        res[f"logsumexp_{name}"] = entry(w.E * K * 4 + w.E * 8 + w.N * K * 4, t, w.E * K)
     del src, grad
     torch.cuda.empty_cache()
     return res

@@ -396,6 +396,21 @@ int ts_group_std_backward(const void *src, const int64_t *index,
                           int64_t index_stride_b, int64_t index_stride_e,
                           int dtype, int unbiased, ts_stream_t stream);
 
+/* scatter_std and scatter_logsumexp through buckets of groups (no counterpart in the reference, whose
+ * torch_scatter/composite/std.py:8-41 and logsumexp.py:8-57 compose scatter operators): the entries are binned
+ * by bucket of neighbouring groups, then src is gathered once and both sweeps of the statistic run in LDS, whatever
+ * the order of the index. ts_group_bins_workspace_bytes() is the scratch this takes, 0 when the route does not apply
+ * (small inputs, rows held by more than 32 lanes, more groups than 16384 buckets hold).
+ * ts_group_std_forward writes the group sums (total, element type), the entries per group (count, int32) and the
+ * standard deviation (out) in one call: what ts_scatter(sum) + ts_scatter_count + ts_group_std leave. It needs that
+ * workspace: TS_ERR_UNSUPPORTED when the route does not apply, TS_ERR_WORKSPACE when the workspace is too small.
+ * ts_group_logsumexp takes the same route by itself when its workspace has that size. */
+size_t ts_group_bins_workspace_bytes(int64_t B, int64_t E, int64_t K, int64_t N, int dtype);
+int ts_group_std_forward(const void *src, const int64_t *index, void *total, int32_t *count, void *out,
+                         int64_t B, int64_t E, int64_t K, int64_t N, int64_t index_stride_b,
+                         int64_t index_stride_e, int dtype, int unbiased, void *workspace,
+                         size_t workspace_bytes, ts_stream_t stream);
+
 /* ---- index formats either side of the reductions. The reference has no operator for these steps:
  * its benchmark takes `row` and `rowptr` from the same sparse matrix (benchmark/scatter_segment.py:38-41)
  * and segment_coo's documentation asks the caller for a sorted index (torch_scatter/segment_coo.py:80-83).

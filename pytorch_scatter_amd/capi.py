@@ -29,7 +29,7 @@ EXPORTS = (
     "ts_scatter", "ts_scatter_workspace_bytes", "ts_scatter_workspace_zero_bytes", "ts_scatter_with_workspace", "ts_scatter_count", "ts_scatter_count_workspace_bytes", "ts_scatter_count_with_workspace", "ts_scatter_sum_count_workspace_bytes", "ts_scatter_sum_count_with_workspace", "ts_divide_by_count", "ts_arg_backward",
     "ts_group_softmax_workspace_bytes", "ts_group_softmax", "ts_group_softmax_backward",
     "ts_group_logsumexp", "ts_group_logsumexp_backward",
-    "ts_group_std", "ts_group_std_backward",
+    "ts_group_std", "ts_group_std_backward", "ts_group_bins_workspace_bytes", "ts_group_std_forward",
     "ts_index_to_indptr", "ts_indptr_to_index_workspace_bytes", "ts_indptr_to_index",
     "ts_sort_index_workspace_bytes", "ts_sort_index",
     "ts_segment_csr_permuted_workspace_bytes", "ts_segment_csr_permuted",
@@ -61,6 +61,7 @@ def lib() -> ctypes.CDLL:
         _lib.ts_scatter_count_workspace_bytes.restype = ctypes.c_size_t
         _lib.ts_scatter_sum_count_workspace_bytes.restype = ctypes.c_size_t
         _lib.ts_sort_index_workspace_bytes.restype = ctypes.c_size_t
+        _lib.ts_group_bins_workspace_bytes.restype = ctypes.c_size_t
         _lib.ts_segment_csr_permuted_workspace_bytes.restype = ctypes.c_size_t
     return _lib
 
@@ -286,9 +287,19 @@ def group_softmax_backward(result, grad_out, index, grad_in, B, E, K, N, sb, se,
     return ws
 
 
-def group_logsumexp(src, index, out, B, E, K, N, sb, se, eps: float = 1e-12):
+def group_bins_workspace_bytes(B, E, K, N, dtype) -> int:
+    """Scratch of the route through buckets of groups (ts_group_bins_workspace_bytes); 0: the route does not apply."""
+    return int(lib().ts_group_bins_workspace_bytes(_i(B), _i(E), _i(K), _i(N), DTYPE[dtype]))
+
+
+def group_logsumexp(src, index, out, B, E, K, N, sb, se, eps: float = 1e-12, bins: bool = True):
+    """bins: hand over the larger workspace with which the call goes through buckets of groups where that applies."""
     _dev(src, index, out)
     ws, nbytes = _group_workspace(out, B, N, K)
+    big = group_bins_workspace_bytes(B, E, K, N, out.dtype) if bins else 0
+    if big > nbytes:
+        nbytes = big
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=out.device)
     with torch.cuda.device(out.device):
         _check(lib().ts_group_logsumexp(_p(src), _p(index), _p(out), _i(B), _i(E), _i(K), _i(N), _i(sb), _i(se),
                                         DTYPE[out.dtype], ctypes.c_double(eps), _p(ws), ctypes.c_size_t(nbytes),
@@ -312,6 +323,19 @@ def group_std(src, index, total, count, out, B, E, K, N, sb, se, unbiased: bool 
                                   _i(sb), _i(se), DTYPE[out.dtype], int(unbiased), _p(ws), ctypes.c_size_t(nbytes),
                                   _stream(out)))
     return ws
+
+
+def group_std_forward(src, index, total, count, out, B, E, K, N, sb, se, unbiased: bool = True):
+    """Group sums, counts and standard deviation in one call through buckets of groups (ts_group_std_forward).
+    Returns the bytes of workspace used; raises where the route does not apply."""
+    _dev(src, index, total, count, out)
+    nbytes = group_bins_workspace_bytes(B, E, K, N, out.dtype)
+    ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=out.device)
+    with torch.cuda.device(out.device):
+        _check(lib().ts_group_std_forward(_p(src), _p(index), _p(total), _p(count), _p(out), _i(B), _i(E), _i(K), _i(N),
+                                          _i(sb), _i(se), DTYPE[out.dtype], int(unbiased), _p(ws),
+                                          ctypes.c_size_t(nbytes), _stream(out)))
+    return nbytes
 
 
 def group_std_backward(src, index, total, count, out, grad_out, grad_in, B, E, K, N, sb, se, unbiased: bool = True):

@@ -910,6 +910,25 @@ int ts_group_softmax_backward(const void *result, const void *grad_out, const in
                            static_cast<hipStream_t>(stream));
 }
 
+namespace {
+// columns per lane of the bucket kernels: 16 bytes when the row allows it
+int group_bins_vec(int64_t K, int dtype, bool aligned) {
+  const int full = kVecBytes / kElemBytes[dtype];
+  return (full > 1 && K % full == 0 && aligned) ? full : 1;
+}
+// TS_GROUP_BINS (tuning aid): 0 the buckets of groups never take a call, 2 they take it at any size
+GroupBinPlan group_bins_plan(int64_t B, int64_t E, int64_t K, int64_t N, int dtype, bool aligned, void *ws, size_t ws_bytes) {
+  const int mode = env_int("TS_GROUP_BINS", 1);
+  if (mode == 0) {
+    GroupBinPlan r;
+    r.ok = false;
+    r.bytes = 0;
+    return r;
+  }
+  return group_bin_plan(B, E, K, N, kElemBytes[dtype], group_bins_vec(K, dtype, aligned), ws, ws_bytes, mode == 2);
+}
+}  // namespace
+
 int ts_group_logsumexp(const void *src, const int64_t *index, void *out, int64_t B, int64_t E, int64_t K, int64_t N,
                        int64_t index_stride_b, int64_t index_stride_e, int dtype, double eps, void *workspace,
                        size_t workspace_bytes, ts_stream_t stream) {
@@ -924,6 +943,22 @@ int ts_group_logsumexp(const void *src, const int64_t *index, void *out, int64_t
   g.src = src;
   g.index = index;
   g.out = out;
+  if (B * E * K > 0) {
+    // a workspace of ts_group_bins_workspace_bytes(): one gather of src through buckets of groups
+    const GroupBinPlan plan = group_bins_plan(B, E, K, N, dtype, aligned16(src), workspace, workspace_bytes);
+    if (plan.ok) {
+      g.B = B;
+      g.E = E;
+      g.K = K;
+      g.N = N;
+      g.sb = index_stride_b;
+      g.se = index_stride_e;
+      g.eps = eps;
+      g.bins = &plan.p;
+      return dispatch_group_softmax(dtype, g, GS_LSE_BINS, group_bins_vec(K, dtype, aligned16(src)),
+                                    static_cast<hipStream_t>(stream));
+    }
+  }
   g.gmax = workspace;
   g.gs = 2 * K;  // a group's keys and sums side by side
   g.gsum = static_cast<char *>(workspace) + (size_t)K * (kElemBytes[dtype] == 8 ? 8 : 4);
@@ -938,6 +973,39 @@ int ts_group_logsumexp(const void *src, const int64_t *index, void *out, int64_t
   const int full = kVecBytes / kElemBytes[dtype];
   const int vec = (full > 1 && K % full == 0 && aligned16(src)) ? full : 1;
   return dispatch_group_softmax(dtype, g, GS_LSE, vec, static_cast<hipStream_t>(stream));
+}
+
+size_t ts_group_bins_workspace_bytes(int64_t B, int64_t E, int64_t K, int64_t N, int dtype) {
+  if (!valid_dtype(dtype) || !is_float_dtype(dtype) || !sizes_ok(B, N, E, K)) return 0;
+  return group_bins_plan(B, E, K, N, dtype, true, nullptr, 0).bytes;
+}
+
+int ts_group_std_forward(const void *src, const int64_t *index, void *total, int32_t *count, void *out, int64_t B,
+                         int64_t E, int64_t K, int64_t N, int64_t index_stride_b, int64_t index_stride_e, int dtype,
+                         int unbiased, void *workspace, size_t workspace_bytes, ts_stream_t stream) {
+  if (!valid_dtype(dtype) || !sizes_ok(B, N, E, K)) return TS_ERR_BAD_ARG;
+  if (!is_float_dtype(dtype)) return TS_ERR_UNSUPPORTED;
+  if (B * N * K == 0) return TS_OK;
+  if (!out || !total || !count || !src || !index) return TS_ERR_BAD_ARG;
+  const bool al = aligned16(src);
+  const GroupBinPlan plan = group_bins_plan(B, E, K, N, dtype, al, workspace, workspace_bytes);
+  if (plan.bytes == 0) return TS_ERR_UNSUPPORTED;
+  if (!plan.ok) return TS_ERR_WORKSPACE;
+  GroupArgs g = {};
+  g.src = src;
+  g.index = index;
+  g.out = out;
+  g.total_w = total;
+  g.count_w = count;
+  g.unbiased = unbiased ? 1 : 0;
+  g.B = B;
+  g.E = E;
+  g.K = K;
+  g.N = N;
+  g.sb = index_stride_b;
+  g.se = index_stride_e;
+  g.bins = &plan.p;
+  return dispatch_group_softmax(dtype, g, GS_STD_BINS, group_bins_vec(K, dtype, al), static_cast<hipStream_t>(stream));
 }
 
 int ts_group_logsumexp_backward(const void *src, const int64_t *index, const void *out, const void *grad_out,

@@ -72,8 +72,11 @@ template <typename T> __device__ __forceinline__ typename OrdKey<typename Acc<T>
 
 enum {
   GS_SOFTMAX = 0, GS_LOG_SOFTMAX = 1, GS_SOFTMAX_BWD = 2, GS_LOG_SOFTMAX_BWD = 3, GS_LSE = 4, GS_LSE_BWD = 5,
-  GS_STD = 6, GS_STD_BWD = 7
+  GS_STD = 6, GS_STD_BWD = 7,
+  GS_STD_BINS = 8, GS_LSE_BINS = 9  // std / logsumexp forward through buckets of groups (group_binned.h)
 };
+
+struct BinArgs;
 
 struct GroupArgs {
   const void *src;       // [B, E, K]: forward input; backward: the forward result y
@@ -95,6 +98,9 @@ struct GroupArgs {
   const int *gate = nullptr;  // the three passes of softmax run only if *gate != 0 (null: always)
   int *flag = nullptr;        // softmax: a word behind the workspace of the three passes, for the one-pass kernels
   size_t ws_bytes = 0;        //          bytes of that workspace (gmax is its start)
+  void *total_w = nullptr;      // std through buckets: the group sums [B, N, K] in the element type are written here,
+  int32_t *count_w = nullptr;   // and the entries per group [B, N] here
+  const BinArgs *bins = nullptr;  // (host) plan of the buckets
 };
 
 // std: the group mean as the reference forms it (composite/std.py:27-31: sum / clamp(count, 1), in the
@@ -621,6 +627,10 @@ inline ScatterArgs group_index_args(const GroupArgs &g) {
   return a;
 }
 
+}  // namespace ts
+#include "group_binned.h"
+namespace ts {
+
 template <typename T, int VEC, int MODE>
 int launch_group_softmax_m(const GroupArgs &g_in, hipStream_t stream) {
   constexpr bool kForward = MODE == GS_SOFTMAX || MODE == GS_LOG_SOFTMAX;
@@ -722,6 +732,8 @@ int launch_group_softmax_v(const GroupArgs &g, int mode, hipStream_t stream) {
   switch (mode) {
   case GS_STD: return launch_group_std_v<T, VEC>(g, false, stream);
   case GS_STD_BWD: return launch_group_std_v<T, VEC>(g, true, stream);
+  case GS_STD_BINS: return launch_group_bins<T, VEC, GS_STD>(g, stream);
+  case GS_LSE_BINS: return launch_group_bins<T, VEC, GS_LSE>(g, stream);
   case GS_LSE: return launch_group_lse_v<T, VEC>(g, false, stream);
   case GS_LSE_BWD: return launch_group_lse_v<T, VEC>(g, true, stream);
   case GS_SOFTMAX: return launch_group_softmax_m<T, VEC, GS_SOFTMAX>(g, stream);

@@ -862,7 +862,10 @@ struct GroupLogSumExpFn : public torch::autograd::Function<GroupLogSumExpFn> {
     auto sizes = src.sizes().vec();
     sizes[dim] = N;
     Tensor out = at::empty(sizes, src.options());
-    Tensor ws = workspace(ts_group_softmax_workspace_bytes(l.B, N, l.K, dtype_code(src)), src);
+    // the larger workspace of the route through buckets of groups, where that route applies
+    const size_t ws_bytes = std::max(ts_group_softmax_workspace_bytes(l.B, N, l.K, dtype_code(src)),
+                                     ts_group_bins_workspace_bytes(l.B, l.E, l.K, N, dtype_code(src)));
+    Tensor ws = workspace(ws_bytes, src);
     check_status(ts_group_logsumexp(src.data_ptr(), index.data_ptr<int64_t>(), out.data_ptr(), l.B, l.E, l.K, N, l.sb,
                                     l.se, dtype_code(src), eps, ws.data_ptr(), static_cast<size_t>(ws.numel()),
                                     stream_of(src)),
@@ -898,17 +901,33 @@ struct GroupStdFn : public torch::autograd::Function<GroupStdFn> {
     c10::DeviceGuard guard(src.device());
     src = src.contiguous();
     const GroupLayout l = group_layout(src, index, dim);
-    Tensor total = std::get<0>(scatter_hip(src, index, dim, std::nullopt, N, TS_SUM)).contiguous();
-    Tensor count = at::empty({l.B * N}, src.options().dtype(at::kInt));
-    check_status(ts_scatter_count(index.data_ptr<int64_t>(), count.data_ptr<int32_t>(), l.B, l.E, N, l.sb, l.se,
-                                  stream_of(src)),
-                 "scatter_std count");
-    Tensor out = at::empty_like(total);
-    Tensor ws = workspace(ts_group_softmax_workspace_bytes(l.B, N, l.K, dtype_code(src)), src);
-    check_status(ts_group_std(src.data_ptr(), index.data_ptr<int64_t>(), total.data_ptr(), count.data_ptr<int32_t>(),
-                              out.data_ptr(), l.B, l.E, l.K, N, l.sb, l.se, dtype_code(src), unbiased ? 1 : 0,
-                              ws.data_ptr(), static_cast<size_t>(ws.numel()), stream_of(src)),
-                 "scatter_std");
+    Tensor total, count, out;
+    const size_t bins_bytes = ts_group_bins_workspace_bytes(l.B, l.E, l.K, N, dtype_code(src));
+    if (bins_bytes > 0 && l.B * N * l.K > 0 && (reinterpret_cast<uintptr_t>(src.data_ptr()) & 15) == 0) {
+      // group sums, counts and result from one gather of src through buckets of groups
+      auto sizes = src.sizes().vec();
+      sizes[dim] = N;
+      total = at::empty(sizes, src.options());
+      count = at::empty({l.B * N}, src.options().dtype(at::kInt));
+      out = at::empty_like(total);
+      Tensor ws = workspace(bins_bytes, src);
+      check_status(ts_group_std_forward(src.data_ptr(), index.data_ptr<int64_t>(), total.data_ptr(),
+                                        count.data_ptr<int32_t>(), out.data_ptr(), l.B, l.E, l.K, N, l.sb, l.se,
+                                        dtype_code(src), unbiased ? 1 : 0, ws.data_ptr(), bins_bytes, stream_of(src)),
+                   "scatter_std");
+    } else {
+      total = std::get<0>(scatter_hip(src, index, dim, std::nullopt, N, TS_SUM)).contiguous();
+      count = at::empty({l.B * N}, src.options().dtype(at::kInt));
+      check_status(ts_scatter_count(index.data_ptr<int64_t>(), count.data_ptr<int32_t>(), l.B, l.E, N, l.sb, l.se,
+                                    stream_of(src)),
+                   "scatter_std count");
+      out = at::empty_like(total);
+      Tensor ws = workspace(ts_group_softmax_workspace_bytes(l.B, N, l.K, dtype_code(src)), src);
+      check_status(ts_group_std(src.data_ptr(), index.data_ptr<int64_t>(), total.data_ptr(), count.data_ptr<int32_t>(),
+                                out.data_ptr(), l.B, l.E, l.K, N, l.sb, l.se, dtype_code(src), unbiased ? 1 : 0,
+                                ws.data_ptr(), static_cast<size_t>(ws.numel()), stream_of(src)),
+                   "scatter_std");
+    }
     ctx->saved_data["dim"] = dim;
     ctx->saved_data["unbiased"] = unbiased;
     ctx->save_for_backward({src, index, total, count, out});

@@ -325,15 +325,37 @@ def test_operator_reference_cases_script_and_fallback(ts, oracle):
 
 
 # ------------------------------------------------------------------ logsumexp
-@pytest.mark.parametrize("shape,kind,dtype", product(SHAPES, ["random", "sorted", "hub"], DTYPES))
-def test_logsumexp_forward_and_backward_capi(capi, oracle, shape, kind, dtype):
+def bucket_lanes(K, dtype):
+    """lanes that hold a row in the bucket kernels: 16 bytes each when the row is a whole number of them, else one column"""
+    full = 16 // torch.empty((), dtype=dtype).element_size()
+    return K // full if K % full == 0 else K
+
+
+# one shape whose hub group fills more than 32 chunks of its bucket (the slabs merged by wavefronts side by side)
+BIN_SHAPES = SHAPES + [(1, 300_000, 8, 2000)]
+
+
+@pytest.mark.parametrize("shape,kind,dtype", product(BIN_SHAPES, ["random", "sorted", "hub"], DTYPES))
+@pytest.mark.parametrize("route", ["passes", "buckets"])
+def test_logsumexp_forward_and_backward_capi(capi, oracle, monkeypatch, shape, kind, dtype, route):
+    """route = buckets: the call goes through buckets of groups (group_binned.h) at any size; a hub group fills
+    several chunks of its bucket, whose slabs are merged."""
     B, E, K, N = shape
+    if route == "buckets":
+        if bucket_lanes(K, dtype) > 32:
+            pytest.skip("rows held by more than 32 lanes stay with the three passes")
+        monkeypatch.setenv("TS_GROUP_BINS", "2")
+        assert capi.group_bins_workspace_bytes(B, E, K, N + 3, dtype) > 0
+    elif E > 100_000:
+        pytest.skip("a shape for the buckets")
+    else:
+        monkeypatch.setenv("TS_GROUP_BINS", "0")
     N = N + 3  # the last groups stay empty
     rng = np.random.default_rng(E * 17 + K)
     src = torch.from_numpy(rng.standard_normal(size=(B, E, K)) * 3).to(dtype)
     index1 = make_index(kind, rng, E, N - 3)
     index = index1.view(1, E, 1).expand(B, E, K)
-    exact = dtype in (torch.float32, torch.float64)
+    exact = dtype in (torch.float32, torch.float64) and E <= 100_000
     ref_src = src if exact else src.double()
     out = torch.full((B, N, K), 7, dtype=dtype, device=DEV)
     capi.group_logsumexp(src.to(DEV), index1.to(DEV), out, B, E, K, N, 0, 1)
@@ -466,6 +488,70 @@ def test_std_forward_and_backward_capi(capi, oracle, shape, kind, dtype, unbiase
         gbound = gbound + 2.0 ** -24  # gradients below 2^-14 are subnormal in fp16: absolute spacing 2^-24
     gerr = (got_g - want_g).abs()
     assert bool((gerr[live] <= gbound[live]).all()), float((gerr[live] - gbound[live]).max())
+
+
+@pytest.mark.parametrize("shape,kind,dtype,unbiased",
+                         product(STD_SHAPES + [(1, 300_000, 8, 2000)], ["random", "sorted", "hub"], DTYPES, [True, False]))
+def test_std_forward_through_buckets_capi(capi, oracle, monkeypatch, shape, kind, dtype, unbiased):
+    """ts_group_std_forward: group sums, counts and standard deviation from one gather of src through buckets of
+    groups (group_binned.h), at any size. Bars as in test_std_forward_and_backward_capi; the count is exact, the group
+    sum is the double-precision sum rounded once."""
+    B, E, K, N = shape
+    exact = dtype in (torch.float32, torch.float64)
+    if kind == "hub" and not exact:
+        pytest.skip("a 16-bit group sum over hundreds of entries is not meaningful")
+    if bucket_lanes(K, dtype) > 32:
+        pytest.skip("rows held by more than 32 lanes stay with the three passes")
+    monkeypatch.setenv("TS_GROUP_BINS", "2")
+    rng = np.random.default_rng(E * 19 + K)
+    src = torch.from_numpy(rng.standard_normal(size=(B, E, K)) * 3 + 1).to(dtype)
+    index1 = make_index(kind, rng, E, N)
+    if E > 10:
+        index1[3] = -1   # outside [0, N): belongs to no group
+        index1[E - 2] = N
+    index = index1.view(1, E, 1).expand(B, E, K)
+    keep = (index1 >= 0) & (index1 < N)
+    total = torch.full((B, N, K), 7, dtype=dtype, device=DEV)
+    count = torch.full((B, N), -7, dtype=torch.int32, device=DEV)
+    out = torch.full((B, N, K), 7, dtype=dtype, device=DEV)
+    used = capi.group_std_forward(src.to(DEV), index1.to(DEV), total, count, out, B, E, K, N, 0, 1, unbiased)
+    torch.cuda.synchronize()
+    assert used > 8 * B * E
+    want_cnt = np.bincount(index1[keep].numpy(), minlength=N)
+    for b in range(B):
+        assert count.cpu().view(B, N)[b].tolist() == want_cnt.tolist()
+    src_k, index_k = src[:, keep], index[:, keep]
+    sum64 = oracle.scatter(src_k.double(), index_k, 1, None, N, "sum")[0]
+    abs64 = oracle.scatter(src_k.double().abs(), index_k, 1, None, N, "sum")[0]
+    e = EPS_T[dtype]
+    # the group sum: lanes add their few entries in fp32 (fp64 for doubles) and meet in double precision; rounded once
+    assert bool(((total.cpu().double() - sum64).abs() <= e * sum64.abs() + min(e, 4e-6) * abs64 + 1e-30).all())
+    ref_src = src_k if exact and E <= 100_000 else src_k.double()
+    want = oracle.scatter_std(ref_src, index_k, 1, None, N, unbiased).double()
+    err = (out.cpu().double() - want).abs()
+    cnt_n = torch.from_numpy(want_cnt).double().view(1, N, 1).clamp(1).expand(B, N, K)
+    mean_abs = abs64 / cnt_n
+    if exact:
+        bound = e * want + (1e-6 if dtype == torch.float32 else 1e-12)
+    else:
+        bound = 8.0 * e * want + 2.0 * e * mean_abs * (1.0 + cnt_n.sqrt())
+    assert bool((err <= bound).all()), float((err - bound).max())
+
+
+def test_bucket_route_declines(capi, monkeypatch):
+    """Where the buckets of groups do not apply the size query says 0 and ts_group_std_forward refuses."""
+    assert capi.group_bins_workspace_bytes(1, 1000, 8, 100, torch.float32) == 0        # small
+    assert capi.group_bins_workspace_bytes(1, 1 << 22, 8, 1 << 20, torch.float32) > 0
+    assert capi.group_bins_workspace_bytes(1, 1 << 22, 8, 1 << 20, torch.int32) == 0   # floating types only
+    assert capi.group_bins_workspace_bytes(1, 1 << 20, 256, 1 << 10, torch.float32) == 0  # 64 lanes per row
+    monkeypatch.setenv("TS_GROUP_BINS", "0")
+    assert capi.group_bins_workspace_bytes(1, 1 << 22, 8, 1 << 20, torch.float32) == 0
+    src = torch.zeros((1000, 8), device=DEV)
+    idx = torch.zeros(1000, dtype=torch.long, device=DEV)
+    total, out = torch.empty((10, 8), device=DEV), torch.empty((10, 8), device=DEV)
+    count = torch.empty(10, dtype=torch.int32, device=DEV)
+    with pytest.raises(RuntimeError):
+        capi.group_std_forward(src, idx, total, count, out, 1, 1000, 8, 10, 0, 1)
 
 
 @pytest.mark.parametrize("dim,unbiased", product([0, 1, 2, -1], [True, False]))
