@@ -266,9 +266,18 @@ def _group_workspace(like, B, N, K):
     return torch.empty(max(nbytes, 1), dtype=torch.uint8, device=like.device), nbytes
 
 
+def group_bins_workspace_bytes(B, E, K, N, dtype) -> int:
+    """Scratch of the route through buckets of groups (ts_group_bins_workspace_bytes); 0: the route does not apply."""
+    return int(lib().ts_group_bins_workspace_bytes(_i(B), _i(E), _i(K), _i(N), DTYPE[dtype]))
+
+
 def group_softmax(src, index, out, B, E, K, N, sb, se, log_space: bool, eps: float = 1e-12):
     _dev(src, index, out)
     ws, nbytes = _group_workspace(out, B, N, K)
+    big = group_bins_workspace_bytes(B, E, K, N, out.dtype)  # where it applies: buckets of groups for an unsorted index
+    if big > nbytes:
+        nbytes = big
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=out.device)
     with torch.cuda.device(out.device):
         _check(lib().ts_group_softmax(_p(src), _p(index), _p(out), _i(B), _i(E), _i(K), _i(N), _i(sb), _i(se),
                                       DTYPE[out.dtype], int(log_space), ctypes.c_double(eps), _p(ws),
@@ -285,11 +294,6 @@ def group_softmax_backward(result, grad_out, index, grad_in, B, E, K, N, sb, se,
                                                int(log_space), _p(ws), ctypes.c_size_t(nbytes),
                                                _stream(grad_in)))
     return ws
-
-
-def group_bins_workspace_bytes(B, E, K, N, dtype) -> int:
-    """Scratch of the route through buckets of groups (ts_group_bins_workspace_bytes); 0: the route does not apply."""
-    return int(lib().ts_group_bins_workspace_bytes(_i(B), _i(E), _i(K), _i(N), DTYPE[dtype]))
 
 
 def group_logsumexp(src, index, out, B, E, K, N, sb, se, eps: float = 1e-12, bins: bool = True):

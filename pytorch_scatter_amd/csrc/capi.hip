@@ -845,6 +845,31 @@ int ts_arg_backward(const void *grad_out, const int64_t *arg, void *grad_in, int
 }
 
 namespace {
+// columns per lane of the bucket kernels: 16 bytes when the row allows it
+int group_bins_vec(int64_t K, int dtype, bool aligned) {
+  const int full = kVecBytes / kElemBytes[dtype];
+  return (full > 1 && K % full == 0 && aligned) ? full : 1;
+}
+// TS_GROUP_BINS (tuning aid): 0 the buckets of groups never take a call, 2 they take it at any size
+GroupBinPlan group_bins_plan(int64_t B, int64_t E, int64_t K, int64_t N, int dtype, bool aligned, void *ws, size_t ws_bytes) {
+  const int mode = env_int("TS_GROUP_BINS", 1);
+  if (mode == 0) {
+    GroupBinPlan r;
+    r.ok = false;
+    r.bytes = 0;
+    return r;
+  }
+  // the buckets' scratch lies behind the workspace of the three passes (softmax keeps its keys, sums and flag there)
+  const size_t front = group_workspace_bytes(B, N, K, kElemBytes[dtype]);
+  GroupBinPlan r = group_bin_plan(B, E, K, N, kElemBytes[dtype], group_bins_vec(K, dtype, aligned),
+                                  ws != nullptr && ws_bytes > front ? static_cast<char *>(ws) + front : nullptr,
+                                  ws_bytes > front ? ws_bytes - front : 0, mode == 2);
+  if (r.bytes > 0) r.bytes += front;
+  return r;
+}
+}  // namespace
+
+namespace {
 int run_group_softmax(const void *src, const void *grad, const int64_t *index, void *out, int64_t B, int64_t E,
                       int64_t K, int64_t N, int64_t sb, int64_t se, int dtype, int mode, double eps, void *workspace,
                       size_t workspace_bytes, hipStream_t stream) {
@@ -884,6 +909,12 @@ int run_group_softmax(const void *src, const void *grad, const int64_t *index, v
   const int full = kVecBytes / kElemBytes[dtype];
   const bool al = aligned16(src) && aligned16(out) && (!grad || aligned16(grad));
   const int vec = (full > 1 && K % full == 0 && al) ? full : 1;
+  // forward with a workspace of ts_group_bins_workspace_bytes(): an index that is not in order goes through buckets of groups
+  GroupBinPlan plan;
+  if (with_keys) {
+    plan = group_bins_plan(B, E, K, N, dtype, al, workspace, workspace_bytes);
+    if (plan.ok && group_bins_vec(K, dtype, al) == vec) g.bins = &plan.p;
+  }
   return dispatch_group_softmax(dtype, g, mode, vec, stream);
 }
 }  // namespace
@@ -909,25 +940,6 @@ int ts_group_softmax_backward(const void *result, const void *grad_out, const in
                            log_space ? GS_LOG_SOFTMAX_BWD : GS_SOFTMAX_BWD, 0.0, workspace, workspace_bytes,
                            static_cast<hipStream_t>(stream));
 }
-
-namespace {
-// columns per lane of the bucket kernels: 16 bytes when the row allows it
-int group_bins_vec(int64_t K, int dtype, bool aligned) {
-  const int full = kVecBytes / kElemBytes[dtype];
-  return (full > 1 && K % full == 0 && aligned) ? full : 1;
-}
-// TS_GROUP_BINS (tuning aid): 0 the buckets of groups never take a call, 2 they take it at any size
-GroupBinPlan group_bins_plan(int64_t B, int64_t E, int64_t K, int64_t N, int dtype, bool aligned, void *ws, size_t ws_bytes) {
-  const int mode = env_int("TS_GROUP_BINS", 1);
-  if (mode == 0) {
-    GroupBinPlan r;
-    r.ok = false;
-    r.bytes = 0;
-    return r;
-  }
-  return group_bin_plan(B, E, K, N, kElemBytes[dtype], group_bins_vec(K, dtype, aligned), ws, ws_bytes, mode == 2);
-}
-}  // namespace
 
 int ts_group_logsumexp(const void *src, const int64_t *index, void *out, int64_t B, int64_t E, int64_t K, int64_t N,
                        int64_t index_stride_b, int64_t index_stride_e, int dtype, double eps, void *workspace,

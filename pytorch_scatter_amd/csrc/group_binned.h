@@ -113,7 +113,7 @@ template <typename T, int MODE> struct GroupBinPart {
   int32_t n;   // std: entries
   __device__ static GroupBinPart identity() {
     GroupBinPart s;
-    s.a = MODE == GS_STD ? 0ull : (uint64_t)OrdKey<F>::enc(-INFINITY);
+    s.a = MODE == GS_STD ? 0ull : MODE == GS_LSE ? (uint64_t)OrdKey<F>::enc(-INFINITY) : (uint64_t)group_empty_key<T>();
     s.b = 0.0;
     s.n = 0;
     return s;
@@ -134,7 +134,14 @@ template <typename T, int MODE> struct GroupBinPart {
       n += o.n;
     } else {
       const KB ka = (KB)a, kb = (KB)o.a;
-      const KB none = OrdKey<F>::enc(-INFINITY);
+      // no maximum yet: logsumexp starts from -inf; softmax from lowest(), and a partial in which nothing beat it
+      // was summed relative to 0 and holds 0 or NaN, taken as is
+      const KB none = MODE == GS_LSE ? OrdKey<F>::enc(-INFINITY) : group_empty_key<T>();
+      if (MODE != GS_LSE && (ka == none || kb == none)) {
+        if (kb > ka) a = o.a;
+        b = b + o.b;
+        return;
+      }
       if (kb > ka) {
         const double fac = ka == none ? 0.0 : (double)exp_acc(OrdKey<F>::dec(ka) - OrdKey<F>::dec(kb));
         b = b * fac + o.b;
@@ -162,6 +169,11 @@ __device__ __forceinline__ void group_bin_emit(const GroupArgs &g, int64_t i, in
     out[i] = from_acc<T>(sqrt_acc(round_elem<T>(round_elem<T>((F)s.b) / div)));
     static_cast<T *>(g.total_w)[i] = from_acc<T>((F)__longlong_as_double((long long)s.a));
     if (k == 0) g.count_w[row] = s.n;
+  } else if constexpr (MODE == GS_SOFTMAX) {
+    // the group's key and sum, side by side, for the elementwise finish of group_softmax.h
+    const int64_t slot = row * g.gs + k;
+    static_cast<KB *>(g.gmax)[slot] = (KB)s.a;
+    static_cast<F *>(g.gsum)[slot] = (F)s.b;
   } else {
     const F m = OrdKey<F>::dec((KB)s.a);
     const F l = round_elem<T>(log_acc(round_elem<T>(round_elem<T>((F)s.b) + (F)g.eps)));
@@ -190,6 +202,7 @@ __global__ __launch_bounds__(kBinBlock) void group_bin_kernel(GroupArgs g, BinAr
   __shared__ int32_t s_wsum[W];
   __shared__ int32_t s_long[kGroupBinMaxLong];  // groups for a wavefront
   __shared__ int s_nlong;
+  if (p.unsorted != nullptr && *p.unsorted != 1) return;  // the caller's one-pass kernels took the call
   const int wg = (int)blockIdx.x;
   const int bucket = p.wg_bucket[wg];
   if (bucket < 0) return;
@@ -354,16 +367,20 @@ __global__ __launch_bounds__(kBinBlock) void group_bin_kernel(GroupArgs g, BinAr
 #pragma unroll
         for (int v = 0; v < VEC; ++v) top[v] = max_acc(top[v], to_acc<T>(y.v[v]));  // a NaN never wins
       });
+      bool won[VEC];
 #pragma unroll
       for (int v = 0; v < VEC; ++v) {
         if (wide) top[v] = meet(top[v], [](F a, F b) { return max_acc(a, b); });
         top[v] = OrdKey<F>::dec(OrdKey<F>::enc(top[v]));  // -0.0 folds onto +0.0
+        // softmax: an entry has to beat lowest(); a group without a winner is shifted by 0 (composite/softmax.py:16-18)
+        won[v] = MODE == GS_LSE || top[v] > to_acc<T>(ElemLim<T>::lowest());
+        if (!won[v]) top[v] = (F)0;
       }
       for_entries([&](const Vec<T, VEC> &y) {
 #pragma unroll
         for (int v = 0; v < VEC; ++v) {
           F z = round_elem<T>(to_acc<T>(y.v[v]) - top[v]);
-          if (z != z) z = -INFINITY;  // NaN entries and -inf - -inf drop out (logsumexp.py:41)
+          if (MODE == GS_LSE && z != z) z = -INFINITY;  // NaN entries and -inf - -inf drop out (logsumexp.py:41)
           acc[v] += round_elem<T>(exp_acc(z));
         }
       });
@@ -371,7 +388,7 @@ __global__ __launch_bounds__(kBinBlock) void group_bin_kernel(GroupArgs g, BinAr
       for (int v = 0; v < VEC; ++v) {
         sum[v] = (double)acc[v];
         if (wide) sum[v] = meet(sum[v], [](double a, double b) { return a + b; });
-        part[v].a = (uint64_t)OrdKey<F>::enc(top[v]);
+        part[v].a = won[v] ? (uint64_t)OrdKey<F>::enc(top[v]) : (uint64_t)group_empty_key<T>();
         part[v].b = sum[v];
         part[v].n = 0;
       }
@@ -416,6 +433,7 @@ __global__ __launch_bounds__(kBinBlock) void group_bin_combine_kernel(GroupArgs 
   __shared__ uint64_t s_pa[W][kCombPos];
   __shared__ double s_pb[W][kCombPos];
   __shared__ int32_t s_pn[W][kCombPos];
+  if (p.unsorted != nullptr && *p.unsorted != 1) return;
   const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
   const int K = (int)g.K, R = 1 << p.rshift, table = K << p.rshift;
   const int64_t words = (int64_t)group_bin_slab_words(table, R);
@@ -489,13 +507,20 @@ __global__ __launch_bounds__(kBinBlock) void group_bin_combine_kernel(GroupArgs 
 }
 
 // count, scan, place (scatter_binned.h), then the chunks and the buckets of several chunks
+// gate (softmax): a word that the caller's one-pass kernels leave at 1 when the index was not in order; every pass
+// here then runs only if it reads 1
 template <typename T, int VEC, int MODE>
-int launch_group_bins(const GroupArgs &g, hipStream_t stream) {
+int launch_group_bins(const GroupArgs &g, hipStream_t stream, int *gate = nullptr) {
   if (g.bins == nullptr) return TS_ERR_BAD_ARG;
-  const BinArgs p = *g.bins;
+  BinArgs p = *g.bins;
+  if (gate != nullptr) {
+    p.unsorted = gate;
+    p.sampled = 1;  // the count pass does not judge the index, it reads the verdict
+  }
   const ScatterArgs a = group_index_args(g);
-  hipLaunchKernelGGL(bin_clear_kernel, dim3((p.nb + kBlock - 1) / kBlock), dim3(kBlock), 0, stream, p.totals, p.nb,
-                     (int *)nullptr);
+  if (gate == nullptr)  // (with a gate: its owner's sample kernel has cleared the totals)
+    hipLaunchKernelGGL(bin_clear_kernel, dim3((p.nb + kBlock - 1) / kBlock), dim3(kBlock), 0, stream, p.totals, p.nb,
+                       (int *)nullptr);
   launch_bin_count(a, p, stream);
   hipLaunchKernelGGL(bin_scan_kernel, dim3(1), dim3(kBinBlock), 0, stream, p);
   if (bin_place_sorted_ok(p))

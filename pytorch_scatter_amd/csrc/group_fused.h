@@ -94,8 +94,11 @@ inline bool group_fused_plan(const GroupArgs &g, int mode, int elem_bytes, void 
 
 // A look at up to 1024 pairs of neighbours spread over the index: *flag = 1 (not in order, the tiles do not
 // run) if at least 1/64 of them descend, else 0 (the tiles run and check every pair).
-static __global__ __launch_bounds__(1024) void group_order_sample_kernel(GroupArgs g, int *flag, int force) {
+// Also clears `clear_n` 8-byte words at `clear` (the bucket totals of the passes that follow an index found out of order).
+static __global__ __launch_bounds__(1024) void group_order_sample_kernel(GroupArgs g, int *flag, int force,
+                                                                          unsigned long long *clear, int clear_n) {
   __shared__ int s_desc, s_pairs;
+  for (int i = threadIdx.x; i < clear_n; i += 1024) clear[i] = 0;
   if (threadIdx.x == 0) { s_desc = 0; s_pairs = 0; }
   __syncthreads();
   const int64_t total = g.B * g.E;
@@ -631,7 +634,8 @@ template <typename T, int CV, int MODE>
 int launch_group_fused(const GroupArgs &g, const FusedArgs &f, bool force, hipStream_t stream) {
   constexpr bool kBackward = MODE == GS_SOFTMAX_BWD || MODE == GS_LOG_SOFTMAX_BWD;
   typedef typename Acc<T>::type F;
-  hipLaunchKernelGGL(group_order_sample_kernel, dim3(1), dim3(1024), 0, stream, g, f.flag, force ? 1 : 0);
+  hipLaunchKernelGGL(group_order_sample_kernel, dim3(1), dim3(1024), 0, stream, g, f.flag, force ? 1 : 0,
+                     g.bins != nullptr ? g.bins->totals : nullptr, g.bins != nullptr ? g.bins->nb : 0);
   const size_t lds = (size_t)f.tile_vecs * 16 * (kBackward ? 2 : 1) + ((size_t)f.te + 2) * 2;
   const unsigned tiles = (unsigned)(g.B * f.nt);
   hipLaunchKernelGGL((group_fused_kernel<T, CV, MODE>), dim3(tiles), dim3(kBlock), lds, stream, g, f);

@@ -650,6 +650,17 @@ int launch_group_softmax_m(const GroupArgs &g_in, hipStream_t stream) {
     if (rc != TS_OK) return rc;
     g.gate = f.flag;
   }
+  if constexpr (kForward) {
+    if (g.bins != nullptr) {
+      // any other index, with the larger workspace: key and sum of every group from one gather of src through
+      // buckets of groups (group_binned.h), then the elementwise finish
+      const int rc = launch_group_bins<T, VEC, GS_SOFTMAX>(g, stream, const_cast<int *>(g.gate));
+      if (rc != TS_OK) return rc;
+      hipLaunchKernelGGL((group_finish_kernel<T, VEC, MODE>), dim3(scatter_grid(n_edges, g.K / VEC, kBlock, 4)),
+                         dim3(kBlock), 0, stream, g);
+      return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
+    }
+  }
   const ScatterArgs a = group_index_args(g);
   const dim3 gd(rg.blocks, rg.ychunks);
   hipLaunchKernelGGL(group_init_kernel<T>, dim3(grid_for(g.B * g.N * g.K)), dim3(kBlock), 0, stream, g,

@@ -818,7 +818,9 @@ struct GroupSoftmaxFn : public torch::autograd::Function<GroupSoftmaxFn> {
     src = src.contiguous();
     const GroupLayout l = group_layout(src, index, dim);
     Tensor out = at::empty_like(src);
-    Tensor ws = workspace(ts_group_softmax_workspace_bytes(l.B, N, l.K, dtype_code(src)), src);
+    // the larger workspace of the route through buckets of groups, where that route applies
+    Tensor ws = workspace(std::max(ts_group_softmax_workspace_bytes(l.B, N, l.K, dtype_code(src)),
+                                   ts_group_bins_workspace_bytes(l.B, l.E, l.K, N, dtype_code(src))), src);
     check_status(ts_group_softmax(src.data_ptr(), index.data_ptr<int64_t>(), out.data_ptr(), l.B, l.E, l.K, N, l.sb,
                                   l.se, dtype_code(src), log_space ? 1 : 0, eps, ws.data_ptr(),
                                   static_cast<size_t>(ws.numel()), stream_of(src)),

@@ -55,6 +55,12 @@ def make_index(kind, rng, E, N):
     return torch.from_numpy(idx)
 
 
+def bucket_lanes(K, dtype):
+    """lanes that hold a row in the bucket kernels: 16 bytes each when the row is a whole number of them, else one column"""
+    full = 16 // torch.empty((), dtype=dtype).element_size()
+    return K // full if K % full == 0 else K
+
+
 def forward_bound(dtype, want64, z64, log_space, exact=True):
     e = EPS_T[dtype]
     if dtype in (torch.float32, torch.float64) and exact:
@@ -116,9 +122,21 @@ def check_against_oracle(capi, oracle, src, grad, index1, shape, dtype):
         assert float(grad_in.cpu().double()[~inside].abs().max() if bool((~inside).any()) else 0.0) == 0.0
 
 
-@pytest.mark.parametrize("shape,kind,dtype", product(SHAPES, ["random", "sorted", "hub"], DTYPES))
-def test_forward_and_backward_capi(capi, oracle, shape, kind, dtype):
+@pytest.mark.parametrize("shape,kind,dtype", product(SHAPES + [(1, 300_000, 8, 2000)], ["random", "sorted", "hub"], DTYPES))
+@pytest.mark.parametrize("route", ["passes", "buckets"])
+def test_forward_and_backward_capi(capi, oracle, monkeypatch, shape, kind, dtype, route):
+    """route = buckets: the forward call finds key and sum of every group through buckets of groups (group_binned.h)
+    at any size, then the elementwise finish; a hub group fills several chunks of its bucket."""
     B, E, K, N = shape
+    if route == "buckets":
+        if bucket_lanes(K, dtype) > 32:
+            pytest.skip("rows held by more than 32 lanes stay with the three passes")
+        monkeypatch.setenv("TS_GROUP_BINS", "2")
+        assert capi.group_bins_workspace_bytes(B, E, K, N, dtype) > 0
+    elif E > 100_000:
+        pytest.skip("a shape for the buckets")
+    else:
+        monkeypatch.setenv("TS_GROUP_BINS", "0")
     rng = np.random.default_rng(E * 13 + K)
     src = torch.from_numpy(rng.standard_normal(size=(B, E, K)) * 3).to(dtype)
     grad = torch.from_numpy(rng.standard_normal(size=(B, E, K))).to(dtype)
@@ -151,10 +169,13 @@ def fused_index(kind, rng, E, N):
 
 @pytest.mark.parametrize("shape,kind,dtype",
                          product(FUSED_SHAPES, ["sorted", "skewed", "outside", "one_descent"], DTYPES))
-@pytest.mark.parametrize("tile", [256, 0])
-def test_one_pass_kernels_capi(capi, oracle, monkeypatch, shape, kind, dtype, tile):
+@pytest.mark.parametrize("tile,bins", [(256, "0"), (0, "0"), (256, "2")])
+def test_one_pass_kernels_capi(capi, oracle, monkeypatch, shape, kind, dtype, tile, bins):
+    """bins = 2: the passes behind the tiles are those through buckets of groups, which run only when the tiles
+    have found the index out of order."""
     B, E, K, N = shape
     monkeypatch.setenv("TS_GROUP_FUSED", "2")
+    monkeypatch.setenv("TS_GROUP_BINS", bins)
     if tile:
         monkeypatch.setenv("TS_GROUP_TILE", str(tile))
     rng = np.random.default_rng(E * 7 + K + N)
@@ -325,12 +346,6 @@ def test_operator_reference_cases_script_and_fallback(ts, oracle):
 
 
 # ------------------------------------------------------------------ logsumexp
-def bucket_lanes(K, dtype):
-    """lanes that hold a row in the bucket kernels: 16 bytes each when the row is a whole number of them, else one column"""
-    full = 16 // torch.empty((), dtype=dtype).element_size()
-    return K // full if K % full == 0 else K
-
-
 # one shape whose hub group fills more than 32 chunks of its bucket (the slabs merged by wavefronts side by side)
 BIN_SHAPES = SHAPES + [(1, 300_000, 8, 2000)]
 
