@@ -373,6 +373,12 @@ int ts_group_logsumexp_backward(const void *src, const int64_t *index,
                                 int64_t N, int64_t index_stride_b,
                                 int64_t index_stride_e, int dtype,
                                 ts_stream_t stream);
+/* The same with ts_group_softmax_workspace_bytes() of scratch (result and grad_out of a group side by side). */
+int ts_group_logsumexp_backward_with_workspace(const void *src, const int64_t *index, const void *out,
+                                               const void *grad_out, void *grad_in, int64_t B, int64_t E,
+                                               int64_t K, int64_t N, int64_t index_stride_b,
+                                               int64_t index_stride_e, int dtype, void *workspace,
+                                               size_t workspace_bytes, ts_stream_t stream);
 
 /* Standard deviation over the entries that share an index, one index per row, given the group sums
  * `total` ([B, N, K], element type: ts_scatter with SUM) and the entries per group `count` ([B, N]
@@ -395,6 +401,15 @@ int ts_group_std_backward(const void *src, const int64_t *index,
                           int64_t B, int64_t E, int64_t K, int64_t N,
                           int64_t index_stride_b, int64_t index_stride_e,
                           int dtype, int unbiased, ts_stream_t stream);
+/* The same backward pass with ts_group_softmax_workspace_bytes() of scratch: what an entry needs of its group (mean and
+ * grad_out / (out * divisor)) is first laid side by side, one memory line per entry instead of four under an index
+ * that is not in order. Without workspace (null): as ts_group_std_backward. */
+int ts_group_std_backward_with_workspace(const void *src, const int64_t *index, const void *total,
+                                         const int32_t *count, const void *out, const void *grad_out,
+                                         void *grad_in, int64_t B, int64_t E, int64_t K, int64_t N,
+                                         int64_t index_stride_b, int64_t index_stride_e, int dtype,
+                                         int unbiased, void *workspace, size_t workspace_bytes,
+                                         ts_stream_t stream);
 
 /* scatter_std and scatter_logsumexp through buckets of groups (no counterpart in the reference, whose
  * torch_scatter/composite/std.py:8-41 and logsumexp.py:8-57 compose scatter operators): the entries are binned

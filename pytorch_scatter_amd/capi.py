@@ -30,6 +30,7 @@ EXPORTS = (
     "ts_group_softmax_workspace_bytes", "ts_group_softmax", "ts_group_softmax_backward",
     "ts_group_logsumexp", "ts_group_logsumexp_backward",
     "ts_group_std", "ts_group_std_backward", "ts_group_bins_workspace_bytes", "ts_group_std_forward",
+    "ts_group_std_backward_with_workspace", "ts_group_logsumexp_backward_with_workspace",
     "ts_index_to_indptr", "ts_indptr_to_index_workspace_bytes", "ts_indptr_to_index",
     "ts_sort_index_workspace_bytes", "ts_sort_index",
     "ts_segment_csr_permuted_workspace_bytes", "ts_segment_csr_permuted",
@@ -311,12 +312,18 @@ def group_logsumexp(src, index, out, B, E, K, N, sb, se, eps: float = 1e-12, bin
     return ws
 
 
-def group_logsumexp_backward(src, index, out, grad_out, grad_in, B, E, K, N, sb, se):
+def group_logsumexp_backward(src, index, out, grad_out, grad_in, B, E, K, N, sb, se, with_workspace: bool = True):
     _dev(src, index, out, grad_out, grad_in)
     with torch.cuda.device(grad_in.device):
-        _check(lib().ts_group_logsumexp_backward(_p(src), _p(index), _p(out), _p(grad_out), _p(grad_in), _i(B),
-                                                 _i(E), _i(K), _i(N), _i(sb), _i(se), DTYPE[grad_in.dtype],
-                                                 _stream(grad_in)))
+        if with_workspace:
+            ws, nbytes = _group_workspace(grad_in, B, N, K)
+            _check(lib().ts_group_logsumexp_backward_with_workspace(
+                _p(src), _p(index), _p(out), _p(grad_out), _p(grad_in), _i(B), _i(E), _i(K), _i(N), _i(sb), _i(se),
+                DTYPE[grad_in.dtype], _p(ws), ctypes.c_size_t(nbytes), _stream(grad_in)))
+        else:
+            _check(lib().ts_group_logsumexp_backward(_p(src), _p(index), _p(out), _p(grad_out), _p(grad_in), _i(B),
+                                                     _i(E), _i(K), _i(N), _i(sb), _i(se), DTYPE[grad_in.dtype],
+                                                     _stream(grad_in)))
 
 
 def group_std(src, index, total, count, out, B, E, K, N, sb, se, unbiased: bool = True):
@@ -342,12 +349,19 @@ def group_std_forward(src, index, total, count, out, B, E, K, N, sb, se, unbiase
     return nbytes
 
 
-def group_std_backward(src, index, total, count, out, grad_out, grad_in, B, E, K, N, sb, se, unbiased: bool = True):
+def group_std_backward(src, index, total, count, out, grad_out, grad_in, B, E, K, N, sb, se, unbiased: bool = True,
+                       with_workspace: bool = True):
     _dev(src, index, total, count, out, grad_out, grad_in)
     with torch.cuda.device(grad_in.device):
-        _check(lib().ts_group_std_backward(_p(src), _p(index), _p(total), _p(count), _p(out), _p(grad_out),
-                                           _p(grad_in), _i(B), _i(E), _i(K), _i(N), _i(sb), _i(se),
-                                           DTYPE[grad_in.dtype], int(unbiased), _stream(grad_in)))
+        if with_workspace:
+            ws, nbytes = _group_workspace(grad_in, B, N, K)
+            _check(lib().ts_group_std_backward_with_workspace(
+                _p(src), _p(index), _p(total), _p(count), _p(out), _p(grad_out), _p(grad_in), _i(B), _i(E), _i(K), _i(N),
+                _i(sb), _i(se), DTYPE[grad_in.dtype], int(unbiased), _p(ws), ctypes.c_size_t(nbytes), _stream(grad_in)))
+        else:
+            _check(lib().ts_group_std_backward(_p(src), _p(index), _p(total), _p(count), _p(out), _p(grad_out),
+                                               _p(grad_in), _i(B), _i(E), _i(K), _i(N), _i(sb), _i(se),
+                                               DTYPE[grad_in.dtype], int(unbiased), _stream(grad_in)))
 
 
 def index_to_indptr(index, indptr, B, E, N, index_batch_stride):

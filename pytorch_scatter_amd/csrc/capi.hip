@@ -845,6 +845,13 @@ int ts_arg_backward(const void *grad_out, const int64_t *arg, void *grad_in, int
 }
 
 namespace {
+// std / logsumexp backward with a workspace of ts_group_softmax_workspace_bytes(): the values an entry needs of its group
+// are laid side by side first (one more launch over [B, N, K]) when there are at least as many entries as groups
+bool group_coef_ok(int64_t B, int64_t E, int64_t N, int64_t K, int dtype, const void *ws, size_t ws_bytes) {
+  if (ws == nullptr || (reinterpret_cast<uintptr_t>(ws) & 31) != 0 || !env_int("TS_GROUP_COEF", 1)) return false;
+  if (E < N) return false;
+  return ws_bytes >= (size_t)(B * N * K) * 2 * (kElemBytes[dtype] == 8 ? 8 : 4);
+}
 // columns per lane of the bucket kernels: 16 bytes when the row allows it
 int group_bins_vec(int64_t K, int dtype, bool aligned) {
   const int full = kVecBytes / kElemBytes[dtype];
@@ -1023,6 +1030,14 @@ int ts_group_std_forward(const void *src, const int64_t *index, void *total, int
 int ts_group_logsumexp_backward(const void *src, const int64_t *index, const void *out, const void *grad_out,
                                 void *grad_in, int64_t B, int64_t E, int64_t K, int64_t N, int64_t index_stride_b,
                                 int64_t index_stride_e, int dtype, ts_stream_t stream) {
+  return ts_group_logsumexp_backward_with_workspace(src, index, out, grad_out, grad_in, B, E, K, N, index_stride_b,
+                                                    index_stride_e, dtype, nullptr, 0, stream);
+}
+
+int ts_group_logsumexp_backward_with_workspace(const void *src, const int64_t *index, const void *out,
+                                               const void *grad_out, void *grad_in, int64_t B, int64_t E, int64_t K,
+                                               int64_t N, int64_t index_stride_b, int64_t index_stride_e, int dtype,
+                                               void *workspace, size_t workspace_bytes, ts_stream_t stream) {
   if (!valid_dtype(dtype) || !sizes_ok(B, N, E, K)) return TS_ERR_BAD_ARG;
   if (!is_float_dtype(dtype)) return TS_ERR_UNSUPPORTED;
   if (B * E * K == 0) return TS_OK;
@@ -1043,6 +1058,7 @@ int ts_group_logsumexp_backward(const void *src, const int64_t *index, const voi
   const int full = kVecBytes / kElemBytes[dtype];
   const bool al = aligned16(src) && aligned16(grad_in) && aligned16(out) && aligned16(grad_out);
   const int vec = (full > 1 && K % full == 0 && al) ? full : 1;
+  if (group_coef_ok(B, E, N, K, dtype, workspace, workspace_bytes)) g.coef = workspace;
   return dispatch_group_softmax(dtype, g, GS_LSE_BWD, vec, static_cast<hipStream_t>(stream));
 }
 
@@ -1081,6 +1097,14 @@ int ts_group_std_backward(const void *src, const int64_t *index, const void *tot
                           const void *out, const void *grad_out, void *grad_in, int64_t B, int64_t E, int64_t K,
                           int64_t N, int64_t index_stride_b, int64_t index_stride_e, int dtype, int unbiased,
                           ts_stream_t stream) {
+  return ts_group_std_backward_with_workspace(src, index, total, count, out, grad_out, grad_in, B, E, K, N, index_stride_b,
+                                              index_stride_e, dtype, unbiased, nullptr, 0, stream);
+}
+
+int ts_group_std_backward_with_workspace(const void *src, const int64_t *index, const void *total, const int32_t *count,
+                                         const void *out, const void *grad_out, void *grad_in, int64_t B, int64_t E,
+                                         int64_t K, int64_t N, int64_t index_stride_b, int64_t index_stride_e, int dtype,
+                                         int unbiased, void *workspace, size_t workspace_bytes, ts_stream_t stream) {
   if (!valid_dtype(dtype) || !sizes_ok(B, N, E, K)) return TS_ERR_BAD_ARG;
   if (!is_float_dtype(dtype)) return TS_ERR_UNSUPPORTED;
   if (B * E * K == 0) return TS_OK;
@@ -1104,6 +1128,7 @@ int ts_group_std_backward(const void *src, const int64_t *index, const void *tot
   const int full = kVecBytes / kElemBytes[dtype];
   const bool al = aligned16(src) && aligned16(grad_in) && aligned16(out) && aligned16(grad_out) && aligned16(total);
   const int vec = (full > 1 && K % full == 0 && al) ? full : 1;
+  if (group_coef_ok(B, E, N, K, dtype, workspace, workspace_bytes)) g.coef = workspace;
   return dispatch_group_softmax(dtype, g, GS_STD_BWD, vec, static_cast<hipStream_t>(stream));
 }
 

@@ -98,6 +98,8 @@ struct GroupArgs {
   const int *gate = nullptr;  // the three passes of softmax run only if *gate != 0 (null: always)
   int *flag = nullptr;        // softmax: a word behind the workspace of the three passes, for the one-pass kernels
   size_t ws_bytes = 0;        //          bytes of that workspace (gmax is its start)
+  const void *coef = nullptr;   // std / logsumexp backward: [B, N, 2, K] in the accumulate type, what an entry needs of its
+                                // group side by side (group_coef_kernel); null: gathered from the group arrays
   void *total_w = nullptr;      // std through buckets: the group sums [B, N, K] in the element type are written here,
   int32_t *count_w = nullptr;   // and the entries per group [B, N] here
   const BinArgs *bins = nullptr;  // (host) plan of the buckets
@@ -471,6 +473,33 @@ void launch_group_sum_lds(const ScatterArgs &a, const GroupArgs &g, int tn, hipS
                      stream, a, g, tn - 1, epb);
 }
 
+// What the backward pass of std / logsumexp needs of a group, side by side in the accumulate type ([B, N, 2, K]):
+//   std        mean = total / max(count, 1),  w = grad / (std * divisor)   ->  grad_in = w * (src - mean)
+//   logsumexp  the forward result,            grad                         ->  grad_in = grad * exp(src - result)
+// With an index that is not in order every entry fetches its group's values from a line of its own per array (std: total,
+// count, std, grad; 9 M x 8 floats: 689 us); here it is one line.
+template <typename T, int MODE>
+__global__ __launch_bounds__(kBlock) void group_coef_kernel(GroupArgs g, void *coef) {
+  typedef typename Acc<T>::type F;
+  const int64_t n = g.B * g.N * g.K;
+  F *rec = static_cast<F *>(coef);
+  const T *o = static_cast<const T *>(g.node_out), *go = static_cast<const T *>(g.node_grad);
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlock) {
+    const int64_t node = i / g.K, k = i - node * g.K;
+    F c0, c1;
+    if (MODE == GS_STD_BWD) {
+      const int32_t cnt = g.count[node];
+      c0 = group_mean<T>(static_cast<const T *>(g.total)[i], cnt);
+      c1 = to_acc<T>(go[i]) / (to_acc<T>(o[i]) * group_divisor<T>(cnt, g.unbiased));
+    } else {
+      c0 = to_acc<T>(o[i]);
+      c1 = to_acc<T>(go[i]);
+    }
+    rec[node * 2 * g.K + k] = c0;
+    rec[node * 2 * g.K + g.K + k] = c1;
+  }
+}
+
 // ---- pass 3: the elementwise finish
 template <typename T, int VEC, int MODE>
 __global__ __launch_bounds__(kBlock) void group_finish_kernel(GroupArgs g) {
@@ -513,6 +542,25 @@ __global__ __launch_bounds__(kBlock) void group_finish_kernel(GroupArgs g) {
           continue;
         }
         const int64_t slot = (bb[u] * g.N + idx[u]) * g.K + k0;
+        if constexpr (MODE == GS_STD_BWD || MODE == GS_LSE_BWD) {
+          if (g.coef != nullptr) {
+            // one line per entry instead of three or four: std (mean, grad / (std * divisor)), logsumexp (result, grad)
+            const F *rec = static_cast<const F *>(g.coef) + (bb[u] * g.N + idx[u]) * 2 * g.K + k0;
+            const Vec<F, VEC> c0 = load_vec<F, VEC>(rec), c1 = load_vec<F, VEC>(rec + g.K);
+#pragma unroll
+            for (int v = 0; v < VEC; ++v) {
+              const F xv = to_acc<T>(x[u].v[v]);
+              if (MODE == GS_STD_BWD) {
+                r.v[v] = from_acc<T>(c1.v[v] * (xv - c0.v[v]));
+              } else {
+                const F w = exp_acc(xv - c0.v[v]);
+                r.v[v] = from_acc<T>(xv != xv || w != w ? (F)0 : c1.v[v] * w);
+              }
+            }
+            store_vec_stream<T, VEC>(out + be * g.K + k0, r);
+            continue;
+          }
+        }
         if constexpr (MODE == GS_STD_BWD) {
           // d std / d src = (src - mean) / (std * divisor); a group whose std is 0 gets 0 / 0 = NaN,
           // as autograd gives for the reference's sqrt at 0
@@ -687,6 +735,9 @@ int launch_group_lse_v(const GroupArgs &g, bool backward, hipStream_t stream) {
   const int64_t n_edges = g.B * g.E;
   if (g.B * g.N >= 0x7FFFFFFFll) return TS_ERR_UNSUPPORTED;
   if (backward) {
+    if (g.coef != nullptr)
+      hipLaunchKernelGGL((group_coef_kernel<T, GS_LSE_BWD>), dim3(grid_for(g.B * g.N * g.K)), dim3(kBlock), 0, stream, g,
+                         const_cast<void *>(g.coef));
     hipLaunchKernelGGL((group_finish_kernel<T, VEC, GS_LSE_BWD>), dim3(scatter_grid(n_edges, g.K / VEC, kBlock, 4)),
                        dim3(kBlock), 0, stream, g);
     return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
@@ -718,6 +769,9 @@ int launch_group_std_v(const GroupArgs &g, bool backward, hipStream_t stream) {
   const int64_t n_edges = g.B * g.E;
   if (g.B * g.N >= 0x7FFFFFFFll) return TS_ERR_UNSUPPORTED;
   if (backward) {
+    if (g.coef != nullptr)
+      hipLaunchKernelGGL((group_coef_kernel<T, GS_STD_BWD>), dim3(grid_for(g.B * g.N * g.K)), dim3(kBlock), 0, stream, g,
+                         const_cast<void *>(g.coef));
     hipLaunchKernelGGL((group_finish_kernel<T, VEC, GS_STD_BWD>), dim3(scatter_grid(n_edges, g.K / VEC, kBlock, 4)),
                        dim3(kBlock), 0, stream, g);
     return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;

@@ -885,9 +885,11 @@ struct GroupLogSumExpFn : public torch::autograd::Function<GroupLogSumExpFn> {
     const int64_t dim = ctx->saved_data["dim"].toInt();
     const GroupLayout l = group_layout(src, index, dim);
     Tensor grad_in = at::empty_like(src);
-    check_status(ts_group_logsumexp_backward(src.data_ptr(), index.data_ptr<int64_t>(), out.data_ptr(),
-                                             grad_out.data_ptr(), grad_in.data_ptr(), l.B, l.E, l.K, out.size(dim),
-                                             l.sb, l.se, dtype_code(src), stream_of(src)),
+    Tensor ws = workspace(ts_group_softmax_workspace_bytes(l.B, out.size(dim), l.K, dtype_code(src)), src);
+    check_status(ts_group_logsumexp_backward_with_workspace(src.data_ptr(), index.data_ptr<int64_t>(), out.data_ptr(),
+                                                            grad_out.data_ptr(), grad_in.data_ptr(), l.B, l.E, l.K,
+                                                            out.size(dim), l.sb, l.se, dtype_code(src), ws.data_ptr(),
+                                                            static_cast<size_t>(ws.numel()), stream_of(src)),
                  "scatter_logsumexp backward");
     return {grad_in, Variable(), Variable(), Variable(), Variable()};
   }
@@ -945,10 +947,12 @@ struct GroupStdFn : public torch::autograd::Function<GroupStdFn> {
     const bool unbiased = ctx->saved_data["unbiased"].toBool();
     const GroupLayout l = group_layout(src, index, dim);
     Tensor grad_in = at::empty_like(src);
-    check_status(ts_group_std_backward(src.data_ptr(), index.data_ptr<int64_t>(), total.data_ptr(),
-                                       count.data_ptr<int32_t>(), out.data_ptr(), grad_out.data_ptr(),
-                                       grad_in.data_ptr(), l.B, l.E, l.K, out.size(dim), l.sb, l.se, dtype_code(src),
-                                       unbiased ? 1 : 0, stream_of(src)),
+    Tensor ws = workspace(ts_group_softmax_workspace_bytes(l.B, out.size(dim), l.K, dtype_code(src)), src);
+    check_status(ts_group_std_backward_with_workspace(src.data_ptr(), index.data_ptr<int64_t>(), total.data_ptr(),
+                                                      count.data_ptr<int32_t>(), out.data_ptr(), grad_out.data_ptr(),
+                                                      grad_in.data_ptr(), l.B, l.E, l.K, out.size(dim), l.sb, l.se,
+                                                      dtype_code(src), unbiased ? 1 : 0, ws.data_ptr(),
+                                                      static_cast<size_t>(ws.numel()), stream_of(src)),
                  "scatter_std backward");
     return {grad_in, Variable(), Variable(), Variable(), Variable()};
   }

@@ -384,15 +384,17 @@ def test_logsumexp_forward_and_backward_capi(capi, oracle, monkeypatch, shape, k
     assert float(out[:, N - 3:, :].abs().max()) == 0.0
 
     grad = torch.from_numpy(rng.standard_normal(size=(B, N, K))).to(dtype)
-    grad_in = torch.empty((B, E, K), dtype=dtype, device=DEV)
-    capi.group_logsumexp_backward(src.to(DEV), index1.to(DEV), out, grad.to(DEV), grad_in, B, E, K, N, 0, 1)
-    torch.cuda.synchronize()
     y64 = out.cpu().double()
     want_g = oracle.scatter_logsumexp_backward(src.double(), y64, grad.double(), index, 1)
-    gerr = (grad_in.cpu().double() - want_g).abs()
     gbound = 8 * e * want_g.abs() * (1 + (src.double() - y64.gather(1, index)).abs()) + \
         (2.0 ** -23 if dtype == torch.float16 else 1e-30)
-    assert bool((gerr <= gbound).all()), ("backward", float((gerr - gbound).max()))
+    for with_workspace in (True, False):  # a group's result and gradient laid side by side first, or gathered
+        grad_in = torch.empty((B, E, K), dtype=dtype, device=DEV)
+        capi.group_logsumexp_backward(src.to(DEV), index1.to(DEV), out, grad.to(DEV), grad_in, B, E, K, N, 0, 1,
+                                      with_workspace)
+        torch.cuda.synchronize()
+        gerr = (grad_in.cpu().double() - want_g).abs()
+        assert bool((gerr <= gbound).all()), ("backward", with_workspace, float((gerr - gbound).max()))
 
 
 def test_logsumexp_operator(ts, oracle):
@@ -486,11 +488,16 @@ def test_std_forward_and_backward_capi(capi, oracle, shape, kind, dtype, unbiase
         bound = 8.0 * e * want + 2.0 * e * mean_abs * (1.0 + cnt_n.sqrt())
     assert bool((err <= bound).all()), float((err - bound).max())
 
-    grad_in = torch.empty((B, E, K), dtype=dtype, device=DEV)
-    capi.group_std_backward(src_d, idx_d, total, count, out, grad.to(DEV), grad_in, B, E, K, N, 0, 1, unbiased)
-    torch.cuda.synchronize()
     std64, want_g = oracle.scatter_std_backward(src.double(), grad.double(), index, 1, N, unbiased)
-    got_g = grad_in.cpu().double()
+    for with_workspace in (True, False):  # mean and grad / (std * divisor) laid side by side first, or gathered
+        grad_in = torch.empty((B, E, K), dtype=dtype, device=DEV)
+        capi.group_std_backward(src_d, idx_d, total, count, out, grad.to(DEV), grad_in, B, E, K, N, 0, 1, unbiased,
+                                with_workspace)
+        torch.cuda.synchronize()
+        check_std_gradient(grad_in.cpu().double(), want_g, std64, grad, index, cnt_n, mean_abs, exact, e, dtype)
+
+
+def check_std_gradient(got_g, want_g, std64, grad, index, cnt_n, mean_abs, exact, e, dtype):
     # a group whose std is 0 (one entry, or equal entries): NaN on both sides
     dead = (std64 == 0).gather(1, index)
     assert bool(torch.isnan(got_g[dead]).all()) and bool(torch.isnan(want_g[dead]).all())
