@@ -246,6 +246,68 @@ def test_one_pass_kernels_take_large_sorted_inputs(capi, monkeypatch, dtype, K):
         assert bool(((a[0] - b[0]).abs() <= 16 * e * (1.0 + a[0].abs())).all())
         assert bool(((a[1] - b[1]).abs() <= 64 * e * (1.0 + a[1].abs())).all())
 
+@pytest.mark.parametrize("kind", ["sorted", "random", "hubs"])
+@pytest.mark.parametrize("dtype,K", [(torch.float32, 8), (torch.float32, 1), (torch.bfloat16, 16), (torch.float64, 3)])
+def test_operators_at_sizes_that_take_the_buckets(ts, dtype, K, kind):
+    """scatter_std, scatter_logsumexp and scatter_softmax through the operators at the library's default settings, at a
+    size from which the route through buckets of groups applies (group_binned.h), against a double-precision
+    evaluation with torch's own index_add_ / scatter_reduce_ on the CPU (on the device a double-precision index_add_
+    is a compare-and-swap loop, which a hub group of 600 k entries stalls for minutes): sorted, random and a power-law
+    index whose hub groups fill many chunks."""
+    E, N = 1_200_000, 150_000
+    if K == 1:
+        E *= 2
+    g = torch.Generator().manual_seed(7)
+    if kind == "hubs":
+        w = torch.arange(1, N + 1, dtype=torch.float64) ** -1.3
+        index = torch.multinomial(w, E, replacement=True, generator=g)
+    else:
+        index = torch.randint(0, N, (E,), generator=g)
+        if kind == "sorted":
+            index = index.sort().values
+    src_cpu = (torch.randn((E, K), generator=g) * 2 + 0.5).to(dtype)
+    src, x = src_cpu.to(DEV), src_cpu.double()
+    index_dev = index.to(DEV)
+    idx2 = index.view(E, 1).expand(E, K)
+    e = EPS_T[dtype]
+    cnt = torch.bincount(index, minlength=N).double().view(N, 1)
+    total = torch.zeros((N, K), dtype=torch.float64, device='cpu').index_add_(0, index, x)
+    mean = total / cnt.clamp(min=1)
+    # std (unbiased)
+    m2 = torch.zeros((N, K), dtype=torch.float64, device='cpu').index_add_(0, index, (x - mean[index]) ** 2)
+    want = (m2 / ((cnt - 1).clamp(min=1) + 1e-6)).sqrt()
+    got = ts.scatter_std(src, index_dev, 0, None, N).double().cpu()
+    mean_abs = torch.zeros((N, K), dtype=torch.float64, device='cpu').index_add_(0, index, x.abs()) / cnt.clamp(min=1)
+    if dtype in (torch.float32, torch.float64):
+        bound = 4 * e * want + 4 * e * mean_abs + 1e-30
+    else:
+        bound = 8.0 * e * want + 2.0 * e * mean_abs * (1.0 + cnt.sqrt())
+    assert bool(((got - want).abs() <= bound).all()), float(((got - want).abs() - bound).max())
+    # logsumexp and softmax
+    gmax = torch.full((N, K), float("-inf"), dtype=torch.float64, device='cpu').scatter_reduce_(0, idx2, x, "amax")
+    z = x - gmax[index]
+    gsum = torch.zeros((N, K), dtype=torch.float64, device='cpu').index_add_(0, index, z.exp())
+    want_lse = torch.where(cnt > 0, gsum.log() + gmax, torch.zeros_like(gsum))
+    got_lse = ts.scatter_logsumexp(src, index_dev, 0, None, N).double().cpu()
+    lse_bound = e * (1.0 + want_lse.abs()) * (4 if dtype in (torch.float32, torch.float64) else 30)
+    assert bool(((got_lse - want_lse).abs() <= lse_bound).all()), float(((got_lse - want_lse).abs() - lse_bound).max())
+    want_sm = z.exp() / gsum[index]
+    got_sm = ts.scatter_softmax(src, index_dev, 0, N).double().cpu()
+    sm_bound = e * (4.0 + z.abs()) * want_sm * (4 if dtype in (torch.float32, torch.float64) else 1) + 1e-30
+    assert bool(((got_sm - want_sm).abs() <= sm_bound).all()), float(((got_sm - want_sm).abs() - sm_bound).max())
+    # the gradient of std through the operator (one line per entry in the backward pass)
+    xs = src.clone().requires_grad_(True)
+    y = ts.scatter_std(xs, index_dev, 0, None, N)
+    go = torch.randn((N, K), generator=g).to(dtype)
+    (gi,) = torch.autograd.grad(y, xs, go.to(DEV))
+    gi, y = gi.cpu(), y.detach().cpu()
+    div = (cnt - 1).clamp(min=1) + 1e-6
+    want_g = (go.double() / (y.detach().double() * div))[index] * (x - mean[index])
+    live = (cnt[index] > 1).expand(E, K) & torch.isfinite(want_g)
+    scale = (go.double().abs() / y.detach().double().clamp_min(1e-300))[index]
+    gb = 16 * e * (want_g.abs() + scale * mean_abs[index] / cnt[index].clamp(min=1)) + (2.0 ** -24 if dtype == torch.float16 else 1e-30)
+    assert bool(((gi.double() - want_g).abs()[live] <= gb[live]).all())
+
 
 def test_special_values_capi(capi, oracle):
     """-inf entries, a group of only -inf, NaN in a group, entries outside [0, N), an empty group."""
