@@ -24,6 +24,9 @@ constexpr int kGroupBinU = 8;         // units (one entry's VEC columns) per lan
 constexpr int kGroupBinRows = 2048;   // groups per bucket at most
 constexpr int kGroupBinSlots = 8192;  // groups x columns of a bucket at most (the slab of a chunk: 16 bytes per slot)
 constexpr int kGroupBinLong = 64;     // entries of a group inside a chunk from which on a wavefront takes the group
+constexpr int kGroupBinCoop = 2;      // up to this many long groups in a chunk, the whole workgroup takes them one by one
+constexpr int kGroupBinCoopLanes = 8;  // and held by at least this many lanes (few entries per step of one wavefront)
+constexpr int kGroupBinCoopCols = 64;  // ... for rows of up to this many columns
 constexpr int kGroupBinMaxLong = 128;  // such groups per chunk at most (a chunk holds at most 8192 entries)
 constexpr int kGroupBinMaxLanes = 32;  // lanes per entry at most (a chunk then holds 256 entries)
 
@@ -47,8 +50,10 @@ inline GroupBinPlan group_bin_plan(int64_t B, int64_t E, int64_t K, int64_t N, i
   if (vec < 1 || K % vec != 0) return r;
   const int64_t lanes = K / vec;
   if (lanes > kGroupBinMaxLanes || K > kGroupBinSlots) return r;
-  // six launches: below a few MB the three passes are ahead
+  // six launches: below a few MB the three passes are ahead; so they are with single values in few, large groups
+  // (their LDS tables hold every group: 4 M values in 4 k groups, random order: logsumexp 70 against 125 us)
   if (!any_size && n_edges * K * elem_bytes < ((int64_t)4 << 20)) return r;
+  if (!any_size && K == 1 && n_edges > 256 * rows) return r;
   const int64_t epw = kWave / lanes;  // entries per row of a wavefront
   const int64_t chunk = (int64_t)(kBinBlock / kWave) * kGroupBinU * epw;
   // groups per bucket: a power of two whose table fits, and so that an average bucket fills at most 0.6 chunks
@@ -202,6 +207,7 @@ __global__ __launch_bounds__(kBinBlock) void group_bin_kernel(GroupArgs g, BinAr
   __shared__ int32_t s_wsum[W];
   __shared__ int32_t s_long[kGroupBinMaxLong];  // groups for a wavefront
   __shared__ int s_nlong;
+  __shared__ double s_part[W][kGroupBinCoopCols];  // where the wavefronts that share a long group meet
   if (p.unsorted != nullptr && *p.unsorted != 1) return;  // the caller's one-pass kernels took the call
   const int wg = (int)blockIdx.x;
   const int bucket = p.wg_bucket[wg];
@@ -286,10 +292,27 @@ __global__ __launch_bounds__(kBinBlock) void group_bin_kernel(GroupArgs g, BinAr
                                           (int64_t)group_bin_slab_words(table, R);
   // the lanes that share a group meet in a butterfly: a wavefront's lanes with the same columns (offsets 32 ... lanes),
   // or `share` neighbouring lanes (offsets share / 2 ... 1)
-  auto stat = [&](int r, int c, int first, int step, int off_hi, int off_lo) {
-    auto meet = [&](auto v, auto op) {
-      for (int off = off_hi; off >= off_lo; off >>= 1) v = op(v, __shfl_xor(v, off));
-      return v;
+  // coop: all wavefronts of the workgroup share the group (a chunk with one or two long groups: the groups of hub nodes, or
+  // few groups of many entries each); their totals meet in LDS, added in wavefront order.
+  auto stat = [&](int r, int c, int first, int step, int off_hi, int off_lo, bool coop) {
+    auto meet = [&](auto (&v)[VEC], auto op) {  // the VEC columns of this lane at once: two barriers per meeting
+#pragma unroll
+      for (int j = 0; j < VEC; ++j)
+        for (int off = off_hi; off >= off_lo; off >>= 1) v[j] = op(v[j], __shfl_xor(v[j], off));
+      if (coop) {
+        if (sub == 0) {
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) s_part[wave][c + j] = (double)v[j];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+          auto t = (decltype(v[j] + v[j]))s_part[0][c + j];
+          for (int w2 = 1; w2 < W; ++w2) t = op(t, (decltype(v[j] + v[j]))s_part[w2][c + j]);
+          v[j] = t;
+        }
+        __syncthreads();
+      }
     };
     const bool wide = off_hi >= off_lo;
     const int e0 = s_off[r], cnt = s_n[r];
@@ -319,11 +342,8 @@ __global__ __launch_bounds__(kBinBlock) void group_bin_kernel(GroupArgs g, BinAr
         for (int v = 0; v < VEC; ++v) acc[v] += to_acc<T>(y.v[v]);
       });
 #pragma unroll
-      for (int v = 0; v < VEC; ++v) {
-        sum[v] = (double)acc[v];
-        if (wide) sum[v] = meet(sum[v], [](double a, double b) { return a + b; });
-        acc[v] = (F)0;
-      }
+      for (int v = 0; v < VEC; ++v) sum[v] = (double)acc[v], acc[v] = (F)0;
+      if (wide) meet(sum, [](double a, double b) { return a + b; });
       if (single) {
         F mean[VEC];
 #pragma unroll
@@ -348,10 +368,8 @@ __global__ __launch_bounds__(kBinBlock) void group_bin_kernel(GroupArgs g, BinAr
         });
       }
 #pragma unroll
-      for (int v = 0; v < VEC; ++v) {
-        m2[v] = (double)acc[v];
-        if (wide) m2[v] = meet(m2[v], [](double a, double b) { return a + b; });
-      }
+      for (int v = 0; v < VEC; ++v) m2[v] = (double)acc[v];
+      if (wide) meet(m2, [](double a, double b) { return a + b; });
 #pragma unroll
       for (int v = 0; v < VEC; ++v) {
         part[v].a = (uint64_t)__double_as_longlong(sum[v]);
@@ -368,9 +386,9 @@ __global__ __launch_bounds__(kBinBlock) void group_bin_kernel(GroupArgs g, BinAr
         for (int v = 0; v < VEC; ++v) top[v] = max_acc(top[v], to_acc<T>(y.v[v]));  // a NaN never wins
       });
       bool won[VEC];
+      if (wide) meet(top, [](F a, F b) { return max_acc(a, b); });
 #pragma unroll
       for (int v = 0; v < VEC; ++v) {
-        if (wide) top[v] = meet(top[v], [](F a, F b) { return max_acc(a, b); });
         top[v] = OrdKey<F>::dec(OrdKey<F>::enc(top[v]));  // -0.0 folds onto +0.0
         // softmax: an entry has to beat lowest(); a group without a winner is shifted by 0 (composite/softmax.py:16-18)
         won[v] = MODE == GS_LSE || top[v] > to_acc<T>(ElemLim<T>::lowest());
@@ -385,9 +403,10 @@ __global__ __launch_bounds__(kBinBlock) void group_bin_kernel(GroupArgs g, BinAr
         }
       });
 #pragma unroll
+      for (int v = 0; v < VEC; ++v) sum[v] = (double)acc[v];
+      if (wide) meet(sum, [](double a, double b) { return a + b; });
+#pragma unroll
       for (int v = 0; v < VEC; ++v) {
-        sum[v] = (double)acc[v];
-        if (wide) sum[v] = meet(sum[v], [](double a, double b) { return a + b; });
         part[v].a = won[v] ? (uint64_t)OrdKey<F>::enc(top[v]) : (uint64_t)group_empty_key<T>();
         part[v].b = sum[v];
         part[v].n = 0;
@@ -417,9 +436,13 @@ __global__ __launch_bounds__(kBinBlock) void group_bin_kernel(GroupArgs g, BinAr
     const int r = live ? i / lanes : 0;
     const bool mine = live && !(nlong > 0 && s_n[r] > kGroupBinLong);
     // (a lane group that has no item still takes part in the butterflies of its wavefront)
-    stat(r, (i - r * lanes) * VEC, mine ? slane : 0x7FFFFFF0, share, share / 2, 1);
+    stat(r, (i - r * lanes) * VEC, mine ? slane : 0x7FFFFFF0, share, share / 2, 1, false);
   }
-  for (int q = wave; q < nlong; q += W) stat(s_long[q], col, sub, epw, kWave / 2, lanes);
+  if (nlong > 0 && nlong <= kGroupBinCoop && K <= kGroupBinCoopCols && lanes >= kGroupBinCoopLanes) {
+    for (int q = 0; q < nlong; ++q) stat(s_long[q], col, wave * epw + sub, W * epw, kWave / 2, lanes, true);
+  } else {
+    for (int q = wave; q < nlong; q += W) stat(s_long[q], col, sub, epw, kWave / 2, lanes, false);
+  }
 }
 
 // Buckets that were not reduced in exactly one chunk: their slabs merged, slab by slab in chunk order, element by
