@@ -309,8 +309,12 @@ def test_operators_at_sizes_that_take_the_buckets(ts, dtype, K, kind):
     assert bool(((gi.double() - want_g).abs()[live] <= gb[live]).all())
 
 
-def test_special_values_capi(capi, oracle):
-    """-inf entries, a group of only -inf, NaN in a group, entries outside [0, N), an empty group."""
+@pytest.mark.parametrize("bins", ["0", "2"])
+def test_special_values_capi(capi, oracle, monkeypatch, bins):
+    """-inf entries, a group of only -inf, NaN in a group, entries outside [0, N), an empty group; through the three
+    passes (bins = 0) and through buckets of groups (bins = 2), softmax and logsumexp. A hub variant repeats the
+    values so that the groups of the first bucket fill several chunks (slabs merged with -inf and NaN partials)."""
+    monkeypatch.setenv("TS_GROUP_BINS", bins)
     src = torch.tensor([0.2, 0, 0.2, -2.1, 3.2, 7, -1, float("-inf"), float("-inf"), float("-inf"),
                         1.0, float("nan"), 2.0, 5.0])
     index = torch.tensor([0, 1, 0, 1, 1, 2, 4, 4, 5, 5, 6, 6, 6, 9])
@@ -325,6 +329,20 @@ def test_special_values_capi(capi, oracle):
         got = out.cpu()
         assert torch.allclose(got[keep], want, rtol=1e-5, atol=1e-7, equal_nan=True), (log_space, got, want)
         assert float(got[~keep].abs().max()) == 0.0
+    for reps in (1, 6000):  # 6000: 78 000 single values in 8 groups, the groups of three entries in three chunks each
+        s, i = src[keep].repeat(reps), index[keep].repeat(reps)
+        out = torch.full((N,), 7.0, device=DEV)
+        capi.group_logsumexp(s.to(DEV), i.to(DEV), out, 1, s.numel(), 1, N, 0, 1)
+        torch.cuda.synchronize()
+        want = oracle.scatter_logsumexp(s.double(), i, 0, None, N)
+        assert torch.allclose(out.cpu().double(), want, rtol=1e-5, atol=1e-6, equal_nan=True), (reps, out, want)
+        for log_space in (False, True):
+            o = torch.empty(s.numel(), device=DEV)
+            capi.group_softmax(s.to(DEV), i.to(DEV), o, 1, s.numel(), 1, N, 0, 1, log_space)
+            torch.cuda.synchronize()
+            w = (oracle.scatter_log_softmax(s.double(), i, 0, 1e-12, N) if log_space
+                 else oracle.scatter_softmax(s.double(), i, 0, dim_size=N))
+            assert torch.allclose(o.cpu().double(), w, rtol=1e-5, atol=1e-6, equal_nan=True), (reps, log_space)
 
 
 def test_workspace_and_argument_checks(capi):
