@@ -874,6 +874,21 @@ GroupBinPlan group_bins_plan(int64_t B, int64_t E, int64_t K, int64_t N, int dty
   if (r.bytes > 0) r.bytes += front;
   return r;
 }
+// std / logsumexp: the one-pass tiles for an index in order, their scratch behind that of the buckets (at ws + skip).
+// TS_GROUP_FUSED (tuning aid): 0 never, 2 at any size and whatever the index looks like.
+FusedReducePlan group_tiles_plan(int64_t B, int64_t E, int64_t K, int dtype, bool aligned, void *ws, size_t ws_bytes,
+                                 size_t skip) {
+  const int mode = env_int("TS_GROUP_FUSED", 1);
+  if (mode == 0 || skip == 0) {
+    FusedReducePlan r;
+    r.ok = false;
+    r.bytes = 0;
+    return r;
+  }
+  return group_reduce_fused_plan(B, E, K, kElemBytes[dtype], aligned,
+                                 ws != nullptr && ws_bytes > skip ? static_cast<char *>(ws) + skip : nullptr,
+                                 ws_bytes > skip ? ws_bytes - skip : 0, mode == 2);
+}
 }  // namespace
 
 namespace {
@@ -974,6 +989,11 @@ int ts_group_logsumexp(const void *src, const int64_t *index, void *out, int64_t
       g.se = index_stride_e;
       g.eps = eps;
       g.bins = &plan.p;
+      const FusedReducePlan tiles = group_tiles_plan(B, E, K, dtype, aligned16(src), workspace, workspace_bytes, plan.bytes);
+      if (tiles.ok) {
+        g.tiles = &tiles.f;
+        g.tiles_force = env_int("TS_GROUP_FUSED", 1) == 2;
+      }
       return dispatch_group_softmax(dtype, g, GS_LSE_BINS, group_bins_vec(K, dtype, aligned16(src)),
                                     static_cast<hipStream_t>(stream));
     }
@@ -996,7 +1016,8 @@ int ts_group_logsumexp(const void *src, const int64_t *index, void *out, int64_t
 
 size_t ts_group_bins_workspace_bytes(int64_t B, int64_t E, int64_t K, int64_t N, int dtype) {
   if (!valid_dtype(dtype) || !is_float_dtype(dtype) || !sizes_ok(B, N, E, K)) return 0;
-  return group_bins_plan(B, E, K, N, dtype, true, nullptr, 0).bytes;
+  const size_t bins = group_bins_plan(B, E, K, N, dtype, true, nullptr, 0).bytes;
+  return bins + group_tiles_plan(B, E, K, dtype, true, nullptr, 0, bins).bytes;
 }
 
 int ts_group_std_forward(const void *src, const int64_t *index, void *total, int32_t *count, void *out, int64_t B,
@@ -1024,6 +1045,11 @@ int ts_group_std_forward(const void *src, const int64_t *index, void *total, int
   g.sb = index_stride_b;
   g.se = index_stride_e;
   g.bins = &plan.p;
+  const FusedReducePlan tiles = group_tiles_plan(B, E, K, dtype, al, workspace, workspace_bytes, plan.bytes);
+  if (tiles.ok) {
+    g.tiles = &tiles.f;
+    g.tiles_force = env_int("TS_GROUP_FUSED", 1) == 2;
+  }
   return dispatch_group_softmax(dtype, g, GS_STD_BINS, group_bins_vec(K, dtype, al), static_cast<hipStream_t>(stream));
 }
 

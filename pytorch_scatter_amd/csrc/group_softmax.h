@@ -77,6 +77,7 @@ enum {
 };
 
 struct BinArgs;
+struct FusedReduceArgs;
 
 struct GroupArgs {
   const void *src;       // [B, E, K]: forward input; backward: the forward result y
@@ -103,6 +104,8 @@ struct GroupArgs {
   void *total_w = nullptr;      // std through buckets: the group sums [B, N, K] in the element type are written here,
   int32_t *count_w = nullptr;   // and the entries per group [B, N] here
   const BinArgs *bins = nullptr;  // (host) plan of the buckets
+  const FusedReduceArgs *tiles = nullptr;  // (host) std / logsumexp: plan of the one-pass tiles in front of the buckets
+  int tiles_force = 0;                     //        ... which run whatever a sample of the index looks like
 };
 
 // std: the group mean as the reference forms it (composite/std.py:27-31: sum / clamp(count, 1), in the
@@ -677,7 +680,18 @@ inline ScatterArgs group_index_args(const GroupArgs &g) {
 
 }  // namespace ts
 #include "group_binned.h"
+#include "group_fused_reduce.h"
 namespace ts {
+
+// std / logsumexp forward: the one-pass tiles for an index in order where they apply, then (gated on their verdict)
+// the passes through buckets of groups
+template <typename T, int VEC, int MODE>
+int launch_group_reduce(const GroupArgs &g, hipStream_t stream) {
+  if (g.tiles == nullptr) return launch_group_bins<T, VEC, MODE>(g, stream);
+  const int rc = launch_group_reduce_fused<T, VEC, MODE>(g, *g.tiles, g.tiles_force != 0, stream);
+  if (rc != TS_OK) return rc;
+  return launch_group_bins<T, VEC, MODE>(g, stream, g.tiles->flag);
+}
 
 template <typename T, int VEC, int MODE>
 int launch_group_softmax_m(const GroupArgs &g_in, hipStream_t stream) {
@@ -797,8 +811,8 @@ int launch_group_softmax_v(const GroupArgs &g, int mode, hipStream_t stream) {
   switch (mode) {
   case GS_STD: return launch_group_std_v<T, VEC>(g, false, stream);
   case GS_STD_BWD: return launch_group_std_v<T, VEC>(g, true, stream);
-  case GS_STD_BINS: return launch_group_bins<T, VEC, GS_STD>(g, stream);
-  case GS_LSE_BINS: return launch_group_bins<T, VEC, GS_LSE>(g, stream);
+  case GS_STD_BINS: return launch_group_reduce<T, VEC, GS_STD>(g, stream);
+  case GS_LSE_BINS: return launch_group_reduce<T, VEC, GS_LSE>(g, stream);
   case GS_LSE: return launch_group_lse_v<T, VEC>(g, false, stream);
   case GS_LSE_BWD: return launch_group_lse_v<T, VEC>(g, true, stream);
   case GS_SOFTMAX: return launch_group_softmax_m<T, VEC, GS_SOFTMAX>(g, stream);

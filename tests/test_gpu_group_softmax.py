@@ -183,6 +183,58 @@ def test_one_pass_kernels_capi(capi, oracle, monkeypatch, shape, kind, dtype, ti
     grad = torch.from_numpy(rng.standard_normal(size=(B, E, K))).to(dtype)
     check_against_oracle(capi, oracle, src, grad, fused_index(kind, rng, E, N), shape, dtype)
 
+@pytest.mark.parametrize("shape,kind,dtype",
+                         product(FUSED_SHAPES + [(1, 40_000, 8, 3000)], ["sorted", "skewed", "outside", "one_descent"], DTYPES))
+@pytest.mark.parametrize("tile", [256, 0])
+def test_std_and_logsumexp_one_pass_tiles_capi(capi, oracle, monkeypatch, shape, kind, dtype, tile):
+    """scatter_std / scatter_logsumexp forward through the one-pass tiles for an index in order
+    (group_fused_reduce.h), switched on at any size: runs inside a tile, runs that cross one border or fill whole
+    tiles (their partials merged), entries outside [0, N), empty groups, and an index with one descent (the tiles
+    notice, the passes through buckets of groups write every result again)."""
+    B, E, K, N = shape
+    monkeypatch.setenv("TS_GROUP_FUSED", "2")
+    monkeypatch.setenv("TS_GROUP_BINS", "2")
+    if tile:
+        monkeypatch.setenv("TS_GROUP_TILE", str(tile))
+    exact = dtype in (torch.float32, torch.float64)
+    if kind == "skewed" and not exact:
+        pytest.skip("a 16-bit group sum over hundreds of entries is not meaningful")
+    rng = np.random.default_rng(E * 23 + K + N)
+    src = torch.from_numpy(rng.standard_normal(size=(B, E, K)) * 3 + 1).to(dtype)
+    index1 = fused_index(kind, rng, E, N)
+    keep = (index1 >= 0) & (index1 < N)
+    index = index1.view(1, E, 1).expand(B, E, K)
+    src_k, index_k = src[:, keep], index[:, keep]
+    e = EPS_T[dtype]
+    want_cnt = np.bincount(index1[keep].numpy(), minlength=N)
+    cnt_n = torch.from_numpy(want_cnt).double().view(1, N, 1).clamp(1).expand(B, N, K)
+    abs64 = oracle.scatter(src_k.double().abs(), index_k, 1, None, N, "sum")[0]
+    sum64 = oracle.scatter(src_k.double(), index_k, 1, None, N, "sum")[0]
+    for unbiased in (True, False):
+        total = torch.full((B, N, K), 7, dtype=dtype, device=DEV)
+        count = torch.full((B, N), -7, dtype=torch.int32, device=DEV)
+        out = torch.full((B, N, K), 7, dtype=dtype, device=DEV)
+        capi.group_std_forward(src.to(DEV), index1.to(DEV), total, count, out, B, E, K, N, 0, 1, unbiased)
+        torch.cuda.synchronize()
+        for b in range(B):
+            assert count.cpu().view(B, N)[b].tolist() == want_cnt.tolist()
+        assert bool(((total.cpu().double() - sum64).abs() <= e * sum64.abs() + min(e, 4e-6) * abs64 + 1e-30).all())
+        want = oracle.scatter_std(src_k if exact else src_k.double(), index_k, 1, None, N, unbiased).double()
+        err = (out.cpu().double() - want).abs()
+        if exact:
+            bound = e * want + (1e-6 if dtype == torch.float32 else 1e-12)
+        else:
+            bound = 8.0 * e * want + 2.0 * e * (abs64 / cnt_n) * (1.0 + cnt_n.sqrt())
+        assert bool((err <= bound).all()), (unbiased, float((err - bound).max()))
+    out = torch.full((B, N, K), 7, dtype=dtype, device=DEV)
+    capi.group_logsumexp(src.to(DEV), index1.to(DEV), out, B, E, K, N, 0, 1)
+    torch.cuda.synchronize()
+    want = oracle.scatter_logsumexp(src_k if exact else src_k.double(), index_k, 1, None, N).double()
+    err = (out.cpu().double() - want).abs()
+    bound = e * (1.0 + want.abs()) if exact else e * (30.0 + want.abs())
+    assert bool((err <= bound).all()), float((err - bound).max())
+
+
 
 def test_one_pass_kernels_leave_their_verdict(capi, monkeypatch):
     """The word behind the workspace of the three passes says whether the tiles found the index in order: 1 after
