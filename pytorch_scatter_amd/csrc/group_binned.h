@@ -82,7 +82,7 @@ inline GroupBinPlan group_bin_plan(int64_t B, int64_t E, int64_t K, int64_t N, i
   const int table = (int)(K << rshift);
   const int64_t n_slabs = 2 * (n_edges / chunk) + 2;  // a bucket of m >= 2 chunks holds more than (m - 1) chunks of entries
   const size_t slab_bytes = group_bin_slab_words(table, 1 << rshift) * 8;
-  if ((size_t)n_slabs * slab_bytes > ((size_t)2 << 30)) return r;
+  if ((size_t)n_slabs * slab_bytes > ((size_t)1 << 30)) return r;  // (an upper bound: every chunk of every bucket among several)
   auto up = [](size_t x) { return (x + 255) & ~(size_t)255; };
   size_t off = 0;
   auto take = [&](size_t bytes) { const size_t o = off; off += up(bytes); return o; };
