@@ -588,32 +588,38 @@ static __global__ __launch_bounds__(kBinBlock) void bin_scan_kernel(BinArgs p) {
 // and inside [0, N)), in rounds of one entry per lane: what a place pass leaves for the segmented reduction that
 // finishes a sorted index
 __device__ __forceinline__ void bin_row_pointers(const ScatterArgs &a, int64_t lo, int tile, GapList &s_gaps) {
-  // (long ranges of rows without entries are written by the wavefront or the workgroup: gap_rows; a round may span
-  // two batches, whose pointers differ, so the list is emptied after every round)
+  // Long ranges of rows without entries are written by the wavefront or, through the list, by the workgroup
+  // (gap_rows): one list for the whole tile, emptied once at the end -- a range that finds the list full stays with
+  // its wavefront. (One barrier pair per round of 1024 entries, and a 64-bit division per entry for the batch row,
+  // made this pass 53 us for 9 M entries, 37 us without.)
+  if (threadIdx.x == 0) s_gaps.n = 0;
+  __syncthreads();
+  const int64_t n_all = a.B * a.E;
   for (int j = 0; j < kBinPer; ++j) {
     if (j * kBinPlaceBlock >= tile) break;  // uniform
-    if (threadIdx.x == 0) s_gaps.n = 0;
-    __syncthreads();
     const int64_t be = lo + threadIdx.x + (int64_t)j * kBinPlaceBlock;
-    const bool live = be < a.B * a.E;
-    const int64_t b = live ? be / a.E : 0, e = live ? be - b * a.E : 0;
+    const bool live = be < n_all;
+    int64_t b = 0, e = live ? be : 0;
+    if (a.B > 1 && live) {
+      b = be / a.E;
+      e = be - b * a.E;
+    }
     const int64_t *idx = a.index + b * a.sb;
     int64_t top = live ? idx[e] : -1;
     int64_t bot = e == 0 ? 0 : idx[e - 1] + 1;
     if (bot < 0) bot = 0;
     if (top > a.N) top = a.N;
     if (!live) top = bot - 1;
-    // the ranges of one round are written through pointers relative to batch 0: lanes of one wavefront may
+    // the ranges are written through pointers relative to batch 0: lanes of one wavefront may
     // belong to two batches
     const int64_t off = b * (a.N + 1);
     gap_rows(a.route_ptr, off + bot, off + top, e, s_gaps);
     const bool last = live && e == a.E - 1;
     const int64_t tl = top < 0 ? 0 : top + 1;
     gap_rows(a.route_ptr, off + tl, last ? off + a.N : off + tl - 1, a.E, s_gaps);
-    __syncthreads();
-    gap_rows_finish(a.route_ptr, s_gaps);
-    __syncthreads();
   }
+  __syncthreads();
+  gap_rows_finish(a.route_ptr, s_gaps);
 }
 
 // (eight wavefronts per SIMD, i.e. at most 64 vector registers: two workgroups per CU at CAP = 8192; left to itself
