@@ -421,6 +421,11 @@ int ts_group_std_backward_with_workspace(const void *src, const int64_t *index, 
  * workspace: TS_ERR_UNSUPPORTED when the route does not apply, TS_ERR_WORKSPACE when the workspace is too small.
  * ts_group_logsumexp takes the same route by itself when its workspace has that size. */
 size_t ts_group_bins_workspace_bytes(int64_t B, int64_t E, int64_t K, int64_t N, int dtype);
+/* The workspace with which every route of ts_group_softmax, ts_group_softmax_backward and ts_group_logsumexp is open
+ * to a call of this shape: the three passes' part (ts_group_softmax_workspace_bytes), the buckets of groups where
+ * they apply, and behind them the records of the one-pass tiles (which otherwise live in the three passes' part and
+ * are declined when that is too small: few groups of many entries). Never smaller than either of the other two. */
+size_t ts_group_workspace_bytes(int64_t B, int64_t E, int64_t K, int64_t N, int dtype);
 int ts_group_std_forward(const void *src, const int64_t *index, void *total, int32_t *count, void *out,
                          int64_t B, int64_t E, int64_t K, int64_t N, int64_t index_stride_b,
                          int64_t index_stride_e, int dtype, int unbiased, void *workspace,

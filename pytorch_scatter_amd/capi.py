@@ -29,7 +29,7 @@ EXPORTS = (
     "ts_scatter", "ts_scatter_workspace_bytes", "ts_scatter_workspace_zero_bytes", "ts_scatter_with_workspace", "ts_scatter_count", "ts_scatter_count_workspace_bytes", "ts_scatter_count_with_workspace", "ts_scatter_sum_count_workspace_bytes", "ts_scatter_sum_count_with_workspace", "ts_divide_by_count", "ts_arg_backward",
     "ts_group_softmax_workspace_bytes", "ts_group_softmax", "ts_group_softmax_backward",
     "ts_group_logsumexp", "ts_group_logsumexp_backward",
-    "ts_group_std", "ts_group_std_backward", "ts_group_bins_workspace_bytes", "ts_group_std_forward",
+    "ts_group_std", "ts_group_std_backward", "ts_group_bins_workspace_bytes", "ts_group_workspace_bytes", "ts_group_std_forward",
     "ts_group_std_backward_with_workspace", "ts_group_logsumexp_backward_with_workspace",
     "ts_index_to_indptr", "ts_indptr_to_index_workspace_bytes", "ts_indptr_to_index",
     "ts_sort_index_workspace_bytes", "ts_sort_index",
@@ -63,6 +63,7 @@ def lib() -> ctypes.CDLL:
         _lib.ts_scatter_sum_count_workspace_bytes.restype = ctypes.c_size_t
         _lib.ts_sort_index_workspace_bytes.restype = ctypes.c_size_t
         _lib.ts_group_bins_workspace_bytes.restype = ctypes.c_size_t
+        _lib.ts_group_workspace_bytes.restype = ctypes.c_size_t
         _lib.ts_segment_csr_permuted_workspace_bytes.restype = ctypes.c_size_t
     return _lib
 
@@ -274,11 +275,9 @@ def group_bins_workspace_bytes(B, E, K, N, dtype) -> int:
 
 def group_softmax(src, index, out, B, E, K, N, sb, se, log_space: bool, eps: float = 1e-12):
     _dev(src, index, out)
-    ws, nbytes = _group_workspace(out, B, N, K)
-    big = group_bins_workspace_bytes(B, E, K, N, out.dtype)  # where it applies: buckets of groups for an unsorted index
-    if big > nbytes:
-        nbytes = big
-        ws = torch.empty(nbytes, dtype=torch.uint8, device=out.device)
+    # the workspace that opens every route: three passes, buckets of groups (unsorted index), one-pass tiles (sorted)
+    nbytes = int(lib().ts_group_workspace_bytes(_i(B), _i(E), _i(K), _i(N), DTYPE[out.dtype]))
+    ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=out.device)
     with torch.cuda.device(out.device):
         _check(lib().ts_group_softmax(_p(src), _p(index), _p(out), _i(B), _i(E), _i(K), _i(N), _i(sb), _i(se),
                                       DTYPE[out.dtype], int(log_space), ctypes.c_double(eps), _p(ws),
@@ -288,7 +287,8 @@ def group_softmax(src, index, out, B, E, K, N, sb, se, log_space: bool, eps: flo
 
 def group_softmax_backward(result, grad_out, index, grad_in, B, E, K, N, sb, se, log_space: bool):
     _dev(result, grad_out, index, grad_in)
-    ws, nbytes = _group_workspace(grad_in, B, N, K)
+    nbytes = int(lib().ts_group_workspace_bytes(_i(B), _i(E), _i(K), _i(N), DTYPE[grad_in.dtype]))
+    ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=grad_in.device)
     with torch.cuda.device(grad_in.device):
         _check(lib().ts_group_softmax_backward(_p(result), _p(grad_out), _p(index), _p(grad_in), _i(B), _i(E),
                                                _i(K), _i(N), _i(sb), _i(se), DTYPE[grad_in.dtype],

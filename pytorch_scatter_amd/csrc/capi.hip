@@ -933,9 +933,17 @@ int run_group_softmax(const void *src, const void *grad, const int64_t *index, v
   const int vec = (full > 1 && K % full == 0 && al) ? full : 1;
   // forward with a workspace of ts_group_bins_workspace_bytes(): an index that is not in order goes through buckets of groups
   GroupBinPlan plan;
+  plan.ok = false;
   if (with_keys) {
     plan = group_bins_plan(B, E, K, N, dtype, al, workspace, workspace_bytes);
     if (plan.ok && group_bins_vec(K, dtype, al) == vec) g.bins = &plan.p;
+  }
+  // a workspace of ts_group_workspace_bytes(): what lies behind the three passes' (and the buckets') part is scratch
+  // for the one-pass tiles
+  const size_t used = plan.ok ? plan.bytes : need;
+  if (workspace_bytes > used) {
+    g.fused_ws = static_cast<char *>(workspace) + used;
+    g.fused_ws_bytes = workspace_bytes - used;
   }
   return dispatch_group_softmax(dtype, g, mode, vec, stream);
 }
@@ -1012,6 +1020,17 @@ int ts_group_logsumexp(const void *src, const int64_t *index, void *out, int64_t
   const int full = kVecBytes / kElemBytes[dtype];
   const int vec = (full > 1 && K % full == 0 && aligned16(src)) ? full : 1;
   return dispatch_group_softmax(dtype, g, GS_LSE, vec, static_cast<hipStream_t>(stream));
+}
+
+size_t ts_group_workspace_bytes(int64_t B, int64_t E, int64_t K, int64_t N, int dtype) {
+  if (!valid_dtype(dtype) || !is_float_dtype(dtype) || !sizes_ok(B, N, E, K)) return 0;
+  const size_t front = group_workspace_bytes(B, N, K, kElemBytes[dtype]);
+  const size_t bins = group_bins_plan(B, E, K, N, dtype, true, nullptr, 0).bytes;
+  const size_t base = bins > 0 ? bins : front;
+  size_t tail = bins > 0 ? group_tiles_plan(B, E, K, dtype, true, nullptr, 0, bins).bytes : 0;
+  const size_t soft = env_int("TS_GROUP_FUSED", 1) != 0 ? group_fused_scratch_bytes(B, E, K, kElemBytes[dtype]) : 0;
+  if (soft > tail) tail = soft;
+  return base + tail;
 }
 
 size_t ts_group_bins_workspace_bytes(int64_t B, int64_t E, int64_t K, int64_t N, int dtype) {

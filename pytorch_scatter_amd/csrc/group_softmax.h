@@ -99,6 +99,8 @@ struct GroupArgs {
   const int *gate = nullptr;  // the three passes of softmax run only if *gate != 0 (null: always)
   int *flag = nullptr;        // softmax: a word behind the workspace of the three passes, for the one-pass kernels
   size_t ws_bytes = 0;        //          bytes of that workspace (gmax is its start)
+  void *fused_ws = nullptr;     // softmax: scratch for the one-pass tiles beyond the workspace of the three passes (whose
+  size_t fused_ws_bytes = 0;    //          front holds their records only while it is large enough: few, large groups)
   const void *coef = nullptr;   // std / logsumexp backward: [B, N, 2, K] in the accumulate type, what an entry needs of its
                                 // group side by side (group_coef_kernel); null: gathered from the group arrays
   void *total_w = nullptr;      // std through buckets: the group sums [B, N, K] in the element type are written here,

@@ -818,9 +818,8 @@ struct GroupSoftmaxFn : public torch::autograd::Function<GroupSoftmaxFn> {
     src = src.contiguous();
     const GroupLayout l = group_layout(src, index, dim);
     Tensor out = at::empty_like(src);
-    // the larger workspace of the route through buckets of groups, where that route applies
-    Tensor ws = workspace(std::max(ts_group_softmax_workspace_bytes(l.B, N, l.K, dtype_code(src)),
-                                   ts_group_bins_workspace_bytes(l.B, l.E, l.K, N, dtype_code(src))), src);
+    // the workspace that opens every route: three passes, buckets of groups, one-pass tiles
+    Tensor ws = workspace(ts_group_workspace_bytes(l.B, l.E, l.K, N, dtype_code(src)), src);
     check_status(ts_group_softmax(src.data_ptr(), index.data_ptr<int64_t>(), out.data_ptr(), l.B, l.E, l.K, N, l.sb,
                                   l.se, dtype_code(src), log_space ? 1 : 0, eps, ws.data_ptr(),
                                   static_cast<size_t>(ws.numel()), stream_of(src)),
@@ -842,7 +841,7 @@ struct GroupSoftmaxFn : public torch::autograd::Function<GroupSoftmaxFn> {
     const bool log_space = ctx->saved_data["log"].toBool();
     const GroupLayout l = group_layout(out, index, dim);
     Tensor grad_in = at::empty_like(out);
-    Tensor ws = workspace(ts_group_softmax_workspace_bytes(l.B, N, l.K, dtype_code(out)), out);
+    Tensor ws = workspace(ts_group_workspace_bytes(l.B, l.E, l.K, N, dtype_code(out)), out);
     check_status(ts_group_softmax_backward(out.data_ptr(), grad_out.data_ptr(), index.data_ptr<int64_t>(),
                                            grad_in.data_ptr(), l.B, l.E, l.K, N, l.sb, l.se, dtype_code(out),
                                            log_space ? 1 : 0, ws.data_ptr(), static_cast<size_t>(ws.numel()),
@@ -865,8 +864,7 @@ struct GroupLogSumExpFn : public torch::autograd::Function<GroupLogSumExpFn> {
     sizes[dim] = N;
     Tensor out = at::empty(sizes, src.options());
     // the larger workspace of the route through buckets of groups, where that route applies
-    const size_t ws_bytes = std::max(ts_group_softmax_workspace_bytes(l.B, N, l.K, dtype_code(src)),
-                                     ts_group_bins_workspace_bytes(l.B, l.E, l.K, N, dtype_code(src)));
+    const size_t ws_bytes = ts_group_workspace_bytes(l.B, l.E, l.K, N, dtype_code(src));
     Tensor ws = workspace(ws_bytes, src);
     check_status(ts_group_logsumexp(src.data_ptr(), index.data_ptr<int64_t>(), out.data_ptr(), l.B, l.E, l.K, N, l.sb,
                                     l.se, dtype_code(src), eps, ws.data_ptr(), static_cast<size_t>(ws.numel()),

@@ -249,7 +249,29 @@ def test_one_pass_kernels_leave_their_verdict(capi, monkeypatch):
         out = torch.empty_like(src)
         ws = capi.group_softmax(src, index, out, B, E, K, N, 0, 1, False)
         torch.cuda.synchronize()
-        assert int(ws[-256:-252].cpu().view(torch.int32)[0]) == verdict, kind
+        front = capi.lib().ts_group_softmax_workspace_bytes(capi._i(B), capi._i(N), capi._i(K), capi.DTYPE[torch.float32])
+        assert int(ws[front - 256:front - 252].cpu().view(torch.int32)[0]) == verdict, kind
+
+
+def test_one_pass_kernels_take_few_large_groups(capi, oracle, monkeypatch):
+    """Few groups of many entries: the tiles' records do not fit the workspace of the three passes (2 x N x K words) and
+    live in the scratch behind it (ts_group_workspace_bytes). The verdict word says that the tiles took the call."""
+    monkeypatch.setenv("TS_GROUP_FUSED", "2")
+    monkeypatch.setenv("TS_GROUP_BINS", "0")
+    monkeypatch.setenv("TS_GROUP_TILE", "256")
+    rng = np.random.default_rng(8)
+    B, E, K, N = 1, 60_000, 4, 6
+    src = torch.from_numpy(rng.standard_normal(size=(B, E, K)) * 2).float()
+    grad = torch.from_numpy(rng.standard_normal(size=(B, E, K))).float()
+    index1 = torch.from_numpy(np.sort(rng.integers(0, N, size=E)))
+    L = capi.lib()
+    front = L.ts_group_softmax_workspace_bytes(capi._i(B), capi._i(N), capi._i(K), capi.DTYPE[torch.float32])
+    assert L.ts_group_workspace_bytes(capi._i(B), capi._i(E), capi._i(K), capi._i(N), capi.DTYPE[torch.float32]) > front
+    out = torch.empty((B, E, K), device=DEV)
+    ws = capi.group_softmax(src.to(DEV), index1.to(DEV), out, B, E, K, N, 0, 1, False)
+    torch.cuda.synchronize()
+    assert int(ws[front - 256:front - 252].cpu().view(torch.int32)[0]) == 0
+    check_against_oracle(capi, oracle, src, grad, index1, (B, E, K, N), torch.float32)
 
 
 def test_one_pass_kernels_special_values(capi, oracle, monkeypatch):
