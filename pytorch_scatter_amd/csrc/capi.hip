@@ -876,8 +876,8 @@ GroupBinPlan group_bins_plan(int64_t B, int64_t E, int64_t K, int64_t N, int dty
 }
 // std / logsumexp: the one-pass tiles for an index in order, their scratch behind that of the buckets (at ws + skip).
 // TS_GROUP_FUSED (tuning aid): 0 never, 2 at any size and whatever the index looks like.
-FusedReducePlan group_tiles_plan(int64_t B, int64_t E, int64_t K, int dtype, bool aligned, void *ws, size_t ws_bytes,
-                                 size_t skip) {
+FusedReducePlan group_tiles_plan(int64_t B, int64_t E, int64_t K, int64_t N, int dtype, bool aligned, void *ws,
+                                 size_t ws_bytes, size_t skip) {
   const int mode = env_int("TS_GROUP_FUSED", 1);
   if (mode == 0 || skip == 0) {
     FusedReducePlan r;
@@ -885,7 +885,7 @@ FusedReducePlan group_tiles_plan(int64_t B, int64_t E, int64_t K, int dtype, boo
     r.bytes = 0;
     return r;
   }
-  return group_reduce_fused_plan(B, E, K, kElemBytes[dtype], aligned,
+  return group_reduce_fused_plan(B, E, K, N, kElemBytes[dtype], aligned,
                                  ws != nullptr && ws_bytes > skip ? static_cast<char *>(ws) + skip : nullptr,
                                  ws_bytes > skip ? ws_bytes - skip : 0, mode == 2);
 }
@@ -997,7 +997,7 @@ int ts_group_logsumexp(const void *src, const int64_t *index, void *out, int64_t
       g.se = index_stride_e;
       g.eps = eps;
       g.bins = &plan.p;
-      const FusedReducePlan tiles = group_tiles_plan(B, E, K, dtype, aligned16(src), workspace, workspace_bytes, plan.bytes);
+      const FusedReducePlan tiles = group_tiles_plan(B, E, K, N, dtype, aligned16(src), workspace, workspace_bytes, plan.bytes);
       if (tiles.ok) {
         g.tiles = &tiles.f;
         g.tiles_force = env_int("TS_GROUP_FUSED", 1) == 2;
@@ -1027,7 +1027,7 @@ size_t ts_group_workspace_bytes(int64_t B, int64_t E, int64_t K, int64_t N, int 
   const size_t front = group_workspace_bytes(B, N, K, kElemBytes[dtype]);
   const size_t bins = group_bins_plan(B, E, K, N, dtype, true, nullptr, 0).bytes;
   const size_t base = bins > 0 ? bins : front;
-  size_t tail = bins > 0 ? group_tiles_plan(B, E, K, dtype, true, nullptr, 0, bins).bytes : 0;
+  size_t tail = bins > 0 ? group_tiles_plan(B, E, K, N, dtype, true, nullptr, 0, bins).bytes : 0;
   const size_t soft = env_int("TS_GROUP_FUSED", 1) != 0 ? group_fused_scratch_bytes(B, E, K, kElemBytes[dtype]) : 0;
   if (soft > tail) tail = soft;
   return base + tail;
@@ -1036,7 +1036,7 @@ size_t ts_group_workspace_bytes(int64_t B, int64_t E, int64_t K, int64_t N, int 
 size_t ts_group_bins_workspace_bytes(int64_t B, int64_t E, int64_t K, int64_t N, int dtype) {
   if (!valid_dtype(dtype) || !is_float_dtype(dtype) || !sizes_ok(B, N, E, K)) return 0;
   const size_t bins = group_bins_plan(B, E, K, N, dtype, true, nullptr, 0).bytes;
-  return bins + group_tiles_plan(B, E, K, dtype, true, nullptr, 0, bins).bytes;
+  return bins + group_tiles_plan(B, E, K, N, dtype, true, nullptr, 0, bins).bytes;
 }
 
 int ts_group_std_forward(const void *src, const int64_t *index, void *total, int32_t *count, void *out, int64_t B,
@@ -1064,7 +1064,7 @@ int ts_group_std_forward(const void *src, const int64_t *index, void *total, int
   g.sb = index_stride_b;
   g.se = index_stride_e;
   g.bins = &plan.p;
-  const FusedReducePlan tiles = group_tiles_plan(B, E, K, dtype, al, workspace, workspace_bytes, plan.bytes);
+  const FusedReducePlan tiles = group_tiles_plan(B, E, K, N, dtype, al, workspace, workspace_bytes, plan.bytes);
   if (tiles.ok) {
     g.tiles = &tiles.f;
     g.tiles_force = env_int("TS_GROUP_FUSED", 1) == 2;

@@ -14,6 +14,9 @@
 
 namespace ts {
 
+constexpr int kReduceRowBytes = 256;  // widest row of these tiles
+constexpr int kReduceVecsWide = 16;   // 16-byte units per lane of a tile of such rows
+
 struct FusedReduceArgs {
   int te;            // entries per tile: kBlock * epl
   int epl;           // neighbouring entries per lane when the runs are found
@@ -33,22 +36,26 @@ struct FusedReducePlan {
   FusedReduceArgs f;
 };
 
-// rows of up to 128 bytes, from 16 MB of input (the launches that return at once under any other index)
-inline FusedReducePlan group_reduce_fused_plan(int64_t B, int64_t E, int64_t K, int elem_bytes, bool aligned, void *ws,
-                                               size_t ws_bytes, bool force) {
+// rows of up to 256 bytes, from 16 MB of input (the launches that return at once under any other index)
+inline FusedReducePlan group_reduce_fused_plan(int64_t B, int64_t E, int64_t K, int64_t N, int elem_bytes, bool aligned,
+                                               void *ws, size_t ws_bytes, bool force) {
   FusedReducePlan r;
   r.ok = false;
   r.bytes = 0;
   const int64_t row = K * elem_bytes;
-  if (row > kFusedRowBytes || E < 2 || !aligned) return r;
+  if (row > kReduceRowBytes || E < 2 || !aligned) return r;
   if (B > 1 && (E * row) % 16 != 0) return r;
   if (!force && B * E * row < ((int64_t)16 << 20)) return r;
-  int64_t te = 32768 / row;
+  // rows of more than 128 bytes (256 entries per tile): not for few groups of many entries, whose runs all cross several
+  // tiles (4 M entries of 64 floats in 4 k groups: std 1034 us, 628 us through the buckets behind)
+  if (!force && row > kFusedRowBytes && E > 64 * N) return r;
+  int64_t te = 32768 / row;  // 32 KB of rows per tile; rows of more than 128 bytes: 256 entries, 64 KB
+  if (te < kBlock) te = kBlock;
   if (const char *env = getenv("TS_GROUP_TILE")) te = atoi(env);  // tuning aid
   int epl = 1;
   while (epl * 2 * kBlock <= te && epl * 2 <= kFusedPer) epl *= 2;
   te = (int64_t)epl * kBlock;
-  if (te * row > (int64_t)kFusedVecs * kBlock * 16) return r;
+  if (te * row > (int64_t)kReduceVecsWide * kBlock * 16) return r;
   FusedReduceArgs &f = r.f;
   f.te = (int)te;
   f.epl = epl;
@@ -86,8 +93,9 @@ __global__ __launch_bounds__(kBlock) void group_reduce_fill_kernel(GroupArgs g, 
   }
 }
 
-template <typename T, int CV, int MODE>
-__global__ __launch_bounds__(kBlock, 4) void group_reduce_fused_kernel(GroupArgs g, FusedReduceArgs f) {
+// NV: 16-byte units of the tile per lane (8: 32 KB of rows, four workgroups per CU; 16: rows of up to 256 bytes, 64 KB)
+template <typename T, int CV, int MODE, int NV>
+__global__ __launch_bounds__(kBlock, NV > 8 ? 2 : 4) void group_reduce_fused_kernel(GroupArgs g, FusedReduceArgs f) {
   typedef typename Acc<T>::type F;
   typedef GroupBinPart<T, MODE> Part;
   typedef uint32_t u4 __attribute__((ext_vector_type(4)));
@@ -109,11 +117,11 @@ __global__ __launch_bounds__(kBlock, 4) void group_reduce_fused_kernel(GroupArgs
 
   // ---- the tile of src: whole 16-byte units, every load of the tile and of the index in flight together
   const int nvec = (int)(((size_t)ne * K * sizeof(T) + 15) / 16);
-  u4 stage[kFusedVecs];
+  u4 stage[NV];
   {
     const u4 *p0 = reinterpret_cast<const u4 *>(static_cast<const T *>(g.src) + (b * g.E + j0) * K);
 #pragma unroll
-    for (int q = 0; q < kFusedVecs; ++q) {
+    for (int q = 0; q < NV; ++q) {
       const int v = tid + q * kBlock;
       if (v < f.tile_vecs && v < nvec) stage[q] = __builtin_nontemporal_load(p0 + v);
     }
@@ -125,7 +133,7 @@ __global__ __launch_bounds__(kBlock, 4) void group_reduce_fused_kernel(GroupArgs
   bool descent = false, lane_enters = false, lane_leaves = false;
   auto stage_to_lds = [&]() {
 #pragma unroll
-    for (int q = 0; q < kFusedVecs; ++q) {
+    for (int q = 0; q < NV; ++q) {
       const int v = tid + q * kBlock;
       if (v < f.tile_vecs && v < nvec) s_dyn[v] = stage[q];
     }
@@ -362,7 +370,14 @@ int launch_group_reduce_fused(const GroupArgs &g, const FusedReduceArgs &f, bool
                      f.flag);
   const size_t lds = (size_t)f.tile_vecs * 16 + ((size_t)f.te + 2) * 2;
   const unsigned tiles = (unsigned)(g.B * f.nt);
-  hipLaunchKernelGGL((group_reduce_fused_kernel<T, CV, MODE>), dim3(tiles), dim3(kBlock), lds, stream, g, f);
+  if ((int64_t)f.tile_vecs > (int64_t)kFusedVecs * kBlock) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void *>(&group_reduce_fused_kernel<T, CV, MODE, kReduceVecsWide>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+      return TS_ERR_LAUNCH;
+    hipLaunchKernelGGL((group_reduce_fused_kernel<T, CV, MODE, kReduceVecsWide>), dim3(tiles), dim3(kBlock), lds, stream, g, f);
+  } else {
+    hipLaunchKernelGGL((group_reduce_fused_kernel<T, CV, MODE, kFusedVecs>), dim3(tiles), dim3(kBlock), lds, stream, g, f);
+  }
   int G = 1;
   while (G < g.K && G < kWave) G *= 2;
   hipLaunchKernelGGL((group_reduce_fragment_kernel<T, MODE>), dim3(tiles), dim3(kWave), 0, stream, g, f, G);

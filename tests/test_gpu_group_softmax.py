@@ -184,7 +184,8 @@ def test_one_pass_kernels_capi(capi, oracle, monkeypatch, shape, kind, dtype, ti
     check_against_oracle(capi, oracle, src, grad, fused_index(kind, rng, E, N), shape, dtype)
 
 @pytest.mark.parametrize("shape,kind,dtype",
-                         product(FUSED_SHAPES + [(1, 40_000, 8, 3000)], ["sorted", "skewed", "outside", "one_descent"], DTYPES))
+                         product(FUSED_SHAPES + [(1, 40_000, 8, 3000), (1, 1200, 64, 30), (2, 700, 48, 9)],
+                                 ["sorted", "skewed", "outside", "one_descent"], DTYPES))
 @pytest.mark.parametrize("tile", [256, 0])
 def test_std_and_logsumexp_one_pass_tiles_capi(capi, oracle, monkeypatch, shape, kind, dtype, tile):
     """scatter_std / scatter_logsumexp forward through the one-pass tiles for an index in order
