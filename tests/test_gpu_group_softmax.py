@@ -797,3 +797,43 @@ def test_std_operator_reference_case_script_and_fallback(ts, oracle):
     # zero-size input
     assert ts.scatter_std(torch.empty(0, 4, device=DEV), torch.empty(0, dtype=torch.long, device=DEV), 0,
                           dim_size=3).shape == (3, 4)
+
+
+@pytest.mark.parametrize("kind", ["sorted", "random"])
+def test_group_operators_under_graph_replay(ts, kind):
+    """scatter_std, scatter_logsumexp and scatter_softmax at a size that takes the one-pass tiles (sorted) or the
+    buckets of groups (random), captured in a graph and replayed three times with fresh inputs and eager work in
+    between: every replay equals the eager call on the same inputs (the passes clear their own counters with kernels,
+    the verdict word of the tiles is rewritten by every call)."""
+    E, N, K = 700_000, 90_000, 8
+    g = torch.Generator().manual_seed(13)
+    index = torch.randint(0, N, (E,), generator=g)
+    if kind == "sorted":
+        index = index.sort().values
+    index = index.to(DEV)
+    static_src = torch.zeros((E, K), device=DEV)
+
+    def step():
+        return (ts.scatter_std(static_src, index, 0, None, N), ts.scatter_logsumexp(static_src, index, 0, None, N),
+                ts.scatter_softmax(static_src, index, 0, N))
+
+    with torch.no_grad():
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(2):
+                step()  # warm-up on a side stream
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            outs = step()
+        for rep in range(3):
+            static_src.copy_(torch.randn((E, K), generator=g).to(DEV))
+            graph.replay()
+            torch.cuda.synchronize()
+            got = [o.clone() for o in outs]
+            eager = step()
+            torch.cuda.synchronize()
+            for a, b in zip(got, eager):
+                assert torch.allclose(a, b, rtol=1e-5, atol=1e-6), (rep, float((a - b).abs().max()))
