@@ -24,6 +24,8 @@ struct FusedReduceArgs {
   int short_run;     // runs of more entries than this inside a tile take eight lanes,
   int long_run;      // of more than this a wavefront
   int64_t nt;        // tiles per batch
+  int kcols;         // columns of a row that a workgroup takes: K, or a slice of 256 bytes of a wider row (then
+  int slices;        // K / kcols workgroups share a tile of entries, each on its own columns)
   int32_t *meta;     // [B * nt][4]: entries of the entering run, first entry of the leaving run, entries, tile is one run that enters and leaves
   uint64_t *pa;      // [B * nt][2][K] partials of the entering / leaving run: GroupBinPart::a
   double *pb;        //                                                        GroupBinPart::b
@@ -36,16 +38,21 @@ struct FusedReducePlan {
   FusedReduceArgs f;
 };
 
-// rows of up to 256 bytes, from 16 MB of input (the launches that return at once under any other index)
+// rows of up to 256 bytes, or of a whole number of 256-byte column slices; from 16 MB of input (the launches that
+// return at once under any other index)
 inline FusedReducePlan group_reduce_fused_plan(int64_t B, int64_t E, int64_t K, int64_t N, int elem_bytes, bool aligned,
                                                void *ws, size_t ws_bytes, bool force) {
   FusedReducePlan r;
   r.ok = false;
   r.bytes = 0;
-  const int64_t row = K * elem_bytes;
-  if (row > kReduceRowBytes || E < 2 || !aligned) return r;
-  if (B > 1 && (E * row) % 16 != 0) return r;
-  if (!force && B * E * row < ((int64_t)16 << 20)) return r;
+  const int64_t row_all = K * elem_bytes;
+  // rows of more than 256 bytes in column slices of 256 bytes (a whole number of them)
+  const int64_t slices = row_all > kReduceRowBytes ? row_all / kReduceRowBytes : 1;
+  if (slices * kReduceRowBytes != row_all && slices > 1) return r;
+  const int64_t row = row_all / slices;
+  if (E < 2 || !aligned) return r;
+  if (B > 1 && (E * row_all) % 16 != 0) return r;
+  if (!force && B * E * row_all < ((int64_t)16 << 20)) return r;
   // rows of more than 128 bytes (256 entries per tile): not for few groups of many entries, whose runs all cross several
   // tiles (4 M entries of 64 floats in 4 k groups: std 1034 us, 628 us through the buckets behind)
   if (!force && row > kFusedRowBytes && E > 64 * N) return r;
@@ -62,7 +69,9 @@ inline FusedReducePlan group_reduce_fused_plan(int64_t B, int64_t E, int64_t K, 
   f.short_run = kFusedShortRun;
   f.long_run = kFusedGroup * kFusedShortRun;
   f.nt = (E + te - 1) / te;
-  if (B * f.nt >= 0x7FFFFFFFll) return r;
+  f.slices = (int)slices;
+  f.kcols = (int)(K / slices);
+  if (B * f.nt >= 0x7FFFFFFFll || slices > 65535) return r;
   f.tile_vecs = (int)((te * row + 15) / 16);
   auto up = [](size_t x) { return (x + 255) & ~(size_t)255; };
   const size_t tiles = (size_t)(B * f.nt);
@@ -108,7 +117,9 @@ __global__ __launch_bounds__(kBlock, NV > 8 ? 2 : 4) void group_reduce_fused_ker
   const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
   if (tid < 6) s_info[tid] = 0;
   __syncthreads();
-  const int K = (int)g.K;
+  const int K = f.kcols;                       // columns of this workgroup, row pitch of the staged tile
+  const int64_t KR = g.K;                      // columns of a row in memory
+  const int k_first = (int)blockIdx.y * K;     // first column of this workgroup's slice
   const int64_t b = blockIdx.x / f.nt, t = blockIdx.x - b * f.nt;
   const int64_t j0 = t * f.te;
   const int ne = (int)(g.E - j0 < f.te ? g.E - j0 : f.te);
@@ -119,11 +130,20 @@ __global__ __launch_bounds__(kBlock, NV > 8 ? 2 : 4) void group_reduce_fused_ker
   const int nvec = (int)(((size_t)ne * K * sizeof(T) + 15) / 16);
   u4 stage[NV];
   {
-    const u4 *p0 = reinterpret_cast<const u4 *>(static_cast<const T *>(g.src) + (b * g.E + j0) * K);
+    const T *tile0 = static_cast<const T *>(g.src) + (b * g.E + j0) * KR + k_first;
+    const u4 *p0 = reinterpret_cast<const u4 *>(tile0);
+    const int vps = K * (int)sizeof(T) / 16;  // (slices: 16-byte units of an entry's slice, a power of two)
 #pragma unroll
     for (int q = 0; q < NV; ++q) {
       const int v = tid + q * kBlock;
-      if (v < f.tile_vecs && v < nvec) stage[q] = __builtin_nontemporal_load(p0 + v);
+      if (v < f.tile_vecs && v < nvec) {
+        if (f.slices == 1) {
+          stage[q] = __builtin_nontemporal_load(p0 + v);  // the tile is one range of memory
+        } else {
+          const int ev = v / vps;
+          stage[q] = __builtin_nontemporal_load(reinterpret_cast<const u4 *>(tile0 + (int64_t)ev * KR) + (v - ev * vps));
+        }
+      }
     }
   }
   const int64_t *idx = g.index + b * g.sb;
@@ -248,7 +268,7 @@ __global__ __launch_bounds__(kBlock, NV > 8 ? 2 : 4) void group_reduce_fused_ker
     }
     if (first != 0) return;
     if (!single) {
-      const int64_t slot = (tile * 2 + (frag_in ? 0 : 1)) * K + c0;
+      const int64_t slot = (tile * 2 + (frag_in ? 0 : 1)) * KR + k_first + c0;
 #pragma unroll
       for (int v = 0; v < CV; ++v) {
         f.pa[slot + v] = part[v].a;
@@ -259,7 +279,7 @@ __global__ __launch_bounds__(kBlock, NV > 8 ? 2 : 4) void group_reduce_fused_ker
     if ((s_start[r] >> 15) != 0) return;  // a run that belongs to no group
     const int64_t row = b * g.N + idx[(j0 + lo) * g.se];
 #pragma unroll
-    for (int v = 0; v < CV; ++v) group_bin_emit<T, MODE>(g, row * K + c0 + v, row, c0 + v, part[v]);
+    for (int v = 0; v < CV; ++v) group_bin_emit<T, MODE>(g, row * KR + k_first + c0 + v, row, k_first + c0 + v, part[v]);
   };
 
   // one lane per (run, columns) for short runs, eight lanes or a wavefront for longer ones
@@ -292,7 +312,7 @@ __global__ __launch_bounds__(kBlock, NV > 8 ? 2 : 4) void group_reduce_fused_ker
     const int r = s_long[kFusedMaxTile / 4 + 1 - q];
     for (int c = 0; c < kc; ++c) run_stat(r, c * CV, lane, kWave);
   }
-  if (tid == 0) {
+  if (tid == 0 && blockIdx.y == 0) {
     const int w_lo = enters ? (s_start[1] & 0x7FFF) : 0;  // nruns == 1: s_start[1] == ne
     const int w_hi = leaves ? (s_start[nruns - 1] & 0x7FFF) : ne;
     const bool one = nruns == 1 && enters && leaves;
@@ -374,9 +394,9 @@ int launch_group_reduce_fused(const GroupArgs &g, const FusedReduceArgs &f, bool
     if (hipFuncSetAttribute(reinterpret_cast<const void *>(&group_reduce_fused_kernel<T, CV, MODE, kReduceVecsWide>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
       return TS_ERR_LAUNCH;
-    hipLaunchKernelGGL((group_reduce_fused_kernel<T, CV, MODE, kReduceVecsWide>), dim3(tiles), dim3(kBlock), lds, stream, g, f);
+    hipLaunchKernelGGL((group_reduce_fused_kernel<T, CV, MODE, kReduceVecsWide>), dim3(tiles, (unsigned)f.slices), dim3(kBlock), lds, stream, g, f);
   } else {
-    hipLaunchKernelGGL((group_reduce_fused_kernel<T, CV, MODE, kFusedVecs>), dim3(tiles), dim3(kBlock), lds, stream, g, f);
+    hipLaunchKernelGGL((group_reduce_fused_kernel<T, CV, MODE, kFusedVecs>), dim3(tiles, (unsigned)f.slices), dim3(kBlock), lds, stream, g, f);
   }
   int G = 1;
   while (G < g.K && G < kWave) G *= 2;
