@@ -938,8 +938,11 @@ int run_group_softmax(const void *src, const void *grad, const int64_t *index, v
     plan = group_bins_plan(B, E, K, N, dtype, al, workspace, workspace_bytes);
     // (rows of up to 128 bytes, where the one-pass tiles take an index in order: for wider rows the three passes are
     // ahead under a sorted index, 1 M x 128 floats 570 against 741 us, and behind under a random one, 663 against 449)
-    if (plan.ok && group_bins_vec(K, dtype, al) == vec &&
-        (K * kElemBytes[dtype] <= kFusedRowBytes || env_int("TS_GROUP_BINS", 1) == 2))
+    // (nor for few groups of many entries in rows of more than 64 bytes, which the tiles decline as well: 4 M x 64 bf16
+    // in 4 k groups, sorted, 890 against 1116 us)
+    const int64_t row_bytes = K * kElemBytes[dtype];
+    const bool tiles_cover = row_bytes <= 64 || (row_bytes <= kFusedRowBytes && E <= 64 * N);
+    if (plan.ok && group_bins_vec(K, dtype, al) == vec && (tiles_cover || env_int("TS_GROUP_BINS", 1) == 2))
       g.bins = &plan.p;
   }
   // a workspace of ts_group_workspace_bytes(): what lies behind the three passes' (and the buckets') part is scratch
