@@ -25,7 +25,8 @@ constexpr int kGroupBinRows = 2048;   // groups per bucket at most
 constexpr int kGroupBinSlots = 8192;  // groups x columns of a bucket at most (the slab of a chunk: 16 bytes per slot)
 constexpr int kGroupBinLong = 64;     // entries of a group inside a chunk from which on a wavefront takes the group
 constexpr int kGroupBinCoop = 2;      // up to this many long groups in a chunk, the whole workgroup takes them one by one
-constexpr int kGroupBinCoopLanes = 8;  // and held by at least this many lanes (few entries per step of one wavefront)
+constexpr int kGroupBinCoopLanes = 8;  // and held by at least this many lanes (few entries per step of one wavefront),
+constexpr int kGroupBinCoopEntries = 2048;  // or a group of at least this many entries
 constexpr int kGroupBinCoopCols = 64;  // ... for rows of up to this many columns
 constexpr int kGroupBinMaxLong = 128;  // such groups per chunk at most (a chunk holds at most 8192 entries)
 constexpr int kGroupBinMaxLanes = 32;  // lanes per entry at most (a chunk then holds 256 entries)
@@ -438,7 +439,15 @@ __global__ __launch_bounds__(kBinBlock) void group_bin_kernel(GroupArgs g, BinAr
     // (a lane group that has no item still takes part in the butterflies of its wavefront)
     stat(r, (i - r * lanes) * VEC, mine ? slane : 0x7FFFFFF0, share, share / 2, 1, false);
   }
-  if (nlong > 0 && nlong <= kGroupBinCoop && K <= kGroupBinCoopCols && lanes >= kGroupBinCoopLanes) {
+  // (rows held by few lanes: only for a group of kGroupBinCoopEntries entries and more, where one wavefront would need
+  // tens of rounds; below that the barriers of the meeting cost more)
+  bool coop = nlong > 0 && nlong <= kGroupBinCoop && K <= kGroupBinCoopCols;
+  if (coop && lanes < kGroupBinCoopLanes) {
+    int most = 0;
+    for (int q = 0; q < nlong; ++q) most = s_n[s_long[q]] > most ? s_n[s_long[q]] : most;
+    coop = most >= kGroupBinCoopEntries;
+  }
+  if (coop) {
     for (int q = 0; q < nlong; ++q) stat(s_long[q], col, wave * epw + sub, W * epw, kWave / 2, lanes, true);
   } else {
     for (int q = wave; q < nlong; q += W) stat(s_long[q], col, sub, epw, kWave / 2, lanes, false);
