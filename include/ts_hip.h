@@ -262,8 +262,10 @@ enum ts_scatter_route {
   TS_ROUTE_MINMAX_BUCKETS = 15,          /* workspace: entries binned by bucket of output rows */
   TS_ROUTE_MINMAX_BUCKETS_OR_SEGMENTED = 16, /* the same; an index found sorted: the segmented reduction */
   TS_ROUTE_MINMAX_64BIT = 17,            /* 64-bit elements: value pass, then position pass */
-  TS_ROUTE_SUM_VALUE_BUCKETS = 18        /* workspace, one 4-byte value per entry: the values travel in the binned words;
+  TS_ROUTE_SUM_VALUE_BUCKETS = 18,       /* workspace, one 4-byte value per entry: the values travel in the binned words;
                                             a sample of the index picks buckets (even), table (skewed) or runs (sorted) */
+  TS_ROUTE_SUM_COUNT_RUNS = 19           /* ts_scatter_sum_count_with_workspace below 2^16 elements: runs, the entries per
+                                            output row counted by the same launch */
 };
 /* Self-test of the fixed-pattern cross-lane helpers the kernels use (DPP row shifts, wave_shr:1,
  * v_permlane16_swap / v_permlane32_swap: csrc/dpp.h): one wavefront applies each helper to x = 3 * lane + 1 and
@@ -296,7 +298,9 @@ int ts_scatter_count_with_workspace(const int64_t *index, int32_t *count, int64_
  * ts_scatter_with_workspace(reduce = sum, index_stride_k = 0) leaves it, count as ts_scatter_count leaves it. When
  * the sum goes through buckets of output rows (ts_scatter_sum_count_workspace_bytes() of scratch: wide rows from
  * 64 MB, single 4-byte values from 2 M entries) the index is read and binned once for both: the adding pass keeps
- * a table of counts beside its sums. Every other case is the two calls in a row. */
+ * a table of counts beside its sums. Where the sum is one launch (runs below 2^16 elements, the table in LDS above,
+ * see ts_scatter_route) that launch counts too, and one launch clears out and count. Every other case is the two
+ * calls in a row. */
 size_t ts_scatter_sum_count_workspace_bytes(int64_t B, int64_t E, int64_t K, int64_t N, int dtype);
 int ts_scatter_sum_count_with_workspace(const void *src, const int64_t *index, void *out,
                                         int32_t *count, int64_t B, int64_t E, int64_t K, int64_t N,

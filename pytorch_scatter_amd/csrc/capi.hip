@@ -291,7 +291,8 @@ const char *ts_scatter_route_name(int route) {
       "sum: buckets or segmented reduction (index checked)", "mul: atomic", "mul: table", "min/max: atomic",
       "min/max: runs", "min/max: runs or table (sample)", "min/max: table", "min/max: table, one value per entry",
       "min/max: slabs, one value per entry", "min/max: buckets", "min/max: buckets or segmented reduction (index checked)",
-      "min/max: 64-bit elements, two passes", "sum: single values in buckets, table or runs (sample)"};
+      "min/max: 64-bit elements, two passes", "sum: single values in buckets, table or runs (sample)",
+      "sum: runs, entries per row counted by the same launch"};
   return route >= 0 && route < (int)(sizeof(names) / sizeof(names[0])) ? names[route] : "unknown";
 }
 
@@ -602,7 +603,8 @@ namespace {
 int scatter_ws_impl(const void *src, const int64_t *index, void *out, int64_t *arg_out, int64_t B,
                     int64_t E, int64_t K, int64_t N, int64_t index_stride_b, int64_t index_stride_e,
                     int64_t index_stride_k, int dtype, int reduce, int out_given, void *workspace,
-                    size_t workspace_bytes, ts_stream_t stream, int32_t *count_out, const int **count_flag) {
+                    size_t workspace_bytes, ts_stream_t stream, int32_t *count_out, const int **count_flag,
+                    int *count_done = nullptr) {
   if (!valid_dtype(dtype) || !sizes_ok(B, N, E, K)) return TS_ERR_BAD_ARG;
   if (reduce != TS_SUM && reduce != TS_MUL && reduce != TS_MIN && reduce != TS_MAX) return TS_ERR_UNSUPPORTED;
   if (B * N * K == 0) return TS_OK;
@@ -623,6 +625,7 @@ int scatter_ws_impl(const void *src, const int64_t *index, void *out, int64_t *a
   a.out_given = out_given ? 1 : 0;
   a.count_out = count_out;
   a.count_flag = count_flag;
+  a.count_done = count_done;
   a.precheck = env_int("TS_SCATTER_PRECHECK", 1);   // tuning aids
   a.lds_cache = env_int("TS_SCATTER_LDS", 1);
   a.lds_epb = env_int("TS_SCATTER_EPB", 0);
@@ -790,10 +793,11 @@ int ts_scatter_sum_count_with_workspace(const void *src, const int64_t *index, v
   }
   if (may_fuse)
     hipLaunchKernelGGL(fill_kernel<int32_t>, dim3(grid_for(B * N)), dim3(kBlock), 0, s, count, B * N, (int32_t)0);
+  // (a small sum clears and counts by itself, in the launches that clear out and add: then `counted` reads 1)
+  int counted = 0;
   const int rc = scatter_ws_impl(src, index, out, nullptr, B, E, K, N, index_stride_b, index_stride_e, 0, dtype, TS_SUM,
-                                 out_given, workspace, workspace_bytes, stream, may_fuse ? count : nullptr,
-                                 may_fuse ? &flag : nullptr);
-  if (rc != TS_OK) return rc;
+                                 out_given, workspace, workspace_bytes, stream, count, may_fuse ? &flag : nullptr, &counted);
+  if (rc != TS_OK || counted) return rc;
   if (flag == nullptr)  // another route: the count on its own (with its own fill)
     return ts_scatter_count_with_workspace(index, count, B, E, N, index_stride_b, index_stride_e, workspace, workspace_bytes,
                                            stream);

@@ -240,6 +240,8 @@ struct ScatterArgs {
                                    // zeroed [B * N] array ...
   const int **count_flag = nullptr;  // ... and leave the buckets' flag here (still null afterwards: the call took another
                                    // route and nothing was counted)
+  int *count_done = nullptr;       // (host) a small sum counts into count_out (not zeroed by the caller) in the launch that
+                                   // adds (scatter_add_count_run_kernel) and sets this to 1: the counts are complete
   int *order_ws = nullptr;         // sum of narrow rows: a word of scratch for the sample of the index that picks the kernel
   int skew_probe = 1;              // min/max: sample the index for skew (needs 256 bytes of workspace): 0 never, 2 at any size
   const int *skew_flag = nullptr;  // min/max kernels behind the probe: run only if (*skew_flag != 0) == (skew_want != 0)
@@ -422,9 +424,10 @@ __global__ __launch_bounds__(kBlock) void scatter_add_pk16_kernel(ScatterArgs a)
 //   emit(node, col, x)         combine EW columns x[0..EW) into the output slot with one atomic
 //   begin_row(heads, entries)  called once per wavefront row of more than one entry, before the
 //                              emissions of its finished runs: number of runs and of entries in it
+// (bx, by: the workgroup's place in the grid of this reduction, blockIdx for a kernel that holds nothing else)
 template <typename P>
 __device__ __forceinline__ void run_reduce_wave(const ScatterArgs &a, const int lshift, const int rows_per_wave,
-                                                P &p, typename P::A *stage) {
+                                                P &p, typename P::A *stage, const unsigned bx, const unsigned by) {
   typedef typename P::A A;
   constexpr int U = P::U;
   constexpr int C = P::C;
@@ -436,11 +439,11 @@ __device__ __forceinline__ void run_reduce_wave(const ScatterArgs &a, const int 
   const int epr = kWave >> lshift; // entries per wavefront row
   const int el = lane >> lshift;
   const int cl = lane & (L - 1);
-  const int64_t colbase = (int64_t)blockIdx.y * (L * C);
+  const int64_t colbase = (int64_t)by * (L * C);
   const int64_t col = colbase + cl * C;
   const bool col_ok = col < a.K;
   const int64_t n_edges = a.B * a.E;
-  const int64_t wave = (int64_t)blockIdx.x * (kBlock / kWave) + (threadIdx.x / kWave);
+  const int64_t wave = (int64_t)bx * (kBlock / kWave) + (threadIdx.x / kWave);
   const int64_t lo = wave * rows_per_wave * epr;
   int64_t hi = lo + (int64_t)rows_per_wave * epr;
   if (hi > n_edges) hi = n_edges;
@@ -548,7 +551,7 @@ __device__ __forceinline__ void run_reduce_wave(const ScatterArgs &a, const int 
 // one extra atomic.
 template <typename P>
 __device__ __forceinline__ void run_serial_wave(const ScatterArgs &a, const int lshift, const int rows_per_wave,
-                                                P &p, typename P::A *stage) {
+                                                P &p, typename P::A *stage, const unsigned bx, const unsigned by) {
   typedef typename P::A A;
   constexpr int U = P::U;
   constexpr int C = P::C;
@@ -559,11 +562,11 @@ __device__ __forceinline__ void run_serial_wave(const ScatterArgs &a, const int 
   const int epr = kWave >> lshift;  // entry slots of the wavefront
   const int el = lane >> lshift;
   const int cl = lane & (L - 1);
-  const int64_t colbase = (int64_t)blockIdx.y * (L * C);
+  const int64_t colbase = (int64_t)by * (L * C);
   const int64_t col = colbase + cl * C;
   const bool col_ok = col < a.K;
   const int64_t n_edges = a.B * a.E;
-  const int64_t wave = (int64_t)blockIdx.x * (kBlock / kWave) + (threadIdx.x / kWave);
+  const int64_t wave = (int64_t)bx * (kBlock / kWave) + (threadIdx.x / kWave);
   const int64_t lo = wave * rows_per_wave * epr;
   int64_t hi = lo + (int64_t)rows_per_wave * epr;
   if (hi > n_edges) hi = n_edges;
@@ -642,11 +645,16 @@ __host__ __device__ inline bool run_is_serial(int lshift, int lane_bytes) { retu
 // were 3 us slower, whichever branch they took)
 template <bool SERIAL, typename P>
 __device__ __forceinline__ void run_wave(const ScatterArgs &a, const int lshift, const int rows_per_wave, P &p,
-                                         typename P::A *stage) {
+                                         typename P::A *stage, const unsigned bx, const unsigned by) {
   if constexpr (SERIAL)
-    run_serial_wave(a, lshift, rows_per_wave, p, stage);
+    run_serial_wave(a, lshift, rows_per_wave, p, stage, bx, by);
   else
-    run_reduce_wave(a, lshift, rows_per_wave, p, stage);
+    run_reduce_wave(a, lshift, rows_per_wave, p, stage, bx, by);
+}
+template <bool SERIAL, typename P>
+__device__ __forceinline__ void run_wave(const ScatterArgs &a, const int lshift, const int rows_per_wave, P &p,
+                                         typename P::A *stage) {
+  run_wave<SERIAL>(a, lshift, rows_per_wave, p, stage, blockIdx.x, blockIdx.y);
 }
 
 // ---- hot rows of a workgroup ------------------------------------------------------
@@ -861,6 +869,44 @@ __global__ __launch_bounds__(kBlock) void scatter_add_run_kernel(ScatterArgs a, 
   }
 }
 
+
+// scatter mean of a small input, where the launches are the cost (five of 3 us each: out cleared, sum, counts
+// cleared, count, divide): one launch clears out and the counts, one launch adds and counts -- the first sum_blocks
+// workgroups along x are the grid of scatter_add_run_kernel, the workgroups behind them (first column chunk only) that
+// of the count, a sum of ones into int32 through the same run reduction.
+template <typename T>
+__global__ __launch_bounds__(kBlock) void fill_out_count_kernel(T *out, int64_t n_out, int32_t *count, int64_t n_count) {
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n_out + n_count; i += (int64_t)gridDim.x * kBlock) {
+    if (i < n_out)
+      out[i] = small_const<T>(0);
+    else
+      count[i - n_out] = 0;
+  }
+}
+template <typename T, int C, int EW, bool SERIAL>
+__global__ __launch_bounds__(kBlock) void scatter_add_count_run_kernel(ScatterArgs a, int lshift, int rows_per_wave,
+                                                                       ScatterArgs cnt, int count_rows_per_wave,
+                                                                       unsigned sum_blocks) {
+  typedef typename Acc<T>::type A;
+  __shared__ A s_stage[kBlock / kWave][kWave * C];
+  if (blockIdx.x < sum_blocks) {
+    AddRun<T, C, EW, false> p;
+    p.src = static_cast<const T *>(a.src);
+    p.out = static_cast<T *>(a.out);
+    p.out_end = p.out + a.B * a.N * a.K;
+    p.K = a.K;
+    run_wave<SERIAL>(a, lshift, rows_per_wave, p, s_stage[threadIdx.x / kWave], blockIdx.x, blockIdx.y);
+  } else if (blockIdx.y == 0) {
+    AddRun<int32_t, 1, 1, false> q;
+    q.src = nullptr;  // adds 1 per entry
+    q.out = static_cast<int32_t *>(cnt.out);
+    q.out_end = q.out + cnt.B * cnt.N;
+    q.K = 1;
+    // (one column per lane and atomic: the staging buffer is not used)
+    run_reduce_wave(cnt, 0, count_rows_per_wave, q, static_cast<typename AddRun<int32_t, 1, 1, false>::A *>(nullptr),
+                    blockIdx.x - sum_blocks, 0u);
+  }
+}
 
 // rows of a wavefront in the kernel above: long enough to carry runs across rows, short enough to
 // leave ~8 K wavefronts
@@ -1410,7 +1456,9 @@ template <typename L> __device__ __forceinline__ void lds_slot_mul(L *slot, L v)
 // hardware atomic at all, so every entry that reaches memory is a compare-and-swap loop whose time grows with
 // the square of the entries that meet in one element (1 M entries of 8 floats, 30 % of them on one row: 89 ms
 // through scatter_atomic_kernel); here a row's entries meet in LDS and memory sees one factor per row and workgroup.
-template <typename T, bool MUL = false>
+// COUNT = true (sums): the entries of every output row are counted as well, into the zeroed int32 array a.count_out
+// (scatter mean), in a table of their own beside the sums; the lane that holds an entry's first column counts it.
+template <typename T, bool MUL = false, bool COUNT = false>
 __global__ __launch_bounds__(kLdsAddBlock) void scatter_add_lds_kernel(ScatterArgs a, int tn_mask, int64_t epb) {
   constexpr int U = 4;
   if (a.skip_flag != nullptr && a.skip_want >= 0) {
@@ -1424,10 +1472,14 @@ __global__ __launch_bounds__(kLdsAddBlock) void scatter_add_lds_kernel(ScatterAr
   typedef typename TableSlot<T>::type LdsAcc;
   __shared__ LdsAcc s_acc[kLdsAcc];
   __shared__ int32_t s_tags[kLdsAccRows];
+  __shared__ int32_t s_cnt[COUNT ? kLdsAccRows : 1];
   const int K = (int)a.K;
   const int tn = tn_mask + 1;
   for (int i = threadIdx.x; i < tn * K; i += kLdsAddBlock) s_acc[i] = (LdsAcc)(MUL ? 1 : 0);
   for (int i = threadIdx.x; i < tn; i += kLdsAddBlock) s_tags[i] = -1;
+  if constexpr (COUNT) {
+    for (int i = threadIdx.x; i < tn; i += kLdsAddBlock) s_cnt[i] = 0;
+  }
   __syncthreads();
 
   const T *src = static_cast<const T *>(a.src);
@@ -1461,6 +1513,9 @@ __global__ __launch_bounds__(kLdsAddBlock) void scatter_add_lds_kernel(ScatterAr
             const int old = atomicCAS(&s_tags[row], -1, node);
             tag = old == -1 ? node : old;
           }
+          if constexpr (COUNT) {
+            if (k == 0) atomicAdd(tag == node ? &s_cnt[row] : a.count_out + node, 1);
+          }
           if (MUL) {
             if (tag == node) {
               lds_slot_mul<LdsAcc>(&s_acc[row * K + k], (LdsAcc)x[u]);
@@ -1478,6 +1533,12 @@ __global__ __launch_bounds__(kLdsAddBlock) void scatter_add_lds_kernel(ScatterAr
     }
   }
   __syncthreads();
+  if constexpr (COUNT) {
+    for (int i = threadIdx.x; i < tn; i += kLdsAddBlock) {
+      const int32_t c = s_cnt[i];
+      if (c != 0) atomicAdd(a.count_out + s_tags[i], c);
+    }
+  }
   if constexpr (MUL) {
     for (int i = threadIdx.x; i < tn * K; i += kLdsAddBlock) {
       const LdsAcc v = s_acc[i];
@@ -1826,6 +1887,42 @@ int launch_scatter_v(const ScatterArgs &args, int reduce, hipStream_t stream) {
   const int64_t n_edges = a.B * a.E;
   const unsigned g_out = grid_for(n_out);
   if (reduce == TS_SUM || reduce == TS_MUL) {
+    // A small sum whose caller wants the entries per output row as well (scatter mean): cleared, added and counted
+    // in two launches (scatter_add_count_run_kernel). Below 2^16 elements, where the run kernel takes every sum.
+    if constexpr (!(std::is_integral<T>::value && sizeof(T) < 4)) {
+      if (reduce == TS_SUM && a.count_out != nullptr && a.count_done != nullptr && n_src > 0 &&
+          n_src < ((int64_t)1 << 16) && a.run_reduce && a.lds_cache != 2 && !a.bin_any_size && a.sk == 0 &&
+          a.B * a.N < 0x7FFFFFFFll) {
+        constexpr int CN = sizeof(T) < 4 ? 4 / (int)sizeof(T) : 1;
+        const bool word_ok = CN == 1 || (a.K % CN == 0 && (reinterpret_cast<uintptr_t>(a.out) & 3) == 0 &&
+                                         (reinterpret_cast<uintptr_t>(a.src) & 3) == 0);
+        const int c = word_ok ? CN : 1;
+        const RunGrid g = run_grid(n_edges, a.K / c, c, c * (int)sizeof(T));
+        const RunGrid gc = run_grid(n_edges, 1, 1, 4);
+        if (g.ok && gc.ok && g.hot_rlog < 0 && (uint64_t)g.blocks + gc.blocks < 0x7FFFFFFFull) {
+          ScatterArgs cnt = a;
+          cnt.src = nullptr;
+          cnt.out = a.count_out;
+          cnt.K = 1;
+          cnt.out_given = 1;
+          const int64_t n_clear = (a.out_given ? 0 : n_out) + a.B * a.N;
+          hipLaunchKernelGGL(fill_out_count_kernel<T>, dim3(grid_for(n_clear)), dim3(kBlock), 0, stream, out,
+                             a.out_given ? (int64_t)0 : n_out, a.count_out, a.B * a.N);
+          const dim3 gd(g.blocks + gc.blocks, g.ychunks);
+          ts_note_scatter_route(TS_ROUTE_SUM_COUNT_RUNS);
+          if (word_ok)
+            TS_LAUNCH_RUN(g.serial, (scatter_add_count_run_kernel<T, CN, CN, true>),
+                          (scatter_add_count_run_kernel<T, CN, CN, false>), gd, stream, a, g.lshift, g.rpw, cnt, gc.rpw,
+                          g.blocks);
+          else
+            TS_LAUNCH_RUN(g.serial, (scatter_add_count_run_kernel<T, 1, 1, true>),
+                          (scatter_add_count_run_kernel<T, 1, 1, false>), gd, stream, a, g.lshift, g.rpw, cnt, gc.rpw,
+                          g.blocks);
+          *a.count_done = 1;
+          return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
+        }
+      }
+    }
     // Large inputs with rows of 64 bytes and more, given a workspace: unless the index is sorted (found out by
     // the first pass), the entries are binned by bucket of output rows and summed in LDS (scatter_binned.h);
     // the kernels launched below then return at once. A sorted index stays with them: they combine its runs
@@ -1872,7 +1969,18 @@ int launch_scatter_v(const ScatterArgs &args, int reduce, hipStream_t stream) {
                   a.run_reduce && n_edges >= 2 * kBinBlock && n_src >= ((int64_t)1 << 23);
       }
     }
-    if (!a.out_given && !routed) {
+    // a caller that wants the entries per output row as well (scatter mean), where the table kernel takes the sum by
+    // itself: it counts too, and the counts are cleared with out
+    bool count_here = false;
+    if constexpr (!(std::is_integral<T>::value && sizeof(T) < 4)) {
+      count_here = a.count_out != nullptr && a.count_done != nullptr && use_lds && !sampled && !three_way && lshift < 0 &&
+                   a.lds_cache != 2 && !a.bin_any_size;
+    }
+    if (count_here) {
+      const int64_t n_clear = (a.out_given ? 0 : n_out) + a.B * a.N;
+      hipLaunchKernelGGL(fill_out_count_kernel<T>, dim3(grid_for(n_clear)), dim3(kBlock), 0, stream, out,
+                         a.out_given ? (int64_t)0 : n_out, a.count_out, a.B * a.N);
+    } else if (!a.out_given && !routed) {
       if (sampled)
         hipLaunchKernelGGL(fill_sample_kernel<T>, dim3(g_out), dim3(kBlock), 0, stream, out, n_out, small_const<T>(0),
                            a, a.order_ws);
@@ -1923,6 +2031,12 @@ int launch_scatter_v(const ScatterArgs &args, int reduce, hipStream_t stream) {
             const int64_t epb = per_cu_chunk_edges(a.lds_epb, n_edges, sum_table_min_chunk(a.K, (int)sizeof(T)),
                                                    131072 / a.K > 2048 ? 131072 / a.K : 2048);
             if (lshift < 0) ts_note_scatter_route(sampled ? TS_ROUTE_SUM_TABLE_OR_RUNS : TS_ROUTE_SUM_TABLE);
+            if (count_here) {
+              hipLaunchKernelGGL((scatter_add_lds_kernel<T, false, true>), dim3((unsigned)((n_edges + epb - 1) / epb)),
+                                 dim3(kLdsAddBlock), 0, stream, t, tn - 1, epb);
+              *a.count_done = 1;
+              return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
+            }
             hipLaunchKernelGGL(scatter_add_lds_kernel<T>, dim3((unsigned)((n_edges + epb - 1) / epb)),
                                dim3(kLdsAddBlock), 0, stream, t, tn - 1, epb);
             if (!sampled && !three_way) return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;

@@ -1798,6 +1798,66 @@ def test_scatter_sum_and_count_in_one_call(capi, case, dtype, out_given, forced,
     assert torch.equal(cnt.cpu(), want_cnt)
 
 
+SMALL_MEAN_CASES = [
+    # B, E, K, N, kind
+    (1, 1, 1, 1, "uniform"), (1, 63, 1, 7, "uniform"), (1, 1000, 1, 100, "sorted"), (2, 777, 3, 50, "uniform"),
+    (1, 4000, 16, 300, "sorted"), (1, 2000, 16, 3, "hub"), (3, 300, 64, 40, "uniform"), (1, 500, 130, 20, "sorted"),
+    (1, 65535, 1, 1000, "hub"), (1, 1023, 33, 2000, "uniform"),
+]
+
+
+TABLE_MEAN_CASES = [
+    (1, 70000, 1, 1000, "hub"), (1, 5000, 16, 300, "uniform"), (2, 3000, 64, 100, "sorted"), (1, 40000, 3, 5000, "uniform"),
+    (1, 300000, 2, 2000, "uniform"), (1, 150000, 8, 100, "sorted"),
+]
+
+
+@pytest.mark.parametrize("case,dtype,out_given", product(
+    SMALL_MEAN_CASES + TABLE_MEAN_CASES,
+    [torch.float32, torch.float64, torch.bfloat16, torch.float16, torch.int32, torch.int64], [False, True]))
+def test_scatter_sum_and_count_in_the_launch_that_adds(capi, case, dtype, out_given):
+    """ts_scatter_sum_count_with_workspace where the sum is one launch: one launch clears out and the counts (which
+    hold rubbish before the call), one launch adds and counts -- below 2^16 elements the run kernel beside a count
+    through runs, above the table kernel with a table of counts. Rows of one column, of an odd number of columns
+    (16-bit elements then go one by one instead of in packed pairs), of 128 bytes and more (every slot walks its own
+    part), several batch rows, a hub row, indices outside [0, N), `out` given."""
+    B, E, K, N, kind = case
+    small = B * E * K < 1 << 16
+    if dtype in (torch.bfloat16, torch.float16) and E > 40 * N:
+        pytest.skip("sums of that many entries are not exactly representable in 16 bits")
+    if dtype in (torch.bfloat16, torch.float16) and kind == "hub":
+        pytest.skip("the sum of a hub row is not exactly representable in 16 bits")
+    rng = np.random.default_rng(E * 31 + K * 7 + N)
+    src = torch.from_numpy(rng.integers(-9, 10, size=(B, E, K))).to(dtype)   # small integers: exact sums in every type
+    if kind == "hub":
+        index = rng.integers(0, N, size=(B, E))
+        index[:, rng.random(E) < 0.5] = N // 2
+    elif kind == "sorted":
+        index = np.sort(rng.integers(0, N, size=(B, E)), axis=1)
+    else:
+        index = rng.integers(0, N, size=(B, E))
+    index = torch.from_numpy(index.astype(np.int64))
+    if E > 100 and kind != "sorted":
+        index[0, 5] = -1
+        index[-1, 77] = N
+    valid = (index >= 0) & (index < N)
+    prev = torch.from_numpy(rng.integers(-5, 6, size=(B, N, K))).to(dtype) if out_given else torch.zeros((B, N, K), dtype=dtype)
+    want = prev.clone().double()
+    for b in range(B):
+        want[b].index_add_(0, index[b][valid[b]], src[b, valid[b]].double())
+    want_cnt = torch.stack([torch.bincount(index[b][valid[b]], minlength=N) for b in range(B)]).int()
+    out = (prev.clone() if out_given else torch.full((B, N, K), 3, dtype=dtype)).to(DEV)
+    cnt = torch.full((B, N), -7, dtype=torch.int32, device=DEV)
+    capi.scatter_sum_count_with_workspace(src.to(DEV), index.to(DEV), out, cnt, B, E, K, N, E, 1, out_given)
+    torch.cuda.synchronize()
+    if small:
+        assert capi.scatter_last_route() == "sum: runs, entries per row counted by the same launch"
+    elif dtype == torch.float32:
+        assert capi.scatter_last_route() == "sum: table"
+    assert torch.equal(out.cpu().double(), want)
+    assert torch.equal(cnt.cpu(), want_cnt)
+
+
 def test_scatter_sum_of_single_values_sorted_index_keeps_the_run_kernels(capi, oracle, monkeypatch):
     """A sorted index: the sample sends the call to the kernels that combine runs; the bucket passes return at once."""
     monkeypatch.setenv("TS_SCATTER_BINNED", "2")
