@@ -292,7 +292,7 @@ const char *ts_scatter_route_name(int route) {
       "min/max: runs", "min/max: runs or table (sample)", "min/max: table", "min/max: table, one value per entry",
       "min/max: slabs, one value per entry", "min/max: buckets", "min/max: buckets or segmented reduction (index checked)",
       "min/max: 64-bit elements, two passes", "sum: single values in buckets, table or runs (sample)",
-      "sum: runs, entries per row counted by the same launch"};
+      "sum: runs, entries per row counted by the same launch", "sum: single values, tables in slabs"};
   return route >= 0 && route < (int)(sizeof(names) / sizeof(names[0])) ? names[route] : "unknown";
 }
 
@@ -570,6 +570,13 @@ size_t ts_scatter_workspace_bytes(int64_t B, int64_t E, int64_t K, int64_t N, in
       // one 4-byte value per entry: (row in bucket, value) words, 8 bytes of scratch per entry
       const size_t payload = bin_plan_payload(B, E, K, N, kElemBytes[dtype], nullptr, 0, any_size).bytes;
       if (payload != 0) return payload;
+      // single 4-byte values from 2^19 entries: a table per workgroup, handed over in slabs (with room for the counts
+      // of scatter mean)
+      if ((dtype == TS_F32 || dtype == TS_I32) && env_int("TS_SCATTER_LDS", 1) == 1 && env_int("TS_SCATTER_SLABS", 1)) {
+        const size_t slabs =
+            s1_plan(B, E, K, N, kElemBytes[dtype], nullptr, 0, true, env_int("TS_SCATTER_SLABS", 1) == 2).bytes;
+        if (slabs != 0) return slabs;
+      }
     }
     if (binned == 0) {
       // one word for the sample of the index that keeps a sorted one away from the table kernel

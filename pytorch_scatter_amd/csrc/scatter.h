@@ -1752,6 +1752,7 @@ inline unsigned grid_for(int64_t n, int per_thread = 1) {
 }  // namespace ts
 #include "scatter_binned.h"
 #include "scatter_k1.h"
+#include "scatter_k1_sum.h"
 namespace ts {
 
 // ---- elementwise helpers --------------------------------------------------------
@@ -1942,6 +1943,33 @@ int launch_scatter_v(const ScatterArgs &args, int reduce, hipStream_t stream) {
             bp = bin_plan_payload(a.B, a.E, a.K, a.N, (int)sizeof(T), a.bin_ws, a.bin_ws_bytes, a.bin_any_size != 0);
             lshift = bp.ok ? 0 : -1;
           }
+        }
+      }
+    }
+    // Single 4-byte values between the sizes of the table kernel and of the value buckets, given a workspace: tables
+    // handed over in slabs (scatter_k1_sum.h), with the counts of scatter mean if the caller wants them.
+    // TS_SCATTER_SLABS (tuning aid): 0 never, 2 at any size.
+    if constexpr (__is_same(T, float) || __is_same(T, int32_t)) {
+      const char *env = getenv("TS_SCATTER_SLABS");
+      const int slab_mode = env ? atoi(env) : 1;
+      if (reduce == TS_SUM && lshift < 0 && n_src > 0 && slab_mode != 0 && a.bin_ws != nullptr && a.sk == 0 && a.se == 1 &&
+          a.lds_cache == 1 && a.src != nullptr && (reinterpret_cast<uintptr_t>(a.src) & 15) == 0 &&
+          (reinterpret_cast<uintptr_t>(a.index) & 15) == 0) {
+        const bool with_count = a.count_out != nullptr && a.count_done != nullptr;
+        const S1Plan sp = s1_plan(a.B, a.E, a.K, a.N, (int)sizeof(T), a.bin_ws, a.bin_ws_bytes, with_count, slab_mode == 2);
+        if (sp.ok) {
+          ScatterArgs s = a;
+          if (!with_count) s.count_out = nullptr;
+          if (with_count) {
+            hipLaunchKernelGGL(fill_out_count_kernel<T>, dim3(grid_for((a.out_given ? 0 : n_out) + a.N)), dim3(kBlock), 0,
+                               stream, out, a.out_given ? (int64_t)0 : n_out, a.count_out, a.N);
+          } else if (!a.out_given) {
+            hipLaunchKernelGGL(fill_kernel<T>, dim3(g_out), dim3(kBlock), 0, stream, out, n_out, small_const<T>(0));
+          }
+          ts_note_scatter_route(TS_ROUTE_SUM_SLABS);
+          launch_scatter_s1<T>(s, sp, stream);
+          if (with_count) *a.count_done = 1;
+          return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
         }
       }
     }

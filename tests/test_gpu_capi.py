@@ -1858,6 +1858,62 @@ def test_scatter_sum_and_count_in_the_launch_that_adds(capi, case, dtype, out_gi
     assert torch.equal(cnt.cpu(), want_cnt)
 
 
+SLAB_CASES = [
+    # E, N, kind, forced (TS_SCATTER_SLABS=2: outside the sizes where the route applies by itself)
+    (600_001, 100_000, "uniform", False), (1 << 20, 300_000, "zipf", False), (700_003, 5000, "sorted", False),
+    (524_290, 524_288, "uniform", False), (2_000_000, 8192, "hub", False),
+    (1, 5, "uniform", True), (4099, 100, "hub", True), (70_000, 9000, "uniform", True), (3, 1, "uniform", True),
+]
+
+
+@pytest.mark.parametrize("case,dtype,out_given,counted", product(
+    SLAB_CASES, [torch.float32, torch.int32], [False, True], [False, True]))
+def test_scatter_sum_of_single_values_through_slabs(capi, case, dtype, out_given, counted, monkeypatch):
+    """Single 4-byte values between the sizes of the table kernel and of the value buckets: a table per workgroup,
+    handed over in slabs, and the counts of scatter mean from the same launches. An index in random order, skewed,
+    with a hub row, in order (tables with few rows are written back with atomics and their slabs stay unused), as
+    many output rows as the route takes, indices outside [0, N), a number of entries that is no multiple of four,
+    `out` given."""
+    E, N, kind, forced = case
+    if forced:
+        monkeypatch.setenv("TS_SCATTER_SLABS", "2")
+    rng = np.random.default_rng(E + N)
+    src = torch.from_numpy(rng.integers(-9, 10, size=(1, E, 1))).to(dtype)   # small integers: exact sums
+    if kind == "zipf":
+        p = np.arange(1, N + 1, dtype=np.float64) ** -1.2
+        index = (rng.choice(N, size=(1, E), p=p / p.sum()) * 7919) % N
+    elif kind == "hub":
+        index = rng.integers(0, N, size=(1, E))
+        index[:, rng.random(E) < 0.4] = N // 3
+    elif kind == "sorted":
+        index = np.sort(rng.integers(0, N, size=(1, E)), axis=1)
+    else:
+        index = rng.integers(0, N, size=(1, E))
+    index = torch.from_numpy(index.astype(np.int64))
+    if E > 100 and kind != "sorted":
+        index[0, 5] = -1
+        index[0, 77] = N
+    valid = (index >= 0) & (index < N)
+    prev = torch.from_numpy(rng.integers(-5, 6, size=(1, N, 1))).to(dtype) if out_given else torch.zeros((1, N, 1), dtype=dtype)
+    want = prev.clone().double()
+    want[0, :, 0].index_add_(0, index[0][valid[0]], src[0, valid[0], 0].double())
+    want_cnt = torch.bincount(index[0][valid[0]], minlength=N).int().view(1, N)
+    out = (prev.clone() if out_given else torch.full((1, N, 1), 3, dtype=dtype)).to(DEV)
+    if counted:
+        cnt = torch.full((1, N), -7, dtype=torch.int32, device=DEV)
+        capi.scatter_sum_count_with_workspace(src.to(DEV), index.to(DEV), out, cnt, 1, E, 1, N, E, 1, out_given)
+    else:
+        capi.scatter_with_workspace(src.to(DEV), index.to(DEV), out, None, 1, E, 1, N, E, 1, 0, capi.SUM, out_given)
+    torch.cuda.synchronize()
+    if counted and E < 1 << 16:   # (a small sum that counts as well has its own launch)
+        assert capi.scatter_last_route() == "sum: runs, entries per row counted by the same launch"
+    else:
+        assert capi.scatter_last_route() == "sum: single values, tables in slabs"
+    assert torch.equal(out.cpu().double(), want)
+    if counted:
+        assert torch.equal(cnt.cpu(), want_cnt)
+
+
 def test_scatter_sum_of_single_values_sorted_index_keeps_the_run_kernels(capi, oracle, monkeypatch):
     """A sorted index: the sample sends the call to the kernels that combine runs; the bucket passes return at once."""
     monkeypatch.setenv("TS_SCATTER_BINNED", "2")

@@ -98,10 +98,12 @@ def test_route_narrow_rows_unsorted(env):
 
 
 @pytest.mark.parametrize("E,route", [((1 << 21) + 4096, "sum: single values in buckets, table or runs (sample)"),
-                                     ((1 << 21) - 4096, "sum: table")])
+                                     ((1 << 21) - 4096, "sum: single values, tables in slabs"),
+                                     ((1 << 19) + 4096, "sum: single values, tables in slabs"),
+                                     ((1 << 19) - 4096, "sum: table")])
 def test_route_single_values_either_side_of_the_value_buckets(env, E, route):
     """One float per entry under an index in random order (the width-1 column of the benchmark table): value
-    buckets from 2^21 entries, the accumulator table below."""
+    buckets from 2^21 entries, tables handed over in slabs from 2^19, the accumulator table below."""
     ts, capi, _ = env
     g = torch.Generator().manual_seed(E)
     N = 270_000
