@@ -794,8 +794,8 @@ int ts_scatter_sum_count_with_workspace(const void *src, const int64_t *index, v
     const bool any_size = env_int("TS_SCATTER_BINNED", 1) == 2;
     bool planned = kAccBytes[dtype] >= 4 && bin_plan(B, E, K, N, kElemBytes[dtype], workspace, workspace_bytes, any_size,
                                                      dtype == TS_I32 ? 4 : 8, false, true).ok;
-    if (!planned && K == 1 && kElemBytes[dtype] == 4)
-      planned = bin_plan_payload(B, E, 1, N, 4, workspace, workspace_bytes, any_size).ok;
+    if (!planned && K <= kBinPayloadCols && (dtype == TS_F32 || dtype == TS_I32))
+      planned = bin_plan_payload(B, E, K, N, 4, workspace, workspace_bytes, any_size).ok;
     may_fuse = planned;
   }
   if (may_fuse)
@@ -827,7 +827,7 @@ int ts_scatter_sum_count_with_workspace(const void *src, const int64_t *index, v
   c.lds_cache = env_int("TS_SCATTER_LDS", 1);
   c.lds_epb = env_int("TS_SCATTER_EPB", 0);
   c.skip_flag = flag;
-  if (K == 1) {
+  if (K <= kBinPayloadCols) {  // (the plans whose sample can answer "skewed")
     ScatterArgs t = c;
     t.skip_want = 2;
     const int64_t epb = per_cu_chunk_edges(c.lds_epb, B * E, sum_table_min_chunk(1, 4), 131072);

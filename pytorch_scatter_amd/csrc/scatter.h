@@ -1937,9 +1937,9 @@ int launch_scatter_v(const ScatterArgs &args, int reduce, hipStream_t stream) {
         bp = bin_plan(a.B, a.E, a.K, a.N, (int)sizeof(T), a.bin_ws, a.bin_ws_bytes, a.bin_any_size != 0,
                       (int)sizeof(typename BinSlot<T>::type), false, true);
         lshift = bp.ok ? bin_lane_shift(bp.p, VEC) : -1;
-        if constexpr (sizeof(T) == 4 && VEC == 1) {
-          // one 4-byte value per entry: the value travels in the binned word (bin_plan_payload)
-          if (!bp.ok && a.K == 1 && a.lds_cache) {
+        if constexpr (sizeof(T) == 4) {
+          // up to eight 4-byte values per entry: the values travel in the binned words (bin_plan_payload)
+          if (!bp.ok && a.K <= kBinPayloadCols && a.lds_cache) {
             bp = bin_plan_payload(a.B, a.E, a.K, a.N, (int)sizeof(T), a.bin_ws, a.bin_ws_bytes, a.bin_any_size != 0);
             lshift = bp.ok ? 0 : -1;
           }

@@ -30,6 +30,11 @@ constexpr int kCombFew = 32;          // many: more than this
 constexpr int kBinCountShift = 10;   // rows per bucket (log2) up to which bin_add_wave_kernel can count entries per row as well
 constexpr int kBinPlaceBlock = 1024;   // (measured slower: 256 lanes x 4 batches, 64 K entries per workgroup, 8 K)
 
+// 4-byte values per entry that travel in binned words, one plane of words per column. Every plane costs what a single
+// value costs (9 M entries onto 1 M rows, uniform index: 129 / 200 / 289 / 379 us for 1 / 2 / 3 / 4 values, 951 us for
+// eight, whose 512-row buckets also outgrow the place pass that sorts its tile) against 440 us for one atomic per row.
+constexpr int kBinPayloadCols = 3;
+
 struct BinArgs {
   int rshift;              // log2 of the rows per bucket
   int kc;                  // columns of a row that one reducing workgroup holds in LDS (K when slices == 1)
@@ -62,6 +67,8 @@ struct BinArgs {
                            // (bin_sample_kernel); then the count pass returns at once as well
   int payload = 0;         // sum of one 4-byte value per entry: the low half of a binned word holds the value's bits
                            // instead of the entry number, so the reducing pass never goes back to src
+  int planes = 1;          // ... of `planes` 4-byte values per entry (rows of up to 32 bytes): one array of words per
+  int64_t plane_words = 0; // column, plane_words apart; an entry has the same place in every one of them
   int32_t *count_out = nullptr;  // sums: the adding pass also counts the entries of every output row into this
                            // [B * N] array (the divisor of a mean, from the same words); row buckets: rshift <= kBinCountShift
 };
@@ -205,7 +212,7 @@ inline BinPlan bin_plan_payload(int64_t B, int64_t E, int64_t K, int64_t N, int 
   r.ok = false;
   r.bytes = 0;
   const int64_t n_edges = B * E, rows = B * N;
-  if (K != 1 || elem_bytes != 4 || n_edges >= 0xFFFFFFFEll || rows >= 0x7FFFFFFFll || rows < 1) return r;
+  if (K < 1 || K > kBinPayloadCols || elem_bytes != 4 || n_edges >= 0xFFFFFFFEll || rows >= 0x7FFFFFFFll || rows < 1) return r;
   // from 2 M entries: an even index gains from there on (74 against 106 us; 2.3 M entries of a graph in random order
   // 85 against 125 us); a skewed one, which the sample hands to the table kernel, pays about 15 us for the launches
   // that return at once (2.3 M entries: 51 against 36 us)
@@ -217,10 +224,14 @@ inline BinPlan bin_plan_payload(int64_t B, int64_t E, int64_t K, int64_t N, int 
   if (const char *env = getenv("TS_BIN_CHUNK")) chunk = atoi(env) > 0 ? atoi(env) : chunk;  // tuning aid
   // rows per bucket: as many as the table holds (4096). Fewer, larger buckets make the place pass cheaper (21 M entries:
   // 256 rows 580 us, 1024 rows 494, 4096 rows 393 for the whole call), which outweighs the longer write-back per chunk.
-  int rshift = 12;
+  // (K values per entry: the table's 4096 slots hold 4096 / K rows, rounded down to a power of two)
+  int top = 12;
+  while (((int64_t)K << top) > 4096) --top;
+  int rshift = top;
   if (const char *env = getenv("TS_BIN_PAYLOAD_RSHIFT")) rshift = atoi(env);  // tuning aid
-  while (rshift < 12 && ((rows + ((int64_t)1 << rshift) - 1) >> rshift) > kBinMaxBuckets) ++rshift;
-  if (rshift > 12) rshift = 12;
+  while (rshift < top && ((rows + ((int64_t)1 << rshift) - 1) >> rshift) > kBinMaxBuckets) ++rshift;
+  if (rshift > top) rshift = top;
+  if (rshift < 0) rshift = 0;
   const int64_t nb = (rows + ((int64_t)1 << rshift) - 1) >> rshift;
   if (nb > kBinMaxBuckets) return r;                       // more output rows than 16384 buckets of 4096 hold
   if (!any_size && n_edges < 2 * nb * 64) return r;        // nearly empty buckets: every one still costs its share
@@ -230,6 +241,8 @@ inline BinPlan bin_plan_payload(int64_t B, int64_t E, int64_t K, int64_t N, int 
   p.slices = 1;
   p.nb = (int)nb;
   p.payload = 1;
+  p.planes = (int)K;
+  p.plane_words = (n_edges + 3) & ~(int64_t)1;  // even, and one pair of padding: the 16-byte loads of the adding pass
   {
     const int64_t rounds = (n_edges + (int64_t)512 * kBinPlaceChunk - 1) / ((int64_t)512 * kBinPlaceChunk);
     int64_t tile = (((n_edges + 512 * rounds - 1) / (512 * rounds)) + kBinPlaceBlock - 1) & ~(int64_t)(kBinPlaceBlock - 1);
@@ -245,7 +258,7 @@ inline BinPlan bin_plan_payload(int64_t B, int64_t E, int64_t K, int64_t N, int 
   auto take = [&](size_t bytes) { const size_t o = off; off += up(bytes); return o; };
   const size_t o_tot = take((size_t)nb * 8), o_cur = take((size_t)nb * 8), o_st = take((size_t)(nb + 1) * 8);
   const size_t o_cs = take((size_t)(nb + 1) * 4), o_wb = take((size_t)p.max_wgs * 4);
-  const size_t o_bin = take((size_t)n_edges * 8), o_flag = take(256);
+  const size_t o_bin = take((size_t)p.plane_words * 8 * (size_t)K), o_flag = take(256);
   r.bytes = off;
   if (ws == nullptr || ws_bytes < off || (reinterpret_cast<uintptr_t>(ws) & 15) != 0) return r;
   char *base = static_cast<char *>(ws);
@@ -383,7 +396,10 @@ static __global__ __launch_bounds__(kBinBlock) void bin_sample_kernel(ScatterArg
 // onto 270 k rows: 51 / 89 us against 77 / 101 us through the buckets -- and sometimes far behind: the same onto 1 M
 // rows 141 / 79 us against 80 / 106 us. A bar of one half below 8 M entries was measured and lost more than it won, the
 // launches that return included; the buckets' time does not depend on where the hot rows lie.)
-static __global__ __launch_bounds__(kBinBlock) void bin_sample_skew_kernel(ScatterArgs a, int *flag) {
+// (quarters: the bar in quarters of the sample. Several values per entry: one half, since the buckets' time grows with
+// the values per entry and the table's does not -- 9 M entries of 3 floats under a Zipf(1.2) index, 64 % repeats:
+// 389 us through the buckets, about 250 through the table.)
+static __global__ __launch_bounds__(kBinBlock) void bin_sample_skew_kernel(ScatterArgs a, int *flag, int quarters) {
   constexpr int kSlots = 2048;
   __shared__ int s_set[kSlots];
   __shared__ int s_desc, s_dup;
@@ -408,7 +424,7 @@ static __global__ __launch_bounds__(kBinBlock) void bin_sample_skew_kernel(Scatt
     }
   }
   __syncthreads();
-  if (threadIdx.x == 0) *flag = s_desc * 64 < kBinBlock ? 0 : (s_dup * 4 >= 3 * kBinBlock ? 2 : 1);
+  if (threadIdx.x == 0) *flag = s_desc * 64 < kBinBlock ? 0 : (s_dup * 4 >= quarters * kBinBlock ? 2 : 1);
 }
 
 // Count pass: entries per bucket (and, for callers that ask, whether the index is in order and inside [0, N)).
@@ -660,10 +676,16 @@ void bin_place_kernel(ScatterArgs a, BinArgs p) {
   for (int j = 0; j < kBinPer; ++j) {
     if (bucket[j] < 0) continue;
     const int64_t be = lo + threadIdx.x + (int64_t)j * kBinPlaceBlock;
-    // (payload: one 4-byte value per entry, K == 1, so entry be of the flattened [B, E] is element be of src)
-    const uint32_t low = (p.payload && a.src != nullptr) ? static_cast<const uint32_t *>(a.src)[be]
-                                                         : (p.payload ? 1u : (uint32_t)be);  // no src: a count of ones
-    p.binned[s_base[bucket[j]] + (uint32_t)rank[j]] = ((uint64_t)(uint32_t)local[j] << 32) | low;
+    // (payload: the 4-byte values of entry be of the flattened [B, E] are elements be * planes ... of src, one plane
+    // of words each)
+    const uint64_t high = (uint64_t)(uint32_t)local[j] << 32;
+    uint64_t *dst = p.binned + s_base[bucket[j]] + (uint32_t)rank[j];
+    if (p.payload && a.src != nullptr) {
+      const uint32_t *vals = static_cast<const uint32_t *>(a.src) + be * p.planes;
+      for (int k = 0; k < p.planes; ++k) dst[(int64_t)k * p.plane_words] = high | vals[k];
+    } else {
+      dst[0] = high | (p.payload ? 1u : (uint32_t)be);  // no src: a count of ones
+    }
   }
 }
 static_assert(kBinPlaceChunk == kBinBatch, "the place pass holds a workgroup's entries in registers: one batch");
@@ -730,21 +752,27 @@ void bin_place_sorted_kernel(ScatterArgs a, BinArgs p) {
     run += h;
   }
   __syncthreads();
-#pragma unroll
-  for (int j = 0; j < kBinPer; ++j) {
-    if (bucket[j] < 0) continue;
-    const int64_t be = lo + threadIdx.x + (int64_t)j * kBinPlaceBlock;
-    const uint32_t low = (p.payload && a.src != nullptr) ? static_cast<const uint32_t *>(a.src)[be]
-                                                         : (p.payload ? 1u : (uint32_t)be);
-    s_stage[s_cnt[bucket[j]] + rank[j]] =
-        ((uint64_t)(uint32_t)bucket[j] << 44) | ((uint64_t)(uint32_t)local[j] << 32) | low;
-  }
-  __syncthreads();
   const int total = run_total(s_wsum);  // the tile's entries with an index inside [0, N)
-  for (int pos = threadIdx.x; pos < total; pos += kBinPlaceBlock) {
-    const uint64_t w = s_stage[pos];
-    const uint32_t b = (uint32_t)(w >> 44);
-    p.binned[s_base[b] + (uint32_t)(pos - s_cnt[b])] = w & (((uint64_t)1 << 44) - 1);
+  // one plane of words after the other through the same stage (a single one unless the entries hold several values)
+  const int planes = (p.payload && a.src != nullptr) ? p.planes : 1;
+  for (int k = 0; k < planes; ++k) {
+    if (k != 0) __syncthreads();  // the stage has been read
+#pragma unroll
+    for (int j = 0; j < kBinPer; ++j) {
+      if (bucket[j] < 0) continue;
+      const int64_t be = lo + threadIdx.x + (int64_t)j * kBinPlaceBlock;
+      const uint32_t low = (p.payload && a.src != nullptr) ? static_cast<const uint32_t *>(a.src)[be * planes + k]
+                                                           : (p.payload ? 1u : (uint32_t)be);
+      s_stage[s_cnt[bucket[j]] + rank[j]] =
+          ((uint64_t)(uint32_t)bucket[j] << 44) | ((uint64_t)(uint32_t)local[j] << 32) | low;
+    }
+    __syncthreads();
+    uint64_t *plane = p.binned + (int64_t)k * p.plane_words;
+    for (int pos = threadIdx.x; pos < total; pos += kBinPlaceBlock) {
+      const uint64_t w = s_stage[pos];
+      const uint32_t b = (uint32_t)(w >> 44);
+      plane[s_base[b] + (uint32_t)(pos - s_cnt[b])] = w & (((uint64_t)1 << 44) - 1);
+    }
   }
 }
 
@@ -1146,26 +1174,30 @@ __global__ __launch_bounds__(kBinBlock) void bin_add_payload_kernel(ScatterArgs 
   const int bucket = p.wg_bucket[wg];
   if (bucket < 0) return;
   const int rows = 1 << p.rshift;
-  for (int i = threadIdx.x; i < rows; i += kBinBlock) {
-    s_acc[i] = (A)0;
-    if (COUNT) s_num[i] = 0;
+  const int planes = p.planes;  // values per entry: slot row * planes + k of the table is element k of the row
+  for (int i = threadIdx.x; i < rows * planes; i += kBinBlock) s_acc[i] = (A)0;
+  if (COUNT) {
+    for (int i = threadIdx.x; i < rows; i += kBinBlock) s_num[i] = 0;
   }
   __syncthreads();
   const int64_t lo = p.starts[bucket] + ((int64_t)wg - p.chunk_start[bucket]) * p.chunk;
   int64_t hi = lo + p.chunk;
   if (hi > p.starts[bucket + 1]) hi = p.starts[bucket + 1];
+  int k = 0;
   auto add = [&](unsigned long long w) {
     T v;
     const uint32_t bits = (uint32_t)w;
     __builtin_memcpy(&v, &bits, 4);
     const uint32_t row = (uint32_t)(w >> 32) & (uint32_t)(rows - 1);
-    __hip_atomic_fetch_add(&s_acc[row], (A)v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-    if (COUNT) __hip_atomic_fetch_add(&s_num[row], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    __hip_atomic_fetch_add(&s_acc[row * planes + k], (A)v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    if (COUNT) {
+      if (k == 0) __hip_atomic_fetch_add(&s_num[row], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
   };
-  if (lo < hi) {
-    // words lo .. hi - 1; the 16-byte loads start at an even word
+  for (k = 0; k < planes && lo < hi; ++k) {
+    // words lo .. hi - 1 of plane k; the 16-byte loads start at an even word (planes are an even number of words apart)
     const int64_t first = lo & ~(int64_t)1;
-    const u64x2 *pairs = reinterpret_cast<const u64x2 *>(p.binned + first);
+    const u64x2 *pairs = reinterpret_cast<const u64x2 *>(p.binned + (int64_t)k * p.plane_words + first);
     const int64_t n_pairs = (hi - first + 1) >> 1;  // the last pair may reach one word past hi: inside the array or its padding
     for (int64_t base = 0; base < n_pairs; base += (int64_t)U * kBinBlock) {
       u64x2 w[U];
@@ -1185,12 +1217,14 @@ __global__ __launch_bounds__(kBinBlock) void bin_add_payload_kernel(ScatterArgs 
     }
   }
   __syncthreads();
-  T *out = static_cast<T *>(a.out) + ((int64_t)bucket << p.rshift);
+  T *out = static_cast<T *>(a.out) + ((int64_t)bucket << p.rshift) * planes;
   const int64_t rows_left = a.B * a.N - ((int64_t)bucket << p.rshift);  // rows that exist
-  for (int i = threadIdx.x; i < rows && i < rows_left; i += kBinBlock) {
+  for (int i = threadIdx.x; i < rows * planes && i < rows_left * planes; i += kBinBlock) {
     const A v = s_acc[i];
     if (v != (A)0) atomic_add_elem<T>(out + i, (T)v);
-    if (COUNT) {
+  }
+  if (COUNT) {
+    for (int i = threadIdx.x; i < rows && i < rows_left; i += kBinBlock) {
       const int32_t c = s_num[i];
       if (c != 0) atomicAdd(p.count_out + ((int64_t)bucket << p.rshift) + i, c);
     }
@@ -1281,7 +1315,7 @@ void launch_binned_add(const ScatterArgs &a, const BinArgs &plan, int lshift, hi
     p.strict = 1;
   }
   if (p.sampled && three_way)
-    hipLaunchKernelGGL(bin_sample_skew_kernel, dim3(1), dim3(kBinBlock), 0, stream, a, p.unsorted);
+    hipLaunchKernelGGL(bin_sample_skew_kernel, dim3(1), dim3(kBinBlock), 0, stream, a, p.unsorted, p.planes > 1 ? 2 : 3);
   else if (p.sampled)
     hipLaunchKernelGGL(bin_sample_kernel, dim3(1), dim3(kBinBlock), 0, stream, a, p.unsorted);
   hipLaunchKernelGGL(bin_clear_kernel, dim3((p.nb + kBlock - 1) / kBlock), dim3(kBlock), 0, stream, p.totals, p.nb,
@@ -1298,7 +1332,7 @@ void launch_binned_add(const ScatterArgs &a, const BinArgs &plan, int lshift, hi
     hipLaunchKernelGGL(bin_place_kernel<kBinSmallCap>, dim3((unsigned)p.n_place), dim3(kBinPlaceBlock), 0, stream, a, p);
   else
     hipLaunchKernelGGL(bin_place_kernel<kBinMaxBuckets>, dim3((unsigned)p.n_place), dim3(kBinPlaceBlock), 0, stream, a, p);
-  if constexpr (sizeof(T) == 4 && VEC == 1) {
+  if constexpr (sizeof(T) == 4) {
     if (p.payload) {
       if (p.count_out != nullptr)
         hipLaunchKernelGGL((bin_add_payload_kernel<T, true>), dim3((unsigned)p.max_wgs), dim3(kBinBlock), 0, stream, a, p);

@@ -1046,8 +1046,13 @@ def test_scatter_sum_narrow_rows_sample_picks_the_kernel(capi, oracle, shape, ki
     index = index1.view(1, E, 1).expand(B, E, K)
     L = capi.lib()
     need = L.ts_scatter_workspace_bytes(capi._i(B), capi._i(E), capi._i(K), capi._i(N), capi.DTYPE[dtype], capi.SUM)
-    by_sample = B * E * K >= (1 << 23) and (K < 32 or dtype == torch.float32)
-    assert need == (256 if by_sample else need) and need in (0, 256)
+    # (rows of up to three floats from 2^21 entries: the value buckets, with scratch for the binned words)
+    value_buckets = dtype == torch.float32 and K <= 3 and B * E >= 1 << 21
+    by_sample = not value_buckets and B * E * K >= (1 << 23) and (K < 32 or dtype == torch.float32)
+    if value_buckets:
+        assert need >= 8 * B * E * K
+    else:
+        assert need == (256 if by_sample else need) and need in (0, 256)
     exact = oracle.scatter(src.double(), index, 1, None, N, "sum")[0]
     absum = oracle.scatter(src.double().abs(), index, 1, None, N, "sum")[0]
     for out_given in (False, True):
@@ -1910,6 +1915,60 @@ def test_scatter_sum_of_single_values_through_slabs(capi, case, dtype, out_given
         assert capi.scatter_last_route() == "sum: runs, entries per row counted by the same launch"
     else:
         assert capi.scatter_last_route() == "sum: single values, tables in slabs"
+    assert torch.equal(out.cpu().double(), want)
+    if counted:
+        assert torch.equal(cnt.cpu(), want_cnt)
+
+
+VALUE_ROW_CASES = [
+    # B, E, K, N, kind, forced (TS_SCATTER_BINNED=2: below the size from which the value buckets take a call)
+    (1, (1 << 21) + 77, 3, 300_000, "uniform", False), (1, (1 << 21) + 2, 2, 1_000_000, "uniform", False),
+    (1, 2_500_001, 3, 40_000, "zipf", False), (1, 2_200_000, 2, 5000, "sorted", False),
+    (1, 90_001, 2, 5000, "uniform", True), (2, 50_003, 3, 3000, "hub", True), (1, 70_000, 2, 9000, "zipf", True),
+    (1, 30_000, 3, 200_000, "uniform", True), (3, 20_001, 2, 100, "uniform", True), (1, 40_000, 3, 700, "sorted", True),
+]
+
+
+@pytest.mark.parametrize("case,dtype,out_given,counted", product(
+    VALUE_ROW_CASES, [torch.float32, torch.int32], [False, True], [False, True]))
+def test_scatter_sum_of_narrow_rows_through_value_buckets(capi, case, dtype, out_given, counted, monkeypatch):
+    """Rows of two or three 4-byte values under an index in no order: the values travel in the binned words, one plane
+    of words per column, and the counts of scatter mean come from the same pass. Row widths that are no power of
+    two, several batch rows, a hub row, a skewed and a sorted index (which the sample hands to the table / run
+    kernels behind the buckets), indices outside [0, N), `out` given."""
+    B, E, K, N, kind, forced = case
+    if forced:
+        monkeypatch.setenv("TS_SCATTER_BINNED", "2")
+    rng = np.random.default_rng(E + N + K)
+    src = torch.from_numpy(rng.integers(-9, 10, size=(B, E, K))).to(dtype)   # small integers: exact sums
+    if kind == "zipf":
+        p = np.arange(1, N + 1, dtype=np.float64) ** -1.2
+        index = (rng.choice(N, size=(B, E), p=p / p.sum()) * 7919) % N
+    elif kind == "hub":
+        index = rng.integers(0, N, size=(B, E))
+        index[:, rng.random(E) < 0.4] = N // 3
+    elif kind == "sorted":
+        index = np.sort(rng.integers(0, N, size=(B, E)), axis=1)
+    else:
+        index = rng.integers(0, N, size=(B, E))
+    index = torch.from_numpy(index.astype(np.int64))
+    if kind != "sorted":
+        index[0, 5] = -1
+        index[-1, 77] = N
+    valid = (index >= 0) & (index < N)
+    prev = torch.from_numpy(rng.integers(-5, 6, size=(B, N, K))).to(dtype) if out_given else torch.zeros((B, N, K), dtype=dtype)
+    want = prev.clone().double()
+    for b in range(B):
+        want[b].index_add_(0, index[b][valid[b]], src[b, valid[b]].double())
+    want_cnt = torch.stack([torch.bincount(index[b][valid[b]], minlength=N) for b in range(B)]).int()
+    out = (prev.clone() if out_given else torch.full((B, N, K), 3, dtype=dtype)).to(DEV)
+    if counted:
+        cnt = torch.full((B, N), -7, dtype=torch.int32, device=DEV)
+        capi.scatter_sum_count_with_workspace(src.to(DEV), index.to(DEV), out, cnt, B, E, K, N, E, 1, out_given)
+    else:
+        capi.scatter_with_workspace(src.to(DEV), index.to(DEV), out, None, B, E, K, N, E, 1, 0, capi.SUM, out_given)
+    torch.cuda.synchronize()
+    assert capi.scatter_last_route() == "sum: single values in buckets, table or runs (sample)"
     assert torch.equal(out.cpu().double(), want)
     if counted:
         assert torch.equal(cnt.cpu(), want_cnt)
