@@ -183,6 +183,10 @@ def sweep_thresholds():
         ("sum: buckets of output rows from 64 MB (K = 32)", "sum", 32, 100_000, [M // 2 - 16384, M // 2 + 16384]),
         ("sum: single values in buckets from 2^21 entries (K = 1; sample of the index)", "sum", 1, 1_000_000,
          [2 * M - 65536, 2 * M + 65536]),
+        ("sum: single values, tables in slabs from 2^19 entries (K = 1)", "sum", 1, 100_000,
+         [M // 2 - 16384, M // 2 + 16384]),
+        ("sum: rows of two values in buckets from 2^21 entries (K = 2; sample of the index)", "sum", 2, 1_000_000,
+         [2 * M - 65536, 2 * M + 65536]),
         ("max: LDS table from 2^20 elements (contended index)", "max", 8, 1000, [M // 8 - 4096, M // 8 + 4096]),
         ("max: one value per entry, slabs from 2^14 entries", "max", 1, 100_000, [M // 64 - 1024, M // 64 + 1024]),
         ("max: buckets of output rows from 24 MB (K = 32, keys of 25 MB)", "max", 32, 100_000,
