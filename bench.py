@@ -546,6 +546,12 @@ def main():
         uni = torch.randint(0, 1_000_000, (wz.E,), generator=g)
         su = wl.ScatterWorkload("X-uniform-deg10-K64", uni, 1_000_000, wz.E, 64, torch.float32)
         table["X-uniform-deg10-K64"] = bench_scatter_config(ts, wl, su, dev, max(it // 2, 3), ["sum", "max"])
+        # narrow rows under the same uniform index: two floats per entry (values travel in binned words), and one
+        # float per entry at a tenth of the size (a table per workgroup, handed over in slabs)
+        su2 = wl.ScatterWorkload("X-uniform-deg10-K2", uni, 1_000_000, wz.E, 2, torch.float32)
+        table["X-uniform-deg10-K2"] = bench_scatter_config(ts, wl, su2, dev, max(it // 2, 3), ["sum"])
+        su1 = wl.ScatterWorkload("X-uniform-deg10-K1-1M", uni[:1_000_000] % 100_000, 100_000, 1_000_000, 1, torch.float32)
+        table["X-uniform-deg10-K1-1M"] = bench_scatter_config(ts, wl, su1, dev, max(it // 2, 3), ["sum"])
         sz64 = wl.ScatterWorkload("X-zipf-unsorted-K64", zipf_index, 1_000_000, wz.E, 64, torch.float32)
         table["X-zipf-unsorted-K64"] = bench_scatter_config(ts, wl, sz64, dev, max(it // 2, 3), ["sum", "max"])
         table["X-sorted-plan-C4-K32"] = bench_sorted_config(ts, wl, wl.c4_scatter_minmax(32), dev, max(it // 2, 3))
