@@ -213,9 +213,9 @@ int ts_scatter(const void *src, const int64_t *index, void *out,
  * other large inputs of 4-byte elements with few entries per output row ask for 256 bytes: one flag,
  * written by a sample of the index, that picks the kernel for a skewed or an even index; so do SUMs
  * at the sizes that go through the accumulator table in LDS (from 2^23 elements on the sample keeps a
- * sorted index with the kernel that combines its runs: about twice as fast). SUM of up to three floats
- * or int32 per entry: from 2^21 entries the values travel in the binned words (8 bytes of scratch per
- * element). SUM of one float or int32 per entry (K == 1, B == 1, N <= 524288, contiguous index, src and
+ * sorted index with the kernel that combines its runs: about twice as fast). SUM of up to four floats
+ * or int32 per entry: from 2^21 entries the values travel with their bucket (8 bytes of scratch per entry
+ * for one value, 4 * (K + 1) for several). SUM of one float or int32 per entry (K == 1, B == 1, N <= 524288, contiguous index, src and
  * index on 16-byte borders) from 2^19 entries: every workgroup keeps a table in LDS and hands it over in a
  * slab of the workspace instead of writing it back with atomics. MIN / MAX: same
  * results as ts_scatter; SUM: the same sum in another order of additions. No counterpart in the reference

@@ -804,7 +804,7 @@ int ts_scatter_sum_count_with_workspace(const void *src, const int64_t *index, v
   int counted = 0;
   const int rc = scatter_ws_impl(src, index, out, nullptr, B, E, K, N, index_stride_b, index_stride_e, 0, dtype, TS_SUM,
                                  out_given, workspace, workspace_bytes, stream, count, may_fuse ? &flag : nullptr, &counted);
-  if (rc != TS_OK || counted) return rc;
+  if (rc != TS_OK || counted == 1) return rc;
   if (flag == nullptr)  // another route: the count on its own (with its own fill)
     return ts_scatter_count_with_workspace(index, count, B, E, N, index_stride_b, index_stride_e, workspace, workspace_bytes,
                                            stream);
@@ -827,7 +827,7 @@ int ts_scatter_sum_count_with_workspace(const void *src, const int64_t *index, v
   c.lds_cache = env_int("TS_SCATTER_LDS", 1);
   c.lds_epb = env_int("TS_SCATTER_EPB", 0);
   c.skip_flag = flag;
-  if (K <= kBinPayloadCols) {  // (the plans whose sample can answer "skewed")
+  if (K <= kBinPayloadCols && counted != 2) {  // (the plans whose sample can answer "skewed"; 2: the sum's table counted)
     ScatterArgs t = c;
     t.skip_want = 2;
     const int64_t epb = per_cu_chunk_edges(c.lds_epb, B * E, sum_table_min_chunk(1, 4), 131072);

@@ -241,7 +241,8 @@ struct ScatterArgs {
   const int **count_flag = nullptr;  // ... and leave the buckets' flag here (still null afterwards: the call took another
                                    // route and nothing was counted)
   int *count_done = nullptr;       // (host) a small sum counts into count_out (not zeroed by the caller) in the launch that
-                                   // adds (scatter_add_count_run_kernel) and sets this to 1: the counts are complete
+                                   // adds (scatter_add_count_run_kernel) and sets this to 1: the counts are complete;
+                                   // 2: the table kernel behind the value buckets counts for the verdict "skewed"
   int *order_ws = nullptr;         // sum of narrow rows: a word of scratch for the sample of the index that picks the kernel
   int skew_probe = 1;              // min/max: sample the index for skew (needs 256 bytes of workspace): 0 never, 2 at any size
   const int *skew_flag = nullptr;  // min/max kernels behind the probe: run only if (*skew_flag != 0) == (skew_want != 0)
@@ -2065,8 +2066,16 @@ int launch_scatter_v(const ScatterArgs &args, int reduce, hipStream_t stream) {
               *a.count_done = 1;
               return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
             }
-            hipLaunchKernelGGL(scatter_add_lds_kernel<T>, dim3((unsigned)((n_edges + epb - 1) / epb)),
-                               dim3(kLdsAddBlock), 0, stream, t, tn - 1, epb);
+            // behind value buckets that count as well: the table kernel, which takes a skewed index from them, counts too
+            // (*count_done = 2 tells the caller, which then has no table of counts to launch for that verdict)
+            if (three_way && lshift >= 0 && bp.p.count_out != nullptr && a.count_done != nullptr) {
+              hipLaunchKernelGGL((scatter_add_lds_kernel<T, false, true>), dim3((unsigned)((n_edges + epb - 1) / epb)),
+                                 dim3(kLdsAddBlock), 0, stream, t, tn - 1, epb);
+              *a.count_done = 2;
+            } else {
+              hipLaunchKernelGGL(scatter_add_lds_kernel<T>, dim3((unsigned)((n_edges + epb - 1) / epb)),
+                                 dim3(kLdsAddBlock), 0, stream, t, tn - 1, epb);
+            }
             if (!sampled && !three_way) return hipGetLastError() == hipSuccess ? TS_OK : TS_ERR_LAUNCH;
           }
         }

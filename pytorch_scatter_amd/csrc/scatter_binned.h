@@ -30,10 +30,9 @@ constexpr int kCombFew = 32;          // many: more than this
 constexpr int kBinCountShift = 10;   // rows per bucket (log2) up to which bin_add_wave_kernel can count entries per row as well
 constexpr int kBinPlaceBlock = 1024;   // (measured slower: 256 lanes x 4 batches, 64 K entries per workgroup, 8 K)
 
-// 4-byte values per entry that travel in binned words, one plane of words per column. Every plane costs what a single
-// value costs (9 M entries onto 1 M rows, uniform index: 129 / 200 / 289 / 379 us for 1 / 2 / 3 / 4 values, 951 us for
-// eight, whose 512-row buckets also outgrow the place pass that sorts its tile) against 440 us for one atomic per row.
-constexpr int kBinPayloadCols = 3;
+// 4-byte values per entry that travel with their bucket (bin_plan_payload): one value in an 8-byte word, several in a
+// record of K + 1 32-bit words (the values, then the row in the bucket)
+constexpr int kBinPayloadCols = 4;
 
 struct BinArgs {
   int rshift;              // log2 of the rows per bucket
@@ -67,8 +66,9 @@ struct BinArgs {
                            // (bin_sample_kernel); then the count pass returns at once as well
   int payload = 0;         // sum of one 4-byte value per entry: the low half of a binned word holds the value's bits
                            // instead of the entry number, so the reducing pass never goes back to src
-  int planes = 1;          // ... of `planes` 4-byte values per entry (rows of up to 32 bytes): one array of words per
-  int64_t plane_words = 0; // column, plane_words apart; an entry has the same place in every one of them
+  int planes = 1;          // ... of `planes` 4-byte values per entry (rows of up to 16 bytes); more than one: binned holds
+                           // records of planes + 1 32-bit words, the values and then the row in the bucket
+  int sort_tile = 6144;    // entries per workgroup of the place pass that sorts its tile in LDS (records: fewer)
   int32_t *count_out = nullptr;  // sums: the adding pass also counts the entries of every output row into this
                            // [B * N] array (the divisor of a mean, from the same words); row buckets: rshift <= kBinCountShift
 };
@@ -213,6 +213,7 @@ inline BinPlan bin_plan_payload(int64_t B, int64_t E, int64_t K, int64_t N, int 
   r.bytes = 0;
   const int64_t n_edges = B * E, rows = B * N;
   if (K < 1 || K > kBinPayloadCols || elem_bytes != 4 || n_edges >= 0xFFFFFFFEll || rows >= 0x7FFFFFFFll || rows < 1) return r;
+  if (K > 1 && n_edges * (K + 1) >= 0xFFFFFFFEll) return r;
   // from 2 M entries: an even index gains from there on (74 against 106 us; 2.3 M entries of a graph in random order
   // 85 against 125 us); a skewed one, which the sample hands to the table kernel, pays about 15 us for the launches
   // that return at once (2.3 M entries: 51 against 36 us)
@@ -234,6 +235,7 @@ inline BinPlan bin_plan_payload(int64_t B, int64_t E, int64_t K, int64_t N, int 
   if (rshift < 0) rshift = 0;
   const int64_t nb = (rows + ((int64_t)1 << rshift) - 1) >> rshift;
   if (nb > kBinMaxBuckets) return r;                       // more output rows than 16384 buckets of 4096 hold
+  if (K > 1 && nb > 2048) return r;                        // records are placed by the pass that sorts its tile only
   if (!any_size && n_edges < 2 * nb * 64) return r;        // nearly empty buckets: every one still costs its share
   BinArgs &p = r.p;
   p.rshift = rshift;
@@ -242,7 +244,8 @@ inline BinPlan bin_plan_payload(int64_t B, int64_t E, int64_t K, int64_t N, int 
   p.nb = (int)nb;
   p.payload = 1;
   p.planes = (int)K;
-  p.plane_words = (n_edges + 3) & ~(int64_t)1;  // even, and one pair of padding: the 16-byte loads of the adding pass
+  // records: as many entries per tile as the 48 KB stage holds, in whole rounds of the workgroup
+  if (K > 1) p.sort_tile = (int)(12288 / (K + 1) / kBinPlaceBlock) * kBinPlaceBlock;
   {
     const int64_t rounds = (n_edges + (int64_t)512 * kBinPlaceChunk - 1) / ((int64_t)512 * kBinPlaceChunk);
     int64_t tile = (((n_edges + 512 * rounds - 1) / (512 * rounds)) + kBinPlaceBlock - 1) & ~(int64_t)(kBinPlaceBlock - 1);
@@ -258,7 +261,7 @@ inline BinPlan bin_plan_payload(int64_t B, int64_t E, int64_t K, int64_t N, int 
   auto take = [&](size_t bytes) { const size_t o = off; off += up(bytes); return o; };
   const size_t o_tot = take((size_t)nb * 8), o_cur = take((size_t)nb * 8), o_st = take((size_t)(nb + 1) * 8);
   const size_t o_cs = take((size_t)(nb + 1) * 4), o_wb = take((size_t)p.max_wgs * 4);
-  const size_t o_bin = take((size_t)p.plane_words * 8 * (size_t)K), o_flag = take(256);
+  const size_t o_bin = take(K > 1 ? (size_t)n_edges * 4 * (size_t)(K + 1) : (size_t)n_edges * 8), o_flag = take(256);
   r.bytes = off;
   if (ws == nullptr || ws_bytes < off || (reinterpret_cast<uintptr_t>(ws) & 15) != 0) return r;
   char *base = static_cast<char *>(ws);
@@ -397,8 +400,7 @@ static __global__ __launch_bounds__(kBinBlock) void bin_sample_kernel(ScatterArg
 // rows 141 / 79 us against 80 / 106 us. A bar of one half below 8 M entries was measured and lost more than it won, the
 // launches that return included; the buckets' time does not depend on where the hot rows lie.)
 // (quarters: the bar in quarters of the sample. Several values per entry: one half, since the buckets' time grows with
-// the values per entry and the table's does not -- 9 M entries of 3 floats under a Zipf(1.2) index, 64 % repeats:
-// 389 us through the buckets, about 250 through the table.)
+// the values per entry and the table's does not.)
 static __global__ __launch_bounds__(kBinBlock) void bin_sample_skew_kernel(ScatterArgs a, int *flag, int quarters) {
   constexpr int kSlots = 2048;
   __shared__ int s_set[kSlots];
@@ -676,16 +678,10 @@ void bin_place_kernel(ScatterArgs a, BinArgs p) {
   for (int j = 0; j < kBinPer; ++j) {
     if (bucket[j] < 0) continue;
     const int64_t be = lo + threadIdx.x + (int64_t)j * kBinPlaceBlock;
-    // (payload: the 4-byte values of entry be of the flattened [B, E] are elements be * planes ... of src, one plane
-    // of words each)
-    const uint64_t high = (uint64_t)(uint32_t)local[j] << 32;
-    uint64_t *dst = p.binned + s_base[bucket[j]] + (uint32_t)rank[j];
-    if (p.payload && a.src != nullptr) {
-      const uint32_t *vals = static_cast<const uint32_t *>(a.src) + be * p.planes;
-      for (int k = 0; k < p.planes; ++k) dst[(int64_t)k * p.plane_words] = high | vals[k];
-    } else {
-      dst[0] = high | (p.payload ? 1u : (uint32_t)be);  // no src: a count of ones
-    }
+    // (payload: one 4-byte value per entry, K == 1, so entry be of the flattened [B, E] is element be of src)
+    const uint32_t low = (p.payload && a.src != nullptr) ? static_cast<const uint32_t *>(a.src)[be]
+                                                         : (p.payload ? 1u : (uint32_t)be);  // no src: a count of ones
+    p.binned[s_base[bucket[j]] + (uint32_t)rank[j]] = ((uint64_t)(uint32_t)local[j] << 32) | low;
   }
 }
 static_assert(kBinPlaceChunk == kBinBatch, "the place pass holds a workgroup's entries in registers: one batch");
@@ -752,27 +748,88 @@ void bin_place_sorted_kernel(ScatterArgs a, BinArgs p) {
     run += h;
   }
   __syncthreads();
-  const int total = run_total(s_wsum);  // the tile's entries with an index inside [0, N)
-  // one plane of words after the other through the same stage (a single one unless the entries hold several values)
-  const int planes = (p.payload && a.src != nullptr) ? p.planes : 1;
-  for (int k = 0; k < planes; ++k) {
-    if (k != 0) __syncthreads();  // the stage has been read
 #pragma unroll
-    for (int j = 0; j < kBinPer; ++j) {
-      if (bucket[j] < 0) continue;
-      const int64_t be = lo + threadIdx.x + (int64_t)j * kBinPlaceBlock;
-      const uint32_t low = (p.payload && a.src != nullptr) ? static_cast<const uint32_t *>(a.src)[be * planes + k]
-                                                           : (p.payload ? 1u : (uint32_t)be);
-      s_stage[s_cnt[bucket[j]] + rank[j]] =
-          ((uint64_t)(uint32_t)bucket[j] << 44) | ((uint64_t)(uint32_t)local[j] << 32) | low;
-    }
-    __syncthreads();
-    uint64_t *plane = p.binned + (int64_t)k * p.plane_words;
-    for (int pos = threadIdx.x; pos < total; pos += kBinPlaceBlock) {
-      const uint64_t w = s_stage[pos];
-      const uint32_t b = (uint32_t)(w >> 44);
-      plane[s_base[b] + (uint32_t)(pos - s_cnt[b])] = w & (((uint64_t)1 << 44) - 1);
-    }
+  for (int j = 0; j < kBinPer; ++j) {
+    if (bucket[j] < 0) continue;
+    const int64_t be = lo + threadIdx.x + (int64_t)j * kBinPlaceBlock;
+    const uint32_t low = (p.payload && a.src != nullptr) ? static_cast<const uint32_t *>(a.src)[be]
+                                                         : (p.payload ? 1u : (uint32_t)be);
+    s_stage[s_cnt[bucket[j]] + rank[j]] =
+        ((uint64_t)(uint32_t)bucket[j] << 44) | ((uint64_t)(uint32_t)local[j] << 32) | low;
+  }
+  __syncthreads();
+  const int total = run_total(s_wsum);  // the tile's entries with an index inside [0, N)
+  for (int pos = threadIdx.x; pos < total; pos += kBinPlaceBlock) {
+    const uint64_t w = s_stage[pos];
+    const uint32_t b = (uint32_t)(w >> 44);
+    p.binned[s_base[b] + (uint32_t)(pos - s_cnt[b])] = w & (((uint64_t)1 << 44) - 1);
+  }
+}
+
+// The same place pass for records of several values (BinArgs::planes > 1): a staged record is planes + 1 32-bit words,
+// the entry's values and then (bucket << 12 | row in the bucket); the tile holds as many entries as fit the stage
+// (BinArgs::sort_tile). The records leave in the order of the stage, 32-bit word by word: neighbouring lanes,
+// neighbouring words of one bucket's run.
+static __global__ __launch_bounds__(kBinPlaceBlock) __attribute__((amdgpu_waves_per_eu(8, 8)))
+void bin_place_records_kernel(ScatterArgs a, BinArgs p) {
+  __shared__ uint32_t s_stage[2 * kBinSortTile];
+  __shared__ int32_t s_cnt[kBinSortBuckets];   // counts, then the tile's exclusive prefix
+  __shared__ uint32_t s_base[kBinSortBuckets];  // first record of the tile's run in every bucket
+  __shared__ int32_t s_wsum[kBinPlaceBlock / kWave];
+  if (p.unsorted != nullptr && *p.unsorted != 1) return;
+  const int64_t lo = (int64_t)blockIdx.x * p.sort_tile;
+  const int64_t hi = lo + p.sort_tile < a.B * a.E ? lo + p.sort_tile : a.B * a.E;
+  for (int i = threadIdx.x; i < p.nb; i += kBinPlaceBlock) s_cnt[i] = 0;
+  __syncthreads();
+  int32_t bucket[kBinPer], local[kBinPer], rank[kBinPer];
+  bool unused = false;
+  bin_buckets(a, p, lo, hi, bucket, local, false, unused);
+#pragma unroll
+  for (int j = 0; j < kBinPer; ++j) rank[j] = bin_take(s_cnt, bucket[j]);
+  __syncthreads();
+  const int per = (p.nb + kBinPlaceBlock - 1) / kBinPlaceBlock;
+  const int b0 = threadIdx.x * per;
+  int32_t mine = 0;
+  for (int j = 0; j < per; ++j) {
+    const int i = b0 + j;
+    if (i >= p.nb) break;
+    const int32_t h = s_cnt[i];
+    if (h != 0) s_base[i] = (uint32_t)atomicAdd(&p.cursor[i], (unsigned long long)h);
+    mine += h;
+  }
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  const int32_t incl = wave_inclusive_sum(mine);
+  if (lane == kWave - 1) s_wsum[wave] = incl;
+  __syncthreads();
+  int32_t run = incl - mine;
+  for (int w2 = 0; w2 < wave; ++w2) run += s_wsum[w2];
+  for (int j = 0; j < per; ++j) {
+    const int i = b0 + j;
+    if (i >= p.nb) break;
+    const int32_t h = s_cnt[i];
+    s_cnt[i] = run;
+    run += h;
+  }
+  __syncthreads();
+  const int K = p.planes, R = K + 1;
+  const uint32_t *src = static_cast<const uint32_t *>(a.src);
+#pragma unroll
+  for (int j = 0; j < kBinPer; ++j) {
+    if (bucket[j] < 0) continue;
+    const int64_t be = lo + threadIdx.x + (int64_t)j * kBinPlaceBlock;
+    uint32_t *rec = s_stage + (s_cnt[bucket[j]] + rank[j]) * R;
+    for (int k = 0; k < K; ++k) rec[k] = src[be * K + k];
+    rec[K] = ((uint32_t)bucket[j] << 12) | (uint32_t)local[j];
+  }
+  __syncthreads();
+  const int total = run_total(s_wsum);  // the tile's entries with an index inside [0, N)
+  uint32_t *words = reinterpret_cast<uint32_t *>(p.binned);
+  for (int d = threadIdx.x; d < total * R; d += kBinPlaceBlock) {
+    const int pos = d / R, j = d - pos * R;
+    const uint32_t tail = s_stage[pos * R + K];
+    const uint32_t b = tail >> 12;
+    const int64_t dest = (int64_t)s_base[b] + (pos - s_cnt[b]);
+    words[dest * R + j] = j == K ? (tail & 0xFFFu) : s_stage[d];
   }
 }
 
@@ -1174,30 +1231,26 @@ __global__ __launch_bounds__(kBinBlock) void bin_add_payload_kernel(ScatterArgs 
   const int bucket = p.wg_bucket[wg];
   if (bucket < 0) return;
   const int rows = 1 << p.rshift;
-  const int planes = p.planes;  // values per entry: slot row * planes + k of the table is element k of the row
-  for (int i = threadIdx.x; i < rows * planes; i += kBinBlock) s_acc[i] = (A)0;
-  if (COUNT) {
-    for (int i = threadIdx.x; i < rows; i += kBinBlock) s_num[i] = 0;
+  for (int i = threadIdx.x; i < rows; i += kBinBlock) {
+    s_acc[i] = (A)0;
+    if (COUNT) s_num[i] = 0;
   }
   __syncthreads();
   const int64_t lo = p.starts[bucket] + ((int64_t)wg - p.chunk_start[bucket]) * p.chunk;
   int64_t hi = lo + p.chunk;
   if (hi > p.starts[bucket + 1]) hi = p.starts[bucket + 1];
-  int k = 0;
   auto add = [&](unsigned long long w) {
     T v;
     const uint32_t bits = (uint32_t)w;
     __builtin_memcpy(&v, &bits, 4);
     const uint32_t row = (uint32_t)(w >> 32) & (uint32_t)(rows - 1);
-    __hip_atomic_fetch_add(&s_acc[row * planes + k], (A)v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-    if (COUNT) {
-      if (k == 0) __hip_atomic_fetch_add(&s_num[row], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-    }
+    __hip_atomic_fetch_add(&s_acc[row], (A)v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    if (COUNT) __hip_atomic_fetch_add(&s_num[row], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
   };
-  for (k = 0; k < planes && lo < hi; ++k) {
-    // words lo .. hi - 1 of plane k; the 16-byte loads start at an even word (planes are an even number of words apart)
+  if (lo < hi) {
+    // words lo .. hi - 1; the 16-byte loads start at an even word
     const int64_t first = lo & ~(int64_t)1;
-    const u64x2 *pairs = reinterpret_cast<const u64x2 *>(p.binned + (int64_t)k * p.plane_words + first);
+    const u64x2 *pairs = reinterpret_cast<const u64x2 *>(p.binned + first);
     const int64_t n_pairs = (hi - first + 1) >> 1;  // the last pair may reach one word past hi: inside the array or its padding
     for (int64_t base = 0; base < n_pairs; base += (int64_t)U * kBinBlock) {
       u64x2 w[U];
@@ -1217,9 +1270,72 @@ __global__ __launch_bounds__(kBinBlock) void bin_add_payload_kernel(ScatterArgs 
     }
   }
   __syncthreads();
-  T *out = static_cast<T *>(a.out) + ((int64_t)bucket << p.rshift) * planes;
+  T *out = static_cast<T *>(a.out) + ((int64_t)bucket << p.rshift);
   const int64_t rows_left = a.B * a.N - ((int64_t)bucket << p.rshift);  // rows that exist
-  for (int i = threadIdx.x; i < rows * planes && i < rows_left * planes; i += kBinBlock) {
+  for (int i = threadIdx.x; i < rows && i < rows_left; i += kBinBlock) {
+    const A v = s_acc[i];
+    if (v != (A)0) atomic_add_elem<T>(out + i, (T)v);
+    if (COUNT) {
+      const int32_t c = s_num[i];
+      if (c != 0) atomicAdd(p.count_out + ((int64_t)bucket << p.rshift) + i, c);
+    }
+  }
+}
+
+// The same sum from records of several values per entry (BinArgs::planes > 1, bin_place_records_kernel): slot
+// row * planes + k of the table is element k of the row.
+template <typename T, bool COUNT = false>
+__global__ __launch_bounds__(kBinBlock) void bin_add_records_kernel(ScatterArgs a, BinArgs p) {
+  static_assert(sizeof(T) == 4, "4-byte values");
+  typedef typename BinSlot<T>::type A;
+  constexpr int U = 4;
+  __shared__ A s_acc[4096];
+  __shared__ int32_t s_num[COUNT ? 4096 : 1];
+  if (p.unsorted != nullptr && *p.unsorted != 1) return;
+  const int wg = (int)blockIdx.x;
+  const int bucket = p.wg_bucket[wg];
+  if (bucket < 0) return;
+  const int rows = 1 << p.rshift;
+  const int K = p.planes, R = K + 1;
+  for (int i = threadIdx.x; i < rows * K; i += kBinBlock) s_acc[i] = (A)0;
+  if (COUNT) {
+    for (int i = threadIdx.x; i < rows; i += kBinBlock) s_num[i] = 0;
+  }
+  __syncthreads();
+  const int64_t lo = p.starts[bucket] + ((int64_t)wg - p.chunk_start[bucket]) * p.chunk;
+  int64_t hi = lo + p.chunk;
+  if (hi > p.starts[bucket + 1]) hi = p.starts[bucket + 1];
+  const uint32_t *words = reinterpret_cast<const uint32_t *>(p.binned);
+  for (int64_t base = lo; base < hi; base += (int64_t)U * kBinBlock) {
+    uint32_t w[U][kBinPayloadCols + 1];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int64_t e = base + (int64_t)u * kBinBlock + threadIdx.x;
+      const uint32_t *rec = words + (e < hi ? e : lo) * R;
+#pragma unroll
+      for (int k = 0; k <= kBinPayloadCols; ++k) w[u][k] = k < R ? __builtin_nontemporal_load(rec + k) : 0u;
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (base + (int64_t)u * kBinBlock + threadIdx.x >= hi) continue;
+      uint32_t tail = 0;
+#pragma unroll
+      for (int k = 0; k <= kBinPayloadCols; ++k) tail = k == K ? w[u][k] : tail;
+      const uint32_t row = tail & (uint32_t)(rows - 1);
+#pragma unroll
+      for (int k = 0; k < kBinPayloadCols; ++k) {
+        if (k >= K) break;
+        T v;
+        __builtin_memcpy(&v, &w[u][k], 4);
+        __hip_atomic_fetch_add(&s_acc[row * K + k], (A)v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      }
+      if (COUNT) __hip_atomic_fetch_add(&s_num[row], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
+  }
+  __syncthreads();
+  T *out = static_cast<T *>(a.out) + ((int64_t)bucket << p.rshift) * K;
+  const int64_t rows_left = a.B * a.N - ((int64_t)bucket << p.rshift);  // rows that exist
+  for (int i = threadIdx.x; i < rows * K && i < rows_left * K; i += kBinBlock) {
     const A v = s_acc[i];
     if (v != (A)0) atomic_add_elem<T>(out + i, (T)v);
   }
@@ -1325,7 +1441,10 @@ void launch_binned_add(const ScatterArgs &a, const BinArgs &plan, int lshift, hi
     hipLaunchKernelGGL(bin_zero_out_kernel<T>, dim3(grid_for(zero_out)), dim3(kBlock), 0, stream, static_cast<T *>(a.out),
                        zero_out, p.unsorted);
   hipLaunchKernelGGL(bin_scan_kernel, dim3(1), dim3(kBinBlock), 0, stream, p);
-  if (bin_place_sorted_ok(p))
+  if (p.payload && p.planes > 1)
+    hipLaunchKernelGGL(bin_place_records_kernel, dim3((unsigned)((a.B * a.E + p.sort_tile - 1) / p.sort_tile)),
+                       dim3(kBinPlaceBlock), 0, stream, a, p);
+  else if (bin_place_sorted_ok(p))
     hipLaunchKernelGGL(bin_place_sorted_kernel, dim3((unsigned)((a.B * a.E + kBinSortTile - 1) / kBinSortTile)),
                        dim3(kBinPlaceBlock), 0, stream, a, p);
   else if (p.nb <= kBinSmallCap)  // 64 KB of cursors, two workgroups per CU; above: 128 KB, one
@@ -1333,6 +1452,13 @@ void launch_binned_add(const ScatterArgs &a, const BinArgs &plan, int lshift, hi
   else
     hipLaunchKernelGGL(bin_place_kernel<kBinMaxBuckets>, dim3((unsigned)p.n_place), dim3(kBinPlaceBlock), 0, stream, a, p);
   if constexpr (sizeof(T) == 4) {
+    if (p.payload && p.planes > 1) {
+      if (p.count_out != nullptr)
+        hipLaunchKernelGGL((bin_add_records_kernel<T, true>), dim3((unsigned)p.max_wgs), dim3(kBinBlock), 0, stream, a, p);
+      else
+        hipLaunchKernelGGL((bin_add_records_kernel<T, false>), dim3((unsigned)p.max_wgs), dim3(kBinBlock), 0, stream, a, p);
+      return;
+    }
     if (p.payload) {
       if (p.count_out != nullptr)
         hipLaunchKernelGGL((bin_add_payload_kernel<T, true>), dim3((unsigned)p.max_wgs), dim3(kBinBlock), 0, stream, a, p);
