@@ -217,7 +217,9 @@ inline BinPlan bin_plan_payload(int64_t B, int64_t E, int64_t K, int64_t N, int 
   // from 2 M entries: an even index gains from there on (74 against 106 us; 2.3 M entries of a graph in random order
   // 85 against 125 us); a skewed one, which the sample hands to the table kernel, pays about 15 us for the launches
   // that return at once (2.3 M entries: 51 against 36 us)
-  if (!any_size && n_edges < ((int64_t)1 << 21)) return r;
+  // (several values per entry: the place pass grows with them, the atomics they replace do not -- three values from
+  // 3 M entries, four from 4 M: 2.2 M / 3 M entries of four floats 121 / 149 us against 115 / 155 us)
+  if (!any_size && n_edges < (K <= 2 ? (int64_t)1 << 21 : K == 3 ? (int64_t)3 << 20 : (int64_t)1 << 22)) return r;
   // chunk: entries per reducing workgroup, about 1024 workgroups, 2048 ... 65536 entries
   int64_t chunk = (n_edges / 1024 + 1023) & ~(int64_t)1023;
   if (chunk < 2048) chunk = 2048;

@@ -1047,7 +1047,7 @@ def test_scatter_sum_narrow_rows_sample_picks_the_kernel(capi, oracle, shape, ki
     L = capi.lib()
     need = L.ts_scatter_workspace_bytes(capi._i(B), capi._i(E), capi._i(K), capi._i(N), capi.DTYPE[dtype], capi.SUM)
     # (rows of up to four floats from 2^21 entries: the value buckets, with scratch for the binned records)
-    value_buckets = dtype == torch.float32 and K <= 4 and B * E >= 1 << 21
+    value_buckets = dtype == torch.float32 and K <= 4 and B * E >= (1 << 21 if K <= 2 else 3 << 20 if K == 3 else 1 << 22)
     by_sample = not value_buckets and B * E * K >= (1 << 23) and (K < 32 or dtype == torch.float32)
     if value_buckets:
         assert need >= 4 * B * E * (K + 1)
@@ -1922,11 +1922,11 @@ def test_scatter_sum_of_single_values_through_slabs(capi, case, dtype, out_given
 
 VALUE_ROW_CASES = [
     # B, E, K, N, kind, forced (TS_SCATTER_BINNED=2: below the size from which the value buckets take a call)
-    (1, (1 << 21) + 77, 3, 300_000, "uniform", False), (1, (1 << 21) + 2, 2, 1_000_000, "uniform", False),
-    (1, 2_500_001, 3, 40_000, "zipf", False), (1, 2_200_000, 2, 5000, "sorted", False),
+    (1, (3 << 20) + 77, 3, 300_000, "uniform", False), (1, (1 << 21) + 2, 2, 1_000_000, "uniform", False),
+    (1, 3_200_001, 3, 40_000, "zipf", False), (1, 2_200_000, 2, 5000, "sorted", False),
     (1, 90_001, 2, 5000, "uniform", True), (2, 50_003, 3, 3000, "hub", True), (1, 70_000, 2, 9000, "zipf", True),
     (1, 30_000, 3, 200_000, "uniform", True), (3, 20_001, 2, 100, "uniform", True), (1, 40_000, 3, 700, "sorted", True),
-    (1, (1 << 21) + 5, 4, 700_000, "uniform", False), (2, 33_333, 4, 2500, "hub", True), (1, 3, 4, 2, "uniform", True),
+    (1, (1 << 22) + 5, 4, 700_000, "uniform", False), (2, 33_333, 4, 2500, "hub", True), (1, 3, 4, 2, "uniform", True),
 ]
 
 
