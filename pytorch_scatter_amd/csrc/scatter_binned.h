@@ -375,8 +375,11 @@ __device__ __forceinline__ int32_t bin_take(int32_t *counter, int32_t bucket) {
 // runs, and finding that out with the full count pass costs 60-150 us for 10 M entries. It is a question of speed
 // only (both paths are correct for any index), so a sample answers it: 1024 evenly spaced entries and their right
 // neighbours, *flag = 1 (not sorted) if at least 1/64 of the pairs descend.
-static __global__ __launch_bounds__(kBinBlock) void bin_sample_kernel(ScatterArgs a, int *flag) {
+// (totals: the buckets' counts [nb], cleared here on the way, which saves their own launch; null: none)
+static __global__ __launch_bounds__(kBinBlock) void bin_sample_kernel(ScatterArgs a, int *flag,
+                                                                      unsigned long long *totals = nullptr, int nb = 0) {
   __shared__ int s_desc;
+  for (int i = threadIdx.x; i < nb; i += kBinBlock) totals[i] = 0;
   if (threadIdx.x == 0) s_desc = 0;
   __syncthreads();
   const int64_t n = a.B * a.E;  // the host launches this only with n >= 2 * kBinBlock
@@ -403,10 +406,12 @@ static __global__ __launch_bounds__(kBinBlock) void bin_sample_kernel(ScatterArg
 // launches that return included; the buckets' time does not depend on where the hot rows lie.)
 // (quarters: the bar in quarters of the sample. Several values per entry: one half, since the buckets' time grows with
 // the values per entry and the table's does not.)
-static __global__ __launch_bounds__(kBinBlock) void bin_sample_skew_kernel(ScatterArgs a, int *flag, int quarters) {
+static __global__ __launch_bounds__(kBinBlock) void bin_sample_skew_kernel(ScatterArgs a, int *flag, int quarters,
+                                                                           unsigned long long *totals, int nb) {
   constexpr int kSlots = 2048;
   __shared__ int s_set[kSlots];
   __shared__ int s_desc, s_dup;
+  for (int i = threadIdx.x; i < nb; i += kBinBlock) totals[i] = 0;  // (the buckets' counts, cleared on the way)
   for (int i = threadIdx.x; i < kSlots; i += kBinBlock) s_set[i] = -1;
   if (threadIdx.x == 0) { s_desc = 0; s_dup = 0; }
   __syncthreads();
@@ -1433,11 +1438,13 @@ void launch_binned_add(const ScatterArgs &a, const BinArgs &plan, int lshift, hi
     p.strict = 1;
   }
   if (p.sampled && three_way)
-    hipLaunchKernelGGL(bin_sample_skew_kernel, dim3(1), dim3(kBinBlock), 0, stream, a, p.unsorted, p.planes > 1 ? 2 : 3);
+    hipLaunchKernelGGL(bin_sample_skew_kernel, dim3(1), dim3(kBinBlock), 0, stream, a, p.unsorted, p.planes > 1 ? 2 : 3,
+                       p.totals, p.nb);
   else if (p.sampled)
-    hipLaunchKernelGGL(bin_sample_kernel, dim3(1), dim3(kBinBlock), 0, stream, a, p.unsorted);
-  hipLaunchKernelGGL(bin_clear_kernel, dim3((p.nb + kBlock - 1) / kBlock), dim3(kBlock), 0, stream, p.totals, p.nb,
-                     p.sampled ? (int *)nullptr : p.unsorted);
+    hipLaunchKernelGGL(bin_sample_kernel, dim3(1), dim3(kBinBlock), 0, stream, a, p.unsorted, p.totals, p.nb);
+  else  // (the sample kernels clear the buckets' counts on the way)
+    hipLaunchKernelGGL(bin_clear_kernel, dim3((p.nb + kBlock - 1) / kBlock), dim3(kBlock), 0, stream, p.totals, p.nb,
+                       p.unsorted);
   launch_bin_count(a, p, stream);
   if (zero_out > 0)
     hipLaunchKernelGGL(bin_zero_out_kernel<T>, dim3(grid_for(zero_out)), dim3(kBlock), 0, stream, static_cast<T *>(a.out),
